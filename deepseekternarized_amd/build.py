@@ -1,0 +1,51 @@
+"""Builds libbp_ternary_hip.so (the gfx950 kernels and their C ABI) in-tree with hipcc.
+
+    python -m deepseekternarized_amd.build
+
+The shared object lands next to this file; it is what ``deepseekternarized_amd.kernels.ternary_hip``
+loads with ctypes. hipcc cross-compiles for gfx950 without a GPU present.
+"""
+
+from __future__ import annotations
+
+import subprocess
+import sys
+from concurrent.futures import ThreadPoolExecutor
+from pathlib import Path
+
+HERE = Path(__file__).resolve().parent
+CSRC = HERE / "csrc"
+LIB = HERE / "libbp_ternary_hip.so"
+SOURCES = ["bp_api.hip", "bp_general.hip", "bp_route.hip", "bp_mfma.hip"]
+# packed FP32 VALU ops are disabled for every device object of this library
+FLAGS = ["--offload-arch=gfx950", "-O3", "-fPIC", "-std=c++17", "-Wall", "-Wno-unused-function",
+         "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops"]
+
+
+def _compile(src: str) -> Path:
+    obj = CSRC / (src + ".o")
+    cmd = ["hipcc", *FLAGS, "-c", str(CSRC / src), "-o", str(obj)]
+    res = subprocess.run(cmd, capture_output=True, text=True)
+    noise = "is not a recognized feature for this target"
+    err = "\n".join(l for l in res.stderr.splitlines() if noise not in l)
+    if res.returncode != 0:
+        raise RuntimeError(f"hipcc failed for {src}:\n{err}")
+    if err.strip():
+        print(err, file=sys.stderr)
+    return obj
+
+
+def build(verbose: bool = True) -> Path:
+    with ThreadPoolExecutor(max_workers=4) as pool:
+        objs = list(pool.map(_compile, SOURCES))
+    cmd = ["hipcc", "--offload-arch=gfx950", "-shared", "-fPIC", *map(str, objs), "-o", str(LIB)]
+    res = subprocess.run(cmd, capture_output=True, text=True)
+    if res.returncode != 0:
+        raise RuntimeError(f"link failed:\n{res.stderr}")
+    if verbose:
+        print(f"built {LIB}")
+    return LIB
+
+
+if __name__ == "__main__":
+    build()

@@ -1,0 +1,110 @@
+// C entry point of the grouped ternary GEMM: argument validation (the checks of the reference
+// launcher, boilerplate/kernels/csrc/ternary_cuda_kernel.cu:109-141, done without any
+// device-to-host copy), kernel selection, and the thread-local error/kernel-name plumbing.
+#include <cstdarg>
+#include <cstdio>
+#include <cstring>
+
+#include "bp_common.h"
+
+namespace bp {
+namespace {
+thread_local char g_error[512] = "";
+thread_local char g_kernel[96] = "";
+thread_local int g_policy = 0;
+}  // namespace
+
+int fail(int code, const char* fmt, ...) {
+  va_list ap;
+  va_start(ap, fmt);
+  vsnprintf(g_error, sizeof(g_error), fmt, ap);
+  va_end(ap);
+  return code;
+}
+
+void note_kernel(const char* name) {
+  strncpy(g_kernel, name, sizeof(g_kernel) - 1);
+  g_kernel[sizeof(g_kernel) - 1] = 0;
+}
+
+int check_launch(const char* what) {
+  const hipError_t e = hipGetLastError();
+  if (e != hipSuccess) return fail(BP_ERR_LAUNCH, "%s: %s", what, hipGetErrorString(e));
+  return BP_OK;
+}
+}  // namespace bp
+
+using namespace bp;
+
+extern "C" const char* bp_last_error(void) { return g_error; }
+extern "C" const char* bp_last_kernel(void) { return g_kernel; }
+extern "C" const char* bp_version(void) { return "bp_ternary_hip gfx950"; }
+
+extern "C" int bp_set_kernel_policy(int policy) {
+  const int old = g_policy;
+  if (policy >= 0 && policy <= 2) g_policy = policy;
+  return old;
+}
+
+static bool valid_scale_dtype(int d) { return d == BP_F32 || d == BP_F16 || d == BP_BF16; }
+static bool valid_act_dtype(int d) { return d == BP_I8 || d == BP_BF16 || d == BP_F16 || d == BP_F32; }
+
+extern "C" int bp_ternary_grouped_gemm(float* out, const void* x, int x_dtype, const float* x_scale,
+                                       const int64_t* offsets, const int64_t* offsets_host,
+                                       const uint8_t* const* packed, const void* const* w_scale, int scale_dtype,
+                                       int n_terms, int64_t T, int64_t N, int64_t K, int64_t Kp, int64_t G,
+                                       int64_t group, int64_t E, int fmt, int64_t max_rows, const int8_t* lut1,
+                                       void* stream) {
+  (void)lut1;  // the kernels carry the table themselves; see bp_tq1_lut for the tensor form
+  g_error[0] = 0;
+  g_kernel[0] = 0;
+  if (!valid_act_dtype(x_dtype)) return fail(BP_ERR_ARG, "unexpected ternary GEMM activation dtype");
+  if (!valid_scale_dtype(scale_dtype)) return fail(BP_ERR_ARG, "unexpected ternary GEMM scale dtype");
+  if (fmt != BP_TQ1 && fmt != BP_TQ2) return fail(BP_ERR_ARG, "fmt must be 1 (TQ1) or 2 (TQ2)");
+  if (n_terms < 1 || n_terms > BP_MAX_TERMS) return fail(BP_ERR_ARG, "n_terms must be in 1..%d", BP_MAX_TERMS);
+  // 127 * group must fit the int32 group accumulator (ternary_cuda_kernel.cu:120-121)
+  if (K <= 0 || K > ((int64_t)1 << 40) || group <= 0 || group > ((int64_t)1 << 24))
+    return fail(BP_ERR_ARG, "invalid ternary GEMM K or group");
+  const int64_t per = fmt == BP_TQ2 ? 4 : 5;
+  if (Kp != K / per + (K % per != 0) || G != K / group + (K % group != 0))
+    return fail(BP_ERR_ARG, "inconsistent ternary GEMM shapes (Kp or G does not match K)");
+  if (T < 0 || N < 0 || E < 0 || T > ((int64_t)1 << 40) || N > ((int64_t)1 << 40))
+    return fail(BP_ERR_ARG, "bad output shape");
+  if (E > 65535) return fail(BP_ERR_ARG, "too many experts for one launch (grid y limit)");
+  if (max_rows < 0) return fail(BP_ERR_ARG, "max_rows must not be negative");
+  if (!offsets && E > 0) return fail(BP_ERR_ARG, "offsets must be a device pointer to E + 1 values");
+  if (!packed || !w_scale) return fail(BP_ERR_ARG, "null term arrays");
+  if (offsets_host) {
+    // the reference validates a host copy of the offsets on every call (ternary_cuda_kernel.cu:130-139)
+    int64_t widest = 0;
+    if (offsets_host[0] != 0 || offsets_host[E] != T)
+      return fail(BP_ERR_OFFSETS, "offsets must start at 0 and end at the row count");
+    for (int64_t e = 0; e < E; ++e) {
+      if (offsets_host[e + 1] < offsets_host[e]) return fail(BP_ERR_OFFSETS, "offsets must be nondecreasing");
+      const int64_t w = offsets_host[e + 1] - offsets_host[e];
+      if (w > widest) widest = w;
+    }
+    if (max_rows < widest) return fail(BP_ERR_ARG, "max_rows is smaller than the largest expert row count");
+    max_rows = widest;
+  }
+  if (max_rows > T) max_rows = T;
+  if (max_rows == 0 || N == 0 || E == 0 || T == 0) return BP_OK;
+  if (!out || !x) return fail(BP_ERR_ARG, "null out or x");
+  if (x_dtype == BP_I8 && !x_scale) return fail(BP_ERR_ARG, "int8 activations need x_scale");
+
+  GemmArgs a;
+  memset(&a, 0, sizeof(a));
+  a.out = out; a.x = x; a.x_scale = x_scale; a.offsets = offsets;
+  for (int t = 0; t < n_terms; ++t) {
+    if (!packed[t] || !w_scale[t]) return fail(BP_ERR_ARG, "null packed or scale pointer in term %d", t);
+    a.packed[t] = packed[t];
+    a.w_scale[t] = w_scale[t];
+  }
+  a.x_dtype = x_dtype; a.scale_dtype = scale_dtype; a.n_terms = n_terms; a.fmt = fmt;
+  a.T = T; a.N = N; a.K = K; a.Kp = Kp; a.G = G; a.group = group; a.E = E; a.max_rows = max_rows;
+
+  hipStream_t s = (hipStream_t)stream;
+  if (g_policy != 1 && mfma_supports(a)) return launch_mfma(a, s);
+  if (g_policy == 2) return fail(BP_ERR_UNSUPPORTED, "shape is outside the tuned kernels (policy 2 forbids the general kernel)");
+  return launch_general(a, s);
+}

@@ -1,0 +1,78 @@
+// Shared declarations for the gfx950 ternary kernels: error reporting, dtype helpers, launch
+// argument blocks. Host and device code of libbp_ternary_hip.so include this.
+#pragma once
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+#include "../../include/bp_ternary.h"
+
+namespace bp {
+
+// ---- host-side error plumbing (thread local, surfaced through bp_last_error) ----
+int fail(int code, const char* fmt, ...);
+void note_kernel(const char* name);
+int check_launch(const char* what);
+
+// ---- argument block of one grouped GEMM call (validated by the C entry point) ----
+struct GemmArgs {
+  float* out;
+  const void* x;
+  const float* x_scale;
+  const int64_t* offsets;
+  const uint8_t* packed[BP_MAX_TERMS];
+  const void* w_scale[BP_MAX_TERMS];
+  int x_dtype, scale_dtype, n_terms, fmt;
+  int64_t T, N, K, Kp, G, group, E, max_rows;
+};
+
+int launch_general(const GemmArgs& a, hipStream_t s);
+// Returns BP_ERR_UNSUPPORTED (without setting an error message) when the shape is outside the
+// tuned kernels' preconditions.
+int launch_mfma(const GemmArgs& a, hipStream_t s);
+bool mfma_supports(const GemmArgs& a);
+
+// ---- device helpers ----
+__device__ __forceinline__ float bf16_bits_to_f32(uint16_t b) { return __uint_as_float(((uint32_t)b) << 16); }
+
+__device__ __forceinline__ uint16_t f32_to_bf16_bits(float f) {  // round to nearest even, NaN kept quiet
+  uint32_t u = __float_as_uint(f);
+  if ((u & 0x7fffffffu) > 0x7f800000u) return (uint16_t)((u >> 16) | 0x0040u);
+  u += 0x7fffu + ((u >> 16) & 1u);
+  return (uint16_t)(u >> 16);
+}
+
+__device__ __forceinline__ float f16_bits_to_f32(uint16_t b) {
+  _Float16 h = __builtin_bit_cast(_Float16, b);
+  return (float)h;
+}
+
+__device__ __forceinline__ float load_scale(const void* p, int dtype, int64_t i) {
+  if (dtype == BP_F32) return ((const float*)p)[i];
+  const uint16_t b = ((const uint16_t*)p)[i];
+  return dtype == BP_F16 ? f16_bits_to_f32(b) : bf16_bits_to_f32(b);
+}
+
+__device__ __forceinline__ float load_act_f32(const void* p, int dtype, int64_t i) {
+  if (dtype == BP_F32) return ((const float*)p)[i];
+  if (dtype == BP_I8) return (float)((const int8_t*)p)[i];
+  const uint16_t b = ((const uint16_t*)p)[i];
+  return dtype == BP_F16 ? f16_bits_to_f32(b) : bf16_bits_to_f32(b);
+}
+
+__device__ __forceinline__ int64_t clamp_i64(int64_t v, int64_t lo, int64_t hi) { return v < lo ? lo : (v > hi ? hi : v); }
+
+// TQ1 digit i of byte v as a trit (boilerplate/ternary/pack.py:62-67): bytes >= 243 decode to 0.
+__device__ __host__ __forceinline__ int tq1_trit(unsigned v, int i) {
+  if (v >= 243u) return 0;
+  const unsigned p = i == 0 ? 1u : i == 1 ? 3u : i == 2 ? 9u : i == 3 ? 27u : 81u;
+  return (int)((v / p) % 3u) - 1;
+}
+
+template <typename T>
+__device__ __forceinline__ T wave_sum(T v) {
+#pragma unroll
+  for (int off = 32; off > 0; off >>= 1) v += __shfl_xor(v, off, 64);
+  return v;
+}
+
+}  // namespace bp

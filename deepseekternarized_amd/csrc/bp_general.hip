@@ -1,0 +1,249 @@
+// General-shape kernels: the any-K / any-group ternary GEMM and the elementwise format kernels
+// (unpack, pack, scale expansion, TQ1 table, int8 activation quantisation).
+//
+// The general GEMM follows the arithmetic of the reference contract literally
+// (boilerplate/kernels/ternary_cuda.py:52-64): exact int32 group sums, then in float32
+// y += float(acc) * scale[g] with the multiply and the add rounded separately, in ascending group
+// order, then y * x_scale. One wavefront owns one output row n of one expert and up to TOK token
+// rows; the 64 lanes stride over the k of a group and the group sum is reduced across the wave.
+#include "bp_common.h"
+
+namespace bp {
+namespace {
+
+constexpr int GEN_WAVES = 4;  // output rows per workgroup
+constexpr int GEN_TOK = 4;    // token rows per pass
+
+__device__ __forceinline__ int decode_trit(const uint8_t* row, int64_t k, int fmt, const int8_t* lut) {
+  if (fmt == BP_TQ2) {
+    const unsigned b = row[k >> 2];
+    return (int)((b >> ((k & 3) * 2)) & 3u) - 1;
+  }
+  const unsigned b = row[k / 5];
+  return lut[b * 5 + (int)(k % 5)];
+}
+
+template <bool INT8>
+__global__ __launch_bounds__(GEN_WAVES * 64) void k_general(GemmArgs a) {
+  __shared__ int8_t lut[256 * 5];
+  for (int i = threadIdx.x; i < 256 * 5; i += blockDim.x) lut[i] = (int8_t)tq1_trit(i / 5, i % 5);
+  __syncthreads();
+  const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+  const int64_t e = blockIdx.y;
+  const int64_t n = (int64_t)blockIdx.x * GEN_WAVES + wave;
+  const int64_t o0 = clamp_i64(a.offsets[e], 0, a.T), o1 = clamp_i64(a.offsets[e + 1], 0, a.T);
+  const int64_t row0 = o0 + (int64_t)blockIdx.z * GEN_TOK;
+  if (n >= a.N || row0 >= o1) return;
+  const int rows = (int)(o1 - row0 < GEN_TOK ? o1 - row0 : GEN_TOK);
+
+  float total[GEN_TOK];
+#pragma unroll
+  for (int r = 0; r < GEN_TOK; ++r) total[r] = 0.f;
+
+  for (int term = 0; term < a.n_terms; ++term) {
+    const uint8_t* wrow = a.packed[term] + (e * a.N + n) * a.Kp;
+    const int64_t sbase = (e * a.N + n) * a.G;
+    float y[GEN_TOK];
+#pragma unroll
+    for (int r = 0; r < GEN_TOK; ++r) y[r] = 0.f;
+    for (int64_t g = 0; g < a.G; ++g) {
+      const int64_t k0 = g * a.group;
+      const int64_t k1 = k0 + a.group < a.K ? k0 + a.group : a.K;
+      const float s = load_scale(a.w_scale[term], a.scale_dtype, sbase + g);
+      if (INT8) {
+        int acc[GEN_TOK];
+#pragma unroll
+        for (int r = 0; r < GEN_TOK; ++r) acc[r] = 0;
+        for (int64_t k = k0 + lane; k < k1; k += 64) {
+          const int t = decode_trit(wrow, k, a.fmt, lut);
+#pragma unroll
+          for (int r = 0; r < GEN_TOK; ++r)
+            if (r < rows) acc[r] += t * (int)((const int8_t*)a.x)[(row0 + r) * a.K + k];
+        }
+#pragma unroll
+        for (int r = 0; r < GEN_TOK; ++r) {
+          const int sum = wave_sum(acc[r]);
+          y[r] = __fadd_rn(y[r], __fmul_rn((float)sum, s));  // out += acc * w_scale[:, g]
+        }
+      } else {
+        float acc[GEN_TOK];
+#pragma unroll
+        for (int r = 0; r < GEN_TOK; ++r) acc[r] = 0.f;
+        for (int64_t k = k0 + lane; k < k1; k += 64) {
+          const int t = decode_trit(wrow, k, a.fmt, lut);
+          if (t != 0) {  // a zero trit never touches x, as in the reference's select-and-add loop
+#pragma unroll
+            for (int r = 0; r < GEN_TOK; ++r)
+              if (r < rows) acc[r] += (float)t * load_act_f32(a.x, a.x_dtype, (row0 + r) * a.K + k);
+          }
+        }
+#pragma unroll
+        for (int r = 0; r < GEN_TOK; ++r) y[r] = __fadd_rn(y[r], __fmul_rn(wave_sum(acc[r]), s));
+      }
+    }
+#pragma unroll
+    for (int r = 0; r < GEN_TOK; ++r) {
+      if (r < rows) {
+        const float v = INT8 ? __fmul_rn(y[r], a.x_scale[row0 + r]) : y[r];
+        total[r] = term == 0 ? v : __fadd_rn(total[r], v);
+      }
+    }
+  }
+  if (lane == 0) {
+#pragma unroll
+    for (int r = 0; r < GEN_TOK; ++r)
+      if (r < rows) a.out[(row0 + r) * a.N + n] = __fadd_rn(a.out[(row0 + r) * a.N + n], total[r]);
+  }
+}
+
+// ---- format kernels ------------------------------------------------------------------------
+
+__global__ __launch_bounds__(256) void k_unpack(int8_t* __restrict__ trits, const uint8_t* __restrict__ packed,
+                                                int64_t N, int64_t K, int64_t Kp, int fmt) {
+  const int per = fmt == BP_TQ2 ? 4 : 5;
+  const int64_t total = N * Kp;
+  for (int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; i < total; i += (int64_t)gridDim.x * blockDim.x) {
+    const int64_t n = i / Kp, b = i % Kp;
+    const unsigned v = packed[i];
+    for (int d = 0; d < per; ++d) {
+      const int64_t k = b * per + d;
+      if (k < K) trits[n * K + k] = (int8_t)(fmt == BP_TQ2 ? (int)((v >> (2 * d)) & 3u) - 1 : tq1_trit(v, d));
+    }
+  }
+}
+
+__global__ __launch_bounds__(256) void k_pack(uint8_t* __restrict__ packed, const int8_t* __restrict__ trits,
+                                              int64_t N, int64_t K, int64_t Kp, int fmt) {
+  const int per = fmt == BP_TQ2 ? 4 : 5;
+  const int64_t total = N * Kp;
+  for (int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; i < total; i += (int64_t)gridDim.x * blockDim.x) {
+    const int64_t n = i / Kp, b = i % Kp;
+    unsigned v = 0, w = 1;
+    for (int d = 0; d < per; ++d) {
+      const int64_t k = b * per + d;
+      const unsigned u = k < K ? (unsigned)(((int)trits[n * K + k] + 1) & 0xff) : 1u;  // pad digit 1
+      if (fmt == BP_TQ2) v |= u << (2 * d);
+      else { v += u * w; w *= 3u; }
+    }
+    packed[i] = (uint8_t)v;
+  }
+}
+
+__global__ __launch_bounds__(256) void k_expand(float* __restrict__ out, const void* __restrict__ in, int dtype, int64_t n) {
+  for (int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; i < n; i += (int64_t)gridDim.x * blockDim.x)
+    out[i] = load_scale(in, dtype, i);
+}
+
+__global__ void k_lut(int8_t* lut) {
+  for (int i = threadIdx.x; i < 256 * 5; i += blockDim.x) lut[i] = (int8_t)tq1_trit(i / 5, i % 5);
+}
+
+// One workgroup per activation row: absmax reduction, then the quantisation pass.
+__global__ __launch_bounds__(256) void k_quant(int8_t* __restrict__ q, float* __restrict__ s, const void* __restrict__ x,
+                                               int dtype, int64_t K) {
+  __shared__ float part[4];
+  const int64_t m = blockIdx.x;
+  float amax = 0.f;
+  bool nan = false;
+  for (int64_t k = threadIdx.x; k < K; k += blockDim.x) {
+    const float v = load_act_f32(x, dtype, m * K + k);
+    nan |= v != v;
+    amax = fmaxf(amax, fabsf(v));
+  }
+  if (nan) amax = __builtin_nanf("");
+  float w = amax;
+#pragma unroll
+  for (int off = 32; off > 0; off >>= 1) {
+    const float o = __shfl_xor(w, off, 64);
+    w = (w != w || o != o) ? __builtin_nanf("") : fmaxf(w, o);
+  }
+  if ((threadIdx.x & 63) == 0) part[threadIdx.x >> 6] = w;
+  __syncthreads();
+  float a = part[0];
+  for (int i = 1; i < 4; ++i) a = (a != a || part[i] != part[i]) ? __builtin_nanf("") : fmaxf(a, part[i]);
+  float sc = __fdiv_rn(a, 127.0f);
+  sc = sc != sc ? sc : fmaxf(sc, 1e-8f);  // clamp(min=1e-8) keeps NaN
+  if (threadIdx.x == 0) s[m] = sc;
+  for (int64_t k = threadIdx.x; k < K; k += blockDim.x) {
+    const float v = load_act_f32(x, dtype, m * K + k);
+    float r = rintf(__fdiv_rn(v, sc));  // round half to even, like torch.round
+    r = fminf(fmaxf(r, -127.f), 127.f);
+    q[m * K + k] = (int8_t)(r != r ? 0 : (int)r);
+  }
+}
+
+int grid_for(int64_t n) {
+  int64_t g = (n + 255) / 256;
+  return (int)(g < 1 ? 1 : (g > 65535 ? 65535 : g));
+}
+
+}  // namespace
+
+int launch_general(const GemmArgs& a, hipStream_t s) {
+  if (a.max_rows <= 0 || a.N == 0 || a.E == 0) return BP_OK;
+  const int64_t zt = (a.max_rows + GEN_TOK - 1) / GEN_TOK;
+  if (zt > 65535) return fail(BP_ERR_ARG, "too many rows per expert for one launch");
+  const dim3 grid((unsigned)((a.N + GEN_WAVES - 1) / GEN_WAVES), (unsigned)a.E, (unsigned)zt);
+  if (a.x_dtype == BP_I8) {
+    note_kernel("general_i8");
+    hipLaunchKernelGGL(k_general<true>, grid, dim3(GEN_WAVES * 64), 0, s, a);
+  } else {
+    note_kernel("general_float");
+    hipLaunchKernelGGL(k_general<false>, grid, dim3(GEN_WAVES * 64), 0, s, a);
+  }
+  return check_launch("general ternary GEMM");
+}
+
+}  // namespace bp
+
+using namespace bp;
+
+static int fmt_dims(int fmt, int64_t N, int64_t K, int64_t* Kp) {
+  if (fmt != BP_TQ1 && fmt != BP_TQ2) return fail(BP_ERR_ARG, "fmt must be 1 (TQ1) or 2 (TQ2)");
+  if (K <= 0 || K > ((int64_t)1 << 40) || N < 0 || N > ((int64_t)1 << 40)) return fail(BP_ERR_ARG, "invalid N or K");
+  const int64_t per = fmt == BP_TQ2 ? 4 : 5;
+  *Kp = K / per + (K % per != 0);
+  return BP_OK;
+}
+
+extern "C" int bp_unpack_trits(int8_t* trits, const uint8_t* packed, int64_t N, int64_t K, int fmt, void* stream) {
+  int64_t Kp;
+  if (int rc = fmt_dims(fmt, N, K, &Kp)) return rc;
+  if (N == 0) return BP_OK;
+  if (!trits || !packed) return fail(BP_ERR_ARG, "null pointer");
+  hipLaunchKernelGGL(k_unpack, dim3(grid_for(N * Kp)), dim3(256), 0, (hipStream_t)stream, trits, packed, N, K, Kp, fmt);
+  return check_launch("unpack");
+}
+
+extern "C" int bp_pack_trits(uint8_t* packed, const int8_t* trits, int64_t N, int64_t K, int fmt, void* stream) {
+  int64_t Kp;
+  if (int rc = fmt_dims(fmt, N, K, &Kp)) return rc;
+  if (N == 0) return BP_OK;
+  if (!trits || !packed) return fail(BP_ERR_ARG, "null pointer");
+  hipLaunchKernelGGL(k_pack, dim3(grid_for(N * Kp)), dim3(256), 0, (hipStream_t)stream, packed, trits, N, K, Kp, fmt);
+  return check_launch("pack");
+}
+
+extern "C" int bp_expand_scales(float* out, const void* scale, int scale_dtype, int64_t n, void* stream) {
+  if (scale_dtype != BP_F16 && scale_dtype != BP_BF16 && scale_dtype != BP_F32) return fail(BP_ERR_ARG, "scale dtype must be f16, bf16 or f32");
+  if (n < 0) return fail(BP_ERR_ARG, "negative element count");
+  if (n == 0) return BP_OK;
+  if (!out || !scale) return fail(BP_ERR_ARG, "null pointer");
+  hipLaunchKernelGGL(k_expand, dim3(grid_for(n)), dim3(256), 0, (hipStream_t)stream, out, scale, scale_dtype, n);
+  return check_launch("expand_scales");
+}
+
+extern "C" int bp_tq1_lut(int8_t* lut, void* stream) {
+  if (!lut) return fail(BP_ERR_ARG, "null pointer");
+  hipLaunchKernelGGL(k_lut, dim3(1), dim3(256), 0, (hipStream_t)stream, lut);
+  return check_launch("tq1_lut");
+}
+
+extern "C" int bp_quant_act_int8(int8_t* q, float* s, const void* x, int x_dtype, int64_t M, int64_t K, void* stream) {
+  if (x_dtype != BP_BF16 && x_dtype != BP_F16 && x_dtype != BP_F32) return fail(BP_ERR_ARG, "activation dtype must be bf16, f16 or f32");
+  if (M < 0 || K <= 0 || M > 0x7fffffff) return fail(BP_ERR_ARG, "invalid M or K");
+  if (M == 0) return BP_OK;
+  if (!q || !s || !x) return fail(BP_ERR_ARG, "null pointer");
+  hipLaunchKernelGGL(k_quant, dim3((unsigned)M), dim3(256), 0, (hipStream_t)stream, q, s, x, x_dtype, K);
+  return check_launch("quant_act_int8");
+}

@@ -1,0 +1,211 @@
+// Token-to-expert routing kernels around the grouped GEMM: stable counting sort of expert ids,
+// row gather (the x[order // k] permute), and the two elementwise stages of an expert MLP
+// (SwiGLU, weighted combine) with the reference engine's bf16 rounding points.
+#include "bp_common.h"
+
+namespace bp {
+namespace {
+
+constexpr int SORT_THREADS = 1024;
+constexpr int SORT_WAVES = SORT_THREADS / 64;
+constexpr int64_t SORT_LDS_INTS = 32768;  // 128 KiB of per-wave histograms in LDS
+
+// One workgroup. Wave w owns the contiguous segment [w*seg, (w+1)*seg) of ids.
+// Pass 1: per-wave histograms. Scan: offsets and, per wave, the first output slot of each expert.
+// Pass 2: every wave walks its segment in order, 64 ids at a time; lanes holding the same expert are
+// ranked by lane index (ballot + popcount), so equal ids keep their input order (stable).
+__global__ __launch_bounds__(SORT_THREADS) void k_sort(int64_t* __restrict__ order, int64_t* __restrict__ offsets,
+                                                        const int64_t* __restrict__ ids, int64_t n, int64_t E,
+                                                        int32_t* __restrict__ ws, int32_t* __restrict__ bad) {
+  extern __shared__ int32_t lds_hist[];
+  int32_t* hist = ws ? ws : lds_hist;  // [SORT_WAVES][E]
+  __shared__ int64_t carry;
+  const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+  for (int64_t i = threadIdx.x; i < SORT_WAVES * E; i += SORT_THREADS) hist[i] = 0;
+  if (threadIdx.x == 0) carry = 0;
+  __syncthreads();
+  const int64_t seg = (n + SORT_WAVES - 1) / SORT_WAVES;
+  const int64_t lo = wave * seg, hi = lo + seg < n ? lo + seg : n;
+  int32_t* mine = hist + wave * E;
+  for (int64_t i = lo + lane; i < hi; i += 64) {
+    const int64_t id = ids[i];
+    if (id >= 0 && id < E) atomicAdd(&mine[id], 1);
+    else if (bad) *bad = 1;
+  }
+  __threadfence();
+  __syncthreads();
+  // exclusive scan over experts of the column sums; chunks of SORT_THREADS experts at a time
+  __shared__ int64_t scan[SORT_THREADS];
+  for (int64_t e0 = 0; e0 < E; e0 += SORT_THREADS) {
+    const int64_t e = e0 + threadIdx.x;
+    int64_t cnt = 0;
+    if (e < E)
+      for (int w = 0; w < SORT_WAVES; ++w) cnt += hist[w * E + e];
+    scan[threadIdx.x] = cnt;
+    __syncthreads();
+    for (int off = 1; off < SORT_THREADS; off <<= 1) {
+      const int64_t v = threadIdx.x >= off ? scan[threadIdx.x - off] : 0;
+      __syncthreads();
+      scan[threadIdx.x] += v;
+      __syncthreads();
+    }
+    const int64_t base = carry + scan[threadIdx.x] - cnt;  // exclusive prefix for expert e
+    if (e < E) {
+      offsets[e] = base;
+      int64_t run = base;
+      for (int w = 0; w < SORT_WAVES; ++w) {  // turn counts into first slots per wave
+        const int32_t c = hist[w * E + e];
+        hist[w * E + e] = (int32_t)run;
+        run += c;
+      }
+    }
+    __syncthreads();
+    if (threadIdx.x == SORT_THREADS - 1) carry += scan[SORT_THREADS - 1];
+    __syncthreads();
+  }
+  if (threadIdx.x == 0) offsets[E] = carry;
+  __threadfence();
+  __syncthreads();
+  for (int64_t i0 = lo; i0 < hi; i0 += 64) {
+    const int64_t i = i0 + lane;
+    const bool live = i < hi;
+    const int64_t id = live ? ids[i] : -1;
+    bool todo = live && id >= 0 && id < E;
+    while (__any(todo)) {
+      const unsigned long long pending = __ballot(todo);
+      const int leader = __ffsll((long long)pending) - 1;
+      const int64_t key = __shfl(id, leader, 64);
+      const bool same = todo && id == key;
+      const unsigned long long m = __ballot(same);
+      int32_t first = 0;
+      if (lane == leader) first = atomicAdd(&mine[key], (int32_t)__popcll(m));  // claims the run of slots
+      first = __shfl(first, leader, 64);
+      if (same) {
+        order[first + __popcll(m & ((1ull << lane) - 1ull))] = i;
+        todo = false;
+      }
+    }
+  }
+}
+
+__global__ __launch_bounds__(256) void k_gather(uint16_t* __restrict__ dst, const uint16_t* __restrict__ src,
+                                                const int64_t* __restrict__ index, int64_t divisor, int64_t src_rows,
+                                                int64_t row_halfs) {
+  const int64_t r = blockIdx.x;
+  int64_t srow = index[r] / divisor;
+  srow = clamp_i64(srow, 0, src_rows - 1);
+  const uint16_t* s = src + srow * row_halfs;
+  uint16_t* d = dst + r * row_halfs;
+  if ((row_halfs & 7) == 0 && (((uintptr_t)src | (uintptr_t)dst) & 15) == 0) {
+    const uint4* s4 = (const uint4*)s;
+    uint4* d4 = (uint4*)d;
+    for (int64_t i = threadIdx.x; i < row_halfs / 8; i += blockDim.x) d4[i] = s4[i];
+  } else {
+    for (int64_t i = threadIdx.x; i < row_halfs; i += blockDim.x) d[i] = s[i];
+  }
+}
+
+__device__ __forceinline__ float round_bf16(float v) { return bf16_bits_to_f32(f32_to_bf16_bits(v)); }
+
+// h = bf16(bf16(silu(bf16 g)) * bf16 u)   (F.silu on a bf16 tensor computes in float32 and rounds once)
+__global__ __launch_bounds__(256) void k_swiglu(uint16_t* __restrict__ h, const float* __restrict__ gate,
+                                                const float* __restrict__ up, int64_t rows, int64_t I, int64_t ld) {
+  const int64_t total = rows * I;
+  for (int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; i < total; i += (int64_t)gridDim.x * blockDim.x) {
+    const int64_t r = i / I, c = i % I;
+    const float g = round_bf16(gate[r * ld + c]);
+    const float u = round_bf16(up[r * ld + c]);
+    const float sg = round_bf16(g / (1.0f + expf(-g)));
+    h[i] = f32_to_bf16_bits(sg * u);
+  }
+}
+
+// out[t, :] = bf16-accumulated sum over the token's slots in ascending expert order.
+__global__ __launch_bounds__(256) void k_combine(uint16_t* __restrict__ out, const float* __restrict__ y,
+                                                 const int64_t* __restrict__ inv, const uint16_t* __restrict__ w,
+                                                 const int64_t* __restrict__ experts, int64_t k, int64_t H) {
+  const int64_t t = blockIdx.x;
+  __shared__ int slot_order[64];
+  if (threadIdx.x == 0) {  // insertion sort of the k slots by expert id (stable)
+    for (int s = 0; s < k; ++s) slot_order[s] = s;
+    for (int i = 1; i < k; ++i) {
+      const int v = slot_order[i];
+      const int64_t ev = experts[t * k + v];
+      int j = i - 1;
+      while (j >= 0 && experts[t * k + slot_order[j]] > ev) { slot_order[j + 1] = slot_order[j]; --j; }
+      slot_order[j + 1] = v;
+    }
+  }
+  __syncthreads();
+  for (int64_t c = threadIdx.x; c < H; c += blockDim.x) {
+    float acc = 0.f;
+    for (int s = 0; s < k; ++s) {
+      const int slot = slot_order[s];
+      const int64_t pos = inv[t * k + slot];
+      const float v = round_bf16(round_bf16(y[pos * H + c]) * bf16_bits_to_f32(w[t * k + slot]));
+      acc = round_bf16(acc + v);
+    }
+    out[t * H + c] = f32_to_bf16_bits(acc);
+  }
+}
+
+}  // namespace
+}  // namespace bp
+
+using namespace bp;
+
+extern "C" int64_t bp_sort_workspace_ints(int64_t n, int64_t E) {
+  (void)n;
+  if (E <= 0) return 0;
+  return SORT_WAVES * E <= SORT_LDS_INTS ? 0 : SORT_WAVES * E;
+}
+
+extern "C" int bp_sort_by_expert(int64_t* order, int64_t* offsets, const int64_t* ids, int64_t n, int64_t E,
+                                 int32_t* workspace, int32_t* bad, void* stream) {
+  if (n < 0 || E < 0 || E > ((int64_t)1 << 24) || n > ((int64_t)1 << 31) - 1) return fail(BP_ERR_ARG, "invalid n or E");
+  if (!offsets || (n > 0 && (!order || !ids))) return fail(BP_ERR_ARG, "null pointer");
+  const int64_t need = bp_sort_workspace_ints(n, E);
+  if (need > 0 && !workspace) return fail(BP_ERR_ARG, "sort_by_expert needs a workspace for this many experts");
+  const size_t lds = need > 0 ? 0 : (size_t)(SORT_WAVES * (E > 0 ? E : 1)) * sizeof(int32_t);
+  static bool attr_set = false;
+  if (!attr_set) {
+    if (hipFuncSetAttribute((const void*)k_sort, hipFuncAttributeMaxDynamicSharedMemorySize, (int)(SORT_LDS_INTS * 4)) != hipSuccess)
+      return fail(BP_ERR_LAUNCH, "cannot raise the dynamic LDS limit for sort_by_expert");
+    attr_set = true;
+  }
+  hipLaunchKernelGGL(k_sort, dim3(1), dim3(SORT_THREADS), lds, (hipStream_t)stream, order, offsets, ids, n, E,
+                     need > 0 ? workspace : (int32_t*)nullptr, bad);
+  return check_launch("sort_by_expert");
+}
+
+extern "C" int bp_gather_rows(void* dst, const void* src, const int64_t* index, int64_t divisor, int64_t rows,
+                              int64_t src_rows, int64_t row_bytes, void* stream) {
+  if (rows < 0 || src_rows < 0 || row_bytes <= 0 || (row_bytes & 1) || divisor <= 0 || rows > 0x7fffffff)
+    return fail(BP_ERR_ARG, "invalid gather dimensions");
+  if (rows == 0) return BP_OK;
+  if (src_rows == 0) return fail(BP_ERR_ARG, "gather from an empty source");
+  if (!dst || !src || !index) return fail(BP_ERR_ARG, "null pointer");
+  hipLaunchKernelGGL(k_gather, dim3((unsigned)rows), dim3(256), 0, (hipStream_t)stream, (uint16_t*)dst,
+                     (const uint16_t*)src, index, divisor, src_rows, row_bytes / 2);
+  return check_launch("gather_rows");
+}
+
+extern "C" int bp_swiglu_bf16(void* h, const float* gate, const float* up, int64_t rows, int64_t I, int64_t ld_in, void* stream) {
+  if (rows < 0 || I <= 0 || ld_in < I) return fail(BP_ERR_ARG, "invalid SwiGLU dimensions");
+  if (rows == 0) return BP_OK;
+  if (!h || !gate || !up) return fail(BP_ERR_ARG, "null pointer");
+  int64_t g = (rows * I + 255) / 256;
+  if (g > 65535) g = 65535;
+  hipLaunchKernelGGL(k_swiglu, dim3((unsigned)g), dim3(256), 0, (hipStream_t)stream, (uint16_t*)h, gate, up, rows, I, ld_in);
+  return check_launch("swiglu");
+}
+
+extern "C" int bp_moe_combine_bf16(void* out, const float* y, const int64_t* inv, const void* w, const int64_t* experts,
+                                   int64_t T, int64_t k, int64_t H, void* stream) {
+  if (T < 0 || k <= 0 || k > 64 || H <= 0 || T > 0x7fffffff) return fail(BP_ERR_ARG, "invalid combine dimensions (top-k up to 64)");
+  if (T == 0) return BP_OK;
+  if (!out || !y || !inv || !w || !experts) return fail(BP_ERR_ARG, "null pointer");
+  hipLaunchKernelGGL(k_combine, dim3((unsigned)T), dim3(256), 0, (hipStream_t)stream, (uint16_t*)out, y, inv,
+                     (const uint16_t*)w, experts, k, H);
+  return check_launch("moe_combine");
+}

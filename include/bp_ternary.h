@@ -1,0 +1,140 @@
+/* C ABI of libbp_ternary_hip.so: the gfx950 (MI355X) implementation of Boilerplate's ternary
+ * expert-linear path. Plain pointers and sizes only; every pointer marked "device" is HIP device
+ * memory on the current device, `stream` is a hipStream_t (NULL = the default stream).
+ *
+ * Conventions shared by all entry points
+ *   - return value 0 = success; anything else is an error code from enum bp_status, and
+ *     bp_last_error() then returns a message for the calling thread. The reference's native
+ *     boundary raises RuntimeError for every rejected argument
+ *     (boilerplate/kernels/csrc/ternary_cuda_kernel.cu:109-141, tests/test_kernel_security.py:25-38);
+ *     the Python layer turns a nonzero return into RuntimeError with that message.
+ *   - nothing is allocated, freed or retained by the library; launches are asynchronous on `stream`.
+ *   - packed weights use the reference layout unchanged (boilerplate/ternary/pack.py:7-16):
+ *     row-major [N, Kp] uint8 per expert, Kp = ceil(K/4) (TQ2, fmt 2) or ceil(K/5) (TQ1, fmt 1);
+ *     one scale per row per `group` consecutive K entries, [N, G], G = ceil(K/group).
+ */
+#ifndef BP_TERNARY_H
+#define BP_TERNARY_H
+
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+enum bp_status {
+  BP_OK = 0,
+  BP_ERR_ARG = 1,      /* malformed argument (shape, dtype code, null pointer, range) */
+  BP_ERR_OFFSETS = 2,  /* host-visible offsets are not 0-based, nondecreasing and T-terminated */
+  BP_ERR_LAUNCH = 3,   /* HIP reported a launch or runtime error */
+  BP_ERR_UNSUPPORTED = 4
+};
+
+enum bp_dtype {
+  BP_I8 = 0,   /* int8 activations with a per-row float32 scale (ternary.ops.quant_act_int8) */
+  BP_BF16 = 1,
+  BP_F16 = 2,
+  BP_F32 = 3
+};
+
+enum bp_fmt { BP_TQ1 = 1, BP_TQ2 = 2 }; /* the reference's fmt codes (kernels/ternary_cuda.py:46-49) */
+
+#define BP_MAX_TERMS 4
+
+/* Message of the last error on the calling thread ("" when none). */
+const char* bp_last_error(void);
+
+/* Library/ISA identification string, e.g. "bp_ternary_hip gfx950". */
+const char* bp_version(void);
+
+/* Grouped (per-expert) ternary GEMM; the dense GEMM/GEMV is the case E = 1.
+ *
+ *   out[t, n] += x_scale[t] * sum_terms sum_g w_scale[term][e(t), n, g] * sum_{k in g} x[t, k] * trit[term][e(t), n, k]
+ *
+ * Replaces ternary_grouped_gemm_cuda (boilerplate/kernels/csrc/ternary_cuda_kernel.cu:103-152, bound
+ * in ternary_cuda.cpp:7-10) and, for float activations, the CPU twin's float path
+ * (boilerplate/kernels/csrc/boilerplate_cpu.cpp:79-128). Differences from the reference signature,
+ * all additive: activations may be int8 (x_scale used), bf16, f16 or f32 (x_scale ignored, may be
+ * NULL); scales may be f32, f16 or bf16 as stored (ternary/ops.py:37 converts to f32 first);
+ * n_terms stacked terms (Mode C, ternary/ops.py:71-79) are summed in one pass over x.
+ *
+ *   out        device f32 [T, N], accumulated into (the caller zero-fills it, as in the reference)
+ *   x          device [T, K] of x_dtype, rows sorted by expert
+ *   x_scale    device f32 [T] (required for BP_I8)
+ *   offsets    device i64 [E + 1]; expert e owns rows offsets[e] .. offsets[e+1]. Values are clamped
+ *              to [0, T] inside the kernels, so malformed device offsets cannot index out of bounds.
+ *   offsets_host  optional host copy of offsets (NULL to skip): when given it is validated exactly
+ *              like the reference does (start 0, end T, nondecreasing, max_rows >= widest expert)
+ *              and a violation returns BP_ERR_OFFSETS. No device-to-host copy is ever made.
+ *   packed     host array of n_terms device pointers, each u8 [E, N, Kp]
+ *   w_scale    host array of n_terms device pointers, each [E, N, G] of scale_dtype
+ *   max_rows   upper bound on offsets[e+1] - offsets[e] (sizes the launch; T is always safe)
+ *   lut1       device i8 [256, 5] TQ1 table as produced by bp_tq1_lut / pack.tq1_lut(); may be NULL
+ *              (the kernels hold the same table as a constant; when given it is ignored)
+ */
+int bp_ternary_grouped_gemm(float* out, const void* x, int x_dtype, const float* x_scale,
+                            const int64_t* offsets, const int64_t* offsets_host,
+                            const uint8_t* const* packed, const void* const* w_scale, int scale_dtype,
+                            int n_terms, int64_t T, int64_t N, int64_t K, int64_t Kp, int64_t G,
+                            int64_t group, int64_t E, int fmt, int64_t max_rows, const int8_t* lut1,
+                            void* stream);
+
+/* Selects the kernel family for bp_ternary_grouped_gemm on the calling thread:
+ *   0 = automatic (tuned kernels where the shape allows, general kernel otherwise)
+ *   1 = general kernel only (any K, group, format; int8 path bit-identical to
+ *       kernels/ternary_cuda.py:52-64 for one term)
+ *   2 = tuned kernels only (BP_ERR_UNSUPPORTED if the shape is not covered)
+ * Returns the previous value. */
+int bp_set_kernel_policy(int policy);
+
+/* Name of the kernel the last bp_ternary_grouped_gemm on this thread launched ("" if none). */
+const char* bp_last_kernel(void);
+
+/* Packed rows -> int8 trits [N, K]; bit-identical to unpack_tq1/unpack_tq2
+ * (boilerplate/ternary/pack.py:48-51,73-74): TQ2 code 3 -> +2, TQ1 bytes >= 243 -> 0. */
+int bp_unpack_trits(int8_t* trits, const uint8_t* packed, int64_t N, int64_t K, int fmt, void* stream);
+
+/* int8 trits [N, K] -> packed rows [N, Kp]; bit-identical to pack_tq1/pack_tq2
+ * (boilerplate/ternary/pack.py:43-45,57-59), pad digit 1. */
+int bp_pack_trits(uint8_t* packed, const int8_t* trits, int64_t N, int64_t K, int fmt, void* stream);
+
+/* Stored scales (f16 or bf16) -> float32, elementwise; the conversion of ternary/ops.py:37. */
+int bp_expand_scales(float* out, const void* scale, int scale_dtype, int64_t n, void* stream);
+
+/* The reference TQ1 table, [256, 5] int8 (boilerplate/ternary/pack.py:62-67), written to device memory. */
+int bp_tq1_lut(int8_t* lut, void* stream);
+
+/* Per-row absmax int8 quantisation (boilerplate/ternary/ops.py:20-25):
+ * s = max(amax|x| / 127, 1e-8), q = clamp(rint(x / s), -127, 127). x [M, K] of x_dtype (bf16/f16/f32). */
+int bp_quant_act_int8(int8_t* q, float* s, const void* x, int x_dtype, int64_t M, int64_t K, void* stream);
+
+/* Stable counting sort of expert ids (boilerplate/kernels/ternary_cuda.py:114-118):
+ * order[i] = index of the i-th entry in expert order (ties keep input order), offsets = [0, cumsum(counts)].
+ * ids device i64 [n] with values in [0, E) (out-of-range ids are reported through *bad, device i32,
+ * set to 1; may be NULL). workspace: device i32 [bp_sort_workspace_ints(n, E)] or NULL when that is 0. */
+int64_t bp_sort_workspace_ints(int64_t n, int64_t E);
+int bp_sort_by_expert(int64_t* order, int64_t* offsets, const int64_t* ids, int64_t n, int64_t E,
+                      int32_t* workspace, int32_t* bad, void* stream);
+
+/* Row gather dst[i, :] = src[index[i] / divisor, :] (the x[order // k] permute of
+ * scripts/eval/ternary_kernel_bench.py:90-93). row_bytes must be a multiple of 2. */
+int bp_gather_rows(void* dst, const void* src, const int64_t* index, int64_t divisor, int64_t rows,
+                   int64_t src_rows, int64_t row_bytes, void* stream);
+
+/* SwiGLU elementwise stage of an expert MLP (boilerplate/engine/standard.py:151-154):
+ * h = bf16(bf16(silu(bf16 gate)) * bf16 up) from the float32 GEMM outputs gate_up [rows, 2*I]
+ * (gate in columns [0, I), up in [I, 2I)); h bf16 [rows, I]. */
+int bp_swiglu_bf16(void* h, const float* gate, const float* up, int64_t rows, int64_t I, int64_t ld_in, void* stream);
+
+/* Weighted combine of expert outputs (boilerplate/engine/standard.py:173-175):
+ * out[token, :] = sum over that token's slots, in ascending expert order, of
+ * bf16(bf16(y[pos, :]) * w[token, slot]), accumulated in bf16 like index_add_ on a bf16 tensor.
+ * y f32 [T*k, H] in expert-sorted order, inv i64 [T*k] = position of pair (token, slot) in that order,
+ * w bf16 [T, k], experts i64 [T, k] (to order the slots of one token), out bf16 [T, H]. */
+int bp_moe_combine_bf16(void* out, const float* y, const int64_t* inv, const void* w, const int64_t* experts,
+                        int64_t T, int64_t k, int64_t H, void* stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* BP_TERNARY_H */
