@@ -98,7 +98,7 @@ def ref_gemm(x, x_scale, packed, w_scale, K, group, fmt, out=None):
 # --------------------------------------------------------------------------- seeded synthetic inputs
 def synth_trits(rng, shape):
     """iid trits with P(-1) = P(+1) = 0.33, P(0) = 0.34."""
-    u = rng.random(shape)
+    u = rng.random(shape, dtype=np.float32)
     return np.where(u < 0.33, -1, np.where(u < 0.66, 1, 0)).astype(np.int8)
 
 
