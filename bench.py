@@ -1,0 +1,226 @@
+"""Benchmark of the ternary expert-linear path on one MI355X.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload NAME] [--no-extras] [--no-cpu]
+
+A step is one pass of the hot path over one batch of synthetic input: one grouped launch that
+streams L distinct packed linears of the named configuration (L chosen so the packed weights exceed
+the 256 MB Infinity Cache, i.e. every step reads its weights from HBM). Inputs are resident in HBM
+before the timed region. Prints ONE JSON line:
+
+  metric/value/unit : weight bytes as stored (packed + fp16 scales, the reference's own definition,
+                      scripts/eval/ternary_kernel_bench.py:75-79) per second of wall time over K steps
+  roofline          : the same bytes over the kernel's own average duration (HIP events on the
+                      launch stream) against the 8 TB/s HBM peak
+  cpu_baseline      : the reference's CPU kernel (oracle/_ref, "reference") or this repository's C
+                      port of it ("port") timed on the host cores on one linear of the same workload
+  also              : secondary measurements (other M, single-linear latency, grouped-expert GEMM TFLOP/s)
+"""
+
+from __future__ import annotations
+
+import argparse
+import json
+import os
+import sys
+import time
+from pathlib import Path
+
+ROOT = Path(__file__).resolve().parent
+if str(ROOT) not in sys.path:
+    sys.path.insert(0, str(ROOT))
+
+HBM_PEAK_GBPS = 8000.0
+MFMA_BF16_PEAK_TFLOPS = 2500.0
+GROUP = 128
+
+WORKLOADS = {
+    # name: (fmt, N, K, M tokens per linear, activation, terms, L linears per launch)
+    "cfg1a_tq1_gemv": ("tq1", 2048, 7168, 1, "bf16", 1, 128),
+    "cfg1b_tq1_gemv": ("tq1", 7168, 2048, 1, "bf16", 1, 128),
+    "cfg1a_tq2_gemv": ("tq2", 2048, 7168, 1, "bf16", 1, 128),
+    "cfg0_tq2_gemv": ("tq2", 2048, 4096, 1, "bf16", 1, 192),
+}
+
+
+def synth(bp, torch, E, N, K, fmt, terms, seed=0):
+    """Draw order (device generator, seed given): per term, per expert: uniform [N, K] -> trits with
+    P(-1) = P(+1) = 0.33, P(0) = 0.34; then all scales fp16(0.02 |N(0,1)|) [E, N, G]; later terms reuse
+    the first term's scales times 0.25."""
+    g = torch.Generator(device="cuda").manual_seed(seed)
+    packed, scales = [], []
+    for t in range(terms):
+        p = torch.empty(E, N, bp.packed_cols(fmt, K), dtype=torch.uint8, device="cuda")
+        for e in range(E):
+            u = torch.rand(N, K, device="cuda", generator=g)
+            p[e] = bp.pack(torch.where(u < 0.33, -1, torch.where(u < 0.66, 1, 0)).to(torch.int8), fmt)
+        if t == 0:
+            s0 = (0.02 * torch.randn(E, N, K // GROUP, device="cuda", generator=g).abs()).half()
+            scales.append(s0)
+        else:
+            scales.append((s0.float() * 0.25).half())
+        packed.append(p)
+    return packed, scales
+
+
+def weight_bytes(packed, scales):
+    return sum(p.numel() + 2 * s.numel() for p, s in zip(packed, scales))
+
+
+class Launch:
+    """One grouped launch over E experts with `rows[e]` token rows each, through the native entry."""
+
+    def __init__(self, bp, torch, packed, scales, K, fmt, x, offsets, max_rows, x_scale=None):
+        self.e, self.torch = bp.ext(), torch
+        self.args = (x, x_scale, offsets, packed, scales, K, GROUP, 2 if fmt == "tq2" else 1, None, max_rows)
+        self.out = torch.zeros(x.size(0), packed[0].size(1), dtype=torch.float32, device="cuda")
+
+    def __call__(self):
+        self.e.ternary_grouped_gemm(self.out, *self.args)
+
+    def time(self, steps, warmup):
+        torch = self.torch
+        for _ in range(warmup):
+            self()
+        ev = [(torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)) for _ in range(steps)]
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        for a, b in ev:
+            a.record()
+            self()
+            b.record()
+        torch.cuda.synchronize()
+        wall = (time.perf_counter() - t0) / steps
+        kern = sum(a.elapsed_time(b) for a, b in ev) / steps / 1e3
+        return wall, kern, self.e.last_kernel()
+
+
+def uniform_launch(bp, torch, fmt, N, K, M, act, terms, L, seed=0):
+    packed, scales = synth(bp, torch, L, N, K, fmt, terms, seed)
+    g = torch.Generator(device="cuda").manual_seed(seed + 1)
+    x = torch.randn(L * M, K, device="cuda", generator=g).to(torch.bfloat16)
+    xs = None
+    if act == "int8":
+        x, xs = bp.quant_act_int8(x)
+    offsets = torch.arange(0, L * M + 1, M, device="cuda", dtype=torch.int64)
+    return Launch(bp, torch, packed, scales, K, fmt, x, offsets, M, xs), weight_bytes(packed, scales)
+
+
+def cpu_baseline(fmt, N, K, M, budget_s=12.0):
+    """Times the CPU ternary kernel on one linear of the workload (float32 activations, as the
+    reference's float path takes them) for about `budget_s` seconds of CPU work."""
+    import numpy as np
+
+    sys.path.insert(0, str(ROOT / "tests"))
+    from _util import c_gemm, orc, oracle_c, ref_gemm, reference_build, synth_trits
+
+    rng = np.random.default_rng(0)
+    trits = synth_trits(rng, (N, K))
+    scale = (0.02 * np.abs(rng.standard_normal((N, K // GROUP)))).astype(np.float16).astype(np.float32)
+    packed = orc.pack(trits, fmt)
+    x = rng.standard_normal((M, K)).astype(np.float32)
+    kind = "reference" if reference_build() is not None else "port"
+    fn = (lambda: ref_gemm(x, None, packed, scale, K, GROUP, fmt)) if kind == "reference" else \
+         (lambda: c_gemm(x, None, packed, scale, K, GROUP, fmt))
+    for _ in range(3):
+        fn()
+    reps, t0 = 0, time.perf_counter()
+    while time.perf_counter() - t0 < budget_s and reps < 20000:
+        fn()
+        reps += 1
+    dt = (time.perf_counter() - t0) / reps
+    wbytes = packed.size + 2 * scale.size
+    cores = oracle_c().bp_oracle_max_threads()
+    return {"value": round(wbytes / dt / 1e9, 3), "unit": "GB/s", "cores": int(cores), "kind": kind,
+            "sample": f"one {fmt} linear N={N} K={K} M={M} fp32 activations, {reps} calls, {dt * 1e3:.3f} ms/call, "
+                      f"OpenMP over all {cores} host threads (os.cpu_count()={os.cpu_count()})"}
+
+
+def skewed_offsets(torch, T, E, k, seed=0):
+    """top-k of softmax(N(0, 1.5) logits) per token -> per-expert row counts (skewed loads)."""
+    g = torch.Generator(device="cuda").manual_seed(seed)
+    logits = torch.randn(T, E, device="cuda", generator=g) * 1.5
+    idx = torch.topk(torch.softmax(logits, -1), k, -1).indices.reshape(-1)
+    return idx
+
+
+def main() -> int:
+    ap = argparse.ArgumentParser(description=__doc__.split("\n\n")[0])
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=50)
+    ap.add_argument("--warmup", type=int, default=5)
+    ap.add_argument("--workload", default="cfg1a_tq1_gemv", choices=sorted(WORKLOADS))
+    ap.add_argument("--no-extras", action="store_true", help="skip the secondary measurements")
+    ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline")
+    a = ap.parse_args()
+    if a.gpus != 1:
+        print("bench.py measures one GPU: this build has no multi-GPU path (run with --gpus 1)", file=sys.stderr)
+        return 2
+
+    import torch
+
+    import deepseekternarized_amd as bp
+
+    if not torch.cuda.is_available() or bp.ext() is None:
+        print("bench.py needs a HIP device and the built libbp_ternary_hip.so", file=sys.stderr)
+        return 1
+    fmt, N, K, M, act, terms, L = WORKLOADS[a.workload]
+    launch, wbytes = uniform_launch(bp, torch, fmt, N, K, M, act, terms, L)
+    wall, kern, kname = launch.time(a.steps, a.warmup)
+    act_bytes = L * M * K * 2 + L * M * N * 4 * 2  # bf16 activations read, f32 output read-modify-write
+
+    also = {}
+    if not a.no_extras:
+        del launch
+        torch.cuda.empty_cache()
+        for m in (4, 16, 32):  # the other decode batch sizes of the configuration
+            l2, wb2 = uniform_launch(bp, torch, fmt, N, K, m, act, terms, L)
+            _, k2, kn2 = l2.time(max(5, a.steps // 2), 2)
+            also[f"M{m}_weight_GBps"] = round(wb2 / k2 / 1e9, 1)
+            also[f"M{m}_kernel"] = kn2
+            del l2
+            torch.cuda.empty_cache()
+        l1, wb1 = uniform_launch(bp, torch, fmt, N, K, M, act, terms, 1)  # one linear per launch (cache-resident, latency bound)
+        w1, k1, _ = l1.time(200, 20)
+        also["single_linear_us_per_call"] = round(w1 * 1e6, 2)
+        also["single_linear_weight_GBps"] = round(wb1 / w1 / 1e9, 1)
+        del l1
+        # grouped-expert prefill GEMM: TQ2, two stacked terms, top-6 skewed routing, 32 rows per expert on average
+        E3, N3, K3, T3, k3 = 96, 2048, 4096, 512, 6
+        packed, scales = synth(bp, torch, E3, N3, K3, "tq2", 2, seed=3)
+        ids = skewed_offsets(torch, T3, E3, k3, seed=3)
+        order, offsets = bp.sort_by_expert(ids, E3)
+        from deepseekternarized_amd.kernels.ternary_hip import gather_rows
+
+        xg = gather_rows(torch.randn(T3, K3, device="cuda").to(torch.bfloat16), order, k3)
+        max_rows = int((offsets[1:] - offsets[:-1]).max())
+        l3 = Launch(bp, torch, packed, scales, K3, "tq2", xg, offsets, max_rows)
+        _, k3t, kn3 = l3.time(max(5, a.steps // 2), 2)
+        flops = 2.0 * T3 * k3 * N3 * K3 * 2  # per-term count
+        also["grouped_gemm"] = {"workload": f"cfg3 gate projection at E={E3} of 384 experts: TQ2 k=2, N={N3}, K={K3}, "
+                                            f"{T3 * k3} routed rows (max {max_rows}/expert), bf16 activations",
+                                "TFLOPs_per_term_count": round(flops / k3t / 1e12, 1),
+                                "frac_of_bf16_mfma_peak": round(flops / k3t / 1e12 / MFMA_BF16_PEAK_TFLOPS, 4),
+                                "weight_GBps": round(weight_bytes(packed, scales) / k3t / 1e9, 1), "kernel": kn3,
+                                "us": round(k3t * 1e6, 1)}
+
+    line = {
+        "metric": "ternary GEMV HBM GB/s (% peak); grouped-expert GEMM TFLOP/s (% MFMA peak)",
+        "value": round(wbytes / wall / 1e9, 1), "unit": "GB/s", "n_gpus": 1, "steps": a.steps, "warmup": a.warmup,
+        "ms_per_step": round(wall * 1e3, 5), "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+        "dtype": "bf16", "data": "synthetic",
+        "config": {"workload": f"{a.workload}: {fmt.upper()} decode GEMV N={N} K={K} M={M} {act} activations, group 128, "
+                               f"fp16 scales, {L} distinct linears per launch ({wbytes / 1e6:.0f} MB of weights, > Infinity Cache)",
+                   "kernel": kname, "bytes_counted": "packed + fp16 scales as stored",
+                   "activation_and_output_bytes_per_step": act_bytes},
+        "roofline": {"bound": "hbm", "achieved": round(wbytes / kern / 1e9, 1), "peak": HBM_PEAK_GBPS, "unit": "GB/s",
+                     "frac": round(wbytes / kern / 1e9 / HBM_PEAK_GBPS, 4), "traffic": None,
+                     "kernel_us": round(kern * 1e6, 2)},
+        "cpu_baseline": None if a.no_cpu else cpu_baseline(fmt, N, K, M),
+        "also": also,
+    }
+    print(json.dumps(line))
+    return 0
+
+
+if __name__ == "__main__":
+    raise SystemExit(main())

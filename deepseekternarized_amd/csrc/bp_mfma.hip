@@ -1,6 +1,367 @@
-// placeholder; replaced by the tuned kernels
+// Tuned gfx950 kernels for group = 128: packed trits are decoded through a bank-replicated LDS
+// lookup table straight into MFMA operands, one 16-row x 16-token tile per instruction.
+//
+//   bf16 activations : v_mfma_f32_16x16x32_bf16, table entry = the trits of one byte as bf16
+//   int8 activations : v_mfma_i32_16x16x64_i8,  table entry = the trits of one byte as int8
+//
+// Accumulators are flushed at every 128-wide K group: total += acc * scale[n, g] in float32, so the
+// scale multiplies the group sum exactly as in the reference contract
+// (boilerplate/kernels/ternary_cuda.py:58-63, boilerplate/kernels/csrc/boilerplate_cpu.cpp:114-124).
+// Stacked terms share one staging of the activations and one output write.
+//
+// Work split: a workgroup of WAVES wavefronts owns WAVES*16*R output rows of one expert and 16*MT of
+// its token rows. The activation tile of the workgroup is staged through LDS in K chunks (global
+// loads one chunk ahead, held in registers across the compute of the current chunk), the packed
+// weights stream from HBM exactly once with loads two steps ahead. Operand A = activations (row i =
+// token), operand B = weights (column j = output row), so a lane ends with 4 tokens x 1 output row
+// and needs one scale per group.
+#include <cstdlib>
+
 #include "bp_common.h"
+
 namespace bp {
-bool mfma_supports(const GemmArgs&) { return false; }
-int launch_mfma(const GemmArgs&, hipStream_t) { return BP_ERR_UNSUPPORTED; }
+namespace {
+
+typedef unsigned u32x2 __attribute__((ext_vector_type(2)));
+typedef unsigned u32x4 __attribute__((ext_vector_type(4)));
+typedef float f32x4 __attribute__((ext_vector_type(4)));
+typedef int i32x4 __attribute__((ext_vector_type(4)));
+typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
+typedef __attribute__((address_space(3))) u32x2 lds_u32x2;
+typedef __attribute__((address_space(3))) u32x4 lds_u32x4;
+typedef __attribute__((address_space(3))) unsigned lds_u32;
+
+// LDS map (absolute addresses; these kernels declare no static LDS, so the dynamic allocation
+// requested at launch starts at LDS address 0):
+//   [0, 32 KiB)        decode table: entry of byte value v, copy c at v * 128 + c * EB
+//   [32 KiB, ...)      activation tile: row t at X_BASE + t * pitch, pitch = KC * XB + 16
+constexpr int LUT_STRIDE = 128;
+constexpr int LUT_BYTES = 256 * LUT_STRIDE;
+constexpr int X_BASE = LUT_BYTES;
+constexpr int X_TILE_BYTES = 48 * 1024;  // table + tile = 80 KiB: two workgroups per CU
+
+__device__ __forceinline__ unsigned bf16_of_trit(int t) {
+  return t == 0 ? 0u : t == 1 ? 0x3f80u : t == -1 ? 0xbf80u : 0x4000u;  // +2 (TQ2 code 3) -> 2.0
 }
+
+// LDS address of the table entry of byte `sel` (0..3) of w: (byte << 7) | lane offset.
+__device__ __forceinline__ unsigned lut_addr(unsigned w, unsigned lane_off, int sel) {
+  return (__builtin_amdgcn_ubfe(w, 8 * sel, 8) << 7) | lane_off;
+}
+
+template <int ACT>
+struct Acc;
+template <>
+struct Acc<BP_BF16> { typedef f32x4 type; };
+template <>
+struct Acc<BP_I8> { typedef i32x4 type; };
+
+template <int SDT>
+__device__ __forceinline__ float scale_at(const u32x4 (&raw)[2], int i) {  // i-th of the 8 scales held in raw
+  if (SDT == BP_F32) return __uint_as_float(raw[i >> 2][i & 3]);
+  const unsigned v = raw[0][i >> 1];
+  if (SDT == BP_F16) return f16_bits_to_f32((uint16_t)((i & 1) ? (v >> 16) : (v & 0xffffu)));
+  return __uint_as_float((i & 1) ? (v & 0xffff0000u) : (v << 16));
+}
+
+// ------------------------------------------------------------------------------------------------
+// TQ2. K % 1024 == 0, N % 16 == 0. One step = 64 packed bytes (256 trits, two groups) per row.
+// Lane (r16 = lane % 16, b = lane / 16) loads bytes [16b, 16b + 16) of its row's 64-byte piece; a
+// v_permlane32_swap pair then leaves every lane with 8 bytes of the first group and 8 bytes of the
+// second, so that all four k-blocks of an MFMA belong to one scale group.
+// After the swap block b holds trits tb(b) .. tb(b)+31 of each group, tb = {0, 64, 32, 96}.
+template <int ACT, int SDT, int R, int MT, int WAVES>
+__global__ __launch_bounds__(WAVES * 64, 4) void k_mfma_tq2(GemmArgs a, int KC) {
+  constexpr int THREADS = WAVES * 64;
+  constexpr int EB = ACT == BP_BF16 ? 8 : 4;   // bytes per table entry
+  constexpr int COPIES = LUT_STRIDE / EB;      // 16 (bf16) or 32 (int8) bank-interleaved copies
+  constexpr int XB = ACT == BP_BF16 ? 2 : 1;   // bytes per activation element
+  constexpr int KM = ACT == BP_BF16 ? 8 : 16;  // k per lane per MFMA
+  constexpr int NJ = 32 / KM;                  // MFMAs per group
+  constexpr int XU = X_TILE_BYTES / 16 / THREADS;  // 16-byte units of the activation tile per thread
+
+  // ---- build the table: thread v < 256 writes the entry of byte value v into every copy
+  if (threadIdx.x < 256) {
+    const unsigned v = threadIdx.x;
+    int t[4];
+#pragma unroll
+    for (int d = 0; d < 4; ++d) t[d] = (int)((v >> (2 * d)) & 3u) - 1;
+    if (ACT == BP_BF16) {
+      u32x2 e;
+      e.x = bf16_of_trit(t[0]) | (bf16_of_trit(t[1]) << 16);
+      e.y = bf16_of_trit(t[2]) | (bf16_of_trit(t[3]) << 16);
+      for (int c = 0; c < COPIES; ++c) *(lds_u32x2*)(v * LUT_STRIDE + c * EB) = e;
+    } else {
+      const unsigned e = (unsigned)(t[0] & 0xff) | ((unsigned)(t[1] & 0xff) << 8) | ((unsigned)(t[2] & 0xff) << 16) |
+                         ((unsigned)(t[3] & 0xff) << 24);
+      for (int c = 0; c < COPIES; ++c) *(lds_u32*)(v * LUT_STRIDE + c * EB) = e;
+    }
+  }
+
+  const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+  const int r16 = lane & 15, b = lane >> 4;
+  const int64_t e = blockIdx.y;
+  const int64_t o0 = clamp_i64(a.offsets[e], 0, a.T), o1 = clamp_i64(a.offsets[e + 1], 0, a.T);
+  const int64_t tok0 = o0 + (int64_t)blockIdx.z * (16 * MT);
+  if (tok0 >= o1) return;  // uniform for the workgroup: no barrier is skipped by part of it
+  const int ntok = (int)(o1 - tok0 < 16 * MT ? o1 - tok0 : 16 * MT);
+  int64_t n0 = ((int64_t)blockIdx.x * WAVES + wave) * (16 * R);
+  const bool wave_live = n0 < a.N;
+  if (!wave_live) n0 = 0;  // keeps addresses valid; the wave still takes part in staging and barriers
+  const unsigned lane_off = (unsigned)((lane % COPIES) * EB);
+  const int tb = 64 * (b & 1) + 32 * (b >> 1);
+
+  // row sub-tiles past N re-read the first sub-tile (branch-free loop body) and are dropped at the store
+  bool rows_valid[R];
+  int64_t row_shift[R];
+#pragma unroll
+  for (int r = 0; r < R; ++r) {
+    rows_valid[r] = wave_live && n0 + 16 * r < a.N;
+    row_shift[r] = rows_valid[r] ? 16 * r : 0;
+  }
+
+  // ---- activation tile geometry
+  const int pitch = KC * XB + 16;
+  const int units_per_row = KC * XB / 16;
+  const int units = ntok * units_per_row;
+  unsigned xaddr[MT];  // LDS address of this lane's token row (+ its k-block offset)
+#pragma unroll
+  for (int mt = 0; mt < MT; ++mt) {
+    int t = 16 * mt + r16;
+    if (t >= ntok) t = ntok - 1;
+    xaddr[mt] = (unsigned)(X_BASE + t * pitch + tb * XB);
+  }
+  const unsigned char* xg = (const unsigned char*)a.x + tok0 * a.K * XB;
+  u32x4 xstage[XU];
+  auto stage_load = [&](int64_t k0) {  // global -> registers, chunk starting at k0
+#pragma unroll
+    for (int i = 0; i < XU; ++i) {
+      const int u = threadIdx.x + i * THREADS;
+      if (u < units) {
+        const int row = u / units_per_row, col = u - row * units_per_row;
+        xstage[i] = *(const u32x4*)(xg + ((int64_t)row * a.K + k0) * XB + col * 16);
+      }
+    }
+  };
+  auto stage_store = [&]() {  // registers -> LDS
+#pragma unroll
+    for (int i = 0; i < XU; ++i) {
+      const int u = threadIdx.x + i * THREADS;
+      if (u < units) {
+        const int row = u / units_per_row, col = u - row * units_per_row;
+        *(lds_u32x4*)(X_BASE + row * pitch + col * 16) = xstage[i];
+      }
+    }
+  };
+
+  f32x4 total[R][MT];
+#pragma unroll
+  for (int r = 0; r < R; ++r)
+#pragma unroll
+    for (int mt = 0; mt < MT; ++mt) total[r][mt] = f32x4{0.f, 0.f, 0.f, 0.f};
+
+  const int64_t steps = a.K / 256;
+  const int steps_per_chunk = KC / 256;
+  const int64_t chunks = (steps + steps_per_chunk - 1) / steps_per_chunk;
+
+  for (int term = 0; term < a.n_terms; ++term) {
+    const unsigned char* wbase = a.packed[term] + ((e * a.N + n0 + r16) * a.Kp + 16 * b);
+    const unsigned char* sbase = (const unsigned char*)a.w_scale[term] + (e * a.N + n0 + r16) * a.G * (SDT == BP_F32 ? 4 : 2);
+    u32x4 wq0[R], wq1[R];           // weights of the next two steps
+    u32x4 sraw[R][2], snext[R][2];  // 8 scales (4 steps) per row sub-tile, and the next 8
+    auto fetch_w = [&](int64_t c, u32x4 (&dst)[R]) {
+      const int64_t cc = c < steps ? c : steps - 1;  // past the end: re-read the last step, no branch
+#pragma unroll
+      for (int r = 0; r < R; ++r) dst[r] = *(const u32x4*)(wbase + row_shift[r] * a.Kp + 64 * cc);
+    };
+    auto fetch_s = [&](int64_t c, u32x4 (&dst)[R][2]) {  // scales of steps c .. c+3 (c % 4 == 0)
+      const int64_t cc = c < steps ? c : 0;
+#pragma unroll
+      for (int r = 0; r < R; ++r) {
+        const unsigned char* p = sbase + (row_shift[r] * a.G + 2 * cc) * (SDT == BP_F32 ? 4 : 2);
+        dst[r][0] = *(const u32x4*)p;
+        if (SDT == BP_F32) dst[r][1] = *(const u32x4*)(p + 16);
+      }
+    };
+    const bool restage = term == 0 || chunks > 1;  // a tile that holds all of K is staged once for all terms
+    if (restage) stage_load(0);
+    fetch_w(0, wq0);
+    fetch_w(1, wq1);
+    fetch_s(0, snext);
+    for (int64_t ch = 0; ch < chunks; ++ch) {
+      if (restage) {
+        __syncthreads();  // every wave is done reading the previous tile (and, first time, the table is built)
+        stage_store();
+        __syncthreads();
+      }
+      if (ch + 1 < chunks) stage_load((ch + 1) * KC);
+      const int64_t c_end = (ch + 1) * steps_per_chunk < steps ? (ch + 1) * steps_per_chunk : steps;
+      for (int64_t c = ch * steps_per_chunk; c < c_end; ++c) {
+        u32x4 w[R];
+#pragma unroll
+        for (int r = 0; r < R; ++r) { w[r] = wq0[r]; wq0[r] = wq1[r]; }
+        fetch_w(c + 2, wq1);
+        if ((c & 3) == 0) {
+#pragma unroll
+          for (int r = 0; r < R; ++r) { sraw[r][0] = snext[r][0]; sraw[r][1] = snext[r][1]; }
+          fetch_s(c + 4, snext);
+        }
+#pragma unroll
+        for (int r = 0; r < R; ++r) {  // regroup: .x/.y = 8 bytes of group 2c, .z/.w = 8 bytes of group 2c+1
+          const auto s0 = __builtin_amdgcn_permlane32_swap(w[r].x, w[r].z, false, false);
+          const auto s1 = __builtin_amdgcn_permlane32_swap(w[r].y, w[r].w, false, false);
+          w[r].x = s0[0]; w[r].z = s0[1];
+          w[r].y = s1[0]; w[r].w = s1[1];
+        }
+        const unsigned xoff = (unsigned)((c - ch * steps_per_chunk) * 256 * XB);
+        const int sidx = (int)(c & 3) * 2;
+#pragma unroll
+        for (int h = 0; h < 2; ++h) {
+          typename Acc<ACT>::type acc[R][MT];
+#pragma unroll
+          for (int r = 0; r < R; ++r)
+#pragma unroll
+            for (int mt = 0; mt < MT; ++mt) acc[r][mt] = typename Acc<ACT>::type{0, 0, 0, 0};
+#pragma unroll
+          for (int j = 0; j < NJ; ++j) {
+            u32x4 xa[MT];
+#pragma unroll
+            for (int mt = 0; mt < MT; ++mt) xa[mt] = *(const lds_u32x4*)(xaddr[mt] + xoff + (h * 128 + j * KM) * XB);
+            u32x4 wb[R];  // decoded operand of every row sub-tile first, then the MFMAs: independent chains
+#pragma unroll
+            for (int r = 0; r < R; ++r) {
+              const unsigned lo = h == 0 ? w[r].x : w[r].z, hi = h == 0 ? w[r].y : w[r].w;
+              if (ACT == BP_BF16) {
+                const unsigned src = j < 2 ? lo : hi;
+                const u32x2 e0 = *(const lds_u32x2*)(lut_addr(src, lane_off, 2 * (j & 1)));
+                const u32x2 e1 = *(const lds_u32x2*)(lut_addr(src, lane_off, 2 * (j & 1) + 1));
+                wb[r] = u32x4{e0.x, e0.y, e1.x, e1.y};
+              } else {
+                const unsigned src = j == 0 ? lo : hi;
+                wb[r].x = *(const lds_u32*)(lut_addr(src, lane_off, 0));
+                wb[r].y = *(const lds_u32*)(lut_addr(src, lane_off, 1));
+                wb[r].z = *(const lds_u32*)(lut_addr(src, lane_off, 2));
+                wb[r].w = *(const lds_u32*)(lut_addr(src, lane_off, 3));
+              }
+            }
+#pragma unroll
+            for (int r = 0; r < R; ++r)
+#pragma unroll
+              for (int mt = 0; mt < MT; ++mt) {
+                if (ACT == BP_BF16)
+                  acc[r][mt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, xa[mt]),
+                                                                       __builtin_bit_cast(bf16x8, wb[r]), acc[r][mt], 0, 0, 0);
+                else
+                  acc[r][mt] = __builtin_amdgcn_mfma_i32_16x16x64_i8(__builtin_bit_cast(i32x4, xa[mt]),
+                                                                     __builtin_bit_cast(i32x4, wb[r]), acc[r][mt], 0, 0, 0);
+              }
+          }
+#pragma unroll
+          for (int r = 0; r < R; ++r) {
+            float s = 0.f;  // scale of group 2c + h: entry sidx + h of the 8 held (sidx is wave-uniform)
+#pragma unroll
+            for (int i = 0; i < 4; ++i)
+              if (sidx == 2 * i) s = scale_at<SDT>(sraw[r], 2 * i + h);
+#pragma unroll
+            for (int mt = 0; mt < MT; ++mt)
+#pragma unroll
+              for (int q = 0; q < 4; ++q) total[r][mt][q] += (float)acc[r][mt][q] * s;
+          }
+        }
+      }
+    }
+  }
+  // ---- epilogue: lane holds tokens 4b + q (q = 0..3) of each token tile, output row n0 + 16r + r16
+#pragma unroll
+  for (int mt = 0; mt < MT; ++mt) {
+#pragma unroll
+    for (int q = 0; q < 4; ++q) {
+      const int t = 16 * mt + 4 * b + q;
+      if (t < ntok) {
+        const int64_t tok = tok0 + t;
+        const float xs = ACT == BP_I8 ? a.x_scale[tok] : 1.0f;
+#pragma unroll
+        for (int r = 0; r < R; ++r) {
+          if (rows_valid[r]) {
+            float* o = a.out + tok * a.N + n0 + 16 * r + r16;
+            *o += total[r][mt][q] * xs;
+          }
+        }
+      }
+    }
+  }
+}
+
+template <int ACT, int SDT, int R, int MT, int WAVES>
+int launch_tq2(const GemmArgs& a, hipStream_t s, const char* name) {
+  constexpr int XB = ACT == BP_BF16 ? 2 : 1;
+  const int64_t rows_per_wg = (int64_t)WAVES * 16 * R;
+  const dim3 grid((unsigned)((a.N + rows_per_wg - 1) / rows_per_wg), (unsigned)a.E,
+                  (unsigned)((a.max_rows + 16 * MT - 1) / (16 * MT)));
+  // chunk length: as much of K as the tile budget holds for the widest token tile, in whole steps
+  const int64_t tokens = a.max_rows < 16 * MT ? a.max_rows : 16 * MT;
+  int64_t kc = (X_TILE_BYTES / tokens - 16) / XB / 256 * 256;
+  if (kc > a.K) kc = a.K;
+  if (kc < 256) return fail(BP_ERR_UNSUPPORTED, "activation tile does not fit");
+  const size_t lds = X_BASE + (size_t)tokens * (kc * XB + 16);
+  static bool attr = false;
+  if (!attr) {
+    if (hipFuncSetAttribute((const void*)k_mfma_tq2<ACT, SDT, R, MT, WAVES>, hipFuncAttributeMaxDynamicSharedMemorySize,
+                            X_BASE + X_TILE_BYTES) != hipSuccess)
+      return fail(BP_ERR_LAUNCH, "cannot raise the dynamic LDS limit");
+    attr = true;
+  }
+  note_kernel(name);
+  hipLaunchKernelGGL((k_mfma_tq2<ACT, SDT, R, MT, WAVES>), grid, dim3(WAVES * 64), lds, s, a, (int)kc);
+  return check_launch(name);
+}
+
+template <int ACT, int R, int MT, int WAVES>
+int launch_tq2_sd(const GemmArgs& a, hipStream_t s, const char* name) {
+  if (a.scale_dtype == BP_F16) return launch_tq2<ACT, BP_F16, R, MT, WAVES>(a, s, name);
+  if (a.scale_dtype == BP_BF16) return launch_tq2<ACT, BP_BF16, R, MT, WAVES>(a, s, name);
+  return launch_tq2<ACT, BP_F32, R, MT, WAVES>(a, s, name);
+}
+
+}  // namespace
+
+bool mfma_supports(const GemmArgs& a) {
+  if (a.group != 128 || a.fmt != BP_TQ2) return false;
+  if (a.x_dtype != BP_BF16 && a.x_dtype != BP_I8) return false;
+  if (a.K % 1024 != 0 || a.N % 16 != 0) return false;
+  if (((uintptr_t)a.x & 15) != 0) return false;
+  for (int t = 0; t < a.n_terms; ++t) {
+    if (((uintptr_t)a.packed[t] & 15) != 0) return false;
+    if (((uintptr_t)a.w_scale[t] & 15) != 0) return false;
+  }
+  if ((a.max_rows + 15) / 16 > 65535) return false;
+  return true;
+}
+
+int launch_mfma(const GemmArgs& a, hipStream_t s) {
+  const bool bf = a.x_dtype == BP_BF16;
+  // rows per wave: keep enough workgroups in flight for small problems
+  const int64_t work = a.E * (a.N / 16);
+  int R = work >= 4096 ? 2 : 1;
+  int MT = a.max_rows > 32 ? 4 : (a.max_rows > 16 ? 2 : 1);
+  int waves = 8;
+  if (const char* t = getenv("BP_TUNE_R")) { const int v = atoi(t); if (v == 1 || v == 2 || v == 4) R = v; }
+  if (const char* t = getenv("BP_TUNE_WAVES")) { const int v = atoi(t); if (v == 8 || v == 16) waves = v; }
+  if (const char* t = getenv("BP_TUNE_MT")) { const int v = atoi(t); if (v == 1 || v == 2 || v == 4) MT = v; }
+  if (MT == 4 && R == 4) R = 2;
+#define BP_CASE(ACTV, RV, MTV, WV, NAME) \
+  if (R == RV && MT == MTV && waves == WV) return launch_tq2_sd<ACTV, RV, MTV, WV>(a, s, NAME "_r" #RV "_m" #MTV "_w" #WV);
+#define BP_ALL(ACTV, NAME)                                                                       \
+  BP_CASE(ACTV, 1, 1, 8, NAME) BP_CASE(ACTV, 2, 1, 8, NAME) BP_CASE(ACTV, 4, 1, 8, NAME)           \
+  BP_CASE(ACTV, 1, 2, 8, NAME) BP_CASE(ACTV, 2, 2, 8, NAME) BP_CASE(ACTV, 4, 2, 8, NAME)           \
+  BP_CASE(ACTV, 1, 4, 8, NAME) BP_CASE(ACTV, 2, 4, 8, NAME)                                        \
+  BP_CASE(ACTV, 1, 1, 16, NAME) BP_CASE(ACTV, 2, 1, 16, NAME) BP_CASE(ACTV, 4, 1, 16, NAME)        \
+  BP_CASE(ACTV, 1, 2, 16, NAME) BP_CASE(ACTV, 2, 2, 16, NAME)                                      \
+  BP_CASE(ACTV, 1, 4, 16, NAME) BP_CASE(ACTV, 2, 4, 16, NAME)
+  if (bf) { BP_ALL(BP_BF16, "mfma_tq2_bf16") } else { BP_ALL(BP_I8, "mfma_tq2_i8") }
+#undef BP_ALL
+#undef BP_CASE
+  return fail(BP_ERR_UNSUPPORTED, "no tuned kernel variant for this tiling");
+}
+
+}  // namespace bp
