@@ -323,18 +323,337 @@ int launch_tq2_sd(const GemmArgs& a, hipStream_t s, const char* name) {
   return launch_tq2<ACT, BP_F32, R, MT, WAVES>(a, s, name);
 }
 
+
+// ------------------------------------------------------------------------------------------------
+// TQ1 (5 trits per byte), bf16 activations. K % 128 == 0, K >= 1024, N % 16 == 0.
+//
+// 640 trits = 128 bytes = 5 scale groups realign byte and group boundaries, so the unit of work is a
+// 128-byte chunk of every row. A byte is atomic: it fills one MFMA k-block with its 5 trits and 3
+// zeros, and the matching activation operand is a 16-byte "slot" holding the 5 activations of that
+// byte and 3 zeros; the activation tile in LDS is laid out slot by slot, so operand reads are aligned.
+// Group g of a chunk touches bytes FB[g] .. FB[g] + NB[g] - 1; k-block b of MFMA m takes byte
+// FB[g] + 7 b + m. A byte shared by two groups is presented to both, with the digits of the other
+// group zeroed (first byte: digits < DF[g]; last byte: digits >= DL[g]); slots past the group's last
+// byte get zero weights.
+//
+// Table entry of byte v: 8 bytes, byte i = high byte of bf16(trit_i / 2) (0x3f, 0xbf or 0), bytes 5..7
+// zero. +-0.5 has a zero low byte, so a v_perm_b32 per operand dword expands the entry to bf16; the
+// factor 2 is folded into the group scale (exact). Zeroing digits is a matter of the perm selector.
+struct __attribute__((packed, aligned(2))) Packed16 { u32x4 v; };
+struct __attribute__((packed, aligned(1))) Packed8 { u32x2 v; };
+
+constexpr unsigned tq1_sel(int dword, int keep_from, int keep_to) {  // selector of operand dword 0..2
+  // operand dword d holds digits 2d (low half) and 2d+1 (high half); a kept digit i reads entry byte i
+  // (bytes 0..3 from the entry's low dword = perm source 1, byte 4 from the high dword = source 0)
+  unsigned sel = 0x0c0c0c0cu;
+  const int lo = 2 * dword, hi = 2 * dword + 1;
+  if (lo < 5 && lo >= keep_from && lo < keep_to) sel = (sel & 0xffff00ffu) | ((unsigned)(lo < 4 ? lo : 4) << 8);
+  if (hi < 5 && hi >= keep_from && hi < keep_to) sel = (sel & 0x00ffffffu) | ((unsigned)(hi < 4 ? hi : 4) << 24);
+  return sel;
+}
+
+template <int SDT, int R, int MT, int WAVES>
+__global__ __launch_bounds__(WAVES * 64) void k_mfma_tq1(GemmArgs a, int CPT /* chunks per activation tile */) {
+  constexpr int THREADS = WAVES * 64;
+  constexpr int XU = (X_TILE_BYTES / 16 + THREADS - 1) / THREADS;  // activation slots staged per thread
+  constexpr int FB[5] = {0, 25, 51, 76, 102};
+  constexpr int DF[5] = {0, 3, 1, 4, 2};
+  constexpr int DL[5] = {3, 1, 4, 2, 5};
+  constexpr int MLAST[5] = {4, 5, 4, 5, 4};  // NB[g] - 1 - 21 with NB = {26, 27, 26, 27, 26}
+
+  // ---- table: entry of byte v, copy c (16 copies) at v * 128 + c * 8
+  if (threadIdx.x < 256) {
+    const unsigned v = threadIdx.x;
+    unsigned hb[5];
+#pragma unroll
+    for (int i = 0; i < 5; ++i) { const int t = tq1_trit(v, i); hb[i] = t > 0 ? 0x3fu : t < 0 ? 0xbfu : 0u; }
+    const u32x2 e = {hb[0] | (hb[1] << 8) | (hb[2] << 16) | (hb[3] << 24), hb[4]};
+    for (int c = 0; c < 16; ++c) *(lds_u32x2*)(v * LUT_STRIDE + c * 8) = e;
+  }
+
+  const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+  const int r16 = lane & 15, b = lane >> 4;
+  const int64_t e = blockIdx.y;
+  const int64_t o0 = clamp_i64(a.offsets[e], 0, a.T), o1 = clamp_i64(a.offsets[e + 1], 0, a.T);
+  const int64_t tok0 = o0 + (int64_t)blockIdx.z * (16 * MT);
+  if (tok0 >= o1) return;  // uniform for the workgroup
+  const int ntok = (int)(o1 - tok0 < 16 * MT ? o1 - tok0 : 16 * MT);
+  int64_t n0 = ((int64_t)blockIdx.x * WAVES + wave) * (16 * R);
+  const bool wave_live = n0 < a.N;
+  if (!wave_live) n0 = 0;
+  const unsigned lane_off = (unsigned)((lane & 15) * 8);
+  const bool is_b0 = b == 0, is_b3 = b == 3;
+
+  bool rows_valid[R];
+  int64_t row_off[R];  // byte offset of row sub-tile r from sub-tile 0, in the packed tensor
+  int64_t srow_off[R];
+#pragma unroll
+  for (int r = 0; r < R; ++r) {
+    rows_valid[r] = wave_live && n0 + 16 * r < a.N;
+    row_off[r] = rows_valid[r] ? 16 * r * a.Kp : 0;
+    srow_off[r] = rows_valid[r] ? 16 * r * a.G * 2 : 0;
+  }
+
+  // ---- activation tile, slot layout: slot s of token t at X_BASE + t * pitch + s * 16
+  const int slots = CPT * 128;
+  const int pitch = slots * 16 + 16;
+  const int units = ntok * slots;
+  unsigned xaddr[MT];
+#pragma unroll
+  for (int mt = 0; mt < MT; ++mt) {
+    int t = 16 * mt + r16;
+    if (t >= ntok) t = ntok - 1;
+    xaddr[mt] = (unsigned)(X_BASE + t * pitch + 7 * 16 * b);
+  }
+  const uint16_t* xg = (const uint16_t*)a.x + tok0 * a.K;
+  u32x4 xstage[XU];
+  auto stage_load = [&](int64_t slot0) {  // global -> registers: slots slot0 .. slot0 + slots of every token
+#pragma unroll
+    for (int i = 0; i < XU; ++i) {
+      const int u = threadIdx.x + i * THREADS;
+      u32x4 v = {0u, 0u, 0u, 0u};
+      if (u < units) {
+        const int row = u / slots, sl = u - row * slots;
+        const int64_t k0 = 5 * (slot0 + sl);
+        const uint16_t* src = xg + (int64_t)row * a.K + k0;
+        if (k0 + 8 <= a.K) {
+          v = ((const Packed16*)src)->v;
+          v.z &= 0xffffu;
+          v.w = 0u;
+        } else if (k0 < a.K) {  // the last slots of a row: element by element, zeros past K
+          unsigned h[5];
+#pragma unroll
+          for (int j = 0; j < 5; ++j) h[j] = k0 + j < a.K ? src[j] : 0u;
+          v = u32x4{h[0] | (h[1] << 16), h[2] | (h[3] << 16), h[4], 0u};
+        }
+      }
+      xstage[i] = v;
+    }
+  };
+  auto stage_store = [&]() {
+#pragma unroll
+    for (int i = 0; i < XU; ++i) {
+      const int u = threadIdx.x + i * THREADS;
+      if (u < units) {
+        const int row = u / slots, sl = u - row * slots;
+        *(lds_u32x4*)(X_BASE + row * pitch + sl * 16) = xstage[i];
+      }
+    }
+  };
+
+  f32x4 total[R][MT];
+#pragma unroll
+  for (int r = 0; r < R; ++r)
+#pragma unroll
+    for (int mt = 0; mt < MT; ++mt) total[r][mt] = f32x4{0.f, 0.f, 0.f, 0.f};
+
+  const int64_t nchunks = (a.K + 639) / 640;  // 128-byte chunks per row (the last may be partial)
+  const int64_t tiles = (nchunks + CPT - 1) / CPT;
+
+  for (int term = 0; term < a.n_terms; ++term) {
+    const unsigned char* wrow = a.packed[term] + (e * a.N + n0 + r16) * a.Kp + 7 * b;
+    const unsigned char* wend = a.packed[term] + a.E * a.N * a.Kp - 8;  // last address an 8-byte load may start at
+    const unsigned char* srow = (const unsigned char*)a.w_scale[term] + (e * a.N + n0 + r16) * a.G * 2;
+    u32x2 wq[R][5];
+    u32x4 sq[R];
+    auto fetch = [&](int64_t c) {  // weights and scales of chunk c (clamped to the last chunk)
+      const int64_t cc = c < nchunks ? c : nchunks - 1;
+      int64_t gi = 5 * cc;
+      if (gi > a.G - 8) gi = a.G - 8;
+      const unsigned char* p0 = wrow + 128 * cc;
+      if (cc + 1 < nchunks) {  // interior chunk: a load may run 3 bytes into the next chunk of the same row
+#pragma unroll
+        for (int r = 0; r < R; ++r)
+#pragma unroll
+          for (int g = 0; g < 5; ++g) wq[r][g] = ((const Packed8*)(p0 + row_off[r] + FB[g]))->v;
+      } else {  // last chunk of the row: never read past the end of the tensor
+#pragma unroll
+        for (int r = 0; r < R; ++r)
+#pragma unroll
+          for (int g = 0; g < 5; ++g) {
+            const unsigned char* p = p0 + row_off[r] + FB[g];
+            const unsigned char* q = p < wend ? p : wend;
+            const u32x2 v = ((const Packed8*)q)->v;
+            const unsigned sh = (unsigned)(p - q) * 8u;
+            const unsigned long long wide = (((unsigned long long)v.y << 32) | v.x) >> (sh < 63u ? sh : 63u);
+            wq[r][g] = u32x2{(unsigned)wide, (unsigned)(wide >> 32)};
+          }
+      }
+#pragma unroll
+      for (int r = 0; r < R; ++r) sq[r] = ((const Packed16*)(srow + srow_off[r] + gi * 2))->v;
+    };
+    const bool restage = term == 0 || tiles > 1;
+    if (restage) stage_load(0);
+    fetch(0);
+    for (int64_t tl = 0; tl < tiles; ++tl) {
+      if (restage) {
+        __syncthreads();
+        stage_store();
+        __syncthreads();
+        if (tl + 1 < tiles) stage_load((tl + 1) * slots);
+      }
+      const int64_t c_end = (tl + 1) * CPT < nchunks ? (tl + 1) * CPT : nchunks;
+      for (int64_t c = tl * CPT; c < c_end; ++c) {
+        u32x2 w[R][5];
+        u32x4 sraw[R];
+#pragma unroll
+        for (int r = 0; r < R; ++r) {
+          sraw[r] = sq[r];
+#pragma unroll
+          for (int g = 0; g < 5; ++g) w[r][g] = wq[r][g];
+        }
+        fetch(c + 1);
+        const int64_t groups_left = a.G - 5 * c;
+        const int ng = groups_left < 5 ? (int)groups_left : 5;
+        int64_t gi = 5 * c;
+        if (gi > a.G - 8) gi = a.G - 8;
+        const int sshift = (int)(5 * c - gi);  // wave-uniform; 0 except in the last chunks of a row
+        const unsigned xoff = (unsigned)((c - tl * CPT) * 2048);
+#pragma unroll
+        for (int g = 0; g < 5; ++g) {
+          if (g < ng) {
+            f32x4 acc[R][MT];
+#pragma unroll
+            for (int r = 0; r < R; ++r)
+#pragma unroll
+              for (int mt = 0; mt < MT; ++mt) acc[r][mt] = f32x4{0.f, 0.f, 0.f, 0.f};
+            // two-stage pipeline over the 7 MFMA slots: the LDS reads of slot m+1 are issued before the
+            // MFMAs of slot m; the scheduling barriers keep the compiler from hoisting all 35 slots at once
+            u32x4 xa[2][MT];
+            u32x2 we[2][R];
+            auto issue = [&](int m, int buf) {
+#pragma unroll
+              for (int mt = 0; mt < MT; ++mt) xa[buf][mt] = *(const lds_u32x4*)(xaddr[mt] + xoff + 16 * (FB[g] + m));
+#pragma unroll
+              for (int r = 0; r < R; ++r) {
+                const unsigned src = m < 4 ? w[r][g].x : w[r][g].y;
+                we[buf][r] = *(const lds_u32x2*)((__builtin_amdgcn_ubfe(src, 8 * (m & 3), 8) << 7) | lane_off);
+              }
+            };
+            issue(0, 0);
+#pragma unroll
+            for (int m = 0; m < 7; ++m) {
+              const int cur = m & 1;
+              if (m + 1 < 7) issue(m + 1, cur ^ 1);
+              // perm selectors of this slot: digits of another group, or a slot past the group, read as zero
+              unsigned s0 = tq1_sel(0, 0, 5), s1 = tq1_sel(1, 0, 5), s2 = tq1_sel(2, 0, 5);
+              if (m == 0 && DF[g] > 0) {
+                s0 = is_b0 ? tq1_sel(0, DF[g], 5) : s0;
+                s1 = is_b0 ? tq1_sel(1, DF[g], 5) : s1;
+              }
+              if (m == MLAST[g] && DL[g] < 5) {
+                s0 = is_b3 ? tq1_sel(0, 0, DL[g]) : s0;
+                s1 = is_b3 ? tq1_sel(1, 0, DL[g]) : s1;
+                s2 = is_b3 ? tq1_sel(2, 0, DL[g]) : s2;
+              }
+              if (m > MLAST[g]) {
+                s0 = is_b3 ? 0x0c0c0c0cu : s0;
+                s1 = is_b3 ? 0x0c0c0c0cu : s1;
+                s2 = is_b3 ? 0x0c0c0c0cu : s2;
+              }
+#pragma unroll
+              for (int r = 0; r < R; ++r) {
+                const u32x2 en = we[cur][r];
+                const u32x4 d = {__builtin_amdgcn_perm(en.y, en.x, s0), __builtin_amdgcn_perm(en.y, en.x, s1),
+                                 __builtin_amdgcn_perm(en.y, en.x, s2), 0u};
+#pragma unroll
+                for (int mt = 0; mt < MT; ++mt)
+                  acc[r][mt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, xa[cur][mt]),
+                                                                       __builtin_bit_cast(bf16x8, d), acc[r][mt], 0, 0, 0);
+              }
+              __builtin_amdgcn_sched_barrier(0);
+            }
+#pragma unroll
+            for (int r = 0; r < R; ++r) {
+              unsigned half = 0;  // 16-bit scale of group 5c + g = entry sshift + g of the 8 loaded
+              if (sshift == 0) {
+                const unsigned v = sraw[r][g >> 1];
+                half = (g & 1) ? (v >> 16) : (v & 0xffffu);
+              } else {
+#pragma unroll
+                for (int i = 0; i < 8; ++i)
+                  if (sshift + g == i) { const unsigned v = sraw[r][i >> 1]; half = (i & 1) ? (v >> 16) : (v & 0xffffu); }
+              }
+              // weights were decoded as +-0.5: the factor 2 goes into the scale (exact)
+              const float sc = 2.0f * (SDT == BP_F16 ? f16_bits_to_f32((uint16_t)half) : __uint_as_float(half << 16));
+#pragma unroll
+              for (int mt = 0; mt < MT; ++mt)
+#pragma unroll
+                for (int q = 0; q < 4; ++q) total[r][mt][q] += acc[r][mt][q] * sc;
+            }
+          }
+        }
+      }
+    }
+  }
+#pragma unroll
+  for (int mt = 0; mt < MT; ++mt) {
+#pragma unroll
+    for (int q = 0; q < 4; ++q) {
+      const int t = 16 * mt + 4 * b + q;
+      if (t < ntok) {
+        const int64_t tok = tok0 + t;
+#pragma unroll
+        for (int r = 0; r < R; ++r) {
+          if (rows_valid[r]) {
+            float* o = a.out + tok * a.N + n0 + 16 * r + r16;
+            *o += total[r][mt][q];
+          }
+        }
+      }
+    }
+  }
+}
+
+template <int SDT, int R, int MT, int WAVES>
+int launch_tq1(const GemmArgs& a, hipStream_t s, const char* name) {
+  const int64_t rows_per_wg = (int64_t)WAVES * 16 * R;
+  const dim3 grid((unsigned)((a.N + rows_per_wg - 1) / rows_per_wg), (unsigned)a.E,
+                  (unsigned)((a.max_rows + 16 * MT - 1) / (16 * MT)));
+  const int64_t tokens = a.max_rows < 16 * MT ? a.max_rows : 16 * MT;
+  const int64_t nchunks = (a.K + 639) / 640;
+  int64_t cpt = (X_TILE_BYTES / tokens - 16) / 2048;  // 128 slots of 16 bytes per chunk and token
+  if (cpt > nchunks) cpt = nchunks;
+  if (cpt < 1) return fail(BP_ERR_UNSUPPORTED, "activation tile does not fit");
+  const size_t lds = X_BASE + (size_t)tokens * (cpt * 2048 + 16);
+  static bool attr = false;
+  if (!attr) {
+    if (hipFuncSetAttribute((const void*)k_mfma_tq1<SDT, R, MT, WAVES>, hipFuncAttributeMaxDynamicSharedMemorySize,
+                            X_BASE + X_TILE_BYTES) != hipSuccess)
+      return fail(BP_ERR_LAUNCH, "cannot raise the dynamic LDS limit");
+    attr = true;
+  }
+  note_kernel(name);
+  hipLaunchKernelGGL((k_mfma_tq1<SDT, R, MT, WAVES>), grid, dim3(WAVES * 64), lds, s, a, (int)cpt);
+  return check_launch(name);
+}
+
+template <int R, int MT, int WAVES>
+int launch_tq1_sd(const GemmArgs& a, hipStream_t s, const char* name) {
+  if (a.scale_dtype == BP_F16) return launch_tq1<BP_F16, R, MT, WAVES>(a, s, name);
+  return launch_tq1<BP_BF16, R, MT, WAVES>(a, s, name);
+}
+
 }  // namespace
 
 bool mfma_supports(const GemmArgs& a) {
-  if (a.group != 128 || a.fmt != BP_TQ2) return false;
-  if (a.x_dtype != BP_BF16 && a.x_dtype != BP_I8) return false;
-  if (a.K % 1024 != 0 || a.N % 16 != 0) return false;
+  if (a.group != 128 || a.N % 16 != 0) return false;
   if (((uintptr_t)a.x & 15) != 0) return false;
-  for (int t = 0; t < a.n_terms; ++t) {
-    if (((uintptr_t)a.packed[t] & 15) != 0) return false;
-    if (((uintptr_t)a.w_scale[t] & 15) != 0) return false;
-  }
   if ((a.max_rows + 15) / 16 > 65535) return false;
+  if (a.fmt == BP_TQ2) {
+    if (a.x_dtype != BP_BF16 && a.x_dtype != BP_I8) return false;
+    if (a.K % 1024 != 0) return false;
+    for (int t = 0; t < a.n_terms; ++t) {
+      if (((uintptr_t)a.packed[t] & 15) != 0) return false;
+      if (((uintptr_t)a.w_scale[t] & 15) != 0) return false;
+    }
+    return true;
+  }
+  // TQ1: bf16 activations, scales as stored (fp16 / bf16)
+  if (a.x_dtype != BP_BF16 || (a.scale_dtype != BP_F16 && a.scale_dtype != BP_BF16)) return false;
+  if (a.K % 128 != 0 || a.K < 1024) return false;
+  for (int t = 0; t < a.n_terms; ++t)
+    if (((uintptr_t)a.w_scale[t] & 1) != 0) return false;
   return true;
 }
 
@@ -349,6 +668,16 @@ int launch_mfma(const GemmArgs& a, hipStream_t s) {
   if (const char* t = getenv("BP_TUNE_WAVES")) { const int v = atoi(t); if (v == 8 || v == 16) waves = v; }
   if (const char* t = getenv("BP_TUNE_MT")) { const int v = atoi(t); if (v == 1 || v == 2 || v == 4) MT = v; }
   if (MT == 4 && R == 4) R = 2;
+  if (a.fmt == BP_TQ1) {
+    if (R == 4) R = 2;
+    MT = 1;  // a 16-token slot-layout tile is the most the LDS budget holds; more rows go to more workgroups
+#define BP_T1(RV, MTV, WV) \
+    if (R == RV && MT == MTV && waves == WV) return launch_tq1_sd<RV, MTV, WV>(a, s, "mfma_tq1_bf16_r" #RV "_m" #MTV "_w" #WV);
+    BP_T1(1, 1, 8) BP_T1(2, 1, 8) BP_T1(1, 2, 8) BP_T1(2, 2, 8)
+    BP_T1(1, 1, 16) BP_T1(2, 1, 16) BP_T1(1, 2, 16) BP_T1(2, 2, 16)
+#undef BP_T1
+    return fail(BP_ERR_UNSUPPORTED, "no tuned TQ1 kernel variant for this tiling");
+  }
 #define BP_CASE(ACTV, RV, MTV, WV, NAME) \
   if (R == RV && MT == MTV && waves == WV) return launch_tq2_sd<ACTV, RV, MTV, WV>(a, s, NAME "_r" #RV "_m" #MTV "_w" #WV);
 #define BP_ALL(ACTV, NAME)                                                                       \
