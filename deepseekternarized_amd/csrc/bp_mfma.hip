@@ -38,7 +38,7 @@ typedef __attribute__((address_space(3))) unsigned lds_u32;
 constexpr int LUT_STRIDE = 128;
 constexpr int LUT_BYTES = 256 * LUT_STRIDE;
 constexpr int X_BASE = LUT_BYTES;
-constexpr int X_TILE_BYTES = 48 * 1024;  // table + tile = 80 KiB: two workgroups per CU
+constexpr int X_TILE_BYTES = 48 * 1024;  // TQ1: table + tile = 80 KiB: two workgroups of 8 waves per CU
 
 __device__ __forceinline__ unsigned bf16_of_trit(int t) {
   return t == 0 ? 0u : t == 1 ? 0x3f80u : t == -1 ? 0xbf80u : 0x4000u;  // +2 (TQ2 code 3) -> 2.0
@@ -70,7 +70,7 @@ __device__ __forceinline__ float scale_at(const u32x4 (&raw)[2], int i) {  // i-
 // v_permlane32_swap pair then leaves every lane with 8 bytes of the first group and 8 bytes of the
 // second, so that all four k-blocks of an MFMA belong to one scale group.
 // After the swap block b holds trits tb(b) .. tb(b)+31 of each group, tb = {0, 64, 32, 96}.
-template <int ACT, int SDT, int R, int MT, int WAVES>
+template <int ACT, int SDT, int R, int MT, int WAVES, int XKB, int ABL = 0>
 __global__ __launch_bounds__(WAVES * 64, 4) void k_mfma_tq2(GemmArgs a, int KC) {
   constexpr int THREADS = WAVES * 64;
   constexpr int EB = ACT == BP_BF16 ? 8 : 4;   // bytes per table entry
@@ -78,7 +78,7 @@ __global__ __launch_bounds__(WAVES * 64, 4) void k_mfma_tq2(GemmArgs a, int KC) 
   constexpr int XB = ACT == BP_BF16 ? 2 : 1;   // bytes per activation element
   constexpr int KM = ACT == BP_BF16 ? 8 : 16;  // k per lane per MFMA
   constexpr int NJ = 32 / KM;                  // MFMAs per group
-  constexpr int XU = X_TILE_BYTES / 16 / THREADS;  // 16-byte units of the activation tile per thread
+  constexpr int XU = XKB * 1024 / 16 / THREADS;  // 16-byte units of the activation tile per thread
 
   // ---- build the table: thread v < 256 writes the entry of byte value v into every copy
   if (threadIdx.x < 256) {
@@ -167,7 +167,10 @@ __global__ __launch_bounds__(WAVES * 64, 4) void k_mfma_tq2(GemmArgs a, int KC) 
   for (int term = 0; term < a.n_terms; ++term) {
     const unsigned char* wbase = a.packed[term] + ((e * a.N + n0 + r16) * a.Kp + 16 * b);
     const unsigned char* sbase = (const unsigned char*)a.w_scale[term] + (e * a.N + n0 + r16) * a.G * (SDT == BP_F32 ? 4 : 2);
-    u32x4 wq0[R], wq1[R];           // weights of the next two steps
+    // Ring of PF steps of packed weights in flight per row sub-tile: with ~4 us of loaded HBM latency a CU
+    // needs > 100 KiB of requests outstanding to stream at full rate (16 waves x PF x R KiB here).
+    constexpr int PF = 4;
+    u32x4 ring[PF][R];
     u32x4 sraw[R][2], snext[R][2];  // 8 scales (4 steps) per row sub-tile, and the next 8
     auto fetch_w = [&](int64_t c, u32x4 (&dst)[R]) {
       const int64_t cc = c < steps ? c : steps - 1;  // past the end: re-read the last step, no branch
@@ -185,87 +188,90 @@ __global__ __launch_bounds__(WAVES * 64, 4) void k_mfma_tq2(GemmArgs a, int KC) 
     };
     const bool restage = term == 0 || chunks > 1;  // a tile that holds all of K is staged once for all terms
     if (restage) stage_load(0);
-    fetch_w(0, wq0);
-    fetch_w(1, wq1);
+#pragma unroll
+    for (int i = 0; i < PF; ++i) fetch_w(i, ring[i]);
     fetch_s(0, snext);
     for (int64_t ch = 0; ch < chunks; ++ch) {
       if (restage) {
         __syncthreads();  // every wave is done reading the previous tile (and, first time, the table is built)
         stage_store();
         __syncthreads();
+        if (ch + 1 < chunks) stage_load((ch + 1) * KC);
       }
-      if (ch + 1 < chunks) stage_load((ch + 1) * KC);
       const int64_t c_end = (ch + 1) * steps_per_chunk < steps ? (ch + 1) * steps_per_chunk : steps;
-      for (int64_t c = ch * steps_per_chunk; c < c_end; ++c) {
-        u32x4 w[R];
+      for (int64_t c4 = ch * steps_per_chunk; c4 < c_end; c4 += PF) {  // KC % 1024 == 0: whole blocks of 4 steps
 #pragma unroll
-        for (int r = 0; r < R; ++r) { w[r] = wq0[r]; wq0[r] = wq1[r]; }
-        fetch_w(c + 2, wq1);
-        if ((c & 3) == 0) {
+        for (int r = 0; r < R; ++r) { sraw[r][0] = snext[r][0]; sraw[r][1] = snext[r][1]; }
+        fetch_s(c4 + 4, snext);
 #pragma unroll
-          for (int r = 0; r < R; ++r) { sraw[r][0] = snext[r][0]; sraw[r][1] = snext[r][1]; }
-          fetch_s(c + 4, snext);
-        }
+        for (int i = 0; i < PF; ++i) {
+          const int64_t c = c4 + i;
+          u32x4 w[R];
 #pragma unroll
-        for (int r = 0; r < R; ++r) {  // regroup: .x/.y = 8 bytes of group 2c, .z/.w = 8 bytes of group 2c+1
-          const auto s0 = __builtin_amdgcn_permlane32_swap(w[r].x, w[r].z, false, false);
-          const auto s1 = __builtin_amdgcn_permlane32_swap(w[r].y, w[r].w, false, false);
-          w[r].x = s0[0]; w[r].z = s0[1];
-          w[r].y = s1[0]; w[r].w = s1[1];
-        }
-        const unsigned xoff = (unsigned)((c - ch * steps_per_chunk) * 256 * XB);
-        const int sidx = (int)(c & 3) * 2;
+          for (int r = 0; r < R; ++r) w[r] = ring[i][r];
+          fetch_w(c + PF, ring[i]);
 #pragma unroll
-        for (int h = 0; h < 2; ++h) {
-          typename Acc<ACT>::type acc[R][MT];
+          for (int r = 0; r < R; ++r) {  // regroup: .x/.y = 8 bytes of group 2c, .z/.w = 8 bytes of group 2c+1
+            const auto s0 = __builtin_amdgcn_permlane32_swap(w[r].x, w[r].z, false, false);
+            const auto s1 = __builtin_amdgcn_permlane32_swap(w[r].y, w[r].w, false, false);
+            w[r].x = s0[0]; w[r].z = s0[1];
+            w[r].y = s1[0]; w[r].w = s1[1];
+          }
+          const unsigned xoff = (unsigned)((c - ch * steps_per_chunk) * 256 * XB);
+          if (ABL == 1) {  // ablation (timing experiments only): memory traffic without decode and MFMA
 #pragma unroll
-          for (int r = 0; r < R; ++r)
+            for (int r = 0; r < R; ++r) total[r][0][0] += __uint_as_float((w[r].x ^ w[r].y ^ w[r].z ^ w[r].w) & 0x3fffffu);
+            continue;
+          }
 #pragma unroll
-            for (int mt = 0; mt < MT; ++mt) acc[r][mt] = typename Acc<ACT>::type{0, 0, 0, 0};
-#pragma unroll
-          for (int j = 0; j < NJ; ++j) {
-            u32x4 xa[MT];
-#pragma unroll
-            for (int mt = 0; mt < MT; ++mt) xa[mt] = *(const lds_u32x4*)(xaddr[mt] + xoff + (h * 128 + j * KM) * XB);
-            u32x4 wb[R];  // decoded operand of every row sub-tile first, then the MFMAs: independent chains
-#pragma unroll
-            for (int r = 0; r < R; ++r) {
-              const unsigned lo = h == 0 ? w[r].x : w[r].z, hi = h == 0 ? w[r].y : w[r].w;
-              if (ACT == BP_BF16) {
-                const unsigned src = j < 2 ? lo : hi;
-                const u32x2 e0 = *(const lds_u32x2*)(lut_addr(src, lane_off, 2 * (j & 1)));
-                const u32x2 e1 = *(const lds_u32x2*)(lut_addr(src, lane_off, 2 * (j & 1) + 1));
-                wb[r] = u32x4{e0.x, e0.y, e1.x, e1.y};
-              } else {
-                const unsigned src = j == 0 ? lo : hi;
-                wb[r].x = *(const lds_u32*)(lut_addr(src, lane_off, 0));
-                wb[r].y = *(const lds_u32*)(lut_addr(src, lane_off, 1));
-                wb[r].z = *(const lds_u32*)(lut_addr(src, lane_off, 2));
-                wb[r].w = *(const lds_u32*)(lut_addr(src, lane_off, 3));
-              }
-            }
+          for (int h = 0; h < 2; ++h) {
+            typename Acc<ACT>::type acc[R][MT];
 #pragma unroll
             for (int r = 0; r < R; ++r)
 #pragma unroll
-              for (int mt = 0; mt < MT; ++mt) {
-                if (ACT == BP_BF16)
-                  acc[r][mt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, xa[mt]),
-                                                                       __builtin_bit_cast(bf16x8, wb[r]), acc[r][mt], 0, 0, 0);
-                else
-                  acc[r][mt] = __builtin_amdgcn_mfma_i32_16x16x64_i8(__builtin_bit_cast(i32x4, xa[mt]),
-                                                                     __builtin_bit_cast(i32x4, wb[r]), acc[r][mt], 0, 0, 0);
+              for (int mt = 0; mt < MT; ++mt) acc[r][mt] = typename Acc<ACT>::type{0, 0, 0, 0};
+#pragma unroll
+            for (int j = 0; j < NJ; ++j) {
+              u32x4 xa[MT];
+#pragma unroll
+              for (int mt = 0; mt < MT; ++mt) xa[mt] = *(const lds_u32x4*)(xaddr[mt] + xoff + (h * 128 + j * KM) * XB);
+              u32x4 wb[R];  // decoded operand of every row sub-tile first, then the MFMAs: independent chains
+#pragma unroll
+              for (int r = 0; r < R; ++r) {
+                const unsigned lo = h == 0 ? w[r].x : w[r].z, hi = h == 0 ? w[r].y : w[r].w;
+                if (ACT == BP_BF16) {
+                  const unsigned src = j < 2 ? lo : hi;
+                  const u32x2 e0 = *(const lds_u32x2*)(lut_addr(src, lane_off, 2 * (j & 1)));
+                  const u32x2 e1 = *(const lds_u32x2*)(lut_addr(src, lane_off, 2 * (j & 1) + 1));
+                  wb[r] = u32x4{e0.x, e0.y, e1.x, e1.y};
+                } else {
+                  const unsigned src = j == 0 ? lo : hi;
+                  wb[r].x = *(const lds_u32*)(lut_addr(src, lane_off, 0));
+                  wb[r].y = *(const lds_u32*)(lut_addr(src, lane_off, 1));
+                  wb[r].z = *(const lds_u32*)(lut_addr(src, lane_off, 2));
+                  wb[r].w = *(const lds_u32*)(lut_addr(src, lane_off, 3));
+                }
               }
-          }
 #pragma unroll
-          for (int r = 0; r < R; ++r) {
-            float s = 0.f;  // scale of group 2c + h: entry sidx + h of the 8 held (sidx is wave-uniform)
+              for (int r = 0; r < R; ++r)
 #pragma unroll
-            for (int i = 0; i < 4; ++i)
-              if (sidx == 2 * i) s = scale_at<SDT>(sraw[r], 2 * i + h);
+                for (int mt = 0; mt < MT; ++mt) {
+                  if (ACT == BP_BF16)
+                    acc[r][mt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, xa[mt]),
+                                                                         __builtin_bit_cast(bf16x8, wb[r]), acc[r][mt], 0, 0, 0);
+                  else
+                    acc[r][mt] = __builtin_amdgcn_mfma_i32_16x16x64_i8(__builtin_bit_cast(i32x4, xa[mt]),
+                                                                       __builtin_bit_cast(i32x4, wb[r]), acc[r][mt], 0, 0, 0);
+                }
+            }
 #pragma unroll
-            for (int mt = 0; mt < MT; ++mt)
+            for (int r = 0; r < R; ++r) {
+              const float s = scale_at<SDT>(sraw[r], 2 * i + h);  // group 2c + h = entry 2i + h of the 8 held
 #pragma unroll
-              for (int q = 0; q < 4; ++q) total[r][mt][q] += (float)acc[r][mt][q] * s;
+              for (int mt = 0; mt < MT; ++mt)
+#pragma unroll
+                for (int q = 0; q < 4; ++q) total[r][mt][q] += (float)acc[r][mt][q] * s;
+            }
           }
         }
       }
@@ -292,37 +298,36 @@ __global__ __launch_bounds__(WAVES * 64, 4) void k_mfma_tq2(GemmArgs a, int KC) 
   }
 }
 
-template <int ACT, int SDT, int R, int MT, int WAVES>
+template <int ACT, int SDT, int R, int MT, int WAVES, int XKB, int ABL = 0>
 int launch_tq2(const GemmArgs& a, hipStream_t s, const char* name) {
   constexpr int XB = ACT == BP_BF16 ? 2 : 1;
   const int64_t rows_per_wg = (int64_t)WAVES * 16 * R;
   const dim3 grid((unsigned)((a.N + rows_per_wg - 1) / rows_per_wg), (unsigned)a.E,
                   (unsigned)((a.max_rows + 16 * MT - 1) / (16 * MT)));
-  // chunk length: as much of K as the tile budget holds for the widest token tile, in whole steps
+  // chunk length: as much of K as the tile budget holds for the widest token tile, in blocks of 4 steps
   const int64_t tokens = a.max_rows < 16 * MT ? a.max_rows : 16 * MT;
-  int64_t kc = (X_TILE_BYTES / tokens - 16) / XB / 256 * 256;
+  int64_t kc = (XKB * 1024 / tokens - 16) / XB / 1024 * 1024;
   if (kc > a.K) kc = a.K;
-  if (kc < 256) return fail(BP_ERR_UNSUPPORTED, "activation tile does not fit");
+  if (kc < 1024) return fail(BP_ERR_UNSUPPORTED, "activation tile does not fit");
   const size_t lds = X_BASE + (size_t)tokens * (kc * XB + 16);
   static bool attr = false;
   if (!attr) {
-    if (hipFuncSetAttribute((const void*)k_mfma_tq2<ACT, SDT, R, MT, WAVES>, hipFuncAttributeMaxDynamicSharedMemorySize,
-                            X_BASE + X_TILE_BYTES) != hipSuccess)
+    if (hipFuncSetAttribute((const void*)k_mfma_tq2<ACT, SDT, R, MT, WAVES, XKB, ABL>, hipFuncAttributeMaxDynamicSharedMemorySize,
+                            X_BASE + XKB * 1024) != hipSuccess)
       return fail(BP_ERR_LAUNCH, "cannot raise the dynamic LDS limit");
     attr = true;
   }
   note_kernel(name);
-  hipLaunchKernelGGL((k_mfma_tq2<ACT, SDT, R, MT, WAVES>), grid, dim3(WAVES * 64), lds, s, a, (int)kc);
+  hipLaunchKernelGGL((k_mfma_tq2<ACT, SDT, R, MT, WAVES, XKB, ABL>), grid, dim3(WAVES * 64), lds, s, a, (int)kc);
   return check_launch(name);
 }
 
-template <int ACT, int R, int MT, int WAVES>
+template <int ACT, int R, int MT, int WAVES, int XKB>
 int launch_tq2_sd(const GemmArgs& a, hipStream_t s, const char* name) {
-  if (a.scale_dtype == BP_F16) return launch_tq2<ACT, BP_F16, R, MT, WAVES>(a, s, name);
-  if (a.scale_dtype == BP_BF16) return launch_tq2<ACT, BP_BF16, R, MT, WAVES>(a, s, name);
-  return launch_tq2<ACT, BP_F32, R, MT, WAVES>(a, s, name);
+  if (a.scale_dtype == BP_F16) return launch_tq2<ACT, BP_F16, R, MT, WAVES, XKB>(a, s, name);
+  if (a.scale_dtype == BP_BF16) return launch_tq2<ACT, BP_BF16, R, MT, WAVES, XKB>(a, s, name);
+  return launch_tq2<ACT, BP_F32, R, MT, WAVES, XKB>(a, s, name);
 }
-
 
 // ------------------------------------------------------------------------------------------------
 // TQ1 (5 trits per byte), bf16 activations. K % 128 == 0, K >= 1024, N % 16 == 0.
@@ -659,34 +664,35 @@ bool mfma_supports(const GemmArgs& a) {
 
 int launch_mfma(const GemmArgs& a, hipStream_t s) {
   const bool bf = a.x_dtype == BP_BF16;
-  // rows per wave: keep enough workgroups in flight for small problems
+  // rows per wave and waves per workgroup: keep enough workgroups in flight for small problems
   const int64_t work = a.E * (a.N / 16);
-  int R = work >= 4096 ? 2 : 1;
-  int MT = a.max_rows > 32 ? 4 : (a.max_rows > 16 ? 2 : 1);
-  int waves = 8;
-  if (const char* t = getenv("BP_TUNE_R")) { const int v = atoi(t); if (v == 1 || v == 2 || v == 4) R = v; }
+  int R = work >= 8192 ? 2 : 1;
+  int MT = a.max_rows > 16 ? 2 : 1;
+  int waves = work >= 2048 ? 16 : 8;
+  if (const char* t = getenv("BP_TUNE_R")) { const int v = atoi(t); if (v == 1 || v == 2) R = v; }
   if (const char* t = getenv("BP_TUNE_WAVES")) { const int v = atoi(t); if (v == 8 || v == 16) waves = v; }
-  if (const char* t = getenv("BP_TUNE_MT")) { const int v = atoi(t); if (v == 1 || v == 2 || v == 4) MT = v; }
-  if (MT == 4 && R == 4) R = 2;
+  if (const char* t = getenv("BP_TUNE_MT")) { const int v = atoi(t); if (v == 1 || v == 2) MT = v; }
   if (a.fmt == BP_TQ1) {
-    if (R == 4) R = 2;
     MT = 1;  // a 16-token slot-layout tile is the most the LDS budget holds; more rows go to more workgroups
-#define BP_T1(RV, MTV, WV) \
-    if (R == RV && MT == MTV && waves == WV) return launch_tq1_sd<RV, MTV, WV>(a, s, "mfma_tq1_bf16_r" #RV "_m" #MTV "_w" #WV);
-    BP_T1(1, 1, 8) BP_T1(2, 1, 8) BP_T1(1, 2, 8) BP_T1(2, 2, 8)
-    BP_T1(1, 1, 16) BP_T1(2, 1, 16) BP_T1(1, 2, 16) BP_T1(2, 2, 16)
+#define BP_T1(RV, WV) \
+    if (R == RV && waves == WV) return launch_tq1_sd<RV, 1, WV>(a, s, "mfma_tq1_bf16_r" #RV "_m1_w" #WV);
+    BP_T1(1, 8) BP_T1(2, 8) BP_T1(1, 16) BP_T1(2, 16)
 #undef BP_T1
     return fail(BP_ERR_UNSUPPORTED, "no tuned TQ1 kernel variant for this tiling");
   }
-#define BP_CASE(ACTV, RV, MTV, WV, NAME) \
-  if (R == RV && MT == MTV && waves == WV) return launch_tq2_sd<ACTV, RV, MTV, WV>(a, s, NAME "_r" #RV "_m" #MTV "_w" #WV);
-#define BP_ALL(ACTV, NAME)                                                                       \
-  BP_CASE(ACTV, 1, 1, 8, NAME) BP_CASE(ACTV, 2, 1, 8, NAME) BP_CASE(ACTV, 4, 1, 8, NAME)           \
-  BP_CASE(ACTV, 1, 2, 8, NAME) BP_CASE(ACTV, 2, 2, 8, NAME) BP_CASE(ACTV, 4, 2, 8, NAME)           \
-  BP_CASE(ACTV, 1, 4, 8, NAME) BP_CASE(ACTV, 2, 4, 8, NAME)                                        \
-  BP_CASE(ACTV, 1, 1, 16, NAME) BP_CASE(ACTV, 2, 1, 16, NAME) BP_CASE(ACTV, 4, 1, 16, NAME)        \
-  BP_CASE(ACTV, 1, 2, 16, NAME) BP_CASE(ACTV, 2, 2, 16, NAME)                                      \
-  BP_CASE(ACTV, 1, 4, 16, NAME) BP_CASE(ACTV, 2, 4, 16, NAME)
+  if (const char* t = getenv("BP_TUNE_ABL")) {
+    if (atoi(t) == 1 && bf && a.scale_dtype == BP_F16 && MT == 1) {
+      if (R == 1) return launch_tq2<BP_BF16, BP_F16, 1, 1, 16, 48, 1>(a, s, "abl_r1_w16");
+      return launch_tq2<BP_BF16, BP_F16, 2, 1, 16, 48, 1>(a, s, "abl_r2_w16");
+    }
+  }
+  if (MT == 2) waves = 16;  // the 32-token tile needs the large LDS budget of a 16-wave workgroup
+#define BP_CASE(ACTV, RV, MTV, WV, XK, NAME) \
+  if (R == RV && MT == MTV && waves == WV) return launch_tq2_sd<ACTV, RV, MTV, WV, XK>(a, s, NAME "_r" #RV "_m" #MTV "_w" #WV);
+#define BP_ALL(ACTV, NAME)                                                        \
+  BP_CASE(ACTV, 1, 1, 8, 48, NAME) BP_CASE(ACTV, 2, 1, 8, 48, NAME)                \
+  BP_CASE(ACTV, 1, 1, 16, 48, NAME) BP_CASE(ACTV, 2, 1, 16, 48, NAME)              \
+  BP_CASE(ACTV, 1, 2, 16, 112, NAME) BP_CASE(ACTV, 2, 2, 16, 112, NAME)
   if (bf) { BP_ALL(BP_BF16, "mfma_tq2_bf16") } else { BP_ALL(BP_I8, "mfma_tq2_i8") }
 #undef BP_ALL
 #undef BP_CASE
