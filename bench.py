@@ -151,6 +151,9 @@ def main() -> int:
     ap.add_argument("--workload", default="cfg1a_tq1_gemv", choices=sorted(WORKLOADS))
     ap.add_argument("--no-extras", action="store_true", help="skip the secondary measurements")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline")
+    ap.add_argument("--calibrate-copy", action="store_true",
+                    help="instead of the workload, run a plain 1 GiB device-to-device copy `steps` times "
+                         "(the known-size kernel that FETCH_SIZE / WRITE_SIZE counter readings are scaled by)")
     a = ap.parse_args()
     if a.gpus != 1:
         print("bench.py measures one GPU: this build has no multi-GPU path (run with --gpus 1)", file=sys.stderr)
@@ -163,6 +166,14 @@ def main() -> int:
     if not torch.cuda.is_available() or bp.ext() is None:
         print("bench.py needs a HIP device and the built libbp_ternary_hip.so", file=sys.stderr)
         return 1
+    if a.calibrate_copy:
+        src = torch.empty(1 << 30, dtype=torch.uint8, device="cuda").random_(0, 255)
+        dst = torch.empty_like(src)
+        for _ in range(a.steps):
+            dst.copy_(src)
+        torch.cuda.synchronize()
+        print(json.dumps({"calibration": "device copy", "bytes_read": 1 << 30, "bytes_written": 1 << 30, "steps": a.steps}))
+        return 0
     fmt, N, K, M, act, terms, L = WORKLOADS[a.workload]
     launch, wbytes = uniform_launch(bp, torch, fmt, N, K, M, act, terms, L)
     wall, kern, kname = launch.time(a.steps, a.warmup)

@@ -666,7 +666,7 @@ int launch_mfma(const GemmArgs& a, hipStream_t s) {
   const bool bf = a.x_dtype == BP_BF16;
   // rows per wave and waves per workgroup: keep enough workgroups in flight for small problems
   const int64_t work = a.E * (a.N / 16);
-  int R = work >= 8192 ? 2 : 1;
+  int R = 1;  // two row sub-tiles per wave spill registers at 4 waves per SIMD; see BP_TUNE_R
   int MT = a.max_rows > 16 ? 2 : 1;
   int waves = work >= 2048 ? 16 : 8;
   if (const char* t = getenv("BP_TUNE_R")) { const int v = atoi(t); if (v == 1 || v == 2) R = v; }
