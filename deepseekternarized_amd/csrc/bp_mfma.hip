@@ -346,6 +346,8 @@ int launch_tq2_sd(const GemmArgs& a, hipStream_t s, const char* name) {
 // factor 2 is folded into the group scale (exact). Zeroing digits is a matter of the perm selector.
 struct __attribute__((packed, aligned(2))) Packed16 { u32x4 v; };
 struct __attribute__((packed, aligned(1))) Packed8 { u32x2 v; };
+constexpr int T1_STRIDE = 256;
+constexpr int T1_X_BASE = 256 * T1_STRIDE;  // activation tile starts after the 64 KiB table
 
 constexpr unsigned tq1_sel(int dword, int keep_from, int keep_to) {  // selector of operand dword 0..2
   // operand dword d holds digits 2d (low half) and 2d+1 (high half); a kept digit i reads entry byte i
@@ -357,7 +359,7 @@ constexpr unsigned tq1_sel(int dword, int keep_from, int keep_to) {  // selector
   return sel;
 }
 
-template <int SDT, int R, int MT, int WAVES>
+template <int SDT, int R, int MT, int WAVES, int ABL = 0>
 __global__ __launch_bounds__(WAVES * 64) void k_mfma_tq1(GemmArgs a, int CPT /* chunks per activation tile */) {
   constexpr int THREADS = WAVES * 64;
   constexpr int XU = (X_TILE_BYTES / 16 + THREADS - 1) / THREADS;  // activation slots staged per thread
@@ -366,14 +368,15 @@ __global__ __launch_bounds__(WAVES * 64) void k_mfma_tq1(GemmArgs a, int CPT /* 
   constexpr int DL[5] = {3, 1, 4, 2, 5};
   constexpr int MLAST[5] = {4, 5, 4, 5, 4};  // NB[g] - 1 - 21 with NB = {26, 27, 26, 27, 26}
 
-  // ---- table: entry of byte v, copy c (16 copies) at v * 128 + c * 8
+  // ---- table: entry of byte v, copy c (16 copies) at v * 256 + c * 8 (the 256-byte stride makes the
+  // address of an entry a single byte permute of the packed word)
   if (threadIdx.x < 256) {
     const unsigned v = threadIdx.x;
     unsigned hb[5];
 #pragma unroll
     for (int i = 0; i < 5; ++i) { const int t = tq1_trit(v, i); hb[i] = t > 0 ? 0x3fu : t < 0 ? 0xbfu : 0u; }
     const u32x2 e = {hb[0] | (hb[1] << 8) | (hb[2] << 16) | (hb[3] << 24), hb[4]};
-    for (int c = 0; c < 16; ++c) *(lds_u32x2*)(v * LUT_STRIDE + c * 8) = e;
+    for (int c = 0; c < 16; ++c) *(lds_u32x2*)(v * T1_STRIDE + c * 8) = e;
   }
 
   const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
@@ -399,7 +402,7 @@ __global__ __launch_bounds__(WAVES * 64) void k_mfma_tq1(GemmArgs a, int CPT /* 
     srow_off[r] = rows_valid[r] ? 16 * r * a.G * 2 : 0;
   }
 
-  // ---- activation tile, slot layout: slot s of token t at X_BASE + t * pitch + s * 16
+  // ---- activation tile, slot layout: slot s of token t at T1_X_BASE + t * pitch + s * 16
   const int slots = CPT * 128;
   const int pitch = slots * 16 + 16;
   const int units = ntok * slots;
@@ -408,8 +411,12 @@ __global__ __launch_bounds__(WAVES * 64) void k_mfma_tq1(GemmArgs a, int CPT /* 
   for (int mt = 0; mt < MT; ++mt) {
     int t = 16 * mt + r16;
     if (t >= ntok) t = ntok - 1;
-    xaddr[mt] = (unsigned)(X_BASE + t * pitch + 7 * 16 * b);
+    xaddr[mt] = (unsigned)(T1_X_BASE + t * pitch + 7 * 16 * b);
   }
+  // The 16-byte pad after every row and the 32 bytes after the last row are read (by slots past a group's
+  // last byte, against zero weights) but never staged: clear them once so they cannot hold NaN patterns.
+  if ((int)threadIdx.x < ntok) *(lds_u32x4*)(T1_X_BASE + threadIdx.x * pitch + slots * 16) = u32x4{0u, 0u, 0u, 0u};
+  if (threadIdx.x < 2) *(lds_u32x4*)(T1_X_BASE + ntok * pitch + threadIdx.x * 16) = u32x4{0u, 0u, 0u, 0u};
   const uint16_t* xg = (const uint16_t*)a.x + tok0 * a.K;
   u32x4 xstage[XU];
   auto stage_load = [&](int64_t slot0) {  // global -> registers: slots slot0 .. slot0 + slots of every token
@@ -441,7 +448,7 @@ __global__ __launch_bounds__(WAVES * 64) void k_mfma_tq1(GemmArgs a, int CPT /* 
       const int u = threadIdx.x + i * THREADS;
       if (u < units) {
         const int row = u / slots, sl = u - row * slots;
-        *(lds_u32x4*)(X_BASE + row * pitch + sl * 16) = xstage[i];
+        *(lds_u32x4*)(T1_X_BASE + row * pitch + sl * 16) = xstage[i];
       }
     }
   };
@@ -459,9 +466,11 @@ __global__ __launch_bounds__(WAVES * 64) void k_mfma_tq1(GemmArgs a, int CPT /* 
     const unsigned char* wrow = a.packed[term] + (e * a.N + n0 + r16) * a.Kp + 7 * b;
     const unsigned char* wend = a.packed[term] + a.E * a.N * a.Kp - 8;  // last address an 8-byte load may start at
     const unsigned char* srow = (const unsigned char*)a.w_scale[term] + (e * a.N + n0 + r16) * a.G * 2;
-    u32x2 wq[R][5];
-    u32x4 sq[R];
-    auto fetch = [&](int64_t c) {  // weights and scales of chunk c (clamped to the last chunk)
+    // queue of PFQ chunks of packed bytes and scales in flight behind the chunk being computed
+    constexpr int PFQ = 2;
+    u32x2 wq[PFQ][R][5];
+    u32x4 sq[PFQ][R];
+    auto fetch = [&](int64_t c, u32x2 (&wd)[R][5], u32x4 (&sd)[R]) {  // chunk c (clamped to the last chunk)
       const int64_t cc = c < nchunks ? c : nchunks - 1;
       int64_t gi = 5 * cc;
       if (gi > a.G - 8) gi = a.G - 8;
@@ -470,7 +479,7 @@ __global__ __launch_bounds__(WAVES * 64) void k_mfma_tq1(GemmArgs a, int CPT /* 
 #pragma unroll
         for (int r = 0; r < R; ++r)
 #pragma unroll
-          for (int g = 0; g < 5; ++g) wq[r][g] = ((const Packed8*)(p0 + row_off[r] + FB[g]))->v;
+          for (int g = 0; g < 5; ++g) wd[r][g] = ((const Packed8*)(p0 + row_off[r] + FB[g]))->v;
       } else {  // last chunk of the row: never read past the end of the tensor
 #pragma unroll
         for (int r = 0; r < R; ++r)
@@ -481,15 +490,16 @@ __global__ __launch_bounds__(WAVES * 64) void k_mfma_tq1(GemmArgs a, int CPT /* 
             const u32x2 v = ((const Packed8*)q)->v;
             const unsigned sh = (unsigned)(p - q) * 8u;
             const unsigned long long wide = (((unsigned long long)v.y << 32) | v.x) >> (sh < 63u ? sh : 63u);
-            wq[r][g] = u32x2{(unsigned)wide, (unsigned)(wide >> 32)};
+            wd[r][g] = u32x2{(unsigned)wide, (unsigned)(wide >> 32)};
           }
       }
 #pragma unroll
-      for (int r = 0; r < R; ++r) sq[r] = ((const Packed16*)(srow + srow_off[r] + gi * 2))->v;
+      for (int r = 0; r < R; ++r) sd[r] = ((const Packed16*)(srow + srow_off[r] + gi * 2))->v;
     };
     const bool restage = term == 0 || tiles > 1;
     if (restage) stage_load(0);
-    fetch(0);
+#pragma unroll
+    for (int i = 0; i < PFQ; ++i) fetch(i, wq[i], sq[i]);
     for (int64_t tl = 0; tl < tiles; ++tl) {
       if (restage) {
         __syncthreads();
@@ -503,17 +513,32 @@ __global__ __launch_bounds__(WAVES * 64) void k_mfma_tq1(GemmArgs a, int CPT /* 
         u32x4 sraw[R];
 #pragma unroll
         for (int r = 0; r < R; ++r) {
-          sraw[r] = sq[r];
+          sraw[r] = sq[0][r];
 #pragma unroll
-          for (int g = 0; g < 5; ++g) w[r][g] = wq[r][g];
+          for (int g = 0; g < 5; ++g) w[r][g] = wq[0][r][g];
         }
-        fetch(c + 1);
+#pragma unroll
+        for (int i = 0; i + 1 < PFQ; ++i)  // rotate the queue (register moves), then refill its tail
+#pragma unroll
+          for (int r = 0; r < R; ++r) {
+            sq[i][r] = sq[i + 1][r];
+#pragma unroll
+            for (int g = 0; g < 5; ++g) wq[i][r][g] = wq[i + 1][r][g];
+          }
+        fetch(c + PFQ, wq[PFQ - 1], sq[PFQ - 1]);
         const int64_t groups_left = a.G - 5 * c;
         const int ng = groups_left < 5 ? (int)groups_left : 5;
         int64_t gi = 5 * c;
         if (gi > a.G - 8) gi = a.G - 8;
         const int sshift = (int)(5 * c - gi);  // wave-uniform; 0 except in the last chunks of a row
         const unsigned xoff = (unsigned)((c - tl * CPT) * 2048);
+        if (ABL == 1) {  // ablation (timing experiments only): memory traffic without decode and MFMA
+#pragma unroll
+          for (int r = 0; r < R; ++r)
+#pragma unroll
+            for (int g = 0; g < 5; ++g) total[r][0][0] += __uint_as_float((w[r][g].x ^ w[r][g].y ^ sraw[r].x) & 0x3fffffu);
+          continue;
+        }
 #pragma unroll
         for (int g = 0; g < 5; ++g) {
           if (g < ng) {
@@ -532,7 +557,8 @@ __global__ __launch_bounds__(WAVES * 64) void k_mfma_tq1(GemmArgs a, int CPT /* 
 #pragma unroll
               for (int r = 0; r < R; ++r) {
                 const unsigned src = m < 4 ? w[r][g].x : w[r][g].y;
-                we[buf][r] = *(const lds_u32x2*)((__builtin_amdgcn_ubfe(src, 8 * (m & 3), 8) << 7) | lane_off);
+                // (byte << 8) | lane offset in one v_perm_b32: result bytes = [lane_off.b0, src.b[m & 3], 0, 0]
+                we[buf][r] = *(const lds_u32x2*)__builtin_amdgcn_perm(src, lane_off, 0x0c0c0000u | ((unsigned)(4 + (m & 3)) << 8));
               }
             };
             issue(0, 0);
@@ -561,6 +587,11 @@ __global__ __launch_bounds__(WAVES * 64) void k_mfma_tq1(GemmArgs a, int CPT /* 
                 const u32x2 en = we[cur][r];
                 const u32x4 d = {__builtin_amdgcn_perm(en.y, en.x, s0), __builtin_amdgcn_perm(en.y, en.x, s1),
                                  __builtin_amdgcn_perm(en.y, en.x, s2), 0u};
+                if (ABL == 2) {  // ablation: everything but the MFMA
+#pragma unroll
+                  for (int mt = 0; mt < MT; ++mt) acc[r][mt][0] += __uint_as_float((d.x ^ d.y ^ d.z ^ xa[cur][mt].x) & 0x3fffffu);
+                  continue;
+                }
 #pragma unroll
                 for (int mt = 0; mt < MT; ++mt)
                   acc[r][mt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, xa[cur][mt]),
@@ -610,7 +641,7 @@ __global__ __launch_bounds__(WAVES * 64) void k_mfma_tq1(GemmArgs a, int CPT /* 
   }
 }
 
-template <int SDT, int R, int MT, int WAVES>
+template <int SDT, int R, int MT, int WAVES, int ABL = 0>
 int launch_tq1(const GemmArgs& a, hipStream_t s, const char* name) {
   const int64_t rows_per_wg = (int64_t)WAVES * 16 * R;
   const dim3 grid((unsigned)((a.N + rows_per_wg - 1) / rows_per_wg), (unsigned)a.E,
@@ -620,16 +651,16 @@ int launch_tq1(const GemmArgs& a, hipStream_t s, const char* name) {
   int64_t cpt = (X_TILE_BYTES / tokens - 16) / 2048;  // 128 slots of 16 bytes per chunk and token
   if (cpt > nchunks) cpt = nchunks;
   if (cpt < 1) return fail(BP_ERR_UNSUPPORTED, "activation tile does not fit");
-  const size_t lds = X_BASE + (size_t)tokens * (cpt * 2048 + 16);
+  const size_t lds = T1_X_BASE + (size_t)tokens * (cpt * 2048 + 16) + 32;
   static bool attr = false;
   if (!attr) {
-    if (hipFuncSetAttribute((const void*)k_mfma_tq1<SDT, R, MT, WAVES>, hipFuncAttributeMaxDynamicSharedMemorySize,
-                            X_BASE + X_TILE_BYTES) != hipSuccess)
+    if (hipFuncSetAttribute((const void*)k_mfma_tq1<SDT, R, MT, WAVES, ABL>, hipFuncAttributeMaxDynamicSharedMemorySize,
+                            T1_X_BASE + X_TILE_BYTES + 32) != hipSuccess)
       return fail(BP_ERR_LAUNCH, "cannot raise the dynamic LDS limit");
     attr = true;
   }
   note_kernel(name);
-  hipLaunchKernelGGL((k_mfma_tq1<SDT, R, MT, WAVES>), grid, dim3(WAVES * 64), lds, s, a, (int)cpt);
+  hipLaunchKernelGGL((k_mfma_tq1<SDT, R, MT, WAVES, ABL>), grid, dim3(WAVES * 64), lds, s, a, (int)cpt);
   return check_launch(name);
 }
 
@@ -674,6 +705,10 @@ int launch_mfma(const GemmArgs& a, hipStream_t s) {
   if (const char* t = getenv("BP_TUNE_MT")) { const int v = atoi(t); if (v == 1 || v == 2) MT = v; }
   if (a.fmt == BP_TQ1) {
     MT = 1;  // a 16-token slot-layout tile is the most the LDS budget holds; more rows go to more workgroups
+    if (const char* t = getenv("BP_TUNE_ABL")) {
+      if (atoi(t) == 1) return launch_tq1<BP_F16, 1, 1, 16, 1>(a, s, "abl1_tq1");
+      if (atoi(t) == 2) return launch_tq1<BP_F16, 1, 1, 16, 2>(a, s, "abl2_tq1");
+    }
 #define BP_T1(RV, WV) \
     if (R == RV && waves == WV) return launch_tq1_sd<RV, 1, WV>(a, s, "mfma_tq1_bf16_r" #RV "_m1_w" #WV);
     BP_T1(1, 8) BP_T1(2, 8) BP_T1(1, 16) BP_T1(2, 16)
