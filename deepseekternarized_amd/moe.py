@@ -1,0 +1,95 @@
+"""Routed-expert MoE layer on the grouped ternary GEMM.
+
+The reference engines run a MoE layer as a Python loop over all experts with one ``TernaryLinear`` call
+per projection (``boilerplate/engine/standard.py:151-176``; the grouped kernel API is not wired into
+them). This module runs the same computation, with the same rounding points, as one sort of the routing,
+one row gather and three grouped launches (gate and up share one launch over a stacked [E, 2I, Kp]
+weight):
+
+    scores = softmax(router_logits.float()); values, indices = topk(scores, k); values -> x.dtype
+    per (token, slot): y = down(silu(gate(x)) * up(x)) * value, each linear rounded to x.dtype,
+    out[token] += y in ascending expert order, accumulated in x.dtype
+
+softmax / topk are torch ops (as in the reference); everything touching packed weights runs in the HIP
+kernels. bf16 activations (``act="bf16"``) or per-row int8 (``act="int8"``, Mode D default).
+"""
+
+from __future__ import annotations
+
+import torch
+
+from .kernels import _lib
+from .kernels.ternary_hip import _fmt_code, _need_ext, gather_rows, grouped_ternary_gemm, sort_by_expert
+from .ternary.ops import quant_act_int8
+
+
+def swiglu_bf16(gate_up: torch.Tensor, inter: int) -> torch.Tensor:
+    """bf16(bf16(silu(bf16 gate)) * bf16 up) from a float32 [rows, 2 * inter] gate|up product
+    (``StandardDecoder._run_mlp``, boilerplate/engine/standard.py:151-154, on bf16 tensors)."""
+    e = _need_ext(gate_up)
+    rows = gate_up.size(0)
+    h = torch.empty(rows, inter, dtype=torch.bfloat16, device=gate_up.device)
+    up = gate_up[:, inter:]
+    with torch.cuda.device(gate_up.device):
+        _lib.check(e.lib.bp_swiglu_bf16(h.data_ptr(), gate_up.data_ptr(), up.data_ptr(), rows, inter, gate_up.stride(0),
+                                        _lib.stream_ptr(gate_up.device)))
+    return h
+
+
+def moe_combine_bf16(y: torch.Tensor, inv: torch.Tensor, values: torch.Tensor, indices: torch.Tensor) -> torch.Tensor:
+    """out[t] = sum over the token's slots, in ascending expert order, of bf16(bf16(y[inv[t, s]]) * values[t, s]),
+    accumulated in bf16 (``output.index_add_`` on a bf16 tensor, boilerplate/engine/standard.py:173-175)."""
+    e = _need_ext(y)
+    T, k = indices.shape
+    H = y.size(1)
+    out = torch.empty(T, H, dtype=torch.bfloat16, device=y.device)
+    with torch.cuda.device(y.device):
+        _lib.check(e.lib.bp_moe_combine_bf16(out.data_ptr(), y.data_ptr(), inv.data_ptr(), values.data_ptr(),
+                                             indices.data_ptr(), T, k, H, _lib.stream_ptr(y.device)))
+    return out
+
+
+class TernaryMoE:
+    """``experts``: per projection a list of stacked terms ``(packed [E, N, Kp] uint8, scale [E, N, G])``:
+    ``gate`` / ``up`` with N = inter, K = hidden; ``down`` with N = hidden, K = inter."""
+
+    def __init__(self, gate, up, down, hidden: int, inter: int, top_k: int, fmt: str, group: int,
+                 act: str = "bf16", renorm: bool = False):
+        _fmt_code(fmt)
+        if act not in ("bf16", "int8"):
+            raise ValueError(f"unknown activation mode {act!r}")
+        if not (len(gate) == len(up) == len(down)):
+            raise ValueError("gate, up and down must hold the same number of stacked terms")
+        self.hidden, self.inter, self.top_k, self.fmt, self.group, self.act, self.renorm = hidden, inter, top_k, fmt, group, act, renorm
+        self.n_experts = gate[0][0].size(0)
+        # gate and up stacked along N once, so both projections of an expert stream in one launch
+        self.gate_up = [(torch.cat([g[0], u[0]], 1).contiguous(), torch.cat([g[1], u[1]], 1).contiguous())
+                        for g, u in zip(gate, up)]
+        self.down = [(p.contiguous(), s.contiguous()) for p, s in down]
+
+    def _linear(self, x, terms, K):
+        if self.act == "int8":
+            q, s = quant_act_int8(x)
+        else:
+            q, s = x, None
+        return grouped_ternary_gemm(q, s, self._offsets, [p for p, _ in terms], [sc for _, sc in terms], K, self.group, self.fmt)
+
+    def __call__(self, x: torch.Tensor, router_logits: torch.Tensor) -> torch.Tensor:
+        shape = x.shape
+        flat = x.reshape(-1, self.hidden).to(torch.bfloat16).contiguous()
+        _need_ext(flat)
+        scores = torch.softmax(router_logits.reshape(flat.size(0), -1).float(), dim=-1)
+        values, indices = torch.topk(scores, self.top_k, dim=-1)
+        if self.renorm:
+            values = values / values.sum(-1, keepdim=True)
+        values = values.to(torch.bfloat16).contiguous()
+        indices = indices.contiguous()
+        order, self._offsets = sort_by_expert(indices.reshape(-1), self.n_experts)
+        inv = torch.empty_like(order)
+        inv[order] = torch.arange(order.numel(), device=order.device)
+        xg = gather_rows(flat, order, self.top_k)                                  # [T*k, H] rows in expert order
+        gu = self._linear(xg, self.gate_up, self.hidden)                           # f32 [T*k, 2I]
+        h = swiglu_bf16(gu, self.inter)                                            # bf16 [T*k, I]
+        y = self._linear(h, self.down, self.inter)                                 # f32 [T*k, H]
+        out = moe_combine_bf16(y, inv, values, indices)
+        return out.view(shape).to(x.dtype)

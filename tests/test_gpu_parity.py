@@ -380,3 +380,30 @@ def test_linearity_at_full_size(bp, fmt):
     eye[np.arange(len(ks)), ks] = 1.0
     want = (trits[:, ks].astype(np.float32) * scale[:, [k // group for k in ks]].astype(np.float32)).T
     assert np.array_equal(f(eye).astype(np.float32), want)  # one nonzero product per output: exact
+
+
+# --------------------------------------------------------------------------- MoE layer (engine call pattern)
+@pytest.mark.parametrize("fmt,act", [("tq1", "bf16"), ("tq2", "bf16"), ("tq2", "int8")])
+def test_moe_layer_matches_reference_call_pattern(bp, fmt, act):
+    """route -> per-expert SwiGLU -> weighted combine with the rounding points of
+    boilerplate/engine/standard.py:151-176, against oracle.moe_layer_ref (top-2 of 8 experts, one empty)."""
+    from deepseekternarized_amd.moe import TernaryMoE
+
+    H, I, E, k, T, group = 1024, 1024, 8, 2, 12, 128
+    rng = np.random.default_rng(21)
+    mats = {}
+    for name, (n, kk) in (("gate", (I, H)), ("up", (I, H)), ("down", (H, I))):
+        tr = synth_trits(rng, (E, n, kk))
+        sc = (0.05 * np.abs(rng.standard_normal((E, n, kk // group)))).astype(np.float16)
+        mats[name] = (np.stack([orc.pack(tr[e], fmt) for e in range(E)]), sc)
+    x = orc.bf16_round(rng.standard_normal((T, H)).astype(np.float32))
+    logits = (rng.standard_normal((T, E)) * 1.5).astype(np.float32)
+    logits[:, 5] = -30.0  # expert 5 is never routed to
+    experts = [tuple([(mats[n][0][e], mats[n][1][e])] for n in ("gate", "up", "down")) for e in range(E)]
+    want = orc.moe_layer_ref(x, logits, experts, k, H, I, group, fmt, act=act)
+    moe = TernaryMoE(*[[(dev(mats[n][0]), dev(mats[n][1]))] for n in ("gate", "up", "down")], H, I, k, fmt, group, act=act)
+    got = moe(bf16_dev(x), dev(logits)).float().cpu().numpy()
+    assert got.shape == (T, H) and np.isfinite(got).all()
+    # both sides round to bf16 at the same points; float32 summation order may flip a few roundings
+    assert rel_l2(got, want) <= 5e-3, rel_l2(got, want)
+    assert np.abs(got - want).max() <= MAX_ABS_BF16 * max(1.0, np.abs(want).max())
