@@ -346,9 +346,17 @@ int launch_tq2_sd(const GemmArgs& a, hipStream_t s, const char* name) {
 // factor 2 is folded into the group scale (exact). Zeroing digits is a matter of the perm selector.
 struct __attribute__((packed, aligned(2))) Packed16 { u32x4 v; };
 struct __attribute__((packed, aligned(1))) Packed8 { u32x2 v; };
-constexpr int T1_STRIDE = 256;
-constexpr int T1_X_BASE = 256 * T1_STRIDE;  // activation tile starts after the 64 KiB table
+constexpr int T1_STRIDE = 128;
+constexpr int T1_WROW = 144;                       // bytes per row of a wave's packed-byte transpose buffer
+constexpr int T1_WBUF_BASE = 256 * T1_STRIDE;      // after the 32 KiB table: WAVES * 16 rows * T1_WROW bytes
+struct __attribute__((packed, aligned(4))) Packed16a4 { u32x4 v; };
 
+template <int WAVES>
+constexpr int t1_tail_base() { return T1_WBUF_BASE + 2 * WAVES * 16 * T1_WROW; }  // two row sub-tiles per wave
+template <int WAVES>
+constexpr int t1_x_base() { return t1_tail_base<WAVES>() + 16 * T1_WROW; }  // + the tensor-tail buffer (16 rows)
+
+// 16 bytes from a 4-byte aligned address, never reading at or past `end` (bytes there read as 1-digits = zero trits)
 constexpr unsigned tq1_sel(int dword, int keep_from, int keep_to) {  // selector of operand dword 0..2
   // operand dword d holds digits 2d (low half) and 2d+1 (high half); a kept digit i reads entry byte i
   // (bytes 0..3 from the entry's low dword = perm source 1, byte 4 from the high dword = source 0)
@@ -362,14 +370,14 @@ constexpr unsigned tq1_sel(int dword, int keep_from, int keep_to) {  // selector
 template <int SDT, int R, int MT, int WAVES, int ABL = 0>
 __global__ __launch_bounds__(WAVES * 64) void k_mfma_tq1(GemmArgs a, int CPT /* chunks per activation tile */) {
   constexpr int THREADS = WAVES * 64;
+  constexpr int T1_X_BASE = t1_x_base<WAVES>();
   constexpr int XU = (X_TILE_BYTES / 16 + THREADS - 1) / THREADS;  // activation slots staged per thread
   constexpr int FB[5] = {0, 25, 51, 76, 102};
   constexpr int DF[5] = {0, 3, 1, 4, 2};
   constexpr int DL[5] = {3, 1, 4, 2, 5};
   constexpr int MLAST[5] = {4, 5, 4, 5, 4};  // NB[g] - 1 - 21 with NB = {26, 27, 26, 27, 26}
 
-  // ---- table: entry of byte v, copy c (16 copies) at v * 256 + c * 8 (the 256-byte stride makes the
-  // address of an entry a single byte permute of the packed word)
+  // ---- table: entry of byte v, copy c (16 copies) at v * 128 + c * 8
   if (threadIdx.x < 256) {
     const unsigned v = threadIdx.x;
     unsigned hb[5];
@@ -401,6 +409,13 @@ __global__ __launch_bounds__(WAVES * 64) void k_mfma_tq1(GemmArgs a, int CPT /* 
     row_off[r] = rows_valid[r] ? 16 * r * a.Kp : 0;
     srow_off[r] = rows_valid[r] ? 16 * r * a.G * 2 : 0;
   }
+
+  // The wide loads of a row's last chunk read up to 135 bytes past the chunk start, i.e. into the rows
+  // that follow (Kp >= 205). The last 16 rows of the tensor have nothing after them: for that sub-tile the
+  // last chunk comes from a small LDS buffer filled once, byte by byte, with loads that stay in bounds.
+  bool is_tail[R];
+#pragma unroll
+  for (int r = 0; r < R; ++r) is_tail[r] = rows_valid[r] && e + 1 == a.E && n0 + 16 * r + 16 >= a.N;
 
   // ---- activation tile, slot layout: slot s of token t at T1_X_BASE + t * pitch + s * 16
   const int slots = CPT * 128;
@@ -463,43 +478,52 @@ __global__ __launch_bounds__(WAVES * 64) void k_mfma_tq1(GemmArgs a, int CPT /* 
   const int64_t tiles = (nchunks + CPT - 1) / CPT;
 
   for (int term = 0; term < a.n_terms; ++term) {
-    const unsigned char* wrow = a.packed[term] + (e * a.N + n0 + r16) * a.Kp + 7 * b;
-    const unsigned char* wend = a.packed[term] + a.E * a.N * a.Kp - 8;  // last address an 8-byte load may start at
+    // Packed bytes: every lane loads two aligned 16-byte pieces of its row's 128-byte chunk (plus one
+    // dword past it), the wave transposes them through its private LDS buffer and every lane reads
+    // back the 7 consecutive bytes of its k-block for each group. Aligned wide loads stream ~1.7x
+    // faster than per-lane 8-byte loads at byte offsets.
+    const unsigned char* wbeg = a.packed[term];
+    const unsigned char* rowp = wbeg + (e * a.N + n0 + r16) * a.Kp;
     const unsigned char* srow = (const unsigned char*)a.w_scale[term] + (e * a.N + n0 + r16) * a.G * 2;
-    // queue of PFQ chunks of packed bytes and scales in flight behind the chunk being computed
-    constexpr int PFQ = 2;
-    u32x2 wq[PFQ][R][5];
-    u32x4 sq[PFQ][R];
-    auto fetch = [&](int64_t c, u32x2 (&wd)[R][5], u32x4 (&sd)[R]) {  // chunk c (clamped to the last chunk)
-      const int64_t cc = c < nchunks ? c : nchunks - 1;
-      int64_t gi = 5 * cc;
-      if (gi > a.G - 8) gi = a.G - 8;
-      const unsigned char* p0 = wrow + 128 * cc;
-      if (cc + 1 < nchunks) {  // interior chunk: a load may run 3 bytes into the next chunk of the same row
+    const unsigned wrbuf = (unsigned)(T1_WBUF_BASE + (wave * 16 + r16) * T1_WROW);  // this lane's row in the wave's buffer
+    const unsigned tailbuf = (unsigned)(t1_tail_base<WAVES>() + r16 * T1_WROW);
 #pragma unroll
-        for (int r = 0; r < R; ++r)
-#pragma unroll
-          for (int g = 0; g < 5; ++g) wd[r][g] = ((const Packed8*)(p0 + row_off[r] + FB[g]))->v;
-      } else {  // last chunk of the row: never read past the end of the tensor
-#pragma unroll
-        for (int r = 0; r < R; ++r)
-#pragma unroll
-          for (int g = 0; g < 5; ++g) {
-            const unsigned char* p = p0 + row_off[r] + FB[g];
-            const unsigned char* q = p < wend ? p : wend;
-            const u32x2 v = ((const Packed8*)q)->v;
-            const unsigned sh = (unsigned)(p - q) * 8u;
-            const unsigned long long wide = (((unsigned long long)v.y << 32) | v.x) >> (sh < 63u ? sh : 63u);
-            wd[r][g] = u32x2{(unsigned)wide, (unsigned)(wide >> 32)};
-          }
+    for (int r = 0; r < R; ++r) {
+      if (is_tail[r]) {  // at most one wave of the launch: guarded byte copy of the last chunk into LDS
+        const unsigned char* wend = wbeg + a.E * a.N * a.Kp;
+        const unsigned char* base = (const unsigned char*)((uintptr_t)(rowp + row_off[r] + 128 * (nchunks - 1)) & ~(uintptr_t)3);
+#pragma unroll 6
+        for (int i = 0; i < 36; ++i) {
+          const int off = i < 16 ? 16 * b + i : (i < 32 ? 64 + 16 * b + (i - 16) : 128 + (i - 32));
+          const unsigned char* q = base + off;
+          *(__attribute__((address_space(3))) unsigned char*)(tailbuf + off) = q < wend ? *q : (unsigned char)121;
+        }
       }
+    }
+    constexpr int PFQ = 2;  // chunks in flight behind the one being computed
+    u32x4 wq[PFQ][R][2];
+    unsigned wt[PFQ][R];
+    unsigned sq[PFQ][R];  // k-blocks 0..2 each fetch one dword = 2 of the 6 scales starting at an even group index
+    const int sb = b < 3 ? b : 2;
+    auto fetch = [&](int64_t c, u32x4 (&wd)[R][2], unsigned (&td)[R], unsigned (&sd)[R]) {  // chunk c (clamped to the last)
+      const int64_t cl = c < nchunks ? c : nchunks - 1;
+      int64_t gi = (5 * cl) & ~(int64_t)1;  // 4-byte aligned start of the 6 scales that cover groups 5c .. 5c+4
+      if (gi > a.G - 6) gi = a.G - 6;
 #pragma unroll
-      for (int r = 0; r < R; ++r) sd[r] = ((const Packed16*)(srow + srow_off[r] + gi * 2))->v;
+      for (int r = 0; r < R; ++r) {
+        const unsigned char* rp = rowp + row_off[r];
+        const int64_t cc = is_tail[r] && cl + 1 == nchunks ? cl - 1 : cl;  // tensor tail: never fetched from here
+        const unsigned char* p = (const unsigned char*)((uintptr_t)(rp + 128 * cc) & ~(uintptr_t)3) + 16 * b;
+        wd[r][0] = ((const Packed16a4*)p)->v;
+        wd[r][1] = ((const Packed16a4*)(p + 64))->v;
+        td[r] = *(const unsigned*)(p - 16 * b + 128);
+        sd[r] = *(const unsigned*)(srow + srow_off[r] + (gi + 2 * sb) * 2);
+      }
     };
     const bool restage = term == 0 || tiles > 1;
     if (restage) stage_load(0);
 #pragma unroll
-    for (int i = 0; i < PFQ; ++i) fetch(i, wq[i], sq[i]);
+    for (int i = 0; i < PFQ; ++i) fetch(i, wq[i], wt[i], sq[i]);
     for (int64_t tl = 0; tl < tiles; ++tl) {
       if (restage) {
         __syncthreads();
@@ -509,34 +533,46 @@ __global__ __launch_bounds__(WAVES * 64) void k_mfma_tq1(GemmArgs a, int CPT /* 
       }
       const int64_t c_end = (tl + 1) * CPT < nchunks ? (tl + 1) * CPT : nchunks;
       for (int64_t c = tl * CPT; c < c_end; ++c) {
-        u32x2 w[R][5];
-        u32x4 sraw[R];
+        // Transpose through the wave's LDS buffer: row r16 of sub-tile r holds the aligned 128 bytes, the
+        // dword after them and the 6 scales; chunk byte j sits at offset j + dlt. LDS operations of one wave
+        // execute in order; the fences only pin the compiler's ordering.
+        unsigned dlt[R], rbuf[R];
 #pragma unroll
         for (int r = 0; r < R; ++r) {
-          sraw[r] = sq[0][r];
-#pragma unroll
-          for (int g = 0; g < 5; ++g) w[r][g] = wq[0][r][g];
+          const bool from_tail = is_tail[r] && c + 1 == nchunks;
+          rbuf[r] = from_tail ? tailbuf : wrbuf + r * T1_WROW * 16 * WAVES;
+          const unsigned rb = rbuf[r];
+          dlt[r] = (unsigned)((uintptr_t)(rowp + row_off[r]) & 3);
+          if (!from_tail) {
+            *(lds_u32x4*)(rb + 16 * b) = wq[0][r][0];
+            *(lds_u32x4*)(rb + 64 + 16 * b) = wq[0][r][1];
+            *(lds_u32*)(rb + 128) = wt[0][r];
+          }
+          *(lds_u32*)(rb + 132 + 4 * sb) = sq[0][r];
         }
+        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+        __builtin_amdgcn_wave_barrier();
 #pragma unroll
         for (int i = 0; i + 1 < PFQ; ++i)  // rotate the queue (register moves), then refill its tail
 #pragma unroll
           for (int r = 0; r < R; ++r) {
             sq[i][r] = sq[i + 1][r];
-#pragma unroll
-            for (int g = 0; g < 5; ++g) wq[i][r][g] = wq[i + 1][r][g];
+            wt[i][r] = wt[i + 1][r];
+            wq[i][r][0] = wq[i + 1][r][0];
+            wq[i][r][1] = wq[i + 1][r][1];
           }
-        fetch(c + PFQ, wq[PFQ - 1], sq[PFQ - 1]);
+        fetch(c + PFQ, wq[PFQ - 1], wt[PFQ - 1], sq[PFQ - 1]);
         const int64_t groups_left = a.G - 5 * c;
         const int ng = groups_left < 5 ? (int)groups_left : 5;
-        int64_t gi = 5 * c;
-        if (gi > a.G - 8) gi = a.G - 8;
-        const int sshift = (int)(5 * c - gi);  // wave-uniform; 0 except in the last chunks of a row
+        int64_t gi = (5 * c) & ~(int64_t)1;
+        if (gi > a.G - 6) gi = a.G - 6;
+        const int sshift = (int)(5 * c - gi);  // wave-uniform position of group 5c among the 6 scales loaded
         const unsigned xoff = (unsigned)((c - tl * CPT) * 2048);
         if (ABL == 1) {  // ablation (timing experiments only): memory traffic without decode and MFMA
 #pragma unroll
           for (int r = 0; r < R; ++r)
 #pragma unroll
-            for (int g = 0; g < 5; ++g) total[r][0][0] += __uint_as_float((w[r][g].x ^ w[r][g].y ^ sraw[r].x) & 0x3fffffu);
+            for (int g = 0; g < 5; ++g) total[r][0][0] += __uint_as_float((*(const lds_u32*)(wrbuf + 24 * g + 4 * b)) & 0x3fffffu);
           continue;
         }
 #pragma unroll
@@ -549,6 +585,16 @@ __global__ __launch_bounds__(WAVES * 64) void k_mfma_tq1(GemmArgs a, int CPT /* 
               for (int mt = 0; mt < MT; ++mt) acc[r][mt] = f32x4{0.f, 0.f, 0.f, 0.f};
             // two-stage pipeline over the 7 MFMA slots: the LDS reads of slot m+1 are issued before the
             // MFMAs of slot m; the scheduling barriers keep the compiler from hoisting all 35 slots at once
+            u32x2 wg[R];  // the 7 bytes of this lane's k-block for group g, read back from the transpose buffer
+#pragma unroll
+            for (int r = 0; r < R; ++r) {
+              const unsigned rb = rbuf[r];
+              const unsigned o = dlt[r] + FB[g] + 7 * b;
+              const unsigned d0 = *(const lds_u32*)(rb + (o & ~3u));
+              const unsigned d1 = *(const lds_u32*)(rb + (o & ~3u) + 4);
+              const unsigned d2 = *(const lds_u32*)(rb + (o & ~3u) + 8);
+              wg[r] = u32x2{__builtin_amdgcn_alignbyte(d1, d0, o & 3u), __builtin_amdgcn_alignbyte(d2, d1, o & 3u)};
+            }
             u32x4 xa[2][MT];
             u32x2 we[2][R];
             auto issue = [&](int m, int buf) {
@@ -556,9 +602,8 @@ __global__ __launch_bounds__(WAVES * 64) void k_mfma_tq1(GemmArgs a, int CPT /* 
               for (int mt = 0; mt < MT; ++mt) xa[buf][mt] = *(const lds_u32x4*)(xaddr[mt] + xoff + 16 * (FB[g] + m));
 #pragma unroll
               for (int r = 0; r < R; ++r) {
-                const unsigned src = m < 4 ? w[r][g].x : w[r][g].y;
-                // (byte << 8) | lane offset in one v_perm_b32: result bytes = [lane_off.b0, src.b[m & 3], 0, 0]
-                we[buf][r] = *(const lds_u32x2*)__builtin_amdgcn_perm(src, lane_off, 0x0c0c0000u | ((unsigned)(4 + (m & 3)) << 8));
+                const unsigned src = m < 4 ? wg[r].x : wg[r].y;
+                we[buf][r] = *(const lds_u32x2*)((__builtin_amdgcn_ubfe(src, 8 * (m & 3), 8) << 7) | lane_off);
               }
             };
             issue(0, 0);
@@ -601,15 +646,7 @@ __global__ __launch_bounds__(WAVES * 64) void k_mfma_tq1(GemmArgs a, int CPT /* 
             }
 #pragma unroll
             for (int r = 0; r < R; ++r) {
-              unsigned half = 0;  // 16-bit scale of group 5c + g = entry sshift + g of the 8 loaded
-              if (sshift == 0) {
-                const unsigned v = sraw[r][g >> 1];
-                half = (g & 1) ? (v >> 16) : (v & 0xffffu);
-              } else {
-#pragma unroll
-                for (int i = 0; i < 8; ++i)
-                  if (sshift + g == i) { const unsigned v = sraw[r][i >> 1]; half = (i & 1) ? (v >> 16) : (v & 0xffffu); }
-              }
+              const unsigned half = *(const __attribute__((address_space(3))) uint16_t*)(rbuf[r] + 132 + 2 * (sshift + g));
               // weights were decoded as +-0.5: the factor 2 goes into the scale (exact)
               const float sc = 2.0f * (SDT == BP_F16 ? f16_bits_to_f32((uint16_t)half) : __uint_as_float(half << 16));
 #pragma unroll
@@ -651,11 +688,11 @@ int launch_tq1(const GemmArgs& a, hipStream_t s, const char* name) {
   int64_t cpt = (X_TILE_BYTES / tokens - 16) / 2048;  // 128 slots of 16 bytes per chunk and token
   if (cpt > nchunks) cpt = nchunks;
   if (cpt < 1) return fail(BP_ERR_UNSUPPORTED, "activation tile does not fit");
-  const size_t lds = T1_X_BASE + (size_t)tokens * (cpt * 2048 + 16) + 32;
+  const size_t lds = t1_x_base<WAVES>() + (size_t)tokens * (cpt * 2048 + 16) + 32;
   static bool attr = false;
   if (!attr) {
     if (hipFuncSetAttribute((const void*)k_mfma_tq1<SDT, R, MT, WAVES, ABL>, hipFuncAttributeMaxDynamicSharedMemorySize,
-                            T1_X_BASE + X_TILE_BYTES + 32) != hipSuccess)
+                            t1_x_base<WAVES>() + X_TILE_BYTES + 32) != hipSuccess)
       return fail(BP_ERR_LAUNCH, "cannot raise the dynamic LDS limit");
     attr = true;
   }
@@ -687,9 +724,9 @@ bool mfma_supports(const GemmArgs& a) {
   }
   // TQ1: bf16 activations, scales as stored (fp16 / bf16)
   if (a.x_dtype != BP_BF16 || (a.scale_dtype != BP_F16 && a.scale_dtype != BP_BF16)) return false;
-  if (a.K % 128 != 0 || a.K < 1024) return false;
+  if (a.K % 256 != 0 || a.K < 1024) return false;  // whole groups, and an even number of them (4-byte aligned scale rows)
   for (int t = 0; t < a.n_terms; ++t)
-    if (((uintptr_t)a.w_scale[t] & 1) != 0) return false;
+    if (((uintptr_t)a.w_scale[t] & 3) != 0) return false;
   return true;
 }
 
