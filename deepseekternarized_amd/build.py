@@ -18,7 +18,7 @@ CSRC = HERE / "csrc"
 LIB = HERE / "libbp_ternary_hip.so"
 SOURCES = ["bp_api.hip", "bp_general.hip", "bp_route.hip", "bp_mfma.hip"]
 # packed FP32 VALU ops are disabled for every device object of this library
-FLAGS = ["--offload-arch=gfx950", "-O3", "-fPIC", "-std=c++17", "-Wall", "-Wno-unused-function",
+FLAGS = ["--offload-arch=gfx950", "-O3", "-fPIC", "-std=c++17", "-Wall", "-Wno-unused-function", "-Wno-int-to-pointer-cast",
          "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops"]
 
 

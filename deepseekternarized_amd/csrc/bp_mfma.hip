@@ -1,8 +1,9 @@
-// Tuned gfx950 kernels for group = 128: packed trits are decoded through a bank-replicated LDS
-// lookup table straight into MFMA operands, one 16-row x 16-token tile per instruction.
+// Tuned gfx950 kernels for group = 128: packed trits are decoded in registers (TQ2: bit arithmetic,
+// TQ1: a bank-replicated LDS table) straight into MFMA operands, one 16-row x 16-token tile per
+// instruction.
 //
-//   bf16 activations : v_mfma_f32_16x16x32_bf16, table entry = the trits of one byte as bf16
-//   int8 activations : v_mfma_i32_16x16x64_i8,  table entry = the trits of one byte as int8
+//   bf16 activations : v_mfma_f32_16x16x32_bf16
+//   int8 activations : v_mfma_i32_16x16x64_i8 (TQ2 only)
 //
 // Accumulators are flushed at every 128-wide K group: total += acc * scale[n, g] in float32, so the
 // scale multiplies the group sum exactly as in the reference contract
@@ -27,26 +28,58 @@ typedef unsigned u32x4 __attribute__((ext_vector_type(4)));
 typedef float f32x4 __attribute__((ext_vector_type(4)));
 typedef int i32x4 __attribute__((ext_vector_type(4)));
 typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
+typedef __bf16 bf16x2 __attribute__((ext_vector_type(2)));
 typedef __attribute__((address_space(3))) u32x2 lds_u32x2;
 typedef __attribute__((address_space(3))) u32x4 lds_u32x4;
 typedef __attribute__((address_space(3))) unsigned lds_u32;
 
-// LDS map (absolute addresses; these kernels declare no static LDS, so the dynamic allocation
-// requested at launch starts at LDS address 0):
-//   [0, 32 KiB)        decode table: entry of byte value v, copy c at v * 128 + c * EB
-//   [32 KiB, ...)      activation tile: row t at X_BASE + t * pitch, pitch = KC * XB + 16
-constexpr int LUT_STRIDE = 128;
-constexpr int LUT_BYTES = 256 * LUT_STRIDE;
-constexpr int X_BASE = LUT_BYTES;
+// These kernels address LDS absolutely: they declare no static LDS, so the dynamic allocation
+// requested at launch starts at LDS address 0.
+// TQ2: the activation tile starts at 0: row t at t * pitch, pitch = KC * XB + 16.
+constexpr int X_BASE = 0;
 constexpr int X_TILE_BYTES = 48 * 1024;  // TQ1: table + tile = 80 KiB: two workgroups of 8 waves per CU
 
 __device__ __forceinline__ unsigned bf16_of_trit(int t) {
   return t == 0 ? 0u : t == 1 ? 0x3f80u : t == -1 ? 0xbf80u : 0x4000u;  // +2 (TQ2 code 3) -> 2.0
 }
 
-// LDS address of the table entry of byte `sel` (0..3) of w: (byte << 7) | lane offset.
-__device__ __forceinline__ unsigned lut_addr(unsigned w, unsigned lane_off, int sel) {
-  return (__builtin_amdgcn_ubfe(w, 8 * sel, 8) << 7) | lane_off;
+// ---- TQ2 decode without a table.
+// bf16: a 2-bit code u placed at bits [7:6] of a bf16 whose other bits are 0x4000 reads 2 + u (the code
+// spans the lowest exponent bit and the highest mantissa bit: 2, 3, 4); placed at bits [5:4] of 0x4100 it
+// reads 8 + u. One v_and_or_b32 per output dword therefore turns two codes of a packed dword (one per
+// 16-bit half) into two bf16 values; three shifts bring all 16 codes of the dword to those two positions.
+// The products then carry sum(x * (c + u)) with c = 2 (odd trits) or 8 (even trits); the accumulator of
+// every group starts from -sum(x * (c + 1)), computed once per workgroup when the activation tile is
+// staged, which leaves sum(x * (u - 1)). Slot order of the two operands made from a packed dword (codes
+// c0..c15, lo/hi bf16 of each operand dword):
+//   first  : (c3,c11) (c2,c10) (c1,c9) (c0,c8)      second : (c5,c13) (c4,c12) (c7,c15) (c6,c14)
+// The activation tile is stored in LDS in that order (permuted inside every 16 elements when staged).
+// The unused code 3 reads +3 or +2 depending on its slot (pack never writes it).
+struct Tq2Consts { unsigned P1, P2, M1, M2; };  // 0x00c000c0, 0x00300030, 0x40004000, 0x41004100 held in registers
+__device__ __forceinline__ void tq2_decode_bf16(unsigned w, const Tq2Consts& k, u32x4& first, u32x4& second) {
+  const unsigned P1 = k.P1, P2 = k.P2, M1 = k.M1, M2 = k.M2;
+  const unsigned wl = w << 4, wr = w >> 4, wr8 = w >> 8;
+  first = u32x4{(w & P1) | M1, (w & P2) | M2, (wl & P1) | M1, (wl & P2) | M2};
+  second = u32x4{(wr & P1) | M1, (wr & P2) | M2, (wr8 & P1) | M1, (wr8 & P2) | M2};
+}
+// int8: dword i of the operand = codes c(i), c(i+4), c(i+8), c(i+12) as digits 0..2; the accumulator
+// starts from -sum(x). The activation tile is stored with every 16 bytes transposed 4 x 4 to match.
+__device__ __forceinline__ u32x4 tq2_decode_i8(unsigned w) {
+  const unsigned m = 0x03030303u;
+  return u32x4{w & m, (w >> 2) & m, (w >> 4) & m, (w >> 6) & m};
+}
+__device__ __forceinline__ void tq2_permute_bf16(const u32x4 a, const u32x4 c, u32x4& o0, u32x4& o1) {
+  const unsigned HI = 0x07060302u, LO = 0x05040100u;
+  o0 = u32x4{__builtin_amdgcn_perm(c.y, a.y, HI), __builtin_amdgcn_perm(c.y, a.y, LO),
+             __builtin_amdgcn_perm(c.x, a.x, HI), __builtin_amdgcn_perm(c.x, a.x, LO)};
+  o1 = u32x4{__builtin_amdgcn_perm(c.z, a.z, HI), __builtin_amdgcn_perm(c.z, a.z, LO),
+             __builtin_amdgcn_perm(c.w, a.w, HI), __builtin_amdgcn_perm(c.w, a.w, LO)};
+}
+__device__ __forceinline__ u32x4 tq2_permute_i8(const u32x4 a) {
+  const unsigned s0 = __builtin_amdgcn_perm(a.y, a.x, 0x05010400u), s1 = __builtin_amdgcn_perm(a.y, a.x, 0x07030602u);
+  const unsigned s2 = __builtin_amdgcn_perm(a.w, a.z, 0x05010400u), s3 = __builtin_amdgcn_perm(a.w, a.z, 0x07030602u);
+  return u32x4{__builtin_amdgcn_perm(s2, s0, 0x05040100u), __builtin_amdgcn_perm(s2, s0, 0x07060302u),
+               __builtin_amdgcn_perm(s3, s1, 0x05040100u), __builtin_amdgcn_perm(s3, s1, 0x07060302u)};
 }
 
 template <int ACT>
@@ -71,32 +104,12 @@ __device__ __forceinline__ float scale_at(const u32x4 (&raw)[2], int i) {  // i-
 // second, so that all four k-blocks of an MFMA belong to one scale group.
 // After the swap block b holds trits tb(b) .. tb(b)+31 of each group, tb = {0, 64, 32, 96}.
 template <int ACT, int SDT, int R, int MT, int WAVES, int XKB, int ABL = 0>
-__global__ __launch_bounds__(WAVES * 64, 4) void k_mfma_tq2(GemmArgs a, int KC) {
+__global__ __launch_bounds__(WAVES * 64, 4) void k_mfma_tq2(GemmArgs a, int KC, int tile_rows) {
   constexpr int THREADS = WAVES * 64;
-  constexpr int EB = ACT == BP_BF16 ? 8 : 4;   // bytes per table entry
-  constexpr int COPIES = LUT_STRIDE / EB;      // 16 (bf16) or 32 (int8) bank-interleaved copies
   constexpr int XB = ACT == BP_BF16 ? 2 : 1;   // bytes per activation element
   constexpr int KM = ACT == BP_BF16 ? 8 : 16;  // k per lane per MFMA
   constexpr int NJ = 32 / KM;                  // MFMAs per group
-  constexpr int XU = XKB * 1024 / 16 / THREADS;  // 16-byte units of the activation tile per thread
-
-  // ---- build the table: thread v < 256 writes the entry of byte value v into every copy
-  if (threadIdx.x < 256) {
-    const unsigned v = threadIdx.x;
-    int t[4];
-#pragma unroll
-    for (int d = 0; d < 4; ++d) t[d] = (int)((v >> (2 * d)) & 3u) - 1;
-    if (ACT == BP_BF16) {
-      u32x2 e;
-      e.x = bf16_of_trit(t[0]) | (bf16_of_trit(t[1]) << 16);
-      e.y = bf16_of_trit(t[2]) | (bf16_of_trit(t[3]) << 16);
-      for (int c = 0; c < COPIES; ++c) *(lds_u32x2*)(v * LUT_STRIDE + c * EB) = e;
-    } else {
-      const unsigned e = (unsigned)(t[0] & 0xff) | ((unsigned)(t[1] & 0xff) << 8) | ((unsigned)(t[2] & 0xff) << 16) |
-                         ((unsigned)(t[3] & 0xff) << 24);
-      for (int c = 0; c < COPIES; ++c) *(lds_u32*)(v * LUT_STRIDE + c * EB) = e;
-    }
-  }
+  constexpr int XU = XKB * 1024 / (16 * XB) / THREADS;  // 16-element units of the activation tile per thread
 
   const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
   const int r16 = lane & 15, b = lane >> 4;
@@ -108,7 +121,6 @@ __global__ __launch_bounds__(WAVES * 64, 4) void k_mfma_tq2(GemmArgs a, int KC) 
   int64_t n0 = ((int64_t)blockIdx.x * WAVES + wave) * (16 * R);
   const bool wave_live = n0 < a.N;
   if (!wave_live) n0 = 0;  // keeps addresses valid; the wave still takes part in staging and barriers
-  const unsigned lane_off = (unsigned)((lane % COPIES) * EB);
   const int tb = 64 * (b & 1) + 32 * (b >> 1);
 
   // row sub-tiles past N re-read the first sub-tile (branch-free loop body) and are dropped at the store
@@ -122,7 +134,7 @@ __global__ __launch_bounds__(WAVES * 64, 4) void k_mfma_tq2(GemmArgs a, int KC) 
 
   // ---- activation tile geometry
   const int pitch = KC * XB + 16;
-  const int units_per_row = KC * XB / 16;
+  const int units_per_row = KC / 16;
   const int units = ntok * units_per_row;
   unsigned xaddr[MT];  // LDS address of this lane's token row (+ its k-block offset)
 #pragma unroll
@@ -131,25 +143,61 @@ __global__ __launch_bounds__(WAVES * 64, 4) void k_mfma_tq2(GemmArgs a, int KC) 
     if (t >= ntok) t = ntok - 1;
     xaddr[mt] = (unsigned)(X_BASE + t * pitch + tb * XB);
   }
+  // Offset removal: corr[g][t] = -sum over the 128 k of group g of x[t, k] * (c(k) + 1) (bf16: c + 1 = 9 for
+  // even k, 3 for odd k; int8: 1), float32 / int32, at corr_base + (g * 16 * MT + t) * 4. A lane starts the
+  // accumulator of a group from the four values of its tokens 4b .. 4b + 3.
+  const unsigned corr_base = (unsigned)(X_BASE + tile_rows * pitch);
+  const unsigned corr_lane = corr_base + (unsigned)(16 * b);
   const unsigned char* xg = (const unsigned char*)a.x + tok0 * a.K * XB;
-  u32x4 xstage[XU];
+  u32x4 xstage[XU][XB];
   auto stage_load = [&](int64_t k0) {  // global -> registers, chunk starting at k0
 #pragma unroll
     for (int i = 0; i < XU; ++i) {
       const int u = threadIdx.x + i * THREADS;
-      if (u < units) {
-        const int row = u / units_per_row, col = u - row * units_per_row;
-        xstage[i] = *(const u32x4*)(xg + ((int64_t)row * a.K + k0) * XB + col * 16);
+      const int row = u / units_per_row, col = u - row * units_per_row;
+      if (u < units && k0 + col * 16 < a.K) {  // the last chunk may be shorter than KC: stay inside the row
+        const unsigned char* p = xg + ((int64_t)row * a.K + k0 + col * 16) * XB;
+#pragma unroll
+        for (int v = 0; v < XB; ++v) xstage[i][v] = *(const u32x4*)(p + 16 * v);
       }
     }
   };
-  auto stage_store = [&]() {  // registers -> LDS
+  auto stage_store = [&]() {  // registers -> LDS, every 16 elements reordered to the decode's slot order
 #pragma unroll
     for (int i = 0; i < XU; ++i) {
       const int u = threadIdx.x + i * THREADS;
       if (u < units) {
         const int row = u / units_per_row, col = u - row * units_per_row;
-        *(lds_u32x4*)(X_BASE + row * pitch + col * 16) = xstage[i];
+        const unsigned dst = (unsigned)(X_BASE + row * pitch + col * 16 * XB);
+        unsigned part;  // this unit's share of the group's offset sum; 8 consecutive lanes hold one group
+        if (ACT == BP_BF16) {
+          u32x4 o0, o1;
+          tq2_permute_bf16(xstage[i][0], xstage[i][XB - 1], o0, o1);
+          *(lds_u32x4*)(dst) = o0;
+          *(lds_u32x4*)(dst + 16) = o1;
+          float f = 0.f;
+          const bf16x2 w93 = __builtin_bit_cast(bf16x2, 0x40404110u);  // (9.0, 3.0): even k in the low half
+#pragma unroll
+          for (int v = 0; v < XB; ++v) {
+            const unsigned dw[4] = {xstage[i][v].x, xstage[i][v].y, xstage[i][v].z, xstage[i][v].w};
+#pragma unroll
+            for (int d = 0; d < 4; ++d) f = __builtin_amdgcn_fdot2_f32_bf16(__builtin_bit_cast(bf16x2, dw[d]), w93, f, false);
+          }
+          f += __shfl_xor(f, 1);
+          f += __shfl_xor(f, 2);
+          f += __shfl_xor(f, 4);
+          part = __float_as_uint(-f);
+        } else {
+          *(lds_u32x4*)(dst) = tq2_permute_i8(xstage[i][0]);
+          int n = 0;
+#pragma unroll
+          for (int d = 0; d < 4; ++d) n = __builtin_amdgcn_sdot4((int)xstage[i][0][d], 0x01010101, n, false);
+          n += __shfl_xor(n, 1);
+          n += __shfl_xor(n, 2);
+          n += __shfl_xor(n, 4);
+          part = (unsigned)(-n);
+        }
+        if ((col & 7) == 0) *(lds_u32*)(corr_base + ((col >> 3) * (16 * MT) + row) * 4) = part;
       }
     }
   };
@@ -159,6 +207,11 @@ __global__ __launch_bounds__(WAVES * 64, 4) void k_mfma_tq2(GemmArgs a, int KC) 
   for (int r = 0; r < R; ++r)
 #pragma unroll
     for (int mt = 0; mt < MT; ++mt) total[r][mt] = f32x4{0.f, 0.f, 0.f, 0.f};
+
+  // decode masks and exponent patterns live in registers: v_and_or_b32 takes no literal operands
+  Tq2Consts kc = {0x00c000c0u, 0x00300030u, 0x40004000u, 0x41004100u};
+  asm volatile("" : "+s"(kc.P1), "+s"(kc.P2));
+  asm volatile("" : "+v"(kc.M1), "+v"(kc.M2));
 
   const int64_t steps = a.K / 256;
   const int steps_per_chunk = KC / 256;
@@ -188,12 +241,18 @@ __global__ __launch_bounds__(WAVES * 64, 4) void k_mfma_tq2(GemmArgs a, int KC) 
     };
     const bool restage = term == 0 || chunks > 1;  // a tile that holds all of K is staged once for all terms
     if (restage) stage_load(0);
-#pragma unroll
-    for (int i = 0; i < PF; ++i) fetch_w(i, ring[i]);
+    // Same issue order as inside the loop (scales, then the weights step by step), pinned with scheduling
+    // barriers: loads return in order, so the loop's waits can then leave the younger loads in flight.
     fetch_s(0, snext);
+    __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+    for (int i = 0; i < PF; ++i) {
+      fetch_w(i, ring[i]);
+      __builtin_amdgcn_sched_barrier(0);
+    }
     for (int64_t ch = 0; ch < chunks; ++ch) {
       if (restage) {
-        __syncthreads();  // every wave is done reading the previous tile (and, first time, the table is built)
+        __syncthreads();  // every wave is done reading the previous tile 
         stage_store();
         __syncthreads();
         if (ch + 1 < chunks) stage_load((ch + 1) * KC);
@@ -205,19 +264,20 @@ __global__ __launch_bounds__(WAVES * 64, 4) void k_mfma_tq2(GemmArgs a, int KC) 
         fetch_s(c4 + 4, snext);
 #pragma unroll
         for (int i = 0; i < PF; ++i) {
+          // One scheduling region per step: the wait for this step's weights stays here instead of joining
+          // the waits of the later steps at the top of the block.
+          __builtin_amdgcn_sched_barrier(0);
           const int64_t c = c4 + i;
           u32x4 w[R];
 #pragma unroll
-          for (int r = 0; r < R; ++r) w[r] = ring[i][r];
-          fetch_w(c + PF, ring[i]);
-#pragma unroll
           for (int r = 0; r < R; ++r) {  // regroup: .x/.y = 8 bytes of group 2c, .z/.w = 8 bytes of group 2c+1
-            const auto s0 = __builtin_amdgcn_permlane32_swap(w[r].x, w[r].z, false, false);
-            const auto s1 = __builtin_amdgcn_permlane32_swap(w[r].y, w[r].w, false, false);
-            w[r].x = s0[0]; w[r].z = s0[1];
-            w[r].y = s1[0]; w[r].w = s1[1];
+            const auto s0 = __builtin_amdgcn_permlane32_swap(ring[i][r].x, ring[i][r].z, false, false);
+            const auto s1 = __builtin_amdgcn_permlane32_swap(ring[i][r].y, ring[i][r].w, false, false);
+            w[r] = u32x4{s0[0], s1[0], s0[1], s1[1]};
           }
-          const unsigned xoff = (unsigned)((c - ch * steps_per_chunk) * 256 * XB);
+          fetch_w(c + PF, ring[i]);
+          const int gl = (int)(c - ch * steps_per_chunk) * 2;  // first of the step's two groups within the tile
+          const unsigned xoff = (unsigned)(gl * 128 * XB);
           if (ABL == 1) {  // ablation (timing experiments only): memory traffic without decode and MFMA
 #pragma unroll
             for (int r = 0; r < R; ++r) total[r][0][0] += __uint_as_float((w[r].x ^ w[r].y ^ w[r].z ^ w[r].w) & 0x3fffffu);
@@ -225,52 +285,42 @@ __global__ __launch_bounds__(WAVES * 64, 4) void k_mfma_tq2(GemmArgs a, int KC) 
           }
 #pragma unroll
           for (int h = 0; h < 2; ++h) {
-            typename Acc<ACT>::type acc[R][MT];
+            typedef typename Acc<ACT>::type acc_t;
+            u32x4 xa[NJ][MT];
+            acc_t base[MT];
 #pragma unroll
-            for (int r = 0; r < R; ++r)
+            for (int mt = 0; mt < MT; ++mt) {
+              base[mt] = __builtin_bit_cast(acc_t, *(const lds_u32x4*)(corr_lane + ((gl + h) * (16 * MT) + 16 * mt) * 4));
 #pragma unroll
-              for (int mt = 0; mt < MT; ++mt) acc[r][mt] = typename Acc<ACT>::type{0, 0, 0, 0};
-#pragma unroll
-            for (int j = 0; j < NJ; ++j) {
-              u32x4 xa[MT];
-#pragma unroll
-              for (int mt = 0; mt < MT; ++mt) xa[mt] = *(const lds_u32x4*)(xaddr[mt] + xoff + (h * 128 + j * KM) * XB);
-              u32x4 wb[R];  // decoded operand of every row sub-tile first, then the MFMAs: independent chains
-#pragma unroll
-              for (int r = 0; r < R; ++r) {
-                const unsigned lo = h == 0 ? w[r].x : w[r].z, hi = h == 0 ? w[r].y : w[r].w;
-                if (ACT == BP_BF16) {
-                  const unsigned src = j < 2 ? lo : hi;
-                  const u32x2 e0 = *(const lds_u32x2*)(lut_addr(src, lane_off, 2 * (j & 1)));
-                  const u32x2 e1 = *(const lds_u32x2*)(lut_addr(src, lane_off, 2 * (j & 1) + 1));
-                  wb[r] = u32x4{e0.x, e0.y, e1.x, e1.y};
-                } else {
-                  const unsigned src = j == 0 ? lo : hi;
-                  wb[r].x = *(const lds_u32*)(lut_addr(src, lane_off, 0));
-                  wb[r].y = *(const lds_u32*)(lut_addr(src, lane_off, 1));
-                  wb[r].z = *(const lds_u32*)(lut_addr(src, lane_off, 2));
-                  wb[r].w = *(const lds_u32*)(lut_addr(src, lane_off, 3));
-                }
-              }
-#pragma unroll
-              for (int r = 0; r < R; ++r)
-#pragma unroll
-                for (int mt = 0; mt < MT; ++mt) {
-                  if (ACT == BP_BF16)
-                    acc[r][mt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, xa[mt]),
-                                                                         __builtin_bit_cast(bf16x8, wb[r]), acc[r][mt], 0, 0, 0);
-                  else
-                    acc[r][mt] = __builtin_amdgcn_mfma_i32_16x16x64_i8(__builtin_bit_cast(i32x4, xa[mt]),
-                                                                       __builtin_bit_cast(i32x4, wb[r]), acc[r][mt], 0, 0, 0);
-                }
+              for (int j = 0; j < NJ; ++j) xa[j][mt] = *(const lds_u32x4*)(xaddr[mt] + xoff + (h * 128 + j * KM) * XB);
             }
 #pragma unroll
             for (int r = 0; r < R; ++r) {
+              const unsigned lo = h == 0 ? w[r].x : w[r].z, hi = h == 0 ? w[r].y : w[r].w;
+              u32x4 wb[NJ];
+              if (ACT == BP_BF16) {
+                tq2_decode_bf16(lo, kc, wb[0], wb[1]);
+                tq2_decode_bf16(hi, kc, wb[NJ - 2], wb[NJ - 1]);
+              } else {
+                wb[0] = tq2_decode_i8(lo);
+                wb[1] = tq2_decode_i8(hi);
+              }
               const float s = scale_at<SDT>(sraw[r], 2 * i + h);  // group 2c + h = entry 2i + h of the 8 held
 #pragma unroll
-              for (int mt = 0; mt < MT; ++mt)
+              for (int mt = 0; mt < MT; ++mt) {
+                acc_t acc = base[mt];
 #pragma unroll
-                for (int q = 0; q < 4; ++q) total[r][mt][q] += (float)acc[r][mt][q] * s;
+                for (int j = 0; j < NJ; ++j) {
+                  if (ACT == BP_BF16)
+                    acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, xa[j][mt]),
+                                                                  __builtin_bit_cast(bf16x8, wb[j]), acc, 0, 0, 0);
+                  else
+                    acc = __builtin_amdgcn_mfma_i32_16x16x64_i8(__builtin_bit_cast(i32x4, xa[j][mt]),
+                                                                __builtin_bit_cast(i32x4, wb[j]), acc, 0, 0, 0);
+                }
+#pragma unroll
+                for (int q = 0; q < 4; ++q) total[r][mt][q] += (float)acc[q] * s;
+              }
             }
           }
         }
@@ -306,10 +356,11 @@ int launch_tq2(const GemmArgs& a, hipStream_t s, const char* name) {
                   (unsigned)((a.max_rows + 16 * MT - 1) / (16 * MT)));
   // chunk length: as much of K as the tile budget holds for the widest token tile, in blocks of 4 steps
   const int64_t tokens = a.max_rows < 16 * MT ? a.max_rows : 16 * MT;
-  int64_t kc = (XKB * 1024 / tokens - 16) / XB / 1024 * 1024;
+  // bytes per k: the tokens' activations plus 16 * MT offset sums of 4 bytes per 128-wide group
+  int64_t kc = 2 * (XKB * 1024 - 16 * tokens) / (2 * tokens * XB + MT) / 1024 * 1024;
   if (kc > a.K) kc = a.K;
   if (kc < 1024) return fail(BP_ERR_UNSUPPORTED, "activation tile does not fit");
-  const size_t lds = X_BASE + (size_t)tokens * (kc * XB + 16);
+  const size_t lds = X_BASE + (size_t)tokens * (kc * XB + 16) + (size_t)(kc / 128) * 16 * MT * 4;
   static bool attr = false;
   if (!attr) {
     if (hipFuncSetAttribute((const void*)k_mfma_tq2<ACT, SDT, R, MT, WAVES, XKB, ABL>, hipFuncAttributeMaxDynamicSharedMemorySize,
@@ -318,7 +369,7 @@ int launch_tq2(const GemmArgs& a, hipStream_t s, const char* name) {
     attr = true;
   }
   note_kernel(name);
-  hipLaunchKernelGGL((k_mfma_tq2<ACT, SDT, R, MT, WAVES, XKB, ABL>), grid, dim3(WAVES * 64), lds, s, a, (int)kc);
+  hipLaunchKernelGGL((k_mfma_tq2<ACT, SDT, R, MT, WAVES, XKB, ABL>), grid, dim3(WAVES * 64), lds, s, a, (int)kc, (int)tokens);
   return check_launch(name);
 }
 

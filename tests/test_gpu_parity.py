@@ -188,6 +188,20 @@ def test_config1_decode_gemv_bf16(bp, fmt, N, K, M):
 
 
 @pytest.mark.parametrize("fmt", ["tq1", "tq2"])
+@pytest.mark.parametrize("M", [1, 16, 32])
+def test_config1_decode_gemv_int8(bp, fmt, M):
+    """Mode D activations (per-row int8) at config-1 size. K = 7168 is not a multiple of the K chunk the
+    kernels stage for 16 token rows, so the last chunk is a short one."""
+    N, K, group = 2048, 7168, 128
+    packed, scales = synth_weights(2, 1, N, K, group, fmt)
+    x = np.random.default_rng(40 + M).standard_normal((M, K)).astype(np.float32)
+    q, qs = orc.quant_act_int8(x)
+    want = c_gemm(q, qs, packed[0][0], scales[0][0].astype(np.float32), K, group, fmt)
+    got = bp.ternary_gemm(dev(q), dev(qs), dev(packed[0][0]), dev(scales[0][0]), K, group, fmt).cpu().numpy()
+    _check(got, want)
+
+
+@pytest.mark.parametrize("fmt", ["tq1", "tq2"])
 @pytest.mark.parametrize("act", ["int8", "bf16"])
 @pytest.mark.parametrize("K,group", [(256, 128), (640, 128), (200, 64), (1024, 256)])
 def test_ternary_linear_stacked_terms(bp, fmt, act, K, group):
