@@ -82,6 +82,17 @@ __device__ __forceinline__ u32x4 tq2_permute_i8(const u32x4 a) {
                __builtin_amdgcn_perm(s3, s1, 0x05040100u), __builtin_amdgcn_perm(s3, s1, 0x07060302u)};
 }
 
+// Weights and scales are read with raw buffer loads: a wave-uniform descriptor (base, byte range) in
+// scalar registers, a 32-bit lane offset and a scalar step offset, so a load needs no vector address
+// arithmetic, and a read past the range returns zeros instead of touching memory.
+__device__ __forceinline__ __amdgpu_buffer_rsrc_t make_rsrc(const void* base, int64_t bytes) {
+  const int n = bytes > 0x7fffffff ? 0x7fffffff : (int)bytes;
+  return __builtin_amdgcn_make_buffer_rsrc(const_cast<void*>(base), (short)0, n, 0x00020000);
+}
+__device__ __forceinline__ u32x4 buf_load16(__amdgpu_buffer_rsrc_t r, unsigned lane_off, unsigned wave_off) {
+  return __builtin_bit_cast(u32x4, __builtin_amdgcn_raw_buffer_load_b128(r, (int)lane_off, (int)wave_off, 0));
+}
+
 template <int ACT>
 struct Acc;
 template <>
@@ -92,7 +103,7 @@ struct Acc<BP_I8> { typedef i32x4 type; };
 template <int SDT>
 __device__ __forceinline__ float scale_at(const u32x4 (&raw)[2], int i) {  // i-th of the 8 scales held in raw
   if (SDT == BP_F32) return __uint_as_float(raw[i >> 2][i & 3]);
-  const unsigned v = raw[0][i >> 1];
+  const unsigned v = raw[i >> 3][(i >> 1) & 3];
   if (SDT == BP_F16) return f16_bits_to_f32((uint16_t)((i & 1) ? (v >> 16) : (v & 0xffffu)));
   return __uint_as_float((i & 1) ? (v & 0xffff0000u) : (v << 16));
 }
@@ -111,7 +122,8 @@ __global__ __launch_bounds__(WAVES * 64, 4) void k_mfma_tq2(GemmArgs a, int KC, 
   constexpr int NJ = 32 / KM;                  // MFMAs per group
   constexpr int XU = XKB * 1024 / (16 * XB) / THREADS;  // 16-element units of the activation tile per thread
 
-  const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+  // the wave index through readfirstlane: everything derived from it stays in scalar registers
+  const int wave = __builtin_amdgcn_readfirstlane((int)(threadIdx.x >> 6)), lane = threadIdx.x & 63;
   const int r16 = lane & 15, b = lane >> 4;
   const int64_t e = blockIdx.y;
   const int64_t o0 = clamp_i64(a.offsets[e], 0, a.T), o1 = clamp_i64(a.offsets[e + 1], 0, a.T);
@@ -213,30 +225,36 @@ __global__ __launch_bounds__(WAVES * 64, 4) void k_mfma_tq2(GemmArgs a, int KC, 
   asm volatile("" : "+s"(kc.P1), "+s"(kc.P2));
   asm volatile("" : "+v"(kc.M1), "+v"(kc.M2));
 
-  const int64_t steps = a.K / 256;
+  const int steps = (int)(a.K / 256);
   const int steps_per_chunk = KC / 256;
-  const int64_t chunks = (steps + steps_per_chunk - 1) / steps_per_chunk;
+  const int chunks = (steps + steps_per_chunk - 1) / steps_per_chunk;
 
   for (int term = 0; term < a.n_terms; ++term) {
-    const unsigned char* wbase = a.packed[term] + ((e * a.N + n0 + r16) * a.Kp + 16 * b);
-    const unsigned char* sbase = (const unsigned char*)a.w_scale[term] + (e * a.N + n0 + r16) * a.G * (SDT == BP_F32 ? 4 : 2);
+    // this wave's rows of the term as two buffers (R sub-tiles of 16 rows; rows past N are not in range)
+    constexpr int SB = SDT == BP_F32 ? 4 : 2;
+    const int64_t rows_here = a.N - n0 < 16 * R ? a.N - n0 : 16 * R;
+    const __amdgpu_buffer_rsrc_t wrs = make_rsrc(a.packed[term] + (e * a.N + n0) * a.Kp, rows_here * a.Kp);
+    const __amdgpu_buffer_rsrc_t srs = make_rsrc((const unsigned char*)a.w_scale[term] + (e * a.N + n0) * a.G * SB, rows_here * a.G * SB);
+    const unsigned woff = (unsigned)r16 * (unsigned)a.Kp + 16u * b;
+    const unsigned soff = (unsigned)r16 * (unsigned)a.G * SB;
     // Ring of PF steps of packed weights in flight per row sub-tile: with ~4 us of loaded HBM latency a CU
     // needs > 100 KiB of requests outstanding to stream at full rate (16 waves x PF x R KiB here).
-    constexpr int PF = 4;
+    constexpr int PF = ABL >= 10 ? 8 : 4;  // (8: timing experiments only; needs K % 2048 == 0 and 2-byte scales)
+    constexpr int AB = ABL % 10;
     u32x4 ring[PF][R];
     u32x4 sraw[R][2], snext[R][2];  // 8 scales (4 steps) per row sub-tile, and the next 8
-    auto fetch_w = [&](int64_t c, u32x4 (&dst)[R]) {
-      const int64_t cc = c < steps ? c : steps - 1;  // past the end: re-read the last step, no branch
+    auto fetch_w = [&](int c, u32x4 (&dst)[R]) {
+      const int cc = c < steps ? c : steps - 1;  // past the end: re-read the last step, no branch
 #pragma unroll
-      for (int r = 0; r < R; ++r) dst[r] = *(const u32x4*)(wbase + row_shift[r] * a.Kp + 64 * cc);
+      for (int r = 0; r < R; ++r) dst[r] = buf_load16(wrs, woff, (unsigned)(row_shift[r] * a.Kp) + 64u * cc);
     };
-    auto fetch_s = [&](int64_t c, u32x4 (&dst)[R][2]) {  // scales of steps c .. c+3 (c % 4 == 0)
-      const int64_t cc = c < steps ? c : 0;
+    auto fetch_s = [&](int c, u32x4 (&dst)[R][2]) {  // scales of steps c .. c+3 (c % 4 == 0)
+      const int cc = c < steps ? c : 0;
 #pragma unroll
       for (int r = 0; r < R; ++r) {
-        const unsigned char* p = sbase + (row_shift[r] * a.G + 2 * cc) * (SDT == BP_F32 ? 4 : 2);
-        dst[r][0] = *(const u32x4*)p;
-        if (SDT == BP_F32) dst[r][1] = *(const u32x4*)(p + 16);
+        const unsigned so = (unsigned)(row_shift[r] * a.G + 2 * cc) * SB;
+        dst[r][0] = buf_load16(srs, soff, so);
+        if (SDT == BP_F32 || PF == 8) dst[r][1] = buf_load16(srs, soff, so + 16);
       }
     };
     const bool restage = term == 0 || chunks > 1;  // a tile that holds all of K is staged once for all terms
@@ -250,24 +268,24 @@ __global__ __launch_bounds__(WAVES * 64, 4) void k_mfma_tq2(GemmArgs a, int KC, 
       fetch_w(i, ring[i]);
       __builtin_amdgcn_sched_barrier(0);
     }
-    for (int64_t ch = 0; ch < chunks; ++ch) {
+    for (int ch = 0; ch < chunks; ++ch) {
       if (restage) {
         __syncthreads();  // every wave is done reading the previous tile 
         stage_store();
         __syncthreads();
-        if (ch + 1 < chunks) stage_load((ch + 1) * KC);
+        if (ch + 1 < chunks) stage_load((int64_t)(ch + 1) * KC);
       }
-      const int64_t c_end = (ch + 1) * steps_per_chunk < steps ? (ch + 1) * steps_per_chunk : steps;
-      for (int64_t c4 = ch * steps_per_chunk; c4 < c_end; c4 += PF) {  // KC % 1024 == 0: whole blocks of 4 steps
+      const int c_end = (ch + 1) * steps_per_chunk < steps ? (ch + 1) * steps_per_chunk : steps;
+      for (int c4 = ch * steps_per_chunk; c4 < c_end; c4 += PF) {  // KC % 1024 == 0: whole blocks of 4 steps
 #pragma unroll
         for (int r = 0; r < R; ++r) { sraw[r][0] = snext[r][0]; sraw[r][1] = snext[r][1]; }
-        fetch_s(c4 + 4, snext);
+        fetch_s(c4 + PF, snext);
 #pragma unroll
         for (int i = 0; i < PF; ++i) {
           // One scheduling region per step: the wait for this step's weights stays here instead of joining
           // the waits of the later steps at the top of the block.
           __builtin_amdgcn_sched_barrier(0);
-          const int64_t c = c4 + i;
+          const int c = c4 + i;
           u32x4 w[R];
 #pragma unroll
           for (int r = 0; r < R; ++r) {  // regroup: .x/.y = 8 bytes of group 2c, .z/.w = 8 bytes of group 2c+1
@@ -276,9 +294,9 @@ __global__ __launch_bounds__(WAVES * 64, 4) void k_mfma_tq2(GemmArgs a, int KC, 
             w[r] = u32x4{s0[0], s1[0], s0[1], s1[1]};
           }
           fetch_w(c + PF, ring[i]);
-          const int gl = (int)(c - ch * steps_per_chunk) * 2;  // first of the step's two groups within the tile
+          const int gl = (c - ch * steps_per_chunk) * 2;  // first of the step's two groups within the tile
           const unsigned xoff = (unsigned)(gl * 128 * XB);
-          if (ABL == 1) {  // ablation (timing experiments only): memory traffic without decode and MFMA
+          if (AB == 1) {  // ablation (timing experiments only): memory traffic without decode and MFMA
 #pragma unroll
             for (int r = 0; r < R; ++r) total[r][0][0] += __uint_as_float((w[r].x ^ w[r].y ^ w[r].z ^ w[r].w) & 0x3fffffu);
             continue;
@@ -290,6 +308,12 @@ __global__ __launch_bounds__(WAVES * 64, 4) void k_mfma_tq2(GemmArgs a, int KC, 
             acc_t base[MT];
 #pragma unroll
             for (int mt = 0; mt < MT; ++mt) {
+              if (AB == 3) {  // ablation: no LDS operand reads
+                base[mt] = acc_t{0, 0, 0, 0};
+#pragma unroll
+                for (int j = 0; j < NJ; ++j) xa[j][mt] = u32x4{kc.M1, kc.M2, kc.M1, kc.M2};
+                continue;
+              }
               base[mt] = __builtin_bit_cast(acc_t, *(const lds_u32x4*)(corr_lane + ((gl + h) * (16 * MT) + 16 * mt) * 4));
 #pragma unroll
               for (int j = 0; j < NJ; ++j) xa[j][mt] = *(const lds_u32x4*)(xaddr[mt] + xoff + (h * 128 + j * KM) * XB);
@@ -298,7 +322,10 @@ __global__ __launch_bounds__(WAVES * 64, 4) void k_mfma_tq2(GemmArgs a, int KC, 
             for (int r = 0; r < R; ++r) {
               const unsigned lo = h == 0 ? w[r].x : w[r].z, hi = h == 0 ? w[r].y : w[r].w;
               u32x4 wb[NJ];
-              if (ACT == BP_BF16) {
+              if (AB == 4) {  // ablation: no decode
+#pragma unroll
+                for (int j = 0; j < NJ; ++j) wb[j] = u32x4{lo, hi, lo | kc.M1, hi | kc.M1};
+              } else if (ACT == BP_BF16) {
                 tq2_decode_bf16(lo, kc, wb[0], wb[1]);
                 tq2_decode_bf16(hi, kc, wb[NJ - 2], wb[NJ - 1]);
               } else {
@@ -311,6 +338,10 @@ __global__ __launch_bounds__(WAVES * 64, 4) void k_mfma_tq2(GemmArgs a, int KC, 
                 acc_t acc = base[mt];
 #pragma unroll
                 for (int j = 0; j < NJ; ++j) {
+                  if (AB == 2) {  // ablation: operands are produced but no MFMA is issued
+                    asm volatile("" ::"v"(xa[j][mt]), "v"(wb[j]));
+                    continue;
+                  }
                   if (ACT == BP_BF16)
                     acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, xa[j][mt]),
                                                                   __builtin_bit_cast(bf16x8, wb[j]), acc, 0, 0, 0);
@@ -804,9 +835,17 @@ int launch_mfma(const GemmArgs& a, hipStream_t s) {
     return fail(BP_ERR_UNSUPPORTED, "no tuned TQ1 kernel variant for this tiling");
   }
   if (const char* t = getenv("BP_TUNE_ABL")) {
-    if (atoi(t) == 1 && bf && a.scale_dtype == BP_F16 && MT == 1) {
-      if (R == 1) return launch_tq2<BP_BF16, BP_F16, 1, 1, 16, 48, 1>(a, s, "abl_r1_w16");
-      return launch_tq2<BP_BF16, BP_F16, 2, 1, 16, 48, 1>(a, s, "abl_r2_w16");
+    if (bf && a.scale_dtype == BP_F16 && MT == 1) {
+      switch (atoi(t)) {
+        case 1: return launch_tq2<BP_BF16, BP_F16, 1, 1, 16, 48, 1>(a, s, "abl1_w16");
+        case 2: return launch_tq2<BP_BF16, BP_F16, 1, 1, 16, 48, 2>(a, s, "abl2_w16");
+        case 3: return launch_tq2<BP_BF16, BP_F16, 1, 1, 16, 48, 3>(a, s, "abl3_w16");
+        case 4: return launch_tq2<BP_BF16, BP_F16, 1, 1, 16, 48, 4>(a, s, "abl4_w16");
+        case 10: return launch_tq2<BP_BF16, BP_F16, 1, 1, 16, 48, 10>(a, s, "abl10_w16");
+        case 11: return launch_tq2<BP_BF16, BP_F16, 1, 1, 16, 48, 11>(a, s, "abl11_w16");
+        case 14: return launch_tq2<BP_BF16, BP_F16, 1, 1, 16, 48, 14>(a, s, "abl14_w16");
+        default: break;
+      }
     }
   }
   if (MT == 2) waves = 16;  // the 32-token tile needs the large LDS budget of a 16-wave workgroup
