@@ -114,7 +114,7 @@ __device__ __forceinline__ float scale_at(const u32x4 (&raw)[2], int i) {  // i-
 // v_permlane32_swap pair then leaves every lane with 8 bytes of the first group and 8 bytes of the
 // second, so that all four k-blocks of an MFMA belong to one scale group.
 // After the swap block b holds trits tb(b) .. tb(b)+31 of each group, tb = {0, 64, 32, 96}.
-template <int ACT, int SDT, int R, int MT, int WAVES, int XKB, int ABL = 0>
+template <int ACT, int SDT, int R, int MT, int WAVES, int XKB, int ABL = 0, int NQ = 4>
 __global__ __launch_bounds__(WAVES * 64, 4) void k_mfma_tq2(GemmArgs a, int KC, int tile_rows) {
   constexpr int THREADS = WAVES * 64;
   constexpr int XB = ACT == BP_BF16 ? 2 : 1;   // bytes per activation element
@@ -241,12 +241,15 @@ __global__ __launch_bounds__(WAVES * 64, 4) void k_mfma_tq2(GemmArgs a, int KC, 
     // needs > 100 KiB of requests outstanding to stream at full rate (16 waves x PF x R KiB here).
     constexpr int PF = ABL >= 10 ? 8 : 4;  // (8: timing experiments only; needs K % 2048 == 0 and 2-byte scales)
     constexpr int AB = ABL % 10;
-    u32x4 ring[PF][R];
+    u32x4 ring[PF][R] = {};
     u32x4 sraw[R][2], snext[R][2];  // 8 scales (4 steps) per row sub-tile, and the next 8
     auto fetch_w = [&](int c, u32x4 (&dst)[R]) {
       const int cc = c < steps ? c : steps - 1;  // past the end: re-read the last step, no branch
 #pragma unroll
-      for (int r = 0; r < R; ++r) dst[r] = buf_load16(wrs, woff, (unsigned)(row_shift[r] * a.Kp) + 64u * cc);
+      for (int r = 0; r < R; ++r) {
+        if (AB == 5) { asm volatile("" : "+v"(dst[r])); continue; }  // ablation: no weight traffic
+        dst[r] = buf_load16(wrs, woff, (unsigned)(row_shift[r] * a.Kp) + 64u * cc);
+      }
     };
     auto fetch_s = [&](int c, u32x4 (&dst)[R][2]) {  // scales of steps c .. c+3 (c % 4 == 0)
       const int cc = c < steps ? c : 0;
@@ -293,10 +296,10 @@ __global__ __launch_bounds__(WAVES * 64, 4) void k_mfma_tq2(GemmArgs a, int KC, 
             const auto s1 = __builtin_amdgcn_permlane32_swap(ring[i][r].y, ring[i][r].w, false, false);
             w[r] = u32x4{s0[0], s1[0], s0[1], s1[1]};
           }
-          fetch_w(c + PF, ring[i]);
           const int gl = (c - ch * steps_per_chunk) * 2;  // first of the step's two groups within the tile
           const unsigned xoff = (unsigned)(gl * 128 * XB);
           if (AB == 1) {  // ablation (timing experiments only): memory traffic without decode and MFMA
+            fetch_w(c + PF, ring[i]);
 #pragma unroll
             for (int r = 0; r < R; ++r) total[r][0][0] += __uint_as_float((w[r].x ^ w[r].y ^ w[r].z ^ w[r].w) & 0x3fffffu);
             continue;
@@ -350,9 +353,17 @@ __global__ __launch_bounds__(WAVES * 64, 4) void k_mfma_tq2(GemmArgs a, int KC, 
                                                                 __builtin_bit_cast(i32x4, wb[j]), acc, 0, 0, 0);
                 }
 #pragma unroll
-                for (int q = 0; q < 4; ++q) total[r][mt][q] += (float)acc[q] * s;
+                for (int q = 0; q < NQ; ++q) total[r][mt][q] += (float)acc[q] * s;
               }
             }
+          }
+          // Ring slots are reloaded once consumed (in place: no register copies), two steps at a time and
+          // back to back: the two 64-byte halves of every 128-byte line then reach the L1 together and go
+          // to L2 as one request instead of two that each occupy a miss slot for the full latency.
+          __builtin_amdgcn_sched_barrier(0);
+          if (i & 1) {
+            fetch_w(c - 1 + PF, ring[i - 1]);
+            fetch_w(c + PF, ring[i]);
           }
         }
       }
@@ -362,7 +373,7 @@ __global__ __launch_bounds__(WAVES * 64, 4) void k_mfma_tq2(GemmArgs a, int KC, 
 #pragma unroll
   for (int mt = 0; mt < MT; ++mt) {
 #pragma unroll
-    for (int q = 0; q < 4; ++q) {
+    for (int q = 0; q < NQ; ++q) {  // NQ = 1: single-token launches keep only the sums of token 0
       const int t = 16 * mt + 4 * b + q;
       if (t < ntok) {
         const int64_t tok = tok0 + t;
@@ -379,7 +390,7 @@ __global__ __launch_bounds__(WAVES * 64, 4) void k_mfma_tq2(GemmArgs a, int KC, 
   }
 }
 
-template <int ACT, int SDT, int R, int MT, int WAVES, int XKB, int ABL = 0>
+template <int ACT, int SDT, int R, int MT, int WAVES, int XKB, int ABL = 0, int NQ = 4>
 int launch_tq2(const GemmArgs& a, hipStream_t s, const char* name) {
   constexpr int XB = ACT == BP_BF16 ? 2 : 1;
   const int64_t rows_per_wg = (int64_t)WAVES * 16 * R;
@@ -394,21 +405,21 @@ int launch_tq2(const GemmArgs& a, hipStream_t s, const char* name) {
   const size_t lds = X_BASE + (size_t)tokens * (kc * XB + 16) + (size_t)(kc / 128) * 16 * MT * 4;
   static bool attr = false;
   if (!attr) {
-    if (hipFuncSetAttribute((const void*)k_mfma_tq2<ACT, SDT, R, MT, WAVES, XKB, ABL>, hipFuncAttributeMaxDynamicSharedMemorySize,
+    if (hipFuncSetAttribute((const void*)k_mfma_tq2<ACT, SDT, R, MT, WAVES, XKB, ABL, NQ>, hipFuncAttributeMaxDynamicSharedMemorySize,
                             X_BASE + XKB * 1024) != hipSuccess)
       return fail(BP_ERR_LAUNCH, "cannot raise the dynamic LDS limit");
     attr = true;
   }
   note_kernel(name);
-  hipLaunchKernelGGL((k_mfma_tq2<ACT, SDT, R, MT, WAVES, XKB, ABL>), grid, dim3(WAVES * 64), lds, s, a, (int)kc, (int)tokens);
+  hipLaunchKernelGGL((k_mfma_tq2<ACT, SDT, R, MT, WAVES, XKB, ABL, NQ>), grid, dim3(WAVES * 64), lds, s, a, (int)kc, (int)tokens);
   return check_launch(name);
 }
 
-template <int ACT, int R, int MT, int WAVES, int XKB>
+template <int ACT, int R, int MT, int WAVES, int XKB, int NQ = 4>
 int launch_tq2_sd(const GemmArgs& a, hipStream_t s, const char* name) {
-  if (a.scale_dtype == BP_F16) return launch_tq2<ACT, BP_F16, R, MT, WAVES, XKB>(a, s, name);
-  if (a.scale_dtype == BP_BF16) return launch_tq2<ACT, BP_BF16, R, MT, WAVES, XKB>(a, s, name);
-  return launch_tq2<ACT, BP_F32, R, MT, WAVES, XKB>(a, s, name);
+  if (a.scale_dtype == BP_F16) return launch_tq2<ACT, BP_F16, R, MT, WAVES, XKB, 0, NQ>(a, s, name);
+  if (a.scale_dtype == BP_BF16) return launch_tq2<ACT, BP_BF16, R, MT, WAVES, XKB, 0, NQ>(a, s, name);
+  return launch_tq2<ACT, BP_F32, R, MT, WAVES, XKB, 0, NQ>(a, s, name);
 }
 
 // ------------------------------------------------------------------------------------------------
@@ -841,6 +852,7 @@ int launch_mfma(const GemmArgs& a, hipStream_t s) {
         case 2: return launch_tq2<BP_BF16, BP_F16, 1, 1, 16, 48, 2>(a, s, "abl2_w16");
         case 3: return launch_tq2<BP_BF16, BP_F16, 1, 1, 16, 48, 3>(a, s, "abl3_w16");
         case 4: return launch_tq2<BP_BF16, BP_F16, 1, 1, 16, 48, 4>(a, s, "abl4_w16");
+        case 5: return launch_tq2<BP_BF16, BP_F16, 1, 1, 16, 48, 5>(a, s, "abl5_w16");
         case 10: return launch_tq2<BP_BF16, BP_F16, 1, 1, 16, 48, 10>(a, s, "abl10_w16");
         case 11: return launch_tq2<BP_BF16, BP_F16, 1, 1, 16, 48, 11>(a, s, "abl11_w16");
         case 14: return launch_tq2<BP_BF16, BP_F16, 1, 1, 16, 48, 14>(a, s, "abl14_w16");
@@ -849,6 +861,18 @@ int launch_mfma(const GemmArgs& a, hipStream_t s) {
     }
   }
   if (MT == 2) waves = 16;  // the 32-token tile needs the large LDS budget of a 16-wave workgroup
+  if (a.max_rows == 1 && R == 2 && MT == 1 && waves == 16) {
+    if (bf) return launch_tq2_sd<BP_BF16, 2, 1, 16, 48, 1>(a, s, "mfma_tq2_bf16_r2_t1_w16");
+    return launch_tq2_sd<BP_I8, 2, 1, 16, 48, 1>(a, s, "mfma_tq2_i8_r2_t1_w16");
+  }
+  if (a.max_rows == 1 && R == 1 && MT == 1) {  // decode GEMV: one token, only its sums are scaled and kept
+    if (bf) {
+      if (waves == 16) return launch_tq2_sd<BP_BF16, 1, 1, 16, 48, 1>(a, s, "mfma_tq2_bf16_r1_t1_w16");
+      return launch_tq2_sd<BP_BF16, 1, 1, 8, 48, 1>(a, s, "mfma_tq2_bf16_r1_t1_w8");
+    }
+    if (waves == 16) return launch_tq2_sd<BP_I8, 1, 1, 16, 48, 1>(a, s, "mfma_tq2_i8_r1_t1_w16");
+    return launch_tq2_sd<BP_I8, 1, 1, 8, 48, 1>(a, s, "mfma_tq2_i8_r1_t1_w8");
+  }
 #define BP_CASE(ACTV, RV, MTV, WV, XK, NAME) \
   if (R == RV && MT == MTV && waves == WV) return launch_tq2_sd<ACTV, RV, MTV, WV, XK>(a, s, NAME "_r" #RV "_m" #MTV "_w" #WV);
 #define BP_ALL(ACTV, NAME)                                                        \
