@@ -37,6 +37,7 @@ typedef __attribute__((address_space(3))) unsigned lds_u32;
 // requested at launch starts at LDS address 0.
 // TQ2: the activation tile starts at 0: row t at t * pitch, pitch = KC * XB + 16.
 constexpr int X_BASE = 0;
+constexpr int TQ2_SCALE_TILE_MAX = 40 * 1024;  // LDS budget for a workgroup's scales (beyond it: read from global memory)
 constexpr int X_TILE_BYTES = 48 * 1024;  // TQ1: table + tile = 80 KiB: two workgroups of 8 waves per CU
 
 __device__ __forceinline__ unsigned bf16_of_trit(int t) {
@@ -114,7 +115,7 @@ __device__ __forceinline__ float scale_at(const u32x4 (&raw)[2], int i) {  // i-
 // v_permlane32_swap pair then leaves every lane with 8 bytes of the first group and 8 bytes of the
 // second, so that all four k-blocks of an MFMA belong to one scale group.
 // After the swap block b holds trits tb(b) .. tb(b)+31 of each group, tb = {0, 64, 32, 96}.
-template <int ACT, int SDT, int R, int MT, int WAVES, int XKB, int ABL = 0, int NQ = 4>
+template <int ACT, int SDT, int R, int MT, int WAVES, int XKB, int ABL = 0, int NQ = 4, int SL = 1>
 __global__ __launch_bounds__(WAVES * 64, 4) void k_mfma_tq2(GemmArgs a, int KC, int tile_rows) {
   constexpr int THREADS = WAVES * 64;
   constexpr int XB = ACT == BP_BF16 ? 2 : 1;   // bytes per activation element
@@ -237,17 +238,30 @@ __global__ __launch_bounds__(WAVES * 64, 4) void k_mfma_tq2(GemmArgs a, int KC, 
     const __amdgpu_buffer_rsrc_t srs = make_rsrc((const unsigned char*)a.w_scale[term] + (e * a.N + n0) * a.G * SB, rows_here * a.G * SB);
     const unsigned woff = (unsigned)r16 * (unsigned)a.Kp + 16u * b;
     const unsigned soff = (unsigned)r16 * (unsigned)a.G * SB;
+    // SL: the scales of the workgroup's rows (all of K, one term) are copied into LDS once, as full cache
+    // lines; read row by row from global memory, every 16-byte piece would be an L1 miss of its own.
+    const unsigned stile = corr_base + (unsigned)((KC / 128) * 16 * MT * 4);
+    const unsigned slane = stile + (unsigned)((wave * 16 * R + r16) * (int)a.G * SB);
+    auto stage_scales = [&]() {
+      const int64_t wg_row0 = (int64_t)blockIdx.x * (WAVES * 16 * R);
+      const int64_t wg_rows = a.N - wg_row0 < WAVES * 16 * R ? a.N - wg_row0 : WAVES * 16 * R;
+      const unsigned char* src = (const unsigned char*)a.w_scale[term] + (e * a.N + wg_row0) * a.G * SB;
+      const int units16 = (int)(wg_rows * a.G * SB / 16);
+      if (term > 0) __syncthreads();  // the previous term's scales are no longer read
+      for (int u = threadIdx.x; u < units16; u += THREADS) *(lds_u32x4*)(stile + 16 * u) = *(const u32x4*)(src + 16 * (int64_t)u);
+      __syncthreads();
+    };
     // Ring of PF steps of packed weights in flight per row sub-tile: with ~4 us of loaded HBM latency a CU
     // needs > 100 KiB of requests outstanding to stream at full rate (16 waves x PF x R KiB here).
-    constexpr int PF = ABL >= 10 ? 8 : 4;  // (8: timing experiments only; needs K % 2048 == 0 and 2-byte scales)
-    constexpr int AB = ABL % 10;
+    constexpr int PF = ABL >= 100 ? 8 : 4;  // (8: timing experiments only; needs K % 2048 == 0 and 2-byte scales)
+    constexpr int AB = ABL % 10, AB2 = ABL / 10 % 10;  // up to two ablations at once
     u32x4 ring[PF][R] = {};
     u32x4 sraw[R][2], snext[R][2];  // 8 scales (4 steps) per row sub-tile, and the next 8
     auto fetch_w = [&](int c, u32x4 (&dst)[R]) {
       const int cc = c < steps ? c : steps - 1;  // past the end: re-read the last step, no branch
 #pragma unroll
       for (int r = 0; r < R; ++r) {
-        if (AB == 5) { asm volatile("" : "+v"(dst[r])); continue; }  // ablation: no weight traffic
+        if (AB == 5 || AB2 == 5) { asm volatile("" : "+v"(dst[r])); continue; }  // ablation: no weight traffic
         dst[r] = buf_load16(wrs, woff, (unsigned)(row_shift[r] * a.Kp) + 64u * cc);
       }
     };
@@ -256,6 +270,11 @@ __global__ __launch_bounds__(WAVES * 64, 4) void k_mfma_tq2(GemmArgs a, int KC, 
 #pragma unroll
       for (int r = 0; r < R; ++r) {
         const unsigned so = (unsigned)(row_shift[r] * a.G + 2 * cc) * SB;
+        if (SL) {
+          dst[r][0] = *(const lds_u32x4*)(slane + so);
+          if (SDT == BP_F32 || PF == 8) dst[r][1] = *(const lds_u32x4*)(slane + so + 16);
+          continue;
+        }
         dst[r][0] = buf_load16(srs, soff, so);
         if (SDT == BP_F32 || PF == 8) dst[r][1] = buf_load16(srs, soff, so + 16);
       }
@@ -264,12 +283,16 @@ __global__ __launch_bounds__(WAVES * 64, 4) void k_mfma_tq2(GemmArgs a, int KC, 
     if (restage) stage_load(0);
     // Same issue order as inside the loop (scales, then the weights step by step), pinned with scheduling
     // barriers: loads return in order, so the loop's waits can then leave the younger loads in flight.
-    fetch_s(0, snext);
+    if (!SL) fetch_s(0, snext);
     __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
     for (int i = 0; i < PF; ++i) {
       fetch_w(i, ring[i]);
       __builtin_amdgcn_sched_barrier(0);
+    }
+    if (SL) {  // behind the loads above, so that their latencies overlap with the copy's
+      stage_scales();
+      fetch_s(0, snext);
     }
     for (int ch = 0; ch < chunks; ++ch) {
       if (restage) {
@@ -311,7 +334,7 @@ __global__ __launch_bounds__(WAVES * 64, 4) void k_mfma_tq2(GemmArgs a, int KC, 
             acc_t base[MT];
 #pragma unroll
             for (int mt = 0; mt < MT; ++mt) {
-              if (AB == 3) {  // ablation: no LDS operand reads
+              if (AB == 3 || AB2 == 3) {  // ablation: no LDS operand reads
                 base[mt] = acc_t{0, 0, 0, 0};
 #pragma unroll
                 for (int j = 0; j < NJ; ++j) xa[j][mt] = u32x4{kc.M1, kc.M2, kc.M1, kc.M2};
@@ -325,7 +348,7 @@ __global__ __launch_bounds__(WAVES * 64, 4) void k_mfma_tq2(GemmArgs a, int KC, 
             for (int r = 0; r < R; ++r) {
               const unsigned lo = h == 0 ? w[r].x : w[r].z, hi = h == 0 ? w[r].y : w[r].w;
               u32x4 wb[NJ];
-              if (AB == 4) {  // ablation: no decode
+              if (AB == 4 || AB2 == 4) {  // ablation: no decode
 #pragma unroll
                 for (int j = 0; j < NJ; ++j) wb[j] = u32x4{lo, hi, lo | kc.M1, hi | kc.M1};
               } else if (ACT == BP_BF16) {
@@ -341,7 +364,7 @@ __global__ __launch_bounds__(WAVES * 64, 4) void k_mfma_tq2(GemmArgs a, int KC, 
                 acc_t acc = base[mt];
 #pragma unroll
                 for (int j = 0; j < NJ; ++j) {
-                  if (AB == 2) {  // ablation: operands are produced but no MFMA is issued
+                  if (AB == 2 || AB2 == 2) {  // ablation: operands are produced but no MFMA is issued
                     asm volatile("" ::"v"(xa[j][mt]), "v"(wb[j]));
                     continue;
                   }
@@ -390,7 +413,7 @@ __global__ __launch_bounds__(WAVES * 64, 4) void k_mfma_tq2(GemmArgs a, int KC, 
   }
 }
 
-template <int ACT, int SDT, int R, int MT, int WAVES, int XKB, int ABL = 0, int NQ = 4>
+template <int ACT, int SDT, int R, int MT, int WAVES, int XKB, int ABL = 0, int NQ = 4, int SL = 1>
 int launch_tq2(const GemmArgs& a, hipStream_t s, const char* name) {
   constexpr int XB = ACT == BP_BF16 ? 2 : 1;
   const int64_t rows_per_wg = (int64_t)WAVES * 16 * R;
@@ -402,24 +425,32 @@ int launch_tq2(const GemmArgs& a, hipStream_t s, const char* name) {
   int64_t kc = 2 * (XKB * 1024 - 16 * tokens) / (2 * tokens * XB + MT) / 1024 * 1024;
   if (kc > a.K) kc = a.K;
   if (kc < 1024) return fail(BP_ERR_UNSUPPORTED, "activation tile does not fit");
-  const size_t lds = X_BASE + (size_t)tokens * (kc * XB + 16) + (size_t)(kc / 128) * 16 * MT * 4;
+  const size_t stile = SL ? (size_t)rows_per_wg * a.G * (SDT == BP_F32 ? 4 : 2) : 0;
+  const size_t lds = X_BASE + (size_t)tokens * (kc * XB + 16) + (size_t)(kc / 128) * 16 * MT * 4 + stile;
   static bool attr = false;
   if (!attr) {
-    if (hipFuncSetAttribute((const void*)k_mfma_tq2<ACT, SDT, R, MT, WAVES, XKB, ABL, NQ>, hipFuncAttributeMaxDynamicSharedMemorySize,
-                            X_BASE + XKB * 1024) != hipSuccess)
+    if (hipFuncSetAttribute((const void*)k_mfma_tq2<ACT, SDT, R, MT, WAVES, XKB, ABL, NQ, SL>, hipFuncAttributeMaxDynamicSharedMemorySize,
+                            X_BASE + XKB * 1024 + (SL ? TQ2_SCALE_TILE_MAX : 0)) != hipSuccess)
       return fail(BP_ERR_LAUNCH, "cannot raise the dynamic LDS limit");
     attr = true;
   }
   note_kernel(name);
-  hipLaunchKernelGGL((k_mfma_tq2<ACT, SDT, R, MT, WAVES, XKB, ABL, NQ>), grid, dim3(WAVES * 64), lds, s, a, (int)kc, (int)tokens);
+  hipLaunchKernelGGL((k_mfma_tq2<ACT, SDT, R, MT, WAVES, XKB, ABL, NQ, SL>), grid, dim3(WAVES * 64), lds, s, a, (int)kc, (int)tokens);
   return check_launch(name);
 }
 
 template <int ACT, int R, int MT, int WAVES, int XKB, int NQ = 4>
 int launch_tq2_sd(const GemmArgs& a, hipStream_t s, const char* name) {
-  if (a.scale_dtype == BP_F16) return launch_tq2<ACT, BP_F16, R, MT, WAVES, XKB, 0, NQ>(a, s, name);
-  if (a.scale_dtype == BP_BF16) return launch_tq2<ACT, BP_BF16, R, MT, WAVES, XKB, 0, NQ>(a, s, name);
-  return launch_tq2<ACT, BP_F32, R, MT, WAVES, XKB, 0, NQ>(a, s, name);
+  // scales through LDS whenever the workgroup's share of one term fits the budget
+  const int64_t tile = (int64_t)WAVES * 16 * R * a.G * (a.scale_dtype == BP_F32 ? 4 : 2);
+  if (tile <= TQ2_SCALE_TILE_MAX) {
+    if (a.scale_dtype == BP_F16) return launch_tq2<ACT, BP_F16, R, MT, WAVES, XKB, 0, NQ, 1>(a, s, name);
+    if (a.scale_dtype == BP_BF16) return launch_tq2<ACT, BP_BF16, R, MT, WAVES, XKB, 0, NQ, 1>(a, s, name);
+    return launch_tq2<ACT, BP_F32, R, MT, WAVES, XKB, 0, NQ, 1>(a, s, name);
+  }
+  if (a.scale_dtype == BP_F16) return launch_tq2<ACT, BP_F16, R, MT, WAVES, XKB, 0, NQ, 0>(a, s, name);
+  if (a.scale_dtype == BP_BF16) return launch_tq2<ACT, BP_BF16, R, MT, WAVES, XKB, 0, NQ, 0>(a, s, name);
+  return launch_tq2<ACT, BP_F32, R, MT, WAVES, XKB, 0, NQ, 0>(a, s, name);
 }
 
 // ------------------------------------------------------------------------------------------------
@@ -829,7 +860,9 @@ int launch_mfma(const GemmArgs& a, hipStream_t s) {
   const int64_t work = a.E * (a.N / 16);
   int R = 1;  // two row sub-tiles per wave spill registers at 4 waves per SIMD; see BP_TUNE_R
   int MT = a.max_rows > 16 ? 2 : 1;
-  int waves = work >= 2048 ? 16 : 8;
+  // 8-wave workgroups run two to a CU, so one's start-up (staging, first loads) overlaps the other's
+  // steady state; the TQ2 single-token kernels are light enough on registers for that to win everywhere.
+  int waves = work >= 2048 && !(a.fmt == BP_TQ2 && a.max_rows == 1) ? 16 : 8;
   if (const char* t = getenv("BP_TUNE_R")) { const int v = atoi(t); if (v == 1 || v == 2) R = v; }
   if (const char* t = getenv("BP_TUNE_WAVES")) { const int v = atoi(t); if (v == 8 || v == 16) waves = v; }
   if (const char* t = getenv("BP_TUNE_MT")) { const int v = atoi(t); if (v == 1 || v == 2) MT = v; }
@@ -853,9 +886,10 @@ int launch_mfma(const GemmArgs& a, hipStream_t s) {
         case 3: return launch_tq2<BP_BF16, BP_F16, 1, 1, 16, 48, 3>(a, s, "abl3_w16");
         case 4: return launch_tq2<BP_BF16, BP_F16, 1, 1, 16, 48, 4>(a, s, "abl4_w16");
         case 5: return launch_tq2<BP_BF16, BP_F16, 1, 1, 16, 48, 5>(a, s, "abl5_w16");
-        case 10: return launch_tq2<BP_BF16, BP_F16, 1, 1, 16, 48, 10>(a, s, "abl10_w16");
-        case 11: return launch_tq2<BP_BF16, BP_F16, 1, 1, 16, 48, 11>(a, s, "abl11_w16");
-        case 14: return launch_tq2<BP_BF16, BP_F16, 1, 1, 16, 48, 14>(a, s, "abl14_w16");
+        case 25: return launch_tq2<BP_BF16, BP_F16, 1, 1, 16, 48, 25>(a, s, "abl25_w16");
+        case 35: return launch_tq2<BP_BF16, BP_F16, 1, 1, 16, 48, 35>(a, s, "abl35_w16");
+        case 45: return launch_tq2<BP_BF16, BP_F16, 1, 1, 16, 48, 45>(a, s, "abl45_w16");
+        case 100: return launch_tq2<BP_BF16, BP_F16, 1, 1, 16, 48, 100>(a, s, "abl100_w16");
         default: break;
       }
     }
