@@ -1,0 +1,65 @@
+// Shared pieces of the tuned gfx950 MFMA kernels (bp_mfma_tq2.hip, bp_mfma_tq1.hip).
+//
+// Packed trits are decoded in registers straight into MFMA operands, one 16-row x 16-token tile per
+// instruction (v_mfma_f32_16x16x32_bf16 for bf16 activations, v_mfma_i32_16x16x64_i8 for int8).
+// Accumulators are flushed at every 128-wide K group: total += acc * scale[n, g] in float32, so the
+// scale multiplies the group sum exactly as in the reference contract
+// (boilerplate/kernels/ternary_cuda.py:58-63, boilerplate/kernels/csrc/boilerplate_cpu.cpp:114-124).
+// Stacked terms share one staging of the activations and one output write.
+//
+// Operand A = activations (row i = token), operand B = weights (column j = output row), so a lane
+// ends with 4 tokens x 1 output row and needs one scale per group.
+//
+// The kernels address LDS absolutely: they declare no static LDS, so the dynamic allocation requested
+// at launch starts at LDS address 0.
+#pragma once
+#include <cstdlib>
+
+#include "bp_common.h"
+
+namespace bp {
+
+// implemented in bp_mfma_tq2.hip / bp_mfma_tq1.hip; R, MT, waves: the tiling chosen by launch_mfma
+int launch_mfma_tq2(const GemmArgs& a, hipStream_t s, int R, int MT, int waves);
+int launch_mfma_tq1(const GemmArgs& a, hipStream_t s, int waves);
+
+namespace {
+
+typedef unsigned u32x2 __attribute__((ext_vector_type(2)));
+typedef unsigned u32x4 __attribute__((ext_vector_type(4)));
+typedef float f32x4 __attribute__((ext_vector_type(4)));
+typedef int i32x4 __attribute__((ext_vector_type(4)));
+typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
+typedef __bf16 bf16x2 __attribute__((ext_vector_type(2)));
+typedef __attribute__((address_space(3))) u32x2 lds_u32x2;
+typedef __attribute__((address_space(3))) u32x4 lds_u32x4;
+typedef __attribute__((address_space(3))) unsigned lds_u32;
+
+// Weights and scales are read with raw buffer loads: a wave-uniform descriptor (base, byte range) in
+// scalar registers, a 32-bit lane offset and a scalar step offset, so a load needs no vector address
+// arithmetic, and a read past the range returns zeros instead of touching memory.
+__device__ __forceinline__ __amdgpu_buffer_rsrc_t make_rsrc(const void* base, int64_t bytes) {
+  const int n = bytes > 0x7fffffff ? 0x7fffffff : (int)bytes;
+  return __builtin_amdgcn_make_buffer_rsrc(const_cast<void*>(base), (short)0, n, 0x00020000);
+}
+__device__ __forceinline__ u32x4 buf_load16(__amdgpu_buffer_rsrc_t r, unsigned lane_off, unsigned wave_off) {
+  return __builtin_bit_cast(u32x4, __builtin_amdgcn_raw_buffer_load_b128(r, (int)lane_off, (int)wave_off, 0));
+}
+
+template <int ACT>
+struct Acc;
+template <>
+struct Acc<BP_BF16> { typedef f32x4 type; };
+template <>
+struct Acc<BP_I8> { typedef i32x4 type; };
+
+template <int SDT>
+__device__ __forceinline__ float scale_at(const u32x4 (&raw)[2], int i) {  // i-th of the 8 scales held in raw
+  if (SDT == BP_F32) return __uint_as_float(raw[i >> 2][i & 3]);
+  const unsigned v = raw[i >> 3][(i >> 1) & 3];
+  if (SDT == BP_F16) return f16_bits_to_f32((uint16_t)((i & 1) ? (v >> 16) : (v & 0xffffu)));
+  return __uint_as_float((i & 1) ? (v & 0xffff0000u) : (v << 16));
+}
+
+}  // namespace
+}  // namespace bp

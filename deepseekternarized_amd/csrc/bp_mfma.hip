@@ -1,837 +1,7 @@
-// Tuned gfx950 kernels for group = 128: packed trits are decoded in registers (TQ2: bit arithmetic,
-// TQ1: a bank-replicated LDS table) straight into MFMA operands, one 16-row x 16-token tile per
-// instruction.
-//
-//   bf16 activations : v_mfma_f32_16x16x32_bf16
-//   int8 activations : v_mfma_i32_16x16x64_i8 (TQ2 only)
-//
-// Accumulators are flushed at every 128-wide K group: total += acc * scale[n, g] in float32, so the
-// scale multiplies the group sum exactly as in the reference contract
-// (boilerplate/kernels/ternary_cuda.py:58-63, boilerplate/kernels/csrc/boilerplate_cpu.cpp:114-124).
-// Stacked terms share one staging of the activations and one output write.
-//
-// Work split: a workgroup of WAVES wavefronts owns WAVES*16*R output rows of one expert and 16*MT of
-// its token rows. The activation tile of the workgroup is staged through LDS in K chunks (global
-// loads one chunk ahead, held in registers across the compute of the current chunk), the packed
-// weights stream from HBM exactly once with loads two steps ahead. Operand A = activations (row i =
-// token), operand B = weights (column j = output row), so a lane ends with 4 tokens x 1 output row
-// and needs one scale per group.
-#include <cstdlib>
-
-#include "bp_common.h"
+// Dispatch of the tuned gfx950 MFMA kernels for group = 128.
+#include "bp_mfma.h"
 
 namespace bp {
-namespace {
-
-typedef unsigned u32x2 __attribute__((ext_vector_type(2)));
-typedef unsigned u32x4 __attribute__((ext_vector_type(4)));
-typedef float f32x4 __attribute__((ext_vector_type(4)));
-typedef int i32x4 __attribute__((ext_vector_type(4)));
-typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
-typedef __bf16 bf16x2 __attribute__((ext_vector_type(2)));
-typedef __attribute__((address_space(3))) u32x2 lds_u32x2;
-typedef __attribute__((address_space(3))) u32x4 lds_u32x4;
-typedef __attribute__((address_space(3))) unsigned lds_u32;
-
-// These kernels address LDS absolutely: they declare no static LDS, so the dynamic allocation
-// requested at launch starts at LDS address 0.
-// TQ2: the activation tile starts at 0: row t at t * pitch, pitch = KC * XB + 16.
-constexpr int X_BASE = 0;
-constexpr int TQ2_SCALE_TILE_MAX = 40 * 1024;  // LDS budget for a workgroup's scales (beyond it: read from global memory)
-constexpr int X_TILE_BYTES = 48 * 1024;  // TQ1: table + tile = 80 KiB: two workgroups of 8 waves per CU
-
-__device__ __forceinline__ unsigned bf16_of_trit(int t) {
-  return t == 0 ? 0u : t == 1 ? 0x3f80u : t == -1 ? 0xbf80u : 0x4000u;  // +2 (TQ2 code 3) -> 2.0
-}
-
-// ---- TQ2 decode without a table.
-// bf16: a 2-bit code u placed at bits [7:6] of a bf16 whose other bits are 0x4000 reads 2 + u (the code
-// spans the lowest exponent bit and the highest mantissa bit: 2, 3, 4); placed at bits [5:4] of 0x4100 it
-// reads 8 + u. One v_and_or_b32 per output dword therefore turns two codes of a packed dword (one per
-// 16-bit half) into two bf16 values; three shifts bring all 16 codes of the dword to those two positions.
-// The products then carry sum(x * (c + u)) with c = 2 (odd trits) or 8 (even trits); the accumulator of
-// every group starts from -sum(x * (c + 1)), computed once per workgroup when the activation tile is
-// staged, which leaves sum(x * (u - 1)). Slot order of the two operands made from a packed dword (codes
-// c0..c15, lo/hi bf16 of each operand dword):
-//   first  : (c3,c11) (c2,c10) (c1,c9) (c0,c8)      second : (c5,c13) (c4,c12) (c7,c15) (c6,c14)
-// The activation tile is stored in LDS in that order (permuted inside every 16 elements when staged).
-// The unused code 3 reads +3 or +2 depending on its slot (pack never writes it).
-struct Tq2Consts { unsigned P1, P2, M1, M2; };  // 0x00c000c0, 0x00300030, 0x40004000, 0x41004100 held in registers
-__device__ __forceinline__ void tq2_decode_bf16(unsigned w, const Tq2Consts& k, u32x4& first, u32x4& second) {
-  const unsigned P1 = k.P1, P2 = k.P2, M1 = k.M1, M2 = k.M2;
-  const unsigned wl = w << 4, wr = w >> 4, wr8 = w >> 8;
-  first = u32x4{(w & P1) | M1, (w & P2) | M2, (wl & P1) | M1, (wl & P2) | M2};
-  second = u32x4{(wr & P1) | M1, (wr & P2) | M2, (wr8 & P1) | M1, (wr8 & P2) | M2};
-}
-// int8: dword i of the operand = codes c(i), c(i+4), c(i+8), c(i+12) as digits 0..2; the accumulator
-// starts from -sum(x). The activation tile is stored with every 16 bytes transposed 4 x 4 to match.
-__device__ __forceinline__ u32x4 tq2_decode_i8(unsigned w) {
-  const unsigned m = 0x03030303u;
-  return u32x4{w & m, (w >> 2) & m, (w >> 4) & m, (w >> 6) & m};
-}
-__device__ __forceinline__ void tq2_permute_bf16(const u32x4 a, const u32x4 c, u32x4& o0, u32x4& o1) {
-  const unsigned HI = 0x07060302u, LO = 0x05040100u;
-  o0 = u32x4{__builtin_amdgcn_perm(c.y, a.y, HI), __builtin_amdgcn_perm(c.y, a.y, LO),
-             __builtin_amdgcn_perm(c.x, a.x, HI), __builtin_amdgcn_perm(c.x, a.x, LO)};
-  o1 = u32x4{__builtin_amdgcn_perm(c.z, a.z, HI), __builtin_amdgcn_perm(c.z, a.z, LO),
-             __builtin_amdgcn_perm(c.w, a.w, HI), __builtin_amdgcn_perm(c.w, a.w, LO)};
-}
-__device__ __forceinline__ u32x4 tq2_permute_i8(const u32x4 a) {
-  const unsigned s0 = __builtin_amdgcn_perm(a.y, a.x, 0x05010400u), s1 = __builtin_amdgcn_perm(a.y, a.x, 0x07030602u);
-  const unsigned s2 = __builtin_amdgcn_perm(a.w, a.z, 0x05010400u), s3 = __builtin_amdgcn_perm(a.w, a.z, 0x07030602u);
-  return u32x4{__builtin_amdgcn_perm(s2, s0, 0x05040100u), __builtin_amdgcn_perm(s2, s0, 0x07060302u),
-               __builtin_amdgcn_perm(s3, s1, 0x05040100u), __builtin_amdgcn_perm(s3, s1, 0x07060302u)};
-}
-
-// Weights and scales are read with raw buffer loads: a wave-uniform descriptor (base, byte range) in
-// scalar registers, a 32-bit lane offset and a scalar step offset, so a load needs no vector address
-// arithmetic, and a read past the range returns zeros instead of touching memory.
-__device__ __forceinline__ __amdgpu_buffer_rsrc_t make_rsrc(const void* base, int64_t bytes) {
-  const int n = bytes > 0x7fffffff ? 0x7fffffff : (int)bytes;
-  return __builtin_amdgcn_make_buffer_rsrc(const_cast<void*>(base), (short)0, n, 0x00020000);
-}
-__device__ __forceinline__ u32x4 buf_load16(__amdgpu_buffer_rsrc_t r, unsigned lane_off, unsigned wave_off) {
-  return __builtin_bit_cast(u32x4, __builtin_amdgcn_raw_buffer_load_b128(r, (int)lane_off, (int)wave_off, 0));
-}
-
-template <int ACT>
-struct Acc;
-template <>
-struct Acc<BP_BF16> { typedef f32x4 type; };
-template <>
-struct Acc<BP_I8> { typedef i32x4 type; };
-
-template <int SDT>
-__device__ __forceinline__ float scale_at(const u32x4 (&raw)[2], int i) {  // i-th of the 8 scales held in raw
-  if (SDT == BP_F32) return __uint_as_float(raw[i >> 2][i & 3]);
-  const unsigned v = raw[i >> 3][(i >> 1) & 3];
-  if (SDT == BP_F16) return f16_bits_to_f32((uint16_t)((i & 1) ? (v >> 16) : (v & 0xffffu)));
-  return __uint_as_float((i & 1) ? (v & 0xffff0000u) : (v << 16));
-}
-
-// ------------------------------------------------------------------------------------------------
-// TQ2. K % 1024 == 0, N % 16 == 0. One step = 64 packed bytes (256 trits, two groups) per row.
-// Lane (r16 = lane % 16, b = lane / 16) loads bytes [16b, 16b + 16) of its row's 64-byte piece; a
-// v_permlane32_swap pair then leaves every lane with 8 bytes of the first group and 8 bytes of the
-// second, so that all four k-blocks of an MFMA belong to one scale group.
-// After the swap block b holds trits tb(b) .. tb(b)+31 of each group, tb = {0, 64, 32, 96}.
-template <int ACT, int SDT, int R, int MT, int WAVES, int XKB, int ABL = 0, int NQ = 4, int SL = 1>
-__global__ __launch_bounds__(WAVES * 64, 4) void k_mfma_tq2(GemmArgs a, int KC, int tile_rows) {
-  constexpr int THREADS = WAVES * 64;
-  constexpr int XB = ACT == BP_BF16 ? 2 : 1;   // bytes per activation element
-  constexpr int KM = ACT == BP_BF16 ? 8 : 16;  // k per lane per MFMA
-  constexpr int NJ = 32 / KM;                  // MFMAs per group
-  constexpr int XU = XKB * 1024 / (16 * XB) / THREADS;  // 16-element units of the activation tile per thread
-
-  // the wave index through readfirstlane: everything derived from it stays in scalar registers
-  const int wave = __builtin_amdgcn_readfirstlane((int)(threadIdx.x >> 6)), lane = threadIdx.x & 63;
-  const int r16 = lane & 15, b = lane >> 4;
-  const int64_t e = blockIdx.y;
-  const int64_t o0 = clamp_i64(a.offsets[e], 0, a.T), o1 = clamp_i64(a.offsets[e + 1], 0, a.T);
-  const int64_t tok0 = o0 + (int64_t)blockIdx.z * (16 * MT);
-  if (tok0 >= o1) return;  // uniform for the workgroup: no barrier is skipped by part of it
-  const int ntok = (int)(o1 - tok0 < 16 * MT ? o1 - tok0 : 16 * MT);
-  int64_t n0 = ((int64_t)blockIdx.x * WAVES + wave) * (16 * R);
-  const bool wave_live = n0 < a.N;
-  if (!wave_live) n0 = 0;  // keeps addresses valid; the wave still takes part in staging and barriers
-  const int tb = 64 * (b & 1) + 32 * (b >> 1);
-
-  // row sub-tiles past N re-read the first sub-tile (branch-free loop body) and are dropped at the store
-  bool rows_valid[R];
-  int64_t row_shift[R];
-#pragma unroll
-  for (int r = 0; r < R; ++r) {
-    rows_valid[r] = wave_live && n0 + 16 * r < a.N;
-    row_shift[r] = rows_valid[r] ? 16 * r : 0;
-  }
-
-  // ---- activation tile geometry
-  const int pitch = KC * XB + 16;
-  const int units_per_row = KC / 16;
-  const int units = ntok * units_per_row;
-  unsigned xaddr[MT];  // LDS address of this lane's token row (+ its k-block offset)
-#pragma unroll
-  for (int mt = 0; mt < MT; ++mt) {
-    int t = 16 * mt + r16;
-    if (t >= ntok) t = ntok - 1;
-    xaddr[mt] = (unsigned)(X_BASE + t * pitch + tb * XB);
-  }
-  // Offset removal: corr[g][t] = -sum over the 128 k of group g of x[t, k] * (c(k) + 1) (bf16: c + 1 = 9 for
-  // even k, 3 for odd k; int8: 1), float32 / int32, at corr_base + (g * 16 * MT + t) * 4. A lane starts the
-  // accumulator of a group from the four values of its tokens 4b .. 4b + 3.
-  const unsigned corr_base = (unsigned)(X_BASE + tile_rows * pitch);
-  const unsigned corr_lane = corr_base + (unsigned)(16 * b);
-  const unsigned char* xg = (const unsigned char*)a.x + tok0 * a.K * XB;
-  u32x4 xstage[XU][XB];
-  auto stage_load = [&](int64_t k0) {  // global -> registers, chunk starting at k0
-#pragma unroll
-    for (int i = 0; i < XU; ++i) {
-      const int u = threadIdx.x + i * THREADS;
-      const int row = u / units_per_row, col = u - row * units_per_row;
-      if (u < units && k0 + col * 16 < a.K) {  // the last chunk may be shorter than KC: stay inside the row
-        const unsigned char* p = xg + ((int64_t)row * a.K + k0 + col * 16) * XB;
-#pragma unroll
-        for (int v = 0; v < XB; ++v) xstage[i][v] = *(const u32x4*)(p + 16 * v);
-      }
-    }
-  };
-  auto stage_store = [&]() {  // registers -> LDS, every 16 elements reordered to the decode's slot order
-#pragma unroll
-    for (int i = 0; i < XU; ++i) {
-      const int u = threadIdx.x + i * THREADS;
-      if (u < units) {
-        const int row = u / units_per_row, col = u - row * units_per_row;
-        const unsigned dst = (unsigned)(X_BASE + row * pitch + col * 16 * XB);
-        unsigned part;  // this unit's share of the group's offset sum; 8 consecutive lanes hold one group
-        if (ACT == BP_BF16) {
-          u32x4 o0, o1;
-          tq2_permute_bf16(xstage[i][0], xstage[i][XB - 1], o0, o1);
-          *(lds_u32x4*)(dst) = o0;
-          *(lds_u32x4*)(dst + 16) = o1;
-          float f = 0.f;
-          const bf16x2 w93 = __builtin_bit_cast(bf16x2, 0x40404110u);  // (9.0, 3.0): even k in the low half
-#pragma unroll
-          for (int v = 0; v < XB; ++v) {
-            const unsigned dw[4] = {xstage[i][v].x, xstage[i][v].y, xstage[i][v].z, xstage[i][v].w};
-#pragma unroll
-            for (int d = 0; d < 4; ++d) f = __builtin_amdgcn_fdot2_f32_bf16(__builtin_bit_cast(bf16x2, dw[d]), w93, f, false);
-          }
-          f += __shfl_xor(f, 1);
-          f += __shfl_xor(f, 2);
-          f += __shfl_xor(f, 4);
-          part = __float_as_uint(-f);
-        } else {
-          *(lds_u32x4*)(dst) = tq2_permute_i8(xstage[i][0]);
-          int n = 0;
-#pragma unroll
-          for (int d = 0; d < 4; ++d) n = __builtin_amdgcn_sdot4((int)xstage[i][0][d], 0x01010101, n, false);
-          n += __shfl_xor(n, 1);
-          n += __shfl_xor(n, 2);
-          n += __shfl_xor(n, 4);
-          part = (unsigned)(-n);
-        }
-        if ((col & 7) == 0) *(lds_u32*)(corr_base + ((col >> 3) * (16 * MT) + row) * 4) = part;
-      }
-    }
-  };
-
-  f32x4 total[R][MT];
-#pragma unroll
-  for (int r = 0; r < R; ++r)
-#pragma unroll
-    for (int mt = 0; mt < MT; ++mt) total[r][mt] = f32x4{0.f, 0.f, 0.f, 0.f};
-
-  // decode masks and exponent patterns live in registers: v_and_or_b32 takes no literal operands
-  Tq2Consts kc = {0x00c000c0u, 0x00300030u, 0x40004000u, 0x41004100u};
-  asm volatile("" : "+s"(kc.P1), "+s"(kc.P2));
-  asm volatile("" : "+v"(kc.M1), "+v"(kc.M2));
-
-  const int steps = (int)(a.K / 256);
-  const int steps_per_chunk = KC / 256;
-  const int chunks = (steps + steps_per_chunk - 1) / steps_per_chunk;
-
-  for (int term = 0; term < a.n_terms; ++term) {
-    // this wave's rows of the term as two buffers (R sub-tiles of 16 rows; rows past N are not in range)
-    constexpr int SB = SDT == BP_F32 ? 4 : 2;
-    const int64_t rows_here = a.N - n0 < 16 * R ? a.N - n0 : 16 * R;
-    const __amdgpu_buffer_rsrc_t wrs = make_rsrc(a.packed[term] + (e * a.N + n0) * a.Kp, rows_here * a.Kp);
-    const __amdgpu_buffer_rsrc_t srs = make_rsrc((const unsigned char*)a.w_scale[term] + (e * a.N + n0) * a.G * SB, rows_here * a.G * SB);
-    const unsigned woff = (unsigned)r16 * (unsigned)a.Kp + 16u * b;
-    const unsigned soff = (unsigned)r16 * (unsigned)a.G * SB;
-    // SL: the scales of the workgroup's rows (all of K, one term) are copied into LDS once, as full cache
-    // lines; read row by row from global memory, every 16-byte piece would be an L1 miss of its own.
-    const unsigned stile = corr_base + (unsigned)((KC / 128) * 16 * MT * 4);
-    const unsigned slane = stile + (unsigned)((wave * 16 * R + r16) * (int)a.G * SB);
-    auto stage_scales = [&]() {
-      const int64_t wg_row0 = (int64_t)blockIdx.x * (WAVES * 16 * R);
-      const int64_t wg_rows = a.N - wg_row0 < WAVES * 16 * R ? a.N - wg_row0 : WAVES * 16 * R;
-      const unsigned char* src = (const unsigned char*)a.w_scale[term] + (e * a.N + wg_row0) * a.G * SB;
-      const int units16 = (int)(wg_rows * a.G * SB / 16);
-      if (term > 0) __syncthreads();  // the previous term's scales are no longer read
-      for (int u = threadIdx.x; u < units16; u += THREADS) *(lds_u32x4*)(stile + 16 * u) = *(const u32x4*)(src + 16 * (int64_t)u);
-      __syncthreads();
-    };
-    // Ring of PF steps of packed weights in flight per row sub-tile: with ~4 us of loaded HBM latency a CU
-    // needs > 100 KiB of requests outstanding to stream at full rate (16 waves x PF x R KiB here).
-    constexpr int PF = ABL >= 100 ? 8 : 4;  // (8: timing experiments only; needs K % 2048 == 0 and 2-byte scales)
-    constexpr int AB = ABL % 10, AB2 = ABL / 10 % 10;  // up to two ablations at once
-    u32x4 ring[PF][R] = {};
-    u32x4 sraw[R][2], snext[R][2];  // 8 scales (4 steps) per row sub-tile, and the next 8
-    auto fetch_w = [&](int c, u32x4 (&dst)[R]) {
-      const int cc = c < steps ? c : steps - 1;  // past the end: re-read the last step, no branch
-#pragma unroll
-      for (int r = 0; r < R; ++r) {
-        if (AB == 5 || AB2 == 5) { asm volatile("" : "+v"(dst[r])); continue; }  // ablation: no weight traffic
-        dst[r] = buf_load16(wrs, woff, (unsigned)(row_shift[r] * a.Kp) + 64u * cc);
-      }
-    };
-    auto fetch_s = [&](int c, u32x4 (&dst)[R][2]) {  // scales of steps c .. c+3 (c % 4 == 0)
-      const int cc = c < steps ? c : 0;
-#pragma unroll
-      for (int r = 0; r < R; ++r) {
-        const unsigned so = (unsigned)(row_shift[r] * a.G + 2 * cc) * SB;
-        if (SL) {
-          dst[r][0] = *(const lds_u32x4*)(slane + so);
-          if (SDT == BP_F32 || PF == 8) dst[r][1] = *(const lds_u32x4*)(slane + so + 16);
-          continue;
-        }
-        dst[r][0] = buf_load16(srs, soff, so);
-        if (SDT == BP_F32 || PF == 8) dst[r][1] = buf_load16(srs, soff, so + 16);
-      }
-    };
-    const bool restage = term == 0 || chunks > 1;  // a tile that holds all of K is staged once for all terms
-    if (restage) stage_load(0);
-    // Same issue order as inside the loop (scales, then the weights step by step), pinned with scheduling
-    // barriers: loads return in order, so the loop's waits can then leave the younger loads in flight.
-    if (!SL) fetch_s(0, snext);
-    __builtin_amdgcn_sched_barrier(0);
-#pragma unroll
-    for (int i = 0; i < PF; ++i) {
-      fetch_w(i, ring[i]);
-      __builtin_amdgcn_sched_barrier(0);
-    }
-    if (SL) {  // behind the loads above, so that their latencies overlap with the copy's
-      stage_scales();
-      fetch_s(0, snext);
-    }
-    for (int ch = 0; ch < chunks; ++ch) {
-      if (restage) {
-        __syncthreads();  // every wave is done reading the previous tile 
-        stage_store();
-        __syncthreads();
-        if (ch + 1 < chunks) stage_load((int64_t)(ch + 1) * KC);
-      }
-      const int c_end = (ch + 1) * steps_per_chunk < steps ? (ch + 1) * steps_per_chunk : steps;
-      for (int c4 = ch * steps_per_chunk; c4 < c_end; c4 += PF) {  // KC % 1024 == 0: whole blocks of 4 steps
-#pragma unroll
-        for (int r = 0; r < R; ++r) { sraw[r][0] = snext[r][0]; sraw[r][1] = snext[r][1]; }
-        fetch_s(c4 + PF, snext);
-#pragma unroll
-        for (int i = 0; i < PF; ++i) {
-          // One scheduling region per step: the wait for this step's weights stays here instead of joining
-          // the waits of the later steps at the top of the block.
-          __builtin_amdgcn_sched_barrier(0);
-          const int c = c4 + i;
-          u32x4 w[R];
-#pragma unroll
-          for (int r = 0; r < R; ++r) {  // regroup: .x/.y = 8 bytes of group 2c, .z/.w = 8 bytes of group 2c+1
-            const auto s0 = __builtin_amdgcn_permlane32_swap(ring[i][r].x, ring[i][r].z, false, false);
-            const auto s1 = __builtin_amdgcn_permlane32_swap(ring[i][r].y, ring[i][r].w, false, false);
-            w[r] = u32x4{s0[0], s1[0], s0[1], s1[1]};
-          }
-          const int gl = (c - ch * steps_per_chunk) * 2;  // first of the step's two groups within the tile
-          const unsigned xoff = (unsigned)(gl * 128 * XB);
-          if (AB == 1) {  // ablation (timing experiments only): memory traffic without decode and MFMA
-            fetch_w(c + PF, ring[i]);
-#pragma unroll
-            for (int r = 0; r < R; ++r) total[r][0][0] += __uint_as_float((w[r].x ^ w[r].y ^ w[r].z ^ w[r].w) & 0x3fffffu);
-            continue;
-          }
-#pragma unroll
-          for (int h = 0; h < 2; ++h) {
-            typedef typename Acc<ACT>::type acc_t;
-            u32x4 xa[NJ][MT];
-            acc_t base[MT];
-#pragma unroll
-            for (int mt = 0; mt < MT; ++mt) {
-              if (AB == 3 || AB2 == 3) {  // ablation: no LDS operand reads
-                base[mt] = acc_t{0, 0, 0, 0};
-#pragma unroll
-                for (int j = 0; j < NJ; ++j) xa[j][mt] = u32x4{kc.M1, kc.M2, kc.M1, kc.M2};
-                continue;
-              }
-              base[mt] = __builtin_bit_cast(acc_t, *(const lds_u32x4*)(corr_lane + ((gl + h) * (16 * MT) + 16 * mt) * 4));
-#pragma unroll
-              for (int j = 0; j < NJ; ++j) xa[j][mt] = *(const lds_u32x4*)(xaddr[mt] + xoff + (h * 128 + j * KM) * XB);
-            }
-#pragma unroll
-            for (int r = 0; r < R; ++r) {
-              const unsigned lo = h == 0 ? w[r].x : w[r].z, hi = h == 0 ? w[r].y : w[r].w;
-              u32x4 wb[NJ];
-              if (AB == 4 || AB2 == 4) {  // ablation: no decode
-#pragma unroll
-                for (int j = 0; j < NJ; ++j) wb[j] = u32x4{lo, hi, lo | kc.M1, hi | kc.M1};
-              } else if (ACT == BP_BF16) {
-                tq2_decode_bf16(lo, kc, wb[0], wb[1]);
-                tq2_decode_bf16(hi, kc, wb[NJ - 2], wb[NJ - 1]);
-              } else {
-                wb[0] = tq2_decode_i8(lo);
-                wb[1] = tq2_decode_i8(hi);
-              }
-              const float s = scale_at<SDT>(sraw[r], 2 * i + h);  // group 2c + h = entry 2i + h of the 8 held
-#pragma unroll
-              for (int mt = 0; mt < MT; ++mt) {
-                acc_t acc = base[mt];
-#pragma unroll
-                for (int j = 0; j < NJ; ++j) {
-                  if (AB == 2 || AB2 == 2) {  // ablation: operands are produced but no MFMA is issued
-                    asm volatile("" ::"v"(xa[j][mt]), "v"(wb[j]));
-                    continue;
-                  }
-                  if (ACT == BP_BF16)
-                    acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, xa[j][mt]),
-                                                                  __builtin_bit_cast(bf16x8, wb[j]), acc, 0, 0, 0);
-                  else
-                    acc = __builtin_amdgcn_mfma_i32_16x16x64_i8(__builtin_bit_cast(i32x4, xa[j][mt]),
-                                                                __builtin_bit_cast(i32x4, wb[j]), acc, 0, 0, 0);
-                }
-#pragma unroll
-                for (int q = 0; q < NQ; ++q) total[r][mt][q] += (float)acc[q] * s;
-              }
-            }
-          }
-          // Ring slots are reloaded once consumed (in place: no register copies), two steps at a time and
-          // back to back: the two 64-byte halves of every 128-byte line then reach the L1 together and go
-          // to L2 as one request instead of two that each occupy a miss slot for the full latency.
-          __builtin_amdgcn_sched_barrier(0);
-          if (i & 1) {
-            fetch_w(c - 1 + PF, ring[i - 1]);
-            fetch_w(c + PF, ring[i]);
-          }
-        }
-      }
-    }
-  }
-  // ---- epilogue: lane holds tokens 4b + q (q = 0..3) of each token tile, output row n0 + 16r + r16
-#pragma unroll
-  for (int mt = 0; mt < MT; ++mt) {
-#pragma unroll
-    for (int q = 0; q < NQ; ++q) {  // NQ = 1: single-token launches keep only the sums of token 0
-      const int t = 16 * mt + 4 * b + q;
-      if (t < ntok) {
-        const int64_t tok = tok0 + t;
-        const float xs = ACT == BP_I8 ? a.x_scale[tok] : 1.0f;
-#pragma unroll
-        for (int r = 0; r < R; ++r) {
-          if (rows_valid[r]) {
-            float* o = a.out + tok * a.N + n0 + 16 * r + r16;
-            *o += total[r][mt][q] * xs;
-          }
-        }
-      }
-    }
-  }
-}
-
-template <int ACT, int SDT, int R, int MT, int WAVES, int XKB, int ABL = 0, int NQ = 4, int SL = 1>
-int launch_tq2(const GemmArgs& a, hipStream_t s, const char* name) {
-  constexpr int XB = ACT == BP_BF16 ? 2 : 1;
-  const int64_t rows_per_wg = (int64_t)WAVES * 16 * R;
-  const dim3 grid((unsigned)((a.N + rows_per_wg - 1) / rows_per_wg), (unsigned)a.E,
-                  (unsigned)((a.max_rows + 16 * MT - 1) / (16 * MT)));
-  // chunk length: as much of K as the tile budget holds for the widest token tile, in blocks of 4 steps
-  const int64_t tokens = a.max_rows < 16 * MT ? a.max_rows : 16 * MT;
-  // bytes per k: the tokens' activations plus 16 * MT offset sums of 4 bytes per 128-wide group
-  int64_t kc = 2 * (XKB * 1024 - 16 * tokens) / (2 * tokens * XB + MT) / 1024 * 1024;
-  if (kc > a.K) kc = a.K;
-  if (kc < 1024) return fail(BP_ERR_UNSUPPORTED, "activation tile does not fit");
-  const size_t stile = SL ? (size_t)rows_per_wg * a.G * (SDT == BP_F32 ? 4 : 2) : 0;
-  const size_t lds = X_BASE + (size_t)tokens * (kc * XB + 16) + (size_t)(kc / 128) * 16 * MT * 4 + stile;
-  static bool attr = false;
-  if (!attr) {
-    if (hipFuncSetAttribute((const void*)k_mfma_tq2<ACT, SDT, R, MT, WAVES, XKB, ABL, NQ, SL>, hipFuncAttributeMaxDynamicSharedMemorySize,
-                            X_BASE + XKB * 1024 + (SL ? TQ2_SCALE_TILE_MAX : 0)) != hipSuccess)
-      return fail(BP_ERR_LAUNCH, "cannot raise the dynamic LDS limit");
-    attr = true;
-  }
-  note_kernel(name);
-  hipLaunchKernelGGL((k_mfma_tq2<ACT, SDT, R, MT, WAVES, XKB, ABL, NQ, SL>), grid, dim3(WAVES * 64), lds, s, a, (int)kc, (int)tokens);
-  return check_launch(name);
-}
-
-template <int ACT, int R, int MT, int WAVES, int XKB, int NQ = 4>
-int launch_tq2_sd(const GemmArgs& a, hipStream_t s, const char* name) {
-  // scales through LDS whenever the workgroup's share of one term fits the budget
-  const int64_t tile = (int64_t)WAVES * 16 * R * a.G * (a.scale_dtype == BP_F32 ? 4 : 2);
-  if (tile <= TQ2_SCALE_TILE_MAX) {
-    if (a.scale_dtype == BP_F16) return launch_tq2<ACT, BP_F16, R, MT, WAVES, XKB, 0, NQ, 1>(a, s, name);
-    if (a.scale_dtype == BP_BF16) return launch_tq2<ACT, BP_BF16, R, MT, WAVES, XKB, 0, NQ, 1>(a, s, name);
-    return launch_tq2<ACT, BP_F32, R, MT, WAVES, XKB, 0, NQ, 1>(a, s, name);
-  }
-  if (a.scale_dtype == BP_F16) return launch_tq2<ACT, BP_F16, R, MT, WAVES, XKB, 0, NQ, 0>(a, s, name);
-  if (a.scale_dtype == BP_BF16) return launch_tq2<ACT, BP_BF16, R, MT, WAVES, XKB, 0, NQ, 0>(a, s, name);
-  return launch_tq2<ACT, BP_F32, R, MT, WAVES, XKB, 0, NQ, 0>(a, s, name);
-}
-
-// ------------------------------------------------------------------------------------------------
-// TQ1 (5 trits per byte), bf16 activations. K % 128 == 0, K >= 1024, N % 16 == 0.
-//
-// 640 trits = 128 bytes = 5 scale groups realign byte and group boundaries, so the unit of work is a
-// 128-byte chunk of every row. A byte is atomic: it fills one MFMA k-block with its 5 trits and 3
-// zeros, and the matching activation operand is a 16-byte "slot" holding the 5 activations of that
-// byte and 3 zeros; the activation tile in LDS is laid out slot by slot, so operand reads are aligned.
-// Group g of a chunk touches bytes FB[g] .. FB[g] + NB[g] - 1; k-block b of MFMA m takes byte
-// FB[g] + 7 b + m. A byte shared by two groups is presented to both, with the digits of the other
-// group zeroed (first byte: digits < DF[g]; last byte: digits >= DL[g]); slots past the group's last
-// byte get zero weights.
-//
-// Table entry of byte v: 8 bytes, byte i = high byte of bf16(trit_i / 2) (0x3f, 0xbf or 0), bytes 5..7
-// zero. +-0.5 has a zero low byte, so a v_perm_b32 per operand dword expands the entry to bf16; the
-// factor 2 is folded into the group scale (exact). Zeroing digits is a matter of the perm selector.
-struct __attribute__((packed, aligned(2))) Packed16 { u32x4 v; };
-struct __attribute__((packed, aligned(1))) Packed8 { u32x2 v; };
-constexpr int T1_STRIDE = 128;
-constexpr int T1_WROW = 144;                       // bytes per row of a wave's packed-byte transpose buffer
-constexpr int T1_WBUF_BASE = 256 * T1_STRIDE;      // after the 32 KiB table: WAVES * 16 rows * T1_WROW bytes
-struct __attribute__((packed, aligned(4))) Packed16a4 { u32x4 v; };
-
-template <int WAVES>
-constexpr int t1_tail_base() { return T1_WBUF_BASE + 2 * WAVES * 16 * T1_WROW; }  // two row sub-tiles per wave
-template <int WAVES>
-constexpr int t1_x_base() { return t1_tail_base<WAVES>() + 16 * T1_WROW; }  // + the tensor-tail buffer (16 rows)
-
-// 16 bytes from a 4-byte aligned address, never reading at or past `end` (bytes there read as 1-digits = zero trits)
-constexpr unsigned tq1_sel(int dword, int keep_from, int keep_to) {  // selector of operand dword 0..2
-  // operand dword d holds digits 2d (low half) and 2d+1 (high half); a kept digit i reads entry byte i
-  // (bytes 0..3 from the entry's low dword = perm source 1, byte 4 from the high dword = source 0)
-  unsigned sel = 0x0c0c0c0cu;
-  const int lo = 2 * dword, hi = 2 * dword + 1;
-  if (lo < 5 && lo >= keep_from && lo < keep_to) sel = (sel & 0xffff00ffu) | ((unsigned)(lo < 4 ? lo : 4) << 8);
-  if (hi < 5 && hi >= keep_from && hi < keep_to) sel = (sel & 0x00ffffffu) | ((unsigned)(hi < 4 ? hi : 4) << 24);
-  return sel;
-}
-
-template <int SDT, int R, int MT, int WAVES, int ABL = 0>
-__global__ __launch_bounds__(WAVES * 64) void k_mfma_tq1(GemmArgs a, int CPT /* chunks per activation tile */) {
-  constexpr int THREADS = WAVES * 64;
-  constexpr int T1_X_BASE = t1_x_base<WAVES>();
-  constexpr int XU = (X_TILE_BYTES / 16 + THREADS - 1) / THREADS;  // activation slots staged per thread
-  constexpr int FB[5] = {0, 25, 51, 76, 102};
-  constexpr int DF[5] = {0, 3, 1, 4, 2};
-  constexpr int DL[5] = {3, 1, 4, 2, 5};
-  constexpr int MLAST[5] = {4, 5, 4, 5, 4};  // NB[g] - 1 - 21 with NB = {26, 27, 26, 27, 26}
-
-  // ---- table: entry of byte v, copy c (16 copies) at v * 128 + c * 8
-  if (threadIdx.x < 256) {
-    const unsigned v = threadIdx.x;
-    unsigned hb[5];
-#pragma unroll
-    for (int i = 0; i < 5; ++i) { const int t = tq1_trit(v, i); hb[i] = t > 0 ? 0x3fu : t < 0 ? 0xbfu : 0u; }
-    const u32x2 e = {hb[0] | (hb[1] << 8) | (hb[2] << 16) | (hb[3] << 24), hb[4]};
-    for (int c = 0; c < 16; ++c) *(lds_u32x2*)(v * T1_STRIDE + c * 8) = e;
-  }
-
-  const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
-  const int r16 = lane & 15, b = lane >> 4;
-  const int64_t e = blockIdx.y;
-  const int64_t o0 = clamp_i64(a.offsets[e], 0, a.T), o1 = clamp_i64(a.offsets[e + 1], 0, a.T);
-  const int64_t tok0 = o0 + (int64_t)blockIdx.z * (16 * MT);
-  if (tok0 >= o1) return;  // uniform for the workgroup
-  const int ntok = (int)(o1 - tok0 < 16 * MT ? o1 - tok0 : 16 * MT);
-  int64_t n0 = ((int64_t)blockIdx.x * WAVES + wave) * (16 * R);
-  const bool wave_live = n0 < a.N;
-  if (!wave_live) n0 = 0;
-  const unsigned lane_off = (unsigned)((lane & 15) * 8);
-  const bool is_b0 = b == 0, is_b3 = b == 3;
-
-  bool rows_valid[R];
-  int64_t row_off[R];  // byte offset of row sub-tile r from sub-tile 0, in the packed tensor
-  int64_t srow_off[R];
-#pragma unroll
-  for (int r = 0; r < R; ++r) {
-    rows_valid[r] = wave_live && n0 + 16 * r < a.N;
-    row_off[r] = rows_valid[r] ? 16 * r * a.Kp : 0;
-    srow_off[r] = rows_valid[r] ? 16 * r * a.G * 2 : 0;
-  }
-
-  // The wide loads of a row's last chunk read up to 135 bytes past the chunk start, i.e. into the rows
-  // that follow (Kp >= 205). The last 16 rows of the tensor have nothing after them: for that sub-tile the
-  // last chunk comes from a small LDS buffer filled once, byte by byte, with loads that stay in bounds.
-  bool is_tail[R];
-#pragma unroll
-  for (int r = 0; r < R; ++r) is_tail[r] = rows_valid[r] && e + 1 == a.E && n0 + 16 * r + 16 >= a.N;
-
-  // ---- activation tile, slot layout: slot s of token t at T1_X_BASE + t * pitch + s * 16
-  const int slots = CPT * 128;
-  const int pitch = slots * 16 + 16;
-  const int units = ntok * slots;
-  unsigned xaddr[MT];
-#pragma unroll
-  for (int mt = 0; mt < MT; ++mt) {
-    int t = 16 * mt + r16;
-    if (t >= ntok) t = ntok - 1;
-    xaddr[mt] = (unsigned)(T1_X_BASE + t * pitch + 7 * 16 * b);
-  }
-  // The 16-byte pad after every row and the 32 bytes after the last row are read (by slots past a group's
-  // last byte, against zero weights) but never staged: clear them once so they cannot hold NaN patterns.
-  if ((int)threadIdx.x < ntok) *(lds_u32x4*)(T1_X_BASE + threadIdx.x * pitch + slots * 16) = u32x4{0u, 0u, 0u, 0u};
-  if (threadIdx.x < 2) *(lds_u32x4*)(T1_X_BASE + ntok * pitch + threadIdx.x * 16) = u32x4{0u, 0u, 0u, 0u};
-  const uint16_t* xg = (const uint16_t*)a.x + tok0 * a.K;
-  u32x4 xstage[XU];
-  auto stage_load = [&](int64_t slot0) {  // global -> registers: slots slot0 .. slot0 + slots of every token
-#pragma unroll
-    for (int i = 0; i < XU; ++i) {
-      const int u = threadIdx.x + i * THREADS;
-      u32x4 v = {0u, 0u, 0u, 0u};
-      if (u < units) {
-        const int row = u / slots, sl = u - row * slots;
-        const int64_t k0 = 5 * (slot0 + sl);
-        const uint16_t* src = xg + (int64_t)row * a.K + k0;
-        if (k0 + 8 <= a.K) {
-          v = ((const Packed16*)src)->v;
-          v.z &= 0xffffu;
-          v.w = 0u;
-        } else if (k0 < a.K) {  // the last slots of a row: element by element, zeros past K
-          unsigned h[5];
-#pragma unroll
-          for (int j = 0; j < 5; ++j) h[j] = k0 + j < a.K ? src[j] : 0u;
-          v = u32x4{h[0] | (h[1] << 16), h[2] | (h[3] << 16), h[4], 0u};
-        }
-      }
-      xstage[i] = v;
-    }
-  };
-  auto stage_store = [&]() {
-#pragma unroll
-    for (int i = 0; i < XU; ++i) {
-      const int u = threadIdx.x + i * THREADS;
-      if (u < units) {
-        const int row = u / slots, sl = u - row * slots;
-        *(lds_u32x4*)(T1_X_BASE + row * pitch + sl * 16) = xstage[i];
-      }
-    }
-  };
-
-  f32x4 total[R][MT];
-#pragma unroll
-  for (int r = 0; r < R; ++r)
-#pragma unroll
-    for (int mt = 0; mt < MT; ++mt) total[r][mt] = f32x4{0.f, 0.f, 0.f, 0.f};
-
-  const int64_t nchunks = (a.K + 639) / 640;  // 128-byte chunks per row (the last may be partial)
-  const int64_t tiles = (nchunks + CPT - 1) / CPT;
-
-  for (int term = 0; term < a.n_terms; ++term) {
-    // Packed bytes: every lane loads two aligned 16-byte pieces of its row's 128-byte chunk (plus one
-    // dword past it), the wave transposes them through its private LDS buffer and every lane reads
-    // back the 7 consecutive bytes of its k-block for each group. Aligned wide loads stream ~1.7x
-    // faster than per-lane 8-byte loads at byte offsets.
-    const unsigned char* wbeg = a.packed[term];
-    const unsigned char* rowp = wbeg + (e * a.N + n0 + r16) * a.Kp;
-    const unsigned char* srow = (const unsigned char*)a.w_scale[term] + (e * a.N + n0 + r16) * a.G * 2;
-    const unsigned wrbuf = (unsigned)(T1_WBUF_BASE + (wave * 16 + r16) * T1_WROW);  // this lane's row in the wave's buffer
-    const unsigned tailbuf = (unsigned)(t1_tail_base<WAVES>() + r16 * T1_WROW);
-#pragma unroll
-    for (int r = 0; r < R; ++r) {
-      if (is_tail[r]) {  // at most one wave of the launch: guarded byte copy of the last chunk into LDS
-        const unsigned char* wend = wbeg + a.E * a.N * a.Kp;
-        const unsigned char* base = (const unsigned char*)((uintptr_t)(rowp + row_off[r] + 128 * (nchunks - 1)) & ~(uintptr_t)3);
-#pragma unroll 6
-        for (int i = 0; i < 36; ++i) {
-          const int off = i < 16 ? 16 * b + i : (i < 32 ? 64 + 16 * b + (i - 16) : 128 + (i - 32));
-          const unsigned char* q = base + off;
-          *(__attribute__((address_space(3))) unsigned char*)(tailbuf + off) = q < wend ? *q : (unsigned char)121;
-        }
-      }
-    }
-    constexpr int PFQ = 2;  // chunks in flight behind the one being computed
-    u32x4 wq[PFQ][R][2];
-    unsigned wt[PFQ][R];
-    unsigned sq[PFQ][R];  // k-blocks 0..2 each fetch one dword = 2 of the 6 scales starting at an even group index
-    const int sb = b < 3 ? b : 2;
-    auto fetch = [&](int64_t c, u32x4 (&wd)[R][2], unsigned (&td)[R], unsigned (&sd)[R]) {  // chunk c (clamped to the last)
-      const int64_t cl = c < nchunks ? c : nchunks - 1;
-      int64_t gi = (5 * cl) & ~(int64_t)1;  // 4-byte aligned start of the 6 scales that cover groups 5c .. 5c+4
-      if (gi > a.G - 6) gi = a.G - 6;
-#pragma unroll
-      for (int r = 0; r < R; ++r) {
-        const unsigned char* rp = rowp + row_off[r];
-        const int64_t cc = is_tail[r] && cl + 1 == nchunks ? cl - 1 : cl;  // tensor tail: never fetched from here
-        const unsigned char* p = (const unsigned char*)((uintptr_t)(rp + 128 * cc) & ~(uintptr_t)3) + 16 * b;
-        wd[r][0] = ((const Packed16a4*)p)->v;
-        wd[r][1] = ((const Packed16a4*)(p + 64))->v;
-        td[r] = *(const unsigned*)(p - 16 * b + 128);
-        sd[r] = *(const unsigned*)(srow + srow_off[r] + (gi + 2 * sb) * 2);
-      }
-    };
-    const bool restage = term == 0 || tiles > 1;
-    if (restage) stage_load(0);
-#pragma unroll
-    for (int i = 0; i < PFQ; ++i) fetch(i, wq[i], wt[i], sq[i]);
-    for (int64_t tl = 0; tl < tiles; ++tl) {
-      if (restage) {
-        __syncthreads();
-        stage_store();
-        __syncthreads();
-        if (tl + 1 < tiles) stage_load((tl + 1) * slots);
-      }
-      const int64_t c_end = (tl + 1) * CPT < nchunks ? (tl + 1) * CPT : nchunks;
-      for (int64_t c = tl * CPT; c < c_end; ++c) {
-        // Transpose through the wave's LDS buffer: row r16 of sub-tile r holds the aligned 128 bytes, the
-        // dword after them and the 6 scales; chunk byte j sits at offset j + dlt. LDS operations of one wave
-        // execute in order; the fences only pin the compiler's ordering.
-        unsigned dlt[R], rbuf[R];
-#pragma unroll
-        for (int r = 0; r < R; ++r) {
-          const bool from_tail = is_tail[r] && c + 1 == nchunks;
-          rbuf[r] = from_tail ? tailbuf : wrbuf + r * T1_WROW * 16 * WAVES;
-          const unsigned rb = rbuf[r];
-          dlt[r] = (unsigned)((uintptr_t)(rowp + row_off[r]) & 3);
-          if (!from_tail) {
-            *(lds_u32x4*)(rb + 16 * b) = wq[0][r][0];
-            *(lds_u32x4*)(rb + 64 + 16 * b) = wq[0][r][1];
-            *(lds_u32*)(rb + 128) = wt[0][r];
-          }
-          *(lds_u32*)(rb + 132 + 4 * sb) = sq[0][r];
-        }
-        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
-        __builtin_amdgcn_wave_barrier();
-#pragma unroll
-        for (int i = 0; i + 1 < PFQ; ++i)  // rotate the queue (register moves), then refill its tail
-#pragma unroll
-          for (int r = 0; r < R; ++r) {
-            sq[i][r] = sq[i + 1][r];
-            wt[i][r] = wt[i + 1][r];
-            wq[i][r][0] = wq[i + 1][r][0];
-            wq[i][r][1] = wq[i + 1][r][1];
-          }
-        fetch(c + PFQ, wq[PFQ - 1], wt[PFQ - 1], sq[PFQ - 1]);
-        const int64_t groups_left = a.G - 5 * c;
-        const int ng = groups_left < 5 ? (int)groups_left : 5;
-        int64_t gi = (5 * c) & ~(int64_t)1;
-        if (gi > a.G - 6) gi = a.G - 6;
-        const int sshift = (int)(5 * c - gi);  // wave-uniform position of group 5c among the 6 scales loaded
-        const unsigned xoff = (unsigned)((c - tl * CPT) * 2048);
-        if (ABL == 1) {  // ablation (timing experiments only): memory traffic without decode and MFMA
-#pragma unroll
-          for (int r = 0; r < R; ++r)
-#pragma unroll
-            for (int g = 0; g < 5; ++g) total[r][0][0] += __uint_as_float((*(const lds_u32*)(wrbuf + 24 * g + 4 * b)) & 0x3fffffu);
-          continue;
-        }
-#pragma unroll
-        for (int g = 0; g < 5; ++g) {
-          if (g < ng) {
-            f32x4 acc[R][MT];
-#pragma unroll
-            for (int r = 0; r < R; ++r)
-#pragma unroll
-              for (int mt = 0; mt < MT; ++mt) acc[r][mt] = f32x4{0.f, 0.f, 0.f, 0.f};
-            // two-stage pipeline over the 7 MFMA slots: the LDS reads of slot m+1 are issued before the
-            // MFMAs of slot m; the scheduling barriers keep the compiler from hoisting all 35 slots at once
-            u32x2 wg[R];  // the 7 bytes of this lane's k-block for group g, read back from the transpose buffer
-#pragma unroll
-            for (int r = 0; r < R; ++r) {
-              const unsigned rb = rbuf[r];
-              const unsigned o = dlt[r] + FB[g] + 7 * b;
-              const unsigned d0 = *(const lds_u32*)(rb + (o & ~3u));
-              const unsigned d1 = *(const lds_u32*)(rb + (o & ~3u) + 4);
-              const unsigned d2 = *(const lds_u32*)(rb + (o & ~3u) + 8);
-              wg[r] = u32x2{__builtin_amdgcn_alignbyte(d1, d0, o & 3u), __builtin_amdgcn_alignbyte(d2, d1, o & 3u)};
-            }
-            u32x4 xa[2][MT];
-            u32x2 we[2][R];
-            auto issue = [&](int m, int buf) {
-#pragma unroll
-              for (int mt = 0; mt < MT; ++mt) xa[buf][mt] = *(const lds_u32x4*)(xaddr[mt] + xoff + 16 * (FB[g] + m));
-#pragma unroll
-              for (int r = 0; r < R; ++r) {
-                const unsigned src = m < 4 ? wg[r].x : wg[r].y;
-                we[buf][r] = *(const lds_u32x2*)((__builtin_amdgcn_ubfe(src, 8 * (m & 3), 8) << 7) | lane_off);
-              }
-            };
-            issue(0, 0);
-#pragma unroll
-            for (int m = 0; m < 7; ++m) {
-              const int cur = m & 1;
-              if (m + 1 < 7) issue(m + 1, cur ^ 1);
-              // perm selectors of this slot: digits of another group, or a slot past the group, read as zero
-              unsigned s0 = tq1_sel(0, 0, 5), s1 = tq1_sel(1, 0, 5), s2 = tq1_sel(2, 0, 5);
-              if (m == 0 && DF[g] > 0) {
-                s0 = is_b0 ? tq1_sel(0, DF[g], 5) : s0;
-                s1 = is_b0 ? tq1_sel(1, DF[g], 5) : s1;
-              }
-              if (m == MLAST[g] && DL[g] < 5) {
-                s0 = is_b3 ? tq1_sel(0, 0, DL[g]) : s0;
-                s1 = is_b3 ? tq1_sel(1, 0, DL[g]) : s1;
-                s2 = is_b3 ? tq1_sel(2, 0, DL[g]) : s2;
-              }
-              if (m > MLAST[g]) {
-                s0 = is_b3 ? 0x0c0c0c0cu : s0;
-                s1 = is_b3 ? 0x0c0c0c0cu : s1;
-                s2 = is_b3 ? 0x0c0c0c0cu : s2;
-              }
-#pragma unroll
-              for (int r = 0; r < R; ++r) {
-                const u32x2 en = we[cur][r];
-                const u32x4 d = {__builtin_amdgcn_perm(en.y, en.x, s0), __builtin_amdgcn_perm(en.y, en.x, s1),
-                                 __builtin_amdgcn_perm(en.y, en.x, s2), 0u};
-                if (ABL == 2) {  // ablation: everything but the MFMA
-#pragma unroll
-                  for (int mt = 0; mt < MT; ++mt) acc[r][mt][0] += __uint_as_float((d.x ^ d.y ^ d.z ^ xa[cur][mt].x) & 0x3fffffu);
-                  continue;
-                }
-#pragma unroll
-                for (int mt = 0; mt < MT; ++mt)
-                  acc[r][mt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, xa[cur][mt]),
-                                                                       __builtin_bit_cast(bf16x8, d), acc[r][mt], 0, 0, 0);
-              }
-              __builtin_amdgcn_sched_barrier(0);
-            }
-#pragma unroll
-            for (int r = 0; r < R; ++r) {
-              const unsigned half = *(const __attribute__((address_space(3))) uint16_t*)(rbuf[r] + 132 + 2 * (sshift + g));
-              // weights were decoded as +-0.5: the factor 2 goes into the scale (exact)
-              const float sc = 2.0f * (SDT == BP_F16 ? f16_bits_to_f32((uint16_t)half) : __uint_as_float(half << 16));
-#pragma unroll
-              for (int mt = 0; mt < MT; ++mt)
-#pragma unroll
-                for (int q = 0; q < 4; ++q) total[r][mt][q] += acc[r][mt][q] * sc;
-            }
-          }
-        }
-      }
-    }
-  }
-#pragma unroll
-  for (int mt = 0; mt < MT; ++mt) {
-#pragma unroll
-    for (int q = 0; q < 4; ++q) {
-      const int t = 16 * mt + 4 * b + q;
-      if (t < ntok) {
-        const int64_t tok = tok0 + t;
-#pragma unroll
-        for (int r = 0; r < R; ++r) {
-          if (rows_valid[r]) {
-            float* o = a.out + tok * a.N + n0 + 16 * r + r16;
-            *o += total[r][mt][q];
-          }
-        }
-      }
-    }
-  }
-}
-
-template <int SDT, int R, int MT, int WAVES, int ABL = 0>
-int launch_tq1(const GemmArgs& a, hipStream_t s, const char* name) {
-  const int64_t rows_per_wg = (int64_t)WAVES * 16 * R;
-  const dim3 grid((unsigned)((a.N + rows_per_wg - 1) / rows_per_wg), (unsigned)a.E,
-                  (unsigned)((a.max_rows + 16 * MT - 1) / (16 * MT)));
-  const int64_t tokens = a.max_rows < 16 * MT ? a.max_rows : 16 * MT;
-  const int64_t nchunks = (a.K + 639) / 640;
-  int64_t cpt = (X_TILE_BYTES / tokens - 16) / 2048;  // 128 slots of 16 bytes per chunk and token
-  if (cpt > nchunks) cpt = nchunks;
-  if (cpt < 1) return fail(BP_ERR_UNSUPPORTED, "activation tile does not fit");
-  const size_t lds = t1_x_base<WAVES>() + (size_t)tokens * (cpt * 2048 + 16) + 32;
-  static bool attr = false;
-  if (!attr) {
-    if (hipFuncSetAttribute((const void*)k_mfma_tq1<SDT, R, MT, WAVES, ABL>, hipFuncAttributeMaxDynamicSharedMemorySize,
-                            t1_x_base<WAVES>() + X_TILE_BYTES + 32) != hipSuccess)
-      return fail(BP_ERR_LAUNCH, "cannot raise the dynamic LDS limit");
-    attr = true;
-  }
-  note_kernel(name);
-  hipLaunchKernelGGL((k_mfma_tq1<SDT, R, MT, WAVES, ABL>), grid, dim3(WAVES * 64), lds, s, a, (int)cpt);
-  return check_launch(name);
-}
-
-template <int R, int MT, int WAVES>
-int launch_tq1_sd(const GemmArgs& a, hipStream_t s, const char* name) {
-  if (a.scale_dtype == BP_F16) return launch_tq1<BP_F16, R, MT, WAVES>(a, s, name);
-  return launch_tq1<BP_BF16, R, MT, WAVES>(a, s, name);
-}
-
-}  // namespace
 
 bool mfma_supports(const GemmArgs& a) {
   if (a.group != 128 || a.N % 16 != 0) return false;
@@ -855,68 +25,19 @@ bool mfma_supports(const GemmArgs& a) {
 }
 
 int launch_mfma(const GemmArgs& a, hipStream_t s) {
-  const bool bf = a.x_dtype == BP_BF16;
   // rows per wave and waves per workgroup: keep enough workgroups in flight for small problems
   const int64_t work = a.E * (a.N / 16);
-  int R = 1;  // two row sub-tiles per wave spill registers at 4 waves per SIMD; see BP_TUNE_R
+  int R = 1;  // two row sub-tiles per wave cost more registers than they save LDS reads; see BP_TUNE_R
   int MT = a.max_rows > 16 ? 2 : 1;
   // 8-wave workgroups run two to a CU, so one's start-up (staging, first loads) overlaps the other's
   // steady state; the TQ2 single-token kernels are light enough on registers for that to win everywhere.
   int waves = work >= 2048 && !(a.fmt == BP_TQ2 && a.max_rows == 1) ? 16 : 8;
+  // development overrides (tuning sweeps)
   if (const char* t = getenv("BP_TUNE_R")) { const int v = atoi(t); if (v == 1 || v == 2) R = v; }
   if (const char* t = getenv("BP_TUNE_WAVES")) { const int v = atoi(t); if (v == 8 || v == 16) waves = v; }
   if (const char* t = getenv("BP_TUNE_MT")) { const int v = atoi(t); if (v == 1 || v == 2) MT = v; }
-  if (a.fmt == BP_TQ1) {
-    MT = 1;  // a 16-token slot-layout tile is the most the LDS budget holds; more rows go to more workgroups
-    if (const char* t = getenv("BP_TUNE_ABL")) {
-      if (atoi(t) == 1) return launch_tq1<BP_F16, 1, 1, 16, 1>(a, s, "abl1_tq1");
-      if (atoi(t) == 2) return launch_tq1<BP_F16, 1, 1, 16, 2>(a, s, "abl2_tq1");
-    }
-#define BP_T1(RV, WV) \
-    if (R == RV && waves == WV) return launch_tq1_sd<RV, 1, WV>(a, s, "mfma_tq1_bf16_r" #RV "_m1_w" #WV);
-    BP_T1(1, 8) BP_T1(2, 8) BP_T1(1, 16) BP_T1(2, 16)
-#undef BP_T1
-    return fail(BP_ERR_UNSUPPORTED, "no tuned TQ1 kernel variant for this tiling");
-  }
-  if (const char* t = getenv("BP_TUNE_ABL")) {
-    if (bf && a.scale_dtype == BP_F16 && MT == 1) {
-      switch (atoi(t)) {
-        case 1: return launch_tq2<BP_BF16, BP_F16, 1, 1, 16, 48, 1>(a, s, "abl1_w16");
-        case 2: return launch_tq2<BP_BF16, BP_F16, 1, 1, 16, 48, 2>(a, s, "abl2_w16");
-        case 3: return launch_tq2<BP_BF16, BP_F16, 1, 1, 16, 48, 3>(a, s, "abl3_w16");
-        case 4: return launch_tq2<BP_BF16, BP_F16, 1, 1, 16, 48, 4>(a, s, "abl4_w16");
-        case 5: return launch_tq2<BP_BF16, BP_F16, 1, 1, 16, 48, 5>(a, s, "abl5_w16");
-        case 25: return launch_tq2<BP_BF16, BP_F16, 1, 1, 16, 48, 25>(a, s, "abl25_w16");
-        case 35: return launch_tq2<BP_BF16, BP_F16, 1, 1, 16, 48, 35>(a, s, "abl35_w16");
-        case 45: return launch_tq2<BP_BF16, BP_F16, 1, 1, 16, 48, 45>(a, s, "abl45_w16");
-        case 100: return launch_tq2<BP_BF16, BP_F16, 1, 1, 16, 48, 100>(a, s, "abl100_w16");
-        default: break;
-      }
-    }
-  }
-  if (MT == 2) waves = 16;  // the 32-token tile needs the large LDS budget of a 16-wave workgroup
-  if (a.max_rows == 1 && R == 2 && MT == 1 && waves == 16) {
-    if (bf) return launch_tq2_sd<BP_BF16, 2, 1, 16, 48, 1>(a, s, "mfma_tq2_bf16_r2_t1_w16");
-    return launch_tq2_sd<BP_I8, 2, 1, 16, 48, 1>(a, s, "mfma_tq2_i8_r2_t1_w16");
-  }
-  if (a.max_rows == 1 && R == 1 && MT == 1) {  // decode GEMV: one token, only its sums are scaled and kept
-    if (bf) {
-      if (waves == 16) return launch_tq2_sd<BP_BF16, 1, 1, 16, 48, 1>(a, s, "mfma_tq2_bf16_r1_t1_w16");
-      return launch_tq2_sd<BP_BF16, 1, 1, 8, 48, 1>(a, s, "mfma_tq2_bf16_r1_t1_w8");
-    }
-    if (waves == 16) return launch_tq2_sd<BP_I8, 1, 1, 16, 48, 1>(a, s, "mfma_tq2_i8_r1_t1_w16");
-    return launch_tq2_sd<BP_I8, 1, 1, 8, 48, 1>(a, s, "mfma_tq2_i8_r1_t1_w8");
-  }
-#define BP_CASE(ACTV, RV, MTV, WV, XK, NAME) \
-  if (R == RV && MT == MTV && waves == WV) return launch_tq2_sd<ACTV, RV, MTV, WV, XK>(a, s, NAME "_r" #RV "_m" #MTV "_w" #WV);
-#define BP_ALL(ACTV, NAME)                                                        \
-  BP_CASE(ACTV, 1, 1, 8, 48, NAME) BP_CASE(ACTV, 2, 1, 8, 48, NAME)                \
-  BP_CASE(ACTV, 1, 1, 16, 48, NAME) BP_CASE(ACTV, 2, 1, 16, 48, NAME)              \
-  BP_CASE(ACTV, 1, 2, 16, 112, NAME) BP_CASE(ACTV, 2, 2, 16, 112, NAME)
-  if (bf) { BP_ALL(BP_BF16, "mfma_tq2_bf16") } else { BP_ALL(BP_I8, "mfma_tq2_i8") }
-#undef BP_ALL
-#undef BP_CASE
-  return fail(BP_ERR_UNSUPPORTED, "no tuned kernel variant for this tiling");
+  if (a.fmt == BP_TQ1) return launch_mfma_tq1(a, s, waves);
+  return launch_mfma_tq2(a, s, R, MT, waves);
 }
 
 }  // namespace bp
