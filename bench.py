@@ -13,7 +13,8 @@ before the timed region. Prints ONE JSON line:
                       launch stream) against the 8 TB/s HBM peak
   cpu_baseline      : the reference's CPU kernel (oracle/_ref, "reference") or this repository's C
                       port of it ("port") timed on the host cores on one linear of the same workload
-  also              : secondary measurements (other M, single-linear latency, grouped-expert GEMM TFLOP/s)
+  also              : secondary measurements (other M, the TQ2 / int8 variants of the GEMV, single-linear
+                      latency, grouped-expert GEMM TFLOP/s, prefill / decode tok/s of the decoder harness)
 """
 
 from __future__ import annotations
@@ -33,12 +34,17 @@ HBM_PEAK_GBPS = 8000.0
 MFMA_BF16_PEAK_TFLOPS = 2500.0
 GROUP = 128
 
+# HBM bytes per launch measured with rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE on this command line (each
+# counter scaled by what it reads for a plain 1 GiB device copy); the summaries are under profiles/.
+MEASURED_TRAFFIC_BYTES = {}
+
 WORKLOADS = {
     # name: (fmt, N, K, M tokens per linear, activation, terms, L linears per launch)
     "cfg1a_tq1_gemv": ("tq1", 2048, 7168, 1, "bf16", 1, 128),
     "cfg1b_tq1_gemv": ("tq1", 7168, 2048, 1, "bf16", 1, 128),
     "cfg1a_tq2_gemv": ("tq2", 2048, 7168, 1, "bf16", 1, 128),
     "cfg0_tq2_gemv": ("tq2", 2048, 4096, 1, "bf16", 1, 192),
+    "cfg1a_tq2_i8_gemv": ("tq2", 2048, 7168, 1, "int8", 1, 128),
 }
 
 
@@ -190,6 +196,16 @@ def main() -> int:
             also[f"M{m}_kernel"] = kn2
             del l2
             torch.cuda.empty_cache()
+        for name in ("cfg1a_tq2_gemv", "cfg1a_tq2_i8_gemv", "cfg1b_tq1_gemv"):  # the same GEMV in the other formats / shapes
+            if name == a.workload:
+                continue
+            f2, n2, k2_, m2, act2, t2, L2 = WORKLOADS[name]
+            l2, wb2 = uniform_launch(bp, torch, f2, n2, k2_, m2, act2, t2, L2)
+            _, kk, kn2 = l2.time(max(5, a.steps // 2), 2)
+            also[name] = {"weight_GBps": round(wb2 / kk / 1e9, 1), "frac_of_hbm_peak": round(wb2 / kk / 1e9 / HBM_PEAK_GBPS, 4),
+                          "kernel": kn2, "us": round(kk * 1e6, 1)}
+            del l2
+            torch.cuda.empty_cache()
         l1, wb1 = uniform_launch(bp, torch, fmt, N, K, M, act, terms, 1)  # one linear per launch (cache-resident, latency bound)
         w1, k1, _ = l1.time(200, 20)
         also["single_linear_us_per_call"] = round(w1 * 1e6, 2)
@@ -213,6 +229,18 @@ def main() -> int:
                                 "frac_of_bf16_mfma_peak": round(flops / k3t / 1e12 / MFMA_BF16_PEAK_TFLOPS, 4),
                                 "weight_GBps": round(weight_bytes(packed, scales) / k3t / 1e9, 1), "kernel": kn3,
                                 "us": round(k3t * 1e6, 1)}
+        del l3, packed, scales, xg
+        torch.cuda.empty_cache()
+        # end-to-end timing loop of the reference's `boilerplate bench` on a random-init OLMoE-shaped Mode D decoder
+        from deepseekternarized_amd.decoder_harness import DecoderConfig, TernaryDecoder, bench_decoder
+
+        cfg = DecoderConfig()
+        r = bench_decoder(TernaryDecoder(cfg), 64, 128, 32)
+        also["decoder_harness"] = {"workload": f"{cfg.layers} layers, hidden {cfg.hidden}, {cfg.experts} experts top-{cfg.top_k}, "
+                                               f"inter {cfg.inter}, {cfg.fmt.upper()}, {cfg.act} activations, random weights; "
+                                               "batch 64, prompt 128, 32 greedy decode steps",
+                                   "prefill_tok_s": r["prefill_tok_s"], "decode_tok_s": r["decode_tok_s"],
+                                   "peak_vram_bytes": r["peak_vram_bytes"], "finite": r["finite"]}
 
     line = {
         "metric": "ternary GEMV HBM GB/s (% peak); grouped-expert GEMM TFLOP/s (% MFMA peak)",
@@ -224,7 +252,7 @@ def main() -> int:
                    "kernel": kname, "bytes_counted": "packed + fp16 scales as stored",
                    "activation_and_output_bytes_per_step": act_bytes},
         "roofline": {"bound": "hbm", "achieved": round(wbytes / kern / 1e9, 1), "peak": HBM_PEAK_GBPS, "unit": "GB/s",
-                     "frac": round(wbytes / kern / 1e9 / HBM_PEAK_GBPS, 4), "traffic": None,
+                     "frac": round(wbytes / kern / 1e9 / HBM_PEAK_GBPS, 4), "traffic": MEASURED_TRAFFIC_BYTES.get(a.workload),
                      "kernel_us": round(kern * 1e6, 2)},
         "cpu_baseline": None if a.no_cpu else cpu_baseline(fmt, N, K, M),
         "also": also,
