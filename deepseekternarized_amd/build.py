@@ -16,7 +16,7 @@ from pathlib import Path
 HERE = Path(__file__).resolve().parent
 CSRC = HERE / "csrc"
 LIB = HERE / "libbp_ternary_hip.so"
-SOURCES = ["bp_api.hip", "bp_general.hip", "bp_route.hip", "bp_mfma.hip", "bp_mfma_tq2.hip", "bp_mfma_tq1.hip"]
+SOURCES = ["bp_api.hip", "bp_general.hip", "bp_route.hip", "bp_mfma.hip", "bp_mfma_tq2.hip", "bp_mfma_tq1.hip", "bp_tq1_gemv.hip"]
 # packed FP32 VALU ops are disabled for every device object of this library
 FLAGS = ["--offload-arch=gfx950", "-O3", "-fPIC", "-std=c++17", "-Wall", "-Wno-unused-function", "-Wno-int-to-pointer-cast",
          "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops"]
@@ -36,7 +36,7 @@ def _compile(src: str) -> Path:
 
 
 def build(verbose: bool = True) -> Path:
-    with ThreadPoolExecutor(max_workers=6) as pool:
+    with ThreadPoolExecutor(max_workers=7) as pool:
         objs = list(pool.map(_compile, SOURCES))
     cmd = ["hipcc", "--offload-arch=gfx950", "-shared", "-fPIC", *map(str, objs), "-o", str(LIB)]
     res = subprocess.run(cmd, capture_output=True, text=True)

@@ -346,7 +346,10 @@ int launch_mfma_tq1(const GemmArgs& a, hipStream_t s, int waves) {
     if (atoi(t) == 4) return launch_tq1<BP_F16, 16, 1, 1, 4>(a, s, "abl4_tq1");
     if (atoi(t) == 5) return launch_tq1<BP_F16, 16, 1, 1, 5>(a, s, "abl5_tq1");
   }
-  if (a.max_rows == 1) {  // decode GEMV: one token, only its sums are scaled and kept
+  if (a.max_rows == 1) {  // decode GEMV
+    const char* t = getenv("BP_TUNE_TQ1");  // development: "mfma" keeps the single-token MFMA variant
+    if (!(t && t[0] == 'm')) return launch_tq1_gemv(a, s, waves);
+    // one token, only its sums are scaled and kept
     if (waves == 16) return launch_tq1_v<16, 1>(a, s, "mfma_tq1_bf16_t1_w16", "mfma_tq1_bf16_t1_w16_gs");
     return launch_tq1_v<8, 1>(a, s, "mfma_tq1_bf16_t1_w8", "mfma_tq1_bf16_t1_w8_gs");
   }
