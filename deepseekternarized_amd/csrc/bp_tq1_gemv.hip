@@ -26,6 +26,7 @@
 namespace bp {
 namespace {
 
+struct __attribute__((packed, aligned(2))) Packed16 { u32x4 v; };
 typedef __attribute__((address_space(3))) float lds_f32;
 
 constexpr int G1_SLOTS = 140;                     // byte slots per chunk: 5 groups x 28
@@ -84,6 +85,15 @@ __global__ __launch_bounds__(WAVES * 64, 4) void k_tq1_gemv(GemmArgs a, int CPT 
         int lo = 128 * g - 5 * j, hi = lo + 128;                   // digits lo <= d < hi belong to group g
         if (a.K - k0 < hi) hi = (int)(a.K - k0);                   // ... and lie inside K
         const int64_t at = tok * a.K + k0;
+        if ((a.x_dtype == BP_BF16 || a.x_dtype == BP_F16) && hi > 0 && lo < 5 && k0 + 8 <= a.K) {
+          // 16-bit activations away from the row's end: one 16-byte load instead of five 2-byte ones
+          const u32x4 q = ((const Packed16*)((const uint16_t*)a.x + at))->v;
+          const unsigned h[5] = {q.x & 0xffffu, q.x >> 16, q.y & 0xffffu, q.y >> 16, q.z & 0xffffu};
+#pragma unroll
+          for (int d = 0; d < 5; ++d)
+            if (d >= lo && d < hi) xstage[i][d] = a.x_dtype == BP_BF16 ? bf16_bits_to_f32((uint16_t)h[d]) : f16_bits_to_f32((uint16_t)h[d]);
+          continue;
+        }
 #pragma unroll
         for (int d = 0; d < 5; ++d) {
           if (d >= lo && d < hi) {
@@ -104,16 +114,18 @@ __global__ __launch_bounds__(WAVES * 64, 4) void k_tq1_gemv(GemmArgs a, int CPT 
       const int u = threadIdx.x + i * THREADS;
       if (u < tile_slots) {
         const float x0 = xstage[i][0], x1 = xstage[i][1], x2 = xstage[i][2], x3 = xstage[i][3], x4 = xstage[i][4];
-        float t[36];
-#pragma unroll
-        for (int r = 0; r < 9; ++r) t[r] = (float)(r % 3 - 1) * x0 + (float)(r / 3 - 1) * x1;
-#pragma unroll
-        for (int q = 0; q < 27; ++q) t[9 + q] = (float)(q % 3 - 1) * x2 + (float)(q / 3 % 3 - 1) * x3 + (float)(q / 9 - 1) * x4;
+        // entry e of the slot: e < 9 -> T9[e], else T27[e - 9]; written four at a time
+        auto entry = [&](int en) -> unsigned {
+          if (en < 9) return __float_as_uint((float)(en % 3 - 1) * x0 + (float)(en / 3 - 1) * x1);
+          const int q = en - 9;
+          return __float_as_uint((float)(q % 3 - 1) * x2 + (float)(q / 3 % 3 - 1) * x3 + (float)(q / 9 - 1) * x4);
+        };
         const unsigned dst = (unsigned)(TB + u * G1_SLOT_BYTES);
 #pragma unroll
-        for (int w = 0; w < 9; ++w)
-          *(lds_u32x4*)(dst + 16 * w) = u32x4{__float_as_uint(t[4 * w]), __float_as_uint(t[4 * w + 1]), __float_as_uint(t[4 * w + 2]),
-                                              __float_as_uint(t[4 * w + 3])};
+        for (int w = 0; w < 9; ++w) {
+          *(lds_u32x4*)(dst + 16 * w) = u32x4{entry(4 * w), entry(4 * w + 1), entry(4 * w + 2), entry(4 * w + 3)};
+          __builtin_amdgcn_sched_barrier(0);  // one store's worth of values live at a time
+        }
       }
     }
   };
