@@ -211,8 +211,39 @@ def main() -> int:
         also["single_linear_us_per_call"] = round(w1 * 1e6, 2)
         also["single_linear_weight_GBps"] = round(wb1 / w1 / 1e9, 1)
         del l1
-        # grouped-expert prefill GEMM: TQ2, two stacked terms, top-6 skewed routing, 32 rows per expert on average
-        E3, N3, K3, T3, k3 = 96, 2048, 4096, 512, 6
+        # one MoE layer of config 2 (TQ1, H=4096, I=2048, 64 experts, top-6, bf16 activations) through TernaryMoE
+        from deepseekternarized_amd.moe import TernaryMoE
+
+        H2, I2, E2, k2 = 4096, 2048, 64, 6
+        gate = synth(bp, torch, E2, I2, H2, "tq1", 1, seed=5)
+        up = synth(bp, torch, E2, I2, H2, "tq1", 1, seed=6)
+        down = synth(bp, torch, E2, H2, I2, "tq1", 1, seed=7)
+        layer_bytes = sum(weight_bytes(*m) for m in (gate, up, down))
+        moe = TernaryMoE([(gate[0][0], gate[1][0])], [(up[0][0], up[1][0])], [(down[0][0], down[1][0])], H2, I2, k2, "tq1", GROUP, act="bf16")
+        del gate, up, down
+        gm = torch.Generator(device="cuda").manual_seed(8)
+        cfg2 = {}
+        for T2 in (1, 32, 256):
+            xt = torch.randn(T2, H2, device="cuda", generator=gm).to(torch.bfloat16)
+            lg = torch.randn(T2, E2, device="cuda", generator=gm) * 1.5
+            for _ in range(3):
+                moe(xt, lg)
+            torch.cuda.synchronize()
+            t0 = time.perf_counter()
+            reps = 20
+            for _ in range(reps):
+                moe(xt, lg)
+            torch.cuda.synchronize()
+            dt = (time.perf_counter() - t0) / reps
+            active = int(torch.unique(torch.topk(torch.softmax(lg.float(), -1), k2, -1).indices).numel())
+            cfg2[f"T{T2}"] = {"ms_per_layer": round(dt * 1e3, 4), "active_experts": active,
+                              "active_weight_GBps": round(layer_bytes / E2 * active / dt / 1e9, 1)}
+        also["cfg2_moe_layer"] = {"workload": f"TQ1 MoE layer H={H2} I={I2} E={E2} top-{k2}, bf16 activations: softmax/top-k, sort, gather, "
+                                              "gate|up grouped GEMM, SwiGLU, down grouped GEMM, weighted combine", **cfg2}
+        del moe
+        torch.cuda.empty_cache()
+        # grouped-expert prefill GEMM of config 3: TQ2, two stacked terms, all 384 experts, 2048 tokens top-6 (skewed routing)
+        E3, N3, K3, T3, k3 = 384, 2048, 4096, 2048, 6
         packed, scales = synth(bp, torch, E3, N3, K3, "tq2", 2, seed=3)
         ids = skewed_offsets(torch, T3, E3, k3, seed=3)
         order, offsets = bp.sort_by_expert(ids, E3)
@@ -223,7 +254,7 @@ def main() -> int:
         l3 = Launch(bp, torch, packed, scales, K3, "tq2", xg, offsets, max_rows)
         _, k3t, kn3 = l3.time(max(5, a.steps // 2), 2)
         flops = 2.0 * T3 * k3 * N3 * K3 * 2  # per-term count
-        also["grouped_gemm"] = {"workload": f"cfg3 gate projection at E={E3} of 384 experts: TQ2 k=2, N={N3}, K={K3}, "
+        also["grouped_gemm"] = {"workload": f"cfg3 gate projection, E={E3} experts: TQ2 k=2, N={N3}, K={K3}, "
                                             f"{T3 * k3} routed rows (max {max_rows}/expert), bf16 activations",
                                 "TFLOPs_per_term_count": round(flops / k3t / 1e12, 1),
                                 "frac_of_bf16_mfma_peak": round(flops / k3t / 1e12 / MFMA_BF16_PEAK_TFLOPS, 4),
@@ -250,6 +281,7 @@ def main() -> int:
         "config": {"workload": f"{a.workload}: {fmt.upper()} decode GEMV N={N} K={K} M={M} {act} activations, group 128, "
                                f"fp16 scales, {L} distinct linears per launch ({wbytes / 1e6:.0f} MB of weights, > Infinity Cache)",
                    "kernel": kname, "bytes_counted": "packed + fp16 scales as stored",
+                   "packed_only_GBps": round(wbytes * (1.0 - 2.0 * (K // GROUP) / (bp.packed_cols(fmt, K) + 2.0 * (K // GROUP))) / kern / 1e9, 1),
                    "activation_and_output_bytes_per_step": act_bytes},
         "roofline": {"bound": "hbm", "achieved": round(wbytes / kern / 1e9, 1), "peak": HBM_PEAK_GBPS, "unit": "GB/s",
                      "frac": round(wbytes / kern / 1e9 / HBM_PEAK_GBPS, 4), "traffic": MEASURED_TRAFFIC_BYTES.get(a.workload),
