@@ -233,8 +233,8 @@ __global__ __launch_bounds__(WAVES * 64, 4) void k_mfma_tq2(GemmArgs a, int KC, 
       fetch_s(0, snext);
     }
     for (int ch = 0; ch < chunks; ++ch) {
-      if (restage) {
-        __syncthreads();  // every wave is done reading the previous tile 
+      if (restage && !((AB == 6 || AB2 == 6) && ch > 0)) {  // (ablation 6: the tile is staged once, results are wrong)
+        __syncthreads();  // every wave is done reading the previous tile
         stage_store();
         __syncthreads();
         if (ch + 1 < chunks) stage_load((int64_t)(ch + 1) * KC);
@@ -365,10 +365,12 @@ int launch_tq2(const GemmArgs& a, hipStream_t s, const char* name) {
   if (kc < 1024) return fail(BP_ERR_UNSUPPORTED, "activation tile does not fit");
   const size_t stile = SL ? (size_t)rows_per_wg * a.G * (SDT == BP_F32 ? 4 : 2) : 0;
   const size_t lds = X_BASE + (size_t)tokens * (kc * XB + 16) + (size_t)(kc / 128) * 16 * MT * 4 + stile;
+  constexpr int lds_cap = X_BASE + XKB * 1024 + (SL ? TQ2_SCALE_TILE_MAX : 0) < 160 * 1024 ? X_BASE + XKB * 1024 + (SL ? TQ2_SCALE_TILE_MAX : 0) : 160 * 1024;
+  if (lds > (size_t)lds_cap) return BP_ERR_UNSUPPORTED;  // (scale tile variant: the caller falls back to scales from global memory)
   static bool attr = false;
   if (!attr) {
     if (hipFuncSetAttribute((const void*)k_mfma_tq2<ACT, SDT, R, MT, WAVES, XKB, ABL, NQ, SL>, hipFuncAttributeMaxDynamicSharedMemorySize,
-                            X_BASE + XKB * 1024 + (SL ? TQ2_SCALE_TILE_MAX : 0)) != hipSuccess)
+                            lds_cap) != hipSuccess)
       return fail(BP_ERR_LAUNCH, "cannot raise the dynamic LDS limit");
     attr = true;
   }
@@ -382,9 +384,11 @@ int launch_tq2_sd(const GemmArgs& a, hipStream_t s, const char* name) {
   // scales through LDS whenever the workgroup's share of one term fits the budget
   const int64_t tile = (int64_t)WAVES * 16 * R * a.G * (a.scale_dtype == BP_F32 ? 4 : 2);
   if (tile <= TQ2_SCALE_TILE_MAX) {
-    if (a.scale_dtype == BP_F16) return launch_tq2<ACT, BP_F16, R, MT, WAVES, XKB, 0, NQ, 1>(a, s, name);
-    if (a.scale_dtype == BP_BF16) return launch_tq2<ACT, BP_BF16, R, MT, WAVES, XKB, 0, NQ, 1>(a, s, name);
-    return launch_tq2<ACT, BP_F32, R, MT, WAVES, XKB, 0, NQ, 1>(a, s, name);
+    int rc;
+    if (a.scale_dtype == BP_F16) rc = launch_tq2<ACT, BP_F16, R, MT, WAVES, XKB, 0, NQ, 1>(a, s, name);
+    else if (a.scale_dtype == BP_BF16) rc = launch_tq2<ACT, BP_BF16, R, MT, WAVES, XKB, 0, NQ, 1>(a, s, name);
+    else rc = launch_tq2<ACT, BP_F32, R, MT, WAVES, XKB, 0, NQ, 1>(a, s, name);
+    if (rc != BP_ERR_UNSUPPORTED) return rc;
   }
   if (a.scale_dtype == BP_F16) return launch_tq2<ACT, BP_F16, R, MT, WAVES, XKB, 0, NQ, 0>(a, s, name);
   if (a.scale_dtype == BP_BF16) return launch_tq2<ACT, BP_BF16, R, MT, WAVES, XKB, 0, NQ, 0>(a, s, name);
@@ -396,6 +400,16 @@ int launch_tq2_sd(const GemmArgs& a, hipStream_t s, const char* name) {
 int launch_mfma_tq2(const GemmArgs& a, hipStream_t s, int R, int MT, int waves) {
   const bool bf = a.x_dtype == BP_BF16;
   if (const char* t = getenv("BP_TUNE_ABL")) {
+    if (bf && a.scale_dtype == BP_F16 && MT == 2) {
+      switch (atoi(t)) {
+        case 2: return launch_tq2<BP_BF16, BP_F16, 1, 2, 16, 112, 2>(a, s, "abl2_m2");
+        case 3: return launch_tq2<BP_BF16, BP_F16, 1, 2, 16, 112, 3>(a, s, "abl3_m2");
+        case 4: return launch_tq2<BP_BF16, BP_F16, 1, 2, 16, 112, 4>(a, s, "abl4_m2");
+        case 5: return launch_tq2<BP_BF16, BP_F16, 1, 2, 16, 112, 5>(a, s, "abl5_m2");
+        case 6: return launch_tq2<BP_BF16, BP_F16, 1, 2, 16, 112, 6>(a, s, "abl6_m2");
+        default: break;
+      }
+    }
     if (bf && a.scale_dtype == BP_F16 && MT == 1) {
       switch (atoi(t)) {
         case 1: return launch_tq2<BP_BF16, BP_F16, 1, 1, 16, 48, 1>(a, s, "abl1_w16");
