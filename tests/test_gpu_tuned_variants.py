@@ -1,0 +1,157 @@
+"""Every code path of the tuned kernels (bp_mfma_tq2.hip, bp_mfma_tq1.hip, bp_tq1_gemv.hip) against the CPU oracle.
+
+The shapes are chosen by what they select inside the launchers, not by size: odd / even packed row
+lengths (row starts at every byte alignment), K that fits one activation / table tile or needs several,
+scales through the LDS tile or - misaligned, or too many groups - from global memory, one or two stacked
+terms, every activation dtype, empty experts, N not a multiple of the rows of a workgroup.
+"""
+
+import numpy as np
+import pytest
+import torch
+
+from _util import c_gemm, orc, rel_l2, synth_weights
+
+pytestmark = pytest.mark.gpu
+
+REL_L2 = 1e-3
+GROUP = 128
+
+
+@pytest.fixture(scope="module")
+def bp():
+    import deepseekternarized_amd as m
+
+    assert torch.cuda.is_available() and m.ext() is not None
+    return m
+
+
+def dev(a):
+    return torch.from_numpy(np.ascontiguousarray(a)).cuda()
+
+
+def _activations(rng, T, K, act):
+    x = rng.standard_normal((T, K)).astype(np.float32)
+    if act == "int8":
+        q, s = orc.quant_act_int8(x)
+        return q, s, dev(q), dev(s)
+    if act == "bf16":
+        x = orc.bf16_round(x)
+        return x, None, dev(x).to(torch.bfloat16), None
+    if act == "f16":
+        x = x.astype(np.float16).astype(np.float32)
+        return x, None, dev(x).half(), None
+    return x, None, dev(x), None
+
+
+def _run(bp, fmt, E, N, K, counts, act, terms=1, seed=0, misalign_scales=False, scale_dtype=np.float16):
+    """Grouped call with `counts[e]` rows per expert; returns (got, want, kernel name)."""
+    rng = np.random.default_rng(seed)
+    packed, scales = synth_weights(seed, E, N, K, GROUP, fmt, terms=terms)
+    offsets = np.concatenate([[0], np.cumsum(counts)]).astype(np.int64)
+    T = int(offsets[-1])
+    x, xs, xd, xsd = _activations(rng, T, K, act)
+    want = np.zeros((T, N), np.float32)
+    for e in range(E):
+        a, b = int(offsets[e]), int(offsets[e + 1])
+        for p, s in zip(packed, scales):
+            if b > a:
+                c_gemm(x[a:b], None if xs is None else xs[a:b], p[e], s[e].astype(np.float32), K, GROUP, fmt, out=want[a:b])
+    pk = [dev(p) for p in packed]
+    if scale_dtype is np.float16:
+        sc = [dev(s) for s in scales]
+    else:
+        sc = [dev(s.astype(np.float32)).to(torch.bfloat16) for s in scales]
+        # the oracle must see the rounded scales
+        want[:] = 0
+        for e in range(E):
+            a, b = int(offsets[e]), int(offsets[e + 1])
+            for p, s in zip(packed, sc):
+                if b > a:
+                    c_gemm(x[a:b], None if xs is None else xs[a:b], p[e], s[e].float().cpu().numpy(), K, GROUP, fmt, out=want[a:b])
+    if misalign_scales:  # a view whose data pointer is 4- but not 16-byte aligned
+        moved = []
+        for s in sc:
+            flat = torch.empty(s.numel() + 2, dtype=s.dtype, device="cuda")
+            flat[2:].copy_(s.reshape(-1))
+            moved.append(flat[2:].view(s.shape))
+            assert moved[-1].data_ptr() % 16 == 4
+        sc = moved
+    got = bp.grouped_ternary_gemm(xd, xsd, offsets.tolist(), pk, sc, K, GROUP, fmt)  # host offsets: max_rows = widest expert
+    return got.cpu().numpy(), want, bp.ext().last_kernel()
+
+
+def _check(got, want):
+    assert np.isfinite(got).all()
+    assert rel_l2(got, want) <= REL_L2, rel_l2(got, want)
+
+
+# --------------------------------------------------------------------------- TQ1 decode GEMV (table lookup)
+@pytest.mark.parametrize("K", [1024, 1280, 2048, 4352, 7168])  # Kp = 205 (odd: rows at every byte alignment), 256, 410, 871, 1434
+@pytest.mark.parametrize("act", ["bf16", "int8"])
+def test_tq1_gemv_row_alignments_and_tiles(bp, K, act):
+    got, want, kern = _run(bp, "tq1", 3, 48, K, [1, 0, 1], act, seed=K)
+    assert kern.startswith("lut_tq1"), kern
+    _check(got, want)
+
+
+@pytest.mark.parametrize("act", ["f16", "f32"])
+def test_tq1_gemv_other_activation_dtypes(bp, act):
+    got, want, kern = _run(bp, "tq1", 2, 32, 2048, [1, 1], act, seed=3)
+    assert kern.startswith("lut_tq1"), kern
+    _check(got, want)
+
+
+def test_tq1_gemv_many_rows_two_terms_bf16_scales(bp):
+    """N spans several workgroups and is not a multiple of their rows; two stacked terms; bf16 scales."""
+    got, want, kern = _run(bp, "tq1", 2, 2048 + 48, 2304, [1, 1], "bf16", terms=2, seed=5, scale_dtype=np.float32)
+    assert kern.startswith("lut_tq1"), kern
+    _check(got, want)
+
+
+def test_tq1_gemv_scales_from_global_memory(bp):
+    """Scale pointers that are not 16-byte aligned, and K with more groups than the LDS tile takes."""
+    got, want, kern = _run(bp, "tq1", 2, 32, 2048, [1, 1], "bf16", seed=6, misalign_scales=True)
+    assert kern.endswith("_gs"), kern
+    _check(got, want)
+    got, want, kern = _run(bp, "tq1", 1, 272, 40960, [1], "bf16", seed=7)  # G = 320: 256 rows x 640 B of scales do not fit
+    assert kern.startswith("lut_tq1"), kern
+    _check(got, want)
+
+
+# --------------------------------------------------------------------------- TQ1 MFMA kernel (2..16 rows per tile)
+@pytest.mark.parametrize("K", [1024, 2048, 7168])
+@pytest.mark.parametrize("counts", [[2, 0, 5], [16, 3, 1], [20, 1, 37]])
+def test_tq1_mfma_tiles(bp, K, counts):
+    got, want, kern = _run(bp, "tq1", 3, 80, K, counts, "bf16", terms=2, seed=K + sum(counts))
+    assert kern.startswith("mfma_tq1"), kern
+    _check(got, want)
+
+
+def test_tq1_mfma_scales_from_global_memory(bp):
+    got, want, kern = _run(bp, "tq1", 2, 32, 2048, [3, 4], "bf16", seed=8, misalign_scales=True)
+    assert kern.startswith("mfma_tq1") and kern.endswith("_gs"), kern
+    _check(got, want)
+
+
+# --------------------------------------------------------------------------- TQ2 MFMA kernel
+@pytest.mark.parametrize("act", ["bf16", "int8"])
+@pytest.mark.parametrize("K,counts", [(1024, [1, 0, 1]), (2048, [1, 1, 1]), (7168, [3, 0, 16]), (4096, [33, 1, 20]), (32768, [1, 2, 0])])
+def test_tq2_mfma_variants(bp, act, K, counts):
+    """Single-token, 16-token and 32-token tiles; K = 32768 has more scales per row than the LDS tile takes."""
+    got, want, kern = _run(bp, "tq2", 3, 2048 + 16 if K <= 2048 else 64, K, counts, act, terms=2 if K == 4096 else 1, seed=K + len(act))
+    assert kern.startswith("mfma_tq2"), kern
+    _check(got, want)
+
+
+def test_tq2_bf16_scales_and_f32_scales(bp):
+    got, want, kern = _run(bp, "tq2", 2, 64, 2048, [1, 9], "bf16", seed=11, scale_dtype=np.float32)
+    assert kern.startswith("mfma_tq2"), kern
+    _check(got, want)
+    # float32 scales through the mirrored API
+    packed, scales = synth_weights(12, 1, 64, 2048, GROUP, "tq2")
+    x = orc.bf16_round(np.random.default_rng(12).standard_normal((5, 2048)).astype(np.float32))
+    want = c_gemm(x, None, packed[0][0], scales[0][0].astype(np.float32), 2048, GROUP, "tq2")
+    got = bp.ternary_gemm_float(dev(x).to(torch.bfloat16), dev(packed[0][0]), dev(scales[0][0]).float(), 2048, GROUP, "tq2")
+    assert bp.ext().last_kernel().startswith("mfma_tq2")
+    _check(got.cpu().numpy(), want)
