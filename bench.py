@@ -136,9 +136,23 @@ def cpu_baseline(fmt, N, K, M, budget_s=12.0):
     dt = (time.perf_counter() - t0) / reps
     wbytes = packed.size + 2 * scale.size
     cores = oracle_c().bp_oracle_max_threads()
+    # the same kernel at 4 threads, the reference's habitual setting (docs/reports/M2.md:114, boilerplate/cli.py:384)
+    import torch
+
+    before = torch.get_num_threads()
+    torch.set_num_threads(4)  # sets the OpenMP team size the compiled reference kernel uses
+    fn4 = fn if kind == "reference" else (lambda: c_gemm(x, None, packed, scale, K, GROUP, fmt, threads=4))
+    fn4()
+    r4, t1 = 0, time.perf_counter()
+    while time.perf_counter() - t1 < budget_s / 3 and r4 < 20000:
+        fn4()
+        r4 += 1
+    dt4 = (time.perf_counter() - t1) / r4
+    torch.set_num_threads(before)
     return {"value": round(wbytes / dt / 1e9, 3), "unit": "GB/s", "cores": int(cores), "kind": kind,
             "sample": f"one {fmt} linear N={N} K={K} M={M} fp32 activations, {reps} calls, {dt * 1e3:.3f} ms/call, "
-                      f"OpenMP over all {cores} host threads (os.cpu_count()={os.cpu_count()})"}
+                      f"OpenMP over all {cores} host threads (os.cpu_count()={os.cpu_count()})",
+            "value_4_threads": round(wbytes / dt4 / 1e9, 3)}
 
 
 def skewed_offsets(torch, T, E, k, seed=0):
