@@ -22,6 +22,8 @@ namespace bp {
 // implemented in bp_mfma_tq2.hip / bp_mfma_tq1.hip; R, MT, waves: the tiling chosen by launch_mfma
 int launch_mfma_tq2(const GemmArgs& a, hipStream_t s, int R, int MT, int waves);
 int launch_mfma_tq1(const GemmArgs& a, hipStream_t s, int waves);
+// bp_gemm_tq2.hip: TQ2 with token tiles of 32 (experts with more than 16 token rows)
+int launch_gemm_tq2(const GemmArgs& a, hipStream_t s);
 // bp_tq1_gemv.hip: TQ1, one token row per expert (max_rows == 1), bf16 activations, table-lookup GEMV
 int launch_tq1_gemv(const GemmArgs& a, hipStream_t s, int waves);
 

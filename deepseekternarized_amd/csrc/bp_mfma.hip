@@ -34,10 +34,11 @@ int launch_mfma(const GemmArgs& a, hipStream_t s) {
   // steady state; the TQ2 single-token kernels are light enough on registers for that to win everywhere.
   int waves = work >= 2048 && !(a.fmt == BP_TQ2 && a.max_rows == 1) ? 16 : 8;
   // development overrides (tuning sweeps)
-  if (const char* t = getenv("BP_TUNE_R")) { const int v = atoi(t); if (v == 1 || v == 2) R = v; }
+  if (const char* t = getenv("BP_TUNE_R")) { const int v = atoi(t); if (v == 1 || v == 2 || v == 4) R = v; }
   if (const char* t = getenv("BP_TUNE_WAVES")) { const int v = atoi(t); if (v == 8 || v == 16) waves = v; }
   if (const char* t = getenv("BP_TUNE_MT")) { const int v = atoi(t); if (v == 1 || v == 2) MT = v; }
   if (a.fmt == BP_TQ1) return launch_mfma_tq1(a, s, waves);
+  if (a.max_rows > 16 && !getenv("BP_TUNE_MT") && !getenv("BP_TUNE_R")) return launch_gemm_tq2(a, s);
   return launch_mfma_tq2(a, s, R, MT, waves);
 }
 

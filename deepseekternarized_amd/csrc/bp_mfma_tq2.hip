@@ -1,51 +1,14 @@
 // TQ2 (4 trits per byte) on MFMA: table-free decode, activations and scales staged through LDS.
 #include "bp_mfma.h"
+#include "bp_tq2_decode.h"
 
 namespace bp {
 namespace {
 
 // The activation tile starts at LDS address 0: row t at t * pitch, pitch = KC * XB + 16.
 constexpr int X_BASE = 0;
-constexpr int TQ2_SCALE_TILE_MAX = 40 * 1024;  // LDS budget for a workgroup's scales (beyond it: read from global memory)
-
-// ---- TQ2 decode without a table.
-// bf16: a 2-bit code u placed at bits [7:6] of a bf16 whose other bits are 0x4000 reads 2 + u (the code
-// spans the lowest exponent bit and the highest mantissa bit: 2, 3, 4); placed at bits [5:4] of 0x4100 it
-// reads 8 + u. One v_and_or_b32 per output dword therefore turns two codes of a packed dword (one per
-// 16-bit half) into two bf16 values; three shifts bring all 16 codes of the dword to those two positions.
-// The products then carry sum(x * (c + u)) with c = 2 (odd trits) or 8 (even trits); the accumulator of
-// every group starts from -sum(x * (c + 1)), computed once per workgroup when the activation tile is
-// staged, which leaves sum(x * (u - 1)). Slot order of the two operands made from a packed dword (codes
-// c0..c15, lo/hi bf16 of each operand dword):
-//   first  : (c3,c11) (c2,c10) (c1,c9) (c0,c8)      second : (c5,c13) (c4,c12) (c7,c15) (c6,c14)
-// The activation tile is stored in LDS in that order (permuted inside every 16 elements when staged).
-// The unused code 3 reads +3 or +2 depending on its slot (pack never writes it).
-struct Tq2Consts { unsigned P1, P2, M1, M2; };  // 0x00c000c0, 0x00300030, 0x40004000, 0x41004100 held in registers
-__device__ __forceinline__ void tq2_decode_bf16(unsigned w, const Tq2Consts& k, u32x4& first, u32x4& second) {
-  const unsigned P1 = k.P1, P2 = k.P2, M1 = k.M1, M2 = k.M2;
-  const unsigned wl = w << 4, wr = w >> 4, wr8 = w >> 8;
-  first = u32x4{(w & P1) | M1, (w & P2) | M2, (wl & P1) | M1, (wl & P2) | M2};
-  second = u32x4{(wr & P1) | M1, (wr & P2) | M2, (wr8 & P1) | M1, (wr8 & P2) | M2};
-}
-// int8: dword i of the operand = codes c(i), c(i+4), c(i+8), c(i+12) as digits 0..2; the accumulator
-// starts from -sum(x). The activation tile is stored with every 16 bytes transposed 4 x 4 to match.
-__device__ __forceinline__ u32x4 tq2_decode_i8(unsigned w) {
-  const unsigned m = 0x03030303u;
-  return u32x4{w & m, (w >> 2) & m, (w >> 4) & m, (w >> 6) & m};
-}
-__device__ __forceinline__ void tq2_permute_bf16(const u32x4 a, const u32x4 c, u32x4& o0, u32x4& o1) {
-  const unsigned HI = 0x07060302u, LO = 0x05040100u;
-  o0 = u32x4{__builtin_amdgcn_perm(c.y, a.y, HI), __builtin_amdgcn_perm(c.y, a.y, LO),
-             __builtin_amdgcn_perm(c.x, a.x, HI), __builtin_amdgcn_perm(c.x, a.x, LO)};
-  o1 = u32x4{__builtin_amdgcn_perm(c.z, a.z, HI), __builtin_amdgcn_perm(c.z, a.z, LO),
-             __builtin_amdgcn_perm(c.w, a.w, HI), __builtin_amdgcn_perm(c.w, a.w, LO)};
-}
-__device__ __forceinline__ u32x4 tq2_permute_i8(const u32x4 a) {
-  const unsigned s0 = __builtin_amdgcn_perm(a.y, a.x, 0x05010400u), s1 = __builtin_amdgcn_perm(a.y, a.x, 0x07030602u);
-  const unsigned s2 = __builtin_amdgcn_perm(a.w, a.z, 0x05010400u), s3 = __builtin_amdgcn_perm(a.w, a.z, 0x07030602u);
-  return u32x4{__builtin_amdgcn_perm(s2, s0, 0x05040100u), __builtin_amdgcn_perm(s2, s0, 0x07060302u),
-               __builtin_amdgcn_perm(s3, s1, 0x05040100u), __builtin_amdgcn_perm(s3, s1, 0x07060302u)};
-}
+// LDS budget for a workgroup's scales (beyond it: read from global memory)
+constexpr int tq2_scale_tile_max(int R) { return R >= 4 ? 64 * 1024 : 40 * 1024; }
 
 // ------------------------------------------------------------------------------------------------
 // TQ2. K % 1024 == 0, N % 16 == 0. One step = 64 packed bytes (256 trits, two groups) per row.
@@ -54,7 +17,7 @@ __device__ __forceinline__ u32x4 tq2_permute_i8(const u32x4 a) {
 // second, so that all four k-blocks of an MFMA belong to one scale group.
 // After the swap block b holds trits tb(b) .. tb(b)+31 of each group, tb = {0, 64, 32, 96}.
 template <int ACT, int SDT, int R, int MT, int WAVES, int XKB, int ABL = 0, int NQ = 4, int SL = 1>
-__global__ __launch_bounds__(WAVES * 64, 4) void k_mfma_tq2(GemmArgs a, int KC, int tile_rows) {
+__global__ __launch_bounds__(WAVES * 64, (WAVES == 8 && R >= 2 && MT == 2) ? 2 : 4) void k_mfma_tq2(GemmArgs a, int KC, int tile_rows) {
   constexpr int THREADS = WAVES * 64;
   constexpr int XB = ACT == BP_BF16 ? 2 : 1;   // bytes per activation element
   constexpr int KM = ACT == BP_BF16 ? 8 : 16;  // k per lane per MFMA
@@ -365,7 +328,8 @@ int launch_tq2(const GemmArgs& a, hipStream_t s, const char* name) {
   if (kc < 1024) return fail(BP_ERR_UNSUPPORTED, "activation tile does not fit");
   const size_t stile = SL ? (size_t)rows_per_wg * a.G * (SDT == BP_F32 ? 4 : 2) : 0;
   const size_t lds = X_BASE + (size_t)tokens * (kc * XB + 16) + (size_t)(kc / 128) * 16 * MT * 4 + stile;
-  constexpr int lds_cap = X_BASE + XKB * 1024 + (SL ? TQ2_SCALE_TILE_MAX : 0) < 160 * 1024 ? X_BASE + XKB * 1024 + (SL ? TQ2_SCALE_TILE_MAX : 0) : 160 * 1024;
+  constexpr int lds_want = X_BASE + XKB * 1024 + (SL ? tq2_scale_tile_max(R) : 0);
+  constexpr int lds_cap = lds_want < 160 * 1024 ? lds_want : 160 * 1024;
   if (lds > (size_t)lds_cap) return BP_ERR_UNSUPPORTED;  // (scale tile variant: the caller falls back to scales from global memory)
   static bool attr = false;
   if (!attr) {
@@ -383,7 +347,7 @@ template <int ACT, int R, int MT, int WAVES, int XKB, int NQ = 4>
 int launch_tq2_sd(const GemmArgs& a, hipStream_t s, const char* name) {
   // scales through LDS whenever the workgroup's share of one term fits the budget
   const int64_t tile = (int64_t)WAVES * 16 * R * a.G * (a.scale_dtype == BP_F32 ? 4 : 2);
-  if (tile <= TQ2_SCALE_TILE_MAX) {
+  if (tile <= tq2_scale_tile_max(R)) {
     int rc;
     if (a.scale_dtype == BP_F16) rc = launch_tq2<ACT, BP_F16, R, MT, WAVES, XKB, 0, NQ, 1>(a, s, name);
     else if (a.scale_dtype == BP_BF16) rc = launch_tq2<ACT, BP_BF16, R, MT, WAVES, XKB, 0, NQ, 1>(a, s, name);
@@ -425,7 +389,7 @@ int launch_mfma_tq2(const GemmArgs& a, hipStream_t s, int R, int MT, int waves) 
       }
     }
   }
-  if (MT == 2) waves = 16;  // the 32-token tile needs the large LDS budget of a 16-wave workgroup
+  if (MT == 2 && !(waves == 8 && R >= 2)) waves = 16;  // the 32-token tile needs the large LDS budget of a 16-wave workgroup
   if (a.max_rows == 1 && R == 2 && MT == 1 && waves == 16) {
     if (bf) return launch_tq2_sd<BP_BF16, 2, 1, 16, 48, 1>(a, s, "mfma_tq2_bf16_r2_t1_w16");
     return launch_tq2_sd<BP_I8, 2, 1, 16, 48, 1>(a, s, "mfma_tq2_i8_r2_t1_w16");
@@ -443,7 +407,8 @@ int launch_mfma_tq2(const GemmArgs& a, hipStream_t s, int R, int MT, int waves) 
 #define BP_ALL(ACTV, NAME)                                                        \
   BP_CASE(ACTV, 1, 1, 8, 48, NAME) BP_CASE(ACTV, 2, 1, 8, 48, NAME)                \
   BP_CASE(ACTV, 1, 1, 16, 48, NAME) BP_CASE(ACTV, 2, 1, 16, 48, NAME)              \
-  BP_CASE(ACTV, 1, 2, 16, 112, NAME) BP_CASE(ACTV, 2, 2, 16, 112, NAME)
+  BP_CASE(ACTV, 1, 2, 16, 112, NAME) BP_CASE(ACTV, 2, 2, 16, 112, NAME)            \
+  BP_CASE(ACTV, 2, 2, 8, 112, NAME) BP_CASE(ACTV, 4, 2, 8, 80, NAME)
   if (bf) { BP_ALL(BP_BF16, "mfma_tq2_bf16") } else { BP_ALL(BP_I8, "mfma_tq2_i8") }
 #undef BP_ALL
 #undef BP_CASE
