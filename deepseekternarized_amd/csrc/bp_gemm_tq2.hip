@@ -5,12 +5,15 @@
 // cores and the LDS, not HBM, set the pace:
 //  * 8 waves per workgroup, two 16-row sub-tiles per wave: the decoded weights of a lane meet 32 tokens,
 //    and every activation operand read from LDS feeds two MFMAs. Two waves per SIMD leave each wave 256
-//    registers, enough to read the next group's operands while the current group is decoded and multiplied.
+//    registers.
 //  * The activation tile is stored fragment-major: the 64 x 16 bytes that one MFMA takes as operand A are
 //    one contiguous KiB in lane order, so an operand read is conflict-free (a token-major tile with a
 //    padded pitch costs 1.6x the LDS time of this layout on gfx950).
-//  * Two activation tiles when LDS allows: the next 1024 k are staged while the current tile is multiplied,
-//    with one barrier per tile.
+//  * Two activation tiles in LDS: the next 1024 k are loaded to registers while the current tile is
+//    multiplied and stored when it ends, with one barrier per tile.
+//  * Workgroups that share an expert's activations run on the same XCD (one L2).
+#include <type_traits>
+
 #include "bp_mfma.h"
 #include "bp_tq2_decode.h"
 
@@ -42,7 +45,6 @@ __global__ __launch_bounds__(GTHREADS, 2) void k_gemm_tq2(GemmArgs a) {
   constexpr int SB = SDT == BP_F32 ? 4 : 2;
   constexpr int PF = 4;  // steps per activation tile
   constexpr int RD = 4;  // steps of packed weights in flight per row sub-tile
-  constexpr int XP = 0;  // 1: operands of the next group are read while the current group is multiplied (64 more registers)
   static_assert(16 * (GKC / 32) == GTHREADS, "one staging item (32 elements of one token) per thread and token sub-tile");
   typedef typename Acc<ACT>::type acc_t;
 
@@ -59,7 +61,7 @@ __global__ __launch_bounds__(GTHREADS, 2) void k_gemm_tq2(GemmArgs a) {
   const int64_t tok0 = o0 + (int64_t)blockIdx.z * (16 * GT);
   if (tok0 >= o1) return;  // uniform for the workgroup
   const int ntok = (int)(o1 - tok0 < 16 * GT ? o1 - tok0 : 16 * GT);
-  const bool two = ntok > 16;  // the second token sub-tile holds tokens (when not, it is multiplied all the same: its LDS content is stale, its sums are never stored)
+  const bool two = ntok > 16;  // the second token sub-tile holds tokens
   int64_t n0 = ((int64_t)wg_tile * GW + wave) * (16 * GR);
   const bool wave_live = n0 < a.N;
   if (!wave_live) n0 = 0;
@@ -76,17 +78,17 @@ __global__ __launch_bounds__(GTHREADS, 2) void k_gemm_tq2(GemmArgs a) {
   const int sq = (lane >> 4), sg = wave;
   const int sb = ((sq & 1) << 1) | (sq >> 1);  // k-block that holds elements 32 q .. 32 q + 31 of a group
   const unsigned char* xg = (const unsigned char*)a.x + tok0 * a.K * XB;
-  // One register set holds half a tile's share (one token sub-tile) at a time: the halves are loaded and
-  // stored in turn while the current tile is multiplied.
+  // The thread's share of the next tile (one item per token sub-tile) is loaded when the current tile starts
+  // and stored to the other LDS tile when it ends: a whole tile time hides the load latency.
   // Loads: an instruction reads, per token row, the four 16-byte pieces of a 64-byte segment with four
   // lanes (16 rows x 64 B: 16 memory requests; one lane per 64-byte item would make 64). bf16: a 16-element
   // permutation unit is two pieces; lanes l and l + 32 hold the two pieces of a unit and trade them with
   // v_permlane32_swap, the lower half of the wave ending with the units of one segment, the upper half
   // with those of the next.
-  u32x4 xs[2][XB];
+  u32x4 xsr[GT][2][XB];
   auto stage_load = [&](int64_t k0, int mt) {
     if (mt == 1 && !two) return;
-    if (ABL / 10 == 1) { asm volatile("" : "+v"(xs[0][0]), "+v"(xs[1][0]), "+v"(xs[0][XB - 1]), "+v"(xs[1][XB - 1])); return; }  // (timing: no activation loads)
+    auto& xs = xsr[mt];
     int row = 16 * mt + r16;
     if (row >= ntok) row = ntok - 1;
     const unsigned char* p = xg + ((int64_t)row * a.K + k0 + sg * 128) * XB;
@@ -111,6 +113,7 @@ __global__ __launch_bounds__(GTHREADS, 2) void k_gemm_tq2(GemmArgs a) {
   };
   auto stage_store = [&](int buf, int mt) {
     if (mt == 1 && !two) return;
+    auto& xs = xsr[mt];
     const unsigned tile = (unsigned)(buf * TILE);
     unsigned part;
     float f = 0.f;
@@ -176,24 +179,12 @@ __global__ __launch_bounds__(GTHREADS, 2) void k_gemm_tq2(GemmArgs a) {
   stage_store(0, 0);
   stage_load(0, 1);
   stage_store(0, 1);
-  if (tiles > 1) stage_load(tile_k0(1), 0);
+  if (tiles > 1) {
+    stage_load(tile_k0(1), 0);
+    stage_load(tile_k0(1), 1);
+  }
   __syncthreads();
   int seq = 0;  // tiles consumed so far
-  // ABL 9 (timing experiments): wave `blockIdx.z` of workgroup (1, 0, 0) writes clock stamps over the output
-  const bool dbg = ABL % 10 == 9 && wg_tile == 1 && e == 0 && blockIdx.z == 0 && wave == 3 && lane == 0;
-  long long* dbgp = (long long*)a.out;
-  int dbgn = 0;
-  auto stamp = [&]() {
-    if (ABL % 10 == 9) {
-      __builtin_amdgcn_sched_barrier(0);
-      const long long t = clock64();
-      if (dbg && dbgn < 400) *(__attribute__((address_space(3))) long long*)(156 * 1024 + 8 * dbgn) = t;  // (LDS: a store to memory would be waited for)
-      ++dbgn;
-      __builtin_amdgcn_sched_barrier(0);
-    }
-  };
-  stamp();
-
   for (int term = 0; term < a.n_terms; ++term) {
     const int64_t rows_here = a.N - n0 < 16 * GR ? a.N - n0 : 16 * GR;
     const __amdgpu_buffer_rsrc_t wrs = make_rsrc(a.packed[term] + (e * a.N + n0) * a.Kp, rows_here * a.Kp);
@@ -207,7 +198,7 @@ __global__ __launch_bounds__(GTHREADS, 2) void k_gemm_tq2(GemmArgs a) {
       const int cc = c < steps ? c : steps - 1;
 #pragma unroll
       for (int r = 0; r < GR; ++r) {
-        if (ABL == 5 || ABL / 10 == 5) { asm volatile("" : "+v"(dst[r])); continue; }
+        if (ABL == 5) { asm volatile("" : "+v"(dst[r])); continue; }
         dst[r] = buf_load16(wrs, woff, (unsigned)(row_shift[r] * a.Kp) + 64u * cc);
       }
     };
@@ -256,116 +247,108 @@ __global__ __launch_bounds__(GTHREADS, 2) void k_gemm_tq2(GemmArgs a) {
       const int c4 = ch * PF;
       fetch_s(c4 + PF, snext);
 
-      u32x4 xa[1 + XP][NJ][GT];
-      acc_t base[1 + XP][GT];
-      auto load_x = [&](int gl, u32x4 (&dx)[NJ][GT], acc_t (&db)[GT]) {
+      // The four steps of the tile, for MTN token sub-tiles (a tile of at most 16 tokens skips the second one).
+      auto run_steps = [&](auto mtn_c) {
+        constexpr int MTN = decltype(mtn_c)::value;
+        // One group's operands at a time; the compiler hoists these reads ahead of the previous group's MFMAs as
+        // far as registers allow (an explicit second operand buffer costs 40 registers and spills the staging data).
+        u32x4 xa[NJ][GT];
+        acc_t base[GT];
+        auto load_x = [&](int gl, u32x4 (&dx)[NJ][GT], acc_t (&db)[GT]) {
 #pragma unroll
-        for (int mt = 0; mt < GT; ++mt) {
-          if (ABL == 3) {
-            db[mt] = acc_t{0, 0, 0, 0};
+          for (int mt = 0; mt < MTN; ++mt) {
+            if (ABL == 3) {
+              db[mt] = acc_t{0, 0, 0, 0};
 #pragma unroll
-            for (int j = 0; j < NJ; ++j) dx[j][mt] = u32x4{kc.M1, kc.M2, kc.M1, kc.M2};
-            continue;
-          }
-          db[mt] = __builtin_bit_cast(acc_t, *(const lds_u32x4*)(cbase + (gl * (16 * GT) + 16 * mt) * 4));
-#pragma unroll
-          for (int j = 0; j < NJ; ++j) dx[j][mt] = *(const lds_u32x4*)(xbase + ((gl * NJ + j) * GT + mt) * 1024);
-        }
-      };
-      stamp();  // chunk start
-      if (XP) load_x(0, xa[0], base[0]);
-#pragma unroll
-      for (int i = 0; i < PF; ++i) {
-        __builtin_amdgcn_sched_barrier(0);
-        const int c = c4 + i;
-        u32x4 w[GR];
-#pragma unroll
-        for (int r = 0; r < GR; ++r) {  // regroup: .x/.y = 8 bytes of group 2c, .z/.w = 8 bytes of group 2c+1
-          const auto s0 = __builtin_amdgcn_permlane32_swap(ring[i % RD][r].x, ring[i % RD][r].z, false, false);
-          const auto s1 = __builtin_amdgcn_permlane32_swap(ring[i % RD][r].y, ring[i % RD][r].w, false, false);
-          w[r] = u32x4{s0[0], s1[0], s0[1], s1[1]};
-        }
-#pragma unroll
-        for (int h = 0; h < 2; ++h) {
-          const int gl = 2 * i + h, cur = XP ? (gl & 1) : 0;
-          // next group's operands: issued here, ahead of this group's decode and MFMAs (the scheduling barrier keeps
-          // the compiler from sinking the reads to their first use, where their latency would be exposed)
-          if (XP) {
-            if (gl + 1 < 2 * PF) load_x(gl + 1, xa[(cur ^ 1) & XP], base[(cur ^ 1) & XP]);
-            __builtin_amdgcn_sched_barrier(0);
-          } else {
-            load_x(gl, xa[0], base[0]);
-          }
-#pragma unroll
-          for (int r = 0; r < GR; ++r) {
-            const unsigned lo = h == 0 ? w[r].x : w[r].z, hi = h == 0 ? w[r].y : w[r].w;
-            u32x4 wb[NJ];
-            if (ABL == 4) {
-#pragma unroll
-              for (int j = 0; j < NJ; ++j) wb[j] = u32x4{lo, hi, lo | kc.M1, hi | kc.M1};
-            } else if (ACT == BP_BF16) {
-              tq2_decode_bf16(lo, kc, wb[0], wb[1]);
-              tq2_decode_bf16(hi, kc, wb[NJ - 2], wb[NJ - 1]);
-            } else {
-              wb[0] = tq2_decode_i8(lo);
-              wb[1] = tq2_decode_i8(hi);
+              for (int j = 0; j < NJ; ++j) dx[j][mt] = u32x4{kc.M1, kc.M2, kc.M1, kc.M2};
+              continue;
             }
-            const float s = scale_at<SDT>(sraw[r], 2 * i + h);
-            acc_t acc[GT];
+            db[mt] = __builtin_bit_cast(acc_t, *(const lds_u32x4*)(cbase + (gl * (16 * GT) + 16 * mt) * 4));
 #pragma unroll
-            for (int mt = 0; mt < GT; ++mt) acc[mt] = base[cur][mt];
+            for (int j = 0; j < NJ; ++j) dx[j][mt] = *(const lds_u32x4*)(xbase + ((gl * NJ + j) * GT + mt) * 1024);
+          }
+        };
 #pragma unroll
-            for (int j = 0; j < NJ; ++j) {  // the two token sub-tiles alternate: no MFMA waits on the one before it
+        for (int i = 0; i < PF; ++i) {
+          __builtin_amdgcn_sched_barrier(0);
+          const int c = c4 + i;
+          u32x4 w[GR];
 #pragma unroll
-              for (int mt = 0; mt < GT; ++mt) {
-                      if (ACT == BP_BF16)
-                  acc[mt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, xa[cur][j][mt]),
-                                                                    __builtin_bit_cast(bf16x8, wb[j]), acc[mt], 0, 0, 0);
-                else
-                  acc[mt] = __builtin_amdgcn_mfma_i32_16x16x64_i8(__builtin_bit_cast(i32x4, xa[cur][j][mt]),
-                                                                  __builtin_bit_cast(i32x4, wb[j]), acc[mt], 0, 0, 0);
+          for (int r = 0; r < GR; ++r) {  // regroup: .x/.y = 8 bytes of group 2c, .z/.w = 8 bytes of group 2c+1
+            const auto s0 = __builtin_amdgcn_permlane32_swap(ring[i % RD][r].x, ring[i % RD][r].z, false, false);
+            const auto s1 = __builtin_amdgcn_permlane32_swap(ring[i % RD][r].y, ring[i % RD][r].w, false, false);
+            w[r] = u32x4{s0[0], s1[0], s0[1], s1[1]};
+          }
+#pragma unroll
+          for (int h = 0; h < 2; ++h) {
+            const int gl = 2 * i + h;
+            load_x(gl, xa, base);
+#pragma unroll
+            for (int r = 0; r < GR; ++r) {
+              const unsigned lo = h == 0 ? w[r].x : w[r].z, hi = h == 0 ? w[r].y : w[r].w;
+              u32x4 wb[NJ];
+              if (ABL == 4) {
+#pragma unroll
+                for (int j = 0; j < NJ; ++j) wb[j] = u32x4{lo, hi, lo | kc.M1, hi | kc.M1};
+              } else if (ACT == BP_BF16) {
+                tq2_decode_bf16(lo, kc, wb[0], wb[1]);
+                tq2_decode_bf16(hi, kc, wb[NJ - 2], wb[NJ - 1]);
+              } else {
+                wb[0] = tq2_decode_i8(lo);
+                wb[1] = tq2_decode_i8(hi);
               }
-            }
+              const float s = scale_at<SDT>(sraw[r], 2 * i + h);
+              acc_t acc[GT];
 #pragma unroll
-            for (int mt = 0; mt < GT; ++mt) {
-    #pragma unroll
-              for (int q = 0; q < 4; ++q) {
-                if (ABL == 7) { if (q == 0) total[r][mt][0] += (float)(acc[mt][0] + acc[mt][1] + acc[mt][2] + acc[mt][3]) * s; continue; }
-                total[r][mt][q] += (float)acc[mt][q] * s;
+              for (int mt = 0; mt < MTN; ++mt) acc[mt] = base[mt];
+#pragma unroll
+              for (int j = 0; j < NJ; ++j) {  // the two token sub-tiles alternate: no MFMA waits on the one before it
+#pragma unroll
+                for (int mt = 0; mt < MTN; ++mt) {
+                  if (ACT == BP_BF16)
+                    acc[mt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, xa[j][mt]),
+                                                                      __builtin_bit_cast(bf16x8, wb[j]), acc[mt], 0, 0, 0);
+                  else
+                    acc[mt] = __builtin_amdgcn_mfma_i32_16x16x64_i8(__builtin_bit_cast(i32x4, xa[j][mt]),
+                                                                    __builtin_bit_cast(i32x4, wb[j]), acc[mt], 0, 0, 0);
+                }
+              }
+#pragma unroll
+              for (int mt = 0; mt < MTN; ++mt) {
+#pragma unroll
+                for (int q = 0; q < 4; ++q) {
+                  if (ABL == 7) { if (q == 0) total[r][mt][0] += (float)(acc[mt][0] + acc[mt][1] + acc[mt][2] + acc[mt][3]) * s; continue; }
+                  total[r][mt][q] += (float)acc[mt][q] * s;
+                }
               }
             }
           }
+          __builtin_amdgcn_sched_barrier(0);
+          if (i & 1) {  // reload the consumed ring slots in place, two steps back to back (whole 128-byte lines)
+            fetch_w(c - 1 + RD, ring[(i - 1) % RD]);
+            fetch_w(c + RD, ring[i % RD]);
+          }
         }
-        __builtin_amdgcn_sched_barrier(0);
-        stamp();  // step done
-        if (i == 1 && more) {  // half-way: first half of the next tile into the other buffer (last read before the previous barrier)
-          stage_store(buf ^ 1, 0);
-          stage_load(tile_k0(seq + 1), 1);
-        }
-        if (i & 1) {  // reload the consumed ring slots in place, two steps back to back (whole 128-byte lines)
-          fetch_w(c - 1 + RD, ring[(i - 1) % RD]);
-          fetch_w(c + RD, ring[i % RD]);
-        }
-      }
 
-      stamp();  // reloads issued
+      };
+      if (two) run_steps(std::integral_constant<int, GT>{});
+      else run_steps(std::integral_constant<int, 1>{});
+
       if (staged) {
         if (more) {
+          stage_store(buf ^ 1, 0);  // the other tile: last read before the previous barrier
           stage_store(buf ^ 1, 1);
-          if (seq + 2 < tiles) stage_load(tile_k0(seq + 2), 0);
+          if (seq + 2 < tiles) {
+            stage_load(tile_k0(seq + 2), 0);
+            stage_load(tile_k0(seq + 2), 1);
+          }
         }
-        stamp();  // staged
         __syncthreads();
-        stamp();  // barrier passed
         ++seq;
       }
     }
   }
 
-  if (ABL % 10 == 9 && wg_tile <= 1 && e == 0 && blockIdx.z == 0) {
-    if (dbg) for (int i = 0; i < dbgn && i < 400; ++i) dbgp[i] = *(__attribute__((address_space(3))) long long*)(156 * 1024 + 8 * i);
-    return;
-  }
   // ---- epilogue: lane holds tokens 4b + q of each token sub-tile, output row n0 + 16r + r16
 #pragma unroll
   for (int mt = 0; mt < GT; ++mt) {
@@ -424,10 +407,6 @@ int launch_gemm_tq2(const GemmArgs& a, hipStream_t s) {
         case 5: return launch_gemm_k<BP_BF16, BP_F16, 1, 5>(a, s, lds, "gemm_abl5");
         case 6: return launch_gemm_k<BP_BF16, BP_F16, 1, 6>(a, s, lds, "gemm_abl6");
         case 7: return launch_gemm_k<BP_BF16, BP_F16, 1, 7>(a, s, lds, "gemm_abl7");
-        case 9: return launch_gemm_k<BP_BF16, BP_F16, 1, 9>(a, s, 160 * 1024, "gemm_abl9");
-        case 59: return launch_gemm_k<BP_BF16, BP_F16, 1, 59>(a, s, 160 * 1024, "gemm_abl59");
-        case 19: return launch_gemm_k<BP_BF16, BP_F16, 1, 19>(a, s, 160 * 1024, "gemm_abl19");
-        case 10: return launch_gemm_k<BP_BF16, BP_F16, 1, 10>(a, s, lds, "gemm_abl10");
         default: break;
       }
     }

@@ -29,17 +29,15 @@ int launch_mfma(const GemmArgs& a, hipStream_t s) {
   // rows per wave and waves per workgroup: keep enough workgroups in flight for small problems
   const int64_t work = a.E * (a.N / 16);
   int R = 1;  // two row sub-tiles per wave cost more registers than they save LDS reads; see BP_TUNE_R
-  int MT = a.max_rows > 16 ? 2 : 1;
   // 8-wave workgroups run two to a CU, so one's start-up (staging, first loads) overlaps the other's
   // steady state; the TQ2 single-token kernels are light enough on registers for that to win everywhere.
   int waves = work >= 2048 && !(a.fmt == BP_TQ2 && a.max_rows == 1) ? 16 : 8;
   // development overrides (tuning sweeps)
-  if (const char* t = getenv("BP_TUNE_R")) { const int v = atoi(t); if (v == 1 || v == 2 || v == 4) R = v; }
+  if (const char* t = getenv("BP_TUNE_R")) { const int v = atoi(t); if (v == 1 || v == 2) R = v; }
   if (const char* t = getenv("BP_TUNE_WAVES")) { const int v = atoi(t); if (v == 8 || v == 16) waves = v; }
-  if (const char* t = getenv("BP_TUNE_MT")) { const int v = atoi(t); if (v == 1 || v == 2) MT = v; }
   if (a.fmt == BP_TQ1) return launch_mfma_tq1(a, s, waves);
-  if (a.max_rows > 16 && !getenv("BP_TUNE_MT") && !getenv("BP_TUNE_R")) return launch_gemm_tq2(a, s);
-  return launch_mfma_tq2(a, s, R, MT, waves);
+  if (a.max_rows > 16) return launch_gemm_tq2(a, s);  // token tiles of 32
+  return launch_mfma_tq2(a, s, R, 1, waves);
 }
 
 }  // namespace bp

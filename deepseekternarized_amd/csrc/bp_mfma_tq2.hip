@@ -8,7 +8,7 @@ namespace {
 // The activation tile starts at LDS address 0: row t at t * pitch, pitch = KC * XB + 16.
 constexpr int X_BASE = 0;
 // LDS budget for a workgroup's scales (beyond it: read from global memory)
-constexpr int tq2_scale_tile_max(int R) { return R >= 4 ? 64 * 1024 : 40 * 1024; }
+constexpr int tq2_scale_tile_max(int) { return 40 * 1024; }
 
 // ------------------------------------------------------------------------------------------------
 // TQ2. K % 1024 == 0, N % 16 == 0. One step = 64 packed bytes (256 trits, two groups) per row.
@@ -17,7 +17,7 @@ constexpr int tq2_scale_tile_max(int R) { return R >= 4 ? 64 * 1024 : 40 * 1024;
 // second, so that all four k-blocks of an MFMA belong to one scale group.
 // After the swap block b holds trits tb(b) .. tb(b)+31 of each group, tb = {0, 64, 32, 96}.
 template <int ACT, int SDT, int R, int MT, int WAVES, int XKB, int ABL = 0, int NQ = 4, int SL = 1>
-__global__ __launch_bounds__(WAVES * 64, (WAVES == 8 && R >= 2 && MT == 2) ? 2 : 4) void k_mfma_tq2(GemmArgs a, int KC, int tile_rows) {
+__global__ __launch_bounds__(WAVES * 64, 4) void k_mfma_tq2(GemmArgs a, int KC, int tile_rows) {
   constexpr int THREADS = WAVES * 64;
   constexpr int XB = ACT == BP_BF16 ? 2 : 1;   // bytes per activation element
   constexpr int KM = ACT == BP_BF16 ? 8 : 16;  // k per lane per MFMA
@@ -364,16 +364,6 @@ int launch_tq2_sd(const GemmArgs& a, hipStream_t s, const char* name) {
 int launch_mfma_tq2(const GemmArgs& a, hipStream_t s, int R, int MT, int waves) {
   const bool bf = a.x_dtype == BP_BF16;
   if (const char* t = getenv("BP_TUNE_ABL")) {
-    if (bf && a.scale_dtype == BP_F16 && MT == 2) {
-      switch (atoi(t)) {
-        case 2: return launch_tq2<BP_BF16, BP_F16, 1, 2, 16, 112, 2>(a, s, "abl2_m2");
-        case 3: return launch_tq2<BP_BF16, BP_F16, 1, 2, 16, 112, 3>(a, s, "abl3_m2");
-        case 4: return launch_tq2<BP_BF16, BP_F16, 1, 2, 16, 112, 4>(a, s, "abl4_m2");
-        case 5: return launch_tq2<BP_BF16, BP_F16, 1, 2, 16, 112, 5>(a, s, "abl5_m2");
-        case 6: return launch_tq2<BP_BF16, BP_F16, 1, 2, 16, 112, 6>(a, s, "abl6_m2");
-        default: break;
-      }
-    }
     if (bf && a.scale_dtype == BP_F16 && MT == 1) {
       switch (atoi(t)) {
         case 1: return launch_tq2<BP_BF16, BP_F16, 1, 1, 16, 48, 1>(a, s, "abl1_w16");
@@ -389,7 +379,6 @@ int launch_mfma_tq2(const GemmArgs& a, hipStream_t s, int R, int MT, int waves) 
       }
     }
   }
-  if (MT == 2 && !(waves == 8 && R >= 2)) waves = 16;  // the 32-token tile needs the large LDS budget of a 16-wave workgroup
   if (a.max_rows == 1 && R == 2 && MT == 1 && waves == 16) {
     if (bf) return launch_tq2_sd<BP_BF16, 2, 1, 16, 48, 1>(a, s, "mfma_tq2_bf16_r2_t1_w16");
     return launch_tq2_sd<BP_I8, 2, 1, 16, 48, 1>(a, s, "mfma_tq2_i8_r2_t1_w16");
@@ -406,9 +395,7 @@ int launch_mfma_tq2(const GemmArgs& a, hipStream_t s, int R, int MT, int waves) 
   if (R == RV && MT == MTV && waves == WV) return launch_tq2_sd<ACTV, RV, MTV, WV, XK>(a, s, NAME "_r" #RV "_m" #MTV "_w" #WV);
 #define BP_ALL(ACTV, NAME)                                                        \
   BP_CASE(ACTV, 1, 1, 8, 48, NAME) BP_CASE(ACTV, 2, 1, 8, 48, NAME)                \
-  BP_CASE(ACTV, 1, 1, 16, 48, NAME) BP_CASE(ACTV, 2, 1, 16, 48, NAME)              \
-  BP_CASE(ACTV, 1, 2, 16, 112, NAME) BP_CASE(ACTV, 2, 2, 16, 112, NAME)            \
-  BP_CASE(ACTV, 2, 2, 8, 112, NAME) BP_CASE(ACTV, 4, 2, 8, 80, NAME)
+  BP_CASE(ACTV, 1, 1, 16, 48, NAME) BP_CASE(ACTV, 2, 1, 16, 48, NAME)
   if (bf) { BP_ALL(BP_BF16, "mfma_tq2_bf16") } else { BP_ALL(BP_I8, "mfma_tq2_i8") }
 #undef BP_ALL
 #undef BP_CASE
