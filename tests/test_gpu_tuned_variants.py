@@ -1,4 +1,4 @@
-"""Every code path of the tuned kernels (bp_mfma_tq2.hip, bp_mfma_tq1.hip, bp_tq1_gemv.hip) against the CPU oracle.
+"""Every code path of the tuned kernels (bp_mfma_tq2.hip, bp_gemm_tq2.hip, bp_mfma_tq1.hip, bp_tq1_gemv.hip) against the CPU oracle.
 
 The shapes are chosen by what they select inside the launchers, not by size: odd / even packed row
 lengths (row starts at every byte alignment), K that fits one activation / table tile or needs several,
@@ -154,4 +154,37 @@ def test_tq2_bf16_scales_and_f32_scales(bp):
     want = c_gemm(x, None, packed[0][0], scales[0][0].astype(np.float32), 2048, GROUP, "tq2")
     got = bp.ternary_gemm_float(dev(x).to(torch.bfloat16), dev(packed[0][0]), dev(scales[0][0]).float(), 2048, GROUP, "tq2")
     assert bp.ext().last_kernel().startswith("mfma_tq2")
+    _check(got.cpu().numpy(), want)
+
+
+# --------------------------------------------------------------------------- TQ2 grouped GEMM (token tiles of 32)
+@pytest.mark.parametrize("act", ["bf16", "int8"])
+@pytest.mark.parametrize(
+    "E,N,K,counts,terms",
+    [
+        (3, 64, 1024, [17, 0, 40], 2),        # one activation tile for all of K, reused by the second term
+        (5, 272, 2048, [32, 33, 1, 64, 16], 1),  # N not a multiple of the 256 rows of a workgroup; full, 1-row and 16-row tiles
+        (11, 48, 3072, [20] * 11, 2),          # more experts than XCDs and not a multiple of 8; odd number of tiles
+        (2, 528, 7168, [48, 31], 1),           # config-3 K, three row tiles
+    ],
+)
+def test_tq2_gemm_tiles(bp, act, E, N, K, counts, terms):
+    got, want, kern = _run(bp, "tq2", E, N, K, counts, act, terms=terms, seed=K + N)
+    assert kern.startswith("gemm_tq2"), kern
+    _check(got, want)
+
+
+def test_tq2_gemm_scales_from_global_memory_and_other_scale_dtypes(bp):
+    """K = 10240: 256 rows x 80 groups of scales do not fit beside two activation tiles; bf16 scales; float32 scales."""
+    got, want, kern = _run(bp, "tq2", 2, 64, 10240, [33, 18], "bf16", seed=21)
+    assert kern == "gemm_tq2_bf16_gs", kern
+    _check(got, want)
+    got, want, kern = _run(bp, "tq2", 2, 64, 2048, [18, 40], "bf16", seed=22, scale_dtype=np.float32)  # bf16 scales
+    assert kern.startswith("gemm_tq2"), kern
+    _check(got, want)
+    packed, scales = synth_weights(23, 1, 80, 2048, GROUP, "tq2")
+    x = orc.bf16_round(np.random.default_rng(23).standard_normal((37, 2048)).astype(np.float32))
+    want = c_gemm(x, None, packed[0][0], scales[0][0].astype(np.float32), 2048, GROUP, "tq2")
+    got = bp.ternary_gemm_float(dev(x).to(torch.bfloat16), dev(packed[0][0]), dev(scales[0][0]).float(), 2048, GROUP, "tq2")
+    assert bp.ext().last_kernel().startswith("gemm_tq2")
     _check(got.cpu().numpy(), want)
