@@ -1,0 +1,144 @@
+"""The Mode C / D checkpoint reader against directories written here in the reference's on-disk layout
+(docs/architecture/format.md:87-134): manifest checks, shapes, SHA-256, stacking of per-expert weights."""
+
+import json
+
+import numpy as np
+import pytest
+import torch
+from safetensors.torch import save_file
+
+from _util import orc, synth_weights
+
+from deepseekternarized_amd.checkpoint import TernaryCheckpoint, tensor_sha256
+
+GROUP = 128
+
+
+def _write(root, weights, shards=2, index=True, with_file=True):
+    """weights: {base: (fmt, N, K, terms, packed list [N, Kp], scales list [N, G], act)}"""
+    tensors, manifest = {}, {"format": "boilerplate", "version": 1, "tensors": {}}
+    for base, (fmt, N, K, terms, packed, scales, act) in weights.items():
+        stored = {}
+        for i in range(terms):
+            tensors[f"{base}.tq{i}.packed"] = torch.from_numpy(np.ascontiguousarray(packed[i]))
+            tensors[f"{base}.tq{i}.scale"] = torch.from_numpy(np.ascontiguousarray(scales[i]))
+            for n in (f"{base}.tq{i}.packed", f"{base}.tq{i}.scale"):
+                t = tensors[n]
+                stored[n] = {"dtype": str(t.dtype).replace("torch.", ""), "shape": list(t.shape), "sha256": tensor_sha256(t)}
+        manifest["tensors"][base] = {"mode": "C", "shape": [N, K], "packing": fmt, "terms": terms, "group": GROUP,
+                                     "scale_dtype": "fp16", "act": act, "gptq": False, "stored": stored}
+    names = sorted(tensors)
+    weight_map = {}
+    for s in range(shards):
+        part = {n: tensors[n] for n in names[s::shards]}
+        fname = f"model-{s + 1:05d}-of-{shards:05d}.safetensors"
+        save_file(part, str(root / fname))
+        for n in part:
+            weight_map[n] = fname
+    if with_file:
+        for m in manifest["tensors"].values():
+            for n, rec in m["stored"].items():
+                rec["file"] = weight_map[n]
+    if index:
+        (root / "model.safetensors.index.json").write_text(json.dumps({"weight_map": weight_map}))
+    manifest["tensors"]["layers.0.attn.wq"] = {"mode": "A", "shape": [8, 8]}
+    (root / "manifest.json").write_text(json.dumps(manifest))
+    return tensors
+
+
+def _experts(fmt, E, N, K, terms, seed, prefix="layers.0.ffn.experts", name="w1", act="int8"):
+    packed, scales = synth_weights(seed, E, N, K, GROUP, fmt, terms=terms)
+    return {f"{prefix}.{e}.{name}": (fmt, N, K, terms, [p[e] for p in packed], [s[e] for s in scales], act) for e in range(E)}, packed, scales
+
+
+@pytest.mark.parametrize("fmt", ["tq1", "tq2"])
+@pytest.mark.parametrize("layout", ["index", "file", "scan"])
+def test_terms_and_stack_match_what_was_written(tmp_path, fmt, layout):
+    w, packed, scales = _experts(fmt, 3, 16, 1280, 2, seed=1)
+    _write(tmp_path, w, index=layout == "index", with_file=layout == "file")
+    ck = TernaryCheckpoint(tmp_path, verify=True)
+    assert ck.bases() == list(w)
+    terms, meta = ck.terms("layers.0.ffn.experts.1.w1")
+    assert meta["packing"] == fmt and len(terms) == 2
+    assert np.array_equal(terms[1].packed.numpy(), packed[1][1]) and np.array_equal(terms[1].scale.numpy(), scales[1][1])
+    stacks, m = ck.stack(list(w), "cpu")
+    assert m == {"N": 16, "K": 1280, "fmt": fmt, "group": GROUP, "act": "int8", "terms": 2}
+    for i in range(2):
+        assert stacks[i][0].shape == packed[i].shape and stacks[i][0].dtype == torch.uint8
+        assert np.array_equal(stacks[i][0].numpy(), packed[i]) and np.array_equal(stacks[i][1].numpy(), scales[i])
+    lin = ck.linear("layers.0.ffn.experts.2.w1")
+    assert (lin.K, lin.fmt, lin.group, lin.act, lin.out_features) == (1280, fmt, GROUP, "int8", 16)
+
+
+def test_refusals(tmp_path):
+    w, _, _ = _experts("tq2", 2, 16, 1024, 1, seed=2)
+    other, _, _ = _experts("tq1", 1, 16, 1024, 1, seed=3, prefix="layers.1.ffn.experts")
+    tensors = _write(tmp_path, {**w, **other})
+    ck = TernaryCheckpoint(tmp_path)
+    with pytest.raises(ValueError, match="mode 'A'"):
+        ck.entry("layers.0.attn.wq")
+    with pytest.raises(KeyError):
+        ck.entry("layers.9.nope")
+    with pytest.raises(ValueError, match="cannot be stacked"):
+        ck.stack(list(w) + list(other), "cpu")
+    with pytest.raises(ValueError, match="no weights"):
+        ck.stack([], "cpu")
+    # a manifest that disagrees with the file
+    man = json.loads((tmp_path / "manifest.json").read_text())
+    base = "layers.0.ffn.experts.0.w1"
+    man["tensors"][base]["shape"] = [16, 2048]
+    (tmp_path / "manifest.json").write_text(json.dumps(man))
+    with pytest.raises(ValueError, match="expected uint8"):
+        TernaryCheckpoint(tmp_path).terms(base)
+    man["tensors"][base]["shape"] = [16, 1024]
+    man["tensors"][base]["stored"][base + ".tq0.packed"]["sha256"] = "0" * 64
+    (tmp_path / "manifest.json").write_text(json.dumps(man))
+    TernaryCheckpoint(tmp_path).terms(base)  # not checked unless asked
+    with pytest.raises(ValueError, match="SHA-256"):
+        TernaryCheckpoint(tmp_path, verify=True).terms(base)
+    assert tensor_sha256(tensors[base + ".tq0.scale"]) == man["tensors"][base]["stored"][base + ".tq0.scale"]["sha256"]
+    man["format"] = "gguf"
+    (tmp_path / "manifest.json").write_text(json.dumps(man))
+    with pytest.raises(ValueError, match="format"):
+        TernaryCheckpoint(tmp_path)
+    (tmp_path / "manifest.json").unlink()
+    with pytest.raises(FileNotFoundError):
+        TernaryCheckpoint(tmp_path)
+
+
+@pytest.mark.gpu
+def test_linear_and_moe_from_checkpoint_match_the_oracle(tmp_path):
+    """A checkpoint with one MoE layer (4 experts, gate / up / down, two terms) read back and run on the GPU."""
+    import deepseekternarized_amd as bp
+    from _util import c_gemm
+
+    H, I, E, k = 1024, 256, 4, 2
+    ws, stacks = {}, {}
+    for name, (N, K), seed in (("w1", (I, H), 5), ("w3", (I, H), 6), ("w2", (H, I), 7)):
+        w, packed, scales = _experts("tq2", E, N, K, 2, seed=seed, name=name, act="bf16")
+        ws.update(w)
+        stacks[name] = (packed, scales)
+    _write(tmp_path, ws, shards=3)
+    ck = TernaryCheckpoint(tmp_path, verify=True)
+    rng = np.random.default_rng(0)
+    x = orc.bf16_round(rng.standard_normal((5, H)).astype(np.float32))
+    # one linear
+    lin = ck.linear("layers.0.ffn.experts.3.w1")
+    got = lin(torch.from_numpy(x).cuda().to(torch.bfloat16), out_dtype=torch.float32).cpu().numpy()
+    want = np.zeros((5, I), np.float32)
+    for p, s in zip(*stacks["w1"]):
+        c_gemm(x, None, p[3], s[3].astype(np.float32), H, GROUP, "tq2", out=want)
+    assert np.linalg.norm(got - want) <= 1e-2 * np.linalg.norm(want)  # bf16 output rounding
+    # the layer: same result as a TernaryMoE built from the stacks that were written
+    moe = ck.moe("layers.0.ffn.experts.{}", E, k, "cuda")
+    from deepseekternarized_amd.moe import TernaryMoE
+
+    dev = lambda a: torch.from_numpy(np.ascontiguousarray(a)).cuda()  # noqa: E731
+    ref = TernaryMoE(*[[(dev(p), dev(s)) for p, s in zip(*stacks[n])] for n in ("w1", "w3", "w2")], hidden=H, inter=I, top_k=k,
+                     fmt="tq2", group=GROUP, act="bf16")
+    xd = dev(x).to(torch.bfloat16)
+    logits = dev(rng.standard_normal((5, E)).astype(np.float32))
+    a, b = moe(xd, logits), ref(xd, logits)
+    assert torch.equal(a, b) and torch.isfinite(a).all()
+    assert bp.ext() is not None
