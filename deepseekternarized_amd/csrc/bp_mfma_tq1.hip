@@ -1,4 +1,7 @@
-// TQ1 (5 trits per byte, base 3) on MFMA, bf16 activations. K % 256 == 0, K >= 1024, N % 16 == 0.
+// TQ1 (5 trits per byte, base 3) on MFMA, bf16 or int8 activations. K % 256 == 0, K >= 1024, N % 16 == 0.
+// int8 activations are widened to bf16 when the tile is staged (exact: |q| <= 127), so a group's sum of
+// q * trit is an exact integer in the float32 accumulator, as in the integer kernels; the token's
+// activation scale multiplies the finished sum.
 //
 // 640 trits = 128 bytes = 5 scale groups realign byte and group boundaries, so the unit of work is a
 // 128-byte chunk of every row. A byte is atomic: it fills one MFMA k-block with its 5 trits and 3
@@ -24,6 +27,7 @@ namespace bp {
 namespace {
 
 struct __attribute__((packed, aligned(2))) Packed16 { u32x4 v; };
+struct __attribute__((packed, aligned(1))) Packed8 { u32x2 v; };
 
 // LDS map: [0, 32 KiB) table, entry of byte v copy c at v * 128 + c * 8; then per wave two row buffers
 // of 16 rows x WROW bytes; then the activation tile; then (SL) the workgroup's scales.
@@ -87,7 +91,9 @@ __global__ __launch_bounds__(WAVES * 64, 4) void k_mfma_tq1(GemmArgs a, int CPT 
   const int units = ntok * tile_slots;
   int t_lane = r16 < ntok ? r16 : ntok - 1;
   const unsigned xaddr = (unsigned)(XB0 + t_lane * pitch + 7 * 16 * b);
+  const bool x_i8 = a.x_dtype == BP_I8;  // uniform
   const uint16_t* xg = (const uint16_t*)a.x + tok0 * a.K;
+  const signed char* xg8 = (const signed char*)a.x + tok0 * a.K;
   u32x4 xstage[XU];
   auto stage_load = [&](int chunk0) {  // global -> registers: the tile that starts at chunk `chunk0`
 #pragma unroll
@@ -104,14 +110,30 @@ __global__ __launch_bounds__(WAVES * 64, 4) void k_mfma_tq1(GemmArgs a, int CPT 
         int lo = 128 * g - 5 * j, hi = lo + 128;                   // digits lo <= d < hi belong to group g
         if (a.K - k0 < hi) hi = (int)(a.K - k0);                   // ... and lie inside K
         if (hi > 0 && lo < 5) {
-          const uint16_t* src = xg + (int64_t)row * a.K + k0;
           unsigned h[5];
-          if (k0 + 8 <= a.K) {
-            const u32x4 q = ((const Packed16*)src)->v;
-            h[0] = q.x & 0xffffu; h[1] = q.x >> 16; h[2] = q.y & 0xffffu; h[3] = q.y >> 16; h[4] = q.z & 0xffffu;
-          } else {  // the last bytes of a row: element by element
+          if (x_i8) {
+            const signed char* src = xg8 + (int64_t)row * a.K + k0;
+            int v8[5];
+            if (k0 + 8 <= a.K) {
+              const u32x2 q = ((const Packed8*)src)->v;
 #pragma unroll
-            for (int d = 0; d < 5; ++d) h[d] = k0 + d < a.K ? src[d] : 0u;
+              for (int d = 0; d < 4; ++d) v8[d] = __builtin_amdgcn_sbfe((int)q.x, 8 * d, 8);
+              v8[4] = __builtin_amdgcn_sbfe((int)q.y, 0, 8);
+            } else {
+#pragma unroll
+              for (int d = 0; d < 5; ++d) v8[d] = k0 + d < a.K ? (int)src[d] : 0;
+            }
+#pragma unroll
+            for (int d = 0; d < 5; ++d) h[d] = __float_as_uint((float)v8[d]) >> 16;  // exact in bf16
+          } else {
+            const uint16_t* src = xg + (int64_t)row * a.K + k0;
+            if (k0 + 8 <= a.K) {
+              const u32x4 q = ((const Packed16*)src)->v;
+              h[0] = q.x & 0xffffu; h[1] = q.x >> 16; h[2] = q.y & 0xffffu; h[3] = q.y >> 16; h[4] = q.z & 0xffffu;
+            } else {  // the last bytes of a row: element by element
+#pragma unroll
+              for (int d = 0; d < 5; ++d) h[d] = k0 + d < a.K ? src[d] : 0u;
+            }
           }
 #pragma unroll
           for (int d = 0; d < 5; ++d) h[d] = d >= lo && d < hi ? h[d] : 0u;
@@ -287,7 +309,7 @@ __global__ __launch_bounds__(WAVES * 64, 4) void k_mfma_tq1(GemmArgs a, int CPT 
     const int t = 4 * b + q;
     if (t < ntok && wave_live) {
       float* o = a.out + (tok0 + t) * a.N + n0 + r16;
-      *o += total[q];
+      *o += x_i8 ? total[q] * a.x_scale[tok0 + t] : total[q];
     }
   }
 }

@@ -120,10 +120,11 @@ def test_tq1_gemv_scales_from_global_memory(bp):
 
 
 # --------------------------------------------------------------------------- TQ1 MFMA kernel (2..16 rows per tile)
+@pytest.mark.parametrize("act", ["bf16", "int8"])
 @pytest.mark.parametrize("K", [1024, 2048, 7168])
 @pytest.mark.parametrize("counts", [[2, 0, 5], [16, 3, 1], [20, 1, 37]])
-def test_tq1_mfma_tiles(bp, K, counts):
-    got, want, kern = _run(bp, "tq1", 3, 80, K, counts, "bf16", terms=2, seed=K + sum(counts))
+def test_tq1_mfma_tiles(bp, K, counts, act):
+    got, want, kern = _run(bp, "tq1", 3, 80, K, counts, act, terms=2, seed=K + sum(counts))
     assert kern.startswith("mfma_tq1"), kern
     _check(got, want)
 
