@@ -16,8 +16,9 @@ bool mfma_supports(const GemmArgs& a) {
     }
     return true;
   }
-  // TQ1: scales as stored (fp16 / bf16); bf16 or int8 activations, or any activation dtype for single-token launches
-  if (a.scale_dtype != BP_F16 && a.scale_dtype != BP_BF16) return false;
+  // TQ1: fp16 / bf16 scales as stored, or float32 ones (the reference's wrappers widen them before the call);
+  // bf16 or int8 activations, or any activation dtype for single-token launches
+  if (a.scale_dtype != BP_F16 && a.scale_dtype != BP_BF16 && a.scale_dtype != BP_F32) return false;
   if (a.x_dtype != BP_BF16 && a.x_dtype != BP_I8 && a.max_rows != 1) return false;
   if (a.K % 256 != 0 || a.K < 1024) return false;  // whole groups, and an even number of them (4-byte aligned scale rows)
   for (int t = 0; t < a.n_terms; ++t)

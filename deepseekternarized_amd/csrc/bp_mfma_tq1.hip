@@ -39,10 +39,15 @@ constexpr int T1_X_BUDGET = 48 * 1024;
 constexpr int T1_LDS_MAX = 160 * 1024;
 // row pitch of the transpose buffers: 132 bytes of data (+ 12 of scales without the scale tile); a multiple
 // of 16 (aligned 16-byte writes) whose 16 rows start in different banks
-template <int SL>
-constexpr int t1_wrow() { return 144; }
-template <int WAVES, int SL>
-constexpr int t1_x_base() { return T1_LUT_BYTES + WAVES * 2 * 16 * t1_wrow<SL>(); }
+// (float32 scales without the scale tile: 24 bytes of scales at offset 136)
+template <int SL, int SDT>
+constexpr int t1_wrow() { return !SL && SDT == BP_F32 ? 160 : 144; }
+template <int WAVES, int SL, int SDT>
+constexpr int t1_x_base() { return T1_LUT_BYTES + WAVES * 2 * 16 * t1_wrow<SL, SDT>(); }
+
+__device__ __forceinline__ u32x2 buf_load8(__amdgpu_buffer_rsrc_t r, unsigned lane_off, unsigned wave_off) {
+  return __builtin_bit_cast(u32x2, __builtin_amdgcn_raw_buffer_load_b64(r, (int)lane_off, (int)wave_off, 0));
+}
 
 __device__ __forceinline__ unsigned buf_load4(__amdgpu_buffer_rsrc_t r, unsigned lane_off, unsigned wave_off) {
   return (unsigned)__builtin_amdgcn_raw_buffer_load_b32(r, (int)lane_off, (int)wave_off, 0);
@@ -54,9 +59,10 @@ __device__ __forceinline__ unsigned buf_load4(__amdgpu_buffer_rsrc_t r, unsigned
 template <int SDT, int WAVES, int NQ, int SL, int MULTI, int ABL = 0>
 __global__ __launch_bounds__(WAVES * 64, 4) void k_mfma_tq1(GemmArgs a, int CPT /* chunks per activation tile */, int tile_rows) {
   constexpr int THREADS = WAVES * 64;
-  constexpr int WROW = t1_wrow<SL>();
+  constexpr int WROW = t1_wrow<SL, SDT>();
   constexpr int WB = T1_LUT_BYTES;
-  constexpr int XB0 = t1_x_base<WAVES, SL>();
+  constexpr int XB0 = t1_x_base<WAVES, SL, SDT>();
+  constexpr int SB = SDT == BP_F32 ? 4 : 2;  // bytes per scale
   constexpr int XU = (T1_X_BUDGET / 16 + THREADS - 1) / THREADS;  // activation slots staged per thread
   constexpr int FB[5] = {0, 25, 51, 76, 102};
 
@@ -159,7 +165,7 @@ __global__ __launch_bounds__(WAVES * 64, 4) void k_mfma_tq1(GemmArgs a, int CPT 
   for (int q = 0; q < NQ; ++q) total[q] = 0.f;
 
   const unsigned stile = (unsigned)(XB0 + tile_rows * pitch);                       // scale tile (SL)
-  const unsigned slane = stile + (unsigned)((wave * 16 + r16) * (int)a.G * 2);      // this lane's row of it
+  const unsigned slane = stile + (unsigned)((wave * 16 + r16) * (int)a.G * SB);     // this lane's row of it
 
   for (int term = 0; term < a.n_terms; ++term) {
     // this wave's 16 rows as a buffer that ends with the tensor; 4-byte aligned base, per-lane row offset
@@ -170,13 +176,14 @@ __global__ __launch_bounds__(WAVES * 64, 4) void k_mfma_tq1(GemmArgs a, int CPT 
     const unsigned ro = mis + (unsigned)r16 * (unsigned)a.Kp;
     const unsigned dlt = ro & 3u;            // chunk byte j of this lane's row sits at offset j + dlt of its buffer row
     const unsigned voff_row = ro & ~3u, voff = voff_row + 16u * b;
-    const __amdgpu_buffer_rsrc_t srs = make_rsrc((const unsigned char*)a.w_scale[term] + (e * a.N + n0) * a.G * 2, 16 * a.G * 2);
+    const __amdgpu_buffer_rsrc_t srs = make_rsrc((const unsigned char*)a.w_scale[term] + (e * a.N + n0) * a.G * SB, 16 * a.G * SB);
     const int sb = b < 3 ? b : 2;
-    const unsigned soff_lane = (unsigned)r16 * (unsigned)a.G * 2u + 4u * sb;
+    const unsigned soff_lane = (unsigned)r16 * (unsigned)a.G * SB + (SDT == BP_F32 ? 8u : 4u) * sb;
     const unsigned rbuf0 = (unsigned)(WB + ((wave * 2) * 16 + r16) * WROW);  // this lane's row in the wave's buffers
 
     u32x4 wq[2][2] = {};
     unsigned wt[2] = {}, sq[2] = {};
+    u32x2 sq2[2] = {};  // (float32 scales)
     auto fetch_pair = [&](int c) {  // chunks c and c + 1 (clamped to the last one)
 #pragma unroll
       for (int j = 0; j < 2; ++j) {
@@ -189,7 +196,9 @@ __global__ __launch_bounds__(WAVES * 64, 4) void k_mfma_tq1(GemmArgs a, int CPT 
         wq[j][0] = buf_load16(wrs, voff, so);
         wq[j][1] = buf_load16(wrs, voff, so + 64);
         wt[j] = buf_load4(wrs, voff_row, so + 128);
-        if (!SL) {  // k-blocks 0..2 fetch one dword each = 2 of the 6 scales starting at an even group index
+        if (!SL && SDT == BP_F32) {  // k-blocks 0..2 fetch two scales each: groups 5 cl .. 5 cl + 5 (past the rows: zeros)
+          sq2[j] = buf_load8(srs, soff_lane, 4u * 5 * cl);
+        } else if (!SL) {  // k-blocks 0..2 fetch one dword each = 2 of the 6 scales starting at an even group index
           int gi = (5 * cl) & ~1;
           if (gi > (int)a.G - 6) gi = (int)a.G - 6;
           sq[j] = buf_load4(srs, soff_lane, 2u * gi);
@@ -204,8 +213,8 @@ __global__ __launch_bounds__(WAVES * 64, 4) void k_mfma_tq1(GemmArgs a, int CPT 
     if (SL) {  // behind the loads above, so that their latencies overlap with the copy's
       const int64_t wg_row0 = (int64_t)blockIdx.x * (WAVES * 16);
       const int64_t wg_rows = a.N - wg_row0 < WAVES * 16 ? a.N - wg_row0 : WAVES * 16;
-      const unsigned char* src = (const unsigned char*)a.w_scale[term] + (e * a.N + wg_row0) * a.G * 2;
-      const int units16 = (int)(wg_rows * a.G * 2 / 16);
+      const unsigned char* src = (const unsigned char*)a.w_scale[term] + (e * a.N + wg_row0) * a.G * SB;
+      const int units16 = (int)(wg_rows * a.G * SB / 16);
       if (term > 0) __syncthreads();  // the previous term's scales are no longer read
       for (int u = threadIdx.x; u < units16; u += THREADS) *(lds_u32x4*)(stile + 16 * u) = *(const u32x4*)(src + 16 * (int64_t)u);
       __syncthreads();
@@ -227,7 +236,8 @@ __global__ __launch_bounds__(WAVES * 64, 4) void k_mfma_tq1(GemmArgs a, int CPT 
           *(lds_u32x4*)(rbj + 16 * b) = wq[j][0];
           *(lds_u32x4*)(rbj + 64 + 16 * b) = wq[j][1];
           *(lds_u32*)(rbj + 128) = wt[j];
-          if (!SL) *(lds_u32*)(rbj + 132 + 4 * sb) = sq[j];
+          if (!SL && SDT == BP_F32) *(lds_u32x2*)(rbj + 136 + 8 * sb) = sq2[j];
+          else if (!SL) *(lds_u32*)(rbj + 132 + 4 * sb) = sq[j];
         }
         __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
         __builtin_amdgcn_wave_barrier();
@@ -257,8 +267,9 @@ __global__ __launch_bounds__(WAVES * 64, 4) void k_mfma_tq1(GemmArgs a, int CPT 
 #pragma unroll
         for (int g = 0; g < 5; ++g) {
           if (g < ng) {
-            unsigned half;  // the group's scale
-            if (SL) half = *(const __attribute__((address_space(3))) uint16_t*)(slane + 2 * (5 * c + g));
+            unsigned half;  // the group's scale (bits as stored)
+            if (SDT == BP_F32) half = SL ? *(const lds_u32*)(slane + 4 * (5 * c + g)) : *(const lds_u32*)(rb + 136 + 4 * g);
+            else if (SL) half = *(const __attribute__((address_space(3))) uint16_t*)(slane + 2 * (5 * c + g));
             else half = *(const __attribute__((address_space(3))) uint16_t*)(rb + 132 + 2 * (sshift + g));
             // the 7 bytes of this lane's k-block for group g, read back from the transpose buffer
             const unsigned o = dlt + FB[g] + 7 * b;
@@ -295,7 +306,7 @@ __global__ __launch_bounds__(WAVES * 64, 4) void k_mfma_tq1(GemmArgs a, int CPT 
               __builtin_amdgcn_sched_barrier(0);
             }
             // weights were decoded as +-0.5: the factor 2 goes into the scale (exact)
-            const float sc = 2.0f * (SDT == BP_F16 ? f16_bits_to_f32((uint16_t)half) : __uint_as_float(half << 16));
+            const float sc = 2.0f * (SDT == BP_F32 ? __uint_as_float(half) : SDT == BP_F16 ? f16_bits_to_f32((uint16_t)half) : __uint_as_float(half << 16));
 #pragma unroll
             for (int q = 0; q < NQ; ++q) total[q] += acc[q] * sc;
           }
@@ -338,7 +349,7 @@ int launch_tq1(const GemmArgs& a, hipStream_t s, const char* name) {
   int64_t cpt = (T1_X_BUDGET / tokens - 16) / T1_XCHUNK;
   if (cpt > nchunks) cpt = nchunks;
   if (cpt < 1) return fail(BP_ERR_UNSUPPORTED, "activation tile does not fit");
-  const size_t lds = t1_x_base<WAVES, SL>() + (size_t)tokens * (cpt * T1_XCHUNK + 16) + (SL ? (size_t)rows_per_wg * a.G * 2 : 0);
+  const size_t lds = t1_x_base<WAVES, SL, SDT>() + (size_t)tokens * (cpt * T1_XCHUNK + 16) + (SL ? (size_t)rows_per_wg * a.G * (SDT == BP_F32 ? 4 : 2) : 0);
   if (lds > (size_t)T1_LDS_MAX) return BP_ERR_UNSUPPORTED;  // the caller tries the next variant
   if (cpt < nchunks) return launch_tq1_k<SDT, WAVES, NQ, SL, 1, ABL>(a, s, name, cpt, tokens, lds);
   return launch_tq1_k<SDT, WAVES, NQ, SL, 0, ABL>(a, s, name, cpt, tokens, lds);
@@ -350,10 +361,12 @@ int launch_tq1_v(const GemmArgs& a, hipStream_t s, const char* name_sl, const ch
   bool aligned = true;
   for (int t = 0; t < a.n_terms; ++t) aligned = aligned && ((uintptr_t)a.w_scale[t] & 15) == 0;
   if (aligned) {
-    const int rc = a.scale_dtype == BP_F16 ? launch_tq1<BP_F16, WAVES, NQ, 1>(a, s, name_sl) : launch_tq1<BP_BF16, WAVES, NQ, 1>(a, s, name_sl);
+    const int rc = a.scale_dtype == BP_F16 ? launch_tq1<BP_F16, WAVES, NQ, 1>(a, s, name_sl)
+                   : a.scale_dtype == BP_BF16 ? launch_tq1<BP_BF16, WAVES, NQ, 1>(a, s, name_sl) : launch_tq1<BP_F32, WAVES, NQ, 1>(a, s, name_sl);
     if (rc != BP_ERR_UNSUPPORTED) return rc;
   }
-  const int rc = a.scale_dtype == BP_F16 ? launch_tq1<BP_F16, WAVES, NQ, 0>(a, s, name_gl) : launch_tq1<BP_BF16, WAVES, NQ, 0>(a, s, name_gl);
+  const int rc = a.scale_dtype == BP_F16 ? launch_tq1<BP_F16, WAVES, NQ, 0>(a, s, name_gl)
+                 : a.scale_dtype == BP_BF16 ? launch_tq1<BP_BF16, WAVES, NQ, 0>(a, s, name_gl) : launch_tq1<BP_F32, WAVES, NQ, 0>(a, s, name_gl);
   if (rc == BP_ERR_UNSUPPORTED) return fail(BP_ERR_UNSUPPORTED, "TQ1 tile does not fit in LDS");
   return rc;
 }

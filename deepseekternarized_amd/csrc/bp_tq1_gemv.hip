@@ -55,6 +55,8 @@ __global__ __launch_bounds__(WAVES * 64, 4) void k_tq1_gemv(GemmArgs a, int CPT 
   constexpr int TB = WAVES * 16 * WROW;  // tables start after the wave buffers
   constexpr int XU = 2;                  // table slots built per thread (launcher keeps CPT * 140 <= XU * THREADS)
   constexpr int FB[5] = {0, 25, 51, 76, 102};
+  constexpr int SB = SDT == BP_F32 ? 4 : 2;  // bytes per scale (float32 scales: scale tile variant only)
+  static_assert(SL || SDT != BP_F32, "float32 scales are read through the LDS tile");
 
   // the wave index through readfirstlane: everything derived from it stays in scalar registers
   const int wave = __builtin_amdgcn_readfirstlane((int)(threadIdx.x >> 6)), lane = threadIdx.x & 63;
@@ -132,7 +134,7 @@ __global__ __launch_bounds__(WAVES * 64, 4) void k_tq1_gemv(GemmArgs a, int CPT 
 
   float total = 0.f;
   const unsigned stile = (unsigned)(TB + CPT * G1_CHUNK_BYTES);                     // scale tile (SL)
-  const unsigned slane = stile + (unsigned)((wave * 16 + r16) * (int)a.G * 2);      // this lane's row of it
+  const unsigned slane = stile + (unsigned)((wave * 16 + r16) * (int)a.G * SB);     // this lane's row of it
   const unsigned rb = (unsigned)((wave * 16 + r16) * WROW);                         // this lane's row in the wave's buffer
 
   for (int term = 0; term < a.n_terms; ++term) {
@@ -174,8 +176,8 @@ __global__ __launch_bounds__(WAVES * 64, 4) void k_tq1_gemv(GemmArgs a, int CPT 
     if (SL) {  // behind the loads above, so that their latencies overlap with the copy's
       const int64_t wg_row0 = (int64_t)blockIdx.x * (WAVES * 16);
       const int64_t wg_rows = a.N - wg_row0 < WAVES * 16 ? a.N - wg_row0 : WAVES * 16;
-      const unsigned char* src = (const unsigned char*)a.w_scale[term] + (e * a.N + wg_row0) * a.G * 2;
-      const int units16 = (int)(wg_rows * a.G * 2 / 16);
+      const unsigned char* src = (const unsigned char*)a.w_scale[term] + (e * a.N + wg_row0) * a.G * SB;
+      const int units16 = (int)(wg_rows * a.G * SB / 16);
       if (term > 0) __syncthreads();  // the previous term's scales are no longer read
       for (int u = threadIdx.x; u < units16; u += THREADS) *(lds_u32x4*)(stile + 16 * u) = *(const u32x4*)(src + 16 * (int64_t)u);
       __syncthreads();
@@ -225,8 +227,9 @@ __global__ __launch_bounds__(WAVES * 64, 4) void k_tq1_gemv(GemmArgs a, int CPT 
 #pragma unroll
       for (int g = 0; g < 5; ++g) {
         if (g < ng) {
-          unsigned half;  // the group's scale
-          if (SL) half = *(const __attribute__((address_space(3))) uint16_t*)(slane + 2 * (5 * c + g));
+          unsigned half;  // the group's scale (bits as stored)
+          if (SDT == BP_F32) half = *(const lds_u32*)(slane + 4 * (5 * c + g));
+          else if (SL) half = *(const __attribute__((address_space(3))) uint16_t*)(slane + 2 * (5 * c + g));
           else half = *(const __attribute__((address_space(3))) uint16_t*)(rb + 136 + 2 * (sshift + g));
           // the 7 bytes of this lane's slots for group g, read back from the transpose buffer
           const unsigned o = dlt + FB[g] + 7 * b;
@@ -252,7 +255,7 @@ __global__ __launch_bounds__(WAVES * 64, 4) void k_tq1_gemv(GemmArgs a, int CPT 
           float acc9 = t9[0], acc27 = t27[0];
 #pragma unroll
           for (int m = 1; m < 7; ++m) { acc9 += t9[m]; acc27 += t27[m]; }
-          const float sc = SDT == BP_F16 ? f16_bits_to_f32((uint16_t)half) : __uint_as_float(half << 16);
+          const float sc = SDT == BP_F32 ? __uint_as_float(half) : SDT == BP_F16 ? f16_bits_to_f32((uint16_t)half) : __uint_as_float(half << 16);
           total += (acc9 + acc27) * sc;
           __builtin_amdgcn_sched_barrier(0);
         }
@@ -287,7 +290,7 @@ template <int SDT, int WAVES, int SL>
 int launch_g1(const GemmArgs& a, hipStream_t s, const char* name) {
   const int64_t rows_per_wg = (int64_t)WAVES * 16;
   const int64_t nchunks = (a.K + 639) / 640;
-  const int64_t fixed = rows_per_wg * g1_wrow<SL>() + (SL ? rows_per_wg * a.G * 2 : 0);
+  const int64_t fixed = rows_per_wg * g1_wrow<SL>() + (SL ? rows_per_wg * a.G * (SDT == BP_F32 ? 4 : 2) : 0);
   int64_t cpt = (G1_LDS_MAX - fixed) / G1_CHUNK_BYTES;
   const int64_t cap = 2 * WAVES * 64 / G1_SLOTS;  // two table slots per thread at most
   if (cpt > cap) cpt = cap;
@@ -302,6 +305,8 @@ template <int WAVES>
 int launch_g1_v(const GemmArgs& a, hipStream_t s, const char* name_sl, const char* name_gl) {
   bool aligned = true;
   for (int t = 0; t < a.n_terms; ++t) aligned = aligned && ((uintptr_t)a.w_scale[t] & 15) == 0;
+  if (a.scale_dtype == BP_F32)  // float32 scales (what the reference's own wrappers pass): scale tile or nothing
+    return aligned ? launch_g1<BP_F32, WAVES, 1>(a, s, name_sl) : BP_ERR_UNSUPPORTED;
   if (aligned) {
     const int rc = a.scale_dtype == BP_F16 ? launch_g1<BP_F16, WAVES, 1>(a, s, name_sl) : launch_g1<BP_BF16, WAVES, 1>(a, s, name_sl);
     if (rc != BP_ERR_UNSUPPORTED) return rc;

@@ -60,6 +60,8 @@ def _run(bp, fmt, E, N, K, counts, act, terms=1, seed=0, misalign_scales=False, 
     pk = [dev(p) for p in packed]
     if scale_dtype is np.float16:
         sc = [dev(s) for s in scales]
+    elif scale_dtype == "f32":  # the stored fp16 values widened, as the reference's wrappers pass them
+        sc = [dev(s.astype(np.float32)) for s in scales]
     else:
         sc = [dev(s.astype(np.float32)).to(torch.bfloat16) for s in scales]
         # the oracle must see the rounded scales
@@ -189,3 +191,14 @@ def test_tq2_gemm_scales_from_global_memory_and_other_scale_dtypes(bp):
     got = bp.ternary_gemm_float(dev(x).to(torch.bfloat16), dev(packed[0][0]), dev(scales[0][0]).float(), 2048, GROUP, "tq2")
     assert bp.ext().last_kernel().startswith("gemm_tq2")
     _check(got.cpu().numpy(), want)
+
+
+# --------------------------------------------------------------------------- float32 scales (TQ1)
+@pytest.mark.parametrize("act", ["bf16", "int8"])
+@pytest.mark.parametrize("K,counts,prefix", [(2048, [1, 0, 1], "lut_tq1"), (7168, [1, 1, 1], "lut_tq1"), (2048, [3, 16, 1], "mfma_tq1"),
+                                              (7168, [20, 2, 9], "mfma_tq1")])
+def test_tq1_float32_scales(bp, act, K, counts, prefix):
+    """boilerplate/kernels/ternary_cuda.py:95-97 hands the kernel `w_scale.float()`: the tuned TQ1 kernels take it."""
+    got, want, kern = _run(bp, "tq1", 3, 272, K, counts, act, terms=2, seed=K + len(act), scale_dtype="f32")
+    assert kern.startswith(prefix), kern
+    _check(got, want)
