@@ -73,7 +73,7 @@ __global__ __launch_bounds__(GTHREADS, 2) void k_gemm_tq2(GemmArgs a) {
     row_shift[r] = rows_valid[r] ? 16 * r : 0;
   }
 
-  const int chunks = (int)(a.K / GKC);
+  const int chunks = (int)((a.K + GKC - 1) / GKC);  // K % 256 == 0: the last tile may hold 1 to 3 steps only
   // ---- activation staging: thread = (token t of 16, quarter q of a group, group g = wave), once per sub-tile
   const int sq = (lane >> 4), sg = wave;
   const int sb = ((sq & 1) << 1) | (sq >> 1);  // k-block that holds elements 32 q .. 32 q + 31 of a group
@@ -88,6 +88,7 @@ __global__ __launch_bounds__(GTHREADS, 2) void k_gemm_tq2(GemmArgs a) {
   u32x4 xsr[GT][2][XB];
   auto stage_load = [&](int64_t k0, int mt) {
     if (mt == 1 && !two) return;
+    if (k0 + sg * 128 >= a.K) return;  // (last tile: this wave's group lies past K; its part of the tile is never read)
     auto& xs = xsr[mt];
     int row = 16 * mt + r16;
     if (row >= ntok) row = ntok - 1;
@@ -279,6 +280,7 @@ __global__ __launch_bounds__(GTHREADS, 2) void k_gemm_tq2(GemmArgs a) {
             const auto s1 = __builtin_amdgcn_permlane32_swap(ring[i % RD][r].y, ring[i % RD][r].w, false, false);
             w[r] = u32x4{s0[0], s1[0], s0[1], s1[1]};
           }
+          if (c < steps)  // (K % 1024 != 0: the last tile ends early)
 #pragma unroll
           for (int h = 0; h < 2; ++h) {
             const int gl = 2 * i + h;
@@ -389,17 +391,18 @@ template <int ACT, int SDT>
 int launch_gemm_sd(const GemmArgs& a, hipStream_t s, const char* name, const char* name_gs) {
   const size_t tiles = 2 * (size_t)gemm_tile_bytes<ACT>();
   const size_t stile = (size_t)GROWS * a.G * (SDT == BP_F32 ? 4 : 2);
-  if (tiles + stile <= 160 * 1024) return launch_gemm_k<ACT, SDT, 1>(a, s, tiles + stile, name);
+  // (scale tile rows are read 16 bytes at a time: they must start 16-byte aligned)
+  if (tiles + stile <= 160 * 1024 && (a.G * (SDT == BP_F32 ? 4 : 2)) % 16 == 0) return launch_gemm_k<ACT, SDT, 1>(a, s, tiles + stile, name);
   return launch_gemm_k<ACT, SDT, 0>(a, s, tiles, name_gs);
 }
 
 }  // namespace
 
-// Preconditions (checked by mfma_supports): group 128, K % 1024 == 0, N % 16 == 0, 16-byte aligned x / packed / scales.
+// Preconditions (checked by mfma_supports): group 128, K % 256 == 0, K >= 1024, N % 16 == 0, 16-byte aligned x / packed / scales.
 int launch_gemm_tq2(const GemmArgs& a, hipStream_t s) {
   if (const char* t = getenv("BP_TUNE_ABL")) {  // timing experiments: parts of the kernel switched off, results are wrong
     const size_t lds = 2 * gemm_tile_bytes<BP_BF16>() + (size_t)GROWS * a.G * 2;
-    if (a.x_dtype == BP_BF16 && a.scale_dtype == BP_F16 && lds <= 160 * 1024) {
+    if (a.x_dtype == BP_BF16 && a.scale_dtype == BP_F16 && lds <= 160 * 1024 && a.K % 1024 == 0) {
       switch (atoi(t)) {
         case 2: return launch_gemm_k<BP_BF16, BP_F16, 1, 2>(a, s, lds, "gemm_abl2");
         case 3: return launch_gemm_k<BP_BF16, BP_F16, 1, 3>(a, s, lds, "gemm_abl3");

@@ -9,7 +9,7 @@ bool mfma_supports(const GemmArgs& a) {
   if ((a.max_rows + 15) / 16 > 65535) return false;
   if (a.fmt == BP_TQ2) {
     if (a.x_dtype != BP_BF16 && a.x_dtype != BP_I8) return false;
-    if (a.K % 1024 != 0) return false;
+    if (a.K % 256 != 0 || a.K < 1024) return false;  // whole steps of 64 packed bytes
     for (int t = 0; t < a.n_terms; ++t) {
       if (((uintptr_t)a.packed[t] & 15) != 0) return false;
       if (((uintptr_t)a.w_scale[t] & 15) != 0) return false;

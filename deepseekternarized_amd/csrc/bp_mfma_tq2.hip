@@ -11,7 +11,7 @@ constexpr int X_BASE = 0;
 constexpr int tq2_scale_tile_max(int) { return 40 * 1024; }
 
 // ------------------------------------------------------------------------------------------------
-// TQ2. K % 1024 == 0, N % 16 == 0. One step = 64 packed bytes (256 trits, two groups) per row.
+// TQ2. K % 256 == 0, N % 16 == 0. One step = 64 packed bytes (256 trits, two groups) per row.
 // Lane (r16 = lane % 16, b = lane / 16) loads bytes [16b, 16b + 16) of its row's 64-byte piece; a
 // v_permlane32_swap pair then leaves every lane with 8 bytes of the first group and 8 bytes of the
 // second, so that all four k-blocks of an MFMA belong to one scale group.
@@ -203,7 +203,7 @@ __global__ __launch_bounds__(WAVES * 64, 4) void k_mfma_tq2(GemmArgs a, int KC, 
         if (ch + 1 < chunks) stage_load((int64_t)(ch + 1) * KC);
       }
       const int c_end = (ch + 1) * steps_per_chunk < steps ? (ch + 1) * steps_per_chunk : steps;
-      for (int c4 = ch * steps_per_chunk; c4 < c_end; c4 += PF) {  // KC % 1024 == 0: whole blocks of 4 steps
+      for (int c4 = ch * steps_per_chunk; c4 < c_end; c4 += PF) {  // blocks of 4 steps; KC % 1024 == 0 unless the tile holds all of K
 #pragma unroll
         for (int r = 0; r < R; ++r) { sraw[r][0] = snext[r][0]; sraw[r][1] = snext[r][1]; }
         fetch_s(c4 + PF, snext);
@@ -228,6 +228,7 @@ __global__ __launch_bounds__(WAVES * 64, 4) void k_mfma_tq2(GemmArgs a, int KC, 
             for (int r = 0; r < R; ++r) total[r][0][0] += __uint_as_float((w[r].x ^ w[r].y ^ w[r].z ^ w[r].w) & 0x3fffffu);
             continue;
           }
+          if (c < steps)  // K % 1024 != 0: the last block of 4 steps is partial (the ring re-read the last step)
 #pragma unroll
           for (int h = 0; h < 2; ++h) {
             typedef typename Acc<ACT>::type acc_t;
@@ -347,7 +348,8 @@ template <int ACT, int R, int MT, int WAVES, int XKB, int NQ = 4>
 int launch_tq2_sd(const GemmArgs& a, hipStream_t s, const char* name) {
   // scales through LDS whenever the workgroup's share of one term fits the budget
   const int64_t tile = (int64_t)WAVES * 16 * R * a.G * (a.scale_dtype == BP_F32 ? 4 : 2);
-  if (tile <= tq2_scale_tile_max(R)) {
+  // (the tile is read 16 bytes at a time from a row's start + 4 c: rows must be 16 bytes apart modulo 16)
+  if (tile <= tq2_scale_tile_max(R) && (a.G * (a.scale_dtype == BP_F32 ? 4 : 2)) % 16 == 0) {
     int rc;
     if (a.scale_dtype == BP_F16) rc = launch_tq2<ACT, BP_F16, R, MT, WAVES, XKB, 0, NQ, 1>(a, s, name);
     else if (a.scale_dtype == BP_BF16) rc = launch_tq2<ACT, BP_BF16, R, MT, WAVES, XKB, 0, NQ, 1>(a, s, name);

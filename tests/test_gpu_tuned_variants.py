@@ -202,3 +202,14 @@ def test_tq1_float32_scales(bp, act, K, counts, prefix):
     got, want, kern = _run(bp, "tq1", 3, 272, K, counts, act, terms=2, seed=K + len(act), scale_dtype="f32")
     assert kern.startswith(prefix), kern
     _check(got, want)
+
+
+# --------------------------------------------------------------------------- TQ2 with K % 1024 != 0 (whole 256-trit steps)
+@pytest.mark.parametrize("act", ["bf16", "int8"])
+@pytest.mark.parametrize("K", [1280, 2304, 11008])
+@pytest.mark.parametrize("counts,prefix", [([1, 1, 0], "mfma_tq2"), ([16, 0, 5], "mfma_tq2"), ([33, 2, 17], "gemm_tq2")])
+def test_tq2_partial_last_block(bp, act, K, counts, prefix):
+    """The last block of four steps (and the last activation tile) is partial; scale rows are not 16-byte multiples."""
+    got, want, kern = _run(bp, "tq2", 3, 48, K, counts, act, terms=2 if K == 2304 else 1, seed=K + sum(counts))
+    assert kern.startswith(prefix), kern
+    _check(got, want)
