@@ -30,7 +30,7 @@ struct __attribute__((packed, aligned(2))) Packed16 { u32x4 v; };
 typedef __attribute__((address_space(3))) float lds_f32;
 
 constexpr int G1_SLOTS = 140;                     // byte slots per chunk: 5 groups x 28
-constexpr int G1_SLOT_BYTES = 36 * 4;             // T9 (9 floats) then T27 (27 floats)
+constexpr int G1_SLOT_BYTES = 44 * 4;             // T9 (9 floats) then T27 (27 floats), padded to 44 banks (see the table tile)
 constexpr int G1_CHUNK_BYTES = G1_SLOTS * G1_SLOT_BYTES;
 // Row pitch of the transpose buffer, a multiple of 16: 136 data bytes (the aligned 128 of the chunk and the 8
 // after them, so that every byte a slot can name - up to chunk byte 129 at a row misalignment of 3 - is a
@@ -71,7 +71,13 @@ __global__ __launch_bounds__(WAVES * 64, 4) void k_tq1_gemv(GemmArgs a, int CPT 
 
   const int nchunks = (int)((a.K + 639) / 640);  // 128-byte chunks per row (the last may be partial)
   const int tile_slots = CPT * G1_SLOTS;
-  // ---- table tile: slot (cl, g, 7 b + m) at TB + ((cl * 5 + g) * 28 + 7 b + m) * 144
+  // ---- table tile: the table of slot (cl, g, 7 b + m) sits at TB + ((cl * 5 + g) * 28 + 4 m + b) * 176.
+  // The LDS has 32 banks and serves a wave's 4-byte reads half a wave at a time (measured): lane groups b = 0, 1
+  // meet in one pass, b = 2, 3 in the other. Their tables lie one slot = 44 banks = 12 (mod 32) apart, so the T9
+  // entries (9 banks) of the two groups of a pass never share a bank; with the tables 7 slots of 36 banks apart
+  // they did for most entries, and half of the kernel's LDS cycles were bank conflicts. (Two T27 tables cannot
+  // be disjoint in 32 banks.) The thread that builds a table is the one whose index equals the table's
+  // position, so a wave's 16-byte stores stay an odd multiple of 4 banks apart (conflict-free).
   float xstage[XU][5];  // the slot's 5 activations, masked (any activation dtype; int8 values are exact in float)
   auto stage_load = [&](int chunk0) {  // global -> registers: the tile that starts at chunk `chunk0`
 #pragma unroll
@@ -81,7 +87,8 @@ __global__ __launch_bounds__(WAVES * 64, 4) void k_tq1_gemv(GemmArgs a, int CPT 
       for (int d = 0; d < 5; ++d) xstage[i][d] = 0.f;
       if (u < tile_slots) {
         const int cl = u / G1_SLOTS, sg = u - cl * G1_SLOTS;
-        const int g = sg / 28, sl = sg - g * 28;                   // sl = 7 b + m: byte FB[g] + sl of the chunk
+        const int g = sg / 28, pos = sg - g * 28;                  // position 4 m + b within the group's tables
+        const int sl = 7 * (pos & 3) + (pos >> 2);                 // sl = 7 b + m: byte FB[g] + sl of the chunk
         const int j = (g == 0 ? 0 : g == 1 ? 25 : g == 2 ? 51 : g == 3 ? 76 : 102) + sl;
         const int64_t k0 = 640 * (int64_t)(chunk0 + cl) + 5 * j;  // first activation of the byte
         int lo = 128 * g - 5 * j, hi = lo + 128;                   // digits lo <= d < hi belong to group g
@@ -122,7 +129,7 @@ __global__ __launch_bounds__(WAVES * 64, 4) void k_tq1_gemv(GemmArgs a, int CPT 
           const int q = en - 9;
           return __float_as_uint((float)(q % 3 - 1) * x2 + (float)(q / 3 % 3 - 1) * x3 + (float)(q / 9 - 1) * x4);
         };
-        const unsigned dst = (unsigned)(TB + u * G1_SLOT_BYTES);
+        const unsigned dst = (unsigned)(TB + u * G1_SLOT_BYTES);  // (the 32 bytes of padding stay unwritten)
 #pragma unroll
         for (int w = 0; w < 9; ++w) {
           *(lds_u32x4*)(dst + 16 * w) = u32x4{entry(4 * w), entry(4 * w + 1), entry(4 * w + 2), entry(4 * w + 3)};
@@ -222,7 +229,7 @@ __global__ __launch_bounds__(WAVES * 64, 4) void k_tq1_gemv(GemmArgs a, int CPT 
       if (gi > (int)a.G - 6) gi = (int)a.G - 6;
       const int sshift = 5 * c - gi;  // position of group 5c among the 6 scales loaded (!SL)
       // this lane's first table of the chunk; the slot within the chunk is an instruction offset
-      unsigned tbl = (unsigned)(TB + (c - tile_c0) * G1_CHUNK_BYTES + 7 * G1_SLOT_BYTES * b);
+      unsigned tbl = (unsigned)(TB + (c - tile_c0) * G1_CHUNK_BYTES + G1_SLOT_BYTES * b);
       asm volatile("" : "+v"(tbl));  // one register; the rest of every table address is q, r and an instruction offset
 #pragma unroll
       for (int g = 0; g < 5; ++g) {
@@ -249,8 +256,8 @@ __global__ __launch_bounds__(WAVES * 64, 4) void k_tq1_gemv(GemmArgs a, int CPT 
           float t9[7], t27[7];
 #pragma unroll
           for (int m = 0; m < 7; ++m) {
-            t9[m] = *(const lds_f32*)(a9[m] + (28 * g + m) * G1_SLOT_BYTES);
-            t27[m] = *(const lds_f32*)(a27[m] + (28 * g + m) * G1_SLOT_BYTES + 36);
+            t9[m] = *(const lds_f32*)(a9[m] + (28 * g + 4 * m) * G1_SLOT_BYTES);
+            t27[m] = *(const lds_f32*)(a27[m] + (28 * g + 4 * m) * G1_SLOT_BYTES + 36);
           }
           float acc9 = t9[0], acc27 = t27[0];
 #pragma unroll
@@ -294,6 +301,7 @@ int launch_g1(const GemmArgs& a, hipStream_t s, const char* name) {
   int64_t cpt = (G1_LDS_MAX - fixed) / G1_CHUNK_BYTES;
   const int64_t cap = 2 * WAVES * 64 / G1_SLOTS;  // two table slots per thread at most
   if (cpt > cap) cpt = cap;
+  if (const char* t = getenv("BP_TUNE_CPT")) { const int v = atoi(t); if (v >= 1 && v < cpt) cpt = v; }  // (development)
   if (cpt > nchunks) cpt = nchunks;
   if (cpt < 1) return BP_ERR_UNSUPPORTED;  // the caller tries the next variant
   const size_t lds = (size_t)(fixed + cpt * G1_CHUNK_BYTES);
