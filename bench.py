@@ -274,7 +274,32 @@ def main() -> int:
                                 "frac_of_bf16_mfma_peak": round(flops / k3t / 1e12 / MFMA_BF16_PEAK_TFLOPS, 4),
                                 "weight_GBps": round(weight_bytes(packed, scales) / k3t / 1e9, 1), "kernel": kn3,
                                 "us": round(k3t * 1e6, 1)}
-        del l3, packed, scales, xg
+        del l3, xg
+        # ... and the whole routed-expert layer of config 3 (gate | up, SwiGLU, down, combine) on the same gate stack
+        from deepseekternarized_amd.moe import TernaryMoE
+
+        H3, I3 = K3, N3
+        up3 = synth(bp, torch, E3, I3, H3, "tq2", 2, seed=4)
+        down3 = synth(bp, torch, E3, H3, I3, "tq2", 2, seed=5)
+        moe3 = TernaryMoE(list(zip(packed, scales)), list(zip(*up3)), list(zip(*down3)), H3, I3, k3, "tq2", GROUP, act="bf16")
+        del packed, scales, up3, down3
+        g3 = torch.Generator(device="cuda").manual_seed(9)
+        x3 = torch.randn(T3, H3, device="cuda", generator=g3).to(torch.bfloat16)
+        lg3 = torch.randn(T3, E3, device="cuda", generator=g3) * 1.5
+        for _ in range(2):
+            moe3(x3, lg3)
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        for _ in range(5):
+            moe3(x3, lg3)
+        torch.cuda.synchronize()
+        dt3 = (time.perf_counter() - t0) / 5
+        fl3 = 2.0 * T3 * k3 * 3 * H3 * I3 * 2  # per-term count, three projections
+        also["cfg3_moe_layer"] = {"workload": f"TQ2 k=2 MoE layer H={H3} I={I3} E={E3} top-{k3}, {T3} tokens, bf16 activations: softmax/top-k, "
+                                              "sort, gather, gate|up grouped GEMM, SwiGLU, down grouped GEMM, weighted combine",
+                                  "ms_per_layer": round(dt3 * 1e3, 3), "TFLOPs_per_term_count": round(fl3 / dt3 / 1e12, 1),
+                                  "frac_of_bf16_mfma_peak": round(fl3 / dt3 / 1e12 / MFMA_BF16_PEAK_TFLOPS, 4)}
+        del moe3, x3, lg3
         torch.cuda.empty_cache()
         # end-to-end timing loop of the reference's `boilerplate bench` on a random-init OLMoE-shaped Mode D decoder
         from deepseekternarized_amd.decoder_harness import DecoderConfig, TernaryDecoder, bench_decoder

@@ -162,13 +162,17 @@ def ternary_gemm_ref(x: torch.Tensor, x_scale: torch.Tensor, packed: torch.Tenso
 
 
 def grouped_ternary_gemm(x: torch.Tensor, x_scale, offsets, packed, w_scale, K: int, group: int, fmt: str,
-                         backend: str = "auto") -> torch.Tensor:
+                         backend: str = "auto", max_rows: int | None = None) -> torch.Tensor:
     """Rows of ``x`` sorted by expert; ``packed`` [E, N, Kp], ``w_scale`` [E, N, G] -> [T, N] float32
     (``boilerplate/kernels/ternary_cuda.py:90-111``).
 
     ``offsets`` given as host data (list, CPU tensor) is validated like the reference does and a
     violation raises ``ValueError("offsets ...")``. ``offsets`` given as a device tensor is used as is,
     with no device-to-host copy; the kernels clamp it, so it cannot cause out-of-bounds accesses.
+    The launch then covers ``max_rows`` rows per expert - an upper bound the caller knows (the token count,
+    when every token picks distinct experts), by default the row count of ``x``; rows of an expert beyond
+    ``max_rows`` would not be computed. With host offsets the widest expert is taken from them and ``max_rows``
+    is ignored.
     """
     code = _fmt_code(fmt)
     if backend not in _BACKENDS:
@@ -186,7 +190,12 @@ def grouped_ternary_gemm(x: torch.Tensor, x_scale, offsets, packed, w_scale, K: 
     e = _need_ext(x)
     dev = x.device
     offs_dev = offsets.to(torch.int64).contiguous() if on_device else host.to(dev, non_blocking=False)
-    max_rows = x.size(0) if host is None else (int(host.diff().max()) if E else 0)
+    if host is not None:
+        max_rows = int(host.diff().max()) if E else 0
+    elif max_rows is None:
+        max_rows = x.size(0)
+    else:
+        max_rows = max(0, min(int(max_rows), x.size(0)))
     out = torch.zeros(x.size(0), pk[0].size(1), dtype=torch.float32, device=dev)
     xs = None if x_scale is None else x_scale.float().contiguous()
     old = e.set_kernel_policy(1 if backend == "torch" else 0)

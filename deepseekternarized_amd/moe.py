@@ -72,7 +72,8 @@ class TernaryMoE:
             q, s = quant_act_int8(x)
         else:
             q, s = x, None
-        return grouped_ternary_gemm(q, s, self._offsets, [p for p, _ in terms], [sc for _, sc in terms], K, self.group, self.fmt)
+        return grouped_ternary_gemm(q, s, self._offsets, [p for p, _ in terms], [sc for _, sc in terms], K, self.group, self.fmt,
+                                    max_rows=self._max_rows)
 
     def __call__(self, x: torch.Tensor, router_logits: torch.Tensor) -> torch.Tensor:
         shape = x.shape
@@ -85,6 +86,12 @@ class TernaryMoE:
         values = values.to(torch.bfloat16).contiguous()
         indices = indices.contiguous()
         order, self._offsets = sort_by_expert(indices.reshape(-1), self.n_experts)
+        # Rows of the widest expert: at most one per token (top-k picks distinct experts). For a few tokens that
+        # bound costs nothing and keeps the layer free of host synchronisation; for many, the launch would cover
+        # tiles that do not exist, so the exact figure is read back, as the reference does
+        # (boilerplate/kernels/ternary_cuda.py:97, `int(offs.diff().max())`).
+        T = flat.size(0)
+        self._max_rows = T if T <= 64 else int((self._offsets[1:] - self._offsets[:-1]).max())
         inv = torch.empty_like(order)
         inv[order] = torch.arange(order.numel(), device=order.device)
         xg = gather_rows(flat, order, self.top_k)                                  # [T*k, H] rows in expert order

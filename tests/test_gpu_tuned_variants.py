@@ -213,3 +213,18 @@ def test_tq2_partial_last_block(bp, act, K, counts, prefix):
     got, want, kern = _run(bp, "tq2", 3, 48, K, counts, act, terms=2 if K == 2304 else 1, seed=K + sum(counts))
     assert kern.startswith(prefix), kern
     _check(got, want)
+
+
+def test_device_offsets_with_row_bound(bp):
+    """Device offsets: the launch covers `max_rows` rows per expert; the exact widest count gives the host-offset result."""
+    rng = np.random.default_rng(31)
+    E, N, K, counts = 5, 64, 2048, [40, 0, 3, 17, 33]
+    packed, scales = synth_weights(31, E, N, K, GROUP, "tq2")
+    offsets = np.concatenate([[0], np.cumsum(counts)]).astype(np.int64)
+    x = dev(orc.bf16_round(rng.standard_normal((int(offsets[-1]), K)).astype(np.float32))).to(torch.bfloat16)
+    pk, sc = [dev(p) for p in packed], [dev(s) for s in scales]
+    want = bp.grouped_ternary_gemm(x, None, offsets.tolist(), pk, sc, K, GROUP, "tq2")
+    got = bp.grouped_ternary_gemm(x, None, dev(offsets), pk, sc, K, GROUP, "tq2", max_rows=max(counts))
+    assert torch.equal(got, want)
+    loose = bp.grouped_ternary_gemm(x, None, dev(offsets), pk, sc, K, GROUP, "tq2")  # default bound: all rows
+    assert torch.equal(loose, want)
