@@ -252,6 +252,19 @@ def main() -> int:
             active = int(torch.unique(torch.topk(torch.softmax(lg.float(), -1), k2, -1).indices).numel())
             cfg2[f"T{T2}"] = {"ms_per_layer": round(dt * 1e3, 4), "active_experts": active,
                               "active_weight_GBps": round(layer_bytes / E2 * active / dt / 1e9, 1)}
+            if T2 <= 64:  # the same layer replayed as one HIP graph (launch-bound at a few tokens)
+                run = moe.graphed(T2)
+                for _ in range(3):
+                    run(xt, lg)
+                torch.cuda.synchronize()
+                t0 = time.perf_counter()
+                for _ in range(reps):
+                    run(xt, lg)
+                torch.cuda.synchronize()
+                dg = (time.perf_counter() - t0) / reps
+                cfg2[f"T{T2}"]["ms_per_layer_hip_graph"] = round(dg * 1e3, 4)
+                cfg2[f"T{T2}"]["active_weight_GBps_hip_graph"] = round(layer_bytes / E2 * active / dg / 1e9, 1)
+                del run
         also["cfg2_moe_layer"] = {"workload": f"TQ1 MoE layer H={H2} I={I2} E={E2} top-{k2}, bf16 activations: softmax/top-k, sort, gather, "
                                               "gate|up grouped GEMM, SwiGLU, down grouped GEMM, weighted combine", **cfg2}
         del moe

@@ -28,7 +28,8 @@ bool mfma_supports(const GemmArgs& a) {
 
 int launch_mfma(const GemmArgs& a, hipStream_t s) {
   // rows per wave and waves per workgroup: keep enough workgroups in flight for small problems
-  const int64_t work = a.E * (a.N / 16);
+  // (an expert without rows exits at once: at most min(E, T) experts do work)
+  const int64_t work = (a.E < a.T ? a.E : a.T) * (a.N / 16);
   int R = 1;  // two row sub-tiles per wave cost more registers than they save LDS reads; see BP_TUNE_R
   // 8-wave workgroups run two to a CU, so one's start-up (staging, first loads) overlaps the other's
   // steady state; the TQ2 single-token kernels are light enough on registers for that to win everywhere.

@@ -88,6 +88,38 @@ __global__ __launch_bounds__(SORT_THREADS) void k_sort(int64_t* __restrict__ ord
   }
 }
 
+// Few ids (n <= SORT_SMALL_N): one pass, no histograms. Element i goes to slot #(valid ids below id_i) + #(equal ids
+// before i) - the stable order - and offsets[e] = #(valid ids below e); every thread scans the ids held in LDS
+// (a broadcast read per step). Decode batches sort a few dozen ids: this takes a quarter of the general kernel's time.
+constexpr int SORT_SMALL_N = 1024;
+__global__ __launch_bounds__(SORT_SMALL_N) void k_sort_small(int64_t* __restrict__ order, int64_t* __restrict__ offsets,
+                                                              const int64_t* __restrict__ ids, int n, int64_t E,
+                                                              int32_t* __restrict__ bad) {
+  __shared__ int32_t sid[SORT_SMALL_N];
+  const int i = threadIdx.x;
+  int32_t mine = 0x7fffffff;  // an id outside [0, E) is left out of the order, as in the general kernel
+  if (i < n) {
+    const int64_t id = ids[i];
+    if (id >= 0 && id < E) mine = (int32_t)id;
+    else if (bad) *bad = 1;
+  }
+  sid[i] = mine;
+  __syncthreads();
+  if (i < n && mine != 0x7fffffff) {
+    int rank = 0;
+    for (int j = 0; j < n; ++j) {
+      const int32_t v = sid[j];
+      rank += (v < mine || (v == mine && j < i)) ? 1 : 0;
+    }
+    order[rank] = i;
+  }
+  for (int64_t e = i; e <= E; e += SORT_SMALL_N) {
+    int cnt = 0;
+    for (int j = 0; j < n; ++j) cnt += sid[j] < e ? 1 : 0;
+    offsets[e] = cnt;
+  }
+}
+
 __global__ __launch_bounds__(256) void k_gather(uint16_t* __restrict__ dst, const uint16_t* __restrict__ src,
                                                 const int64_t* __restrict__ index, int64_t divisor, int64_t src_rows,
                                                 int64_t row_halfs) {
@@ -121,30 +153,55 @@ __global__ __launch_bounds__(256) void k_swiglu(uint16_t* __restrict__ h, const 
 }
 
 // out[t, :] = bf16-accumulated sum over the token's slots in ascending expert order.
+// One workgroup per (token, 1024 columns): the slots' rows and weights are looked up once, in expert order, then
+// every thread reads its 4 columns of all k rows (independent loads) and accumulates them in that order.
+constexpr int COMBINE_COLS = 1024;
 __global__ __launch_bounds__(256) void k_combine(uint16_t* __restrict__ out, const float* __restrict__ y,
                                                  const int64_t* __restrict__ inv, const uint16_t* __restrict__ w,
                                                  const int64_t* __restrict__ experts, int64_t k, int64_t H) {
   const int64_t t = blockIdx.x;
-  __shared__ int slot_order[64];
-  if (threadIdx.x == 0) {  // insertion sort of the k slots by expert id (stable)
-    for (int s = 0; s < k; ++s) slot_order[s] = s;
-    for (int i = 1; i < k; ++i) {
-      const int v = slot_order[i];
-      const int64_t ev = experts[t * k + v];
-      int j = i - 1;
-      while (j >= 0 && experts[t * k + slot_order[j]] > ev) { slot_order[j + 1] = slot_order[j]; --j; }
-      slot_order[j + 1] = v;
-    }
+  __shared__ int64_t expert_of[64];
+  __shared__ int64_t row_of[64];
+  __shared__ float weight_of[64];
+  const int sl = threadIdx.x;
+  int64_t my_expert = 0;
+  if (sl < k) expert_of[sl] = my_expert = experts[t * k + sl];
+  __syncthreads();
+  if (sl < k) {  // position of slot sl in ascending expert order (ties: slot order), as a rank among the k slots
+    int rank = 0;
+    for (int j = 0; j < k; ++j) rank += (expert_of[j] < my_expert || (expert_of[j] == my_expert && j < sl)) ? 1 : 0;
+    row_of[rank] = inv[t * k + sl];
+    weight_of[rank] = bf16_bits_to_f32(w[t * k + sl]);
   }
   __syncthreads();
-  for (int64_t c = threadIdx.x; c < H; c += blockDim.x) {
-    float acc = 0.f;
-    for (int s = 0; s < k; ++s) {
-      const int slot = slot_order[s];
-      const int64_t pos = inv[t * k + slot];
-      const float v = round_bf16(round_bf16(y[pos * H + c]) * bf16_bits_to_f32(w[t * k + slot]));
-      acc = round_bf16(acc + v);
+  const int64_t c0 = (int64_t)blockIdx.y * COMBINE_COLS + 4 * threadIdx.x;
+  if (c0 >= H) return;
+  if ((H & 3) == 0) {  // rows of y are 16-byte aligned: four columns per load
+    float acc[4] = {0.f, 0.f, 0.f, 0.f};
+    for (int s0 = 0; s0 < k; s0 += 8) {  // up to 8 rows in flight
+      float4 v[8];
+      const int ns = k - s0 < 8 ? (int)(k - s0) : 8;
+#pragma unroll
+      for (int s = 0; s < 8; ++s)
+        if (s < ns) v[s] = *(const float4*)(y + row_of[s0 + s] * H + c0);
+#pragma unroll
+      for (int s = 0; s < 8; ++s) {
+        if (s < ns) {
+          const float ws = weight_of[s0 + s];
+          const float e[4] = {v[s].x, v[s].y, v[s].z, v[s].w};
+#pragma unroll
+          for (int i = 0; i < 4; ++i) acc[i] = round_bf16(acc[i] + round_bf16(round_bf16(e[i]) * ws));
+        }
+      }
     }
+    const uint32_t lo = (uint32_t)f32_to_bf16_bits(acc[0]) | ((uint32_t)f32_to_bf16_bits(acc[1]) << 16);
+    const uint32_t hi = (uint32_t)f32_to_bf16_bits(acc[2]) | ((uint32_t)f32_to_bf16_bits(acc[3]) << 16);
+    *(uint2*)(out + t * H + c0) = make_uint2(lo, hi);
+    return;
+  }
+  for (int64_t c = c0; c < H && c < c0 + 4; ++c) {
+    float acc = 0.f;
+    for (int s = 0; s < k; ++s) acc = round_bf16(acc + round_bf16(round_bf16(y[row_of[s] * H + c]) * weight_of[s]));
     out[t * H + c] = f32_to_bf16_bits(acc);
   }
 }
@@ -166,6 +223,10 @@ extern "C" int bp_sort_by_expert(int64_t* order, int64_t* offsets, const int64_t
   if (!offsets || (n > 0 && (!order || !ids))) return fail(BP_ERR_ARG, "null pointer");
   const int64_t need = bp_sort_workspace_ints(n, E);
   if (need > 0 && !workspace) return fail(BP_ERR_ARG, "sort_by_expert needs a workspace for this many experts");
+  if (n <= SORT_SMALL_N && E < ((int64_t)1 << 24)) {
+    hipLaunchKernelGGL(k_sort_small, dim3(1), dim3(SORT_SMALL_N), 0, (hipStream_t)stream, order, offsets, ids, (int)n, E, bad);
+    return check_launch("sort_by_expert");
+  }
   const size_t lds = need > 0 ? 0 : (size_t)(SORT_WAVES * (E > 0 ? E : 1)) * sizeof(int32_t);
   static bool attr_set = false;
   if (!attr_set) {
@@ -205,7 +266,7 @@ extern "C" int bp_moe_combine_bf16(void* out, const float* y, const int64_t* inv
   if (T < 0 || k <= 0 || k > 64 || H <= 0 || T > 0x7fffffff) return fail(BP_ERR_ARG, "invalid combine dimensions (top-k up to 64)");
   if (T == 0) return BP_OK;
   if (!out || !y || !inv || !w || !experts) return fail(BP_ERR_ARG, "null pointer");
-  hipLaunchKernelGGL(k_combine, dim3((unsigned)T), dim3(256), 0, (hipStream_t)stream, (uint16_t*)out, y, inv,
+  hipLaunchKernelGGL(k_combine, dim3((unsigned)T, (unsigned)((H + COMBINE_COLS - 1) / COMBINE_COLS)), dim3(256), 0, (hipStream_t)stream, (uint16_t*)out, y, inv,
                      (const uint16_t*)w, experts, k, H);
   return check_launch("moe_combine");
 }

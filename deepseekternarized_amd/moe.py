@@ -100,3 +100,35 @@ class TernaryMoE:
         y = self._linear(h, self.down, self.inter)                                 # f32 [T*k, H]
         out = moe_combine_bf16(y, inv, values, indices)
         return out.view(shape).to(x.dtype)
+
+    def graphed(self, tokens: int, dtype: torch.dtype = torch.bfloat16, device="cuda"):
+        """The layer for a fixed number of tokens as one HIP graph: ``run(x [tokens, hidden], router_logits [tokens, E])``
+        copies its arguments into the graph's input buffers, replays the captured launches and returns the graph's
+        output buffer (overwritten by the next replay). With a handful of tokens the layer is a dozen launches of a few
+        microseconds each, and issuing them costs more than running them; a replay issues them at once.
+        Only for ``tokens <= 64``: beyond that the layer reads the widest expert's row count back to the host, which
+        cannot be captured."""
+        if not 1 <= tokens <= 64:
+            raise ValueError("graphed() covers 1..64 tokens (larger batches read the routing back to the host)")
+        xs = torch.zeros(tokens, self.hidden, dtype=dtype, device=device)
+        ls = torch.zeros(tokens, self.n_experts, dtype=torch.float32, device=device)
+        side = torch.cuda.Stream(device=device)
+        side.wait_stream(torch.cuda.current_stream(device))
+        with torch.cuda.stream(side):  # warm-up outside the capture: kernel attributes, lazy module loads, allocator state
+            for _ in range(2):
+                self(xs, ls)
+        torch.cuda.current_stream(device).wait_stream(side)
+        torch.cuda.synchronize(device)
+        graph = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(graph):
+            out = self(xs, ls)
+
+        def run(x: torch.Tensor, router_logits: torch.Tensor) -> torch.Tensor:
+            xs.copy_(x.reshape(tokens, self.hidden))
+            ls.copy_(router_logits.reshape(tokens, self.n_experts))
+            graph.replay()
+            return out
+
+        run.graph = graph  # keeps the graph (and its memory pool) alive with the callable
+        return run
+

@@ -228,3 +228,28 @@ def test_device_offsets_with_row_bound(bp):
     assert torch.equal(got, want)
     loose = bp.grouped_ternary_gemm(x, None, dev(offsets), pk, sc, K, GROUP, "tq2")  # default bound: all rows
     assert torch.equal(loose, want)
+
+
+@pytest.mark.parametrize("fmt,act,tokens", [("tq1", "bf16", 1), ("tq2", "int8", 5), ("tq2", "bf16", 40)])
+def test_moe_layer_graph_replays_match_eager(bp, fmt, act, tokens):
+    """The captured layer against the eager one, on several replays with different inputs and eager work in between."""
+    from deepseekternarized_amd.moe import TernaryMoE
+
+    H, I, E, k = 1024, 256, 8, 2
+    stacks = []
+    for (N, K), seed in (((I, H), 41), ((I, H), 42), ((H, I), 43)):
+        packed, scales = synth_weights(seed, E, N, K, GROUP, fmt, terms=2)
+        stacks.append([(dev(p), dev(s)) for p, s in zip(packed, scales)])
+    moe = TernaryMoE(*stacks, hidden=H, inter=I, top_k=k, fmt=fmt, group=GROUP, act=act)
+    run = moe.graphed(tokens)
+    g = torch.Generator(device="cuda").manual_seed(44)
+    for rep in range(4):
+        x = torch.randn(tokens, H, device="cuda", generator=g).to(torch.bfloat16)
+        logits = torch.randn(tokens, E, device="cuda", generator=g)
+        want = moe(x, logits).clone()  # eager launches between the replays
+        torch.cuda.synchronize()
+        got = run(x, logits).clone()
+        torch.cuda.synchronize()
+        assert torch.isfinite(got).all() and torch.equal(got, want), (rep, (got.float() - want.float()).abs().max().item())
+    with pytest.raises(ValueError):
+        moe.graphed(65)
