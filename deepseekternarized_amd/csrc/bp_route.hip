@@ -88,32 +88,41 @@ __global__ __launch_bounds__(SORT_THREADS) void k_sort(int64_t* __restrict__ ord
   }
 }
 
-// Few ids (n <= SORT_SMALL_N): one pass, no histograms. Element i goes to slot #(valid ids below id_i) + #(equal ids
+// Few ids (n <= SORT_SMALL_N = 128): one pass, no histograms. Element i goes to slot #(valid ids below id_i) + #(equal ids
 // before i) - the stable order - and offsets[e] = #(valid ids below e); every thread scans the ids held in LDS
 // (a broadcast read per step). Decode batches sort a few dozen ids: this takes a quarter of the general kernel's time.
-constexpr int SORT_SMALL_N = 1024;
-__global__ __launch_bounds__(SORT_SMALL_N) void k_sort_small(int64_t* __restrict__ order, int64_t* __restrict__ offsets,
-                                                              const int64_t* __restrict__ ids, int n, int64_t E,
-                                                              int32_t* __restrict__ bad) {
+constexpr int SORT_SMALL_THREADS = 64;
+constexpr int SORT_SMALL_N = 2 * SORT_SMALL_THREADS;  // (beyond ~150 ids the scan of all ids per element loses to the histograms)
+__global__ __launch_bounds__(SORT_SMALL_THREADS) void k_sort_small(int64_t* __restrict__ order, int64_t* __restrict__ offsets,
+                                                                    const int64_t* __restrict__ ids, int n, int64_t E,
+                                                                    int32_t* __restrict__ bad) {
   __shared__ int32_t sid[SORT_SMALL_N];
-  const int i = threadIdx.x;
-  int32_t mine = 0x7fffffff;  // an id outside [0, E) is left out of the order, as in the general kernel
-  if (i < n) {
-    const int64_t id = ids[i];
-    if (id >= 0 && id < E) mine = (int32_t)id;
-    else if (bad) *bad = 1;
-  }
-  sid[i] = mine;
-  __syncthreads();
-  if (i < n && mine != 0x7fffffff) {
-    int rank = 0;
-    for (int j = 0; j < n; ++j) {
-      const int32_t v = sid[j];
-      rank += (v < mine || (v == mine && j < i)) ? 1 : 0;
+  int32_t mine[2];
+#pragma unroll
+  for (int q = 0; q < 2; ++q) {
+    const int i = threadIdx.x + q * SORT_SMALL_THREADS;
+    mine[q] = 0x7fffffff;  // an id outside [0, E) is left out of the order, as in the general kernel
+    if (i < n) {
+      const int64_t id = ids[i];
+      if (id >= 0 && id < E) mine[q] = (int32_t)id;
+      else if (bad) *bad = 1;
     }
-    order[rank] = i;
+    sid[i] = mine[q];
   }
-  for (int64_t e = i; e <= E; e += SORT_SMALL_N) {
+  __syncthreads();
+#pragma unroll
+  for (int q = 0; q < 2; ++q) {
+    const int i = threadIdx.x + q * SORT_SMALL_THREADS;
+    if (i < n && mine[q] != 0x7fffffff) {
+      int rank = 0;
+      for (int j = 0; j < n; ++j) {
+        const int32_t v = sid[j];
+        rank += (v < mine[q] || (v == mine[q] && j < i)) ? 1 : 0;
+      }
+      order[rank] = i;
+    }
+  }
+  for (int64_t e = threadIdx.x; e <= E; e += SORT_SMALL_THREADS) {
     int cnt = 0;
     for (int j = 0; j < n; ++j) cnt += sid[j] < e ? 1 : 0;
     offsets[e] = cnt;
@@ -224,7 +233,7 @@ extern "C" int bp_sort_by_expert(int64_t* order, int64_t* offsets, const int64_t
   const int64_t need = bp_sort_workspace_ints(n, E);
   if (need > 0 && !workspace) return fail(BP_ERR_ARG, "sort_by_expert needs a workspace for this many experts");
   if (n <= SORT_SMALL_N && E < ((int64_t)1 << 24)) {
-    hipLaunchKernelGGL(k_sort_small, dim3(1), dim3(SORT_SMALL_N), 0, (hipStream_t)stream, order, offsets, ids, (int)n, E, bad);
+    hipLaunchKernelGGL(k_sort_small, dim3(1), dim3(SORT_SMALL_THREADS), 0, (hipStream_t)stream, order, offsets, ids, (int)n, E, bad);
     return check_launch("sort_by_expert");
   }
   const size_t lds = need > 0 ? 0 : (size_t)(SORT_WAVES * (E > 0 ? E : 1)) * sizeof(int32_t);
