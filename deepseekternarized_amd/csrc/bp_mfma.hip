@@ -38,7 +38,11 @@ int launch_mfma(const GemmArgs& a, hipStream_t s) {
   if (const char* t = getenv("BP_TUNE_R")) { const int v = atoi(t); if (v == 1 || v == 2) R = v; }
   if (const char* t = getenv("BP_TUNE_WAVES")) { const int v = atoi(t); if (v == 8 || v == 16) waves = v; }
   if (a.fmt == BP_TQ1) return launch_mfma_tq1(a, s, waves);
-  if (a.max_rows > 16) return launch_gemm_tq2(a, s);  // token tiles of 32
+  // Experts with more than 16 rows get token tiles of 32 - unless the batch is sparse (on average at most 8 rows per
+  // expert) and the bound small: then nearly every expert fits one 16-token tile of the lighter kernel, and the few
+  // that do not (or a loose upper bound from a caller that keeps the routing on the device) cost a second tile.
+  const bool sparse = a.T <= 8 * a.E && a.max_rows <= 64;
+  if (a.max_rows > 16 && !sparse) return launch_gemm_tq2(a, s);
   return launch_mfma_tq2(a, s, R, 1, waves);
 }
 
