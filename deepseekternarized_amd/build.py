@@ -22,12 +22,35 @@ FLAGS = ["--offload-arch=gfx950", "-O3", "-fPIC", "-std=c++17", "-Wall", "-Wno-u
          "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops"]
 
 
+# These kernels address LDS absolutely (their dynamic allocation must start at LDS address 0): a kernel of theirs
+# with static LDS - e.g. a register array the compiler moved there because it was indexed dynamically - would
+# compute on the wrong bytes, so the build refuses it.
+NO_STATIC_LDS = {"bp_mfma_tq2.hip", "bp_gemm_tq2.hip", "bp_mfma_tq1.hip", "bp_tq1_gemv.hip"}
+_REMARK = "[-Rpass-analysis=kernel-resource-usage]"
+
+
 def _compile(src: str) -> Path:
     obj = CSRC / (src + ".o")
-    cmd = ["hipcc", *FLAGS, "-c", str(CSRC / src), "-o", str(obj)]
+    check = src in NO_STATIC_LDS
+    cmd = ["hipcc", *FLAGS, *(["-Rpass-analysis=kernel-resource-usage"] if check else []), "-c", str(CSRC / src), "-o", str(obj)]
     res = subprocess.run(cmd, capture_output=True, text=True)
     noise = "is not a recognized feature for this target"
-    err = "\n".join(l for l in res.stderr.splitlines() if noise not in l)
+    lines = [l for l in res.stderr.splitlines() if noise not in l]
+    if check:  # drop the resource remarks (and the source excerpts printed under them) after reading the LDS sizes
+        kept, name, skip = [], "?", 0
+        for l in lines:
+            if _REMARK in l:
+                if "Function Name:" in l:
+                    name = l.split("Function Name:")[1].split()[0]
+                if "LDS Size [bytes/block]:" in l and int(l.split("LDS Size [bytes/block]:")[1].split()[0]) != 0:
+                    raise RuntimeError(f"{src}: kernel {name} uses static LDS; these kernels address LDS absolutely")
+                skip = 2
+            elif skip and (l.lstrip().startswith("|") or l.lstrip()[:1].isdigit()):
+                skip -= 1
+            else:
+                kept.append(l)
+        lines = kept
+    err = "\n".join(lines)
     if res.returncode != 0:
         raise RuntimeError(f"hipcc failed for {src}:\n{err}")
     if err.strip():

@@ -170,6 +170,7 @@ __global__ __launch_bounds__(GTHREADS, 2) void k_gemm_tq2(GemmArgs a) {
   asm volatile("" : "+v"(kc.M1), "+v"(kc.M2));
 
   const int steps = (int)(a.K / 256);
+  const int gs = a.group == 256 ? 1 : 0;  // scale groups of 256: the two 128-wide halves of a step share a scale (read from global memory)
   const int tiles = chunks == 1 ? 1 : a.n_terms * chunks;  // activation tiles to stage (one tile serves all terms)
   const unsigned stile = (unsigned)(2 * TILE);
   const unsigned xlane = (unsigned)(lane * 16);
@@ -207,7 +208,7 @@ __global__ __launch_bounds__(GTHREADS, 2) void k_gemm_tq2(GemmArgs a) {
       const int cc = c < steps ? c : 0;
 #pragma unroll
       for (int r = 0; r < GR; ++r) {
-        const unsigned so = (unsigned)(row_shift[r] * a.G + 2 * cc) * SB;
+        const unsigned so = (unsigned)(row_shift[r] * a.G + ((2 * cc) >> gs)) * SB;
         if (SL) {
           dst[r][0] = *(const lds_u32x4*)(slane + so);
           if (SDT == BP_F32) dst[r][1] = *(const lds_u32x4*)(slane + so + 16);
@@ -299,7 +300,9 @@ __global__ __launch_bounds__(GTHREADS, 2) void k_gemm_tq2(GemmArgs a) {
                 wb[0] = tq2_decode_i8(lo);
                 wb[1] = tq2_decode_i8(hi);
               }
-              const float s = scale_at<SDT>(sraw[r], 2 * i + h);
+              // (scale groups of 256: one scale per step; both candidates are read with constant indices)
+            const float s_step = scale_at<SDT>(sraw[r], i), s_group = scale_at<SDT>(sraw[r], 2 * i + h);
+            const float s = gs ? s_step : s_group;
               acc_t acc[GT];
 #pragma unroll
               for (int mt = 0; mt < MTN; ++mt) acc[mt] = base[mt];
@@ -376,8 +379,8 @@ template <int ACT, int SDT, int SL, int ABL = 0>
 int launch_gemm_k(const GemmArgs& a, hipStream_t s, size_t lds, const char* name) {
   static bool attr = false;
   if (!attr) {
-    if (hipFuncSetAttribute((const void*)k_gemm_tq2<ACT, SDT, SL, ABL>, hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024) != hipSuccess)
-      return fail(BP_ERR_LAUNCH, "cannot raise the dynamic LDS limit");
+    const hipError_t rc = hipFuncSetAttribute((const void*)k_gemm_tq2<ACT, SDT, SL, ABL>, hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
+    if (rc != hipSuccess) return fail(BP_ERR_LAUNCH, "cannot raise the dynamic LDS limit of the grouped GEMM kernel: %s", hipGetErrorString(rc));
     attr = true;
   }
   const dim3 grid((unsigned)((a.N + GROWS - 1) / GROWS * ((a.E + 7) / 8 * 8)), 1, (unsigned)((a.max_rows + 16 * GT - 1) / (16 * GT)));
@@ -392,7 +395,7 @@ int launch_gemm_sd(const GemmArgs& a, hipStream_t s, const char* name, const cha
   const size_t tiles = 2 * (size_t)gemm_tile_bytes<ACT>();
   const size_t stile = (size_t)GROWS * a.G * (SDT == BP_F32 ? 4 : 2);
   // (scale tile rows are read 16 bytes at a time: they must start 16-byte aligned)
-  if (tiles + stile <= 160 * 1024 && (a.G * (SDT == BP_F32 ? 4 : 2)) % 16 == 0) return launch_gemm_k<ACT, SDT, 1>(a, s, tiles + stile, name);
+  if (tiles + stile <= 160 * 1024 && (a.G * (SDT == BP_F32 ? 4 : 2)) % 16 == 0 && a.group == 128) return launch_gemm_k<ACT, SDT, 1>(a, s, tiles + stile, name);
   return launch_gemm_k<ACT, SDT, 0>(a, s, tiles, name_gs);
 }
 
@@ -402,7 +405,7 @@ int launch_gemm_sd(const GemmArgs& a, hipStream_t s, const char* name, const cha
 int launch_gemm_tq2(const GemmArgs& a, hipStream_t s) {
   if (const char* t = getenv("BP_TUNE_ABL")) {  // timing experiments: parts of the kernel switched off, results are wrong
     const size_t lds = 2 * gemm_tile_bytes<BP_BF16>() + (size_t)GROWS * a.G * 2;
-    if (a.x_dtype == BP_BF16 && a.scale_dtype == BP_F16 && lds <= 160 * 1024 && a.K % 1024 == 0) {
+    if (a.x_dtype == BP_BF16 && a.scale_dtype == BP_F16 && lds <= 160 * 1024 && a.K % 1024 == 0 && a.group == 128) {
       switch (atoi(t)) {
         case 2: return launch_gemm_k<BP_BF16, BP_F16, 1, 2>(a, s, lds, "gemm_abl2");
         case 3: return launch_gemm_k<BP_BF16, BP_F16, 1, 3>(a, s, lds, "gemm_abl3");

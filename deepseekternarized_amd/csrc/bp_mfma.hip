@@ -4,7 +4,8 @@
 namespace bp {
 
 bool mfma_supports(const GemmArgs& a) {
-  if (a.group != 128 || a.N % 16 != 0) return false;
+  // scale groups of 128, or of 256 (two 128-wide work groups per scale) from K = 2048 up
+  if ((a.group != 128 && !(a.group == 256 && a.K >= 2048)) || a.N % 16 != 0) return false;
   if (((uintptr_t)a.x & 15) != 0) return false;
   if ((a.max_rows + 15) / 16 > 65535) return false;
   if (a.fmt == BP_TQ2) {
@@ -21,6 +22,7 @@ bool mfma_supports(const GemmArgs& a) {
   if (a.scale_dtype != BP_F16 && a.scale_dtype != BP_BF16 && a.scale_dtype != BP_F32) return false;
   if (a.x_dtype != BP_BF16 && a.x_dtype != BP_I8 && a.max_rows != 1) return false;
   if (a.K % 256 != 0 || a.K < 1024) return false;  // whole groups, and an even number of them (4-byte aligned scale rows)
+  if (a.group == 256 && a.K % 512 != 0) return false;
   for (int t = 0; t < a.n_terms; ++t)
     if (((uintptr_t)a.w_scale[t] & 3) != 0) return false;
   return true;

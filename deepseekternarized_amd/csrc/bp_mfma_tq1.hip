@@ -90,6 +90,7 @@ __global__ __launch_bounds__(WAVES * 64, 4) void k_mfma_tq1(GemmArgs a, int CPT 
   const unsigned lane_off = (unsigned)(r16 * 8);
 
   const int nchunks = (int)((a.K + 639) / 640);  // 128-byte chunks per row (the last may be partial)
+  const int gs = a.group == 256 ? 1 : 0;         // scale groups of 256: two 128-wide work groups share a scale
 
   // ---- activation tile: slot (cl, g, 7 b + m) of token t at XB0 + t * pitch + ((cl * 5 + g) * 28 + 7 b + m) * 16
   const int tile_slots = CPT * T1_SLOTS;
@@ -197,9 +198,9 @@ __global__ __launch_bounds__(WAVES * 64, 4) void k_mfma_tq1(GemmArgs a, int CPT 
         wq[j][1] = buf_load16(wrs, voff, so + 64);
         wt[j] = buf_load4(wrs, voff_row, so + 128);
         if (!SL && SDT == BP_F32) {  // k-blocks 0..2 fetch two scales each: groups 5 cl .. 5 cl + 5 (past the rows: zeros)
-          sq2[j] = buf_load8(srs, soff_lane, 4u * 5 * cl);
+          sq2[j] = buf_load8(srs, soff_lane, 4u * ((5 * cl) >> gs));
         } else if (!SL) {  // k-blocks 0..2 fetch one dword each = 2 of the 6 scales starting at an even group index
-          int gi = (5 * cl) & ~1;
+          int gi = ((5 * cl) >> gs) & ~1;
           if (gi > (int)a.G - 6) gi = (int)a.G - 6;
           sq[j] = buf_load4(srs, soff_lane, 2u * gi);
         }
@@ -253,11 +254,11 @@ __global__ __launch_bounds__(WAVES * 64, 4) void k_mfma_tq1(GemmArgs a, int CPT 
           if (next_tile < nchunks) stage_load(next_tile);
         }
         const unsigned rb = rbuf0 + (c & 1) * 16 * WROW;
-        const int groups_left = (int)a.G - 5 * c;
+        const int groups_left = ((int)a.G << gs) - 5 * c;  // 128-wide work groups left in the row
         const int ng = groups_left < 5 ? groups_left : 5;
-        int gi = (5 * c) & ~1;
+        int gi = ((5 * c) >> gs) & ~1;
         if (gi > (int)a.G - 6) gi = (int)a.G - 6;
-        const int sshift = 5 * c - gi;  // position of group 5c among the 6 scales loaded (!SL)
+        const int sshift = -gi;  // scale s of the row sits at position s - gi among the 6 loaded (!SL)
         const unsigned xoff = (unsigned)((c - tile_c0) * T1_XCHUNK);
         if (ABL == 1) {  // ablation (timing experiments only): memory traffic without decode and MFMA
 #pragma unroll
@@ -268,9 +269,10 @@ __global__ __launch_bounds__(WAVES * 64, 4) void k_mfma_tq1(GemmArgs a, int CPT 
         for (int g = 0; g < 5; ++g) {
           if (g < ng) {
             unsigned half;  // the group's scale (bits as stored)
-            if (SDT == BP_F32) half = SL ? *(const lds_u32*)(slane + 4 * (5 * c + g)) : *(const lds_u32*)(rb + 136 + 4 * g);
-            else if (SL) half = *(const __attribute__((address_space(3))) uint16_t*)(slane + 2 * (5 * c + g));
-            else half = *(const __attribute__((address_space(3))) uint16_t*)(rb + 132 + 2 * (sshift + g));
+            const int sidx = (5 * c + g) >> gs;  // the 128-wide group's scale (group 256: two of them share one)
+            if (SDT == BP_F32) half = SL ? *(const lds_u32*)(slane + 4 * sidx) : *(const lds_u32*)(rb + 136 + 4 * (sidx - ((5 * c) >> gs)));
+            else if (SL) half = *(const __attribute__((address_space(3))) uint16_t*)(slane + 2 * sidx);
+            else half = *(const __attribute__((address_space(3))) uint16_t*)(rb + 132 + 2 * (sshift + sidx));
             // the 7 bytes of this lane's k-block for group g, read back from the transpose buffer
             const unsigned o = dlt + FB[g] + 7 * b;
             const unsigned d0 = *(const lds_u32*)(rb + (o & ~3u));

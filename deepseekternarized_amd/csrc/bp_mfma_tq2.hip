@@ -128,6 +128,7 @@ __global__ __launch_bounds__(WAVES * 64, 4) void k_mfma_tq2(GemmArgs a, int KC, 
   asm volatile("" : "+v"(kc.M1), "+v"(kc.M2));
 
   const int steps = (int)(a.K / 256);
+  const int gs = a.group == 256 ? 1 : 0;  // scale groups of 256: the two 128-wide halves of a step share a scale (read from global memory)
   const int steps_per_chunk = KC / 256;
   const int chunks = (steps + steps_per_chunk - 1) / steps_per_chunk;
 
@@ -170,7 +171,7 @@ __global__ __launch_bounds__(WAVES * 64, 4) void k_mfma_tq2(GemmArgs a, int KC, 
       const int cc = c < steps ? c : 0;
 #pragma unroll
       for (int r = 0; r < R; ++r) {
-        const unsigned so = (unsigned)(row_shift[r] * a.G + 2 * cc) * SB;
+        const unsigned so = (unsigned)(row_shift[r] * a.G + ((2 * cc) >> gs)) * SB;
         if (SL) {
           dst[r][0] = *(const lds_u32x4*)(slane + so);
           if (SDT == BP_F32 || PF == 8) dst[r][1] = *(const lds_u32x4*)(slane + so + 16);
@@ -260,7 +261,9 @@ __global__ __launch_bounds__(WAVES * 64, 4) void k_mfma_tq2(GemmArgs a, int KC, 
                 wb[0] = tq2_decode_i8(lo);
                 wb[1] = tq2_decode_i8(hi);
               }
-              const float s = scale_at<SDT>(sraw[r], 2 * i + h);  // group 2c + h = entry 2i + h of the 8 held
+              // group 2c + h = entry 2i + h of the 8 held (scale groups of 256: one scale per step, entry i)
+              const float s_step = scale_at<SDT>(sraw[r], i), s_group = scale_at<SDT>(sraw[r], 2 * i + h);  // (both with constant indices)
+              const float s = gs ? s_step : s_group;
 #pragma unroll
               for (int mt = 0; mt < MT; ++mt) {
                 acc_t acc = base[mt];
@@ -349,7 +352,7 @@ int launch_tq2_sd(const GemmArgs& a, hipStream_t s, const char* name) {
   // scales through LDS whenever the workgroup's share of one term fits the budget
   const int64_t tile = (int64_t)WAVES * 16 * R * a.G * (a.scale_dtype == BP_F32 ? 4 : 2);
   // (the tile is read 16 bytes at a time from a row's start + 4 c: rows must be 16 bytes apart modulo 16)
-  if (tile <= tq2_scale_tile_max(R) && (a.G * (a.scale_dtype == BP_F32 ? 4 : 2)) % 16 == 0) {
+  if (tile <= tq2_scale_tile_max(R) && (a.G * (a.scale_dtype == BP_F32 ? 4 : 2)) % 16 == 0 && a.group == 128) {
     int rc;
     if (a.scale_dtype == BP_F16) rc = launch_tq2<ACT, BP_F16, R, MT, WAVES, XKB, 0, NQ, 1>(a, s, name);
     else if (a.scale_dtype == BP_BF16) rc = launch_tq2<ACT, BP_BF16, R, MT, WAVES, XKB, 0, NQ, 1>(a, s, name);

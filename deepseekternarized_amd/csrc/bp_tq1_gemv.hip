@@ -70,6 +70,7 @@ __global__ __launch_bounds__(WAVES * 64, 4) void k_tq1_gemv(GemmArgs a, int CPT 
   if (!wave_live) n0 = 0;  // keeps addresses valid; the wave still takes part in staging and barriers
 
   const int nchunks = (int)((a.K + 639) / 640);  // 128-byte chunks per row (the last may be partial)
+  const int gs = a.group == 256 ? 1 : 0;         // scale groups of 256: two 128-wide work groups share a scale
   const int tile_slots = CPT * G1_SLOTS;
   // ---- table tile: the table of slot (cl, g, 7 b + m) sits at TB + ((cl * 5 + g) * 28 + 4 m + b) * 176.
   // The LDS has 32 banks and serves a wave's 4-byte reads half a wave at a time (measured): lane groups b = 0, 1
@@ -169,7 +170,7 @@ __global__ __launch_bounds__(WAVES * 64, 4) void k_tq1_gemv(GemmArgs a, int CPT 
         wq[j][1] = buf_load16(wrs, voff, so + 64);
         wt[j] = g1_load8(wrs, voff_row, so + 128);
         if (!SL) {  // k-blocks 0..2 fetch one dword each = 2 of the 6 scales starting at an even group index
-          int gi = (5 * cl) & ~1;
+          int gi = ((5 * cl) >> gs) & ~1;
           if (gi > (int)a.G - 6) gi = (int)a.G - 6;
           sq[j] = g1_load4(srs, soff_lane, 2u * gi);
         }
@@ -223,11 +224,11 @@ __global__ __launch_bounds__(WAVES * 64, 4) void k_tq1_gemv(GemmArgs a, int CPT 
         next_tile += CPT;
         if (next_tile < nchunks) stage_load(next_tile);
       }
-      const int groups_left = (int)a.G - 5 * c;
+      const int groups_left = ((int)a.G << gs) - 5 * c;  // 128-wide work groups left in the row
       const int ng = groups_left < 5 ? groups_left : 5;
-      int gi = (5 * c) & ~1;
+      int gi = ((5 * c) >> gs) & ~1;
       if (gi > (int)a.G - 6) gi = (int)a.G - 6;
-      const int sshift = 5 * c - gi;  // position of group 5c among the 6 scales loaded (!SL)
+      const int sshift = -gi;  // scale s of the row sits at position s - gi among the 6 loaded (!SL)
       // this lane's first table of the chunk; the slot within the chunk is an instruction offset
       unsigned tbl = (unsigned)(TB + (c - tile_c0) * G1_CHUNK_BYTES + G1_SLOT_BYTES * b);
       asm volatile("" : "+v"(tbl));  // one register; the rest of every table address is q, r and an instruction offset
@@ -235,9 +236,10 @@ __global__ __launch_bounds__(WAVES * 64, 4) void k_tq1_gemv(GemmArgs a, int CPT 
       for (int g = 0; g < 5; ++g) {
         if (g < ng) {
           unsigned half;  // the group's scale (bits as stored)
-          if (SDT == BP_F32) half = *(const lds_u32*)(slane + 4 * (5 * c + g));
-          else if (SL) half = *(const __attribute__((address_space(3))) uint16_t*)(slane + 2 * (5 * c + g));
-          else half = *(const __attribute__((address_space(3))) uint16_t*)(rb + 136 + 2 * (sshift + g));
+          const int sidx = (5 * c + g) >> gs;  // the 128-wide group's scale (group 256: two of them share one)
+          if (SDT == BP_F32) half = *(const lds_u32*)(slane + 4 * sidx);
+          else if (SL) half = *(const __attribute__((address_space(3))) uint16_t*)(slane + 2 * sidx);
+          else half = *(const __attribute__((address_space(3))) uint16_t*)(rb + 136 + 2 * (sshift + sidx));
           // the 7 bytes of this lane's slots for group g, read back from the transpose buffer
           const unsigned o = dlt + FB[g] + 7 * b;
           const unsigned d0 = *(const lds_u32*)(rb + (o & ~3u));

@@ -44,10 +44,10 @@ def _activations(rng, T, K, act):
     return x, None, dev(x), None
 
 
-def _run(bp, fmt, E, N, K, counts, act, terms=1, seed=0, misalign_scales=False, scale_dtype=np.float16):
+def _run(bp, fmt, E, N, K, counts, act, terms=1, seed=0, misalign_scales=False, scale_dtype=np.float16, group=GROUP):
     """Grouped call with `counts[e]` rows per expert; returns (got, want, kernel name)."""
     rng = np.random.default_rng(seed)
-    packed, scales = synth_weights(seed, E, N, K, GROUP, fmt, terms=terms)
+    packed, scales = synth_weights(seed, E, N, K, group, fmt, terms=terms)
     offsets = np.concatenate([[0], np.cumsum(counts)]).astype(np.int64)
     T = int(offsets[-1])
     x, xs, xd, xsd = _activations(rng, T, K, act)
@@ -56,7 +56,7 @@ def _run(bp, fmt, E, N, K, counts, act, terms=1, seed=0, misalign_scales=False, 
         a, b = int(offsets[e]), int(offsets[e + 1])
         for p, s in zip(packed, scales):
             if b > a:
-                c_gemm(x[a:b], None if xs is None else xs[a:b], p[e], s[e].astype(np.float32), K, GROUP, fmt, out=want[a:b])
+                c_gemm(x[a:b], None if xs is None else xs[a:b], p[e], s[e].astype(np.float32), K, group, fmt, out=want[a:b])
     pk = [dev(p) for p in packed]
     if scale_dtype is np.float16:
         sc = [dev(s) for s in scales]
@@ -70,7 +70,7 @@ def _run(bp, fmt, E, N, K, counts, act, terms=1, seed=0, misalign_scales=False, 
             a, b = int(offsets[e]), int(offsets[e + 1])
             for p, s in zip(packed, sc):
                 if b > a:
-                    c_gemm(x[a:b], None if xs is None else xs[a:b], p[e], s[e].float().cpu().numpy(), K, GROUP, fmt, out=want[a:b])
+                    c_gemm(x[a:b], None if xs is None else xs[a:b], p[e], s[e].float().cpu().numpy(), K, group, fmt, out=want[a:b])
     if misalign_scales:  # a view whose data pointer is 4- but not 16-byte aligned
         moved = []
         for s in sc:
@@ -79,7 +79,7 @@ def _run(bp, fmt, E, N, K, counts, act, terms=1, seed=0, misalign_scales=False, 
             moved.append(flat[2:].view(s.shape))
             assert moved[-1].data_ptr() % 16 == 4
         sc = moved
-    got = bp.grouped_ternary_gemm(xd, xsd, offsets.tolist(), pk, sc, K, GROUP, fmt)  # host offsets: max_rows = widest expert
+    got = bp.grouped_ternary_gemm(xd, xsd, offsets.tolist(), pk, sc, K, group, fmt)  # host offsets: max_rows = widest expert
     return got.cpu().numpy(), want, bp.ext().last_kernel()
 
 
@@ -253,3 +253,17 @@ def test_moe_layer_graph_replays_match_eager(bp, fmt, act, tokens):
         assert torch.isfinite(got).all() and torch.equal(got, want), (rep, (got.float() - want.float()).abs().max().item())
     with pytest.raises(ValueError):
         moe.graphed(65)
+
+
+# --------------------------------------------------------------------------- scale groups of 256
+@pytest.mark.parametrize("act", ["bf16", "int8"])
+@pytest.mark.parametrize("fmt,K,counts,prefix", [
+    ("tq2", 2048, [1, 0, 1], "mfma_tq2"), ("tq2", 7168, [16, 2, 5], "mfma_tq2"), ("tq2", 3072, [40, 1, 20], "gemm_tq2"),
+    ("tq1", 2048, [1, 1, 0], "lut_tq1"), ("tq1", 7168, [1, 0, 1], "lut_tq1"), ("tq1", 7168, [9, 16, 2], "mfma_tq1"),
+    ("tq1", 2560, [3, 0, 20], "mfma_tq1"),
+])
+def test_group_256(bp, act, fmt, K, counts, prefix):
+    """configs/policy/std_absmean_tq{1,2}_g256.yaml: one scale per 256 weights; the tuned kernels treat it as two 128-wide groups."""
+    got, want, kern = _run(bp, fmt, 3, 272, K, counts, act, terms=2, seed=K + sum(counts), group=256)
+    assert kern.startswith(prefix), kern
+    _check(got, want)
