@@ -330,6 +330,11 @@ int launch_g1_v(const GemmArgs& a, hipStream_t s, const char* name_sl, const cha
 
 // max_rows == 1 (checked by the caller); any activation dtype
 int launch_tq1_gemv(const GemmArgs& a, hipStream_t s, int waves) {
+  const char* t = getenv("BP_TUNE_TQ1");  // development: "lut" keeps the table kernel
+  if (!(t && t[0] == 'l')) {
+    const int rc = launch_tq1_gemv_fp4(a, s);
+    if (rc != BP_ERR_UNSUPPORTED) return rc;
+  }
   if (waves == 16) return launch_g1_v<16>(a, s, "lut_tq1_t1_w16", "lut_tq1_t1_w16_gs");
   return launch_g1_v<8>(a, s, "lut_tq1_t1_w8", "lut_tq1_t1_w8_gs");
 }

@@ -1,0 +1,477 @@
+// TQ1 single-token GEMV (decode, one token row per expert) on the block-float matrix instruction
+// v_mfma_f32_16x16x128_f8f6f4, weights as fp4 (E2M1 holds -1, 0, +1 exactly), activations as fp8 (E4M3) pieces.
+//
+// Contract as everywhere (boilerplate/kernels/ternary_cuda.py:58-63): out[n] += sum_g scale[n, g] * sum_{k in g}
+// x[k] * trit[n, k], float32 accumulation. What bounds a TQ1 GEMV on this chip is the work per packed byte: base-3
+// digits have no bit fields, so a byte must go through a table, and a table of partial sums costs two LDS reads
+// and ~10 vector operations per byte (bp_tq1_gemv.hip: a third of the HBM rate at best). Here a byte costs ONE
+// conflict-free LDS read and two vector operations:
+//
+//  * The table maps a byte to its five digits as five fp4 codes in one dword (three more nibbles stay 0). A
+//    lane's dword is used as is as a quarter of its operand B of the matrix instruction, so there is no unpacking.
+//    The table is replicated once per LDS bank (entry v, copy c at v * 128 + 4 c; a lane reads copy lane % 32), so
+//    no two lanes of a half-wave ever share a bank.
+//  * K order inside a matrix instruction is free as long as both operands agree, so the bytes a lane loaded (16
+//    consecutive bytes of its row per load, rows of a 16-row tile across lanes % 16, the four 16-byte quarters
+//    of a 64-byte span across lanes / 16) are multiplied where they are: no transpose through LDS.
+//  * The 16 rows of operand A are not tokens (there is one token) but (scale group, piece): a 128-byte chunk of a
+//    row holds 640 digits = 5 scale groups, and an activation is split into 3 fp8 pieces (below), 15 rows in all.
+//    Row (g, p) holds piece p of the activations of group g and zeros elsewhere, so one accumulator tile collects
+//    the 5 group sums of a chunk separately although groups end in the middle of bytes, and the group scales
+//    are applied once per chunk: total += scale[n, g] * (C[g, 0] + C[g, 1] + C[g, 2] / 256) / prescale[g].
+//    Rows 4 g + p are the pieces of group g < 4 and rows 3, 7, 11 those of group 4, so a lane of the result (rows
+//    4 kb + i) holds the three pieces of group kb and one piece of group 4.
+//  * fp8 pieces: the activations of a 128-wide group are multiplied by a power of two that brings the group's
+//    largest magnitude into [128, 256), then y = p0 + p1 + p2 / 256 with p0 = y truncated to E4M3 (4 significant bits), p1 = the
+//    remainder truncated likewise, p2 = 256 x the second remainder, truncated. bf16 (8 significant bits) and
+//    int8 activations are represented exactly by p0 + p1 down to 2^-9 of the scaled range and to 2^-17 with p2,
+//    fp16 (11 bits) by the three; what is dropped is below 2^-20 of the group's largest magnitude. Products
+//    fp8 x fp4 are exact and accumulate in float32. float32 activations are left to the table kernel.
+//
+// Operand A is read from an LDS tile built once per workgroup. It is stored compactly: per chunk, per matrix
+// instruction j = 0..7 and per 16-byte half of an A lane's operand (= the 2 x 8 digit slots of two consecutive
+// packed bytes) one block per piece with the digits outside the block's first group zeroed, a second block for
+// each of the 4 byte pairs that straddle a group boundary (digits outside the second group zeroed), and a block
+// of zeros. A lane (row (g, p)) reads the block of its piece if the byte pair lies in its group, else the zero
+// block; which one is a per-lane offset computed once.
+//
+// Rows start at any byte (Kp = ceil(K / 5) is not a multiple of 4), loads are dword-aligned (a misaligned
+// 16-byte load costs a quarter of the achievable HBM rate), and every row must present the same bytes to the
+// shared operand A: a lane shifts its window by its row's misalignment with v_alignbyte, taking the dword that
+// follows its 16 bytes from the lane that loaded it (ds_bpermute).
+//
+// Operand layout of the instruction with A = fp8 (8 VGPRs), B = fp4 (4 VGPRs), established by one-hot probing
+// on gfx950: B lane (n = lane % 16, kb = lane / 16), VGPR w, nibble q is paired with A lane (m = lane % 16,
+// kbA = 2 (kb % 2) + w / 2), VGPR 4 (kb / 2) + 2 (w % 2) + q / 4, byte q % 4; C lane (n, lg) holds rows 4 lg + i.
+#include <type_traits>
+
+#include "bp_mfma.h"
+
+namespace bp {
+namespace {
+
+typedef int i32x8 __attribute__((ext_vector_type(8)));
+template <int V>
+using IC = std::integral_constant<int, V>;
+struct __attribute__((packed, aligned(2))) F4Packed16 { u32x4 v; };
+struct __attribute__((packed, aligned(2))) F4Packed4 { unsigned v; };
+
+constexpr int F4_LUT_BYTES = 256 * 128;          // byte -> 5 fp4 codes, one copy per bank
+constexpr int F4_LO_BYTES = 64 * 3 * 16;         // per chunk: 64 byte pairs x 3 pieces x 16 bytes
+constexpr int F4_HI_OFF = F4_LO_BYTES;           // then 4 group boundaries x 3 pieces x 16 bytes
+constexpr int F4_ZERO_OFF = F4_HI_OFF + 4 * 3 * 16;
+constexpr int F4_PRE_OFF = F4_ZERO_OFF + 16;     // 8 words: the prescale of the chunk's 5 groups (3 unused)
+constexpr int F4_INV_OFF = F4_PRE_OFF + 32;      // 8 floats: their inverses (the unused ones are 0)
+constexpr int F4_CHUNK_BYTES = F4_INV_OFF + 32;  // 3344
+constexpr int F4_LDS_MAX = 160 * 1024;
+constexpr int F4_GR = 2;                         // 16-row tiles per wave (they share the reads of operand A)
+constexpr int F4_RD = 2;                         // chunks of packed bytes in registers per tile (the ring of loads in flight)
+constexpr int F4_BD = 2;                         // table reads run this many (instruction, tile) pairs ahead of the matrix instructions
+constexpr int F4_AD = 1;                         // 1: operand A is read one instruction ahead into a second set of registers
+
+__device__ __forceinline__ u32x2 f4_load8(__amdgpu_buffer_rsrc_t r, unsigned lane_off, unsigned wave_off) {
+  return __builtin_bit_cast(u32x2, __builtin_amdgcn_raw_buffer_load_b64(r, (int)lane_off, (int)wave_off, 0));
+}
+
+// first packed byte (of the chunk's 128) of the byte pair behind half `hf` of A lane quarter `kbA` in instruction j
+__device__ __forceinline__ int f4_pair_byte(int j, int kbA, int hf) {
+  return 64 * (j >> 2) + 16 * (2 * hf + (kbA >> 1)) + 4 * (j & 3) + 2 * (kbA & 1);
+}
+
+// ABL (development): timing ablations - 1 no chunk loop, 2 no table reads, 3 no operand A reads, 4 no matrix instructions, 5 no byte extraction (and the loads are not waited for),
+// 6 bytes extracted from registers that are not loaded (no loads at all), 7 = 2 + 3 + 4 (loads and byte extraction only),
+// 8 = 7 without the byte extraction (loads and their realignment only)
+template <int SDT, int WAVES, int ABL = 0>
+__global__ __launch_bounds__(WAVES * 64, 4) void k_tq1_gemv_fp4(GemmArgs a, int nchunks, int bpw /* row blocks per workgroup */) {
+  constexpr int THREADS = WAVES * 64, GR = F4_GR, RD = F4_RD, BD = F4_BD, AD = F4_AD;
+  constexpr int AT = F4_LUT_BYTES;           // the operand A tile starts after the table
+  constexpr int SB = SDT == BP_F32 ? 4 : 2;  // bytes per scale
+
+  const int wave = __builtin_amdgcn_readfirstlane((int)(threadIdx.x >> 6)), lane = threadIdx.x & 63;
+  const int r16 = lane & 15, kb = lane >> 4;
+  const int64_t e = blockIdx.y;
+  const int64_t o0 = clamp_i64(a.offsets[e], 0, a.T), o1 = clamp_i64(a.offsets[e + 1], 0, a.T);
+  if (o0 >= o1) return;  // uniform for the workgroup; only the expert's first token row is used (max_rows == 1)
+  const int64_t tok = o0;
+  const int gs = a.group == 256 ? 1 : 0;  // scale groups of 256: two 128-wide work groups share a scale
+  const bool x16 = a.x_dtype == BP_BF16 || a.x_dtype == BP_F16;
+  auto widen16 = [&](unsigned h) { return a.x_dtype == BP_BF16 ? bf16_bits_to_f32((uint16_t)h) : f16_bits_to_f32((uint16_t)h); };
+
+  // ---- the byte table: entry v = digits d0..d4 of v as fp4 codes (-1 -> 0xA, 0 -> 0, +1 -> 0x2) in nibbles 0..4;
+  // computed once per value into copy 0, then spread over the other 31 copies.
+  // Alongside: the largest magnitude of every 128-wide group of the token (LDS maximum over the float bits).
+  if (threadIdx.x < 256) {
+    unsigned v = threadIdx.x, ent = 0;
+    if (v < 243) {
+#pragma unroll
+      for (int d = 0; d < 5; ++d) {
+        const unsigned q = v / 3, dig = v - 3 * q;
+        ent |= (dig == 0 ? 0xAu : dig == 2 ? 0x2u : 0u) << (4 * d);
+        v = q;
+      }
+    }
+    *(lds_u32*)(128 * threadIdx.x) = ent;
+  }
+  for (int g = threadIdx.x; g < nchunks * 8; g += THREADS) *(lds_u32*)(AT + (g >> 3) * F4_CHUNK_BYTES + F4_PRE_OFF + 4 * (g & 7)) = 0u;
+  __syncthreads();
+  for (int idx = threadIdx.x; idx < 256 * 32; idx += THREADS) *(lds_u32*)(4 * idx) = *(const lds_u32*)(128 * (idx >> 5));
+  if (a.x_dtype != BP_I8) {  // (int8 values fit as they are: prescale 1)
+    for (int64_t k0 = 8 * (int64_t)threadIdx.x; k0 < a.K; k0 += 8 * THREADS) {  // 8 values of one group per thread
+      unsigned m = 0;
+      if (x16 && k0 + 8 <= a.K) {
+        const u32x4 q = ((const F4Packed16*)((const uint16_t*)a.x + tok * a.K + k0))->v;
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+          const unsigned lo = __float_as_uint(widen16(q[i] & 0xffffu)) & 0x7fffffffu, hi = __float_as_uint(widen16(q[i] >> 16)) & 0x7fffffffu;
+          m = m > lo ? m : lo;
+          m = m > hi ? m : hi;
+        }
+      } else {
+        for (int i = 0; i < 8 && k0 + i < a.K; ++i) {
+          const unsigned v = __float_as_uint(load_act_f32(a.x, a.x_dtype, tok * a.K + k0 + i)) & 0x7fffffffu;
+          m = m > v ? m : v;
+        }
+      }
+      const int gg = (int)(k0 >> 7);
+      __hip_atomic_fetch_max((lds_u32*)(AT + (gg / 5) * F4_CHUNK_BYTES + F4_PRE_OFF + 4 * (gg % 5)), m, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
+    }
+  }
+  __syncthreads();
+  // the maxima become prescales 2^sh (sh brings the group's largest magnitude into [128, 256)) and their inverses
+  for (int g = threadIdx.x; g < nchunks * 8; g += THREADS) {
+    const unsigned at = (unsigned)(AT + (g >> 3) * F4_CHUNK_BYTES + 4 * (g & 7));
+    const bool real = (g & 7) < 5 && 128 * (int64_t)(5 * (g >> 3) + (g & 7)) < a.K;
+    int sh = 0;
+    if (real && a.x_dtype != BP_I8) {
+      sh = 134 - (int)((*(const lds_u32*)(at + F4_PRE_OFF) >> 23) & 255u);
+      sh = sh > 120 ? 120 : sh < -120 ? -120 : sh;
+    }
+    *(lds_u32*)(at + F4_PRE_OFF) = (unsigned)(sh + 127) << 23;
+    *(lds_u32*)(at + F4_INV_OFF) = real ? (unsigned)(127 - sh) << 23 : 0u;
+  }
+  __syncthreads();
+
+  // ---- operand A tile: one item = the 10 activations behind a byte pair -> 3 pieces x (first-group block, second-group block)
+  for (int it = threadIdx.x; it < nchunks * 64; it += THREADS) {
+    const int c = it >> 6, blk = it & 63;
+    const int tt0 = 5 * f4_pair_byte(blk >> 3, (blk >> 1) & 3, blk & 1), glo = tt0 >> 7, ghi = (tt0 + 9) >> 7;
+    const unsigned dst = (unsigned)(AT + c * F4_CHUNK_BYTES);
+    const float pre_lo = __uint_as_float(*(const lds_u32*)(dst + F4_PRE_OFF + 4 * glo));
+    const float pre_hi = __uint_as_float(*(const lds_u32*)(dst + F4_PRE_OFF + 4 * ghi));
+    const int64_t k0 = 640 * (int64_t)c + tt0;
+    float y[10];
+    if (x16 && k0 + 10 <= a.K) {  // 20 bytes at an even address
+      const uint16_t* src = (const uint16_t*)a.x + tok * a.K + k0;
+      const u32x4 q = ((const F4Packed16*)src)->v;
+      const unsigned q4 = ((const F4Packed4*)(src + 8))->v;
+#pragma unroll
+      for (int i = 0; i < 4; ++i) { y[2 * i] = widen16(q[i] & 0xffffu); y[2 * i + 1] = widen16(q[i] >> 16); }
+      y[8] = widen16(q4 & 0xffffu);
+      y[9] = widen16(q4 >> 16);
+    } else {
+#pragma unroll
+      for (int t = 0; t < 10; ++t) y[t] = k0 + t < a.K ? load_act_f32(a.x, a.x_dtype, tok * a.K + k0 + t) : 0.f;
+    }
+    u32x4 lo[3] = {}, hi[3] = {};
+#pragma unroll
+    for (int t = 0; t < 10; t += 2) {  // two activations per conversion
+      const bool in0 = ((tt0 + t) >> 7) == glo, in1 = ((tt0 + t + 1) >> 7) == glo;
+      float r0 = y[t] * (in0 ? pre_lo : pre_hi), r1 = y[t + 1] * (in1 ? pre_lo : pre_hi);
+      const int pos0 = 8 * (t / 5) + t % 5, pos1 = 8 * ((t + 1) / 5) + (t + 1) % 5;  // digit slots of the block
+#pragma unroll
+      for (int p = 0; p < 3; ++p) {
+        const int w = __builtin_amdgcn_cvt_pk_fp8_f32(p == 2 ? r0 * 256.f : r0, p == 2 ? r1 * 256.f : r1, 0, false);
+        if (p < 2) {
+          r0 -= __builtin_amdgcn_cvt_f32_fp8(w, 0);
+          r1 -= __builtin_amdgcn_cvt_f32_fp8(w, 1);
+        }
+        const unsigned c0 = (unsigned)w & 0xffu, c1 = ((unsigned)w >> 8) & 0xffu;
+        lo[p][pos0 >> 2] |= (in0 ? c0 : 0u) << (8 * (pos0 & 3));
+        hi[p][pos0 >> 2] |= (in0 ? 0u : c0) << (8 * (pos0 & 3));
+        lo[p][pos1 >> 2] |= (in1 ? c1 : 0u) << (8 * (pos1 & 3));
+        hi[p][pos1 >> 2] |= (in1 ? 0u : c1) << (8 * (pos1 & 3));
+      }
+    }
+#pragma unroll
+    for (int p = 0; p < 3; ++p) *(lds_u32x4*)(dst + 16 * (3 * blk + p)) = lo[p];
+    if (ghi != glo) {
+#pragma unroll
+      for (int p = 0; p < 3; ++p) *(lds_u32x4*)(dst + F4_HI_OFF + 16 * (3 * (ghi - 1) + p)) = hi[p];
+    }
+    if (blk == 0) *(lds_u32x4*)(dst + F4_ZERO_OFF) = u32x4{0u, 0u, 0u, 0u};
+  }
+  __syncthreads();
+
+  // ---- this lane as a row of operand A: rows 4 g + p = piece p of group g < 4; rows 3, 7, 11 = pieces of group 4; row 15 unused
+  const int am_g = (r16 & 3) < 3 ? r16 >> 2 : 4, am_p = (r16 & 3) < 3 ? r16 & 3 : r16 >> 2;
+  unsigned aoff[4];  // 16-byte block (index within the chunk's part of the tile) of instruction j, half hf: byte 2 (j % 2) + hf of aoff[j / 2]
+#pragma unroll
+  for (int j = 0; j < 8; ++j) {
+    unsigned both = 0;
+#pragma unroll
+    for (int hf = 0; hf < 2; ++hf) {
+      const int blk = j * 8 + kb * 2 + hf;
+      const int tt0 = 5 * f4_pair_byte(j, kb, hf), glo = tt0 >> 7, ghi = (tt0 + 9) >> 7;
+      unsigned o = F4_ZERO_OFF / 16;
+      if (r16 < 15 && am_g == glo) o = 3 * blk + am_p;
+      else if (r16 < 15 && am_g == ghi) o = F4_HI_OFF / 16 + 3 * (ghi - 1) + am_p;
+      both |= o << (8 * hf);
+    }
+    if (j & 1) aoff[j >> 1] |= both << 16;
+    else aoff[j >> 1] = both;
+  }
+  // ---- this lane as a column of the result: rows 4 kb + i of C: pieces 0..2 of group kb, and piece kb of group 4
+  const float f4th = kb == 3 ? 0.f : kb == 2 ? 1.f / 256.f : 1.f;
+  const unsigned lane4 = (unsigned)(lane & 31) << 2;
+  const unsigned next_lane4 = (unsigned)((lane + 16) & 63) << 2, last_lane4 = (unsigned)(48 + r16) << 2;
+
+  // The tables serve `bpw` blocks of WAVES x 32 rows, one after the other (the build is paid once per workgroup).
+  for (int pass = 0; pass < bpw; ++pass) {
+  int64_t n0 = (((int64_t)blockIdx.x * bpw + pass) * WAVES + wave) * (16 * GR);
+  const bool wave_live = n0 < a.N;
+  if (!wave_live) n0 = 0;  // keeps addresses valid (the wave's results are not stored)
+  float total[GR];
+#pragma unroll
+  for (int s = 0; s < GR; ++s) total[s] = 0.f;
+
+  for (int term = 0; term < a.n_terms; ++term) {
+    // this wave's rows as a buffer that ends with the tensor; dword-aligned base, per-lane row offset
+    const unsigned char* wbeg = a.packed[term];
+    const unsigned char* wave_rows = wbeg + (e * a.N + n0) * a.Kp;
+    const unsigned mis = (unsigned)((uintptr_t)wave_rows & 3);
+    const __amdgpu_buffer_rsrc_t wrs = make_rsrc(wave_rows - mis, (wbeg + a.E * a.N * a.Kp) - (wave_rows - mis));
+    const unsigned ro = mis + (unsigned)r16 * (unsigned)a.Kp;
+    const unsigned dlt = ro & 3u;  // the lane's window starts dlt bytes before its bytes of the row
+    const unsigned voff = (ro & ~3u) + 16u * kb;
+    unsigned tile_off[GR], tile_soff[GR];  // (scalar) a tile past N repeats tile 0 and is not stored
+#pragma unroll
+    for (int s = 0; s < GR; ++s) {
+      const bool live = n0 + 16 * s < a.N;
+      tile_off[s] = live ? 16u * s * (unsigned)a.Kp : 0u;
+      tile_soff[s] = live ? 16u * s * (unsigned)a.G * SB : 0u;  // a multiple of 4
+    }
+    const unsigned char* sbeg = (const unsigned char*)a.w_scale[term];
+    const unsigned char* wave_scales = sbeg + (e * a.N + n0) * a.G * SB;
+    const unsigned smis = (unsigned)((uintptr_t)wave_scales & 3);
+    const __amdgpu_buffer_rsrc_t srs = make_rsrc(wave_scales - smis, (sbeg + a.E * a.N * a.G * SB) - (wave_scales - smis));
+    const unsigned srow = smis + (unsigned)r16 * (unsigned)a.G * SB;
+
+    // RD chunks in registers per tile; the two 64-byte halves of a chunk are refilled separately, each as soon as its
+    // last byte has gone into a table read, so a load has between RD - 1 and RD - 1/2 chunk times to land.
+    u32x4 W[RD][GR][2];
+    u32x2 SQ[GR];  // the scales of one chunk: refilled for the next chunk as soon as they have been applied
+    auto fetch_w = [&](int c, int slot, int h) {
+      const unsigned so = 128u * (c < nchunks ? c : nchunks - 1) + 64u * h;
+#pragma unroll
+      for (int s = 0; s < GR; ++s) W[slot][s][h] = buf_load16(wrs, voff, so + tile_off[s]);
+    };
+    auto scale_at = [&](int c) -> unsigned {  // offset of the dword that holds the scale of group kb of chunk c
+      const unsigned idx = (unsigned)((5 * (c < nchunks ? c : nchunks - 1) + kb) >> gs);
+      return (srow + SB * idx) & ~3u;
+    };
+    auto fetch_s = [&](unsigned at) {  // 8 bytes from there
+#pragma unroll
+      for (int s = 0; s < GR; ++s) SQ[s] = f4_load8(srs, at, tile_soff[s]);
+    };
+    // (chunk slots and pipeline stages are compile-time constants: every register array below is indexed statically)
+    auto step = [&](int c, auto cur_c) {
+      constexpr int cur = decltype(cur_c)::value, nxt = (cur + 1) % RD;
+      f32x4 C[GR];
+#pragma unroll
+      for (int s = 0; s < GR; ++s) C[s] = f32x4{0.f, 0.f, 0.f, 0.f};
+      const unsigned cbase = (unsigned)(AT + c * F4_CHUNK_BYTES);
+      // packed bytes of (instruction j, tile s) = dword j % 4 of the lane's window j / 4, shifted to the row's alignment;
+      // the dword after a window is the first one of the next quarter's window (for the last quarter: of the first
+      // quarter's next window, which for the second window is the next chunk's)
+      unsigned w4[GR], last[GR];  // (last: the last dword of the second window, kept while its registers are refilled)
+      auto bytes_of = [&](int j, int s) -> unsigned {
+        const int h = j >> 2, i = j & 3;
+        if (ABL == 5) return 0u;
+        if (ABL == 6) return __builtin_amdgcn_alignbyte(aoff[(j + 1) & 3], aoff[j & 3] + j, dlt);  // same arithmetic, nothing loaded
+        if (j == 7) return __builtin_amdgcn_alignbyte(w4[s], last[s], dlt);
+        return __builtin_amdgcn_alignbyte(i < 3 ? W[cur][s][h][i < 3 ? i + 1 : 0] : w4[s], W[cur][s][h][i], dlt);
+      };
+      auto table = [&](unsigned d, u32x4& B) {
+#pragma unroll
+        for (int w = 0; w < 4; ++w) {
+          const unsigned at = ABL == 5 ? (unsigned)(w << 7) | lane4 : ABL == 8 ? d : (((d >> (8 * w)) & 0xffu) << 7) | lane4;
+          B[w] = ABL == 2 || ABL == 7 || ABL == 8 ? at : *(const lds_u32*)at;
+        }
+      };
+      auto a_read = [&](int j, u32x4& lo, u32x4& hi) {
+        if (ABL == 3 || ABL == 7 || ABL == 8) { lo = u32x4{cbase, dlt, lane4, cbase}; hi = lo; return; }
+        lo = *(const lds_u32x4*)((((aoff[j >> 1] >> (16 * (j & 1))) & 0xffu) << 4) + cbase);
+        hi = *(const lds_u32x4*)((((aoff[j >> 1] >> (16 * (j & 1) + 8)) & 0xffu) << 4) + cbase);
+      };
+      // software pipeline over the 16 (instruction, tile) pairs t = 2 j + s: table reads BD pairs ahead, operand A one
+      // instruction ahead if AD; the scheduling barriers keep the compiler from sinking the reads back to their uses
+      u32x4 Bq[BD + 1];
+      u32x4 Alo[AD + 1], Ahi[AD + 1];
+      auto lookup = [&](auto p_c) {  // table reads of pair p
+        constexpr int p = decltype(p_c)::value, j = p >> 1, s = p & 1;
+        if (j == 3)  // the dword after the first window: the first one of the next quarter's first window, or of the own second window
+          w4[s] = (unsigned)__builtin_amdgcn_ds_bpermute((int)next_lane4, (int)(kb == 0 ? W[cur][s][1].x : W[cur][s][0].x));
+        if (p == 14) {
+          // The dword after the second window comes from the next quarter's second window, for the last quarter
+          // from the next chunk. What the last instruction still needs of this chunk is set aside, the chunk's
+          // registers are refilled (RD chunks on), and only then is the next chunk's first dword waited for: the
+          // wave never waits with fewer than RD - 1 chunks in flight behind the one it waits for.
+          unsigned same[GR];
+#pragma unroll
+          for (int q = 0; q < GR; ++q) {
+            // (a copy the compiler cannot merge with its source: kept in the same register, it would make the refill
+            // below load into other registers and copy them at the end of the loop - after waiting for the load)
+            asm volatile("v_mov_b32 %0, %1" : "=v"(last[q]) : "v"(W[cur][q][1].w));
+            same[q] = (unsigned)__builtin_amdgcn_ds_bpermute((int)next_lane4, (int)W[cur][q][1].x);
+          }
+          fetch_w(c + RD, cur, 0);  // both windows together: the two loads of a row's 128 bytes then meet in the L1
+          fetch_w(c + RD, cur, 1);
+#pragma unroll
+          for (int q = 0; q < GR; ++q) {
+            const unsigned far = (unsigned)__builtin_amdgcn_ds_bpermute((int)next_lane4, (int)W[nxt][q][0].x);
+            w4[q] = kb == 3 ? far : same[q];
+          }
+        }
+        table(bytes_of(j, s), Bq[p % (BD + 1)]);
+      };
+      a_read(0, Alo[0], Ahi[0]);
+      lookup(IC<0>{});
+      if (BD > 1) lookup(IC<BD - 1>{});
+      auto stage = [&](auto t_c) {
+        constexpr int t = decltype(t_c)::value, j = t >> 1, s = t & 1;
+        if (t + BD < 16) lookup(IC<(t + BD < 16 ? t + BD : 0)>{});
+        if (AD && s == 0 && j + 1 < 8) a_read(j + 1, Alo[(j + 1) & AD], Ahi[(j + 1) & AD]);
+
+        __builtin_amdgcn_sched_barrier(0);
+        const u32x4 alo = Alo[j & AD], ahi = Ahi[j & AD];
+        const i32x8 A = {(int)alo.x, (int)alo.y, (int)alo.z, (int)alo.w, (int)ahi.x, (int)ahi.y, (int)ahi.z, (int)ahi.w};
+        const u32x4 bq = Bq[t % (BD + 1)];
+        const i32x8 B = {(int)bq.x, (int)bq.y, (int)bq.z, (int)bq.w, 0, 0, 0, 0};
+        if (ABL == 4 || ABL == 7 || ABL == 8) asm volatile("; operands stay live" ::"v"(bq), "v"(alo), "v"(ahi));
+        else C[s] = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(A, B, C[s], 0 /* A: E4M3 */, 4 /* B: E2M1 */, 0, 0, 0, 0);
+        if (!AD && s == 1 && j + 1 < 8) a_read(j + 1, Alo[0], Ahi[0]);  // both tiles have issued with this operand
+        __builtin_amdgcn_sched_barrier(0);
+      };
+      stage(IC<0>{}); stage(IC<1>{}); stage(IC<2>{}); stage(IC<3>{}); stage(IC<4>{}); stage(IC<5>{}); stage(IC<6>{}); stage(IC<7>{});
+      stage(IC<8>{}); stage(IC<9>{}); stage(IC<10>{}); stage(IC<11>{}); stage(IC<12>{}); stage(IC<13>{}); stage(IC<14>{}); stage(IC<15>{});
+      // the chunk's 5 group sums under their scales: this lane holds group kb (3 pieces) and a piece of group 4, whose
+      // scale sits next to that of group 3 in the lanes kb = 3
+      const float inv_a = __uint_as_float(*(const lds_u32*)(cbase + F4_INV_OFF + 4 * kb));
+      const float inv_4 = __uint_as_float(*(const lds_u32*)(cbase + F4_INV_OFF + 16)) * f4th;
+      const unsigned ia = (unsigned)((5 * c + kb) >> gs), ib = (unsigned)((5 * c + kb + 1) >> gs);
+#pragma unroll
+      for (int s = 0; s < GR; ++s) {
+        unsigned ra, rb;  // the scale of group kb, and the one after it (bits as stored)
+        if (SDT == BP_F32) {
+          ra = SQ[s].x;
+          rb = ib == ia ? ra : SQ[s].y;
+        } else {
+          const unsigned v = __builtin_amdgcn_alignbyte(SQ[s].y, SQ[s].x, (srow + SB * ia) & 3u);
+          ra = v & 0xffffu;
+          rb = ib == ia ? ra : v >> 16;
+        }
+        const unsigned r4 = (unsigned)__builtin_amdgcn_ds_bpermute((int)last_lane4, (int)rb);
+        const float sa = SDT == BP_F32 ? __uint_as_float(ra) : SDT == BP_F16 ? f16_bits_to_f32((uint16_t)ra) : __uint_as_float(ra << 16);
+        const float s4 = SDT == BP_F32 ? __uint_as_float(r4) : SDT == BP_F16 ? f16_bits_to_f32((uint16_t)r4) : __uint_as_float(r4 << 16);
+        total[s] += sa * inv_a * (C[s][0] + C[s][1] + C[s][2] * (1.f / 256.f)) + s4 * inv_4 * C[s][3];
+      }
+      fetch_s(scale_at(c + 1));
+    };
+
+    // The first loads, in the order of use and with the scales last: the waits at the head of the loop are counted
+    // along this path too, and here as there the 4 loads of the next chunk and the 2 of the scales are the ones
+    // in flight behind the chunk that is needed.
+    const unsigned first_scale = scale_at(0);
+    __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+    for (int u = 0; u < RD; ++u) {
+      fetch_w(u, u, 0);
+      fetch_w(u, u, 1);
+    }
+    __builtin_amdgcn_sched_barrier(0);
+    fetch_s(first_scale);
+    __builtin_amdgcn_sched_barrier(0);
+    // RD chunks per iteration with no way around any of them: the compiler counts the loads in flight along every
+    // path into the head of the loop, and a path on which fewer are in flight would make every iteration wait
+    const int full_end = ABL == 1 ? 0 : nchunks - nchunks % RD;
+    for (int c0 = 0; c0 < full_end; c0 += RD) {
+      step(c0, IC<0>{});
+      step(c0 + 1, IC<1 % RD>{});
+      if (RD > 2) step(c0 + 2, IC<2 % RD>{});
+    }
+    if (ABL != 1 && nchunks - full_end > 0) step(full_end, IC<0>{});  // uniform
+    if (ABL != 1 && nchunks - full_end > 1) step(full_end + 1, IC<1 % RD>{});
+  }
+  // ---- epilogue: the four quarter lanes of a row hold its partial sums
+#pragma unroll
+  for (int s = 0; s < GR; ++s) {
+    float t = total[s];
+    t += __shfl_xor(t, 16);
+    t += __shfl_xor(t, 32);
+    if (kb == 0 && wave_live && n0 + 16 * s < a.N) {
+      float* o = a.out + tok * a.N + n0 + 16 * s + r16;
+      *o += a.x_dtype == BP_I8 ? t * a.x_scale[tok] : t;
+    }
+  }
+  }  // pass
+}
+template <int SDT, int WAVES, int ABL = 0>
+int launch_f4_k(const GemmArgs& a, hipStream_t s, const char* name, int nchunks, size_t lds) {
+  static bool attr = false;
+  static int cus = 0;
+  if (!attr) {
+    const hipError_t rc = hipFuncSetAttribute((const void*)k_tq1_gemv_fp4<SDT, WAVES, ABL>, hipFuncAttributeMaxDynamicSharedMemorySize, F4_LDS_MAX);
+    if (rc != hipSuccess) return fail(BP_ERR_LAUNCH, "cannot raise the dynamic LDS limit: %s", hipGetErrorString(rc));
+    int dev = 0;
+    if (hipGetDevice(&dev) != hipSuccess || hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || cus < 1) cus = 256;
+    attr = true;
+  }
+  // Every workgroup builds the tables of its expert's token, so a workgroup takes as many row blocks as still leaves
+  // every CU its full set of resident workgroups (16 waves): one round of workgroups, one build each.
+  const int64_t rows_per_block = (int64_t)WAVES * 16 * F4_GR;
+  const int64_t blocks = (a.N + rows_per_block - 1) / rows_per_block;  // per expert
+  const int64_t resident = (int64_t)cus * (16 / WAVES);
+  const int64_t experts = a.E < a.T ? a.E : a.T;  // (an expert without a token returns at once)
+  int64_t bpw = blocks * experts / resident;
+  bpw = bpw < 1 ? 1 : bpw > blocks ? blocks : bpw;
+  const dim3 grid((unsigned)((blocks + bpw - 1) / bpw), (unsigned)a.E, 1u);
+  note_kernel(name);
+  hipLaunchKernelGGL((k_tq1_gemv_fp4<SDT, WAVES, ABL>), grid, dim3(WAVES * 64), lds, s, a, nchunks, (int)bpw);
+  return check_launch(name);
+}
+
+template <int SDT>
+int launch_f4(const GemmArgs& a, hipStream_t s) {
+  const int64_t nchunks = (a.K + 639) / 640;
+  const size_t lds = (size_t)(F4_LUT_BYTES + nchunks * F4_CHUNK_BYTES);
+  if (lds > (size_t)F4_LDS_MAX) return BP_ERR_UNSUPPORTED;
+  if (const char* t = getenv("BP_TUNE_F4ABL")) {  // development: timing ablations
+    if (SDT == BP_F16 && atoi(t) == 1) return launch_f4_k<BP_F16, 8, 1>(a, s, "abl1_fp4", (int)nchunks, lds);
+    if (SDT == BP_F16 && atoi(t) == 2) return launch_f4_k<BP_F16, 8, 2>(a, s, "abl2_fp4", (int)nchunks, lds);
+    if (SDT == BP_F16 && atoi(t) == 3) return launch_f4_k<BP_F16, 8, 3>(a, s, "abl3_fp4", (int)nchunks, lds);
+    if (SDT == BP_F16 && atoi(t) == 4) return launch_f4_k<BP_F16, 8, 4>(a, s, "abl4_fp4", (int)nchunks, lds);
+    if (SDT == BP_F16 && atoi(t) == 5) return launch_f4_k<BP_F16, 8, 5>(a, s, "abl5_fp4", (int)nchunks, lds);
+    if (SDT == BP_F16 && atoi(t) == 6) return launch_f4_k<BP_F16, 8, 6>(a, s, "abl6_fp4", (int)nchunks, lds);
+    if (SDT == BP_F16 && atoi(t) == 7) return launch_f4_k<BP_F16, 8, 7>(a, s, "abl7_fp4", (int)nchunks, lds);
+    if (SDT == BP_F16 && atoi(t) == 8) return launch_f4_k<BP_F16, 8, 8>(a, s, "abl8_fp4", (int)nchunks, lds);
+  }
+  // two workgroups of 8 waves per CU when their tiles fit side by side, else one of 16
+  if (lds <= (size_t)F4_LDS_MAX / 2) return launch_f4_k<SDT, 8>(a, s, "fp4_tq1_t1_w8", (int)nchunks, lds);
+  return launch_f4_k<SDT, 16>(a, s, "fp4_tq1_t1_w16", (int)nchunks, lds);
+}
+
+}  // namespace
+
+// max_rows == 1 (checked by the caller). BP_ERR_UNSUPPORTED (no message): the caller falls back to the table kernel.
+int launch_tq1_gemv_fp4(const GemmArgs& a, hipStream_t s) {
+  if (a.x_dtype != BP_BF16 && a.x_dtype != BP_F16 && a.x_dtype != BP_I8) return BP_ERR_UNSUPPORTED;
+  if (a.N % 16 != 0 || a.Kp != (a.K + 4) / 5 || (a.group != 128 && a.group != 256)) return BP_ERR_UNSUPPORTED;
+  for (int t = 0; t < a.n_terms; ++t)
+    if (a.scale_dtype == BP_F32 && ((uintptr_t)a.w_scale[t] & 3) != 0) return BP_ERR_UNSUPPORTED;
+  if (a.scale_dtype == BP_F16) return launch_f4<BP_F16>(a, s);
+  if (a.scale_dtype == BP_BF16) return launch_f4<BP_BF16>(a, s);
+  if (a.scale_dtype == BP_F32) return launch_f4<BP_F32>(a, s);
+  return BP_ERR_UNSUPPORTED;
+}
+
+}  // namespace bp

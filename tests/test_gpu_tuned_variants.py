@@ -88,37 +88,79 @@ def _check(got, want):
     assert rel_l2(got, want) <= REL_L2, rel_l2(got, want)
 
 
-# --------------------------------------------------------------------------- TQ1 decode GEMV (table lookup)
+# --------------------------------------------------------------------------- TQ1 decode GEMV
+# Two kernels: fp8 x fp4 matrix instructions (16-bit and int8 activations, tables that fit in LDS) and the table
+# lookup of partial sums (everything else; BP_TUNE_TQ1=lut selects it for every call, read at each call).
+@pytest.fixture(params=["fp4", "lut"])
+def gemv_kernel(request, monkeypatch):
+    if request.param == "lut":
+        monkeypatch.setenv("BP_TUNE_TQ1", "lut")
+    else:
+        monkeypatch.delenv("BP_TUNE_TQ1", raising=False)
+    return request.param + "_tq1"
+
+
 @pytest.mark.parametrize("K", [1024, 1280, 2048, 4352, 7168])  # Kp = 205 (odd: rows at every byte alignment), 256, 410, 871, 1434
 @pytest.mark.parametrize("act", ["bf16", "int8"])
-def test_tq1_gemv_row_alignments_and_tiles(bp, K, act):
+def test_tq1_gemv_row_alignments_and_tiles(bp, K, act, gemv_kernel):
     got, want, kern = _run(bp, "tq1", 3, 48, K, [1, 0, 1], act, seed=K)
-    assert kern.startswith("lut_tq1"), kern
+    assert kern.startswith(gemv_kernel), kern
     _check(got, want)
 
 
-@pytest.mark.parametrize("act", ["f16", "f32"])
-def test_tq1_gemv_other_activation_dtypes(bp, act):
+@pytest.mark.parametrize("act,prefix", [("f16", "fp4_tq1"), ("f32", "lut_tq1")])
+def test_tq1_gemv_other_activation_dtypes(bp, act, prefix, gemv_kernel):
     got, want, kern = _run(bp, "tq1", 2, 32, 2048, [1, 1], act, seed=3)
-    assert kern.startswith("lut_tq1"), kern
+    assert kern.startswith(prefix if gemv_kernel == "fp4_tq1" else "lut_tq1"), kern
     _check(got, want)
 
 
-def test_tq1_gemv_many_rows_two_terms_bf16_scales(bp):
+def test_tq1_gemv_many_rows_two_terms_bf16_scales(bp, gemv_kernel):
     """N spans several workgroups and is not a multiple of their rows; two stacked terms; bf16 scales."""
     got, want, kern = _run(bp, "tq1", 2, 2048 + 48, 2304, [1, 1], "bf16", terms=2, seed=5, scale_dtype=np.float32)
-    assert kern.startswith("lut_tq1"), kern
+    assert kern.startswith(gemv_kernel), kern
     _check(got, want)
 
 
-def test_tq1_gemv_scales_from_global_memory(bp):
-    """Scale pointers that are not 16-byte aligned, and K with more groups than the LDS tile takes."""
+def test_tq1_gemv_scales_from_global_memory(bp, monkeypatch):
+    """Table kernel: scale pointers that are not 16-byte aligned, and K with more groups than the LDS tile takes."""
+    monkeypatch.setenv("BP_TUNE_TQ1", "lut")
     got, want, kern = _run(bp, "tq1", 2, 32, 2048, [1, 1], "bf16", seed=6, misalign_scales=True)
-    assert kern.endswith("_gs"), kern
+    assert kern.startswith("lut_tq1") and kern.endswith("_gs"), kern
     _check(got, want)
-    got, want, kern = _run(bp, "tq1", 1, 272, 40960, [1], "bf16", seed=7)  # G = 320: 256 rows x 640 B of scales do not fit
+    monkeypatch.delenv("BP_TUNE_TQ1")
+    got, want, kern = _run(bp, "tq1", 2, 32, 2048, [1, 1], "bf16", seed=6, misalign_scales=True)
+    assert kern.startswith("fp4_tq1"), kern
+    _check(got, want)
+    got, want, kern = _run(bp, "tq1", 1, 272, 40960, [1], "bf16", seed=7)  # 64 chunks: the operand tile does not fit in LDS
     assert kern.startswith("lut_tq1"), kern
     _check(got, want)
+    got, want, kern = _run(bp, "tq1", 1, 272, 16384, [1], "bf16", seed=8)  # 26 chunks: one workgroup of 16 waves per CU
+    assert kern == "fp4_tq1_t1_w16", kern
+    _check(got, want)
+
+
+@pytest.mark.parametrize("act", ["bf16", "f16"])
+def test_tq1_gemv_fp8_pieces_keep_small_activations(bp, act):
+    """The fp8 x fp4 kernel splits an activation into three E4M3 pieces under a per-group power-of-two prescale;
+    what it drops is below 2^-20 of the largest magnitude of the 128-wide group. Activations spread over 5 decades,
+    with outliers 1000 x the typical value, must still come out far inside the tolerance of the other paths."""
+    rng = np.random.default_rng(11)
+    E, N, K = 2, 64, 4352
+    packed, scales = synth_weights(11, E, N, K, GROUP, "tq1")
+    x = rng.standard_normal((E, K)).astype(np.float32) * np.exp(rng.uniform(-6, 6, (E, K))).astype(np.float32)
+    x[:, ::97] *= 1000.0
+    x = orc.bf16_round(x) if act == "bf16" else np.clip(x, -6e4, 6e4).astype(np.float16).astype(np.float32)
+    want = np.zeros((E, N), np.float32)
+    for e in range(E):
+        c_gemm(x[e:e + 1], None, packed[0][e], scales[0][e].astype(np.float32), K, GROUP, "tq1", out=want[e:e + 1])
+    xd = dev(x).to(torch.bfloat16) if act == "bf16" else dev(x).half()
+    got = bp.grouped_ternary_gemm(xd, None, [0, 1, 2], [dev(packed[0])], [dev(scales[0])], K, GROUP, "tq1").cpu().numpy()
+    assert bp.ext().last_kernel().startswith("fp4_tq1")
+    assert rel_l2(got, want) <= 1e-4, rel_l2(got, want)  # (measured 4e-5; the other paths are held to 1e-3)
+    z = np.zeros_like(x)  # all-zero activations: the prescale has nothing to go by
+    got = bp.grouped_ternary_gemm(dev(z).to(torch.bfloat16), None, [0, 1, 2], [dev(packed[0])], [dev(scales[0])], K, GROUP, "tq1")
+    assert torch.equal(got, torch.zeros_like(got))
 
 
 # --------------------------------------------------------------------------- TQ1 MFMA kernel (2..16 rows per tile)
@@ -195,7 +237,7 @@ def test_tq2_gemm_scales_from_global_memory_and_other_scale_dtypes(bp):
 
 # --------------------------------------------------------------------------- float32 scales (TQ1)
 @pytest.mark.parametrize("act", ["bf16", "int8"])
-@pytest.mark.parametrize("K,counts,prefix", [(2048, [1, 0, 1], "lut_tq1"), (7168, [1, 1, 1], "lut_tq1"), (2048, [3, 16, 1], "mfma_tq1"),
+@pytest.mark.parametrize("K,counts,prefix", [(2048, [1, 0, 1], "fp4_tq1"), (7168, [1, 1, 1], "fp4_tq1"), (2048, [3, 16, 1], "mfma_tq1"),
                                               (7168, [20, 2, 9], "mfma_tq1")])
 def test_tq1_float32_scales(bp, act, K, counts, prefix):
     """boilerplate/kernels/ternary_cuda.py:95-97 hands the kernel `w_scale.float()`: the tuned TQ1 kernels take it."""
@@ -259,7 +301,7 @@ def test_moe_layer_graph_replays_match_eager(bp, fmt, act, tokens):
 @pytest.mark.parametrize("act", ["bf16", "int8"])
 @pytest.mark.parametrize("fmt,K,counts,prefix", [
     ("tq2", 2048, [1, 0, 1], "mfma_tq2"), ("tq2", 7168, [16, 2, 5], "mfma_tq2"), ("tq2", 3072, [40, 1, 20], "gemm_tq2"),
-    ("tq1", 2048, [1, 1, 0], "lut_tq1"), ("tq1", 7168, [1, 0, 1], "lut_tq1"), ("tq1", 7168, [9, 16, 2], "mfma_tq1"),
+    ("tq1", 2048, [1, 1, 0], "fp4_tq1"), ("tq1", 7168, [1, 0, 1], "fp4_tq1"), ("tq1", 7168, [9, 16, 2], "mfma_tq1"),
     ("tq1", 2560, [3, 0, 20], "mfma_tq1"),
 ])
 def test_group_256(bp, act, fmt, K, counts, prefix):
