@@ -22,11 +22,14 @@
 //    Rows 4 g + p are the pieces of group g < 4 and rows 3, 7, 11 those of group 4, so a lane of the result (rows
 //    4 kb + i) holds the three pieces of group kb and one piece of group 4.
 //  * fp8 pieces: the activations of a 128-wide group are multiplied by a power of two that brings the group's
-//    largest magnitude into [128, 256), then y = p0 + p1 + p2 / 256 with p0 = y truncated to E4M3 (4 significant bits), p1 = the
-//    remainder truncated likewise, p2 = 256 x the second remainder, truncated. bf16 (8 significant bits) and
-//    int8 activations are represented exactly by p0 + p1 down to 2^-9 of the scaled range and to 2^-17 with p2,
-//    fp16 (11 bits) by the three; what is dropped is below 2^-20 of the group's largest magnitude. Products
-//    fp8 x fp4 are exact and accumulate in float32. float32 activations are left to the table kernel.
+//    largest magnitude into [128, 256), then y = p0 + p1 + p2 / 256 with p0 = y rounded to E4M3 (4 significant
+//    bits), p1 = the remainder rounded likewise, p2 = 256 x the second remainder, rounded (v_cvt_pk_fp8_f32: OCP
+//    E4M3, round to nearest even, and v_cvt_f32_fp8 back; checked on gfx950). bf16 (8 significant bits) and int8
+//    activations are exactly p0 + p1 down to 2^-10 of the group's largest magnitude, fp16 (11 bits) exactly the
+//    three; below that a value keeps 4 more bits through p2, and what is dropped is less than 2^-20 of the group's
+//    largest magnitude. Products fp8 x fp4 are exact and accumulate in float32. float32 activations (24 bits)
+//    are left to the table kernel. Activations that are not finite give results that are not meaningful here
+//    (the other kernels propagate NaN / Inf).
 //
 // Operand A is read from an LDS tile built once per workgroup. It is stored compactly: per chunk, per matrix
 // instruction j = 0..7 and per 16-byte half of an A lane's operand (= the 2 x 8 digit slots of two consecutive
@@ -64,10 +67,14 @@ constexpr int F4_PRE_OFF = F4_ZERO_OFF + 16;     // 8 words: the prescale of the
 constexpr int F4_INV_OFF = F4_PRE_OFF + 32;      // 8 floats: their inverses (the unused ones are 0)
 constexpr int F4_CHUNK_BYTES = F4_INV_OFF + 32;  // 3344
 constexpr int F4_LDS_MAX = 160 * 1024;
-constexpr int F4_GR = 2;                         // 16-row tiles per wave (they share the reads of operand A)
-constexpr int F4_RD = 2;                         // chunks of packed bytes in registers per tile (the ring of loads in flight)
-constexpr int F4_BD = 2;                         // table reads run this many (instruction, tile) pairs ahead of the matrix instructions
-constexpr int F4_AD = 1;                         // 1: operand A is read one instruction ahead into a second set of registers
+// Measured on E = 128, N = 2048, K = 7168: one 16-row tile per wave with 4 chunks in flight reads 504 MB from memory
+// per launch, two tiles with 2 chunks each 638 MB (405 MB are packed bytes and scales). Rows of 1434 bytes share
+// 128-byte lines between consecutive chunks; the sooner a wave returns to a row, the more of those lines it still
+// finds in the L2.
+constexpr int F4_GR = 1;                         // 16-row tiles per wave (more than one share the reads of operand A)
+constexpr int F4_RD = 4;                         // chunks of packed bytes in registers per tile (the ring of loads in flight)
+constexpr int F4_BD = 1;                         // table reads run this many (instruction, tile) pairs ahead of the matrix instructions
+constexpr int F4_AD = 0;                         // 1: operand A is read one instruction ahead into a second set of registers
 
 __device__ __forceinline__ u32x2 f4_load8(__amdgpu_buffer_rsrc_t r, unsigned lane_off, unsigned wave_off) {
   return __builtin_bit_cast(u32x2, __builtin_amdgcn_raw_buffer_load_b64(r, (int)lane_off, (int)wave_off, 0));
@@ -225,7 +232,7 @@ __global__ __launch_bounds__(WAVES * 64, 4) void k_tq1_gemv_fp4(GemmArgs a, int 
   const unsigned lane4 = (unsigned)(lane & 31) << 2;
   const unsigned next_lane4 = (unsigned)((lane + 16) & 63) << 2, last_lane4 = (unsigned)(48 + r16) << 2;
 
-  // The tables serve `bpw` blocks of WAVES x 32 rows, one after the other (the build is paid once per workgroup).
+  // The tables serve `bpw` blocks of WAVES x GR x 16 rows, one after the other (the build is paid once per workgroup).
   for (int pass = 0; pass < bpw; ++pass) {
   int64_t n0 = (((int64_t)blockIdx.x * bpw + pass) * WAVES + wave) * (16 * GR);
   const bool wave_live = n0 < a.N;
@@ -305,13 +312,14 @@ __global__ __launch_bounds__(WAVES * 64, 4) void k_tq1_gemv_fp4(GemmArgs a, int 
       };
       // software pipeline over the 16 (instruction, tile) pairs t = 2 j + s: table reads BD pairs ahead, operand A one
       // instruction ahead if AD; the scheduling barriers keep the compiler from sinking the reads back to their uses
+      constexpr int NT = 8 * GR;  // (instruction, tile) pairs of a chunk
       u32x4 Bq[BD + 1];
       u32x4 Alo[AD + 1], Ahi[AD + 1];
       auto lookup = [&](auto p_c) {  // table reads of pair p
-        constexpr int p = decltype(p_c)::value, j = p >> 1, s = p & 1;
+        constexpr int p = decltype(p_c)::value, j = p / GR, s = p % GR;
         if (j == 3)  // the dword after the first window: the first one of the next quarter's first window, or of the own second window
           w4[s] = (unsigned)__builtin_amdgcn_ds_bpermute((int)next_lane4, (int)(kb == 0 ? W[cur][s][1].x : W[cur][s][0].x));
-        if (p == 14) {
+        if (p == 7 * GR) {
           // The dword after the second window comes from the next quarter's second window, for the last quarter
           // from the next chunk. What the last instruction still needs of this chunk is set aside, the chunk's
           // registers are refilled (RD chunks on), and only then is the next chunk's first dword waited for: the
@@ -337,9 +345,10 @@ __global__ __launch_bounds__(WAVES * 64, 4) void k_tq1_gemv_fp4(GemmArgs a, int 
       a_read(0, Alo[0], Ahi[0]);
       lookup(IC<0>{});
       if (BD > 1) lookup(IC<BD - 1>{});
+      static_assert(BD <= 2 && GR <= 2 && RD <= 4, "the stage list below covers 16 pairs, the chunk loop 4 slots");
       auto stage = [&](auto t_c) {
-        constexpr int t = decltype(t_c)::value, j = t >> 1, s = t & 1;
-        if (t + BD < 16) lookup(IC<(t + BD < 16 ? t + BD : 0)>{});
+        constexpr int t = decltype(t_c)::value, j = t / GR, s = t % GR;
+        if (t + BD < NT) lookup(IC<(t + BD < NT ? t + BD : 0)>{});
         if (AD && s == 0 && j + 1 < 8) a_read(j + 1, Alo[(j + 1) & AD], Ahi[(j + 1) & AD]);
 
         __builtin_amdgcn_sched_barrier(0);
@@ -349,11 +358,13 @@ __global__ __launch_bounds__(WAVES * 64, 4) void k_tq1_gemv_fp4(GemmArgs a, int 
         const i32x8 B = {(int)bq.x, (int)bq.y, (int)bq.z, (int)bq.w, 0, 0, 0, 0};
         if (ABL == 4 || ABL == 7 || ABL == 8) asm volatile("; operands stay live" ::"v"(bq), "v"(alo), "v"(ahi));
         else C[s] = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(A, B, C[s], 0 /* A: E4M3 */, 4 /* B: E2M1 */, 0, 0, 0, 0);
-        if (!AD && s == 1 && j + 1 < 8) a_read(j + 1, Alo[0], Ahi[0]);  // both tiles have issued with this operand
+        if (!AD && s == GR - 1 && j + 1 < 8) a_read(j + 1, Alo[0], Ahi[0]);  // every tile has issued with this operand
         __builtin_amdgcn_sched_barrier(0);
       };
-      stage(IC<0>{}); stage(IC<1>{}); stage(IC<2>{}); stage(IC<3>{}); stage(IC<4>{}); stage(IC<5>{}); stage(IC<6>{}); stage(IC<7>{});
-      stage(IC<8>{}); stage(IC<9>{}); stage(IC<10>{}); stage(IC<11>{}); stage(IC<12>{}); stage(IC<13>{}); stage(IC<14>{}); stage(IC<15>{});
+#define BP_F4_STAGE(T) if (T < NT) stage(IC<(T < NT ? T : 0)>{})
+      BP_F4_STAGE(0); BP_F4_STAGE(1); BP_F4_STAGE(2); BP_F4_STAGE(3); BP_F4_STAGE(4); BP_F4_STAGE(5); BP_F4_STAGE(6); BP_F4_STAGE(7);
+      BP_F4_STAGE(8); BP_F4_STAGE(9); BP_F4_STAGE(10); BP_F4_STAGE(11); BP_F4_STAGE(12); BP_F4_STAGE(13); BP_F4_STAGE(14); BP_F4_STAGE(15);
+#undef BP_F4_STAGE
       // the chunk's 5 group sums under their scales: this lane holds group kb (3 pieces) and a piece of group 4, whose
       // scale sits next to that of group 3 in the lanes kb = 3
       const float inv_a = __uint_as_float(*(const lds_u32*)(cbase + F4_INV_OFF + 4 * kb));
@@ -398,9 +409,11 @@ __global__ __launch_bounds__(WAVES * 64, 4) void k_tq1_gemv_fp4(GemmArgs a, int 
       step(c0, IC<0>{});
       step(c0 + 1, IC<1 % RD>{});
       if (RD > 2) step(c0 + 2, IC<2 % RD>{});
+      if (RD > 3) step(c0 + 3, IC<3 % RD>{});
     }
     if (ABL != 1 && nchunks - full_end > 0) step(full_end, IC<0>{});  // uniform
     if (ABL != 1 && nchunks - full_end > 1) step(full_end + 1, IC<1 % RD>{});
+    if (ABL != 1 && nchunks - full_end > 2) step(full_end + 2, IC<2 % RD>{});
   }
   // ---- epilogue: the four quarter lanes of a row hold its partial sums
 #pragma unroll
@@ -415,6 +428,12 @@ __global__ __launch_bounds__(WAVES * 64, 4) void k_tq1_gemv_fp4(GemmArgs a, int 
   }
   }  // pass
 }
+int f4_cus() {  // compute units of the current device (256 if the query fails)
+  int dev = 0, cus = 0;
+  if (hipGetDevice(&dev) != hipSuccess || hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || cus < 1) cus = 256;
+  return cus;
+}
+
 template <int SDT, int WAVES, int ABL = 0>
 int launch_f4_k(const GemmArgs& a, hipStream_t s, const char* name, int nchunks, size_t lds) {
   static bool attr = false;
@@ -422,8 +441,7 @@ int launch_f4_k(const GemmArgs& a, hipStream_t s, const char* name, int nchunks,
   if (!attr) {
     const hipError_t rc = hipFuncSetAttribute((const void*)k_tq1_gemv_fp4<SDT, WAVES, ABL>, hipFuncAttributeMaxDynamicSharedMemorySize, F4_LDS_MAX);
     if (rc != hipSuccess) return fail(BP_ERR_LAUNCH, "cannot raise the dynamic LDS limit: %s", hipGetErrorString(rc));
-    int dev = 0;
-    if (hipGetDevice(&dev) != hipSuccess || hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || cus < 1) cus = 256;
+    cus = f4_cus();
     attr = true;
   }
   // Every workgroup builds the tables of its expert's token, so a workgroup takes as many row blocks as still leaves
@@ -456,7 +474,13 @@ int launch_f4(const GemmArgs& a, hipStream_t s) {
     if (SDT == BP_F16 && atoi(t) == 8) return launch_f4_k<BP_F16, 8, 8>(a, s, "abl8_fp4", (int)nchunks, lds);
   }
   // two workgroups of 8 waves per CU when their tiles fit side by side, else one of 16
-  if (lds <= (size_t)F4_LDS_MAX / 2) return launch_f4_k<SDT, 8>(a, s, "fp4_tq1_t1_w8", (int)nchunks, lds);
+  // Two workgroups of 8 waves per CU when their tiles fit side by side and the call is small; one of 16 waves when
+  // there are row blocks enough for every CU anyway (the tables are then built once per CU instead of twice).
+  static const int cus = f4_cus();
+  const int64_t experts = a.E < a.T ? a.E : a.T;
+  bool wide = lds > (size_t)F4_LDS_MAX / 2 || ((a.N + 255) / 256) * experts >= 4 * (int64_t)cus;
+  if (const char* tw = getenv("BP_TUNE_F4W")) wide = lds > (size_t)F4_LDS_MAX / 2 || atoi(tw) == 16;  // (development)
+  if (!wide) return launch_f4_k<SDT, 8>(a, s, "fp4_tq1_t1_w8", (int)nchunks, lds);
   return launch_f4_k<SDT, 16>(a, s, "fp4_tq1_t1_w16", (int)nchunks, lds);
 }
 
