@@ -74,6 +74,7 @@ constexpr int F4_LDS_MAX = 160 * 1024;
 constexpr int F4_GR = 1;                         // 16-row tiles per wave (more than one share the reads of operand A)
 constexpr int F4_RD = 4;                         // chunks of packed bytes in registers per tile (the ring of loads in flight)
 constexpr int F4_BD = 1;                         // table reads run this many (instruction, tile) pairs ahead of the matrix instructions
+constexpr int F4_PAIRS = 1;                      // 1: chunks are refilled two at a time (RD even)
 constexpr int F4_AD = 0;                         // 1: operand A is read one instruction ahead into a second set of registers
 
 __device__ __forceinline__ u32x2 f4_load8(__amdgpu_buffer_rsrc_t r, unsigned lane_off, unsigned wave_off) {
@@ -90,7 +91,8 @@ __device__ __forceinline__ int f4_pair_byte(int j, int kbA, int hf) {
 // 8 = 7 without the byte extraction (loads and their realignment only)
 template <int SDT, int WAVES, int ABL = 0>
 __global__ __launch_bounds__(WAVES * 64, 4) void k_tq1_gemv_fp4(GemmArgs a, int nchunks, int bpw /* row blocks per workgroup */) {
-  constexpr int THREADS = WAVES * 64, GR = F4_GR, RD = F4_RD, BD = F4_BD, AD = F4_AD;
+  constexpr int THREADS = WAVES * 64, GR = F4_GR, RD = F4_RD, BD = F4_BD, AD = F4_AD, PAIRS = F4_PAIRS;
+  static_assert(!PAIRS || RD % 2 == 0, "pairs of chunks need an even ring");
   constexpr int AT = F4_LUT_BYTES;           // the operand A tile starts after the table
   constexpr int SB = SDT == BP_F32 ? 4 : 2;  // bytes per scale
 
@@ -332,8 +334,18 @@ __global__ __launch_bounds__(WAVES * 64, 4) void k_tq1_gemv_fp4(GemmArgs a, int 
             asm volatile("v_mov_b32 %0, %1" : "=v"(last[q]) : "v"(W[cur][q][1].w));
             same[q] = (unsigned)__builtin_amdgcn_ds_bpermute((int)next_lane4, (int)W[cur][q][1].x);
           }
-          fetch_w(c + RD, cur, 0);  // both windows together: the two loads of a row's 128 bytes then meet in the L1
-          fetch_w(c + RD, cur, 1);
+          // Both windows together (the two loads of a row's 128 bytes then meet in the L1), and with PAIRS two
+          // chunks together, after the second one of a pair has been consumed: 256 consecutive bytes of a row per
+          // visit, so the 128-byte line that two chunks share is fetched once.
+          if (!PAIRS) {
+            fetch_w(c + RD, cur, 0);
+            fetch_w(c + RD, cur, 1);
+          } else if (cur & 1) {
+            fetch_w(c + RD - 1, cur - 1, 0);
+            fetch_w(c + RD - 1, cur - 1, 1);
+            fetch_w(c + RD, cur, 0);
+            fetch_w(c + RD, cur, 1);
+          }
 #pragma unroll
           for (int q = 0; q < GR; ++q) {
             const unsigned far = (unsigned)__builtin_amdgcn_ds_bpermute((int)next_lane4, (int)W[nxt][q][0].x);
