@@ -234,53 +234,67 @@ __global__ __launch_bounds__(WAVES * 64, 4) void k_tq1_gemv_fp4(GemmArgs a, int 
   const unsigned lane4 = (unsigned)(lane & 31) << 2;
   const unsigned next_lane4 = (unsigned)((lane + 16) & 63) << 2, last_lane4 = (unsigned)(48 + r16) << 2;
 
-  // The tables serve `bpw` blocks of WAVES x GR x 16 rows, one after the other (the build is paid once per workgroup).
-  for (int pass = 0; pass < bpw; ++pass) {
-  int64_t n0 = (((int64_t)blockIdx.x * bpw + pass) * WAVES + wave) * (16 * GR);
-  const bool wave_live = n0 < a.N;
-  if (!wave_live) n0 = 0;  // keeps addresses valid (the wave's results are not stored)
-  float total[GR];
-#pragma unroll
-  for (int s = 0; s < GR; ++s) total[s] = 0.f;
-
+  // The tables serve `bpw` blocks of WAVES x GR x 16 rows, one after the other (the build is paid once per workgroup),
+  // term by term: a term's blocks form one stream of chunks, and when the chunks of a row fill the ring a whole
+  // number of times the refills run on into the next block, so the loads do not drain between blocks.
+  const bool chain = nchunks % RD == 0;
+  auto block_row0 = [&](int pass) -> int64_t {  // first row of this wave's tile(s) in block `pass`; 0 (valid, not stored) past N
+    const int64_t r = (((int64_t)blockIdx.x * bpw + pass) * WAVES + wave) * (16 * GR);
+    return r < a.N ? r : 0;
+  };
   for (int term = 0; term < a.n_terms; ++term) {
-    // this wave's rows as a buffer that ends with the tensor; dword-aligned base, per-lane row offset
+    // the expert's rows as a buffer that ends with the tensor; dword-aligned base, per-lane row offset. A block
+    // starts a multiple of 16 rows = of 4 bytes further on, so the misalignment is the same for all blocks.
     const unsigned char* wbeg = a.packed[term];
-    const unsigned char* wave_rows = wbeg + (e * a.N + n0) * a.Kp;
-    const unsigned mis = (unsigned)((uintptr_t)wave_rows & 3);
-    const __amdgpu_buffer_rsrc_t wrs = make_rsrc(wave_rows - mis, (wbeg + a.E * a.N * a.Kp) - (wave_rows - mis));
+    const unsigned char* expert_rows = wbeg + e * a.N * a.Kp;
+    const unsigned mis = (unsigned)((uintptr_t)expert_rows & 3);
+    const __amdgpu_buffer_rsrc_t wrs = make_rsrc(expert_rows - mis, (wbeg + a.E * a.N * a.Kp) - (expert_rows - mis));
     const unsigned ro = mis + (unsigned)r16 * (unsigned)a.Kp;
     const unsigned dlt = ro & 3u;  // the lane's window starts dlt bytes before its bytes of the row
     const unsigned voff = (ro & ~3u) + 16u * kb;
-    unsigned tile_off[GR], tile_soff[GR];  // (scalar) a tile past N repeats tile 0 and is not stored
-#pragma unroll
-    for (int s = 0; s < GR; ++s) {
-      const bool live = n0 + 16 * s < a.N;
-      tile_off[s] = live ? 16u * s * (unsigned)a.Kp : 0u;
-      tile_soff[s] = live ? 16u * s * (unsigned)a.G * SB : 0u;  // a multiple of 4
-    }
     const unsigned char* sbeg = (const unsigned char*)a.w_scale[term];
-    const unsigned char* wave_scales = sbeg + (e * a.N + n0) * a.G * SB;
-    const unsigned smis = (unsigned)((uintptr_t)wave_scales & 3);
-    const __amdgpu_buffer_rsrc_t srs = make_rsrc(wave_scales - smis, (sbeg + a.E * a.N * a.G * SB) - (wave_scales - smis));
+    const unsigned char* expert_scales = sbeg + e * a.N * a.G * SB;
+    const unsigned smis = (unsigned)((uintptr_t)expert_scales & 3);
+    const __amdgpu_buffer_rsrc_t srs = make_rsrc(expert_scales - smis, (sbeg + a.E * a.N * a.G * SB) - (expert_scales - smis));
     const unsigned srow = smis + (unsigned)r16 * (unsigned)a.G * SB;
-
-    // RD chunks in registers per tile; the two 64-byte halves of a chunk are refilled separately, each as soon as its
-    // last byte has gone into a table read, so a load has between RD - 1 and RD - 1/2 chunk times to land.
     u32x4 W[RD][GR][2];
     u32x2 SQ[GR];  // the scales of one chunk: refilled for the next chunk as soon as they have been applied
+
+  for (int pass = 0; pass < bpw; ++pass) {
+    const int64_t n0 = block_row0(pass), n0_next = pass + 1 < bpw ? block_row0(pass + 1) : n0;
+    const bool wave_live = (((int64_t)blockIdx.x * bpw + pass) * WAVES + wave) * (16 * GR) < a.N;
+    float total[GR];
+#pragma unroll
+    for (int s = 0; s < GR; ++s) total[s] = 0.f;
+    // chunk c of this block, or (c >= nchunks, chained) chunk c - nchunks of the next one: row offset (scalar) and chunk
+    auto target = [&](int c, int64_t& row0, int& cc) {
+      const bool over = chain && c >= nchunks && pass + 1 < bpw;
+      row0 = over ? n0_next : n0;
+      cc = over ? c - nchunks : (c < nchunks ? c : nchunks - 1);
+    };
+
+    // RD chunks in registers per tile; a chunk's registers are refilled (RD chunks on) as soon as its last byte has
+    // gone into a table read.
     auto fetch_w = [&](int c, int slot, int h) {
-      const unsigned so = 128u * (c < nchunks ? c : nchunks - 1) + 64u * h;
+      int64_t row0;
+      int cc;
+      target(c, row0, cc);
 #pragma unroll
-      for (int s = 0; s < GR; ++s) W[slot][s][h] = buf_load16(wrs, voff, so + tile_off[s]);
+      for (int s = 0; s < GR; ++s) {
+        const int64_t row = row0 + 16 * s < a.N ? row0 + 16 * s : row0;  // a tile past N repeats tile 0 and is not stored
+        W[slot][s][h] = buf_load16(wrs, voff, (unsigned)(row * a.Kp) + 128u * cc + 64u * h);
+      }
     };
-    auto scale_at = [&](int c) -> unsigned {  // offset of the dword that holds the scale of group kb of chunk c
-      const unsigned idx = (unsigned)((5 * (c < nchunks ? c : nchunks - 1) + kb) >> gs);
-      return (srow + SB * idx) & ~3u;
-    };
-    auto fetch_s = [&](unsigned at) {  // 8 bytes from there
+    auto fetch_s = [&](int c) {  // 8 bytes from the dword that holds the scale of group kb of chunk c
+      int64_t row0;
+      int cc;
+      target(c, row0, cc);
+      const unsigned at = (srow + SB * (unsigned)((5 * cc + kb) >> gs)) & ~3u;
 #pragma unroll
-      for (int s = 0; s < GR; ++s) SQ[s] = f4_load8(srs, at, tile_soff[s]);
+      for (int s = 0; s < GR; ++s) {
+        const int64_t row = row0 + 16 * s < a.N ? row0 + 16 * s : row0;
+        SQ[s] = f4_load8(srs, at, (unsigned)(row * a.G * SB));
+      }
     };
     // (chunk slots and pipeline stages are compile-time constants: every register array below is indexed statically)
     auto step = [&](int c, auto cur_c) {
@@ -398,22 +412,22 @@ __global__ __launch_bounds__(WAVES * 64, 4) void k_tq1_gemv_fp4(GemmArgs a, int 
         const float s4 = SDT == BP_F32 ? __uint_as_float(r4) : SDT == BP_F16 ? f16_bits_to_f32((uint16_t)r4) : __uint_as_float(r4 << 16);
         total[s] += sa * inv_a * (C[s][0] + C[s][1] + C[s][2] * (1.f / 256.f)) + s4 * inv_4 * C[s][3];
       }
-      fetch_s(scale_at(c + 1));
+      fetch_s(c + 1);
     };
 
-    // The first loads, in the order of use and with the scales last: the waits at the head of the loop are counted
-    // along this path too, and here as there the 4 loads of the next chunk and the 2 of the scales are the ones
-    // in flight behind the chunk that is needed.
-    const unsigned first_scale = scale_at(0);
-    __builtin_amdgcn_sched_barrier(0);
+    // The first loads (of a term, or of every block if the blocks are not chained), in the order of use and with the
+    // scales last: the waits at the head of the loop are counted along this path too, and here as there the
+    // loads of later chunks and of the scales are the ones in flight behind the chunk that is needed.
+    if (pass == 0 || !chain) {
 #pragma unroll
-    for (int u = 0; u < RD; ++u) {
-      fetch_w(u, u, 0);
-      fetch_w(u, u, 1);
+      for (int u = 0; u < RD; ++u) {
+        fetch_w(u, u, 0);
+        fetch_w(u, u, 1);
+      }
+      __builtin_amdgcn_sched_barrier(0);
+      fetch_s(0);
+      __builtin_amdgcn_sched_barrier(0);
     }
-    __builtin_amdgcn_sched_barrier(0);
-    fetch_s(first_scale);
-    __builtin_amdgcn_sched_barrier(0);
     // RD chunks per iteration with no way around any of them: the compiler counts the loads in flight along every
     // path into the head of the loop, and a path on which fewer are in flight would make every iteration wait
     const int full_end = ABL == 1 ? 0 : nchunks - nchunks % RD;
@@ -426,8 +440,7 @@ __global__ __launch_bounds__(WAVES * 64, 4) void k_tq1_gemv_fp4(GemmArgs a, int 
     if (ABL != 1 && nchunks - full_end > 0) step(full_end, IC<0>{});  // uniform
     if (ABL != 1 && nchunks - full_end > 1) step(full_end + 1, IC<1 % RD>{});
     if (ABL != 1 && nchunks - full_end > 2) step(full_end + 2, IC<2 % RD>{});
-  }
-  // ---- epilogue: the four quarter lanes of a row hold its partial sums
+  // ---- the four quarter lanes of a row hold its partial sums (of this term: the output is added to)
 #pragma unroll
   for (int s = 0; s < GR; ++s) {
     float t = total[s];
@@ -439,6 +452,7 @@ __global__ __launch_bounds__(WAVES * 64, 4) void k_tq1_gemv_fp4(GemmArgs a, int 
     }
   }
   }  // pass
+  }  // term
 }
 int f4_cus() {  // compute units of the current device (256 if the query fails)
   int dev = 0, cus = 0;
