@@ -25,7 +25,7 @@
 //    largest magnitude into [128, 256), then y = p0 + p1 + p2 / 256 with p0 = y rounded to E4M3 (4 significant
 //    bits), p1 = the remainder rounded likewise, p2 = 256 x the second remainder, rounded (v_cvt_pk_fp8_f32: OCP
 //    E4M3, round to nearest even, and v_cvt_f32_fp8 back; checked on gfx950). bf16 (8 significant bits) and int8
-//    activations are exactly p0 + p1 down to 2^-10 of the group's largest magnitude, fp16 (11 bits) exactly the
+//    activations are exactly p0 + p1 down to 2^-9 of the group's largest magnitude, fp16 (11 bits) exactly the
 //    three; below that a value keeps 4 more bits through p2, and what is dropped is less than 2^-20 of the group's
 //    largest magnitude. Products fp8 x fp4 are exact and accumulate in float32. float32 activations (24 bits)
 //    are left to the table kernel. Activations that are not finite give results that are not meaningful here
