@@ -187,6 +187,10 @@ __global__ __launch_bounds__(GTHREADS, 2) void k_gemm_tq2(GemmArgs a) {
   }
   __syncthreads();
   int seq = 0;  // tiles consumed so far
+  // The whole loop nest is instantiated once per number of token sub-tiles and the choice made outside it: a branch
+  // inside would end in a merge of the two paths' registers, and a register that a load in flight is about to write
+  // can only be merged after waiting for that load - the weight ring would drain at the end of every tile.
+  auto all_terms = [&](auto mtn_c) {
   for (int term = 0; term < a.n_terms; ++term) {
     const int64_t rows_here = a.N - n0 < 16 * GR ? a.N - n0 : 16 * GR;
     const __amdgpu_buffer_rsrc_t wrs = make_rsrc(a.packed[term] + (e * a.N + n0) * a.Kp, rows_here * a.Kp);
@@ -336,8 +340,7 @@ __global__ __launch_bounds__(GTHREADS, 2) void k_gemm_tq2(GemmArgs a) {
         }
 
       };
-      if (two) run_steps(std::integral_constant<int, GT>{});
-      else run_steps(std::integral_constant<int, 1>{});
+      run_steps(mtn_c);
 
       if (staged) {
         if (more) {
@@ -353,6 +356,9 @@ __global__ __launch_bounds__(GTHREADS, 2) void k_gemm_tq2(GemmArgs a) {
       }
     }
   }
+  };
+  if (two) all_terms(std::integral_constant<int, GT>{});
+  else all_terms(std::integral_constant<int, 1>{});
 
   // ---- epilogue: lane holds tokens 4b + q of each token sub-tile, output row n0 + 16r + r16
 #pragma unroll

@@ -471,7 +471,7 @@ int launch_f4_k(const GemmArgs& a, hipStream_t s, const char* name, int nchunks,
     attr = true;
   }
   // Every workgroup builds the tables of its expert's token, so a workgroup takes as many row blocks as still leaves
-  // every CU its full set of resident workgroups (16 waves): one round of workgroups, one build each.
+  // every CU its full set of resident workgroups (16 waves): all workgroups resident at once, one build each.
   const int64_t rows_per_block = (int64_t)WAVES * 16 * F4_GR;
   const int64_t blocks = (a.N + rows_per_block - 1) / rows_per_block;  // per expert
   const int64_t resident = (int64_t)cus * (16 / WAVES);
