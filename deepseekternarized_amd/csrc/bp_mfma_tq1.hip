@@ -101,62 +101,78 @@ __global__ __launch_bounds__(WAVES * 64, 4) void k_mfma_tq1(GemmArgs a, int CPT 
   const bool x_i8 = a.x_dtype == BP_I8;  // uniform
   const uint16_t* xg = (const uint16_t*)a.x + tok0 * a.K;
   const signed char* xg8 = (const signed char*)a.x + tok0 * a.K;
+  // 16-bit activations are staged without waiting for a load right after issuing it (a wait would also drain the
+  // packed bytes in flight): stage_load only requests a slot's activations - 16 raw bytes into the slot's registers -
+  // and stage_store, a tile later, picks the slot's 5 values out of them, zeroes the digits of other groups and
+  // writes the slot. int8 activations and the last bytes of a row are finished at once.
   u32x4 xstage[XU];
+  struct Slot { int row, rem, lo, hi; int64_t k0; bool any, fast; };
+  auto slot_of = [&](int u, int chunk0) -> Slot {
+    Slot t;
+    t.row = u / tile_slots;
+    t.rem = u - t.row * tile_slots;
+    const int cl = t.rem / T1_SLOTS, sg = t.rem - cl * T1_SLOTS;
+    const int g = sg / 28, sl = sg - g * 28;                   // sl = 7 b + m: byte FB[g] + sl of the chunk
+    const int j = (g == 0 ? 0 : g == 1 ? 25 : g == 2 ? 51 : g == 3 ? 76 : 102) + sl;
+    t.k0 = 640 * (int64_t)(chunk0 + cl) + 5 * j;               // first activation of the byte
+    t.lo = 128 * g - 5 * j;                                    // digits lo <= d < hi belong to group g
+    t.hi = t.lo + 128;
+    if (a.K - t.k0 < t.hi) t.hi = (int)(a.K - t.k0);           // ... and lie inside K
+    t.any = t.hi > 0 && t.lo < 5;
+    t.fast = t.k0 + 8 <= a.K;
+    return t;
+  };
+  auto finish = [&](const unsigned (&h)[5], const Slot& t) -> u32x4 {  // 5 bf16 patterns -> the slot, other groups' digits zeroed
+    unsigned m[5];
+#pragma unroll
+    for (int d = 0; d < 5; ++d) m[d] = d >= t.lo && d < t.hi ? h[d] : 0u;
+    return u32x4{m[0] | (m[1] << 16), m[2] | (m[3] << 16), m[4], 0u};
+  };
   auto stage_load = [&](int chunk0) {  // global -> registers: the tile that starts at chunk `chunk0`
 #pragma unroll
     for (int i = 0; i < XU; ++i) {
       const int u = threadIdx.x + i * THREADS;
       u32x4 v = {0u, 0u, 0u, 0u};
       if (u < units) {
-        const int row = u / tile_slots, rem = u - row * tile_slots;
-        const int cl = rem / T1_SLOTS, sg = rem - cl * T1_SLOTS;
-        const int g = sg / 28, sl = sg - g * 28;                   // sl = 7 b + m: byte FB[g] + sl of the chunk
-        const int j = (g == 0 ? 0 : g == 1 ? 25 : g == 2 ? 51 : g == 3 ? 76 : 102) + sl;
-        const int64_t kc0 = 640 * (int64_t)(chunk0 + cl);
-        const int64_t k0 = kc0 + 5 * j;                            // first activation of the byte
-        int lo = 128 * g - 5 * j, hi = lo + 128;                   // digits lo <= d < hi belong to group g
-        if (a.K - k0 < hi) hi = (int)(a.K - k0);                   // ... and lie inside K
-        if (hi > 0 && lo < 5) {
+        const Slot t = slot_of(u, chunk0);
+        if (t.any && t.fast && !x_i8) {
+          v = ((const Packed16*)(xg + (int64_t)t.row * a.K + t.k0))->v;
+        } else if (t.any && t.fast) {  // int8: widened at once (deferring it as well was measured slower)
+          const u32x2 q = ((const Packed8*)(xg8 + (int64_t)t.row * a.K + t.k0))->v;
           unsigned h[5];
-          if (x_i8) {
-            const signed char* src = xg8 + (int64_t)row * a.K + k0;
-            int v8[5];
-            if (k0 + 8 <= a.K) {
-              const u32x2 q = ((const Packed8*)src)->v;
 #pragma unroll
-              for (int d = 0; d < 4; ++d) v8[d] = __builtin_amdgcn_sbfe((int)q.x, 8 * d, 8);
-              v8[4] = __builtin_amdgcn_sbfe((int)q.y, 0, 8);
-            } else {
+          for (int d = 0; d < 5; ++d) h[d] = __float_as_uint((float)(int)__builtin_amdgcn_sbfe(d < 4 ? q.x : q.y, 8 * (d & 3), 8)) >> 16;  // (the builtin returns unsigned) exact in bf16
+          v = finish(h, t);
+        } else if (t.any) {  // the last bytes of a row: element by element
+          unsigned h[5];
 #pragma unroll
-              for (int d = 0; d < 5; ++d) v8[d] = k0 + d < a.K ? (int)src[d] : 0;
-            }
-#pragma unroll
-            for (int d = 0; d < 5; ++d) h[d] = __float_as_uint((float)v8[d]) >> 16;  // exact in bf16
-          } else {
-            const uint16_t* src = xg + (int64_t)row * a.K + k0;
-            if (k0 + 8 <= a.K) {
-              const u32x4 q = ((const Packed16*)src)->v;
-              h[0] = q.x & 0xffffu; h[1] = q.x >> 16; h[2] = q.y & 0xffffu; h[3] = q.y >> 16; h[4] = q.z & 0xffffu;
-            } else {  // the last bytes of a row: element by element
-#pragma unroll
-              for (int d = 0; d < 5; ++d) h[d] = k0 + d < a.K ? src[d] : 0u;
-            }
+          for (int d = 0; d < 5; ++d) {
+            if (x_i8) h[d] = t.k0 + d < a.K ? __float_as_uint((float)(int)xg8[(int64_t)t.row * a.K + t.k0 + d]) >> 16 : 0u;  // exact in bf16
+            else h[d] = t.k0 + d < a.K ? (unsigned)xg[(int64_t)t.row * a.K + t.k0 + d] : 0u;
           }
-#pragma unroll
-          for (int d = 0; d < 5; ++d) h[d] = d >= lo && d < hi ? h[d] : 0u;
-          v = u32x4{h[0] | (h[1] << 16), h[2] | (h[3] << 16), h[4], 0u};
+          v = finish(h, t);
         }
       }
       xstage[i] = v;
     }
   };
-  auto stage_store = [&]() {
+  auto stage_store = [&](int chunk0) {  // registers -> LDS: the tile that starts at chunk `chunk0`, requested by stage_load(chunk0)
 #pragma unroll
     for (int i = 0; i < XU; ++i) {
       const int u = threadIdx.x + i * THREADS;
       if (u < units) {
-        const int row = u / tile_slots, rem = u - row * tile_slots;
-        *(lds_u32x4*)(XB0 + row * pitch + rem * 16) = xstage[i];
+        u32x4 v = xstage[i];
+        if (x_i8) {  // (uniform) finished at the load: only the slot's place is needed
+          const int row = u / tile_slots, rem = u - row * tile_slots;
+          *(lds_u32x4*)(XB0 + row * pitch + rem * 16) = v;
+        } else {
+          const Slot t = slot_of(u, chunk0);
+          if (t.any && t.fast) {
+            const unsigned h[5] = {v.x & 0xffffu, v.x >> 16, v.y & 0xffffu, v.y >> 16, v.z & 0xffffu};
+            v = finish(h, t);
+          }
+          *(lds_u32x4*)(XB0 + t.row * pitch + t.rem * 16) = v;
+        }
       }
     }
   };
@@ -222,7 +238,7 @@ __global__ __launch_bounds__(WAVES * 64, 4) void k_mfma_tq1(GemmArgs a, int CPT 
     }
     if (!MULTI && term == 0) {
       __syncthreads();  // (the table is built)
-      stage_store();
+      stage_store(0);
       __syncthreads();
     }
 
@@ -247,7 +263,7 @@ __global__ __launch_bounds__(WAVES * 64, 4) void k_mfma_tq1(GemmArgs a, int CPT 
       {
         if (MULTI && c == next_tile) {  // uniform for the workgroup
           __syncthreads();  // every wave is done reading the previous tile (and, first time, the table is built)
-          stage_store();
+          stage_store(c);
           __syncthreads();
           tile_c0 = c;
           next_tile += CPT;
