@@ -60,12 +60,11 @@ struct __attribute__((packed, aligned(2))) F4Packed16 { u32x4 v; };
 struct __attribute__((packed, aligned(2))) F4Packed4 { unsigned v; };
 
 constexpr int F4_LUT_BYTES = 256 * 128;          // byte -> 5 fp4 codes, one copy per bank
-constexpr int F4_LO_BYTES = 64 * 3 * 16;         // per chunk: 64 byte pairs x 3 pieces x 16 bytes
-constexpr int F4_HI_OFF = F4_LO_BYTES;           // then 4 group boundaries x 3 pieces x 16 bytes
-constexpr int F4_ZERO_OFF = F4_HI_OFF + 4 * 3 * 16;
-constexpr int F4_PRE_OFF = F4_ZERO_OFF + 16;     // 8 words: the prescale of the chunk's 5 groups (3 unused)
-constexpr int F4_INV_OFF = F4_PRE_OFF + 32;      // 8 floats: their inverses (the unused ones are 0)
-constexpr int F4_CHUNK_BYTES = F4_INV_OFF + 32;  // 3344
+// Operand A tile, per chunk: 64 byte pairs x PC pieces x 16 bytes, then 4 group boundaries x PC pieces x 16 bytes, a
+// block of zeros, 8 words = the prescales of the chunk's 5 groups (3 unused), 8 floats = their inverses (the unused
+// ones are 0): 3344 bytes with 3 pieces, 2256 with 2.
+constexpr int f4_pieces(int ntok) { return ntok == 1 ? 3 : 2; }
+constexpr int f4_chunk_bytes(int ntok) { return (64 + 4) * f4_pieces(ntok) * 16 + 16 + 32 + 32; }
 constexpr int F4_LDS_MAX = 160 * 1024;
 // Measured on E = 128, N = 2048, K = 7168: one 16-row tile per wave with 4 chunks in flight reads 504 MB from memory
 // per launch, two tiles with 2 chunks each 638 MB (405 MB are packed bytes and scales). Rows of 1434 bytes share
@@ -89,19 +88,31 @@ __device__ __forceinline__ int f4_pair_byte(int j, int kbA, int hf) {
 // ABL (development): timing ablations - 1 no chunk loop, 2 no table reads, 3 no operand A reads, 4 no matrix instructions, 5 no byte extraction (and the loads are not waited for),
 // 6 bytes extracted from registers that are not loaded (no loads at all), 7 = 2 + 3 + 4 (loads and byte extraction only),
 // 8 = 7 without the byte extraction (loads and their realignment only)
-template <int SDT, int WAVES, int ABL = 0>
+//
+// NTOK > 1: up to NTOK token rows per expert (small decode batches). Every token has its own operand A tile, matrix
+// instructions and accumulators; the packed bytes and the table reads are shared. To fit 4 tiles beside the table,
+// an activation is then split into TWO fp8 pieces (PC = 2: exact for bf16 / int8 values down to 2^-9 of their group's
+// largest magnitude, at most 2^-17 of it dropped below), rows 2 g + p of operand A; with 4 tokens the ring of loads
+// is two chunks (the matrix instructions and the operand reads, not the loads, are what a wave waits for).
+template <int SDT, int WAVES, int ABL = 0, int NTOK = 1>
 __global__ __launch_bounds__(WAVES * 64, 4) void k_tq1_gemv_fp4(GemmArgs a, int nchunks, int bpw /* row blocks per workgroup */) {
-  constexpr int THREADS = WAVES * 64, GR = F4_GR, RD = F4_RD, BD = F4_BD, AD = F4_AD, PAIRS = F4_PAIRS;
+  constexpr int THREADS = WAVES * 64, GR = F4_GR, RD = NTOK <= 2 ? F4_RD : 2, BD = F4_BD, AD = F4_AD, PAIRS = NTOK <= 2 ? F4_PAIRS : 0;
   static_assert(!PAIRS || RD % 2 == 0, "pairs of chunks need an even ring");
-  constexpr int AT = F4_LUT_BYTES;           // the operand A tile starts after the table
+  static_assert(NTOK == 1 || (GR == 1 && AD == 0), "several tokens: one tile per wave, one operand A buffer");
+  constexpr int PC = f4_pieces(NTOK);        // fp8 pieces per activation
+  constexpr int F4_HI_OFF = 64 * PC * 16, F4_ZERO_OFF = F4_HI_OFF + 4 * PC * 16, F4_PRE_OFF = F4_ZERO_OFF + 16;
+  constexpr int F4_INV_OFF = F4_PRE_OFF + 32, F4_CHUNK_BYTES = f4_chunk_bytes(NTOK);
+  constexpr int AT = F4_LUT_BYTES;           // the operand A tiles (one per token) start after the table
   constexpr int SB = SDT == BP_F32 ? 4 : 2;  // bytes per scale
 
   const int wave = __builtin_amdgcn_readfirstlane((int)(threadIdx.x >> 6)), lane = threadIdx.x & 63;
   const int r16 = lane & 15, kb = lane >> 4;
   const int64_t e = blockIdx.y;
   const int64_t o0 = clamp_i64(a.offsets[e], 0, a.T), o1 = clamp_i64(a.offsets[e + 1], 0, a.T);
-  if (o0 >= o1) return;  // uniform for the workgroup; only the expert's first token row is used (max_rows == 1)
+  if (o0 >= o1) return;  // uniform for the workgroup; the expert's first NTOK token rows are used (max_rows <= NTOK)
   const int64_t tok = o0;
+  const int ntok = o1 - o0 < NTOK ? (int)(o1 - o0) : NTOK;
+  const int tile_bytes = nchunks * F4_CHUNK_BYTES;  // one token's tile
   const int gs = a.group == 256 ? 1 : 0;  // scale groups of 256: two 128-wide work groups share a scale
   const bool x16 = a.x_dtype == BP_BF16 || a.x_dtype == BP_F16;
   auto widen16 = [&](unsigned h) { return a.x_dtype == BP_BF16 ? bf16_bits_to_f32((uint16_t)h) : f16_bits_to_f32((uint16_t)h); };
@@ -121,14 +132,20 @@ __global__ __launch_bounds__(WAVES * 64, 4) void k_tq1_gemv_fp4(GemmArgs a, int 
     }
     *(lds_u32*)(128 * threadIdx.x) = ent;
   }
-  for (int g = threadIdx.x; g < nchunks * 8; g += THREADS) *(lds_u32*)(AT + (g >> 3) * F4_CHUNK_BYTES + F4_PRE_OFF + 4 * (g & 7)) = 0u;
+  for (int g = threadIdx.x; g < ntok * nchunks * 8; g += THREADS) {
+    const int tt = g / (nchunks * 8), gc = g - tt * nchunks * 8;
+    *(lds_u32*)(AT + tt * tile_bytes + (gc >> 3) * F4_CHUNK_BYTES + F4_PRE_OFF + 4 * (gc & 7)) = 0u;
+  }
   __syncthreads();
   for (int idx = threadIdx.x; idx < 256 * 32; idx += THREADS) *(lds_u32*)(4 * idx) = *(const lds_u32*)(128 * (idx >> 5));
+  for (int tt = 0; tt < ntok; ++tt) {
+  const int64_t xrow = (tok + tt) * a.K;
+  const int TB = AT + tt * tile_bytes;
   if (a.x_dtype != BP_I8) {  // (int8 values fit as they are: prescale 1)
     for (int64_t k0 = 8 * (int64_t)threadIdx.x; k0 < a.K; k0 += 8 * THREADS) {  // 8 values of one group per thread
       unsigned m = 0;
       if (x16 && k0 + 8 <= a.K) {
-        const u32x4 q = ((const F4Packed16*)((const uint16_t*)a.x + tok * a.K + k0))->v;
+        const u32x4 q = ((const F4Packed16*)((const uint16_t*)a.x + xrow + k0))->v;
 #pragma unroll
         for (int i = 0; i < 4; ++i) {
           const unsigned lo = __float_as_uint(widen16(q[i] & 0xffffu)) & 0x7fffffffu, hi = __float_as_uint(widen16(q[i] >> 16)) & 0x7fffffffu;
@@ -137,18 +154,20 @@ __global__ __launch_bounds__(WAVES * 64, 4) void k_tq1_gemv_fp4(GemmArgs a, int 
         }
       } else {
         for (int i = 0; i < 8 && k0 + i < a.K; ++i) {
-          const unsigned v = __float_as_uint(load_act_f32(a.x, a.x_dtype, tok * a.K + k0 + i)) & 0x7fffffffu;
+          const unsigned v = __float_as_uint(load_act_f32(a.x, a.x_dtype, xrow + k0 + i)) & 0x7fffffffu;
           m = m > v ? m : v;
         }
       }
       const int gg = (int)(k0 >> 7);
-      __hip_atomic_fetch_max((lds_u32*)(AT + (gg / 5) * F4_CHUNK_BYTES + F4_PRE_OFF + 4 * (gg % 5)), m, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
+      __hip_atomic_fetch_max((lds_u32*)(TB + (gg / 5) * F4_CHUNK_BYTES + F4_PRE_OFF + 4 * (gg % 5)), m, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
     }
+  }
   }
   __syncthreads();
   // the maxima become prescales 2^sh (sh brings the group's largest magnitude into [128, 256)) and their inverses
-  for (int g = threadIdx.x; g < nchunks * 8; g += THREADS) {
-    const unsigned at = (unsigned)(AT + (g >> 3) * F4_CHUNK_BYTES + 4 * (g & 7));
+  for (int gt = threadIdx.x; gt < ntok * nchunks * 8; gt += THREADS) {
+    const int tt = gt / (nchunks * 8), g = gt - tt * nchunks * 8;
+    const unsigned at = (unsigned)(AT + tt * tile_bytes + (g >> 3) * F4_CHUNK_BYTES + 4 * (g & 7));
     const bool real = (g & 7) < 5 && 128 * (int64_t)(5 * (g >> 3) + (g & 7)) < a.K;
     int sh = 0;
     if (real && a.x_dtype != BP_I8) {
@@ -161,16 +180,18 @@ __global__ __launch_bounds__(WAVES * 64, 4) void k_tq1_gemv_fp4(GemmArgs a, int 
   __syncthreads();
 
   // ---- operand A tile: one item = the 10 activations behind a byte pair -> 3 pieces x (first-group block, second-group block)
-  for (int it = threadIdx.x; it < nchunks * 64; it += THREADS) {
+  for (int itt = threadIdx.x; itt < ntok * nchunks * 64; itt += THREADS) {
+    const int tt = itt / (nchunks * 64), it = itt - tt * nchunks * 64;
+    const int64_t xrow = (tok + tt) * a.K;
     const int c = it >> 6, blk = it & 63;
     const int tt0 = 5 * f4_pair_byte(blk >> 3, (blk >> 1) & 3, blk & 1), glo = tt0 >> 7, ghi = (tt0 + 9) >> 7;
-    const unsigned dst = (unsigned)(AT + c * F4_CHUNK_BYTES);
+    const unsigned dst = (unsigned)(AT + tt * tile_bytes + c * F4_CHUNK_BYTES);
     const float pre_lo = __uint_as_float(*(const lds_u32*)(dst + F4_PRE_OFF + 4 * glo));
     const float pre_hi = __uint_as_float(*(const lds_u32*)(dst + F4_PRE_OFF + 4 * ghi));
     const int64_t k0 = 640 * (int64_t)c + tt0;
     float y[10];
     if (x16 && k0 + 10 <= a.K) {  // 20 bytes at an even address
-      const uint16_t* src = (const uint16_t*)a.x + tok * a.K + k0;
+      const uint16_t* src = (const uint16_t*)a.x + xrow + k0;
       const u32x4 q = ((const F4Packed16*)src)->v;
       const unsigned q4 = ((const F4Packed4*)(src + 8))->v;
 #pragma unroll
@@ -179,18 +200,18 @@ __global__ __launch_bounds__(WAVES * 64, 4) void k_tq1_gemv_fp4(GemmArgs a, int 
       y[9] = widen16(q4 >> 16);
     } else {
 #pragma unroll
-      for (int t = 0; t < 10; ++t) y[t] = k0 + t < a.K ? load_act_f32(a.x, a.x_dtype, tok * a.K + k0 + t) : 0.f;
+      for (int t = 0; t < 10; ++t) y[t] = k0 + t < a.K ? load_act_f32(a.x, a.x_dtype, xrow + k0 + t) : 0.f;
     }
-    u32x4 lo[3] = {}, hi[3] = {};
+    u32x4 lo[PC] = {}, hi[PC] = {};
 #pragma unroll
     for (int t = 0; t < 10; t += 2) {  // two activations per conversion
       const bool in0 = ((tt0 + t) >> 7) == glo, in1 = ((tt0 + t + 1) >> 7) == glo;
       float r0 = y[t] * (in0 ? pre_lo : pre_hi), r1 = y[t + 1] * (in1 ? pre_lo : pre_hi);
       const int pos0 = 8 * (t / 5) + t % 5, pos1 = 8 * ((t + 1) / 5) + (t + 1) % 5;  // digit slots of the block
 #pragma unroll
-      for (int p = 0; p < 3; ++p) {
+      for (int p = 0; p < PC; ++p) {
         const int w = __builtin_amdgcn_cvt_pk_fp8_f32(p == 2 ? r0 * 256.f : r0, p == 2 ? r1 * 256.f : r1, 0, false);
-        if (p < 2) {
+        if (p + 1 < PC) {
           r0 -= __builtin_amdgcn_cvt_f32_fp8(w, 0);
           r1 -= __builtin_amdgcn_cvt_f32_fp8(w, 1);
         }
@@ -202,17 +223,19 @@ __global__ __launch_bounds__(WAVES * 64, 4) void k_tq1_gemv_fp4(GemmArgs a, int 
       }
     }
 #pragma unroll
-    for (int p = 0; p < 3; ++p) *(lds_u32x4*)(dst + 16 * (3 * blk + p)) = lo[p];
+    for (int p = 0; p < PC; ++p) *(lds_u32x4*)(dst + 16 * (PC * blk + p)) = lo[p];
     if (ghi != glo) {
 #pragma unroll
-      for (int p = 0; p < 3; ++p) *(lds_u32x4*)(dst + F4_HI_OFF + 16 * (3 * (ghi - 1) + p)) = hi[p];
+      for (int p = 0; p < PC; ++p) *(lds_u32x4*)(dst + F4_HI_OFF + 16 * (PC * (ghi - 1) + p)) = hi[p];
     }
     if (blk == 0) *(lds_u32x4*)(dst + F4_ZERO_OFF) = u32x4{0u, 0u, 0u, 0u};
   }
   __syncthreads();
 
   // ---- this lane as a row of operand A: rows 4 g + p = piece p of group g < 4; rows 3, 7, 11 = pieces of group 4; row 15 unused
-  const int am_g = (r16 & 3) < 3 ? r16 >> 2 : 4, am_p = (r16 & 3) < 3 ? r16 & 3 : r16 >> 2;
+  // (two pieces: rows 2 g + p, rows 10..15 unused)
+  const int am_g = PC == 2 ? r16 >> 1 : (r16 & 3) < 3 ? r16 >> 2 : 4, am_p = PC == 2 ? r16 & 1 : (r16 & 3) < 3 ? r16 & 3 : r16 >> 2;
+  const bool am_used = PC == 2 ? r16 < 10 : r16 < 15;
   unsigned aoff[4];  // 16-byte block (index within the chunk's part of the tile) of instruction j, half hf: byte 2 (j % 2) + hf of aoff[j / 2]
 #pragma unroll
   for (int j = 0; j < 8; ++j) {
@@ -222,8 +245,8 @@ __global__ __launch_bounds__(WAVES * 64, 4) void k_tq1_gemv_fp4(GemmArgs a, int 
       const int blk = j * 8 + kb * 2 + hf;
       const int tt0 = 5 * f4_pair_byte(j, kb, hf), glo = tt0 >> 7, ghi = (tt0 + 9) >> 7;
       unsigned o = F4_ZERO_OFF / 16;
-      if (r16 < 15 && am_g == glo) o = 3 * blk + am_p;
-      else if (r16 < 15 && am_g == ghi) o = F4_HI_OFF / 16 + 3 * (ghi - 1) + am_p;
+      if (am_used && am_g == glo) o = PC * blk + am_p;
+      else if (am_used && am_g == ghi) o = F4_HI_OFF / 16 + PC * (ghi - 1) + am_p;
       both |= o << (8 * hf);
     }
     if (j & 1) aoff[j >> 1] |= both << 16;
@@ -263,9 +286,9 @@ __global__ __launch_bounds__(WAVES * 64, 4) void k_tq1_gemv_fp4(GemmArgs a, int 
   for (int pass = 0; pass < bpw; ++pass) {
     const int64_t n0 = block_row0(pass), n0_next = pass + 1 < bpw ? block_row0(pass + 1) : n0;
     const bool wave_live = (((int64_t)blockIdx.x * bpw + pass) * WAVES + wave) * (16 * GR) < a.N;
-    float total[GR];
+    float total[NTOK > 1 ? NTOK : GR];  // per token, or (one token) per row tile
 #pragma unroll
-    for (int s = 0; s < GR; ++s) total[s] = 0.f;
+    for (int s = 0; s < (NTOK > 1 ? NTOK : GR); ++s) total[s] = 0.f;
     // chunk c of this block, or (c >= nchunks, chained) chunk c - nchunks of the next one: row offset (scalar) and chunk
     auto target = [&](int c, int64_t& row0, int& cc) {
       const bool over = chain && c >= nchunks && pass + 1 < bpw;
@@ -289,7 +312,7 @@ __global__ __launch_bounds__(WAVES * 64, 4) void k_tq1_gemv_fp4(GemmArgs a, int 
       int64_t row0;
       int cc;
       target(c, row0, cc);
-      const unsigned at = (srow + SB * (unsigned)((5 * cc + kb) >> gs)) & ~3u;
+      const unsigned at = (srow + SB * (unsigned)((5 * cc + (PC == 3 ? kb : 2 * kb)) >> gs)) & ~3u;
 #pragma unroll
       for (int s = 0; s < GR; ++s) {
         const int64_t row = row0 + 16 * s < a.N ? row0 + 16 * s : row0;
@@ -299,9 +322,10 @@ __global__ __launch_bounds__(WAVES * 64, 4) void k_tq1_gemv_fp4(GemmArgs a, int 
     // (chunk slots and pipeline stages are compile-time constants: every register array below is indexed statically)
     auto step = [&](int c, auto cur_c) {
       constexpr int cur = decltype(cur_c)::value, nxt = (cur + 1) % RD;
-      f32x4 C[GR];
+      constexpr int NC = NTOK > 1 ? NTOK : GR;  // accumulator tiles: one per token, or (one token) one per row tile
+      f32x4 C[NC];
 #pragma unroll
-      for (int s = 0; s < GR; ++s) C[s] = f32x4{0.f, 0.f, 0.f, 0.f};
+      for (int s = 0; s < NC; ++s) C[s] = f32x4{0.f, 0.f, 0.f, 0.f};
       const unsigned cbase = (unsigned)(AT + c * F4_CHUNK_BYTES);
       // packed bytes of (instruction j, tile s) = dword j % 4 of the lane's window j / 4, shifted to the row's alignment;
       // the dword after a window is the first one of the next quarter's window (for the last quarter: of the first
@@ -321,10 +345,15 @@ __global__ __launch_bounds__(WAVES * 64, 4) void k_tq1_gemv_fp4(GemmArgs a, int 
           B[w] = ABL == 2 || ABL == 7 || ABL == 8 ? at : *(const lds_u32*)at;
         }
       };
-      auto a_read = [&](int j, u32x4& lo, u32x4& hi) {
+      auto a_read = [&](int j, u32x4& lo, u32x4& hi, int tt = 0) {
         if (ABL == 3 || ABL == 7 || ABL == 8) { lo = u32x4{cbase, dlt, lane4, cbase}; hi = lo; return; }
-        lo = *(const lds_u32x4*)((((aoff[j >> 1] >> (16 * (j & 1))) & 0xffu) << 4) + cbase);
-        hi = *(const lds_u32x4*)((((aoff[j >> 1] >> (16 * (j & 1) + 8)) & 0xffu) << 4) + cbase);
+        const unsigned tbase = cbase + (unsigned)(tt * tile_bytes);
+        unsigned ao = aoff[j >> 1];
+        // (several tokens: the block offsets are extracted anew at every use; hoisted out of the chunk loop, the
+        // 16 NTOK addresses of a lane would not fit its registers)
+        if (NTOK > 1) asm volatile("; packed block offsets" : "+v"(ao));
+        lo = *(const lds_u32x4*)((((ao >> (16 * (j & 1))) & 0xffu) << 4) + tbase);
+        hi = *(const lds_u32x4*)((((ao >> (16 * (j & 1) + 8)) & 0xffu) << 4) + tbase);
       };
       // software pipeline over the 16 (instruction, tile) pairs t = 2 j + s: table reads BD pairs ahead, operand A one
       // instruction ahead if AD; the scheduling barriers keep the compiler from sinking the reads back to their uses
@@ -368,7 +397,7 @@ __global__ __launch_bounds__(WAVES * 64, 4) void k_tq1_gemv_fp4(GemmArgs a, int 
         }
         table(bytes_of(j, s), Bq[p % (BD + 1)]);
       };
-      a_read(0, Alo[0], Ahi[0]);
+      if (NTOK == 1) a_read(0, Alo[0], Ahi[0]);
       lookup(IC<0>{});
       if (BD > 1) lookup(IC<BD - 1>{});
       static_assert(BD <= 2 && GR <= 2 && RD <= 4, "the stage list below covers 16 pairs, the chunk loop 4 slots");
@@ -377,11 +406,26 @@ __global__ __launch_bounds__(WAVES * 64, 4) void k_tq1_gemv_fp4(GemmArgs a, int 
         if (t + BD < NT) lookup(IC<(t + BD < NT ? t + BD : 0)>{});
         if (AD && s == 0 && j + 1 < 8) a_read(j + 1, Alo[(j + 1) & AD], Ahi[(j + 1) & AD]);
 
+        const u32x4 bq = Bq[t % (BD + 1)];
+        const i32x8 B = {(int)bq.x, (int)bq.y, (int)bq.z, (int)bq.w, 0, 0, 0, 0};
+        if (NTOK > 1) {
+          // The same packed bytes against every token's operand A, one token at a time (the scheduling barriers keep
+          // the compiler from reading all the operands first: 8 registers each). Tiles of tokens the expert does not
+          // have hold whatever LDS held; their accumulators are not used.
+#pragma unroll
+          for (int tt = 0; tt < NTOK; ++tt) {
+            __builtin_amdgcn_sched_barrier(0);
+            a_read(j, Alo[0], Ahi[0], tt);
+            const u32x4 alo = Alo[0], ahi = Ahi[0];
+            const i32x8 A = {(int)alo.x, (int)alo.y, (int)alo.z, (int)alo.w, (int)ahi.x, (int)ahi.y, (int)ahi.z, (int)ahi.w};
+            C[tt] = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(A, B, C[tt], 0 /* A: E4M3 */, 4 /* B: E2M1 */, 0, 0, 0, 0);
+          }
+          __builtin_amdgcn_sched_barrier(0);
+          return;
+        }
         __builtin_amdgcn_sched_barrier(0);
         const u32x4 alo = Alo[j & AD], ahi = Ahi[j & AD];
         const i32x8 A = {(int)alo.x, (int)alo.y, (int)alo.z, (int)alo.w, (int)ahi.x, (int)ahi.y, (int)ahi.z, (int)ahi.w};
-        const u32x4 bq = Bq[t % (BD + 1)];
-        const i32x8 B = {(int)bq.x, (int)bq.y, (int)bq.z, (int)bq.w, 0, 0, 0, 0};
         if (ABL == 4 || ABL == 7 || ABL == 8) asm volatile("; operands stay live" ::"v"(bq), "v"(alo), "v"(ahi));
         else C[s] = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(A, B, C[s], 0 /* A: E4M3 */, 4 /* B: E2M1 */, 0, 0, 0, 0);
         if (!AD && s == GR - 1 && j + 1 < 8) a_read(j + 1, Alo[0], Ahi[0]);  // every tile has issued with this operand
@@ -391,14 +435,13 @@ __global__ __launch_bounds__(WAVES * 64, 4) void k_tq1_gemv_fp4(GemmArgs a, int 
       BP_F4_STAGE(0); BP_F4_STAGE(1); BP_F4_STAGE(2); BP_F4_STAGE(3); BP_F4_STAGE(4); BP_F4_STAGE(5); BP_F4_STAGE(6); BP_F4_STAGE(7);
       BP_F4_STAGE(8); BP_F4_STAGE(9); BP_F4_STAGE(10); BP_F4_STAGE(11); BP_F4_STAGE(12); BP_F4_STAGE(13); BP_F4_STAGE(14); BP_F4_STAGE(15);
 #undef BP_F4_STAGE
-      // the chunk's 5 group sums under their scales: this lane holds group kb (3 pieces) and a piece of group 4, whose
-      // scale sits next to that of group 3 in the lanes kb = 3
-      const float inv_a = __uint_as_float(*(const lds_u32*)(cbase + F4_INV_OFF + 4 * kb));
-      const float inv_4 = __uint_as_float(*(const lds_u32*)(cbase + F4_INV_OFF + 16)) * f4th;
-      const unsigned ia = (unsigned)((5 * c + kb) >> gs), ib = (unsigned)((5 * c + kb + 1) >> gs);
+      // the chunk's 5 group sums under their scales. Three pieces: this lane holds group kb (3 pieces) and a piece of
+      // group 4, whose scale sits next to that of group 3 in the lanes kb = 3. Two pieces: groups 2 kb and 2 kb + 1.
+      const int g_first = PC == 3 ? kb : 2 * kb;
+      const unsigned ia = (unsigned)((5 * c + g_first) >> gs), ib = (unsigned)((5 * c + g_first + 1) >> gs);
 #pragma unroll
       for (int s = 0; s < GR; ++s) {
-        unsigned ra, rb;  // the scale of group kb, and the one after it (bits as stored)
+        unsigned ra, rb;  // the scale of group g_first, and the one after it (bits as stored)
         if (SDT == BP_F32) {
           ra = SQ[s].x;
           rb = ib == ia ? ra : SQ[s].y;
@@ -407,10 +450,22 @@ __global__ __launch_bounds__(WAVES * 64, 4) void k_tq1_gemv_fp4(GemmArgs a, int 
           ra = v & 0xffffu;
           rb = ib == ia ? ra : v >> 16;
         }
-        const unsigned r4 = (unsigned)__builtin_amdgcn_ds_bpermute((int)last_lane4, (int)rb);
         const float sa = SDT == BP_F32 ? __uint_as_float(ra) : SDT == BP_F16 ? f16_bits_to_f32((uint16_t)ra) : __uint_as_float(ra << 16);
-        const float s4 = SDT == BP_F32 ? __uint_as_float(r4) : SDT == BP_F16 ? f16_bits_to_f32((uint16_t)r4) : __uint_as_float(r4 << 16);
-        total[s] += sa * inv_a * (C[s][0] + C[s][1] + C[s][2] * (1.f / 256.f)) + s4 * inv_4 * C[s][3];
+        if (PC == 3) {
+          const float inv_a = __uint_as_float(*(const lds_u32*)(cbase + F4_INV_OFF + 4 * kb));
+          const float inv_4 = __uint_as_float(*(const lds_u32*)(cbase + F4_INV_OFF + 16)) * f4th;
+          const unsigned r4 = (unsigned)__builtin_amdgcn_ds_bpermute((int)last_lane4, (int)rb);
+          const float s4 = SDT == BP_F32 ? __uint_as_float(r4) : SDT == BP_F16 ? f16_bits_to_f32((uint16_t)r4) : __uint_as_float(r4 << 16);
+          total[s] += sa * inv_a * (C[s][0] + C[s][1] + C[s][2] * (1.f / 256.f)) + s4 * inv_4 * C[s][3];
+        } else {  // (one row tile per wave: s == 0)
+          const float sb = SDT == BP_F32 ? __uint_as_float(rb) : SDT == BP_F16 ? f16_bits_to_f32((uint16_t)rb) : __uint_as_float(rb << 16);
+#pragma unroll
+          for (int tt = 0; tt < NTOK; ++tt) {  // (the inverses of groups past the chunk's five are 0)
+            const unsigned ivb = cbase + (unsigned)(tt * tile_bytes) + F4_INV_OFF + 8 * kb;
+            const float inv_a = __uint_as_float(*(const lds_u32*)ivb), inv_b = __uint_as_float(*(const lds_u32*)(ivb + 4));
+            total[tt] += sa * inv_a * (C[tt][0] + C[tt][1]) + sb * inv_b * (C[tt][2] + C[tt][3]);
+          }
+        }
       }
       fetch_s(c + 1);
     };
@@ -442,13 +497,14 @@ __global__ __launch_bounds__(WAVES * 64, 4) void k_tq1_gemv_fp4(GemmArgs a, int 
     if (ABL != 1 && nchunks - full_end > 2) step(full_end + 2, IC<2 % RD>{});
   // ---- the four quarter lanes of a row hold its partial sums (of this term: the output is added to)
 #pragma unroll
-  for (int s = 0; s < GR; ++s) {
+  for (int s = 0; s < (NTOK > 1 ? NTOK : GR); ++s) {
     float t = total[s];
     t += __shfl_xor(t, 16);
     t += __shfl_xor(t, 32);
-    if (kb == 0 && wave_live && n0 + 16 * s < a.N) {
-      float* o = a.out + tok * a.N + n0 + 16 * s + r16;
-      *o += a.x_dtype == BP_I8 ? t * a.x_scale[tok] : t;
+    const int tile = NTOK > 1 ? 0 : s, tt = NTOK > 1 ? s : 0;
+    if (kb == 0 && wave_live && n0 + 16 * tile < a.N && tt < ntok) {
+      float* o = a.out + (tok + tt) * a.N + n0 + 16 * tile + r16;
+      *o += a.x_dtype == BP_I8 ? t * a.x_scale[tok + tt] : t;
     }
   }
   }  // pass
@@ -460,12 +516,12 @@ int f4_cus() {  // compute units of the current device (256 if the query fails)
   return cus;
 }
 
-template <int SDT, int WAVES, int ABL = 0>
+template <int SDT, int WAVES, int ABL = 0, int NTOK = 1>
 int launch_f4_k(const GemmArgs& a, hipStream_t s, const char* name, int nchunks, size_t lds) {
   static bool attr = false;
   static int cus = 0;
   if (!attr) {
-    const hipError_t rc = hipFuncSetAttribute((const void*)k_tq1_gemv_fp4<SDT, WAVES, ABL>, hipFuncAttributeMaxDynamicSharedMemorySize, F4_LDS_MAX);
+    const hipError_t rc = hipFuncSetAttribute((const void*)k_tq1_gemv_fp4<SDT, WAVES, ABL, NTOK>, hipFuncAttributeMaxDynamicSharedMemorySize, F4_LDS_MAX);
     if (rc != hipSuccess) return fail(BP_ERR_LAUNCH, "cannot raise the dynamic LDS limit: %s", hipGetErrorString(rc));
     cus = f4_cus();
     attr = true;
@@ -480,16 +536,23 @@ int launch_f4_k(const GemmArgs& a, hipStream_t s, const char* name, int nchunks,
   bpw = bpw < 1 ? 1 : bpw > blocks ? blocks : bpw;
   const dim3 grid((unsigned)((blocks + bpw - 1) / bpw), (unsigned)a.E, 1u);
   note_kernel(name);
-  hipLaunchKernelGGL((k_tq1_gemv_fp4<SDT, WAVES, ABL>), grid, dim3(WAVES * 64), lds, s, a, nchunks, (int)bpw);
+  hipLaunchKernelGGL((k_tq1_gemv_fp4<SDT, WAVES, ABL, NTOK>), grid, dim3(WAVES * 64), lds, s, a, nchunks, (int)bpw);
   return check_launch(name);
 }
 
-template <int SDT>
+template <int SDT, int NTOK>
 int launch_f4(const GemmArgs& a, hipStream_t s) {
   const int64_t nchunks = (a.K + 639) / 640;
-  const size_t lds = (size_t)(F4_LUT_BYTES + nchunks * F4_CHUNK_BYTES);
+  const size_t lds = (size_t)(F4_LUT_BYTES + NTOK * nchunks * f4_chunk_bytes(NTOK));
   if (lds > (size_t)F4_LDS_MAX) return BP_ERR_UNSUPPORTED;
-  if (const char* t = getenv("BP_TUNE_F4ABL")) {  // development: timing ablations
+  static const int cus = f4_cus();
+  const int64_t experts = a.E < a.T ? a.E : a.T;
+  if (NTOK > 1) {
+    const bool wide = lds > (size_t)F4_LDS_MAX / 2 || ((a.N + 255) / 256) * experts >= 4 * (int64_t)cus;
+    if (!wide) return launch_f4_k<SDT, 8, 0, NTOK>(a, s, NTOK == 2 ? "fp4_tq1_m2_w8" : "fp4_tq1_m4_w8", (int)nchunks, lds);
+    return launch_f4_k<SDT, 16, 0, NTOK>(a, s, NTOK == 2 ? "fp4_tq1_m2_w16" : "fp4_tq1_m4_w16", (int)nchunks, lds);
+  }
+  if (const char* t = getenv("BP_TUNE_F4ABL")) {  // development: timing ablations (one token)
     if (SDT == BP_F16 && atoi(t) == 1) return launch_f4_k<BP_F16, 8, 1>(a, s, "abl1_fp4", (int)nchunks, lds);
     if (SDT == BP_F16 && atoi(t) == 2) return launch_f4_k<BP_F16, 8, 2>(a, s, "abl2_fp4", (int)nchunks, lds);
     if (SDT == BP_F16 && atoi(t) == 3) return launch_f4_k<BP_F16, 8, 3>(a, s, "abl3_fp4", (int)nchunks, lds);
@@ -499,11 +562,8 @@ int launch_f4(const GemmArgs& a, hipStream_t s) {
     if (SDT == BP_F16 && atoi(t) == 7) return launch_f4_k<BP_F16, 8, 7>(a, s, "abl7_fp4", (int)nchunks, lds);
     if (SDT == BP_F16 && atoi(t) == 8) return launch_f4_k<BP_F16, 8, 8>(a, s, "abl8_fp4", (int)nchunks, lds);
   }
-  // two workgroups of 8 waves per CU when their tiles fit side by side, else one of 16
   // Two workgroups of 8 waves per CU when their tiles fit side by side and the call is small; one of 16 waves when
   // there are row blocks enough for every CU anyway (the tables are then built once per CU instead of twice).
-  static const int cus = f4_cus();
-  const int64_t experts = a.E < a.T ? a.E : a.T;
   bool wide = lds > (size_t)F4_LDS_MAX / 2 || ((a.N + 255) / 256) * experts >= 4 * (int64_t)cus;
   if (const char* tw = getenv("BP_TUNE_F4W")) wide = lds > (size_t)F4_LDS_MAX / 2 || atoi(tw) == 16;  // (development)
   if (!wide) return launch_f4_k<SDT, 8>(a, s, "fp4_tq1_t1_w8", (int)nchunks, lds);
@@ -512,15 +572,28 @@ int launch_f4(const GemmArgs& a, hipStream_t s) {
 
 }  // namespace
 
-// max_rows == 1 (checked by the caller). BP_ERR_UNSUPPORTED (no message): the caller falls back to the table kernel.
+// max_rows <= 4 (checked by the caller): one token row per expert, or 2 / up to 4 (two fp8 pieces per activation).
+// BP_ERR_UNSUPPORTED (no message): the caller falls back to its other kernels.
 int launch_tq1_gemv_fp4(const GemmArgs& a, hipStream_t s) {
   if (a.x_dtype != BP_BF16 && a.x_dtype != BP_F16 && a.x_dtype != BP_I8) return BP_ERR_UNSUPPORTED;
+  if (a.max_rows > 1 && a.x_dtype == BP_F16) return BP_ERR_UNSUPPORTED;  // (11 significant bits need the third piece)
+  if (a.max_rows < 1 || a.max_rows > 4) return BP_ERR_UNSUPPORTED;
   if (a.N % 16 != 0 || a.Kp != (a.K + 4) / 5 || (a.group != 128 && a.group != 256)) return BP_ERR_UNSUPPORTED;
   for (int t = 0; t < a.n_terms; ++t)
     if (a.scale_dtype == BP_F32 && ((uintptr_t)a.w_scale[t] & 3) != 0) return BP_ERR_UNSUPPORTED;
-  if (a.scale_dtype == BP_F16) return launch_f4<BP_F16>(a, s);
-  if (a.scale_dtype == BP_BF16) return launch_f4<BP_BF16>(a, s);
-  if (a.scale_dtype == BP_F32) return launch_f4<BP_F32>(a, s);
+  if (a.max_rows == 1) {
+    if (a.scale_dtype == BP_F16) return launch_f4<BP_F16, 1>(a, s);
+    if (a.scale_dtype == BP_BF16) return launch_f4<BP_BF16, 1>(a, s);
+    if (a.scale_dtype == BP_F32) return launch_f4<BP_F32, 1>(a, s);
+  } else if (a.max_rows == 2) {
+    if (a.scale_dtype == BP_F16) return launch_f4<BP_F16, 2>(a, s);
+    if (a.scale_dtype == BP_BF16) return launch_f4<BP_BF16, 2>(a, s);
+    if (a.scale_dtype == BP_F32) return launch_f4<BP_F32, 2>(a, s);
+  } else {
+    if (a.scale_dtype == BP_F16) return launch_f4<BP_F16, 4>(a, s);
+    if (a.scale_dtype == BP_BF16) return launch_f4<BP_BF16, 4>(a, s);
+    if (a.scale_dtype == BP_F32) return launch_f4<BP_F32, 4>(a, s);
+  }
   return BP_ERR_UNSUPPORTED;
 }
 

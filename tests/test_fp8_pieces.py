@@ -78,6 +78,26 @@ def test_three_pieces_reconstruct_a_group(kind):
             assert np.array_equal((p0 + p1 + p2 / 256.0)[big], y[big])
 
 
+@pytest.mark.parametrize("kind", ["bf16", "int8"])
+def test_two_pieces_for_small_batches(kind):
+    """The small-batch variant keeps two pieces (bf16 / int8 activations only): exact down to 2^-9 of the group's largest
+    magnitude, and what is dropped below that is at most 2^-17 of it."""
+    rng = np.random.default_rng(5)
+    for trial in range(200):
+        x = rng.standard_normal(128) * np.exp(rng.uniform(-8, 8, 128))
+        if kind == "bf16":
+            x = (x.astype(np.float32).view(np.uint32) & 0xFFFF0000).view(np.float32).astype(np.float64)
+            y, _ = _prescaled(x)
+        else:
+            y = np.clip(np.rint(x * 20), -127, 127)
+        amax = max(np.abs(y).max(), 128.0)
+        p0, p1, _ = split3(y)
+        err = np.abs(y - (p0 + p1))
+        assert err.max() <= 2.0 ** -17 * amax, (kind, trial, err.max())
+        big = np.abs(y) >= 2.0 ** -9 * amax
+        assert np.array_equal((p0 + p1)[big], y[big])
+
+
 def test_pieces_stay_in_range():
     """No piece can overflow E4M3 (the conversion does not saturate: 500 became NaN on the hardware)."""
     y = np.concatenate([np.linspace(-255.99, 255.99, 100001), [255.9999, -255.9999, 2.0 ** -9, 2.0 ** -10]])

@@ -173,8 +173,40 @@ def test_tq1_mfma_tiles(bp, K, counts, act):
     _check(got, want)
 
 
-def test_tq1_mfma_scales_from_global_memory(bp):
+@pytest.mark.parametrize("act", ["bf16", "int8"])
+@pytest.mark.parametrize("K", [1024, 2048, 7168])
+@pytest.mark.parametrize("counts", [[2, 0, 1], [2, 2, 2], [4, 3, 1], [3, 0, 0]])
+def test_tq1_fp4_small_batches(bp, K, counts, act):
+    """2 and up to 4 token rows per expert: one operand tile per token (two fp8 pieces), the packed bytes read once."""
+    got, want, kern = _run(bp, "tq1", 3, 80, K, counts, act, terms=2, seed=K + 7 * sum(counts))
+    assert kern.startswith("fp4_tq1_m2" if max(counts) <= 2 else "fp4_tq1_m4"), kern
+    _check(got, want)
+
+
+def test_tq1_small_batches_other_kernels(bp, monkeypatch):
+    """fp16 activations (11 significant bits: more than two fp8 pieces hold) and rows of K whose 4 tiles x 26 chunks
+    do not fit beside the table go to the kernels they went to before; the development switch keeps the multi-row
+    MFMA kernel."""
+    got, want, kern = _run(bp, "tq1", 3, 80, 2048, [2, 4, 1], "f16", seed=21)
+    assert not kern.startswith("fp4_tq1"), kern
+    _check(got, want)
+    got, want, kern = _run(bp, "tq1", 2, 32, 16384, [4, 2], "bf16", seed=22)
+    assert not kern.startswith("fp4_tq1"), kern
+    _check(got, want)
+    monkeypatch.setenv("BP_TUNE_TQ1", "mfma")
+    got, want, kern = _run(bp, "tq1", 3, 80, 2048, [2, 4, 1], "bf16", seed=23)
+    assert kern.startswith("mfma_tq1"), kern
+    _check(got, want)
+
+
+def test_tq1_fp4_small_batches_misaligned_scales(bp):
     got, want, kern = _run(bp, "tq1", 2, 32, 2048, [3, 4], "bf16", seed=8, misalign_scales=True)
+    assert kern.startswith("fp4_tq1_m4"), kern
+    _check(got, want)
+
+
+def test_tq1_mfma_scales_from_global_memory(bp):
+    got, want, kern = _run(bp, "tq1", 2, 32, 2048, [5, 4], "bf16", seed=8, misalign_scales=True)
     assert kern.startswith("mfma_tq1") and kern.endswith("_gs"), kern
     _check(got, want)
 
