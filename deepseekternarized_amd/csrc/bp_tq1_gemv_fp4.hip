@@ -89,16 +89,21 @@ __device__ __forceinline__ int f4_pair_byte(int j, int kbA, int hf) {
 // 6 bytes extracted from registers that are not loaded (no loads at all), 7 = 2 + 3 + 4 (loads and byte extraction only),
 // 8 = 7 without the byte extraction (loads and their realignment only)
 //
-// NTOK > 1: up to NTOK token rows per expert (small decode batches). Every token has its own operand A tile, matrix
-// instructions and accumulators; the packed bytes and the table reads are shared. To fit 4 tiles beside the table,
-// an activation is then split into TWO fp8 pieces (PC = 2: exact for bf16 / int8 values down to 2^-9 of their group's
-// largest magnitude, at most 2^-17 of it dropped below), rows 2 g + p of operand A; with 4 tokens the ring of loads
-// is two chunks (the matrix instructions and the operand reads, not the loads, are what a wave waits for).
+// NTOK > 1: up to NTOK token rows per expert (small decode batches). Every token has its own operand A tile; the
+// packed bytes and the table reads are shared. To fit 4 tiles beside the table, an activation is then split into
+// TWO fp8 pieces (PC = 2: exact for bf16 / int8 values down to 2^-9 of their group's largest magnitude, at most
+// 2^-17 of it dropped below), and one matrix instruction serves TWO tokens: the 64-byte window (half a chunk, 320
+// digits) that instructions 0..3, and the one that instructions 4..7 multiply holds digits of only 3 groups
+// (0, 1, 2 and 2, 3, 4), so a token needs 3 group slots x 2 pieces = 6 rows instead of 10 if each window has its
+// own accumulator tile. Row 4 s + 2 t + p = piece p of token t (of the pair) in slot s; slot s is group s in the
+// first window and group 3, 4, 2 (s = 0, 1, 2) in the second, so a lane of the result (rows 4 lg + i) holds both
+// tokens' pieces of one group per window. 8 matrix instructions per chunk and token pair.
 template <int SDT, int WAVES, int ABL = 0, int NTOK = 1>
 __global__ __launch_bounds__(WAVES * 64, 4) void k_tq1_gemv_fp4(GemmArgs a, int nchunks, int bpw /* row blocks per workgroup */) {
-  constexpr int THREADS = WAVES * 64, GR = F4_GR, RD = NTOK <= 2 ? F4_RD : 2, BD = F4_BD, AD = F4_AD, PAIRS = NTOK <= 2 ? F4_PAIRS : 0;
+  constexpr int THREADS = WAVES * 64, GR = F4_GR, RD = F4_RD, BD = F4_BD, AD = F4_AD, PAIRS = F4_PAIRS;
   static_assert(!PAIRS || RD % 2 == 0, "pairs of chunks need an even ring");
-  static_assert(NTOK == 1 || (GR == 1 && AD == 0), "several tokens: one tile per wave, one operand A buffer");
+  static_assert(NTOK == 1 || (GR == 1 && AD == 0 && NTOK % 2 == 0), "several tokens: one tile per wave, one operand A buffer, token pairs");
+  constexpr int NP = NTOK / 2;               // token pairs
   constexpr int PC = f4_pieces(NTOK);        // fp8 pieces per activation
   constexpr int F4_HI_OFF = 64 * PC * 16, F4_ZERO_OFF = F4_HI_OFF + 4 * PC * 16, F4_PRE_OFF = F4_ZERO_OFF + 16;
   constexpr int F4_INV_OFF = F4_PRE_OFF + 32, F4_CHUNK_BYTES = f4_chunk_bytes(NTOK);
@@ -233,9 +238,10 @@ __global__ __launch_bounds__(WAVES * 64, 4) void k_tq1_gemv_fp4(GemmArgs a, int 
   __syncthreads();
 
   // ---- this lane as a row of operand A: rows 4 g + p = piece p of group g < 4; rows 3, 7, 11 = pieces of group 4; row 15 unused
-  // (two pieces: rows 2 g + p, rows 10..15 unused)
-  const int am_g = PC == 2 ? r16 >> 1 : (r16 & 3) < 3 ? r16 >> 2 : 4, am_p = PC == 2 ? r16 & 1 : (r16 & 3) < 3 ? r16 & 3 : r16 >> 2;
-  const bool am_used = PC == 2 ? r16 < 10 : r16 < 15;
+  // (several tokens: row 4 s + 2 t + p = piece p of the pair's token t in group slot s < 3, rows 12..15 unused)
+  const int am_g = PC == 2 ? r16 >> 2 : (r16 & 3) < 3 ? r16 >> 2 : 4, am_p = PC == 2 ? r16 & 1 : (r16 & 3) < 3 ? r16 & 3 : r16 >> 2;
+  const bool am_used = PC == 2 ? r16 < 12 : r16 < 15;
+  const unsigned lane_tok = PC == 2 ? (unsigned)(((r16 >> 1) & 1) * tile_bytes) : 0u;  // the lane's token of a pair: its tile
   unsigned aoff[4];  // 16-byte block (index within the chunk's part of the tile) of instruction j, half hf: byte 2 (j % 2) + hf of aoff[j / 2]
 #pragma unroll
   for (int j = 0; j < 8; ++j) {
@@ -244,9 +250,11 @@ __global__ __launch_bounds__(WAVES * 64, 4) void k_tq1_gemv_fp4(GemmArgs a, int 
     for (int hf = 0; hf < 2; ++hf) {
       const int blk = j * 8 + kb * 2 + hf;
       const int tt0 = 5 * f4_pair_byte(j, kb, hf), glo = tt0 >> 7, ghi = (tt0 + 9) >> 7;
+      // (several tokens: the group behind the lane's slot in this instruction's window)
+      const int g = PC == 3 || j < 4 ? am_g : am_g == 0 ? 3 : am_g == 1 ? 4 : 2;
       unsigned o = F4_ZERO_OFF / 16;
-      if (am_used && am_g == glo) o = PC * blk + am_p;
-      else if (am_used && am_g == ghi) o = F4_HI_OFF / 16 + PC * (ghi - 1) + am_p;
+      if (am_used && g == glo) o = PC * blk + am_p;
+      else if (am_used && g == ghi) o = F4_HI_OFF / 16 + PC * (ghi - 1) + am_p;
       both |= o << (8 * hf);
     }
     if (j & 1) aoff[j >> 1] |= both << 16;
@@ -286,7 +294,7 @@ __global__ __launch_bounds__(WAVES * 64, 4) void k_tq1_gemv_fp4(GemmArgs a, int 
   for (int pass = 0; pass < bpw; ++pass) {
     const int64_t n0 = block_row0(pass), n0_next = pass + 1 < bpw ? block_row0(pass + 1) : n0;
     const bool wave_live = (((int64_t)blockIdx.x * bpw + pass) * WAVES + wave) * (16 * GR) < a.N;
-    float total[NTOK > 1 ? NTOK : GR];  // per token, or (one token) per row tile
+    float total[NTOK > 1 ? NTOK : GR];  // per token (this lane's two groups of every chunk), or (one token) per row tile
 #pragma unroll
     for (int s = 0; s < (NTOK > 1 ? NTOK : GR); ++s) total[s] = 0.f;
     // chunk c of this block, or (c >= nchunks, chained) chunk c - nchunks of the next one: row offset (scalar) and chunk
@@ -308,11 +316,21 @@ __global__ __launch_bounds__(WAVES * 64, 4) void k_tq1_gemv_fp4(GemmArgs a, int 
         W[slot][s][h] = buf_load16(wrs, voff, (unsigned)(row * a.Kp) + 128u * cc + 64u * h);
       }
     };
+    // (several tokens: the lane's group of the first window and the one of the second: lg and 3, 4, 2, 2 for lg = 0..3;
+    // the lanes lg = 3 hold unused rows: their accumulators are 0)
+    const int g_w0 = kb < 3 ? kb : 2, g_w1 = kb == 0 ? 3 : kb == 1 ? 4 : 2;
     auto fetch_s = [&](int c) {  // 8 bytes from the dword that holds the scale of group kb of chunk c
       int64_t row0;
       int cc;
       target(c, row0, cc);
-      const unsigned at = (srow + SB * (unsigned)((5 * cc + (PC == 3 ? kb : 2 * kb)) >> gs)) & ~3u;
+      if (PC == 2) {  // the two dwords that hold the scales of the lane's two groups
+        const unsigned at0 = (srow + SB * (unsigned)((5 * cc + g_w0) >> gs)) & ~3u, at1 = (srow + SB * (unsigned)((5 * cc + g_w1) >> gs)) & ~3u;
+        const unsigned wo = (unsigned)(row0 * a.G * SB);
+        SQ[0].x = (unsigned)__builtin_amdgcn_raw_buffer_load_b32(srs, (int)at0, (int)wo, 0);
+        SQ[0].y = (unsigned)__builtin_amdgcn_raw_buffer_load_b32(srs, (int)at1, (int)wo, 0);
+        return;
+      }
+      const unsigned at = (srow + SB * (unsigned)((5 * cc + kb) >> gs)) & ~3u;
 #pragma unroll
       for (int s = 0; s < GR; ++s) {
         const int64_t row = row0 + 16 * s < a.N ? row0 + 16 * s : row0;
@@ -322,7 +340,7 @@ __global__ __launch_bounds__(WAVES * 64, 4) void k_tq1_gemv_fp4(GemmArgs a, int 
     // (chunk slots and pipeline stages are compile-time constants: every register array below is indexed statically)
     auto step = [&](int c, auto cur_c) {
       constexpr int cur = decltype(cur_c)::value, nxt = (cur + 1) % RD;
-      constexpr int NC = NTOK > 1 ? NTOK : GR;  // accumulator tiles: one per token, or (one token) one per row tile
+      constexpr int NC = NTOK > 1 ? NTOK : GR;  // accumulator tiles: per token pair and window, or (one token) one per row tile
       f32x4 C[NC];
 #pragma unroll
       for (int s = 0; s < NC; ++s) C[s] = f32x4{0.f, 0.f, 0.f, 0.f};
@@ -345,9 +363,9 @@ __global__ __launch_bounds__(WAVES * 64, 4) void k_tq1_gemv_fp4(GemmArgs a, int 
           B[w] = ABL == 2 || ABL == 7 || ABL == 8 ? at : *(const lds_u32*)at;
         }
       };
-      auto a_read = [&](int j, u32x4& lo, u32x4& hi, int tt = 0) {
+      auto a_read = [&](int j, u32x4& lo, u32x4& hi, int pair = 0) {
         if (ABL == 3 || ABL == 7 || ABL == 8) { lo = u32x4{cbase, dlt, lane4, cbase}; hi = lo; return; }
-        const unsigned tbase = cbase + (unsigned)(tt * tile_bytes);
+        const unsigned tbase = cbase + lane_tok + (unsigned)(2 * pair * tile_bytes);
         unsigned ao = aoff[j >> 1];
         // (several tokens: the block offsets are extracted anew at every use; hoisted out of the chunk loop, the
         // 16 NTOK addresses of a lane would not fit its registers)
@@ -409,16 +427,17 @@ __global__ __launch_bounds__(WAVES * 64, 4) void k_tq1_gemv_fp4(GemmArgs a, int 
         const u32x4 bq = Bq[t % (BD + 1)];
         const i32x8 B = {(int)bq.x, (int)bq.y, (int)bq.z, (int)bq.w, 0, 0, 0, 0};
         if (NTOK > 1) {
-          // The same packed bytes against every token's operand A, one token at a time (the scheduling barriers keep
-          // the compiler from reading all the operands first: 8 registers each). Tiles of tokens the expert does not
-          // have hold whatever LDS held; their accumulators are not used.
+          // The same packed bytes against every token pair's operand A, one pair at a time (the scheduling barriers
+          // keep the compiler from reading all the operands first: 8 registers each). Tiles of tokens the expert does
+          // not have hold whatever LDS held; their rows of the accumulators are not used.
 #pragma unroll
-          for (int tt = 0; tt < NTOK; ++tt) {
+          for (int pr = 0; pr < NP; ++pr) {
             __builtin_amdgcn_sched_barrier(0);
-            a_read(j, Alo[0], Ahi[0], tt);
+            a_read(j, Alo[0], Ahi[0], pr);
             const u32x4 alo = Alo[0], ahi = Ahi[0];
             const i32x8 A = {(int)alo.x, (int)alo.y, (int)alo.z, (int)alo.w, (int)ahi.x, (int)ahi.y, (int)ahi.z, (int)ahi.w};
-            C[tt] = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(A, B, C[tt], 0 /* A: E4M3 */, 4 /* B: E2M1 */, 0, 0, 0, 0);
+            constexpr int ci = j >> 2;  // the window's accumulator tile
+            C[2 * pr + ci] = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(A, B, C[2 * pr + ci], 0 /* A: E4M3 */, 4 /* B: E2M1 */, 0, 0, 0, 0);
           }
           __builtin_amdgcn_sched_barrier(0);
           return;
@@ -436,15 +455,18 @@ __global__ __launch_bounds__(WAVES * 64, 4) void k_tq1_gemv_fp4(GemmArgs a, int 
       BP_F4_STAGE(8); BP_F4_STAGE(9); BP_F4_STAGE(10); BP_F4_STAGE(11); BP_F4_STAGE(12); BP_F4_STAGE(13); BP_F4_STAGE(14); BP_F4_STAGE(15);
 #undef BP_F4_STAGE
       // the chunk's 5 group sums under their scales. Three pieces: this lane holds group kb (3 pieces) and a piece of
-      // group 4, whose scale sits next to that of group 3 in the lanes kb = 3. Two pieces: groups 2 kb and 2 kb + 1.
-      const int g_first = PC == 3 ? kb : 2 * kb;
-      const unsigned ia = (unsigned)((5 * c + g_first) >> gs), ib = (unsigned)((5 * c + g_first + 1) >> gs);
+      // group 4, whose scale sits next to that of group 3 in the lanes kb = 3. Several tokens: one group per window.
+      const int g_first = PC == 3 ? kb : g_w0;
+      const unsigned ia = (unsigned)((5 * c + g_first) >> gs), ib = (unsigned)((5 * c + (PC == 3 ? g_first + 1 : g_w1)) >> gs);
 #pragma unroll
       for (int s = 0; s < GR; ++s) {
         unsigned ra, rb;  // the scale of group g_first, and the one after it (bits as stored)
         if (SDT == BP_F32) {
           ra = SQ[s].x;
           rb = ib == ia ? ra : SQ[s].y;
+        } else if (PC == 2) {
+          ra = (SQ[s].x >> (8u * ((srow + SB * ia) & 3u))) & 0xffffu;
+          rb = (SQ[s].y >> (8u * ((srow + SB * ib) & 3u))) & 0xffffu;
         } else {
           const unsigned v = __builtin_amdgcn_alignbyte(SQ[s].y, SQ[s].x, (srow + SB * ia) & 3u);
           ra = v & 0xffffu;
@@ -460,10 +482,12 @@ __global__ __launch_bounds__(WAVES * 64, 4) void k_tq1_gemv_fp4(GemmArgs a, int 
         } else {  // (one row tile per wave: s == 0)
           const float sb = SDT == BP_F32 ? __uint_as_float(rb) : SDT == BP_F16 ? f16_bits_to_f32((uint16_t)rb) : __uint_as_float(rb << 16);
 #pragma unroll
-          for (int tt = 0; tt < NTOK; ++tt) {  // (the inverses of groups past the chunk's five are 0)
-            const unsigned ivb = cbase + (unsigned)(tt * tile_bytes) + F4_INV_OFF + 8 * kb;
-            const float inv_a = __uint_as_float(*(const lds_u32*)ivb), inv_b = __uint_as_float(*(const lds_u32*)(ivb + 4));
-            total[tt] += sa * inv_a * (C[tt][0] + C[tt][1]) + sb * inv_b * (C[tt][2] + C[tt][3]);
+          for (int tt = 0; tt < NTOK; ++tt) {  // rows 4 lg + 2 (tt % 2) + p of the pair's two tiles
+            const unsigned ivb = cbase + (unsigned)(tt * tile_bytes) + F4_INV_OFF;
+            const float inv_a = __uint_as_float(*(const lds_u32*)(ivb + 4 * g_w0)), inv_b = __uint_as_float(*(const lds_u32*)(ivb + 4 * g_w1));
+            const f32x4 c0 = C[2 * (tt >> 1)], c1 = C[2 * (tt >> 1) + 1];
+            const float s0 = (tt & 1) ? c0[2] + c0[3] : c0[0] + c0[1], s1 = (tt & 1) ? c1[2] + c1[3] : c1[0] + c1[1];
+            total[tt] += sa * inv_a * s0 + sb * inv_b * s1;
           }
         }
       }
