@@ -203,7 +203,7 @@ def main() -> int:
     if not a.no_extras:
         del launch
         torch.cuda.empty_cache()
-        for m in (4, 16, 32):  # the other decode batch sizes of the configuration
+        for m in (2, 4, 16, 32):  # the other decode batch sizes of the configuration
             l2, wb2 = uniform_launch(bp, torch, fmt, N, K, m, act, terms, L)
             _, k2, kn2 = l2.time(max(5, a.steps // 2), 2)
             also[f"M{m}_weight_GBps"] = round(wb2 / k2 / 1e9, 1)

@@ -97,10 +97,11 @@ __device__ __forceinline__ int f4_pair_byte(int j, int kbA, int hf) {
 // (0, 1, 2 and 2, 3, 4), so a token needs 3 group slots x 2 pieces = 6 rows instead of 10 if each window has its
 // own accumulator tile. Row 4 s + 2 t + p = piece p of token t (of the pair) in slot s; slot s is group s in the
 // first window and group 3, 4, 2 (s = 0, 1, 2) in the second, so a lane of the result (rows 4 lg + i) holds both
-// tokens' pieces of one group per window. 8 matrix instructions per chunk and token pair.
+// tokens' pieces of one group per window. 8 matrix instructions per chunk and token pair; with two pairs the ring
+// of loads is two chunks (registers; the loads are not what a wave then waits for).
 template <int SDT, int WAVES, int ABL = 0, int NTOK = 1>
 __global__ __launch_bounds__(WAVES * 64, 4) void k_tq1_gemv_fp4(GemmArgs a, int nchunks, int bpw /* row blocks per workgroup */) {
-  constexpr int THREADS = WAVES * 64, GR = F4_GR, RD = F4_RD, BD = F4_BD, AD = F4_AD, PAIRS = F4_PAIRS;
+  constexpr int THREADS = WAVES * 64, GR = F4_GR, RD = NTOK <= 2 ? F4_RD : 2, BD = F4_BD, AD = F4_AD, PAIRS = NTOK <= 2 ? F4_PAIRS : 0;
   static_assert(!PAIRS || RD % 2 == 0, "pairs of chunks need an even ring");
   static_assert(NTOK == 1 || (GR == 1 && AD == 0 && NTOK % 2 == 0), "several tokens: one tile per wave, one operand A buffer, token pairs");
   constexpr int NP = NTOK / 2;               // token pairs

@@ -177,7 +177,8 @@ def test_tq1_mfma_tiles(bp, K, counts, act):
 @pytest.mark.parametrize("K", [1024, 2048, 7168])
 @pytest.mark.parametrize("counts", [[2, 0, 1], [2, 2, 2], [4, 3, 1], [3, 0, 0]])
 def test_tq1_fp4_small_batches(bp, K, counts, act):
-    """2 and up to 4 token rows per expert: one operand tile per token (two fp8 pieces), the packed bytes read once."""
+    """2 and up to 4 token rows per expert: one operand tile per token (two fp8 pieces), one matrix instruction per
+    token pair; experts with fewer rows than the launch's variant holds leave rows of the operand unused."""
     got, want, kern = _run(bp, "tq1", 3, 80, K, counts, act, terms=2, seed=K + 7 * sum(counts))
     assert kern.startswith("fp4_tq1_m2" if max(counts) <= 2 else "fp4_tq1_m4"), kern
     _check(got, want)
