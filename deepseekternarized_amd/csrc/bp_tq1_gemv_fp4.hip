@@ -118,7 +118,8 @@ __global__ __launch_bounds__(WAVES * 64, 4) void k_tq1_gemv_fp4(GemmArgs a, int 
   if (o0 >= o1) return;  // uniform for the workgroup; the expert's first NTOK token rows are used (max_rows <= NTOK)
   const int64_t tok = o0;
   const int ntok = o1 - o0 < NTOK ? (int)(o1 - o0) : NTOK;
-  const int tile_bytes = nchunks * F4_CHUNK_BYTES;  // one token's tile
+  // the tiles of the NTOK tokens are interleaved chunk by chunk (a pair's tiles are a constant apart)
+  auto tile_at = [](int tt, int c) { return AT + (c * NTOK + tt) * F4_CHUNK_BYTES; };
   const int gs = a.group == 256 ? 1 : 0;  // scale groups of 256: two 128-wide work groups share a scale
   const bool x16 = a.x_dtype == BP_BF16 || a.x_dtype == BP_F16;
   auto widen16 = [&](unsigned h) { return a.x_dtype == BP_BF16 ? bf16_bits_to_f32((uint16_t)h) : f16_bits_to_f32((uint16_t)h); };
@@ -140,13 +141,12 @@ __global__ __launch_bounds__(WAVES * 64, 4) void k_tq1_gemv_fp4(GemmArgs a, int 
   }
   for (int g = threadIdx.x; g < ntok * nchunks * 8; g += THREADS) {
     const int tt = g / (nchunks * 8), gc = g - tt * nchunks * 8;
-    *(lds_u32*)(AT + tt * tile_bytes + (gc >> 3) * F4_CHUNK_BYTES + F4_PRE_OFF + 4 * (gc & 7)) = 0u;
+    *(lds_u32*)(tile_at(tt, gc >> 3) + F4_PRE_OFF + 4 * (gc & 7)) = 0u;
   }
   __syncthreads();
   for (int idx = threadIdx.x; idx < 256 * 32; idx += THREADS) *(lds_u32*)(4 * idx) = *(const lds_u32*)(128 * (idx >> 5));
   for (int tt = 0; tt < ntok; ++tt) {
   const int64_t xrow = (tok + tt) * a.K;
-  const int TB = AT + tt * tile_bytes;
   if (a.x_dtype != BP_I8) {  // (int8 values fit as they are: prescale 1)
     for (int64_t k0 = 8 * (int64_t)threadIdx.x; k0 < a.K; k0 += 8 * THREADS) {  // 8 values of one group per thread
       unsigned m = 0;
@@ -165,7 +165,7 @@ __global__ __launch_bounds__(WAVES * 64, 4) void k_tq1_gemv_fp4(GemmArgs a, int 
         }
       }
       const int gg = (int)(k0 >> 7);
-      __hip_atomic_fetch_max((lds_u32*)(TB + (gg / 5) * F4_CHUNK_BYTES + F4_PRE_OFF + 4 * (gg % 5)), m, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
+      __hip_atomic_fetch_max((lds_u32*)(tile_at(tt, gg / 5) + F4_PRE_OFF + 4 * (gg % 5)), m, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
     }
   }
   }
@@ -173,7 +173,7 @@ __global__ __launch_bounds__(WAVES * 64, 4) void k_tq1_gemv_fp4(GemmArgs a, int 
   // the maxima become prescales 2^sh (sh brings the group's largest magnitude into [128, 256)) and their inverses
   for (int gt = threadIdx.x; gt < ntok * nchunks * 8; gt += THREADS) {
     const int tt = gt / (nchunks * 8), g = gt - tt * nchunks * 8;
-    const unsigned at = (unsigned)(AT + tt * tile_bytes + (g >> 3) * F4_CHUNK_BYTES + 4 * (g & 7));
+    const unsigned at = (unsigned)(tile_at(tt, g >> 3) + 4 * (g & 7));
     const bool real = (g & 7) < 5 && 128 * (int64_t)(5 * (g >> 3) + (g & 7)) < a.K;
     int sh = 0;
     if (real && a.x_dtype != BP_I8) {
@@ -191,7 +191,7 @@ __global__ __launch_bounds__(WAVES * 64, 4) void k_tq1_gemv_fp4(GemmArgs a, int 
     const int64_t xrow = (tok + tt) * a.K;
     const int c = it >> 6, blk = it & 63;
     const int tt0 = 5 * f4_pair_byte(blk >> 3, (blk >> 1) & 3, blk & 1), glo = tt0 >> 7, ghi = (tt0 + 9) >> 7;
-    const unsigned dst = (unsigned)(AT + tt * tile_bytes + c * F4_CHUNK_BYTES);
+    const unsigned dst = (unsigned)tile_at(tt, c);
     const float pre_lo = __uint_as_float(*(const lds_u32*)(dst + F4_PRE_OFF + 4 * glo));
     const float pre_hi = __uint_as_float(*(const lds_u32*)(dst + F4_PRE_OFF + 4 * ghi));
     const int64_t k0 = 640 * (int64_t)c + tt0;
@@ -242,7 +242,7 @@ __global__ __launch_bounds__(WAVES * 64, 4) void k_tq1_gemv_fp4(GemmArgs a, int 
   // (several tokens: row 4 s + 2 t + p = piece p of the pair's token t in group slot s < 3, rows 12..15 unused)
   const int am_g = PC == 2 ? r16 >> 2 : (r16 & 3) < 3 ? r16 >> 2 : 4, am_p = PC == 2 ? r16 & 1 : (r16 & 3) < 3 ? r16 & 3 : r16 >> 2;
   const bool am_used = PC == 2 ? r16 < 12 : r16 < 15;
-  const unsigned lane_tok = PC == 2 ? (unsigned)(((r16 >> 1) & 1) * tile_bytes) : 0u;  // the lane's token of a pair: its tile
+  const unsigned lane_tok = PC == 2 ? (unsigned)(((r16 >> 1) & 1) * F4_CHUNK_BYTES) : 0u;  // the lane's token of a pair: its tile
   unsigned aoff[4];  // 16-byte block (index within the chunk's part of the tile) of instruction j, half hf: byte 2 (j % 2) + hf of aoff[j / 2]
 #pragma unroll
   for (int j = 0; j < 8; ++j) {
@@ -345,7 +345,7 @@ __global__ __launch_bounds__(WAVES * 64, 4) void k_tq1_gemv_fp4(GemmArgs a, int 
       f32x4 C[NC];
 #pragma unroll
       for (int s = 0; s < NC; ++s) C[s] = f32x4{0.f, 0.f, 0.f, 0.f};
-      const unsigned cbase = (unsigned)(AT + c * F4_CHUNK_BYTES);
+      const unsigned cbase = (unsigned)tile_at(0, c);
       // packed bytes of (instruction j, tile s) = dword j % 4 of the lane's window j / 4, shifted to the row's alignment;
       // the dword after a window is the first one of the next quarter's window (for the last quarter: of the first
       // quarter's next window, which for the second window is the next chunk's)
@@ -364,15 +364,10 @@ __global__ __launch_bounds__(WAVES * 64, 4) void k_tq1_gemv_fp4(GemmArgs a, int 
           B[w] = ABL == 2 || ABL == 7 || ABL == 8 ? at : *(const lds_u32*)at;
         }
       };
-      auto a_read = [&](int j, u32x4& lo, u32x4& hi, int pair = 0) {
+      auto a_read = [&](int j, u32x4& lo, u32x4& hi) {  // (one token)
         if (ABL == 3 || ABL == 7 || ABL == 8) { lo = u32x4{cbase, dlt, lane4, cbase}; hi = lo; return; }
-        const unsigned tbase = cbase + lane_tok + (unsigned)(2 * pair * tile_bytes);
-        unsigned ao = aoff[j >> 1];
-        // (several tokens: the block offsets are extracted anew at every use; hoisted out of the chunk loop, the
-        // 16 NTOK addresses of a lane would not fit its registers)
-        if (NTOK > 1) asm volatile("; packed block offsets" : "+v"(ao));
-        lo = *(const lds_u32x4*)((((ao >> (16 * (j & 1))) & 0xffu) << 4) + tbase);
-        hi = *(const lds_u32x4*)((((ao >> (16 * (j & 1) + 8)) & 0xffu) << 4) + tbase);
+        lo = *(const lds_u32x4*)((((aoff[j >> 1] >> (16 * (j & 1))) & 0xffu) << 4) + cbase);
+        hi = *(const lds_u32x4*)((((aoff[j >> 1] >> (16 * (j & 1) + 8)) & 0xffu) << 4) + cbase);
       };
       // software pipeline over the 16 (instruction, tile) pairs t = 2 j + s: table reads BD pairs ahead, operand A one
       // instruction ahead if AD; the scheduling barriers keep the compiler from sinking the reads back to their uses
@@ -431,11 +426,16 @@ __global__ __launch_bounds__(WAVES * 64, 4) void k_tq1_gemv_fp4(GemmArgs a, int 
           // The same packed bytes against every token pair's operand A, one pair at a time (the scheduling barriers
           // keep the compiler from reading all the operands first: 8 registers each). Tiles of tokens the expert does
           // not have hold whatever LDS held; their rows of the accumulators are not used.
+          unsigned ao = aoff[j >> 1];
+          // (the block offsets are extracted anew at every use: left visible, the compiler hoists the 16 addresses of
+          // a lane out of the chunk loop, and they do not fit its registers)
+          asm volatile("; packed block offsets" : "+v"(ao));
+          const unsigned lo_at = (((ao >> (16 * (j & 1))) & 0xffu) << 4) + cbase + lane_tok;
+          const unsigned hi_at = (((ao >> (16 * (j & 1) + 8)) & 0xffu) << 4) + cbase + lane_tok;
 #pragma unroll
           for (int pr = 0; pr < NP; ++pr) {
             __builtin_amdgcn_sched_barrier(0);
-            a_read(j, Alo[0], Ahi[0], pr);
-            const u32x4 alo = Alo[0], ahi = Ahi[0];
+            const u32x4 alo = *(const lds_u32x4*)(lo_at + 2 * pr * F4_CHUNK_BYTES), ahi = *(const lds_u32x4*)(hi_at + 2 * pr * F4_CHUNK_BYTES);
             const i32x8 A = {(int)alo.x, (int)alo.y, (int)alo.z, (int)alo.w, (int)ahi.x, (int)ahi.y, (int)ahi.z, (int)ahi.w};
             constexpr int ci = j >> 2;  // the window's accumulator tile
             C[2 * pr + ci] = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(A, B, C[2 * pr + ci], 0 /* A: E4M3 */, 4 /* B: E2M1 */, 0, 0, 0, 0);
@@ -484,7 +484,7 @@ __global__ __launch_bounds__(WAVES * 64, 4) void k_tq1_gemv_fp4(GemmArgs a, int 
           const float sb = SDT == BP_F32 ? __uint_as_float(rb) : SDT == BP_F16 ? f16_bits_to_f32((uint16_t)rb) : __uint_as_float(rb << 16);
 #pragma unroll
           for (int tt = 0; tt < NTOK; ++tt) {  // rows 4 lg + 2 (tt % 2) + p of the pair's two tiles
-            const unsigned ivb = cbase + (unsigned)(tt * tile_bytes) + F4_INV_OFF;
+            const unsigned ivb = cbase + (unsigned)(tt * F4_CHUNK_BYTES) + F4_INV_OFF;
             const float inv_a = __uint_as_float(*(const lds_u32*)(ivb + 4 * g_w0)), inv_b = __uint_as_float(*(const lds_u32*)(ivb + 4 * g_w1));
             const f32x4 c0 = C[2 * (tt >> 1)], c1 = C[2 * (tt >> 1) + 1];
             const float s0 = (tt & 1) ? c0[2] + c0[3] : c0[0] + c0[1], s1 = (tt & 1) ? c1[2] + c1[3] : c1[0] + c1[1];
