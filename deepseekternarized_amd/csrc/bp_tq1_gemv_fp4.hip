@@ -574,8 +574,8 @@ int launch_f4(const GemmArgs& a, hipStream_t s) {
   const int64_t experts = a.E < a.T ? a.E : a.T;
   if (NTOK > 1) {
     const bool wide = lds > (size_t)F4_LDS_MAX / 2 || ((a.N + 255) / 256) * experts >= 4 * (int64_t)cus;
-    if (!wide) return launch_f4_k<SDT, 8, 0, NTOK>(a, s, NTOK == 2 ? "fp4_tq1_m2_w8" : "fp4_tq1_m4_w8", (int)nchunks, lds);
-    return launch_f4_k<SDT, 16, 0, NTOK>(a, s, NTOK == 2 ? "fp4_tq1_m2_w16" : "fp4_tq1_m4_w16", (int)nchunks, lds);
+    if (!wide) return launch_f4_k<SDT, 8, 0, NTOK>(a, s, NTOK == 2 ? "fp4_tq1_m2_w8" : NTOK == 4 ? "fp4_tq1_m4_w8" : NTOK == 6 ? "fp4_tq1_m6_w8" : "fp4_tq1_m8_w8", (int)nchunks, lds);
+    return launch_f4_k<SDT, 16, 0, NTOK>(a, s, NTOK == 2 ? "fp4_tq1_m2_w16" : NTOK == 4 ? "fp4_tq1_m4_w16" : NTOK == 6 ? "fp4_tq1_m6_w16" : "fp4_tq1_m8_w16", (int)nchunks, lds);
   }
   if (const char* t = getenv("BP_TUNE_F4ABL")) {  // development: timing ablations (one token)
     if (SDT == BP_F16 && atoi(t) == 1) return launch_f4_k<BP_F16, 8, 1>(a, s, "abl1_fp4", (int)nchunks, lds);
@@ -597,12 +597,12 @@ int launch_f4(const GemmArgs& a, hipStream_t s) {
 
 }  // namespace
 
-// max_rows <= 4 (checked by the caller): one token row per expert, or 2 / up to 4 (two fp8 pieces per activation).
+// One token row per expert, or up to 2 / 4 / 6 / 8 (two fp8 pieces per activation) while the tiles fit in LDS.
 // BP_ERR_UNSUPPORTED (no message): the caller falls back to its other kernels.
 int launch_tq1_gemv_fp4(const GemmArgs& a, hipStream_t s) {
   if (a.x_dtype != BP_BF16 && a.x_dtype != BP_F16 && a.x_dtype != BP_I8) return BP_ERR_UNSUPPORTED;
   if (a.max_rows > 1 && a.x_dtype == BP_F16) return BP_ERR_UNSUPPORTED;  // (11 significant bits need the third piece)
-  if (a.max_rows < 1 || a.max_rows > 4) return BP_ERR_UNSUPPORTED;
+  if (a.max_rows < 1 || a.max_rows > 8) return BP_ERR_UNSUPPORTED;
   if (a.N % 16 != 0 || a.Kp != (a.K + 4) / 5 || (a.group != 128 && a.group != 256)) return BP_ERR_UNSUPPORTED;
   for (int t = 0; t < a.n_terms; ++t)
     if (a.scale_dtype == BP_F32 && ((uintptr_t)a.w_scale[t] & 3) != 0) return BP_ERR_UNSUPPORTED;
@@ -614,10 +614,18 @@ int launch_tq1_gemv_fp4(const GemmArgs& a, hipStream_t s) {
     if (a.scale_dtype == BP_F16) return launch_f4<BP_F16, 2>(a, s);
     if (a.scale_dtype == BP_BF16) return launch_f4<BP_BF16, 2>(a, s);
     if (a.scale_dtype == BP_F32) return launch_f4<BP_F32, 2>(a, s);
-  } else {
+  } else if (a.max_rows <= 4) {
     if (a.scale_dtype == BP_F16) return launch_f4<BP_F16, 4>(a, s);
     if (a.scale_dtype == BP_BF16) return launch_f4<BP_BF16, 4>(a, s);
     if (a.scale_dtype == BP_F32) return launch_f4<BP_F32, 4>(a, s);
+  } else if (a.max_rows <= 6) {  // (6 tiles fit beside the table for K <= 5760)
+    if (a.scale_dtype == BP_F16) return launch_f4<BP_F16, 6>(a, s);
+    if (a.scale_dtype == BP_BF16) return launch_f4<BP_BF16, 6>(a, s);
+    if (a.scale_dtype == BP_F32) return launch_f4<BP_F32, 6>(a, s);
+  } else {  // (8 tiles fit beside the table for K <= 4480)
+    if (a.scale_dtype == BP_F16) return launch_f4<BP_F16, 8>(a, s);
+    if (a.scale_dtype == BP_BF16) return launch_f4<BP_BF16, 8>(a, s);
+    if (a.scale_dtype == BP_F32) return launch_f4<BP_F32, 8>(a, s);
   }
   return BP_ERR_UNSUPPORTED;
 }

@@ -169,18 +169,21 @@ def test_tq1_gemv_fp8_pieces_keep_small_activations(bp, act):
 @pytest.mark.parametrize("counts", [[2, 0, 5], [16, 3, 1], [20, 1, 37]])
 def test_tq1_mfma_tiles(bp, K, counts, act):
     got, want, kern = _run(bp, "tq1", 3, 80, K, counts, act, terms=2, seed=K + sum(counts))
-    assert kern.startswith("mfma_tq1"), kern
+    # (up to 6 / 8 rows per expert go to the fp8 x fp4 kernel while their operand tiles fit beside its table: K <= 5760 / 4480)
+    assert kern.startswith("fp4_tq1_m6" if max(counts) <= 6 and K <= 5760 else "mfma_tq1"), kern
     _check(got, want)
 
 
 @pytest.mark.parametrize("act", ["bf16", "int8"])
-@pytest.mark.parametrize("K", [1024, 2048, 7168])
-@pytest.mark.parametrize("counts", [[2, 0, 1], [2, 2, 2], [4, 3, 1], [3, 0, 0]])
+@pytest.mark.parametrize("K", [1024, 2048, 5120, 7168])
+@pytest.mark.parametrize("counts", [[2, 0, 1], [2, 2, 2], [4, 3, 1], [3, 0, 0], [8, 5, 1], [1, 6, 7], [5, 6, 0]])
 def test_tq1_fp4_small_batches(bp, K, counts, act):
-    """2 and up to 4 token rows per expert: one operand tile per token (two fp8 pieces), one matrix instruction per
-    token pair; experts with fewer rows than the launch's variant holds leave rows of the operand unused."""
+    """2, up to 4 and (K <= 5760 / 4480) up to 6 / 8 token rows per expert: one operand tile per token (two fp8 pieces), one matrix
+    instruction per token pair; experts with fewer rows than the launch's variant holds leave rows of the operand unused."""
     got, want, kern = _run(bp, "tq1", 3, 80, K, counts, act, terms=2, seed=K + 7 * sum(counts))
-    assert kern.startswith("fp4_tq1_m2" if max(counts) <= 2 else "fp4_tq1_m4"), kern
+    m = max(counts)
+    want_kernel = "fp4_tq1_m2" if m <= 2 else "fp4_tq1_m4" if m <= 4 else "fp4_tq1_m6" if m <= 6 and K <= 5760 else "fp4_tq1_m8" if K <= 4480 else "mfma_tq1"
+    assert kern.startswith(want_kernel), kern
     _check(got, want)
 
 
@@ -207,7 +210,7 @@ def test_tq1_fp4_small_batches_misaligned_scales(bp):
 
 
 def test_tq1_mfma_scales_from_global_memory(bp):
-    got, want, kern = _run(bp, "tq1", 2, 32, 2048, [5, 4], "bf16", seed=8, misalign_scales=True)
+    got, want, kern = _run(bp, "tq1", 2, 32, 2048, [9, 4], "bf16", seed=8, misalign_scales=True)
     assert kern.startswith("mfma_tq1") and kern.endswith("_gs"), kern
     _check(got, want)
 
