@@ -100,7 +100,7 @@ __device__ __forceinline__ int f4_pair_byte(int j, int kbA, int hf) {
 // tokens' pieces of one group per window. 8 matrix instructions per chunk and token pair; with two pairs the ring
 // of loads is two chunks (registers; the loads are not what a wave then waits for).
 template <int SDT, int WAVES, int ABL = 0, int NTOK = 1>
-__global__ __launch_bounds__(WAVES * 64, 4) void k_tq1_gemv_fp4(GemmArgs a, int nchunks, int bpw /* row blocks per workgroup */) {
+__global__ __launch_bounds__(WAVES * 64, 4) void k_tq1_gemv_fp4(GemmArgs a, int total_chunks, int first_chunk, int nchunks, int bpw /* row blocks per workgroup */) {
   constexpr int THREADS = WAVES * 64, GR = F4_GR, RD = NTOK <= 2 ? F4_RD : 2, BD = F4_BD, AD = F4_AD, PAIRS = NTOK <= 2 ? F4_PAIRS : 0;
   static_assert(!PAIRS || RD % 2 == 0, "pairs of chunks need an even ring");
   static_assert(NTOK == 1 || (GR == 1 && AD == 0 && NTOK % 2 == 0), "several tokens: one tile per wave, one operand A buffer, token pairs");
@@ -139,16 +139,25 @@ __global__ __launch_bounds__(WAVES * 64, 4) void k_tq1_gemv_fp4(GemmArgs a, int 
     }
     *(lds_u32*)(128 * threadIdx.x) = ent;
   }
+  // A launch covers the chunks first_chunk .. first_chunk + nchunks - 1 of every row (all of them unless the tokens'
+  // tiles of all chunks do not fit in LDS: then the host launches once per segment of K, and the output takes the
+  // segments' partial sums one launch after the other). Chunk c below is chunk cb + c of the rows.
+  const int cb = NTOK == 1 ? 0 : first_chunk;
+  // The last bytes of a chunk are completed from the first dword of the chunk after it (rows start at any byte). At
+  // the end of a row that dword meets activations that are 0; at the end of a segment it is needed, so the chunk
+  // after a segment that is not the last one is loaded as well.
+  const int last_load = NTOK > 1 && cb + nchunks < total_chunks ? nchunks : nchunks - 1;
   for (int g = threadIdx.x; g < ntok * nchunks * 8; g += THREADS) {
     const int tt = g / (nchunks * 8), gc = g - tt * nchunks * 8;
     *(lds_u32*)(tile_at(tt, gc >> 3) + F4_PRE_OFF + 4 * (gc & 7)) = 0u;
   }
   __syncthreads();
   for (int idx = threadIdx.x; idx < 256 * 32; idx += THREADS) *(lds_u32*)(4 * idx) = *(const lds_u32*)(128 * (idx >> 5));
+  const int64_t kbeg = 640 * (int64_t)cb, kend = a.K < 640 * (int64_t)(cb + nchunks) ? a.K : 640 * (int64_t)(cb + nchunks);
   for (int tt = 0; tt < ntok; ++tt) {
   const int64_t xrow = (tok + tt) * a.K;
   if (a.x_dtype != BP_I8) {  // (int8 values fit as they are: prescale 1)
-    for (int64_t k0 = 8 * (int64_t)threadIdx.x; k0 < a.K; k0 += 8 * THREADS) {  // 8 values of one group per thread
+    for (int64_t k0 = kbeg + 8 * (int64_t)threadIdx.x; k0 < kend; k0 += 8 * THREADS) {  // 8 values of one group per thread
       unsigned m = 0;
       if (x16 && k0 + 8 <= a.K) {
         const u32x4 q = ((const F4Packed16*)((const uint16_t*)a.x + xrow + k0))->v;
@@ -164,7 +173,7 @@ __global__ __launch_bounds__(WAVES * 64, 4) void k_tq1_gemv_fp4(GemmArgs a, int 
           m = m > v ? m : v;
         }
       }
-      const int gg = (int)(k0 >> 7);
+      const int gg = (int)((k0 - kbeg) >> 7);
       __hip_atomic_fetch_max((lds_u32*)(tile_at(tt, gg / 5) + F4_PRE_OFF + 4 * (gg % 5)), m, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
     }
   }
@@ -174,7 +183,7 @@ __global__ __launch_bounds__(WAVES * 64, 4) void k_tq1_gemv_fp4(GemmArgs a, int 
   for (int gt = threadIdx.x; gt < ntok * nchunks * 8; gt += THREADS) {
     const int tt = gt / (nchunks * 8), g = gt - tt * nchunks * 8;
     const unsigned at = (unsigned)(tile_at(tt, g >> 3) + 4 * (g & 7));
-    const bool real = (g & 7) < 5 && 128 * (int64_t)(5 * (g >> 3) + (g & 7)) < a.K;
+    const bool real = (g & 7) < 5 && 128 * (int64_t)(5 * (cb + (g >> 3)) + (g & 7)) < a.K;
     int sh = 0;
     if (real && a.x_dtype != BP_I8) {
       sh = 134 - (int)((*(const lds_u32*)(at + F4_PRE_OFF) >> 23) & 255u);
@@ -194,7 +203,7 @@ __global__ __launch_bounds__(WAVES * 64, 4) void k_tq1_gemv_fp4(GemmArgs a, int 
     const unsigned dst = (unsigned)tile_at(tt, c);
     const float pre_lo = __uint_as_float(*(const lds_u32*)(dst + F4_PRE_OFF + 4 * glo));
     const float pre_hi = __uint_as_float(*(const lds_u32*)(dst + F4_PRE_OFF + 4 * ghi));
-    const int64_t k0 = 640 * (int64_t)c + tt0;
+    const int64_t k0 = 640 * (int64_t)(cb + c) + tt0;
     float y[10];
     if (x16 && k0 + 10 <= a.K) {  // 20 bytes at an even address
       const uint16_t* src = (const uint16_t*)a.x + xrow + k0;
@@ -269,7 +278,7 @@ __global__ __launch_bounds__(WAVES * 64, 4) void k_tq1_gemv_fp4(GemmArgs a, int 
   // The tables serve `bpw` blocks of WAVES x GR x 16 rows, one after the other (the build is paid once per workgroup),
   // term by term: a term's blocks form one stream of chunks, and when the chunks of a row fill the ring a whole
   // number of times the refills run on into the next block, so the loads do not drain between blocks.
-  const bool chain = nchunks % RD == 0;
+  const bool chain = nchunks % RD == 0 && last_load == nchunks - 1;
   auto block_row0 = [&](int pass) -> int64_t {  // first row of this wave's tile(s) in block `pass`; 0 (valid, not stored) past N
     const int64_t r = (((int64_t)blockIdx.x * bpw + pass) * WAVES + wave) * (16 * GR);
     return r < a.N ? r : 0;
@@ -302,7 +311,7 @@ __global__ __launch_bounds__(WAVES * 64, 4) void k_tq1_gemv_fp4(GemmArgs a, int 
     auto target = [&](int c, int64_t& row0, int& cc) {
       const bool over = chain && c >= nchunks && pass + 1 < bpw;
       row0 = over ? n0_next : n0;
-      cc = over ? c - nchunks : (c < nchunks ? c : nchunks - 1);
+      cc = over ? c - nchunks : (c < last_load ? c : last_load);
     };
 
     // RD chunks in registers per tile; a chunk's registers are refilled (RD chunks on) as soon as its last byte has
@@ -314,7 +323,7 @@ __global__ __launch_bounds__(WAVES * 64, 4) void k_tq1_gemv_fp4(GemmArgs a, int 
 #pragma unroll
       for (int s = 0; s < GR; ++s) {
         const int64_t row = row0 + 16 * s < a.N ? row0 + 16 * s : row0;  // a tile past N repeats tile 0 and is not stored
-        W[slot][s][h] = buf_load16(wrs, voff, (unsigned)(row * a.Kp) + 128u * cc + 64u * h);
+        W[slot][s][h] = buf_load16(wrs, voff, (unsigned)(row * a.Kp) + 128u * (unsigned)(cb + cc) + 64u * h);
       }
     };
     // (several tokens: the lane's group of the first window and the one of the second: lg and 3, 4, 2, 2 for lg = 0..3;
@@ -325,13 +334,13 @@ __global__ __launch_bounds__(WAVES * 64, 4) void k_tq1_gemv_fp4(GemmArgs a, int 
       int cc;
       target(c, row0, cc);
       if (PC == 2) {  // the two dwords that hold the scales of the lane's two groups
-        const unsigned at0 = (srow + SB * (unsigned)((5 * cc + g_w0) >> gs)) & ~3u, at1 = (srow + SB * (unsigned)((5 * cc + g_w1) >> gs)) & ~3u;
+        const unsigned at0 = (srow + SB * (unsigned)((5 * (cb + cc) + g_w0) >> gs)) & ~3u, at1 = (srow + SB * (unsigned)((5 * (cb + cc) + g_w1) >> gs)) & ~3u;
         const unsigned wo = (unsigned)(row0 * a.G * SB);
         SQ[0].x = (unsigned)__builtin_amdgcn_raw_buffer_load_b32(srs, (int)at0, (int)wo, 0);
         SQ[0].y = (unsigned)__builtin_amdgcn_raw_buffer_load_b32(srs, (int)at1, (int)wo, 0);
         return;
       }
-      const unsigned at = (srow + SB * (unsigned)((5 * cc + kb) >> gs)) & ~3u;
+      const unsigned at = (srow + SB * (unsigned)((5 * (cb + cc) + kb) >> gs)) & ~3u;
 #pragma unroll
       for (int s = 0; s < GR; ++s) {
         const int64_t row = row0 + 16 * s < a.N ? row0 + 16 * s : row0;
@@ -458,7 +467,7 @@ __global__ __launch_bounds__(WAVES * 64, 4) void k_tq1_gemv_fp4(GemmArgs a, int 
       // the chunk's 5 group sums under their scales. Three pieces: this lane holds group kb (3 pieces) and a piece of
       // group 4, whose scale sits next to that of group 3 in the lanes kb = 3. Several tokens: one group per window.
       const int g_first = PC == 3 ? kb : g_w0;
-      const unsigned ia = (unsigned)((5 * c + g_first) >> gs), ib = (unsigned)((5 * c + (PC == 3 ? g_first + 1 : g_w1)) >> gs);
+      const unsigned ia = (unsigned)((5 * (cb + c) + g_first) >> gs), ib = (unsigned)((5 * (cb + c) + (PC == 3 ? g_first + 1 : g_w1)) >> gs);
 #pragma unroll
       for (int s = 0; s < GR; ++s) {
         unsigned ra, rb;  // the scale of group g_first, and the one after it (bits as stored)
@@ -542,7 +551,7 @@ int f4_cus() {  // compute units of the current device (256 if the query fails)
 }
 
 template <int SDT, int WAVES, int ABL = 0, int NTOK = 1>
-int launch_f4_k(const GemmArgs& a, hipStream_t s, const char* name, int nchunks, size_t lds) {
+int launch_f4_k(const GemmArgs& a, hipStream_t s, const char* name, int nchunks, size_t lds, int seg_chunks = 0) {  // seg_chunks: chunks per launch (0: all)
   static bool attr = false;
   static int cus = 0;
   if (!attr) {
@@ -561,21 +570,29 @@ int launch_f4_k(const GemmArgs& a, hipStream_t s, const char* name, int nchunks,
   bpw = bpw < 1 ? 1 : bpw > blocks ? blocks : bpw;
   const dim3 grid((unsigned)((blocks + bpw - 1) / bpw), (unsigned)a.E, 1u);
   note_kernel(name);
-  hipLaunchKernelGGL((k_tq1_gemv_fp4<SDT, WAVES, ABL, NTOK>), grid, dim3(WAVES * 64), lds, s, a, nchunks, (int)bpw);
-  return check_launch(name);
+  const int per = seg_chunks > 0 ? seg_chunks : nchunks;
+  for (int cb = 0; cb < nchunks; cb += per) {
+    hipLaunchKernelGGL((k_tq1_gemv_fp4<SDT, WAVES, ABL, NTOK>), grid, dim3(WAVES * 64), lds, s, a, nchunks, cb, nchunks - cb < per ? nchunks - cb : per, (int)bpw);
+    const int rc = check_launch(name);
+    if (rc != BP_OK) return rc;
+  }
+  return BP_OK;
 }
 
 template <int SDT, int NTOK>
 int launch_f4(const GemmArgs& a, hipStream_t s) {
   const int64_t nchunks = (a.K + 639) / 640;
-  const size_t lds = (size_t)(F4_LUT_BYTES + NTOK * nchunks * f4_chunk_bytes(NTOK));
-  if (lds > (size_t)F4_LDS_MAX) return BP_ERR_UNSUPPORTED;
+  // several tokens: K in as many equal segments as make the tokens' tiles of one segment fit beside the table
+  const int64_t fit = (F4_LDS_MAX - F4_LUT_BYTES) / (NTOK * f4_chunk_bytes(NTOK));
+  const int64_t nseg = NTOK == 1 ? 1 : (nchunks + fit - 1) / fit, seg = (nchunks + nseg - 1) / nseg;
+  const size_t lds = (size_t)(F4_LUT_BYTES + NTOK * seg * f4_chunk_bytes(NTOK));
+  if (lds > (size_t)F4_LDS_MAX || nseg > 4) return BP_ERR_UNSUPPORTED;
   static const int cus = f4_cus();
   const int64_t experts = a.E < a.T ? a.E : a.T;
   if (NTOK > 1) {
     const bool wide = lds > (size_t)F4_LDS_MAX / 2 || ((a.N + 255) / 256) * experts >= 4 * (int64_t)cus;
-    if (!wide) return launch_f4_k<SDT, 8, 0, NTOK>(a, s, NTOK == 2 ? "fp4_tq1_m2_w8" : NTOK == 4 ? "fp4_tq1_m4_w8" : NTOK == 6 ? "fp4_tq1_m6_w8" : "fp4_tq1_m8_w8", (int)nchunks, lds);
-    return launch_f4_k<SDT, 16, 0, NTOK>(a, s, NTOK == 2 ? "fp4_tq1_m2_w16" : NTOK == 4 ? "fp4_tq1_m4_w16" : NTOK == 6 ? "fp4_tq1_m6_w16" : "fp4_tq1_m8_w16", (int)nchunks, lds);
+    if (!wide) return launch_f4_k<SDT, 8, 0, NTOK>(a, s, NTOK == 2 ? "fp4_tq1_m2_w8" : NTOK == 4 ? "fp4_tq1_m4_w8" : NTOK == 6 ? "fp4_tq1_m6_w8" : "fp4_tq1_m8_w8", (int)nchunks, lds, (int)seg);
+    return launch_f4_k<SDT, 16, 0, NTOK>(a, s, NTOK == 2 ? "fp4_tq1_m2_w16" : NTOK == 4 ? "fp4_tq1_m4_w16" : NTOK == 6 ? "fp4_tq1_m6_w16" : "fp4_tq1_m8_w16", (int)nchunks, lds, (int)seg);
   }
   if (const char* t = getenv("BP_TUNE_F4ABL")) {  // development: timing ablations (one token)
     if (SDT == BP_F16 && atoi(t) == 1) return launch_f4_k<BP_F16, 8, 1>(a, s, "abl1_fp4", (int)nchunks, lds);
@@ -618,11 +635,11 @@ int launch_tq1_gemv_fp4(const GemmArgs& a, hipStream_t s) {
     if (a.scale_dtype == BP_F16) return launch_f4<BP_F16, 4>(a, s);
     if (a.scale_dtype == BP_BF16) return launch_f4<BP_BF16, 4>(a, s);
     if (a.scale_dtype == BP_F32) return launch_f4<BP_F32, 4>(a, s);
-  } else if (a.max_rows <= 6) {  // (6 tiles fit beside the table for K <= 5760)
+  } else if (a.max_rows <= 6) {
     if (a.scale_dtype == BP_F16) return launch_f4<BP_F16, 6>(a, s);
     if (a.scale_dtype == BP_BF16) return launch_f4<BP_BF16, 6>(a, s);
     if (a.scale_dtype == BP_F32) return launch_f4<BP_F32, 6>(a, s);
-  } else {  // (8 tiles fit beside the table for K <= 4480)
+  } else {
     if (a.scale_dtype == BP_F16) return launch_f4<BP_F16, 8>(a, s);
     if (a.scale_dtype == BP_BF16) return launch_f4<BP_BF16, 8>(a, s);
     if (a.scale_dtype == BP_F32) return launch_f4<BP_F32, 8>(a, s);

@@ -169,8 +169,8 @@ def test_tq1_gemv_fp8_pieces_keep_small_activations(bp, act):
 @pytest.mark.parametrize("counts", [[2, 0, 5], [16, 3, 1], [20, 1, 37]])
 def test_tq1_mfma_tiles(bp, K, counts, act):
     got, want, kern = _run(bp, "tq1", 3, 80, K, counts, act, terms=2, seed=K + sum(counts))
-    # (up to 6 / 8 rows per expert go to the fp8 x fp4 kernel while their operand tiles fit beside its table: K <= 5760 / 4480)
-    assert kern.startswith("fp4_tq1_m6" if max(counts) <= 6 and K <= 5760 else "mfma_tq1"), kern
+    # (up to 8 rows per expert go to the fp8 x fp4 kernel)
+    assert kern.startswith("fp4_tq1_m6" if max(counts) <= 6 else "mfma_tq1"), kern
     _check(got, want)
 
 
@@ -178,23 +178,31 @@ def test_tq1_mfma_tiles(bp, K, counts, act):
 @pytest.mark.parametrize("K", [1024, 2048, 5120, 7168])
 @pytest.mark.parametrize("counts", [[2, 0, 1], [2, 2, 2], [4, 3, 1], [3, 0, 0], [8, 5, 1], [1, 6, 7], [5, 6, 0]])
 def test_tq1_fp4_small_batches(bp, K, counts, act):
-    """2, up to 4 and (K <= 5760 / 4480) up to 6 / 8 token rows per expert: one operand tile per token (two fp8 pieces), one matrix
-    instruction per token pair; experts with fewer rows than the launch's variant holds leave rows of the operand unused."""
+    """Up to 2, 4, 6, 8 token rows per expert: one operand tile per token (two fp8 pieces), one matrix instruction per
+    token pair; experts with fewer rows than the launch's variant holds leave rows of the operand unused. Where the
+    tiles of all of K do not fit in LDS (K = 5120 with 8 tokens, K = 7168 with 6 or 8) K is cut into segments, one
+    launch each."""
     got, want, kern = _run(bp, "tq1", 3, 80, K, counts, act, terms=2, seed=K + 7 * sum(counts))
     m = max(counts)
-    want_kernel = "fp4_tq1_m2" if m <= 2 else "fp4_tq1_m4" if m <= 4 else "fp4_tq1_m6" if m <= 6 and K <= 5760 else "fp4_tq1_m8" if K <= 4480 else "mfma_tq1"
+    want_kernel = "fp4_tq1_m2" if m <= 2 else "fp4_tq1_m4" if m <= 4 else "fp4_tq1_m6" if m <= 6 else "fp4_tq1_m8"
     assert kern.startswith(want_kernel), kern
     _check(got, want)
 
 
 def test_tq1_small_batches_other_kernels(bp, monkeypatch):
-    """fp16 activations (11 significant bits: more than two fp8 pieces hold) and rows of K whose 4 tiles x 26 chunks
-    do not fit beside the table go to the kernels they went to before; the development switch keeps the multi-row
-    MFMA kernel."""
+    """fp16 activations (11 significant bits: more than two fp8 pieces hold) and K that would take more than 4 segments
+    go to the kernels they went to before; the development switch keeps the multi-row MFMA kernel. K = 16384 with 4
+    tokens runs as two segments of 13 chunks, with 8 tokens as four of 7 (the last one 5)."""
     got, want, kern = _run(bp, "tq1", 3, 80, 2048, [2, 4, 1], "f16", seed=21)
     assert not kern.startswith("fp4_tq1"), kern
     _check(got, want)
     got, want, kern = _run(bp, "tq1", 2, 32, 16384, [4, 2], "bf16", seed=22)
+    assert kern.startswith("fp4_tq1_m4"), kern
+    _check(got, want)
+    got, want, kern = _run(bp, "tq1", 2, 32, 16384, [8, 3], "int8", seed=24)
+    assert kern.startswith("fp4_tq1_m8"), kern
+    _check(got, want)
+    got, want, kern = _run(bp, "tq1", 2, 32, 20480, [7, 8], "bf16", seed=25)  # 32 chunks: 5 segments of 7
     assert not kern.startswith("fp4_tq1"), kern
     _check(got, want)
     monkeypatch.setenv("BP_TUNE_TQ1", "mfma")
