@@ -100,7 +100,7 @@ __device__ __forceinline__ int f4_pair_byte(int j, int kbA, int hf) {
 // tokens' pieces of one group per window. 8 matrix instructions per chunk and token pair; with two pairs the ring
 // of loads is two chunks (registers; the loads are not what a wave then waits for).
 template <int SDT, int WAVES, int ABL = 0, int NTOK = 1>
-__global__ __launch_bounds__(WAVES * 64, 4) void k_tq1_gemv_fp4(GemmArgs a, int total_chunks, int first_chunk, int nchunks, int bpw /* row blocks per workgroup */) {
+__global__ __launch_bounds__(WAVES * 64, 4) void k_tq1_gemv_fp4(GemmArgs a, int total_chunks, int first_chunk, int nchunks, int bpw /* row blocks per workgroup */, int first_row) {
   constexpr int THREADS = WAVES * 64, GR = F4_GR, RD = NTOK <= 2 ? F4_RD : 2, BD = F4_BD, AD = F4_AD, PAIRS = NTOK <= 2 ? F4_PAIRS : 0;
   static_assert(!PAIRS || RD % 2 == 0, "pairs of chunks need an even ring");
   static_assert(NTOK == 1 || (GR == 1 && AD == 0 && NTOK % 2 == 0), "several tokens: one tile per wave, one operand A buffer, token pairs");
@@ -115,9 +115,12 @@ __global__ __launch_bounds__(WAVES * 64, 4) void k_tq1_gemv_fp4(GemmArgs a, int 
   const int r16 = lane & 15, kb = lane >> 4;
   const int64_t e = blockIdx.y;
   const int64_t o0 = clamp_i64(a.offsets[e], 0, a.T), o1 = clamp_i64(a.offsets[e + 1], 0, a.T);
-  if (o0 >= o1) return;  // uniform for the workgroup; the expert's first NTOK token rows are used (max_rows <= NTOK)
-  const int64_t tok = o0;
-  const int ntok = o1 - o0 < NTOK ? (int)(o1 - o0) : NTOK;
+  // A launch takes the expert's token rows first_row .. first_row + NTOK - 1 (one token: its first row); an expert with
+  // more rows than that gets further launches, one without any in this range is done at once (uniform).
+  const int64_t tok = o0 + (NTOK == 1 ? 0 : first_row);
+  if (tok >= o1) return;
+  const int ntok = o1 - tok < NTOK ? (int)(o1 - tok) : NTOK;
+  const int npairs = (ntok + 1) >> 1;  // token pairs the expert has in this launch: the others' matrix instructions are left out
   // the tiles of the NTOK tokens are interleaved chunk by chunk (a pair's tiles are a constant apart)
   auto tile_at = [](int tt, int c) { return AT + (c * NTOK + tt) * F4_CHUNK_BYTES; };
   const int gs = a.group == 256 ? 1 : 0;  // scale groups of 256: two 128-wide work groups share a scale
@@ -283,6 +286,10 @@ __global__ __launch_bounds__(WAVES * 64, 4) void k_tq1_gemv_fp4(GemmArgs a, int 
     const int64_t r = (((int64_t)blockIdx.x * bpw + pass) * WAVES + wave) * (16 * GR);
     return r < a.N ? r : 0;
   };
+  // (the whole loop nest once per number of token pairs the expert has in this launch, chosen outside it: a branch
+  // around the absent pairs' matrix instructions inside the chunk loop cost 18-43 spilled registers)
+  auto all_terms = [&](auto npr_c) {
+  constexpr int NPR = decltype(npr_c)::value;  // token pairs processed
   for (int term = 0; term < a.n_terms; ++term) {
     // the expert's rows as a buffer that ends with the tensor; dword-aligned base, per-lane row offset. A block
     // starts a multiple of 16 rows = of 4 bytes further on, so the misalignment is the same for all blocks.
@@ -442,7 +449,7 @@ __global__ __launch_bounds__(WAVES * 64, 4) void k_tq1_gemv_fp4(GemmArgs a, int 
           const unsigned lo_at = (((ao >> (16 * (j & 1))) & 0xffu) << 4) + cbase + lane_tok;
           const unsigned hi_at = (((ao >> (16 * (j & 1) + 8)) & 0xffu) << 4) + cbase + lane_tok;
 #pragma unroll
-          for (int pr = 0; pr < NP; ++pr) {
+          for (int pr = 0; pr < NPR; ++pr) {
             __builtin_amdgcn_sched_barrier(0);
             const u32x4 alo = *(const lds_u32x4*)(lo_at + 2 * pr * F4_CHUNK_BYTES), ahi = *(const lds_u32x4*)(hi_at + 2 * pr * F4_CHUNK_BYTES);
             const i32x8 A = {(int)alo.x, (int)alo.y, (int)alo.z, (int)alo.w, (int)ahi.x, (int)ahi.y, (int)ahi.z, (int)ahi.w};
@@ -492,7 +499,7 @@ __global__ __launch_bounds__(WAVES * 64, 4) void k_tq1_gemv_fp4(GemmArgs a, int 
         } else {  // (one row tile per wave: s == 0)
           const float sb = SDT == BP_F32 ? __uint_as_float(rb) : SDT == BP_F16 ? f16_bits_to_f32((uint16_t)rb) : __uint_as_float(rb << 16);
 #pragma unroll
-          for (int tt = 0; tt < NTOK; ++tt) {  // rows 4 lg + 2 (tt % 2) + p of the pair's two tiles
+          for (int tt = 0; tt < 2 * NPR; ++tt) {  // rows 4 lg + 2 (tt % 2) + p of the pair's two tiles
             const unsigned ivb = cbase + (unsigned)(tt * F4_CHUNK_BYTES) + F4_INV_OFF;
             const float inv_a = __uint_as_float(*(const lds_u32*)(ivb + 4 * g_w0)), inv_b = __uint_as_float(*(const lds_u32*)(ivb + 4 * g_w1));
             const f32x4 c0 = C[2 * (tt >> 1)], c1 = C[2 * (tt >> 1) + 1];
@@ -543,6 +550,11 @@ __global__ __launch_bounds__(WAVES * 64, 4) void k_tq1_gemv_fp4(GemmArgs a, int 
   }
   }  // pass
   }  // term
+  };
+  if (NP >= 2 && npairs == 1) all_terms(IC<1>{});
+  else if (NP >= 3 && npairs == 2) all_terms(IC<(NP >= 3 ? 2 : NP)>{});
+  else if (NP >= 4 && npairs == 3) all_terms(IC<(NP >= 4 ? 3 : NP)>{});
+  else all_terms(IC<NP>{});
 }
 int f4_cus() {  // compute units of the current device (256 if the query fails)
   int dev = 0, cus = 0;
@@ -551,7 +563,7 @@ int f4_cus() {  // compute units of the current device (256 if the query fails)
 }
 
 template <int SDT, int WAVES, int ABL = 0, int NTOK = 1>
-int launch_f4_k(const GemmArgs& a, hipStream_t s, const char* name, int nchunks, size_t lds, int seg_chunks = 0) {  // seg_chunks: chunks per launch (0: all)
+int launch_f4_k(const GemmArgs& a, hipStream_t s, const char* name, int nchunks, size_t lds, int seg_chunks = 0 /* chunks per launch (0: all) */, int first_row = 0) {
   static bool attr = false;
   static int cus = 0;
   if (!attr) {
@@ -572,7 +584,7 @@ int launch_f4_k(const GemmArgs& a, hipStream_t s, const char* name, int nchunks,
   note_kernel(name);
   const int per = seg_chunks > 0 ? seg_chunks : nchunks;
   for (int cb = 0; cb < nchunks; cb += per) {
-    hipLaunchKernelGGL((k_tq1_gemv_fp4<SDT, WAVES, ABL, NTOK>), grid, dim3(WAVES * 64), lds, s, a, nchunks, cb, nchunks - cb < per ? nchunks - cb : per, (int)bpw);
+    hipLaunchKernelGGL((k_tq1_gemv_fp4<SDT, WAVES, ABL, NTOK>), grid, dim3(WAVES * 64), lds, s, a, nchunks, cb, nchunks - cb < per ? nchunks - cb : per, (int)bpw, first_row);
     const int rc = check_launch(name);
     if (rc != BP_OK) return rc;
   }
@@ -580,7 +592,7 @@ int launch_f4_k(const GemmArgs& a, hipStream_t s, const char* name, int nchunks,
 }
 
 template <int SDT, int NTOK>
-int launch_f4(const GemmArgs& a, hipStream_t s) {
+int launch_f4(const GemmArgs& a, hipStream_t s, int first_row = 0) {
   const int64_t nchunks = (a.K + 639) / 640;
   // several tokens: K in as many equal segments as make the tokens' tiles of one segment fit beside the table
   const int64_t fit = (F4_LDS_MAX - F4_LUT_BYTES) / (NTOK * f4_chunk_bytes(NTOK));
@@ -591,8 +603,8 @@ int launch_f4(const GemmArgs& a, hipStream_t s) {
   const int64_t experts = a.E < a.T ? a.E : a.T;
   if (NTOK > 1) {
     const bool wide = lds > (size_t)F4_LDS_MAX / 2 || ((a.N + 255) / 256) * experts >= 4 * (int64_t)cus;
-    if (!wide) return launch_f4_k<SDT, 8, 0, NTOK>(a, s, NTOK == 2 ? "fp4_tq1_m2_w8" : NTOK == 4 ? "fp4_tq1_m4_w8" : NTOK == 6 ? "fp4_tq1_m6_w8" : "fp4_tq1_m8_w8", (int)nchunks, lds, (int)seg);
-    return launch_f4_k<SDT, 16, 0, NTOK>(a, s, NTOK == 2 ? "fp4_tq1_m2_w16" : NTOK == 4 ? "fp4_tq1_m4_w16" : NTOK == 6 ? "fp4_tq1_m6_w16" : "fp4_tq1_m8_w16", (int)nchunks, lds, (int)seg);
+    if (!wide) return launch_f4_k<SDT, 8, 0, NTOK>(a, s, NTOK == 2 ? "fp4_tq1_m2_w8" : NTOK == 4 ? "fp4_tq1_m4_w8" : NTOK == 6 ? "fp4_tq1_m6_w8" : "fp4_tq1_m8_w8", (int)nchunks, lds, (int)seg, first_row);
+    return launch_f4_k<SDT, 16, 0, NTOK>(a, s, NTOK == 2 ? "fp4_tq1_m2_w16" : NTOK == 4 ? "fp4_tq1_m4_w16" : NTOK == 6 ? "fp4_tq1_m6_w16" : "fp4_tq1_m8_w16", (int)nchunks, lds, (int)seg, first_row);
   }
   if (const char* t = getenv("BP_TUNE_F4ABL")) {  // development: timing ablations (one token)
     if (SDT == BP_F16 && atoi(t) == 1) return launch_f4_k<BP_F16, 8, 1>(a, s, "abl1_fp4", (int)nchunks, lds);
@@ -614,36 +626,44 @@ int launch_f4(const GemmArgs& a, hipStream_t s) {
 
 }  // namespace
 
-// One token row per expert, or up to 2 / 4 / 6 / 8 (two fp8 pieces per activation) while the tiles fit in LDS.
+// One token row per expert, or up to 2 / 4 / 6 / 8 (two fp8 pieces per activation), or - when most experts have few
+// rows (T <= 4 E) - up to 32 as launches of 8 rows each and the rest: an expert costs what its own rows cost (and
+// nothing in a launch whose rows it does not have), so a launch in which a few experts have many rows, or whose
+// max_rows is only an upper bound, is not held to that pace.
 // BP_ERR_UNSUPPORTED (no message): the caller falls back to its other kernels.
+namespace {
+template <int SDT>
+int launch_f4_rows(const GemmArgs& a, hipStream_t s, int64_t rows, int first_row) {
+  if (rows <= 1 && first_row == 0) return launch_f4<SDT, 1>(a, s);
+  if (rows <= 2) return launch_f4<SDT, 2>(a, s, first_row);
+  if (rows <= 4) return launch_f4<SDT, 4>(a, s, first_row);
+  if (rows <= 6) return launch_f4<SDT, 6>(a, s, first_row);
+  return launch_f4<SDT, 8>(a, s, first_row);
+}
+template <int SDT>
+int launch_f4_any(const GemmArgs& a, hipStream_t s) {
+  for (int64_t first = 0; first < a.max_rows; first += 8) {
+    const int rc = launch_f4_rows<SDT>(a, s, a.max_rows - first < 8 ? a.max_rows - first : 8, (int)first);
+    if (rc != BP_OK) return rc;
+  }
+  return BP_OK;
+}
+}  // namespace
+
 int launch_tq1_gemv_fp4(const GemmArgs& a, hipStream_t s) {
   if (a.x_dtype != BP_BF16 && a.x_dtype != BP_F16 && a.x_dtype != BP_I8) return BP_ERR_UNSUPPORTED;
   if (a.max_rows > 1 && a.x_dtype == BP_F16) return BP_ERR_UNSUPPORTED;  // (11 significant bits need the third piece)
-  if (a.max_rows < 1 || a.max_rows > 8) return BP_ERR_UNSUPPORTED;
+  if (a.max_rows < 1 || a.max_rows > 32 || (a.max_rows > 8 && a.T > 4 * a.E)) return BP_ERR_UNSUPPORTED;
   if (a.N % 16 != 0 || a.Kp != (a.K + 4) / 5 || (a.group != 128 && a.group != 256)) return BP_ERR_UNSUPPORTED;
   for (int t = 0; t < a.n_terms; ++t)
     if (a.scale_dtype == BP_F32 && ((uintptr_t)a.w_scale[t] & 3) != 0) return BP_ERR_UNSUPPORTED;
-  if (a.max_rows == 1) {
-    if (a.scale_dtype == BP_F16) return launch_f4<BP_F16, 1>(a, s);
-    if (a.scale_dtype == BP_BF16) return launch_f4<BP_BF16, 1>(a, s);
-    if (a.scale_dtype == BP_F32) return launch_f4<BP_F32, 1>(a, s);
-  } else if (a.max_rows == 2) {
-    if (a.scale_dtype == BP_F16) return launch_f4<BP_F16, 2>(a, s);
-    if (a.scale_dtype == BP_BF16) return launch_f4<BP_BF16, 2>(a, s);
-    if (a.scale_dtype == BP_F32) return launch_f4<BP_F32, 2>(a, s);
-  } else if (a.max_rows <= 4) {
-    if (a.scale_dtype == BP_F16) return launch_f4<BP_F16, 4>(a, s);
-    if (a.scale_dtype == BP_BF16) return launch_f4<BP_BF16, 4>(a, s);
-    if (a.scale_dtype == BP_F32) return launch_f4<BP_F32, 4>(a, s);
-  } else if (a.max_rows <= 6) {
-    if (a.scale_dtype == BP_F16) return launch_f4<BP_F16, 6>(a, s);
-    if (a.scale_dtype == BP_BF16) return launch_f4<BP_BF16, 6>(a, s);
-    if (a.scale_dtype == BP_F32) return launch_f4<BP_F32, 6>(a, s);
-  } else {
-    if (a.scale_dtype == BP_F16) return launch_f4<BP_F16, 8>(a, s);
-    if (a.scale_dtype == BP_BF16) return launch_f4<BP_BF16, 8>(a, s);
-    if (a.scale_dtype == BP_F32) return launch_f4<BP_F32, 8>(a, s);
+  if (a.max_rows > 8) {  // (both launches must be possible before the first one adds to the output)
+    const int64_t nchunks = (a.K + 639) / 640, fit = (F4_LDS_MAX - F4_LUT_BYTES) / (8 * f4_chunk_bytes(8));
+    if ((nchunks + fit - 1) / fit > 4) return BP_ERR_UNSUPPORTED;
   }
+  if (a.scale_dtype == BP_F16) return launch_f4_any<BP_F16>(a, s);
+  if (a.scale_dtype == BP_BF16) return launch_f4_any<BP_BF16>(a, s);
+  if (a.scale_dtype == BP_F32) return launch_f4_any<BP_F32>(a, s);
   return BP_ERR_UNSUPPORTED;
 }
 

@@ -189,6 +189,17 @@ def test_tq1_fp4_small_batches(bp, K, counts, act):
     _check(got, want)
 
 
+@pytest.mark.parametrize("act", ["bf16", "int8"])
+@pytest.mark.parametrize("K,counts,last", [(2048, [9, 1, 0, 2, 1, 0, 12, 1], "fp4_tq1_m4"), (7168, [1, 16, 0, 3, 2, 1, 1, 5], "fp4_tq1_m8"),
+                                           (4096, [2, 2, 10, 0, 0, 0, 1, 7], "fp4_tq1_m2"), (2048, [27, 0, 1, 0, 0, 0, 1, 3], "fp4_tq1_m4")])
+def test_tq1_fp4_few_large_experts(bp, K, counts, last, act):
+    """Up to 16 rows in a few experts while most have few (T <= 4 E): a launch for every expert's first 8 rows and one
+    for the rest; experts with fewer rows than a launch's variant holds run the loop nest of their own pair count."""
+    got, want, kern = _run(bp, "tq1", len(counts), 48, K, counts, act, terms=2, seed=K + 3)
+    assert kern.startswith(last), kern
+    _check(got, want)
+
+
 def test_tq1_small_batches_other_kernels(bp, monkeypatch):
     """fp16 activations (11 significant bits: more than two fp8 pieces hold) and K that would take more than 4 segments
     go to the kernels they went to before; the development switch keeps the multi-row MFMA kernel. K = 16384 with 4
