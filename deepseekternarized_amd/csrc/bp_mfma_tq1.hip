@@ -406,7 +406,7 @@ int launch_mfma_tq1(const GemmArgs& a, hipStream_t s, int waves) {
     if (waves == 16) return launch_tq1_v<16, 1>(a, s, "mfma_tq1_bf16_t1_w16", "mfma_tq1_bf16_t1_w16_gs");
     return launch_tq1_v<8, 1>(a, s, "mfma_tq1_bf16_t1_w8", "mfma_tq1_bf16_t1_w8_gs");
   }
-  if (a.max_rows <= 32) {  // small decode batches: the fp8 x fp4 kernel with one operand tile per token
+  if (a.max_rows <= 64) {  // small decode batches: the fp8 x fp4 kernel with one operand tile per token
     const char* t = getenv("BP_TUNE_TQ1");  // development: "mfma" / "lut" keep this kernel
     if (!(t && (t[0] == 'm' || t[0] == 'l'))) {
       const int rc = launch_tq1_gemv_fp4(a, s);

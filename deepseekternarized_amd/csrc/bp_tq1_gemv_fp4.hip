@@ -627,7 +627,7 @@ int launch_f4(const GemmArgs& a, hipStream_t s, int first_row = 0) {
 }  // namespace
 
 // One token row per expert, or up to 2 / 4 / 6 / 8 (two fp8 pieces per activation), or - when most experts have few
-// rows (T <= 4 E) - up to 32 as launches of 8 rows each and the rest: an expert costs what its own rows cost (and
+// rows (T <= 4 E) - up to 64 as launches of 8 rows each and the rest: an expert costs what its own rows cost (and
 // nothing in a launch whose rows it does not have), so a launch in which a few experts have many rows, or whose
 // max_rows is only an upper bound, is not held to that pace.
 // BP_ERR_UNSUPPORTED (no message): the caller falls back to its other kernels.
@@ -653,7 +653,7 @@ int launch_f4_any(const GemmArgs& a, hipStream_t s) {
 int launch_tq1_gemv_fp4(const GemmArgs& a, hipStream_t s) {
   if (a.x_dtype != BP_BF16 && a.x_dtype != BP_F16 && a.x_dtype != BP_I8) return BP_ERR_UNSUPPORTED;
   if (a.max_rows > 1 && a.x_dtype == BP_F16) return BP_ERR_UNSUPPORTED;  // (11 significant bits need the third piece)
-  if (a.max_rows < 1 || a.max_rows > 32 || (a.max_rows > 8 && a.T > 4 * a.E)) return BP_ERR_UNSUPPORTED;
+  if (a.max_rows < 1 || a.max_rows > 64 || (a.max_rows > 8 && a.T > 4 * a.E)) return BP_ERR_UNSUPPORTED;
   if (a.N % 16 != 0 || a.Kp != (a.K + 4) / 5 || (a.group != 128 && a.group != 256)) return BP_ERR_UNSUPPORTED;
   for (int t = 0; t < a.n_terms; ++t)
     if (a.scale_dtype == BP_F32 && ((uintptr_t)a.w_scale[t] & 3) != 0) return BP_ERR_UNSUPPORTED;

@@ -44,8 +44,9 @@ def _activations(rng, T, K, act):
     return x, None, dev(x), None
 
 
-def _run(bp, fmt, E, N, K, counts, act, terms=1, seed=0, misalign_scales=False, scale_dtype=np.float16, group=GROUP):
-    """Grouped call with `counts[e]` rows per expert; returns (got, want, kernel name)."""
+def _run(bp, fmt, E, N, K, counts, act, terms=1, seed=0, misalign_scales=False, scale_dtype=np.float16, group=GROUP, max_rows=None):
+    """Grouped call with `counts[e]` rows per expert; returns (got, want, kernel name). `max_rows`: offsets on the
+    device and that upper bound, as a caller that does not read the counts back passes them."""
     rng = np.random.default_rng(seed)
     packed, scales = synth_weights(seed, E, N, K, group, fmt, terms=terms)
     offsets = np.concatenate([[0], np.cumsum(counts)]).astype(np.int64)
@@ -79,7 +80,10 @@ def _run(bp, fmt, E, N, K, counts, act, terms=1, seed=0, misalign_scales=False, 
             moved.append(flat[2:].view(s.shape))
             assert moved[-1].data_ptr() % 16 == 4
         sc = moved
-    got = bp.grouped_ternary_gemm(xd, xsd, offsets.tolist(), pk, sc, K, group, fmt)  # host offsets: max_rows = widest expert
+    if max_rows is None:
+        got = bp.grouped_ternary_gemm(xd, xsd, offsets.tolist(), pk, sc, K, group, fmt)  # host offsets: max_rows = widest expert
+    else:
+        got = bp.grouped_ternary_gemm(xd, xsd, torch.from_numpy(offsets).cuda(), pk, sc, K, group, fmt, max_rows=max_rows)
     return got.cpu().numpy(), want, bp.ext().last_kernel()
 
 
@@ -197,6 +201,18 @@ def test_tq1_fp4_few_large_experts(bp, K, counts, last, act):
     for the rest; experts with fewer rows than a launch's variant holds run the loop nest of their own pair count."""
     got, want, kern = _run(bp, "tq1", len(counts), 48, K, counts, act, terms=2, seed=K + 3)
     assert kern.startswith(last), kern
+    _check(got, want)
+
+
+def test_tq1_fp4_upper_bound_max_rows(bp):
+    """max_rows as an upper bound (64 for a decode step of 64 tokens) with offsets on the device: 8 launches of 8 rows,
+    most of them without any row to take."""
+    counts = [3, 0, 1, 11, 2, 0, 0, 1, 2, 5, 1, 1, 0, 2, 1, 1, 4, 0, 2, 1]
+    got, want, kern = _run(bp, "tq1", len(counts), 48, 2048, counts, "bf16", terms=2, seed=31, max_rows=64)
+    assert kern.startswith("fp4_tq1_m6"), kern  # (the bound is capped at the 38 rows of the call: 4 launches of 8 rows and one of 6)
+    _check(got, want)
+    got, want, kern = _run(bp, "tq1", 3, 48, 2048, [30, 1, 2], "bf16", seed=32, max_rows=33)  # T > 4 E
+    assert kern.startswith("mfma_tq1"), kern
     _check(got, want)
 
 
