@@ -36,7 +36,7 @@ GROUP = 128
 
 # HBM bytes per launch measured with rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE on this command line (each
 # counter scaled by what it reads for a plain 1 GiB device copy); the summaries are under profiles/.
-MEASURED_TRAFFIC_BYTES = {"cfg1a_tq1_gemv": 522049229, "cfg1a_tq2_gemv": 516034150, "cfg1a_tq2_i8_gemv": 508708761}
+MEASURED_TRAFFIC_BYTES = {"cfg1a_tq1_gemv": 522121318, "cfg1a_tq2_gemv": 516034150, "cfg1a_tq2_i8_gemv": 508708761}
 
 WORKLOADS = {
     # name: (fmt, N, K, M tokens per linear, activation, terms, L linears per launch)
