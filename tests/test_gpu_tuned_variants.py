@@ -126,6 +126,15 @@ def test_tq1_gemv_many_rows_two_terms_bf16_scales(bp, gemv_kernel):
     _check(got, want)
 
 
+def test_tq1_fp4_small_batches_many_rows_bf16_scales(bp):
+    """The small-batch variants over several workgroups and row blocks (N not a multiple of their rows), bf16 scales,
+    int8 activations with their per-row scales."""
+    for counts, act, want_kernel in [([2, 1], "bf16", "fp4_tq1_m2"), ([3, 4], "int8", "fp4_tq1_m4"), ([8, 5], "bf16", "fp4_tq1_m8")]:
+        got, want, kern = _run(bp, "tq1", 2, 2048 + 48, 2304, counts, act, terms=2, seed=6, scale_dtype=np.float32)
+        assert kern.startswith(want_kernel), kern
+        _check(got, want)
+
+
 def test_tq1_gemv_scales_from_global_memory(bp, monkeypatch):
     """Table kernel: scale pointers that are not 16-byte aligned, and K with more groups than the LDS tile takes."""
     monkeypatch.setenv("BP_TUNE_TQ1", "lut")
@@ -309,7 +318,8 @@ def test_tq2_gemm_scales_from_global_memory_and_other_scale_dtypes(bp):
 # --------------------------------------------------------------------------- float32 scales (TQ1)
 @pytest.mark.parametrize("act", ["bf16", "int8"])
 @pytest.mark.parametrize("K,counts,prefix", [(2048, [1, 0, 1], "fp4_tq1"), (7168, [1, 1, 1], "fp4_tq1"), (2048, [3, 16, 1], "mfma_tq1"),
-                                              (7168, [20, 2, 9], "mfma_tq1")])
+                                              (7168, [20, 2, 9], "mfma_tq1"), (2048, [2, 1, 0], "fp4_tq1_m2"), (7168, [3, 4, 1], "fp4_tq1_m4"),
+                                              (7168, [7, 0, 5], "fp4_tq1_m8"), (2304, [12, 0, 0], "fp4_tq1_m4")])
 def test_tq1_float32_scales(bp, act, K, counts, prefix):
     """boilerplate/kernels/ternary_cuda.py:95-97 hands the kernel `w_scale.float()`: the tuned TQ1 kernels take it."""
     got, want, kern = _run(bp, "tq1", 3, 272, K, counts, act, terms=2, seed=K + len(act), scale_dtype="f32")
@@ -373,7 +383,8 @@ def test_moe_layer_graph_replays_match_eager(bp, fmt, act, tokens):
 @pytest.mark.parametrize("fmt,K,counts,prefix", [
     ("tq2", 2048, [1, 0, 1], "mfma_tq2"), ("tq2", 7168, [16, 2, 5], "mfma_tq2"), ("tq2", 3072, [40, 1, 20], "gemm_tq2"),
     ("tq1", 2048, [1, 1, 0], "fp4_tq1"), ("tq1", 7168, [1, 0, 1], "fp4_tq1"), ("tq1", 7168, [9, 16, 2], "mfma_tq1"),
-    ("tq1", 2560, [3, 0, 20], "mfma_tq1"),
+    ("tq1", 2560, [3, 0, 20], "mfma_tq1"), ("tq1", 2048, [2, 2, 1], "fp4_tq1_m2"), ("tq1", 7168, [4, 0, 3], "fp4_tq1_m4"),
+    ("tq1", 7168, [1, 6, 5], "fp4_tq1_m6"), ("tq1", 2560, [1, 0, 11], "fp4_tq1_m4"),
 ])
 def test_group_256(bp, act, fmt, K, counts, prefix):
     """configs/policy/std_absmean_tq{1,2}_g256.yaml: one scale per 256 weights; the tuned kernels treat it as two 128-wide groups."""
