@@ -323,10 +323,12 @@ def cfg2_weights(bp):
     return trits, scale, packed
 
 
-@pytest.mark.parametrize("T", [1, 32, 256])
-def test_config2_grouped_tq1_full_shape_sampled(bp, cfg2_weights, T):
+@pytest.mark.parametrize("T,bound", [(1, None), (32, None), (32, 32), (40, 40), (256, None)])
+def test_config2_grouped_tq1_full_shape_sampled(bp, cfg2_weights, T, bound):
     """64 experts, gate projection 2048 x 4096 TQ1, top-6 skewed routing; every routed row checked on a
-    sample of output columns against the float64 oracle (the full oracle product would take minutes)."""
+    sample of output columns against the float64 oracle (the full oracle product would take minutes).
+    `bound`: max_rows as the MoE layer passes it for a few tokens (the token count, an upper bound on the widest
+    expert's rows, so that nothing is read back): the call then runs as launches of 8 rows per expert."""
     from deepseekternarized_amd.kernels.ternary_hip import gather_rows
 
     E, N, K, group, k, fmt = 64, 2048, 4096, 128, 6, "tq1"
@@ -336,7 +338,9 @@ def test_config2_grouped_tq1_full_shape_sampled(bp, cfg2_weights, T):
     _, idx = _route(rng, T, E, k)
     order, offsets = bp.sort_by_expert(dev(idx.reshape(-1)), E)
     xg = gather_rows(bf16_dev(x), order, k)
-    got = bp.grouped_ternary_gemm(xg, None, offsets, packed, dev(scale), K, group, fmt).cpu().numpy()
+    got = bp.grouped_ternary_gemm(xg, None, offsets, packed, dev(scale), K, group, fmt, max_rows=bound).cpu().numpy()
+    if bound is not None:
+        assert bp.ext().last_kernel().startswith("fp4_tq1_m"), bp.ext().last_kernel()
     worder, woffsets = orc.sort_by_expert(idx.reshape(-1), E)
     assert np.array_equal(order.cpu().numpy(), worder)
     cols = rng.choice(N, 48, replace=False)
