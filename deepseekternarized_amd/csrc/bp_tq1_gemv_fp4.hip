@@ -653,7 +653,9 @@ int launch_f4_any(const GemmArgs& a, hipStream_t s) {
 int launch_tq1_gemv_fp4(const GemmArgs& a, hipStream_t s) {
   if (a.x_dtype != BP_BF16 && a.x_dtype != BP_F16 && a.x_dtype != BP_I8) return BP_ERR_UNSUPPORTED;
   if (a.max_rows > 1 && a.x_dtype == BP_F16) return BP_ERR_UNSUPPORTED;  // (11 significant bits need the third piece)
-  if (a.max_rows < 1 || a.max_rows > 64 || (a.max_rows > 8 && a.T > 4 * a.E)) return BP_ERR_UNSUPPORTED;
+  int64_t few = 4;  // "most experts have few rows": at most this many routed rows per expert on average
+  if (const char* t = getenv("BP_TUNE_F4T")) few = atoi(t);  // (development)
+  if (a.max_rows < 1 || a.max_rows > 64 || (a.max_rows > 8 && a.T > few * a.E)) return BP_ERR_UNSUPPORTED;
   if (a.N % 16 != 0 || a.Kp != (a.K + 4) / 5 || (a.group != 128 && a.group != 256)) return BP_ERR_UNSUPPORTED;
   for (int t = 0; t < a.n_terms; ++t)
     if (a.scale_dtype == BP_F32 && ((uintptr_t)a.w_scale[t] & 3) != 0) return BP_ERR_UNSUPPORTED;
