@@ -102,16 +102,26 @@ class Launch:
             torch.cuda.synchronize()
         for _ in range(warmup):
             self()
-        ev = [(torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)) for _ in range(steps)]
-        torch.cuda.synchronize()
-        t0 = time.perf_counter()
-        for a, b in ev:
-            a.record()
-            self()
-            b.record()
-        torch.cuda.synchronize()
-        wall = (time.perf_counter() - t0) / steps
-        kern = sum(a.elapsed_time(b) for a, b in ev) / steps / 1e3
+        # The boxes show an occasional stall of ~30 ms in the middle of back-to-back launches (about one per several
+        # seconds, whatever the kernel). A timed sequence in which one launch took more than 20 x the median launch
+        # is taken again, once; `self.retimed` says so.
+        self.retimed = 0
+        for attempt in range(2):
+            ev = [(torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)) for _ in range(steps)]
+            torch.cuda.synchronize()
+            t0 = time.perf_counter()
+            for a, b in ev:
+                a.record()
+                self()
+                b.record()
+            torch.cuda.synchronize()
+            wall = (time.perf_counter() - t0) / steps
+            each = sorted(a.elapsed_time(b) for a, b in ev)
+            if attempt == 0 and steps >= 5 and each[-1] > 20.0 * each[len(each) // 2]:
+                self.retimed = 1
+                continue
+            break
+        kern = sum(each) / steps / 1e3
         return wall, kern, self.e.last_kernel()
 
 
@@ -215,6 +225,7 @@ def main() -> int:
     fmt, N, K, M, act, terms, L = WORKLOADS[a.workload]
     launch, wbytes = uniform_launch(bp, torch, fmt, N, K, M, act, terms, L)
     wall, kern, kname = launch.time(a.steps, a.warmup)
+    retimed = launch.retimed
     act_bytes = L * M * K * 2 + L * M * N * 4 * 2  # bf16 activations read, f32 output read-modify-write
 
     also = {}
@@ -350,7 +361,7 @@ def main() -> int:
         "dtype": "bf16", "data": "synthetic",
         "config": {"workload": f"{a.workload}: {fmt.upper()} decode GEMV N={N} K={K} M={M} {act} activations, group 128, "
                                f"fp16 scales, {L} distinct linears per launch ({wbytes / 1e6:.0f} MB of weights, > Infinity Cache)",
-                   "kernel": kname, "bytes_counted": "packed + fp16 scales as stored", "device_spin_up_s": SPIN_UP_S,
+                   "kernel": kname, "bytes_counted": "packed + fp16 scales as stored", "device_spin_up_s": SPIN_UP_S, "retimed_after_stall": retimed,
                    "packed_only_GBps": round(wbytes * (1.0 - 2.0 * (K // GROUP) / (bp.packed_cols(fmt, K) + 2.0 * (K // GROUP))) / kern / 1e9, 1),
                    "activation_and_output_bytes_per_step": act_bytes},
         "roofline": {"bound": "hbm", "achieved": round(wbytes / kern / 1e9, 1), "peak": HBM_PEAK_GBPS, "unit": "GB/s",
