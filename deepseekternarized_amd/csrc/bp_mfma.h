@@ -26,7 +26,8 @@ int launch_mfma_tq1(const GemmArgs& a, hipStream_t s, int waves);
 int launch_gemm_tq2(const GemmArgs& a, hipStream_t s);
 // bp_tq1_gemv.hip: TQ1, one token row per expert (max_rows == 1), bf16 activations, table-lookup GEMV
 int launch_tq1_gemv(const GemmArgs& a, hipStream_t s, int waves);
-// bp_tq1_gemv_fp4.hip: the same through the fp8 x fp4 matrix instruction (16-bit and int8 activations);
+// bp_tq1_gemv_fp4.hip: the same through the fp8 x fp4 matrix instruction (16-bit and int8 activations), and small
+// batches: up to 8 token rows per expert, or up to 64 in launches of 8 when the experts average at most 4 rows;
 // BP_ERR_UNSUPPORTED without a message when the call is outside its preconditions
 int launch_tq1_gemv_fp4(const GemmArgs& a, hipStream_t s);
 

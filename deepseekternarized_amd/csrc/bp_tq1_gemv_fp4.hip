@@ -1,4 +1,5 @@
-// TQ1 single-token GEMV (decode, one token row per expert) on the block-float matrix instruction
+// TQ1 decode GEMV (one token row per expert; small batches of up to 8 rows per expert and launch: NTOK below) on the
+// block-float matrix instruction
 // v_mfma_f32_16x16x128_f8f6f4, weights as fp4 (E2M1 holds -1, 0, +1 exactly), activations as fp8 (E4M3) pieces.
 //
 // Contract as everywhere (boilerplate/kernels/ternary_cuda.py:58-63): out[n] += sum_g scale[n, g] * sum_{k in g}
