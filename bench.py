@@ -48,6 +48,8 @@ WORKLOADS = {
     "cfg1b_tq1_gemv": ("tq1", 7168, 2048, 1, "bf16", 1, 128),
     "cfg1a_tq1_m2": ("tq1", 2048, 7168, 2, "bf16", 1, 128),
     "cfg1a_tq1_m4": ("tq1", 2048, 7168, 4, "bf16", 1, 128),
+    "cfg1a_tq1_m16": ("tq1", 2048, 7168, 16, "bf16", 1, 128),
+    "cfg1a_tq2_m16": ("tq2", 2048, 7168, 16, "bf16", 1, 128),
     "cfg1a_tq2_gemv": ("tq2", 2048, 7168, 1, "bf16", 1, 128),
     "cfg0_tq2_gemv": ("tq2", 2048, 4096, 1, "bf16", 1, 192),
     "cfg1a_tq2_i8_gemv": ("tq2", 2048, 7168, 1, "int8", 1, 128),
