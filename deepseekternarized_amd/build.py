@@ -1,6 +1,6 @@
 """Builds libbp_ternary_hip.so (the gfx950 kernels and their C ABI) in-tree with hipcc.
 
-    python -m deepseekternarized_amd.build
+    python -m deepseekternarized_amd.build [--incremental]
 
 The shared object lands next to this file; it is what ``deepseekternarized_amd.kernels.ternary_hip``
 loads with ctypes. hipcc cross-compiles for gfx950 without a GPU present.
@@ -58,9 +58,21 @@ def _compile(src: str) -> Path:
     return obj
 
 
-def build(verbose: bool = True) -> Path:
+def _fresh(src: str) -> bool:
+    """The object of `src` is newer than the source and every header (used by --incremental only)."""
+    obj = CSRC / (src + ".o")
+    if not obj.exists():
+        return False
+    deps = [CSRC / src, *CSRC.glob("*.h"), HERE.parent / "include" / "bp_ternary.h", Path(__file__)]
+    return all(obj.stat().st_mtime > d.stat().st_mtime for d in deps)
+
+
+def build(verbose: bool = True, incremental: bool = False) -> Path:
+    """Compiles every source (``incremental``: only those older than their inputs) and links the library."""
+    todo = [s for s in SOURCES if not (incremental and _fresh(s))]
     with ThreadPoolExecutor(max_workers=7) as pool:
-        objs = list(pool.map(_compile, SOURCES))
+        list(pool.map(_compile, todo))
+    objs = [CSRC / (s + ".o") for s in SOURCES]
     cmd = ["hipcc", "--offload-arch=gfx950", "-shared", "-fPIC", *map(str, objs), "-o", str(LIB)]
     res = subprocess.run(cmd, capture_output=True, text=True)
     if res.returncode != 0:
@@ -71,4 +83,4 @@ def build(verbose: bool = True) -> Path:
 
 
 if __name__ == "__main__":
-    build()
+    build(incremental="--incremental" in sys.argv[1:])

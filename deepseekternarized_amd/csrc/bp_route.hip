@@ -1,13 +1,26 @@
 // Token-to-expert routing kernels around the grouped GEMM: stable counting sort of expert ids,
 // row gather (the x[order // k] permute), and the two elementwise stages of an expert MLP
 // (SwiGLU, weighted combine) with the reference engine's bf16 rounding points.
+#include <mutex>
+
 #include "bp_common.h"
+
+// Histograms of bp_sort_by_expert_static: device memory that belongs to the library (one copy per GPU the library
+// runs on, held until the process ends), so that entry point needs no workspace and allocates nothing. In host code
+// the name `scratch` is only a stand-in: the array's device address is looked up once per device (g_scratch_ptr).
+static __device__ __align__(256) int32_t scratch[16 * BP_SORT_STATIC_MAX_EXPERTS];  // 16 waves x E counters: 4 MiB
 
 namespace bp {
 namespace {
 
+constexpr int64_t SORT_STATIC_MAX_E = BP_SORT_STATIC_MAX_EXPERTS;
+constexpr int SORT_MAX_DEVICES = 64;
+std::mutex g_scratch_mutex;
+int32_t* g_scratch_ptr[SORT_MAX_DEVICES] = {};
+
 constexpr int SORT_THREADS = 1024;
 constexpr int SORT_WAVES = SORT_THREADS / 64;
+static_assert(SORT_WAVES == 16, "the static histogram array is sized for 16 waves");
 constexpr int64_t SORT_LDS_INTS = 32768;  // 128 KiB of per-wave histograms in LDS
 
 // One workgroup. Wave w owns the contiguous segment [w*seg, (w+1)*seg) of ids.
@@ -226,26 +239,54 @@ extern "C" int64_t bp_sort_workspace_ints(int64_t n, int64_t E) {
   return SORT_WAVES * E <= SORT_LDS_INTS ? 0 : SORT_WAVES * E;
 }
 
+static int launch_sort(int64_t* order, int64_t* offsets, const int64_t* ids, int64_t n, int64_t E, int32_t* hist_mem,
+                       int32_t* bad, hipStream_t stream) {
+  if (n <= SORT_SMALL_N && E < ((int64_t)1 << 24)) {
+    hipLaunchKernelGGL(k_sort_small, dim3(1), dim3(SORT_SMALL_THREADS), 0, stream, order, offsets, ids, (int)n, E, bad);
+    return check_launch("sort_by_expert");
+  }
+  const size_t lds = hist_mem ? 0 : (size_t)(SORT_WAVES * (E > 0 ? E : 1)) * sizeof(int32_t);
+  static std::once_flag attr_once;
+  static hipError_t attr_rc = hipSuccess;
+  std::call_once(attr_once, [] {
+    attr_rc = hipFuncSetAttribute((const void*)k_sort, hipFuncAttributeMaxDynamicSharedMemorySize, (int)(SORT_LDS_INTS * 4));
+  });
+  if (attr_rc != hipSuccess) return fail(BP_ERR_LAUNCH, "cannot raise the dynamic LDS limit for sort_by_expert");
+  hipLaunchKernelGGL(k_sort, dim3(1), dim3(SORT_THREADS), lds, stream, order, offsets, ids, n, E, hist_mem, bad);
+  return check_launch("sort_by_expert");
+}
+
 extern "C" int bp_sort_by_expert(int64_t* order, int64_t* offsets, const int64_t* ids, int64_t n, int64_t E,
                                  int32_t* workspace, int32_t* bad, void* stream) {
   if (n < 0 || E < 0 || E > ((int64_t)1 << 24) || n > ((int64_t)1 << 31) - 1) return fail(BP_ERR_ARG, "invalid n or E");
   if (!offsets || (n > 0 && (!order || !ids))) return fail(BP_ERR_ARG, "null pointer");
   const int64_t need = bp_sort_workspace_ints(n, E);
   if (need > 0 && !workspace) return fail(BP_ERR_ARG, "sort_by_expert needs a workspace for this many experts");
-  if (n <= SORT_SMALL_N && E < ((int64_t)1 << 24)) {
-    hipLaunchKernelGGL(k_sort_small, dim3(1), dim3(SORT_SMALL_THREADS), 0, (hipStream_t)stream, order, offsets, ids, (int)n, E, bad);
-    return check_launch("sort_by_expert");
+  return launch_sort(order, offsets, ids, n, E, need > 0 ? workspace : (int32_t*)nullptr, bad, (hipStream_t)stream);
+}
+
+extern "C" int bp_sort_by_expert_static(int64_t* order, int64_t* offsets, const int64_t* ids, int64_t n, int64_t E,
+                                        int32_t* bad, void* stream) {
+  if (n < 0 || E < 0 || n > ((int64_t)1 << 31) - 1) return fail(BP_ERR_ARG, "invalid n or E");
+  if (E > SORT_STATIC_MAX_E)
+    return fail(BP_ERR_ARG, "bp_sort_by_expert_static takes at most %lld experts (its histograms live in a fixed device array); "
+                            "use bp_sort_by_expert with a workspace", (long long)SORT_STATIC_MAX_E);
+  if (!offsets || (n > 0 && (!order || !ids))) return fail(BP_ERR_ARG, "null pointer");
+  int32_t* hist_mem = nullptr;
+  if (bp_sort_workspace_ints(n, E) > 0 && n > SORT_SMALL_N) {  // (otherwise the histograms fit in LDS, or none are used)
+    int dev = 0;
+    if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= SORT_MAX_DEVICES) return fail(BP_ERR_LAUNCH, "cannot identify the current device");
+    std::lock_guard<std::mutex> lock(g_scratch_mutex);
+    if (!g_scratch_ptr[dev]) {  // each GPU holds its own copy of the array at its own address
+      void* p = nullptr;
+      const hipError_t rc = hipGetSymbolAddress(&p, HIP_SYMBOL(scratch));
+      if (rc != hipSuccess || !p) return fail(BP_ERR_LAUNCH, "hipGetSymbolAddress(scratch): %s", hipGetErrorString(rc));
+      g_scratch_ptr[dev] = (int32_t*)p;
+    }
+    hist_mem = g_scratch_ptr[dev];
   }
-  const size_t lds = need > 0 ? 0 : (size_t)(SORT_WAVES * (E > 0 ? E : 1)) * sizeof(int32_t);
-  static bool attr_set = false;
-  if (!attr_set) {
-    if (hipFuncSetAttribute((const void*)k_sort, hipFuncAttributeMaxDynamicSharedMemorySize, (int)(SORT_LDS_INTS * 4)) != hipSuccess)
-      return fail(BP_ERR_LAUNCH, "cannot raise the dynamic LDS limit for sort_by_expert");
-    attr_set = true;
-  }
-  hipLaunchKernelGGL(k_sort, dim3(1), dim3(SORT_THREADS), lds, (hipStream_t)stream, order, offsets, ids, n, E,
-                     need > 0 ? workspace : (int32_t*)nullptr, bad);
-  return check_launch("sort_by_expert");
+  // the kernel zero-fills the SORT_WAVES * E counters it uses before counting: nothing of an earlier call is read
+  return launch_sort(order, offsets, ids, n, E, hist_mem, bad, (hipStream_t)stream);
 }
 
 extern "C" int bp_gather_rows(void* dst, const void* src, const int64_t* index, int64_t divisor, int64_t rows,

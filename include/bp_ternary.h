@@ -116,6 +116,17 @@ int64_t bp_sort_workspace_ints(int64_t n, int64_t E);
 int bp_sort_by_expert(int64_t* order, int64_t* offsets, const int64_t* ids, int64_t n, int64_t E,
                       int32_t* workspace, int32_t* bad, void* stream);
 
+/* bp_sort_by_expert without a workspace argument and without any allocation. It has no counterpart in the
+ * reference; it is for callers that cannot allocate device memory (code under HIP graph capture, tight serving
+ * loops, harnesses that forbid hipMalloc). The per-wave histograms that bp_sort_by_expert takes as `workspace`
+ * live in a fixed 4 MiB device array inside the library (one per GPU, held until the process ends), so E is limited
+ * to BP_SORT_STATIC_MAX_EXPERTS (more: BP_ERR_ARG). Results are identical to bp_sort_by_expert's. All calls on
+ * one GPU share that array: calls that overlap in time on one GPU (different streams) race; calls on one
+ * stream are ordered and each clears the counters it uses itself. */
+#define BP_SORT_STATIC_MAX_EXPERTS 65536
+int bp_sort_by_expert_static(int64_t* order, int64_t* offsets, const int64_t* ids, int64_t n, int64_t E,
+                             int32_t* bad, void* stream);
+
 /* Row gather dst[i, :] = src[index[i] / divisor, :] (the x[order // k] permute of
  * scripts/eval/ternary_kernel_bench.py:90-93). row_bytes must be a multiple of 2. */
 int bp_gather_rows(void* dst, const void* src, const int64_t* index, int64_t divisor, int64_t rows,
