@@ -413,6 +413,13 @@ int launch_mfma_tq1(const GemmArgs& a, hipStream_t s, int waves) {
       if (rc != BP_ERR_UNSUPPORTED) return rc;
     }
   }
+  {  // more rows per expert: token tiles of 32 on the fp8 x fp4 matrix instruction
+    const char* t = getenv("BP_TUNE_TQ1");  // development: "mfma" keeps the 16-token kernel below
+    if (!(t && t[0] == 'm')) {
+      const int rc = launch_gemm_tq1(a, s);
+      if (rc != BP_ERR_UNSUPPORTED) return rc;
+    }
+  }
   if (waves == 16) return launch_tq1_v<16, 4>(a, s, "mfma_tq1_bf16_m1_w16", "mfma_tq1_bf16_m1_w16_gs");
   return launch_tq1_v<8, 4>(a, s, "mfma_tq1_bf16_m1_w8", "mfma_tq1_bf16_m1_w8_gs");
 }

@@ -1,4 +1,4 @@
-"""Every code path of the tuned kernels (bp_mfma_tq2.hip, bp_gemm_tq2.hip, bp_mfma_tq1.hip, bp_tq1_gemv.hip) against the CPU oracle.
+"""Every code path of the tuned kernels (bp_mfma_tq2.hip, bp_gemm_tq2.hip, bp_mfma_tq1.hip, bp_gemm_tq1.hip, bp_tq1_gemv.hip, bp_tq1_gemv_fp4.hip) against the CPU oracle.
 
 The shapes are chosen by what they select inside the launchers, not by size: odd / even packed row
 lengths (row starts at every byte alignment), K that fits one activation / table tile or needs several,
@@ -176,15 +176,65 @@ def test_tq1_gemv_fp8_pieces_keep_small_activations(bp, act):
     assert torch.equal(got, torch.zeros_like(got))
 
 
-# --------------------------------------------------------------------------- TQ1 MFMA kernel (2..16 rows per tile)
+# --------------------------------------------------------------------------- TQ1 grouped GEMM (token tiles of 32) and the 16-token MFMA kernel
+@pytest.fixture(params=["gemm", "mfma"])
+def tq1_rows_kernel(request, monkeypatch):
+    """More than 8 rows per expert: the fp8 x fp4 grouped GEMM; BP_TUNE_TQ1=mfma keeps the older 16-token kernel covered."""
+    if request.param == "mfma":
+        monkeypatch.setenv("BP_TUNE_TQ1", "mfma")
+    else:
+        monkeypatch.delenv("BP_TUNE_TQ1", raising=False)
+    return request.param + "_tq1"
+
+
 @pytest.mark.parametrize("act", ["bf16", "int8"])
 @pytest.mark.parametrize("K", [1024, 2048, 7168])
 @pytest.mark.parametrize("counts", [[2, 0, 5], [16, 3, 1], [20, 1, 37]])
-def test_tq1_mfma_tiles(bp, K, counts, act):
+def test_tq1_mfma_tiles(bp, K, counts, act, tq1_rows_kernel):
     got, want, kern = _run(bp, "tq1", 3, 80, K, counts, act, terms=2, seed=K + sum(counts))
-    # (up to 8 rows per expert go to the fp8 x fp4 kernel)
-    assert kern.startswith("fp4_tq1_m6" if max(counts) <= 6 else "mfma_tq1"), kern
+    # (up to 8 rows per expert go to the small-batch fp8 x fp4 kernel)
+    assert kern.startswith(tq1_rows_kernel if max(counts) > 6 or tq1_rows_kernel == "mfma_tq1" else "fp4_tq1_m6"), kern
     _check(got, want)
+
+
+@pytest.mark.parametrize("act", ["bf16", "int8"])
+@pytest.mark.parametrize(
+    "E,N,K,counts,terms",
+    [
+        (3, 80, 1280, [33, 0, 64], 1),          # Kp = 256: every row dword-aligned; exactly two chunks; full 32-token tiles and a 1-token one
+        (5, 528, 2048, [20, 1, 37, 9, 32], 2),   # two row blocks, the second with 16 of its 512 rows; Kp = 410: rows at two byte alignments
+        (11, 48, 4096, [17] * 11, 1),            # more experts than XCDs and not a multiple of 8; 7 chunks, the last one with 2 groups (its second window is skipped)
+        (2, 1040, 7168, [48, 31], 1),            # config-1 K: 12 chunks, the last one with a single group; three row blocks
+        (3, 64, 1024, [9, 100, 15], 2),          # the smallest K the tuned kernels take; four token tiles in one expert
+    ],
+)
+def test_tq1_gemm_tiles(bp, act, E, N, K, counts, terms):
+    got, want, kern = _run(bp, "tq1", E, N, K, counts, act, terms=terms, seed=K + N)
+    assert kern.startswith("gemm_tq1"), kern
+    _check(got, want)
+
+
+@pytest.mark.parametrize("ntok", [9, 16, 32])
+def test_tq1_gemm_fp8_pieces_keep_small_activations(bp, ntok):
+    """The grouped GEMM splits an activation into two E4M3 pieces under a power-of-two scale per block of 20: exact for
+    bf16 values down to 2^-9 of the block's largest magnitude. Activations spread over 5 decades with outliers 1000 x
+    the typical value must still come out far inside the general tolerance."""
+    rng = np.random.default_rng(13)
+    E, N, K = 2, 64, 4352
+    packed, scales = synth_weights(13, E, N, K, GROUP, "tq1")
+    T = E * ntok
+    x = rng.standard_normal((T, K)).astype(np.float32) * np.exp(rng.uniform(-6, 6, (T, K))).astype(np.float32)
+    x[:, ::97] *= 1000.0
+    x = orc.bf16_round(x)
+    want = np.zeros((T, N), np.float32)
+    for e in range(E):
+        c_gemm(x[e * ntok:(e + 1) * ntok], None, packed[0][e], scales[0][e].astype(np.float32), K, GROUP, "tq1", out=want[e * ntok:(e + 1) * ntok])
+    got = bp.grouped_ternary_gemm(dev(x).to(torch.bfloat16), None, [0, ntok, 2 * ntok], [dev(packed[0])], [dev(scales[0])], K, GROUP, "tq1").cpu().numpy()
+    assert bp.ext().last_kernel().startswith("gemm_tq1")
+    assert rel_l2(got, want) <= 2e-4, rel_l2(got, want)
+    z = np.zeros_like(x)  # all-zero activations: the block scale has nothing to go by
+    got = bp.grouped_ternary_gemm(dev(z).to(torch.bfloat16), None, [0, ntok, 2 * ntok], [dev(packed[0])], [dev(scales[0])], K, GROUP, "tq1")
+    assert torch.equal(got, torch.zeros_like(got))
 
 
 @pytest.mark.parametrize("act", ["bf16", "int8"])
@@ -221,7 +271,7 @@ def test_tq1_fp4_upper_bound_max_rows(bp):
     assert kern.startswith("fp4_tq1_m6"), kern  # (the bound is capped at the 38 rows of the call: 4 launches of 8 rows and one of 6)
     _check(got, want)
     got, want, kern = _run(bp, "tq1", 3, 48, 2048, [30, 1, 2], "bf16", seed=32, max_rows=33)  # T > 4 E
-    assert kern.startswith("mfma_tq1"), kern
+    assert kern.startswith("gemm_tq1"), kern
     _check(got, want)
 
 
@@ -253,7 +303,11 @@ def test_tq1_fp4_small_batches_misaligned_scales(bp):
     _check(got, want)
 
 
-def test_tq1_mfma_scales_from_global_memory(bp):
+def test_tq1_mfma_scales_from_global_memory(bp, monkeypatch):
+    got, want, kern = _run(bp, "tq1", 2, 32, 2048, [9, 4], "bf16", seed=8, misalign_scales=True)
+    assert kern.startswith("gemm_tq1"), kern
+    _check(got, want)
+    monkeypatch.setenv("BP_TUNE_TQ1", "mfma")
     got, want, kern = _run(bp, "tq1", 2, 32, 2048, [9, 4], "bf16", seed=8, misalign_scales=True)
     assert kern.startswith("mfma_tq1") and kern.endswith("_gs"), kern
     _check(got, want)
@@ -317,8 +371,8 @@ def test_tq2_gemm_scales_from_global_memory_and_other_scale_dtypes(bp):
 
 # --------------------------------------------------------------------------- float32 scales (TQ1)
 @pytest.mark.parametrize("act", ["bf16", "int8"])
-@pytest.mark.parametrize("K,counts,prefix", [(2048, [1, 0, 1], "fp4_tq1"), (7168, [1, 1, 1], "fp4_tq1"), (2048, [3, 16, 1], "mfma_tq1"),
-                                              (7168, [20, 2, 9], "mfma_tq1"), (2048, [2, 1, 0], "fp4_tq1_m2"), (7168, [3, 4, 1], "fp4_tq1_m4"),
+@pytest.mark.parametrize("K,counts,prefix", [(2048, [1, 0, 1], "fp4_tq1"), (7168, [1, 1, 1], "fp4_tq1"), (2048, [3, 16, 1], "gemm_tq1"),
+                                              (7168, [20, 2, 9], "gemm_tq1"), (2048, [2, 1, 0], "fp4_tq1_m2"), (7168, [3, 4, 1], "fp4_tq1_m4"),
                                               (7168, [7, 0, 5], "fp4_tq1_m8"), (2304, [12, 0, 0], "fp4_tq1_m4")])
 def test_tq1_float32_scales(bp, act, K, counts, prefix):
     """boilerplate/kernels/ternary_cuda.py:95-97 hands the kernel `w_scale.float()`: the tuned TQ1 kernels take it."""
@@ -382,8 +436,8 @@ def test_moe_layer_graph_replays_match_eager(bp, fmt, act, tokens):
 @pytest.mark.parametrize("act", ["bf16", "int8"])
 @pytest.mark.parametrize("fmt,K,counts,prefix", [
     ("tq2", 2048, [1, 0, 1], "mfma_tq2"), ("tq2", 7168, [16, 2, 5], "mfma_tq2"), ("tq2", 3072, [40, 1, 20], "gemm_tq2"),
-    ("tq1", 2048, [1, 1, 0], "fp4_tq1"), ("tq1", 7168, [1, 0, 1], "fp4_tq1"), ("tq1", 7168, [9, 16, 2], "mfma_tq1"),
-    ("tq1", 2560, [3, 0, 20], "mfma_tq1"), ("tq1", 2048, [2, 2, 1], "fp4_tq1_m2"), ("tq1", 7168, [4, 0, 3], "fp4_tq1_m4"),
+    ("tq1", 2048, [1, 1, 0], "fp4_tq1"), ("tq1", 7168, [1, 0, 1], "fp4_tq1"), ("tq1", 7168, [9, 16, 2], "gemm_tq1"),
+    ("tq1", 2560, [3, 0, 20], "gemm_tq1"), ("tq1", 2048, [2, 2, 1], "fp4_tq1_m2"), ("tq1", 7168, [4, 0, 3], "fp4_tq1_m4"),
     ("tq1", 7168, [1, 6, 5], "fp4_tq1_m6"), ("tq1", 2560, [1, 0, 11], "fp4_tq1_m4"),
 ])
 def test_group_256(bp, act, fmt, K, counts, prefix):
