@@ -9,8 +9,9 @@ operator called without a HIP device or without the built library raises.
 from .kernels.ternary_hip import (ext, grouped_ternary_gemm, sort_by_expert, ternary_gemm,  # noqa: F401
                                   ternary_gemm_float, ternary_gemm_ref)
 from .ternary.ops import PackedTerm, TernaryLinear, quant_act_int8  # noqa: F401
+from .ternary.fit import TernaryTerm, absmean_ternary, packed_term  # noqa: F401
 from .ternary.pack import (FORMATS, bits_per_weight, pack, packed_cols, tq1_lut, unpack)  # noqa: F401
 
 __all__ = ["ext", "ternary_gemm", "ternary_gemm_float", "ternary_gemm_ref", "grouped_ternary_gemm",
            "sort_by_expert", "PackedTerm", "TernaryLinear", "quant_act_int8", "FORMATS", "bits_per_weight",
-           "pack", "unpack", "packed_cols", "tq1_lut"]
+           "pack", "unpack", "packed_cols", "tq1_lut", "TernaryTerm", "absmean_ternary", "packed_term"]

@@ -75,11 +75,27 @@ class TernaryCheckpoint:
         return m
 
     # ------------------------------------------------------------------ tensors
+    def _contained(self, fname: str) -> Path:
+        """``root / fname`` for a file name that comes from the checkpoint itself (manifest, shard index), or
+        ValueError: no absolute or drive paths, no backslashes, no ``.`` / ``..`` / empty components, and - after
+        resolving symlinks - nothing outside the checkpoint directory (the rules of ``checkpoint_path``,
+        boilerplate/checkpoint/paths.py:6-22)."""
+        from pathlib import PurePosixPath, PureWindowsPath
+
+        if (not isinstance(fname, str) or not fname or "\x00" in fname or "\\" in fname or PurePosixPath(fname).is_absolute()
+                or PureWindowsPath(fname).drive or any(part in (".", "..", "") for part in fname.split("/"))):
+            raise ValueError(f"unsafe checkpoint path: {fname!r}")
+        root = self.root.resolve()
+        path = (root / fname).resolve()
+        if not path.is_relative_to(root):
+            raise ValueError(f"checkpoint path escapes its directory: {fname!r}")
+        return path
+
     def _open(self, fname: str):
         if fname not in self._handles:
             from safetensors import safe_open
 
-            self._handles[fname] = safe_open(str(self.root / fname), framework="pt", device="cpu")
+            self._handles[fname] = safe_open(str(self._contained(fname)), framework="pt", device="cpu")
         return self._handles[fname]
 
     def _locate(self, name: str, stored: dict | None) -> str:

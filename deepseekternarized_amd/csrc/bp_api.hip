@@ -3,6 +3,7 @@
 // device-to-host copy), kernel selection, and the thread-local error/kernel-name plumbing.
 #include <cstdarg>
 #include <cstdio>
+#include <cstdlib>
 #include <cstring>
 
 #include "bp_common.h"
@@ -27,6 +28,26 @@ void note_kernel(const char* name) {
   g_kernel[sizeof(g_kernel) - 1] = 0;
 }
 
+namespace {
+Tuning g_tuning = {0, 0, 0, 0, -1, 0};
+std::once_flag g_tuning_once;
+void read_tuning() {
+  Tuning t = {0, 0, 0, 0, -1, 0};
+  if (const char* v = getenv("BP_TUNE_R")) t.r = atoi(v);
+  if (const char* v = getenv("BP_TUNE_WAVES")) t.waves = atoi(v);
+  if (const char* v = getenv("BP_TUNE_TQ1")) t.tq1 = v[0];
+  if (const char* v = getenv("BP_TUNE_F4W")) t.f4w = atoi(v);
+  if (const char* v = getenv("BP_TUNE_F4T")) t.f4t = atoi(v);
+  if (const char* v = getenv("BP_TUNE_CPT")) t.cpt = atoi(v);
+  g_tuning = t;
+}
+}  // namespace
+
+const Tuning& tuning() {
+  std::call_once(g_tuning_once, read_tuning);
+  return g_tuning;
+}
+
 int check_launch(const char* what) {
   const hipError_t e = hipGetLastError();
   if (e != hipSuccess) return fail(BP_ERR_LAUNCH, "%s: %s", what, hipGetErrorString(e));
@@ -39,6 +60,11 @@ using namespace bp;
 extern "C" const char* bp_last_error(void) { return g_error; }
 extern "C" const char* bp_last_kernel(void) { return g_kernel; }
 extern "C" const char* bp_version(void) { return "bp_ternary_hip gfx950"; }
+
+extern "C" void bp_reload_tuning(void) {
+  tuning();  // (the first read has happened)
+  read_tuning();
+}
 
 extern "C" int bp_set_kernel_policy(int policy) {
   const int old = g_policy;

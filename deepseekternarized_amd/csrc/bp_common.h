@@ -4,6 +4,8 @@
 #include <hip/hip_runtime.h>
 #include <stdint.h>
 
+#include <mutex>
+
 #include "../../include/bp_ternary.h"
 
 namespace bp {
@@ -24,6 +26,34 @@ struct GemmArgs {
   int x_dtype, scale_dtype, n_terms, fmt;
   int64_t T, N, K, Kp, G, group, E, max_rows;
 };
+
+// Development overrides of the kernel selection (environment variables BP_TUNE_*), read once when the library is first
+// used; bp_reload_tuning() reads them again (the tests switch kernels that way). 0 / unset = automatic.
+struct Tuning {
+  int r;       // BP_TUNE_R: 16-row tiles per wave of the TQ2 kernel (1, 2)
+  int waves;   // BP_TUNE_WAVES: waves per workgroup (8, 16)
+  char tq1;    // BP_TUNE_TQ1: 'l' table-lookup GEMV, 'm' 16-token MFMA kernel (first letter of the value)
+  int f4w;     // BP_TUNE_F4W: waves per workgroup of the fp8 x fp4 GEMV (8, 16)
+  int f4t;     // BP_TUNE_F4T: routed rows per expert up to which launches of 8 rows are used (-1 = default)
+  int cpt;     // BP_TUNE_CPT: chunks per table pass of the table-lookup GEMV
+};
+const Tuning& tuning();
+
+// Raises a kernel's dynamic LDS limit, once per device and kernel (thread-safe).
+template <auto Kernel>
+int raise_lds_limit(int bytes) {
+  static std::mutex m;
+  static bool done[64] = {};
+  int dev = 0;
+  if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64) return fail(BP_ERR_LAUNCH, "cannot identify the current device");
+  std::lock_guard<std::mutex> lock(m);
+  if (!done[dev]) {
+    const hipError_t rc = hipFuncSetAttribute((const void*)Kernel, hipFuncAttributeMaxDynamicSharedMemorySize, bytes);
+    if (rc != hipSuccess) return fail(BP_ERR_LAUNCH, "cannot raise the dynamic LDS limit of a kernel: %s", hipGetErrorString(rc));
+    done[dev] = true;
+  }
+  return BP_OK;
+}
 
 int launch_general(const GemmArgs& a, hipStream_t s);
 // Returns BP_ERR_UNSUPPORTED (without setting an error message) when the shape is outside the

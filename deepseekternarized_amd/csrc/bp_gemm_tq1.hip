@@ -461,12 +461,7 @@ __global__ __launch_bounds__(Q_THREADS, 2) void k_gemm_tq1(GemmArgs a) {
 
 template <int ACT, int SDT>
 int launch_gemm_tq1_k(const GemmArgs& a, hipStream_t s, const char* name) {
-  static bool attr = false;
-  if (!attr) {
-    const hipError_t rc = hipFuncSetAttribute((const void*)k_gemm_tq1<ACT, SDT>, hipFuncAttributeMaxDynamicSharedMemorySize, q_lds_bytes(SDT == BP_F32 ? 4 : 2));
-    if (rc != hipSuccess) return fail(BP_ERR_LAUNCH, "cannot raise the dynamic LDS limit of the TQ1 grouped GEMM kernel: %s", hipGetErrorString(rc));
-    attr = true;
-  }
+  if (const int rc = raise_lds_limit<k_gemm_tq1<ACT, SDT>>(q_lds_bytes(SDT == BP_F32 ? 4 : 2))) return rc;
   const int64_t row_blocks = (a.N + Q_ROWS - 1) / Q_ROWS;
   const dim3 grid((unsigned)(row_blocks * ((a.E + 7) / 8 * 8)), 1, (unsigned)((a.max_rows + 31) / 32));
   note_kernel(name);

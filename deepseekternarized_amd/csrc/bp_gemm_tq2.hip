@@ -383,12 +383,7 @@ __global__ __launch_bounds__(GTHREADS, 2) void k_gemm_tq2(GemmArgs a) {
 
 template <int ACT, int SDT, int SL, int ABL = 0>
 int launch_gemm_k(const GemmArgs& a, hipStream_t s, size_t lds, const char* name) {
-  static bool attr = false;
-  if (!attr) {
-    const hipError_t rc = hipFuncSetAttribute((const void*)k_gemm_tq2<ACT, SDT, SL, ABL>, hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
-    if (rc != hipSuccess) return fail(BP_ERR_LAUNCH, "cannot raise the dynamic LDS limit of the grouped GEMM kernel: %s", hipGetErrorString(rc));
-    attr = true;
-  }
+  if (const int rc = raise_lds_limit<k_gemm_tq2<ACT, SDT, SL, ABL>>(160 * 1024)) return rc;
   const dim3 grid((unsigned)((a.N + GROWS - 1) / GROWS * ((a.E + 7) / 8 * 8)), 1, (unsigned)((a.max_rows + 16 * GT - 1) / (16 * GT)));
   note_kernel(name);
   hipLaunchKernelGGL((k_gemm_tq2<ACT, SDT, SL, ABL>), grid, dim3(GTHREADS), lds, s, a);
@@ -409,7 +404,8 @@ int launch_gemm_sd(const GemmArgs& a, hipStream_t s, const char* name, const cha
 
 // Preconditions (checked by mfma_supports): group 128, K % 256 == 0, K >= 1024, N % 16 == 0, 16-byte aligned x / packed / scales.
 int launch_gemm_tq2(const GemmArgs& a, hipStream_t s) {
-  if (const char* t = getenv("BP_TUNE_ABL")) {  // timing experiments: parts of the kernel switched off, results are wrong
+#ifdef BP_DEV_ABLATIONS  // timing ablations (results are wrong): development builds only
+  if (const char* t = getenv("BP_TUNE_ABL")) {
     const size_t lds = 2 * gemm_tile_bytes<BP_BF16>() + (size_t)GROWS * a.G * 2;
     if (a.x_dtype == BP_BF16 && a.scale_dtype == BP_F16 && lds <= 160 * 1024 && a.K % 1024 == 0 && a.group == 128) {
       switch (atoi(t)) {
@@ -423,6 +419,7 @@ int launch_gemm_tq2(const GemmArgs& a, hipStream_t s) {
       }
     }
   }
+#endif
   if (a.x_dtype == BP_BF16) {
     if (a.scale_dtype == BP_F16) return launch_gemm_sd<BP_BF16, BP_F16>(a, s, "gemm_tq2_bf16", "gemm_tq2_bf16_gs");
     if (a.scale_dtype == BP_BF16) return launch_gemm_sd<BP_BF16, BP_BF16>(a, s, "gemm_tq2_bf16", "gemm_tq2_bf16_gs");

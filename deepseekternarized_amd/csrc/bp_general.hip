@@ -177,6 +177,58 @@ int grid_for(int64_t n) {
   return (int)(g < 1 ? 1 : (g > 65535 ? 65535 : g));
 }
 
+// BitNet b1.58 absmean quantizer fused with the packing (boilerplate/ternary/fit.py:78-96, boilerplate/qat/bitlinear.py:75-80):
+// per row and group s = scale_dtype(sum |w| / count) - the sum taken in ascending k, the last group counting its own
+// columns - then trit = s > 0 ? clamp(rint(w / max(s, 1e-30)), -1, 1) : 0, packed in the reference layout (pad digit 1).
+// One workgroup per row: its G scales first (kept in LDS and written out), then its packed bytes.
+constexpr int ABSMEAN_MAX_G = 8192;
+__global__ __launch_bounds__(256) void k_absmean_pack(uint8_t* __restrict__ packed, void* __restrict__ scale, int8_t* __restrict__ trits,
+                                                      const void* __restrict__ w, int w_dtype, int scale_dtype, int64_t K, int64_t Kp,
+                                                      int64_t G, int64_t group, int fmt) {
+  __shared__ float srow[ABSMEAN_MAX_G];
+  const int64_t n = blockIdx.x;
+  const int64_t wrow = n * K;
+  for (int64_t g = threadIdx.x; g < G; g += blockDim.x) {
+    const int64_t k0 = g * group, k1 = k0 + group < K ? k0 + group : K;
+    float sum = 0.f;
+    for (int64_t k = k0; k < k1; ++k) sum += fabsf(load_act_f32(w, w_dtype, wrow + k));
+    const float mean = sum / (float)(k1 - k0);
+    float rounded;
+    if (scale_dtype == BP_F16) {
+      const _Float16 h = (_Float16)mean;
+      ((_Float16*)scale)[n * G + g] = h;
+      rounded = (float)h;
+    } else {
+      const uint16_t b = f32_to_bf16_bits(mean);
+      ((uint16_t*)scale)[n * G + g] = b;
+      rounded = bf16_bits_to_f32(b);
+    }
+    srow[g] = rounded;
+  }
+  __syncthreads();
+  const int per = fmt == BP_TQ2 ? 4 : 5;
+  for (int64_t c = threadIdx.x; c < Kp; c += blockDim.x) {
+    unsigned byte = 0, mul = 1;
+    for (int i = 0; i < per; ++i) {
+      const int64_t k = c * per + i;
+      int t = 0;
+      if (k < K) {
+        const float s = srow[k / group];
+        if (s > 0.f) {
+          float r = rintf(load_act_f32(w, w_dtype, wrow + k) / fmaxf(s, 1e-30f));
+          r = r < -1.f ? -1.f : r > 1.f ? 1.f : r;
+          t = (int)r;  // (a NaN weight compares false twice and converts to 0)
+        }
+        if (trits) trits[wrow + k] = (int8_t)t;
+      }
+      const unsigned u = (unsigned)(t + 1);
+      if (fmt == BP_TQ2) byte |= u << (2 * i);
+      else { byte += u * mul; mul *= 3; }
+    }
+    packed[n * Kp + c] = (uint8_t)byte;
+  }
+}
+
 }  // namespace
 
 int launch_general(const GemmArgs& a, hipStream_t s) {
@@ -246,4 +298,21 @@ extern "C" int bp_quant_act_int8(int8_t* q, float* s, const void* x, int x_dtype
   if (!q || !s || !x) return fail(BP_ERR_ARG, "null pointer");
   hipLaunchKernelGGL(k_quant, dim3((unsigned)M), dim3(256), 0, (hipStream_t)stream, q, s, x, x_dtype, K);
   return check_launch("quant_act_int8");
+}
+
+extern "C" int bp_absmean_pack(uint8_t* packed, void* scale, int scale_dtype, int8_t* trits, const void* w, int w_dtype,
+                               int64_t N, int64_t K, int64_t group, int fmt, void* stream) {
+  int64_t Kp;
+  if (int rc = fmt_dims(fmt, N, K, &Kp)) return rc;
+  if (w_dtype != BP_BF16 && w_dtype != BP_F16 && w_dtype != BP_F32) return fail(BP_ERR_ARG, "weight dtype must be bf16, f16 or f32");
+  if (scale_dtype != BP_F16 && scale_dtype != BP_BF16) return fail(BP_ERR_ARG, "scale_dtype must be float16 or bfloat16");
+  if (group <= 0) return fail(BP_ERR_ARG, "weight must be a matrix with a nonempty input dimension and positive group");
+  const int64_t G = K / group + (K % group != 0);
+  if (G > ABSMEAN_MAX_G) return fail(BP_ERR_ARG, "more than %d scale groups per row", ABSMEAN_MAX_G);
+  if (N > 0x7fffffff) return fail(BP_ERR_ARG, "too many rows");
+  if (N == 0) return BP_OK;
+  if (!packed || !scale || !w) return fail(BP_ERR_ARG, "null pointer");
+  hipLaunchKernelGGL(k_absmean_pack, dim3((unsigned)N), dim3(256), 0, (hipStream_t)stream, packed, scale, trits, w, w_dtype, scale_dtype, K, Kp,
+                     G, group, fmt);
+  return check_launch("absmean_pack");
 }

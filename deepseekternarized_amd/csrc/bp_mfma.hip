@@ -37,8 +37,8 @@ int launch_mfma(const GemmArgs& a, hipStream_t s) {
   // steady state; the TQ2 single-token kernels are light enough on registers for that to win everywhere.
   int waves = work >= 2048 && !(a.fmt == BP_TQ2 && a.max_rows == 1) ? 16 : 8;
   // development overrides (tuning sweeps)
-  if (const char* t = getenv("BP_TUNE_R")) { const int v = atoi(t); if (v == 1 || v == 2) R = v; }
-  if (const char* t = getenv("BP_TUNE_WAVES")) { const int v = atoi(t); if (v == 8 || v == 16) waves = v; }
+  if (tuning().r == 1 || tuning().r == 2) R = tuning().r;
+  if (tuning().waves == 8 || tuning().waves == 16) waves = tuning().waves;
   if (a.fmt == BP_TQ1) return launch_mfma_tq1(a, s, waves);
   // Experts with more than 16 rows get token tiles of 32 - unless the batch is sparse (on average at most 8 rows per
   // expert) and the bound small: then nearly every expert fits one 16-token tile of the lighter kernel, and the few

@@ -347,12 +347,7 @@ template <int SDT, int WAVES, int NQ, int SL, int MULTI, int ABL = 0>
 int launch_tq1_k(const GemmArgs& a, hipStream_t s, const char* name, int64_t cpt, int64_t tokens, size_t lds) {
   const int64_t rows_per_wg = (int64_t)WAVES * 16;
   const dim3 grid((unsigned)((a.N + rows_per_wg - 1) / rows_per_wg), (unsigned)a.E, (unsigned)((a.max_rows + 15) / 16));
-  static bool attr = false;
-  if (!attr) {
-    if (hipFuncSetAttribute((const void*)k_mfma_tq1<SDT, WAVES, NQ, SL, MULTI, ABL>, hipFuncAttributeMaxDynamicSharedMemorySize, T1_LDS_MAX) != hipSuccess)
-      return fail(BP_ERR_LAUNCH, "cannot raise the dynamic LDS limit");
-    attr = true;
-  }
+  if (const int rc = raise_lds_limit<k_mfma_tq1<SDT, WAVES, NQ, SL, MULTI, ABL>>(T1_LDS_MAX)) return rc;
   note_kernel(name);
   hipLaunchKernelGGL((k_mfma_tq1<SDT, WAVES, NQ, SL, MULTI, ABL>), grid, dim3(WAVES * 64), lds, s, a, (int)cpt, (int)tokens);
   return check_launch(name);
@@ -392,30 +387,29 @@ int launch_tq1_v(const GemmArgs& a, hipStream_t s, const char* name_sl, const ch
 }  // namespace
 
 int launch_mfma_tq1(const GemmArgs& a, hipStream_t s, int waves) {
-  if (const char* t = getenv("BP_TUNE_ABL")) {  // development: timing ablations
+#ifdef BP_DEV_ABLATIONS  // timing ablations (results are wrong): development builds only
+  if (const char* t = getenv("BP_TUNE_ABL")) {
     if (atoi(t) == 1) return launch_tq1<BP_F16, 16, 1, 1, 1>(a, s, "abl1_tq1");
     if (atoi(t) == 2) return launch_tq1<BP_F16, 16, 1, 1, 2>(a, s, "abl2_tq1");
     if (atoi(t) == 3) return launch_tq1<BP_F16, 16, 1, 1, 3>(a, s, "abl3_tq1");
     if (atoi(t) == 4) return launch_tq1<BP_F16, 16, 1, 1, 4>(a, s, "abl4_tq1");
     if (atoi(t) == 5) return launch_tq1<BP_F16, 16, 1, 1, 5>(a, s, "abl5_tq1");
   }
+#endif
   if (a.max_rows == 1) {  // decode GEMV
-    const char* t = getenv("BP_TUNE_TQ1");  // development: "mfma" keeps the single-token MFMA variant
-    if (!(t && t[0] == 'm')) return launch_tq1_gemv(a, s, waves);
+    if (tuning().tq1 != 'm') return launch_tq1_gemv(a, s, waves);  // (development: "mfma" keeps the single-token MFMA variant)
     // one token, only its sums are scaled and kept
     if (waves == 16) return launch_tq1_v<16, 1>(a, s, "mfma_tq1_bf16_t1_w16", "mfma_tq1_bf16_t1_w16_gs");
     return launch_tq1_v<8, 1>(a, s, "mfma_tq1_bf16_t1_w8", "mfma_tq1_bf16_t1_w8_gs");
   }
   if (a.max_rows <= 64) {  // small decode batches: the fp8 x fp4 kernel with one operand tile per token
-    const char* t = getenv("BP_TUNE_TQ1");  // development: "mfma" / "lut" keep this kernel
-    if (!(t && (t[0] == 'm' || t[0] == 'l'))) {
+    if (tuning().tq1 != 'm' && tuning().tq1 != 'l') {  // (development: "mfma" / "lut" keep the kernels below)
       const int rc = launch_tq1_gemv_fp4(a, s);
       if (rc != BP_ERR_UNSUPPORTED) return rc;
     }
   }
   {  // more rows per expert: token tiles of 32 on the fp8 x fp4 matrix instruction
-    const char* t = getenv("BP_TUNE_TQ1");  // development: "mfma" keeps the 16-token kernel below
-    if (!(t && t[0] == 'm')) {
+    if (tuning().tq1 != 'm') {  // (development: "mfma" keeps the 16-token kernel below)
       const int rc = launch_gemm_tq1(a, s);
       if (rc != BP_ERR_UNSUPPORTED) return rc;
     }

@@ -335,13 +335,7 @@ int launch_tq2(const GemmArgs& a, hipStream_t s, const char* name) {
   constexpr int lds_want = X_BASE + XKB * 1024 + (SL ? tq2_scale_tile_max(R) : 0);
   constexpr int lds_cap = lds_want < 160 * 1024 ? lds_want : 160 * 1024;
   if (lds > (size_t)lds_cap) return BP_ERR_UNSUPPORTED;  // (scale tile variant: the caller falls back to scales from global memory)
-  static bool attr = false;
-  if (!attr) {
-    if (hipFuncSetAttribute((const void*)k_mfma_tq2<ACT, SDT, R, MT, WAVES, XKB, ABL, NQ, SL>, hipFuncAttributeMaxDynamicSharedMemorySize,
-                            lds_cap) != hipSuccess)
-      return fail(BP_ERR_LAUNCH, "cannot raise the dynamic LDS limit");
-    attr = true;
-  }
+  if (const int rc = raise_lds_limit<k_mfma_tq2<ACT, SDT, R, MT, WAVES, XKB, ABL, NQ, SL>>(lds_cap)) return rc;
   note_kernel(name);
   hipLaunchKernelGGL((k_mfma_tq2<ACT, SDT, R, MT, WAVES, XKB, ABL, NQ, SL>), grid, dim3(WAVES * 64), lds, s, a, (int)kc, (int)tokens);
   return check_launch(name);
@@ -368,6 +362,7 @@ int launch_tq2_sd(const GemmArgs& a, hipStream_t s, const char* name) {
 
 int launch_mfma_tq2(const GemmArgs& a, hipStream_t s, int R, int MT, int waves) {
   const bool bf = a.x_dtype == BP_BF16;
+#ifdef BP_DEV_ABLATIONS  // timing ablations (results are wrong): development builds only
   if (const char* t = getenv("BP_TUNE_ABL")) {
     if (bf && a.scale_dtype == BP_F16 && MT == 1) {
       switch (atoi(t)) {
@@ -384,6 +379,7 @@ int launch_mfma_tq2(const GemmArgs& a, hipStream_t s, int R, int MT, int waves) 
       }
     }
   }
+#endif
   if (a.max_rows == 1 && R == 2 && MT == 1 && waves == 16) {
     if (bf) return launch_tq2_sd<BP_BF16, 2, 1, 16, 48, 1>(a, s, "mfma_tq2_bf16_r2_t1_w16");
     return launch_tq2_sd<BP_I8, 2, 1, 16, 48, 1>(a, s, "mfma_tq2_i8_r2_t1_w16");

@@ -246,12 +246,7 @@ static int launch_sort(int64_t* order, int64_t* offsets, const int64_t* ids, int
     return check_launch("sort_by_expert");
   }
   const size_t lds = hist_mem ? 0 : (size_t)(SORT_WAVES * (E > 0 ? E : 1)) * sizeof(int32_t);
-  static std::once_flag attr_once;
-  static hipError_t attr_rc = hipSuccess;
-  std::call_once(attr_once, [] {
-    attr_rc = hipFuncSetAttribute((const void*)k_sort, hipFuncAttributeMaxDynamicSharedMemorySize, (int)(SORT_LDS_INTS * 4));
-  });
-  if (attr_rc != hipSuccess) return fail(BP_ERR_LAUNCH, "cannot raise the dynamic LDS limit for sort_by_expert");
+  if (const int rc = raise_lds_limit<k_sort>((int)(SORT_LDS_INTS * 4))) return rc;
   hipLaunchKernelGGL(k_sort, dim3(1), dim3(SORT_THREADS), lds, stream, order, offsets, ids, n, E, hist_mem, bad);
   return check_launch("sort_by_expert");
 }

@@ -284,12 +284,7 @@ template <int SDT, int WAVES, int SL, int MULTI>
 int launch_g1_k(const GemmArgs& a, hipStream_t s, const char* name, int64_t cpt, size_t lds) {
   const int64_t rows_per_wg = (int64_t)WAVES * 16;
   const dim3 grid((unsigned)((a.N + rows_per_wg - 1) / rows_per_wg), (unsigned)a.E, 1u);
-  static bool attr = false;
-  if (!attr) {
-    if (hipFuncSetAttribute((const void*)k_tq1_gemv<SDT, WAVES, SL, MULTI>, hipFuncAttributeMaxDynamicSharedMemorySize, G1_LDS_MAX) != hipSuccess)
-      return fail(BP_ERR_LAUNCH, "cannot raise the dynamic LDS limit");
-    attr = true;
-  }
+  if (const int rc = raise_lds_limit<k_tq1_gemv<SDT, WAVES, SL, MULTI>>(G1_LDS_MAX)) return rc;
   note_kernel(name);
   hipLaunchKernelGGL((k_tq1_gemv<SDT, WAVES, SL, MULTI>), grid, dim3(WAVES * 64), lds, s, a, (int)cpt);
   return check_launch(name);
@@ -303,7 +298,7 @@ int launch_g1(const GemmArgs& a, hipStream_t s, const char* name) {
   int64_t cpt = (G1_LDS_MAX - fixed) / G1_CHUNK_BYTES;
   const int64_t cap = 2 * WAVES * 64 / G1_SLOTS;  // two table slots per thread at most
   if (cpt > cap) cpt = cap;
-  if (const char* t = getenv("BP_TUNE_CPT")) { const int v = atoi(t); if (v >= 1 && v < cpt) cpt = v; }  // (development)
+  if (tuning().cpt >= 1 && tuning().cpt < cpt) cpt = tuning().cpt;  // (development)
   if (cpt > nchunks) cpt = nchunks;
   if (cpt < 1) return BP_ERR_UNSUPPORTED;  // the caller tries the next variant
   const size_t lds = (size_t)(fixed + cpt * G1_CHUNK_BYTES);
@@ -330,8 +325,7 @@ int launch_g1_v(const GemmArgs& a, hipStream_t s, const char* name_sl, const cha
 
 // max_rows == 1 (checked by the caller); any activation dtype
 int launch_tq1_gemv(const GemmArgs& a, hipStream_t s, int waves) {
-  const char* t = getenv("BP_TUNE_TQ1");  // development: "lut" keeps the table kernel
-  if (!(t && t[0] == 'l')) {
+  if (tuning().tq1 != 'l') {  // (development: "lut" keeps the table kernel)
     const int rc = launch_tq1_gemv_fp4(a, s);
     if (rc != BP_ERR_UNSUPPORTED) return rc;
   }

@@ -29,8 +29,9 @@
 //    activations are exactly p0 + p1 down to 2^-9 of the group's largest magnitude, fp16 (11 bits) exactly the
 //    three; below that a value keeps 4 more bits through p2, and what is dropped is less than 2^-20 of the group's
 //    largest magnitude. Products fp8 x fp4 are exact and accumulate in float32. float32 activations (24 bits)
-//    are left to the table kernel. Activations that are not finite give results that are not meaningful here
-//    (the other kernels propagate NaN / Inf).
+//    are left to the table kernel. A NaN or an infinity among a group's activations makes the token's outputs NaN
+//    (the group's inverse prescale is NaN); the reference skips zero weights, so there only rows with a nonzero weight
+//    at that k become non-finite.
 //
 // Operand A is read from an LDS tile built once per workgroup. It is stored compactly: per chunk, per matrix
 // instruction j = 0..7 and per 16-byte half of an A lane's operand (= the 2 x 8 digit slots of two consecutive
@@ -189,12 +190,17 @@ __global__ __launch_bounds__(WAVES * 64, 4) void k_tq1_gemv_fp4(GemmArgs a, int 
     const unsigned at = (unsigned)(tile_at(tt, g >> 3) + 4 * (g & 7));
     const bool real = (g & 7) < 5 && 128 * (int64_t)(5 * (cb + (g >> 3)) + (g & 7)) < a.K;
     int sh = 0;
+    bool finite = true;
     if (real && a.x_dtype != BP_I8) {
-      sh = 134 - (int)((*(const lds_u32*)(at + F4_PRE_OFF) >> 23) & 255u);
+      const int ex = (int)((*(const lds_u32*)(at + F4_PRE_OFF) >> 23) & 255u);
+      finite = ex != 255;  // a NaN or an infinity among the group's activations
+      sh = 134 - ex;
       sh = sh > 120 ? 120 : sh < -120 ? -120 : sh;
     }
     *(lds_u32*)(at + F4_PRE_OFF) = (unsigned)(sh + 127) << 23;
-    *(lds_u32*)(at + F4_INV_OFF) = real ? (unsigned)(127 - sh) << 23 : 0u;
+    // (the inverse prescale multiplies every row's group sum: NaN for a group with a non-finite activation, so the
+    // token's outputs are NaN rather than finite and wrong)
+    *(lds_u32*)(at + F4_INV_OFF) = !real ? 0u : finite ? (unsigned)(127 - sh) << 23 : 0x7fc00000u;
   }
   __syncthreads();
 
@@ -557,22 +563,24 @@ __global__ __launch_bounds__(WAVES * 64, 4) void k_tq1_gemv_fp4(GemmArgs a, int 
   else if (NP >= 4 && npairs == 3) all_terms(IC<(NP >= 4 ? 3 : NP)>{});
   else all_terms(IC<NP>{});
 }
-int f4_cus() {  // compute units of the current device (256 if the query fails)
-  int dev = 0, cus = 0;
-  if (hipGetDevice(&dev) != hipSuccess || hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || cus < 1) cus = 256;
-  return cus;
+int f4_cus() {  // compute units of the current device (256 if the query fails); looked up once per device
+  static std::mutex m;
+  static int known[64] = {};
+  int dev = 0;
+  if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64) return 256;
+  std::lock_guard<std::mutex> lock(m);
+  if (known[dev] == 0) {
+    int cus = 0;
+    if (hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || cus < 1) cus = 256;
+    known[dev] = cus;
+  }
+  return known[dev];
 }
 
 template <int SDT, int WAVES, int ABL = 0, int NTOK = 1>
 int launch_f4_k(const GemmArgs& a, hipStream_t s, const char* name, int nchunks, size_t lds, int seg_chunks = 0 /* chunks per launch (0: all) */, int first_row = 0) {
-  static bool attr = false;
-  static int cus = 0;
-  if (!attr) {
-    const hipError_t rc = hipFuncSetAttribute((const void*)k_tq1_gemv_fp4<SDT, WAVES, ABL, NTOK>, hipFuncAttributeMaxDynamicSharedMemorySize, F4_LDS_MAX);
-    if (rc != hipSuccess) return fail(BP_ERR_LAUNCH, "cannot raise the dynamic LDS limit: %s", hipGetErrorString(rc));
-    cus = f4_cus();
-    attr = true;
-  }
+  if (const int rc = raise_lds_limit<k_tq1_gemv_fp4<SDT, WAVES, ABL, NTOK>>(F4_LDS_MAX)) return rc;
+  const int cus = f4_cus();
   // Every workgroup builds the tables of its expert's token, so a workgroup takes as many row blocks as still leaves
   // every CU its full set of resident workgroups (16 waves): all workgroups resident at once, one build each.
   const int64_t rows_per_block = (int64_t)WAVES * 16 * F4_GR;
@@ -600,14 +608,15 @@ int launch_f4(const GemmArgs& a, hipStream_t s, int first_row = 0) {
   const int64_t nseg = NTOK == 1 ? 1 : (nchunks + fit - 1) / fit, seg = (nchunks + nseg - 1) / nseg;
   const size_t lds = (size_t)(F4_LUT_BYTES + NTOK * seg * f4_chunk_bytes(NTOK));
   if (lds > (size_t)F4_LDS_MAX || nseg > 4) return BP_ERR_UNSUPPORTED;
-  static const int cus = f4_cus();
+  const int cus = f4_cus();
   const int64_t experts = a.E < a.T ? a.E : a.T;
   if (NTOK > 1) {
     const bool wide = lds > (size_t)F4_LDS_MAX / 2 || ((a.N + 255) / 256) * experts >= 4 * (int64_t)cus;
     if (!wide) return launch_f4_k<SDT, 8, 0, NTOK>(a, s, NTOK == 2 ? "fp4_tq1_m2_w8" : NTOK == 4 ? "fp4_tq1_m4_w8" : NTOK == 6 ? "fp4_tq1_m6_w8" : "fp4_tq1_m8_w8", (int)nchunks, lds, (int)seg, first_row);
     return launch_f4_k<SDT, 16, 0, NTOK>(a, s, NTOK == 2 ? "fp4_tq1_m2_w16" : NTOK == 4 ? "fp4_tq1_m4_w16" : NTOK == 6 ? "fp4_tq1_m6_w16" : "fp4_tq1_m8_w16", (int)nchunks, lds, (int)seg, first_row);
   }
-  if (const char* t = getenv("BP_TUNE_F4ABL")) {  // development: timing ablations (one token)
+#ifdef BP_DEV_ABLATIONS  // timing ablations (results are wrong): development builds only
+  if (const char* t = getenv("BP_TUNE_F4ABL")) {
     if (SDT == BP_F16 && atoi(t) == 1) return launch_f4_k<BP_F16, 8, 1>(a, s, "abl1_fp4", (int)nchunks, lds);
     if (SDT == BP_F16 && atoi(t) == 2) return launch_f4_k<BP_F16, 8, 2>(a, s, "abl2_fp4", (int)nchunks, lds);
     if (SDT == BP_F16 && atoi(t) == 3) return launch_f4_k<BP_F16, 8, 3>(a, s, "abl3_fp4", (int)nchunks, lds);
@@ -617,10 +626,11 @@ int launch_f4(const GemmArgs& a, hipStream_t s, int first_row = 0) {
     if (SDT == BP_F16 && atoi(t) == 7) return launch_f4_k<BP_F16, 8, 7>(a, s, "abl7_fp4", (int)nchunks, lds);
     if (SDT == BP_F16 && atoi(t) == 8) return launch_f4_k<BP_F16, 8, 8>(a, s, "abl8_fp4", (int)nchunks, lds);
   }
+#endif
   // Two workgroups of 8 waves per CU when their tiles fit side by side and the call is small; one of 16 waves when
   // there are row blocks enough for every CU anyway (the tables are then built once per CU instead of twice).
   bool wide = lds > (size_t)F4_LDS_MAX / 2 || ((a.N + 255) / 256) * experts >= 4 * (int64_t)cus;
-  if (const char* tw = getenv("BP_TUNE_F4W")) wide = lds > (size_t)F4_LDS_MAX / 2 || atoi(tw) == 16;  // (development)
+  if (tuning().f4w) wide = lds > (size_t)F4_LDS_MAX / 2 || tuning().f4w == 16;  // (development)
   if (!wide) return launch_f4_k<SDT, 8>(a, s, "fp4_tq1_t1_w8", (int)nchunks, lds);
   return launch_f4_k<SDT, 16>(a, s, "fp4_tq1_t1_w16", (int)nchunks, lds);
 }
@@ -655,7 +665,7 @@ int launch_tq1_gemv_fp4(const GemmArgs& a, hipStream_t s) {
   if (a.x_dtype != BP_BF16 && a.x_dtype != BP_F16 && a.x_dtype != BP_I8) return BP_ERR_UNSUPPORTED;
   if (a.max_rows > 1 && a.x_dtype == BP_F16) return BP_ERR_UNSUPPORTED;  // (11 significant bits need the third piece)
   int64_t few = 4;  // "most experts have few rows": at most this many routed rows per expert on average
-  if (const char* t = getenv("BP_TUNE_F4T")) few = atoi(t);  // (development)
+  if (tuning().f4t >= 0) few = tuning().f4t;  // (development)
   if (a.max_rows < 1 || a.max_rows > 64 || (a.max_rows > 8 && a.T > few * a.E)) return BP_ERR_UNSUPPORTED;
   if (a.N % 16 != 0 || a.Kp != (a.K + 4) / 5 || (a.group != 128 && a.group != 256)) return BP_ERR_UNSUPPORTED;
   for (int t = 0; t < a.n_terms; ++t)

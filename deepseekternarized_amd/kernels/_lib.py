@@ -20,12 +20,14 @@ SIGNATURES = {
     "bp_version": (C.c_char_p, []),
     "bp_last_kernel": (C.c_char_p, []),
     "bp_set_kernel_policy": (_i, [_i]),
+    "bp_reload_tuning": (None, []),
     "bp_ternary_grouped_gemm": (_i, [_p, _p, _i, _p, _p, _p, _p, _p, _i, _i, _l, _l, _l, _l, _l, _l, _l, _i, _l, _p, _p]),
     "bp_unpack_trits": (_i, [_p, _p, _l, _l, _i, _p]),
     "bp_pack_trits": (_i, [_p, _p, _l, _l, _i, _p]),
     "bp_expand_scales": (_i, [_p, _p, _i, _l, _p]),
     "bp_tq1_lut": (_i, [_p, _p]),
     "bp_quant_act_int8": (_i, [_p, _p, _p, _i, _l, _l, _p]),
+    "bp_absmean_pack": (_i, [_p, _p, _i, _p, _p, _i, _l, _l, _l, _i, _p]),
     "bp_sort_workspace_ints": (_l, [_l, _l]),
     "bp_sort_by_expert": (_i, [_p, _p, _p, _l, _l, _p, _p, _p]),
     "bp_sort_by_expert_static": (_i, [_p, _p, _p, _l, _l, _p, _p]),

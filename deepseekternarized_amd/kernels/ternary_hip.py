@@ -121,6 +121,22 @@ def _need_ext(x):
     return e
 
 
+_dense_offsets_cache: dict = {}
+
+
+def dense_offsets(device, rows: int) -> torch.Tensor:
+    """The device offsets ``[0, rows]`` of a one-expert (dense) call, made once per device and row count and kept:
+    a dense linear then costs no host-to-device copy per call."""
+    key = (device, rows)
+    t = _dense_offsets_cache.get(key)
+    if t is None:
+        if len(_dense_offsets_cache) > 4096:
+            _dense_offsets_cache.clear()
+        t = torch.tensor([0, rows], dtype=torch.int64, device=device)
+        _dense_offsets_cache[key] = t
+    return t
+
+
 def _as_terms(packed, w_scale):
     pk = list(packed) if isinstance(packed, (list, tuple)) else [packed]
     sc = list(w_scale) if isinstance(w_scale, (list, tuple)) else [w_scale]
@@ -136,9 +152,9 @@ def ternary_gemm(x: torch.Tensor, x_scale: torch.Tensor, packed, w_scale, K: int
     if x.dtype != torch.int8:
         raise TypeError("ternary_gemm takes int8 activations (see quant_act_int8)")
     pk, sc = _as_terms(packed, w_scale)
-    offsets = [0, x.size(0)]
-    return grouped_ternary_gemm(x, x_scale, offsets, [p[None] for p in pk], [s[None] for s in sc], K, group, fmt,
-                                backend=backend)
+    _need_ext(x)
+    return grouped_ternary_gemm(x, x_scale, dense_offsets(x.device, x.size(0)), [p[None] for p in pk], [s[None] for s in sc], K, group,
+                                fmt, backend=backend, max_rows=x.size(0))
 
 
 def ternary_gemm_float(x: torch.Tensor, packed, w_scale, K: int, group: int, fmt: str,
@@ -149,8 +165,9 @@ def ternary_gemm_float(x: torch.Tensor, packed, w_scale, K: int, group: int, fmt
     if x.dtype not in (torch.bfloat16, torch.float16, torch.float32):
         raise TypeError("ternary_gemm_float takes bf16, f16 or f32 activations")
     pk, sc = _as_terms(packed, w_scale)
-    return grouped_ternary_gemm(x, None, [0, x.size(0)], [p[None] for p in pk], [s[None] for s in sc], K, group, fmt,
-                                backend=backend)
+    _need_ext(x)
+    return grouped_ternary_gemm(x, None, dense_offsets(x.device, x.size(0)), [p[None] for p in pk], [s[None] for s in sc], K, group, fmt,
+                                backend=backend, max_rows=x.size(0))
 
 
 def ternary_gemm_ref(x: torch.Tensor, x_scale: torch.Tensor, packed: torch.Tensor, w_scale: torch.Tensor,
@@ -198,29 +215,40 @@ def grouped_ternary_gemm(x: torch.Tensor, x_scale, offsets, packed, w_scale, K: 
         max_rows = max(0, min(int(max_rows), x.size(0)))
     out = torch.zeros(x.size(0), pk[0].size(1), dtype=torch.float32, device=dev)
     xs = None if x_scale is None else x_scale.float().contiguous()
-    old = e.set_kernel_policy(1 if backend == "torch" else 0)
+    args = (out, x.contiguous(), xs, offs_dev, [p.contiguous() for p in pk], [s.contiguous() for s in sc], K, group, code, None, max_rows)
+    if backend != "torch":  # (the kernel policy is per thread and 0 unless someone changed it: nothing to set or restore)
+        e.ternary_grouped_gemm(*args, offsets_host=host)
+        return out
+    old = e.set_kernel_policy(1)
     try:
-        e.ternary_grouped_gemm(out, x.contiguous(), xs, offs_dev, [p.contiguous() for p in pk],
-                               [s.contiguous() for s in sc], K, group, code, None, max_rows, offsets_host=host)
+        e.ternary_grouped_gemm(*args, offsets_host=host)
     finally:
         e.set_kernel_policy(old)
     return out
 
 
-def sort_by_expert(expert_ids: torch.Tensor, n_experts: int) -> tuple[torch.Tensor, torch.Tensor]:
+def sort_by_expert(expert_ids: torch.Tensor, n_experts: int, validate: bool = False) -> tuple[torch.Tensor, torch.Tensor]:
     """Flattened top-k expert ids [T*k] -> (row order sorting them by expert, offsets [E + 1])
     (``boilerplate/kernels/ternary_cuda.py:114-118``): a stable counting sort on the device.
-    The result stays on the device; no host synchronisation happens."""
+    The result stays on the device; no host synchronisation happens.
+
+    Ids outside ``[0, n_experts)`` - which the reference's ``bincount`` / ``argsort`` reject or sort to the ends - are
+    left out of the count: ``offsets[-1]`` is then smaller than the number of ids and the tail of ``order`` holds -1.
+    ``validate=True`` reads a device flag back (one host synchronisation) and raises ValueError for such ids instead."""
     e = _need_ext(expert_ids)
     ids = expert_ids.to(torch.int64).contiguous().view(-1)
     n, dev = ids.numel(), ids.device
-    order = torch.empty(n, dtype=torch.int64, device=dev)
+    order = torch.full((n,), -1, dtype=torch.int64, device=dev) if validate else torch.empty(n, dtype=torch.int64, device=dev)
     offsets = torch.empty(n_experts + 1, dtype=torch.int64, device=dev)
     need = e.lib.bp_sort_workspace_ints(n, n_experts)
     ws = torch.empty(need, dtype=torch.int32, device=dev) if need else None
+    bad = torch.zeros(1, dtype=torch.int32, device=dev) if validate else None
     with torch.cuda.device(dev):
         _lib.check(e.lib.bp_sort_by_expert(order.data_ptr(), offsets.data_ptr(), ids.data_ptr(), n, n_experts,
-                                           ws.data_ptr() if ws is not None else None, None, _lib.stream_ptr(dev)))
+                                           ws.data_ptr() if ws is not None else None,
+                                           bad.data_ptr() if bad is not None else None, _lib.stream_ptr(dev)))
+    if validate and int(bad.item()):
+        raise ValueError(f"expert ids must lie in [0, {n_experts})")
     return order, offsets
 
 

@@ -13,7 +13,7 @@ from dataclasses import dataclass
 import torch
 
 from ..kernels import _lib
-from ..kernels.ternary_hip import _fmt_code, _need_ext, grouped_ternary_gemm
+from ..kernels.ternary_hip import _fmt_code, _need_ext, dense_offsets, grouped_ternary_gemm
 
 
 def quant_act_int8(x: torch.Tensor) -> tuple[torch.Tensor, torch.Tensor]:
@@ -65,6 +65,21 @@ class TernaryLinear:
     def out_features(self) -> int:
         return self.terms[0].packed.size(0)
 
+    def dequantized(self, device=None) -> torch.Tensor:
+        """The dense float32 [N, K] weight ``sum_terms trits * scale`` (boilerplate/ternary/ops.py:51-58), computed on
+        the device from the decoded trits and the widened scales (``bp_unpack_trits``, ``bp_expand_scales``) with the
+        reference's operation order, and kept. ``device``: where the terms are not on a HIP device yet."""
+        from .pack import expand_scales, unpack
+
+        if getattr(self, "_deq", None) is None:
+            dev = torch.device(device) if device is not None else self.terms[0].packed.device
+            w = None
+            for packed, scale in self._on(dev):
+                d = unpack(packed[0], self.fmt, self.K).float() * expand_scales(scale[0]).repeat_interleave(self.group, -1)[:, : self.K]
+                w = d if w is None else w + d
+            self._deq = w
+        return self._deq
+
     def __call__(self, x: torch.Tensor, out_dtype=torch.bfloat16) -> torch.Tensor:
         shape = x.shape
         x2 = x.reshape(-1, self.K)
@@ -74,6 +89,6 @@ class TernaryLinear:
             q, s = quant_act_int8(x2)
         else:
             q, s = (x2 if x2.dtype in (torch.bfloat16, torch.float16, torch.float32) else x2.float()).contiguous(), None
-        out = grouped_ternary_gemm(q, s, [0, x2.size(0)], [p for p, _ in terms], [sc for _, sc in terms],
-                                   self.K, self.group, self.fmt, backend=self.backend)
+        out = grouped_ternary_gemm(q, s, dense_offsets(x2.device, x2.size(0)), [p for p, _ in terms], [sc for _, sc in terms],
+                                   self.K, self.group, self.fmt, backend=self.backend, max_rows=x2.size(0))
         return out.view(*shape[:-1], -1).to(out_dtype)

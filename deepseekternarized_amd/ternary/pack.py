@@ -87,6 +87,30 @@ def tq1_lut(device=None) -> torch.Tensor:
     return out
 
 
+class _LazyLut:
+    """``_TQ1_LUT`` of the reference (boilerplate/ternary/pack.py:70, a module-level [256, 5] int8 tensor that
+    ``ternary/ops.py:17`` imports and hands to the kernels). Here the table is produced by the device on first use,
+    per device, because importing this package must not need a GPU: ``_TQ1_LUT.to(device)`` and ``_TQ1_LUT.tensor()``
+    return it."""
+
+    def __init__(self):
+        self._by_device = {}
+
+    def to(self, device=None) -> torch.Tensor:
+        dev = torch.device(device if device is not None else "cuda")
+        if dev.type == "cuda" and dev.index is None:
+            dev = torch.device("cuda", torch.cuda.current_device())
+        if dev not in self._by_device:
+            self._by_device[dev] = tq1_lut(dev)
+        return self._by_device[dev]
+
+    def tensor(self) -> torch.Tensor:
+        return self.to(None)
+
+
+_TQ1_LUT = _LazyLut()
+
+
 def expand_scales(scale: torch.Tensor) -> torch.Tensor:
     """Stored fp16/bf16 scales -> float32 (``t.scale.float()``, boilerplate/ternary/ops.py:37)."""
     e = _need_ext(scale)

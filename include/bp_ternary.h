@@ -87,6 +87,11 @@ int bp_ternary_grouped_gemm(float* out, const void* x, int x_dtype, const float*
  * Returns the previous value. */
 int bp_set_kernel_policy(int policy);
 
+/* The kernel selection has development overrides (environment variables BP_TUNE_*), read once when the library is first
+ * used. This reads them again; it is for tests and tuning sweeps that switch kernels inside one process, and has no
+ * counterpart in the reference. */
+void bp_reload_tuning(void);
+
 /* Name of the kernel the last bp_ternary_grouped_gemm on this thread launched ("" if none). */
 const char* bp_last_kernel(void);
 
@@ -107,6 +112,17 @@ int bp_tq1_lut(int8_t* lut, void* stream);
 /* Per-row absmax int8 quantisation (boilerplate/ternary/ops.py:20-25):
  * s = max(amax|x| / 127, 1e-8), q = clamp(rint(x / s), -127, 127). x [M, K] of x_dtype (bf16/f16/f32). */
 int bp_quant_act_int8(int8_t* q, float* s, const void* x, int x_dtype, int64_t M, int64_t K, void* stream);
+
+/* BitNet b1.58 absmean quantizer and packer in one kernel: the producer of Mode D weights
+ * (absmean_ternary, boilerplate/ternary/fit.py:78-96, followed by pack as in BitLinear.packed_term,
+ * boilerplate/qat/bitlinear.py:75-80). Per row and `group` columns: s = scale_dtype(sum |w| / columns in the group)
+ * (float32 sum in ascending column order), trit = s > 0 ? clamp(rint(w / s), -1, 1) : 0.
+ *   packed  device u8 [N, Kp] in the layout of bp_pack_trits
+ *   scale   device [N, G] of scale_dtype (BP_F16 or BP_BF16), G = ceil(K / group)
+ *   trits   device i8 [N, K], or NULL when only the packed form is wanted
+ *   w       device [N, K] of w_dtype (BP_F32, BP_BF16, BP_F16) */
+int bp_absmean_pack(uint8_t* packed, void* scale, int scale_dtype, int8_t* trits, const void* w, int w_dtype,
+                    int64_t N, int64_t K, int64_t group, int fmt, void* stream);
 
 /* Stable counting sort of expert ids (boilerplate/kernels/ternary_cuda.py:114-118):
  * order[i] = index of the i-th entry in expert order (ties keep input order), offsets = [0, cumsum(counts)].

@@ -135,6 +135,37 @@ def quant_act_int8(x: np.ndarray) -> tuple[np.ndarray, np.ndarray]:
 
 
 # --------------------------------------------------------------------------- GEMM reference
+def absmean_ternary(weight: np.ndarray, group: int, scale_dtype: str = "f16") -> tuple[np.ndarray, np.ndarray]:
+    """BitNet b1.58 absmean quantizer (boilerplate/ternary/fit.py:78-96): per row and group of `group` columns (the
+    last group may be shorter and counts its own columns) s = scale_dtype(sum |w| / count), then
+    trits = s > 0 ? clamp(rint(w / max(s, 1e-30)), -1, 1) : 0 in float32. Returns (trits int8 [N, K], scale as float32
+    holding the fp16 / bf16-rounded values [N, G]).
+
+    The float32 sum is taken in ascending column order here; the reference's ``torch.sum`` leaves the order to the
+    library, so a scale could differ in its last stored bit where the sum lands within one float32 rounding of a
+    fp16 rounding boundary. Pinned by the literal known-answer test of the reference (tests/test_qat.py:11-17: short
+    last group, all-zero row) and by exact small-integer cases where the order cannot matter."""
+    w = np.asarray(weight, np.float32)
+    if w.ndim != 2 or group <= 0 or w.shape[1] == 0:
+        raise ValueError("weight must be a matrix with a nonempty input dimension and positive group")
+    if scale_dtype not in ("f16", "bf16"):
+        raise ValueError("scale_dtype must be float16 or bfloat16")
+    N, K = w.shape
+    G = -(-K // group)
+    scale = np.zeros((N, G), np.float32)
+    trits = np.zeros((N, K), np.int8)
+    for g in range(G):
+        k0, k1 = g * group, min(K, (g + 1) * group)
+        a = np.abs(w[:, k0:k1])
+        total = np.add.accumulate(a, axis=1, dtype=np.float32)[:, -1]  # sequential float32 sum
+        mean = (total / np.float32(k1 - k0)).astype(np.float32)
+        s = mean.astype(np.float16).astype(np.float32) if scale_dtype == "f16" else bf16_round(mean)
+        scale[:, g] = s
+        q = np.rint(w[:, k0:k1] / np.maximum(s, np.float32(1e-30))[:, None]).clip(-1, 1)
+        trits[:, k0:k1] = np.where(s[:, None] > 0, q, 0).astype(np.int8)
+    return trits, scale
+
+
 def _fmt_check(fmt: str) -> None:
     """boilerplate/kernels/ternary_cuda.py:46-49."""
     if fmt not in ("tq1", "tq2"):

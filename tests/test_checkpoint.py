@@ -142,3 +142,45 @@ def test_linear_and_moe_from_checkpoint_match_the_oracle(tmp_path):
     a, b = moe(xd, logits), ref(xd, logits)
     assert torch.equal(a, b) and torch.isfinite(a).all()
     assert bp.ext() is not None
+
+
+@pytest.mark.parametrize("bad", ["../outside.safetensors", "/etc/passwd", "sub/../../x.safetensors", "a\\b.safetensors", "./x.safetensors", ""])
+@pytest.mark.parametrize("where", ["manifest", "index"])
+def test_file_names_from_the_checkpoint_cannot_leave_its_directory(tmp_path, bad, where):
+    """boilerplate/checkpoint/paths.py:6-22: names that come from manifest.json or the shard index are confined to the
+    checkpoint directory (no absolute paths, `..`, backslashes, empty components, or symlinks that lead outside)."""
+    root = tmp_path / "ck"
+    root.mkdir()
+    w, _, _ = _experts("tq2", 1, 16, 1280, 1, seed=3)
+    _write(root, w, shards=1, index=True, with_file=True)
+    base = next(iter(w))
+    if where == "manifest":
+        m = json.loads((root / "manifest.json").read_text())
+        for rec in m["tensors"][base]["stored"].values():
+            rec["file"] = bad
+        (root / "manifest.json").write_text(json.dumps(m))
+    else:
+        m = json.loads((root / "manifest.json").read_text())
+        for rec in m["tensors"][base]["stored"].values():
+            rec.pop("file", None)
+        (root / "manifest.json").write_text(json.dumps(m))
+        idx = json.loads((root / "model.safetensors.index.json").read_text())
+        idx["weight_map"] = {n: bad for n in idx["weight_map"]}
+        (root / "model.safetensors.index.json").write_text(json.dumps(idx))
+    ck = TernaryCheckpoint(root)
+    with pytest.raises(ValueError, match="checkpoint path"):
+        ck.terms(base)
+
+
+def test_symlinked_shard_outside_the_directory_is_refused(tmp_path):
+    root, outside = tmp_path / "ck", tmp_path / "elsewhere"
+    root.mkdir()
+    outside.mkdir()
+    w, _, _ = _experts("tq2", 1, 16, 1280, 1, seed=4)
+    _write(root, w, shards=1, index=True, with_file=True)
+    shard = next(root.glob("*.safetensors"))
+    moved = outside / shard.name
+    shard.rename(moved)
+    shard.symlink_to(moved)
+    with pytest.raises(ValueError, match="escapes"):
+        TernaryCheckpoint(root).terms(next(iter(w)))

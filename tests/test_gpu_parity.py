@@ -426,3 +426,93 @@ def test_moe_layer_matches_reference_call_pattern(bp, fmt, act):
     # both sides round to bf16 at the same points; float32 summation order may flip a few roundings
     assert rel_l2(got, want) <= 5e-3, rel_l2(got, want)
     assert np.abs(got - want).max() <= MAX_ABS_BF16 * max(1.0, np.abs(want).max())
+
+
+# --------------------------------------------------------------------------- producer: absmean quantizer + packer
+def test_absmean_known_answer_of_the_reference(bp):
+    """reference tests/test_qat.py:11-17, literally: a short last group and an all-zero row."""
+    weight = torch.tensor([[0.0, -2.0, 4.0, 3.0, -1.0], [0.0, 0.0, 0.0, 0.0, 0.0]], device="cuda")
+    result = bp.absmean_ternary(weight, group=3)
+    assert torch.equal(result.scale.cpu(), torch.tensor([[2.0, 2.0], [0.0, 0.0]], dtype=torch.float16))
+    assert torch.equal(result.trits.cpu(), torch.tensor([[0, -1, 1, 1, 0], [0, 0, 0, 0, 0]], dtype=torch.int8))
+    with pytest.raises(ValueError):
+        bp.absmean_ternary(weight, group=0)
+    with pytest.raises(ValueError):
+        bp.absmean_ternary(weight, group=3, scale_dtype=torch.float32)
+    with pytest.raises(ValueError):
+        bp.packed_term(weight, 3, "tq3")
+
+
+@pytest.mark.parametrize("wdtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("sdtype", [torch.float16, torch.bfloat16])
+@pytest.mark.parametrize("K,group", [(131, 64), (640, 128), (4099, 256), (7, 3)])
+def test_absmean_and_packed_term_bit_exact(bp, wdtype, sdtype, K, group):
+    """Trits, scales and packed bytes bit-identical to the oracle (same float32 summation order), and
+    packed_term == pack(absmean trits) for both formats (boilerplate/qat/bitlinear.py:75-80)."""
+    rng = np.random.default_rng(K + group)
+    w = rng.standard_normal((37, K)).astype(np.float32) * np.exp(rng.uniform(-3, 3, (37, 1))).astype(np.float32)
+    w[5] = 0.0
+    w[6, : K // 2] = 0.0
+    wt = dev(w).to(wdtype)
+    w_seen = wt.float().cpu().numpy()
+    want_trits, want_scale = orc.absmean_ternary(w_seen, group, "f16" if sdtype == torch.float16 else "bf16")
+    term = bp.absmean_ternary(wt, group, sdtype)
+    assert term.scale.dtype == sdtype and term.trits.dtype == torch.int8
+    assert np.array_equal(term.scale.float().cpu().numpy(), want_scale)
+    assert np.array_equal(term.trits.cpu().numpy(), want_trits)
+    for fmt in ("tq1", "tq2"):
+        pt = bp.packed_term(wt, group, fmt, sdtype)
+        assert np.array_equal(pt.packed.cpu().numpy(), orc.pack(want_trits, fmt))
+        assert torch.equal(pt.scale, term.scale)
+
+
+def test_packed_term_feeds_the_linear_like_the_training_graph(bp):
+    """reference tests/test_qat.py:52-59 (BitLinear training graph == packed engine), K=131, group 64: the packed term
+    made on the device, run through TernaryLinear, equals the dequantized product."""
+    rng = np.random.default_rng(52)
+    K, N, group = 131, 24, 64
+    w = dev(rng.standard_normal((N, K)).astype(np.float32))
+    x = bf16_dev(rng.standard_normal((5, K)).astype(np.float32))
+    for fmt in ("tq1", "tq2"):
+        lin = bp.TernaryLinear([bp.packed_term(w, group, fmt)], K, fmt, group, act="int8")
+        q, s = bp.quant_act_int8(x)
+        want = (q.float() * s[:, None]) @ lin.dequantized().t()
+        got = lin(x, out_dtype=torch.float32)
+        torch.testing.assert_close(got, want, rtol=1e-3, atol=1e-3)
+
+
+# --------------------------------------------------------------------------- operator-layer pieces of the reference interface
+@pytest.mark.parametrize("fmt", ["tq1", "tq2"])
+def test_dequantized_matches_the_reference_formula(bp, fmt):
+    """boilerplate/ternary/ops.py:51-58: sum over terms of unpack(packed).float() * scale.float().repeat_interleave(group)[:, :K]."""
+    N, K, group = 37, 200, 64
+    packed, scales = synth_weights(9, 1, N, K, group, fmt, terms=2)
+    lin = bp.TernaryLinear([bp.PackedTerm(dev(p[0]), dev(s[0])) for p, s in zip(packed, scales)], K, fmt, group)
+    want = None
+    for p, s in zip(packed, scales):
+        d = orc.unpack(p[0], fmt, K).astype(np.float32) * np.repeat(s[0].astype(np.float32), group, axis=1)[:, :K]
+        want = d if want is None else want + d
+    got = lin.dequantized()
+    assert got.dtype == torch.float32 and got.is_cuda and np.array_equal(got.cpu().numpy(), want)
+    assert lin.dequantized() is got  # kept
+
+
+def test_module_level_tq1_table(bp):
+    from deepseekternarized_amd.ternary.pack import _TQ1_LUT
+
+    t = _TQ1_LUT.to("cuda")
+    assert t.dtype == torch.int8 and tuple(t.shape) == (256, 5) and np.array_equal(t.cpu().numpy(), orc.tq1_lut())
+    assert _TQ1_LUT.to("cuda") is t
+
+
+def test_sort_by_expert_ids_out_of_range(bp):
+    """Ids outside [0, E): left out of the count by default (documented divergence: the reference's bincount raises for
+    negative ids); `validate=True` raises."""
+    ids = torch.tensor([3, 0, 7, -1, 2, 8, 0], device="cuda")
+    order, offsets = bp.sort_by_expert(ids, 8)
+    assert offsets.cpu().tolist() == [0, 2, 2, 3, 4, 4, 4, 4, 5]
+    assert order.cpu().tolist()[:5] == [1, 6, 4, 0, 2]
+    with pytest.raises(ValueError):
+        bp.sort_by_expert(ids, 8, validate=True)
+    order, offsets = bp.sort_by_expert(ids.clamp(0, 7), 8, validate=True)
+    assert offsets.cpu().tolist()[-1] == 7 and sorted(order.cpu().tolist()) == list(range(7))

@@ -94,13 +94,10 @@ def _check(got, want):
 
 # --------------------------------------------------------------------------- TQ1 decode GEMV
 # Two kernels: fp8 x fp4 matrix instructions (16-bit and int8 activations, tables that fit in LDS) and the table
-# lookup of partial sums (everything else; BP_TUNE_TQ1=lut selects it for every call, read at each call).
+# lookup of partial sums (everything else; BP_TUNE_TQ1=lut selects it for every call; the `tune` fixture makes the library read the switch again).
 @pytest.fixture(params=["fp4", "lut"])
-def gemv_kernel(request, monkeypatch):
-    if request.param == "lut":
-        monkeypatch.setenv("BP_TUNE_TQ1", "lut")
-    else:
-        monkeypatch.delenv("BP_TUNE_TQ1", raising=False)
+def gemv_kernel(request, tune):
+    tune("BP_TUNE_TQ1", "lut" if request.param == "lut" else None)
     return request.param + "_tq1"
 
 
@@ -135,13 +132,13 @@ def test_tq1_fp4_small_batches_many_rows_bf16_scales(bp):
         _check(got, want)
 
 
-def test_tq1_gemv_scales_from_global_memory(bp, monkeypatch):
+def test_tq1_gemv_scales_from_global_memory(bp, tune):
     """Table kernel: scale pointers that are not 16-byte aligned, and K with more groups than the LDS tile takes."""
-    monkeypatch.setenv("BP_TUNE_TQ1", "lut")
+    tune("BP_TUNE_TQ1", "lut")
     got, want, kern = _run(bp, "tq1", 2, 32, 2048, [1, 1], "bf16", seed=6, misalign_scales=True)
     assert kern.startswith("lut_tq1") and kern.endswith("_gs"), kern
     _check(got, want)
-    monkeypatch.delenv("BP_TUNE_TQ1")
+    tune("BP_TUNE_TQ1", None)
     got, want, kern = _run(bp, "tq1", 2, 32, 2048, [1, 1], "bf16", seed=6, misalign_scales=True)
     assert kern.startswith("fp4_tq1"), kern
     _check(got, want)
@@ -178,12 +175,9 @@ def test_tq1_gemv_fp8_pieces_keep_small_activations(bp, act):
 
 # --------------------------------------------------------------------------- TQ1 grouped GEMM (token tiles of 32) and the 16-token MFMA kernel
 @pytest.fixture(params=["gemm", "mfma"])
-def tq1_rows_kernel(request, monkeypatch):
+def tq1_rows_kernel(request, tune):
     """More than 8 rows per expert: the fp8 x fp4 grouped GEMM; BP_TUNE_TQ1=mfma keeps the older 16-token kernel covered."""
-    if request.param == "mfma":
-        monkeypatch.setenv("BP_TUNE_TQ1", "mfma")
-    else:
-        monkeypatch.delenv("BP_TUNE_TQ1", raising=False)
+    tune("BP_TUNE_TQ1", "mfma" if request.param == "mfma" else None)
     return request.param + "_tq1"
 
 
@@ -275,7 +269,7 @@ def test_tq1_fp4_upper_bound_max_rows(bp):
     _check(got, want)
 
 
-def test_tq1_small_batches_other_kernels(bp, monkeypatch):
+def test_tq1_small_batches_other_kernels(bp, tune):
     """fp16 activations (11 significant bits: more than two fp8 pieces hold) and K that would take more than 4 segments
     go to the kernels they went to before; the development switch keeps the multi-row MFMA kernel. K = 16384 with 4
     tokens runs as two segments of 13 chunks, with 8 tokens as four of 7 (the last one 5)."""
@@ -291,7 +285,7 @@ def test_tq1_small_batches_other_kernels(bp, monkeypatch):
     got, want, kern = _run(bp, "tq1", 2, 32, 20480, [7, 8], "bf16", seed=25)  # 32 chunks: 5 segments of 7
     assert not kern.startswith("fp4_tq1"), kern
     _check(got, want)
-    monkeypatch.setenv("BP_TUNE_TQ1", "mfma")
+    tune("BP_TUNE_TQ1", "mfma")
     got, want, kern = _run(bp, "tq1", 3, 80, 2048, [2, 4, 1], "bf16", seed=23)
     assert kern.startswith("mfma_tq1"), kern
     _check(got, want)
@@ -303,11 +297,11 @@ def test_tq1_fp4_small_batches_misaligned_scales(bp):
     _check(got, want)
 
 
-def test_tq1_mfma_scales_from_global_memory(bp, monkeypatch):
+def test_tq1_mfma_scales_from_global_memory(bp, tune):
     got, want, kern = _run(bp, "tq1", 2, 32, 2048, [9, 4], "bf16", seed=8, misalign_scales=True)
     assert kern.startswith("gemm_tq1"), kern
     _check(got, want)
-    monkeypatch.setenv("BP_TUNE_TQ1", "mfma")
+    tune("BP_TUNE_TQ1", "mfma")
     got, want, kern = _run(bp, "tq1", 2, 32, 2048, [9, 4], "bf16", seed=8, misalign_scales=True)
     assert kern.startswith("mfma_tq1") and kern.endswith("_gs"), kern
     _check(got, want)
@@ -445,3 +439,41 @@ def test_group_256(bp, act, fmt, K, counts, prefix):
     got, want, kern = _run(bp, fmt, 3, 272, K, counts, act, terms=2, seed=K + sum(counts), group=256)
     assert kern.startswith(prefix), kern
     _check(got, want)
+
+
+# --------------------------------------------------------------------------- activations that are not finite
+@pytest.mark.parametrize("fmt,counts,prefix", [
+    ("tq1", [1, 1], "fp4_tq1_t1"), ("tq1", [4, 3], "fp4_tq1_m4"), ("tq1", [20, 12], "gemm_tq1"),
+    ("tq2", [1, 1], "mfma_tq2"), ("tq2", [9, 16], "mfma_tq2"), ("tq2", [40, 33], "gemm_tq2"),
+])
+def test_non_finite_activations_never_give_finite_wrong_values(bp, fmt, counts, prefix):
+    """The reference's CPU kernel skips zero weights (boilerplate/kernels/csrc/boilerplate_cpu.cpp:70-77), so a NaN or an
+    infinite activation makes exactly the outputs with a nonzero weight at that k non-finite. The tuned kernels multiply
+    zeros too (0 x Inf = NaN) or scale whole blocks: they may make more outputs of that token non-finite, but every
+    output the reference makes non-finite must be non-finite here, and tokens without such an activation are untouched."""
+    E, N, K = 2, 64, 2048
+    rng = np.random.default_rng(5)
+    packed, scales = synth_weights(17, E, N, K, GROUP, fmt)
+    trits = np.stack([orc.unpack(packed[0][e], fmt, K) for e in range(E)])
+    offsets = np.concatenate([[0], np.cumsum(counts)]).astype(np.int64)
+    T = int(offsets[-1])
+    x = orc.bf16_round(rng.standard_normal((T, K)).astype(np.float32))
+    bad_tok = [0, T - 1]  # the first token of expert 0 gets a NaN, the last token of expert 1 an infinity
+    x[0, 777] = np.nan
+    x[T - 1, 130] = np.inf
+    got = bp.grouped_ternary_gemm(dev(x).to(torch.bfloat16), None, offsets.tolist(), [dev(packed[0])], [dev(scales[0])], K, GROUP, fmt).cpu().numpy()
+    assert bp.ext().last_kernel().startswith(prefix), bp.ext().last_kernel()
+    assert not np.isfinite(got[0, trits[0][:, 777] != 0]).any()
+    assert not np.isfinite(got[T - 1, trits[1][:, 130] != 0]).any()
+    clean = np.setdiff1d(np.arange(T), bad_tok)
+    if clean.size:
+        want = np.zeros((T, N), np.float32)
+        for e in range(E):
+            a, b = int(offsets[e]), int(offsets[e + 1])
+            c_gemm(np.nan_to_num(x[a:b], nan=0.0, posinf=0.0), None, packed[0][e], scales[0][e].astype(np.float32), K, GROUP, fmt, out=want[a:b])
+        assert np.isfinite(got[clean]).all()
+        assert rel_l2(got[clean], want[clean]) <= REL_L2
+    # the reference-order kernel skips zero weights exactly like the reference
+    ref = bp.grouped_ternary_gemm(dev(x), None, offsets.tolist(), [dev(packed[0])], [dev(scales[0])], K, GROUP, fmt, backend="torch").cpu().numpy()
+    assert np.array_equal(~np.isfinite(ref[0]), trits[0][:, 777] != 0)
+    assert np.array_equal(~np.isfinite(ref[T - 1]), trits[1][:, 130] != 0)

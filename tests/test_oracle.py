@@ -197,3 +197,24 @@ def test_moe_layer_matches_per_token_dense():
             h = orc.silu(x[t] @ g.T) * (x[t] @ u.T)
             want[t] += (h @ d.T) * scores[t, e]
     assert np.linalg.norm(got - want) / np.linalg.norm(want) < 2e-2  # bf16 rounding at every stage
+
+
+def test_absmean_ternary_known_answers():
+    """The literal known-answer test of the reference (tests/test_qat.py:11-17: a short last group and an all-zero row),
+    then cases that closed forms fix: small integers (every sum exact in any order), the clamp, ties to even."""
+    w = np.array([[0.0, -2.0, 4.0, 3.0, -1.0], [0.0, 0.0, 0.0, 0.0, 0.0]], np.float32)
+    trits, scale = orc.absmean_ternary(w, 3)
+    assert np.array_equal(scale, np.array([[2.0, 2.0], [0.0, 0.0]], np.float32))
+    assert np.array_equal(trits, np.array([[0, -1, 1, 1, 0], [0, 0, 0, 0, 0]], np.int8))
+    # group mean 2: w / s = 0.5, 1.5, -0.5, -2.5 -> rint (ties to even) 0, 2, -0, -2 -> clamp 0, 1, 0, -1
+    trits, scale = orc.absmean_ternary(np.array([[1.0, 3.0, -1.0, -5.0, 1.0, 1.0, 2.0, 2.0]], np.float32), 8)
+    assert scale[0, 0] == 2.0 and np.array_equal(trits[0], [0, 1, 0, -1, 0, 0, 1, 1])
+    # the scale is rounded to the stored format BEFORE the division: mean 1/3 -> fp16 0.33325195, bf16 0.333984375
+    w = np.array([[1.0, 0.0, 0.0, 0.1666, 0.1667, 0.0]], np.float32)
+    for dt, s in (("f16", np.float32(np.float16(1 / 3))), ("bf16", orc.bf16_round(np.array([1 / 3], np.float32))[0])):
+        trits, scale = orc.absmean_ternary(w[:, :3], 3, dt)
+        assert scale[0, 0] == s and np.array_equal(trits[0], [1, 0, 0])
+    with pytest.raises(ValueError):
+        orc.absmean_ternary(np.zeros((2, 0), np.float32), 3)
+    with pytest.raises(ValueError):
+        orc.absmean_ternary(np.zeros((2, 4), np.float32), 0)
