@@ -2,9 +2,12 @@
 
     python bench.py [--gpus 1] [--steps K] [--warmup W] [--spin-up SECONDS] [--workload NAME] [--no-extras] [--no-cpu]
 
-A step is one pass of the hot path over one batch of synthetic input: one grouped launch that
-streams L distinct packed linears of the named configuration (L chosen so the packed weights exceed
-the 256 MB Infinity Cache, i.e. every step reads its weights from HBM). Inputs are resident in HBM
+A step is one pass of the hot path over one batch of synthetic input. For the decode workloads (the default is
+BASELINE config 1: TQ1, K = 7168, N = 2048, one token, bf16) it is one grouped launch that streams L distinct packed
+linears of the named configuration (L chosen so the packed weights exceed the 256 MB Infinity Cache, i.e. every step
+reads its weights from HBM). `--workload cfg3_grouped` times the grouped-expert GEMM of config 3 (value in TFLOP/s,
+roofline against the bf16 MFMA peak), `--workload cfg2_moe_T{1,32,256}` one routed-expert layer of config 2; these
+single-workload runs are also what counter collection (rocprofv3 --pmc) is run on. Inputs are resident in HBM
 before the timed region. Every timed launch sequence is preceded by --spin-up seconds (default 0.3) of the same
 launch, untimed, then the W warm-up steps: an idle device runs its first milliseconds of work at lower clocks.
 Prints ONE JSON line:
@@ -36,9 +39,37 @@ HBM_PEAK_GBPS = 8000.0
 MFMA_BF16_PEAK_TFLOPS = 2500.0
 GROUP = 128
 
-# HBM bytes per launch measured with rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE on this command line (each
-# counter scaled by what it reads for a plain 1 GiB device copy); the summaries are under profiles/.
-MEASURED_TRAFFIC_BYTES = {"cfg1a_tq1_gemv": 522121318, "cfg1a_tq2_gemv": 516034150, "cfg1a_tq2_i8_gemv": 508708761}
+# HBM bytes per launch measured with rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE (each counter scaled by what it reads for a
+# plain 1 GiB device copy) are kept in profiles/hbm_traffic.json, keyed by workload, with the kernel they were
+# measured on: the figure is only printed while that kernel is still the one the launch runs.
+TRAFFIC_FILE = ROOT / "profiles" / "hbm_traffic.json"
+
+
+def measured_traffic(workload, kernel):
+    try:
+        rec = json.loads(TRAFFIC_FILE.read_text()).get(workload)
+    except (OSError, ValueError):
+        return None
+    if not rec or rec.get("kernel") != kernel:
+        return None
+    return int(rec["fetch_bytes"]) + int(rec["write_bytes"])
+
+
+def arithmetic_of(kernel):
+    """What the kernel named by bp_last_kernel() multiplies in (the `dtype` field of the line is the activation type)."""
+    if kernel.startswith("fp4_tq1_t1"):
+        return "activations as 3 E4M3 pieces under a per-group power-of-two prescale x E2M1 weights (v_mfma_f32_16x16x128_f8f6f4), fp32 accumulate, fp16 scale per 128-group applied in fp32"
+    if kernel.startswith("fp4_tq1_m"):
+        return "activations as 2 E4M3 pieces under a per-group power-of-two prescale x E2M1 weights (v_mfma_f32_16x16x128_f8f6f4), fp32 accumulate"
+    if kernel.startswith("gemm_tq1"):
+        return "activations as 2 E4M3 pieces under E8M0 block scales (blocks of 20) x E2M1 weights (v_mfma_scale_f32_16x16x128_f8f6f4), fp32 accumulate, scale per 128-group applied in fp32"
+    if kernel.startswith(("mfma_tq2_bf16", "gemm_tq2_bf16", "mfma_tq1")):
+        return "bf16 activations x bf16-decoded trits (v_mfma_f32_16x16x32_bf16), fp32 accumulate, scale per 128-group applied in fp32"
+    if kernel.startswith(("mfma_tq2_i8", "gemm_tq2_i8")):
+        return "int8 activations x int8 digits (v_mfma_i32_16x16x64_i8), exact int32 group sums, scales applied in fp32"
+    if kernel.startswith("lut_tq1"):
+        return "fp32 partial-sum tables, fp32 accumulate"
+    return "fp32 (reference operation order)"
 
 SPIN_UP_S = 0.3  # untimed repetitions of a launch before its warm-up and timed steps (see Launch.time)
 
@@ -49,6 +80,9 @@ WORKLOADS = {
     "cfg1a_tq1_m2": ("tq1", 2048, 7168, 2, "bf16", 1, 128),
     "cfg1a_tq1_m4": ("tq1", 2048, 7168, 4, "bf16", 1, 128),
     "cfg1a_tq1_m16": ("tq1", 2048, 7168, 16, "bf16", 1, 128),
+    "cfg1a_tq1_m32": ("tq1", 2048, 7168, 32, "bf16", 1, 128),
+    "cfg1b_tq1_m16": ("tq1", 7168, 2048, 16, "bf16", 1, 128),
+    "cfg1b_tq1_m32": ("tq1", 7168, 2048, 32, "bf16", 1, 128),
     "cfg1a_tq2_m16": ("tq2", 2048, 7168, 16, "bf16", 1, 128),
     "cfg1a_tq2_gemv": ("tq2", 2048, 7168, 1, "bf16", 1, 128),
     "cfg0_tq2_gemv": ("tq2", 2048, 4096, 1, "bf16", 1, 192),
@@ -207,6 +241,86 @@ def skewed_offsets(torch, T, E, k, seed=0):
     return idx
 
 
+def cfg3_grouped_launch(bp, torch):
+    """The grouped-expert prefill GEMM of config 3: TQ2, two stacked terms, all 384 experts, 2048 tokens top-6 (skewed routing)."""
+    from deepseekternarized_amd.kernels.ternary_hip import gather_rows
+
+    E3, N3, K3, T3, k3 = 384, 2048, 4096, 2048, 6
+    packed, scales = synth(bp, torch, E3, N3, K3, "tq2", 2, seed=3)
+    ids = skewed_offsets(torch, T3, E3, k3, seed=3)
+    order, offsets = bp.sort_by_expert(ids, E3)
+    xg = gather_rows(torch.randn(T3, K3, device="cuda").to(torch.bfloat16), order, k3)
+    max_rows = int((offsets[1:] - offsets[:-1]).max())
+    launch = Launch(bp, torch, packed, scales, K3, "tq2", xg, offsets, max_rows)
+    flops = 2.0 * T3 * k3 * N3 * K3 * 2  # per-term count
+    desc = (f"cfg3 gate projection, E={E3} experts: TQ2 k=2, N={N3}, K={K3}, {T3 * k3} routed rows (max {max_rows}/expert), "
+            "bf16 activations")
+    return launch, flops, weight_bytes(packed, scales), desc, (packed, scales)
+
+
+def cfg2_moe(bp, torch):
+    """One MoE layer of config 2 (TQ1, H=4096, I=2048, 64 experts, top-6, bf16 activations) as a TernaryMoE."""
+    from deepseekternarized_amd.moe import TernaryMoE
+
+    H2, I2, E2, k2 = 4096, 2048, 64, 6
+    gate = synth(bp, torch, E2, I2, H2, "tq1", 1, seed=5)
+    up = synth(bp, torch, E2, I2, H2, "tq1", 1, seed=6)
+    down = synth(bp, torch, E2, H2, I2, "tq1", 1, seed=7)
+    layer_bytes = sum(weight_bytes(*m) for m in (gate, up, down))
+    moe = TernaryMoE([(gate[0][0], gate[1][0])], [(up[0][0], up[1][0])], [(down[0][0], down[1][0])], H2, I2, k2, "tq1", GROUP, act="bf16")
+    return moe, layer_bytes, (H2, I2, E2, k2)
+
+
+def emit(line) -> int:
+    print(json.dumps(line))
+    return 0
+
+
+def run_cfg3_grouped(bp, torch, a) -> int:
+    launch, flops, wbytes, desc, _ = cfg3_grouped_launch(bp, torch)
+    wall, kern, kname = launch.time(a.steps, a.warmup)
+    return emit({
+        "metric": "ternary GEMV HBM GB/s (% peak); grouped-expert GEMM TFLOP/s (% MFMA peak)",
+        "value": round(flops / wall / 1e12, 1), "unit": "TFLOP/s", "n_gpus": 1, "steps": a.steps, "warmup": a.warmup,
+        "ms_per_step": round(wall * 1e3, 5), "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+        "dtype": "bf16", "data": "synthetic",
+        "config": {"workload": "cfg3_grouped: " + desc, "kernel": kname, "arithmetic": arithmetic_of(kname),
+                   "flops_counted": "2 x routed rows x N x K per term (two terms)", "device_spin_up_s": SPIN_UP_S,
+                   "retimed_after_stall": launch.retimed, "weight_GBps": round(wbytes / kern / 1e9, 1)},
+        "roofline": {"bound": "mfma", "achieved": round(flops / kern / 1e12, 1), "peak": MFMA_BF16_PEAK_TFLOPS, "unit": "TFLOP/s",
+                     "frac": round(flops / kern / 1e12 / MFMA_BF16_PEAK_TFLOPS, 4), "traffic": measured_traffic("cfg3_grouped", kname),
+                     "kernel_us": round(kern * 1e6, 2)},
+        "cpu_baseline": None, "also": {}})
+
+
+def run_cfg2_moe(bp, torch, a, T2) -> int:
+    moe, layer_bytes, (H2, I2, E2, k2) = cfg2_moe(bp, torch)
+    gm = torch.Generator(device="cuda").manual_seed(8)
+    xt = torch.randn(T2, H2, device="cuda", generator=gm).to(torch.bfloat16)
+    lg = torch.randn(T2, E2, device="cuda", generator=gm) * 1.5
+    t_end = time.perf_counter() + SPIN_UP_S
+    while time.perf_counter() < t_end:
+        moe(xt, lg)
+        torch.cuda.synchronize()
+    dt = wall_per_call(torch, lambda: moe(xt, lg), a.steps, a.warmup)
+    active = int(torch.unique(torch.topk(torch.softmax(lg.float(), -1), k2, -1).indices).numel())
+    kname = bp.ext().last_kernel()
+    abytes = layer_bytes / E2 * active
+    return emit({
+        "metric": "ternary GEMV HBM GB/s (% peak); grouped-expert GEMM TFLOP/s (% MFMA peak)",
+        "value": round(abytes / dt / 1e9, 1), "unit": "GB/s", "n_gpus": 1, "steps": a.steps, "warmup": a.warmup,
+        "ms_per_step": round(dt * 1e3, 5), "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+        "dtype": "bf16", "data": "synthetic",
+        "config": {"workload": f"cfg2_moe_T{T2}: TQ1 MoE layer H={H2} I={I2} E={E2} top-{k2}, {T2} tokens, bf16 activations: softmax/top-k, sort, "
+                               f"gather, gate|up grouped GEMM, SwiGLU, down grouped GEMM, weighted combine; {active} active experts",
+                   "kernel": kname, "arithmetic": arithmetic_of(kname), "bytes_counted": "packed + fp16 scales of the active experts",
+                   "device_spin_up_s": SPIN_UP_S},
+        "roofline": {"bound": "hbm", "achieved": round(abytes / dt / 1e9, 1), "peak": HBM_PEAK_GBPS, "unit": "GB/s",
+                     "frac": round(abytes / dt / 1e9 / HBM_PEAK_GBPS, 4), "traffic": None, "layer_us": round(dt * 1e6, 2),
+                     "note": "whole layer (a dozen launches) by wall clock, not one kernel"},
+        "cpu_baseline": None, "also": {}})
+
+
 def main() -> int:
     global SPIN_UP_S
     ap = argparse.ArgumentParser(description=__doc__.split("\n\n")[0])
@@ -214,7 +328,7 @@ def main() -> int:
     ap.add_argument("--steps", type=int, default=200)
     ap.add_argument("--warmup", type=int, default=20)
     ap.add_argument("--spin-up", type=float, default=SPIN_UP_S, help="seconds of untimed launches before warm-up and timed steps (0: none, for counter runs)")
-    ap.add_argument("--workload", default="cfg1a_tq1_gemv", choices=sorted(WORKLOADS))
+    ap.add_argument("--workload", default="cfg1a_tq1_gemv", choices=sorted(WORKLOADS) + ["cfg3_grouped", "cfg2_moe_T1", "cfg2_moe_T32", "cfg2_moe_T256"])
     ap.add_argument("--no-extras", action="store_true", help="skip the secondary measurements")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline")
     ap.add_argument("--calibrate-copy", action="store_true",
@@ -241,6 +355,10 @@ def main() -> int:
         print(json.dumps({"calibration": "device copy", "bytes_read": 1 << 30, "bytes_written": 1 << 30, "steps": a.steps}))
         return 0
     SPIN_UP_S = max(0.0, a.spin_up)
+    if a.workload == "cfg3_grouped":
+        return run_cfg3_grouped(bp, torch, a)
+    if a.workload.startswith("cfg2_moe_T"):
+        return run_cfg2_moe(bp, torch, a, int(a.workload[len("cfg2_moe_T"):]))
     fmt, N, K, M, act, terms, L = WORKLOADS[a.workload]
     launch, wbytes = uniform_launch(bp, torch, fmt, N, K, M, act, terms, L)
     wall, kern, kname = launch.time(a.steps, a.warmup)
@@ -274,15 +392,7 @@ def main() -> int:
         also["single_linear_weight_GBps"] = round(wb1 / w1 / 1e9, 1)
         del l1
         # one MoE layer of config 2 (TQ1, H=4096, I=2048, 64 experts, top-6, bf16 activations) through TernaryMoE
-        from deepseekternarized_amd.moe import TernaryMoE
-
-        H2, I2, E2, k2 = 4096, 2048, 64, 6
-        gate = synth(bp, torch, E2, I2, H2, "tq1", 1, seed=5)
-        up = synth(bp, torch, E2, I2, H2, "tq1", 1, seed=6)
-        down = synth(bp, torch, E2, H2, I2, "tq1", 1, seed=7)
-        layer_bytes = sum(weight_bytes(*m) for m in (gate, up, down))
-        moe = TernaryMoE([(gate[0][0], gate[1][0])], [(up[0][0], up[1][0])], [(down[0][0], down[1][0])], H2, I2, k2, "tq1", GROUP, act="bf16")
-        del gate, up, down
+        moe, layer_bytes, (H2, I2, E2, k2) = cfg2_moe(bp, torch)
         gm = torch.Generator(device="cuda").manual_seed(8)
         cfg2 = {}
         for T2 in (1, 32, 256):
@@ -305,23 +415,12 @@ def main() -> int:
         torch.cuda.empty_cache()
         # grouped-expert prefill GEMM of config 3: TQ2, two stacked terms, all 384 experts, 2048 tokens top-6 (skewed routing)
         E3, N3, K3, T3, k3 = 384, 2048, 4096, 2048, 6
-        packed, scales = synth(bp, torch, E3, N3, K3, "tq2", 2, seed=3)
-        ids = skewed_offsets(torch, T3, E3, k3, seed=3)
-        order, offsets = bp.sort_by_expert(ids, E3)
-        from deepseekternarized_amd.kernels.ternary_hip import gather_rows
-
-        xg = gather_rows(torch.randn(T3, K3, device="cuda").to(torch.bfloat16), order, k3)
-        max_rows = int((offsets[1:] - offsets[:-1]).max())
-        l3 = Launch(bp, torch, packed, scales, K3, "tq2", xg, offsets, max_rows)
+        l3, flops, wb3, desc3, (packed, scales) = cfg3_grouped_launch(bp, torch)
         _, k3t, kn3 = l3.time(max(5, a.steps // 2), 2)
-        flops = 2.0 * T3 * k3 * N3 * K3 * 2  # per-term count
-        also["grouped_gemm"] = {"workload": f"cfg3 gate projection, E={E3} experts: TQ2 k=2, N={N3}, K={K3}, "
-                                            f"{T3 * k3} routed rows (max {max_rows}/expert), bf16 activations",
-                                "TFLOPs_per_term_count": round(flops / k3t / 1e12, 1),
+        also["grouped_gemm"] = {"workload": desc3, "TFLOPs_per_term_count": round(flops / k3t / 1e12, 1),
                                 "frac_of_bf16_mfma_peak": round(flops / k3t / 1e12 / MFMA_BF16_PEAK_TFLOPS, 4),
-                                "weight_GBps": round(weight_bytes(packed, scales) / k3t / 1e9, 1), "kernel": kn3,
-                                "us": round(k3t * 1e6, 1)}
-        del l3, xg
+                                "weight_GBps": round(wb3 / k3t / 1e9, 1), "kernel": kn3, "us": round(k3t * 1e6, 1)}
+        del l3
         # ... and the whole routed-expert layer of config 3 (gate | up, SwiGLU, down, combine) on the same gate stack
         from deepseekternarized_amd.moe import TernaryMoE
 
@@ -345,12 +444,15 @@ def main() -> int:
         from deepseekternarized_amd.decoder_harness import DecoderConfig, TernaryDecoder, bench_decoder
 
         cfg = DecoderConfig()
-        r = bench_decoder(TernaryDecoder(cfg), 64, 128, 32)
+        model = TernaryDecoder(cfg)
+        r = bench_decoder(model, 64, 128, 128)
+        rg = bench_decoder(model, 64, 128, 128, graph=True)  # the same decode steps replayed as one HIP graph each
         also["decoder_harness"] = {"workload": f"{cfg.layers} layers, hidden {cfg.hidden}, {cfg.experts} experts top-{cfg.top_k}, "
                                                f"inter {cfg.inter}, {cfg.fmt.upper()}, {cfg.act} activations, random weights; "
-                                               "batch 64, prompt 128, 32 greedy decode steps",
+                                               "batch 64, prompt 128, 128 greedy decode steps",
                                    "prefill_tok_s": r["prefill_tok_s"], "decode_tok_s": r["decode_tok_s"],
-                                   "peak_vram_bytes": r["peak_vram_bytes"], "finite": r["finite"]}
+                                   "decode_tok_s_hip_graph": rg["decode_tok_s"],
+                                   "peak_vram_bytes": r["peak_vram_bytes"], "finite": r["finite"] and rg["finite"]}
 
     line = {
         "metric": "ternary GEMV HBM GB/s (% peak); grouped-expert GEMM TFLOP/s (% MFMA peak)",
@@ -359,17 +461,16 @@ def main() -> int:
         "dtype": "bf16", "data": "synthetic",
         "config": {"workload": f"{a.workload}: {fmt.upper()} decode GEMV N={N} K={K} M={M} {act} activations, group 128, "
                                f"fp16 scales, {L} distinct linears per launch ({wbytes / 1e6:.0f} MB of weights, > Infinity Cache)",
-                   "kernel": kname, "bytes_counted": "packed + fp16 scales as stored", "device_spin_up_s": SPIN_UP_S, "retimed_after_stall": retimed,
+                   "kernel": kname, "arithmetic": arithmetic_of(kname), "bytes_counted": "packed + fp16 scales as stored", "device_spin_up_s": SPIN_UP_S, "retimed_after_stall": retimed,
                    "packed_only_GBps": round(wbytes * (1.0 - 2.0 * (K // GROUP) / (bp.packed_cols(fmt, K) + 2.0 * (K // GROUP))) / kern / 1e9, 1),
                    "activation_and_output_bytes_per_step": act_bytes},
         "roofline": {"bound": "hbm", "achieved": round(wbytes / kern / 1e9, 1), "peak": HBM_PEAK_GBPS, "unit": "GB/s",
-                     "frac": round(wbytes / kern / 1e9 / HBM_PEAK_GBPS, 4), "traffic": MEASURED_TRAFFIC_BYTES.get(a.workload),
+                     "frac": round(wbytes / kern / 1e9 / HBM_PEAK_GBPS, 4), "traffic": measured_traffic(a.workload, kname),
                      "kernel_us": round(kern * 1e6, 2)},
         "cpu_baseline": None if a.no_cpu else cpu_baseline(fmt, N, K, M),
         "also": also,
     }
-    print(json.dumps(line))
-    return 0
+    return emit(line)
 
 
 if __name__ == "__main__":

@@ -136,8 +136,102 @@ class TernaryDecoder:
         return F.linear(x, self.head).float(), new_past
 
 
-def bench_decoder(model: TernaryDecoder, batch: int, prompt_len: int, gen_len: int, seed: int = 0) -> dict:
-    """The timing loop of ``boilerplate bench`` (cli.py:161-184): 8-token warm-up, timed prefill, greedy decode."""
+class GraphedDecode:
+    """Greedy decoding of one token per sequence as ONE HIP graph replay per step.
+
+    A decode step of this model is about forty kernel launches per layer, each a few microseconds of device time, so
+    issued one by one from Python the step is bound by the host. The step is therefore written with static shapes -
+    a KV cache preallocated to ``max_len`` positions, the current length held in a device scalar, attention over all
+    ``max_len`` positions with the unwritten ones masked - and captured once; ``step()`` replays it. Batches up to 64
+    sequences (the routed-expert layer needs no host read-back up to there). The eager path (``forward`` with a
+    concatenated cache, as the reference's engine does it) stays the reference for this one: same kernels, same
+    rounding points; only the softmax rows are longer (masked tail), which can move its float32 sum by an ulp."""
+
+    def __init__(self, model: TernaryDecoder, cache, max_len: int):
+        cfg = model.cfg
+        self.model, self.max_len = model, max_len
+        b, h, n, d = cache[0][0].shape
+        if not 1 <= b <= 64:
+            raise ValueError("graphed decoding covers batches of 1..64 sequences")
+        if n >= max_len:
+            raise ValueError("max_len must exceed the cached length")
+        dev = cache[0][0].device
+        self.k = [torch.zeros(b, h, max_len, d, dtype=k.dtype, device=dev) for k, _ in cache]
+        self.v = [torch.zeros(b, h, max_len, d, dtype=v.dtype, device=dev) for _, v in cache]
+        for i, (k, v) in enumerate(cache):
+            self.k[i][:, :, :n].copy_(k)
+            self.v[i][:, :, :n].copy_(v)
+        self.pos = torch.full((1,), n, dtype=torch.int64, device=dev)  # positions written so far = index of the next one
+        self.ids = torch.zeros(b, dtype=torch.int64, device=dev)
+        pos_all = torch.arange(max_len, dtype=torch.float32, device=dev)
+        inv = cfg.theta ** (-torch.arange(0, model.head_dim, 2, dtype=torch.float32, device=dev) / model.head_dim)
+        fr = torch.outer(pos_all, inv)
+        ang = torch.cat((fr, fr), dim=-1)
+        self.cos, self.sin = ang.cos().to(model.dtype), ang.sin().to(model.dtype)  # [max_len, head_dim]
+        self.arange = torch.arange(max_len, device=dev)
+        self.logits = None
+        side = torch.cuda.Stream(device=dev)
+        side.wait_stream(torch.cuda.current_stream(dev))
+        with torch.cuda.stream(side):  # warm-up outside the capture (kernel attributes, cached offsets, allocator state)
+            saved = (self.pos.clone(), [k.clone() for k in self.k], [v.clone() for v in self.v])
+            for _ in range(2):
+                self._step()
+            self.pos.copy_(saved[0])
+            for i in range(len(self.k)):
+                self.k[i].copy_(saved[1][i])
+                self.v[i].copy_(saved[2][i])
+            del saved
+        torch.cuda.current_stream(dev).wait_stream(side)
+        torch.cuda.synchronize(dev)
+        self.graph = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(self.graph):
+            self.logits = self._step()
+
+    @torch.inference_mode()
+    def _step(self):
+        m, cfg = self.model, self.model.cfg
+        x = F.embedding(self.ids[:, None], m.embedding).to(m.dtype)  # [b, 1, H]
+        cos, sin = self.cos.index_select(0, self.pos)[None, None], self.sin.index_select(0, self.pos)[None, None]
+        mask = (self.arange > self.pos)[None, None, None, :]  # positions not written yet
+
+        def rot(t):
+            a, b = t.chunk(2, dim=-1)
+            return torch.cat((-b, a), dim=-1)
+
+        for index, layer in enumerate(m.layers):
+            residual = x
+            z = m._norm(x, layer.input_norm)
+            q, k, v = m.linear(layer.q, z), m.linear(layer.k, z), m.linear(layer.v, z)
+            b = q.size(0)
+            q = q.view(b, 1, cfg.heads, m.head_dim).transpose(1, 2)
+            k = k.view(b, 1, cfg.heads, m.head_dim).transpose(1, 2)
+            v = v.view(b, 1, cfg.heads, m.head_dim).transpose(1, 2)
+            q, k = q * cos + rot(q) * sin, k * cos + rot(k) * sin
+            self.k[index].index_copy_(2, self.pos, k)
+            self.v[index].index_copy_(2, self.pos, v)
+            scores = (q @ self.k[index].transpose(-2, -1)) / math.sqrt(m.head_dim)
+            scores = scores.masked_fill(mask, torch.finfo(scores.dtype).min)
+            attention = torch.softmax(scores, dim=-1, dtype=torch.float32).to(q.dtype) @ self.v[index]
+            x = residual + m.linear(layer.o, attention.transpose(1, 2).reshape(b, 1, -1).contiguous())
+            residual = x
+            z = m._norm(x, layer.post_norm)
+            x = residual + m.moe(layer, z)
+        x = m._norm(x, m.final_norm)
+        logits = F.linear(x, m.head).float()[:, 0]
+        self.pos.add_(1)
+        return logits
+
+    def step(self, ids: torch.Tensor) -> torch.Tensor:
+        """ids [batch] (the tokens just chosen) -> float32 logits [batch, vocab] of the next position (the graph's
+        output buffer: overwritten by the next step)."""
+        self.ids.copy_(ids)
+        self.graph.replay()
+        return self.logits
+
+
+def bench_decoder(model: TernaryDecoder, batch: int, prompt_len: int, gen_len: int, seed: int = 0, graph: bool = False) -> dict:
+    """The timing loop of ``boilerplate bench`` (cli.py:161-184): 8-token warm-up, timed prefill, greedy decode.
+    ``graph``: the decode steps as HIP graph replays (:class:`GraphedDecode`; capture is outside the timed region)."""
     g = torch.Generator().manual_seed(seed)
     prompts = torch.randint(0, model.cfg.vocab, (batch, prompt_len), generator=g)
     model.forward(prompts[:, :8])
@@ -147,13 +241,20 @@ def bench_decoder(model: TernaryDecoder, batch: int, prompt_len: int, gen_len: i
     torch.cuda.synchronize()
     t_pre = time.perf_counter() - t0
     nxt = logits[:, -1].argmax(-1)
+    if graph:
+        dec = GraphedDecode(model, cache, prompt_len + gen_len + 1)
+        torch.cuda.synchronize()
     t0 = time.perf_counter()
     for _ in range(gen_len):
-        logits, cache = model.forward(nxt[:, None], cache)
-        nxt = logits[:, -1].argmax(-1)
+        if graph:
+            logits = dec.step(nxt)
+            nxt = logits.argmax(-1)
+        else:
+            logits, cache = model.forward(nxt[:, None], cache)
+            nxt = logits[:, -1].argmax(-1)
     torch.cuda.synchronize()
     t_dec = time.perf_counter() - t0
-    return {"batch": batch, "prompt_len": prompt_len, "gen_len": gen_len,
+    return {"batch": batch, "prompt_len": prompt_len, "gen_len": gen_len, "decode_as_hip_graph": bool(graph),
             "prefill_tok_s": round(batch * prompt_len / t_pre, 2),
             "decode_tok_s": round(batch * gen_len / t_dec, 3) if gen_len else None,
             "prefill_s": round(t_pre, 4), "decode_s": round(t_dec, 4),
