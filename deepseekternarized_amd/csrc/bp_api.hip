@@ -129,11 +129,19 @@ extern "C" int bp_ternary_grouped_gemm(float* out, const void* x, int x_dtype, c
   a.x_dtype = x_dtype; a.scale_dtype = scale_dtype; a.n_terms = n_terms; a.fmt = fmt;
   a.T = T; a.N = N; a.K = K; a.Kp = Kp; a.G = G; a.group = group; a.E = E; a.max_rows = max_rows;
 
-  hipStream_t s = (hipStream_t)stream;
+  return run_gemm(a, (hipStream_t)stream);
+}
+
+namespace bp {
+int kernel_policy() { return g_policy; }
+
+int run_gemm(const GemmArgs& a, hipStream_t s) {
   if (g_policy != 1 && mfma_supports(a)) {
     const int rc = launch_mfma(a, s);
     if (rc != BP_ERR_UNSUPPORTED) return rc;  // (a tuned variant may turn a launch down, e.g. when its LDS tiles do not fit)
   }
+  if (a.tiles) return fail(BP_ERR_UNSUPPORTED, "tile-list mode needs one of the 32-token-tile kernels");
   if (g_policy == 2) return fail(BP_ERR_UNSUPPORTED, "shape is outside the tuned kernels (policy 2 forbids the general kernel)");
   return launch_general(a, s);
 }
+}  // namespace bp

@@ -25,7 +25,39 @@ struct GemmArgs {
   const void* w_scale[BP_MAX_TERMS];
   int x_dtype, scale_dtype, n_terms, fmt;
   int64_t T, N, K, Kp, G, group, E, max_rows;
+  // Tile-list mode of the 32-token-tile kernels (set by callers that keep the routing on the device, where the widest
+  // expert's row count is unknown to the host): tiles = (expert, first row) pairs of the token tiles that exist, in
+  // expert order, tile_count[0] of them (device memory, written by a kernel earlier on the stream); the launch covers
+  // tile_cap entries and workgroups past the count leave at once. NULL: token tiles are counted by blockIdx.z up to max_rows.
+  const int32_t* tiles;
+  const int32_t* tile_count;
+  int64_t tile_cap;
+  int overwrite;  // tile-list mode: the kernel's result replaces `out` instead of being added to it (one launch covers all of K and all terms)
 };
+
+__device__ __forceinline__ int64_t clamp_i64(int64_t v, int64_t lo, int64_t hi) { return v < lo ? lo : (v > hi ? hi : v); }
+
+// Which token tile of 32 rows a workgroup takes: `slot` is its expert (list entry in tile-list mode), z its token tile.
+struct TileRef {
+  int64_t e, tok0, o1;
+  bool live;
+};
+__device__ __forceinline__ TileRef tile_ref(const GemmArgs& a, int64_t slot, unsigned z) {
+  TileRef r = {0, 0, 0, false};
+  if (a.tiles) {
+    if (slot >= a.tile_count[0] || slot >= a.tile_cap) return r;
+    r.e = a.tiles[2 * slot];
+    r.tok0 = a.tiles[2 * slot + 1];
+    r.o1 = clamp_i64(a.offsets[r.e + 1], 0, a.T);
+  } else {
+    if (slot >= a.E) return r;
+    r.e = slot;
+    r.o1 = clamp_i64(a.offsets[slot + 1], 0, a.T);
+    r.tok0 = clamp_i64(a.offsets[slot], 0, a.T) + (int64_t)z * 32;
+  }
+  r.live = r.tok0 < r.o1;
+  return r;
+}
 
 // Development overrides of the kernel selection (environment variables BP_TUNE_*), read once when the library is first
 // used; bp_reload_tuning() reads them again (the tests switch kernels that way). 0 / unset = automatic.
@@ -55,6 +87,10 @@ int raise_lds_limit(int bytes) {
   return BP_OK;
 }
 
+// Kernel selection for a validated argument block (the body of bp_ternary_grouped_gemm after its checks).
+int run_gemm(const GemmArgs& a, hipStream_t s);
+// True when a launch in tile-list mode would run on one of the 32-token-tile kernels (which honour tiles / overwrite).
+bool gemm_tiles_supported(const GemmArgs& a);
 int launch_general(const GemmArgs& a, hipStream_t s);
 // Returns BP_ERR_UNSUPPORTED (without setting an error message) when the shape is outside the
 // tuned kernels' preconditions.
@@ -89,7 +125,6 @@ __device__ __forceinline__ float load_act_f32(const void* p, int dtype, int64_t 
   return dtype == BP_F16 ? f16_bits_to_f32(b) : bf16_bits_to_f32(b);
 }
 
-__device__ __forceinline__ int64_t clamp_i64(int64_t v, int64_t lo, int64_t hi) { return v < lo ? lo : (v > hi ? hi : v); }
 
 // TQ1 digit i of byte v as a trit (boilerplate/ternary/pack.py:62-67): bytes >= 243 decode to 0.
 __device__ __host__ __forceinline__ int tq1_trit(unsigned v, int i) {

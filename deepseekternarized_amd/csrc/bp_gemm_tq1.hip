@@ -72,11 +72,9 @@ __global__ __launch_bounds__(Q_THREADS, 2) void k_gemm_tq1(GemmArgs a) {
   // activations, so they get linear indices 8 apart (same XCD, one L2).
   const int row_blocks = (int)((a.N + Q_ROWS - 1) / Q_ROWS);
   const int wg_block = (int)((blockIdx.x >> 3) % (unsigned)row_blocks);
-  const int64_t e = (blockIdx.x & 7) + 8 * (int64_t)((blockIdx.x >> 3) / (unsigned)row_blocks);
-  if (e >= a.E) return;
-  const int64_t o0 = clamp_i64(a.offsets[e], 0, a.T), o1 = clamp_i64(a.offsets[e + 1], 0, a.T);
-  const int64_t tok0 = o0 + (int64_t)blockIdx.z * 32;
-  if (tok0 >= o1) return;  // uniform for the workgroup
+  const TileRef tr = tile_ref(a, (blockIdx.x & 7) + 8 * (int64_t)((blockIdx.x >> 3) / (unsigned)row_blocks), blockIdx.z);
+  if (!tr.live) return;  // uniform for the workgroup
+  const int64_t e = tr.e, tok0 = tr.tok0, o1 = tr.o1;
   const int ntok = (int)(o1 - tok0 < 32 ? o1 - tok0 : 32);
   const bool two = ntok > 16;  // the second token tile holds tokens
   const int64_t n_base = (int64_t)wg_block * Q_ROWS;
@@ -448,7 +446,7 @@ __global__ __launch_bounds__(Q_THREADS, 2) void k_gemm_tq1(GemmArgs a) {
             const int64_t row = n_wave + 16 * r;
             if (row < a.N) {
               float* o = a.out + tok * a.N + row + r16;
-              *o += total[r][t][i] * xs;
+              *o = (a.overwrite ? 0.f : *o) + total[r][t][i] * xs;
             }
           }
         }
@@ -463,7 +461,8 @@ template <int ACT, int SDT>
 int launch_gemm_tq1_k(const GemmArgs& a, hipStream_t s, const char* name) {
   if (const int rc = raise_lds_limit<k_gemm_tq1<ACT, SDT>>(q_lds_bytes(SDT == BP_F32 ? 4 : 2))) return rc;
   const int64_t row_blocks = (a.N + Q_ROWS - 1) / Q_ROWS;
-  const dim3 grid((unsigned)(row_blocks * ((a.E + 7) / 8 * 8)), 1, (unsigned)((a.max_rows + 31) / 32));
+  const int64_t slots = a.tiles ? a.tile_cap : a.E;
+  const dim3 grid((unsigned)(row_blocks * ((slots + 7) / 8 * 8)), 1, a.tiles ? 1u : (unsigned)((a.max_rows + 31) / 32));
   note_kernel(name);
   hipLaunchKernelGGL((k_gemm_tq1<ACT, SDT>), grid, dim3(Q_THREADS), q_lds_bytes(SDT == BP_F32 ? 4 : 2), s, a);
   return check_launch(name);

@@ -52,14 +52,13 @@ __global__ __launch_bounds__(GTHREADS, 2) void k_gemm_tq2(GemmArgs a) {
   const int r16 = lane & 15, b = lane >> 4;
   // Workgroups are dealt to the 8 XCDs round-robin by linear index; each XCD has its own L2. The row tiles of
   // one expert read the same activations, so they get linear indices 8 apart (same XCD, consecutive in time):
-  // linear index L -> expert (L % 8) + 8 * (L / 8 / row_tiles), row tile (L / 8) % row_tiles.
+  // linear index L -> expert (L % 8) + 8 * (L / 8 / row_tiles), row tile (L / 8) % row_tiles (tile-list mode: list entry
+  // instead of expert).
   const int row_tiles = (int)((a.N + GROWS - 1) / GROWS);
   const int wg_tile = (int)((blockIdx.x >> 3) % (unsigned)row_tiles);
-  const int64_t e = (blockIdx.x & 7) + 8 * (int64_t)((blockIdx.x >> 3) / (unsigned)row_tiles);
-  if (e >= a.E) return;
-  const int64_t o0 = clamp_i64(a.offsets[e], 0, a.T), o1 = clamp_i64(a.offsets[e + 1], 0, a.T);
-  const int64_t tok0 = o0 + (int64_t)blockIdx.z * (16 * GT);
-  if (tok0 >= o1) return;  // uniform for the workgroup
+  const TileRef tr = tile_ref(a, (blockIdx.x & 7) + 8 * (int64_t)((blockIdx.x >> 3) / (unsigned)row_tiles), blockIdx.z);
+  if (!tr.live) return;  // uniform for the workgroup
+  const int64_t e = tr.e, tok0 = tr.tok0, o1 = tr.o1;
   const int ntok = (int)(o1 - tok0 < 16 * GT ? o1 - tok0 : 16 * GT);
   const bool two = ntok > 16;  // the second token sub-tile holds tokens
   int64_t n0 = ((int64_t)wg_tile * GW + wave) * (16 * GR);
@@ -373,7 +372,7 @@ __global__ __launch_bounds__(GTHREADS, 2) void k_gemm_tq2(GemmArgs a) {
         for (int r = 0; r < GR; ++r) {
           if (rows_valid[r]) {
             float* o = a.out + tok * a.N + n0 + 16 * r + r16;
-            *o += total[r][mt][q] * xs;
+            *o = (a.overwrite ? 0.f : *o) + total[r][mt][q] * xs;
           }
         }
       }
@@ -384,7 +383,8 @@ __global__ __launch_bounds__(GTHREADS, 2) void k_gemm_tq2(GemmArgs a) {
 template <int ACT, int SDT, int SL, int ABL = 0>
 int launch_gemm_k(const GemmArgs& a, hipStream_t s, size_t lds, const char* name) {
   if (const int rc = raise_lds_limit<k_gemm_tq2<ACT, SDT, SL, ABL>>(160 * 1024)) return rc;
-  const dim3 grid((unsigned)((a.N + GROWS - 1) / GROWS * ((a.E + 7) / 8 * 8)), 1, (unsigned)((a.max_rows + 16 * GT - 1) / (16 * GT)));
+  const int64_t slots = a.tiles ? a.tile_cap : a.E;
+  const dim3 grid((unsigned)((a.N + GROWS - 1) / GROWS * ((slots + 7) / 8 * 8)), 1, a.tiles ? 1u : (unsigned)((a.max_rows + 16 * GT - 1) / (16 * GT)));
   note_kernel(name);
   hipLaunchKernelGGL((k_gemm_tq2<ACT, SDT, SL, ABL>), grid, dim3(GTHREADS), lds, s, a);
   return check_launch(name);

@@ -28,7 +28,17 @@ bool mfma_supports(const GemmArgs& a) {
   return true;
 }
 
+bool gemm_tiles_supported(const GemmArgs& a) {
+  if (!mfma_supports(a) || (a.x_dtype != BP_BF16 && a.x_dtype != BP_I8)) return false;
+  if (a.fmt == BP_TQ1) return a.K <= ((int64_t)1 << 24) && a.N * a.Kp <= ((int64_t)1 << 31) - 4096;
+  return true;
+}
+
 int launch_mfma(const GemmArgs& a, hipStream_t s) {
+  if (a.tiles) {  // tile-list mode: only the 32-token-tile kernels read the list
+    if (!gemm_tiles_supported(a)) return BP_ERR_UNSUPPORTED;
+    return a.fmt == BP_TQ1 ? launch_gemm_tq1(a, s) : launch_gemm_tq2(a, s);
+  }
   // rows per wave and waves per workgroup: keep enough workgroups in flight for small problems
   // (an expert without rows exits at once: at most min(E, T) experts do work)
   const int64_t work = (a.E < a.T ? a.E : a.T) * (a.N / 16);

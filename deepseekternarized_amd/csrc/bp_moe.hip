@@ -1,0 +1,211 @@
+// One routed-expert MoE layer as one call: sort of the routing, row gather, gate|up grouped GEMM, SwiGLU, down grouped
+// GEMM, weighted combine - the per-expert loop of boilerplate/engine/standard.py:156-176 after the router's top-k, with
+// the same rounding points (every linear rounded to bf16, products with the routing weight rounded to bf16, the sum
+// over a token's experts accumulated in bf16 in ascending expert order).
+//
+// Nothing is read back to the host. The reference sizes its grouped launch from `int(offsets.diff().max())`
+// (boilerplate/kernels/ternary_cuda.py:97), a device-to-host copy in the middle of the layer; here a kernel writes
+// the list of 32-row token tiles that exist (k_tile_list), and the grouped GEMMs run over that list. Up to 64 tokens
+// no expert can have more than 64 rows, and the launch is sized by that bound instead (the small-batch kernels).
+//
+// All intermediate tensors live in a workspace the caller provides (bp_moe_layer_workspace_bytes): the library
+// allocates nothing, so the call can be captured in a HIP graph.
+#include <string.h>
+
+#include "bp_mfma.h"
+
+namespace bp {
+int kernel_policy();  // bp_api.hip
+namespace {
+
+constexpr int TILE_ROWS = 32;  // token tile of k_gemm_tq1 / k_gemm_tq2
+
+// (expert, first row) of every 32-row token tile, in expert order; count[0] = their number. One workgroup; experts in
+// chunks of 1024 with a running total.
+__global__ __launch_bounds__(1024) void k_tile_list(int32_t* __restrict__ tiles, int32_t* __restrict__ count, const int64_t* __restrict__ offsets,
+                                                    int64_t E, int64_t T, int64_t cap) {
+  __shared__ int part[16];
+  __shared__ int carry;
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  if (threadIdx.x == 0) carry = 0;
+  __syncthreads();
+  for (int64_t base = 0; base < E; base += 1024) {
+    const int64_t e = base + threadIdx.x;
+    int64_t o0 = 0, rows = 0;
+    if (e < E) {
+      o0 = clamp_i64(offsets[e], 0, T);
+      const int64_t o1 = clamp_i64(offsets[e + 1], 0, T);
+      rows = o1 > o0 ? o1 - o0 : 0;
+    }
+    const int mine = (int)((rows + TILE_ROWS - 1) / TILE_ROWS);
+    int incl = mine;  // inclusive prefix sum within the wave
+#pragma unroll
+    for (int d = 1; d < 64; d <<= 1) {
+      const int up = __shfl_up(incl, d, 64);
+      if (lane >= d) incl += up;
+    }
+    if (lane == 63) part[wave] = incl;
+    __syncthreads();
+    int before = carry;
+    for (int w = 0; w < wave; ++w) before += part[w];
+    int64_t at = before + incl - mine;
+    for (int j = 0; j < mine; ++j, ++at) {
+      if (at < cap) {
+        tiles[2 * at] = (int32_t)e;
+        tiles[2 * at + 1] = (int32_t)(o0 + (int64_t)j * TILE_ROWS);
+      }
+    }
+    __syncthreads();
+    if (threadIdx.x == 1023) carry = before + incl;
+    __syncthreads();
+  }
+  if (threadIdx.x == 0) count[0] = carry < cap ? carry : (int)cap;
+}
+
+// inv[order[i]] = i: where pair (token, slot) sits in expert order
+__global__ __launch_bounds__(256) void k_invert(int64_t* __restrict__ inv, const int64_t* __restrict__ order, int64_t n) {
+  const int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x;
+  if (i < n) {
+    const int64_t o = order[i];
+    if (o >= 0 && o < n) inv[o] = i;
+  }
+}
+
+__global__ __launch_bounds__(256) void k_zero16(u32x4* __restrict__ p, int64_t n16) {
+  for (int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x; i < n16; i += (int64_t)gridDim.x * 256) p[i] = u32x4{0u, 0u, 0u, 0u};
+}
+
+struct Carve {
+  unsigned char* base;
+  size_t used;
+  void* take(size_t bytes) {
+    void* p = base ? base + used : nullptr;
+    used += (bytes + 255) & ~(size_t)255;
+    return p;
+  }
+};
+
+struct Plan {
+  int64_t* order;
+  int64_t* offsets;
+  int64_t* inv;
+  int32_t* sort_ws;
+  int32_t* tiles;
+  int32_t* tile_count;
+  void* xg;       // gathered rows, bf16 [T k, H]
+  int8_t* q;      // int8 activations of the wider of the two GEMM inputs
+  float* q_scale;
+  float* gu;      // f32 [T k, 2 I]
+  void* h;        // bf16 [T k, I]
+  float* y;       // f32 [T k, H]
+  int64_t tile_cap;
+  size_t bytes;
+};
+
+Plan plan(void* workspace, int64_t T, int64_t H, int64_t I, int64_t E, int64_t k, int act) {
+  Carve c = {(unsigned char*)workspace, 0};
+  Plan p;
+  const int64_t n = T * k;
+  p.order = (int64_t*)c.take(8 * (size_t)n);
+  p.offsets = (int64_t*)c.take(8 * (size_t)(E + 1));
+  p.inv = (int64_t*)c.take(8 * (size_t)n);
+  p.sort_ws = (int32_t*)c.take(4 * (size_t)bp_sort_workspace_ints(n, E));
+  p.tile_cap = (n + TILE_ROWS - 1) / TILE_ROWS + E;
+  p.tiles = (int32_t*)c.take(8 * (size_t)p.tile_cap);
+  p.tile_count = (int32_t*)c.take(4);
+  p.xg = c.take(2 * (size_t)n * H);
+  p.q = (int8_t*)c.take(act == BP_I8 ? (size_t)n * (H > I ? H : I) : 0);
+  p.q_scale = (float*)c.take(act == BP_I8 ? 4 * (size_t)n : 0);
+  p.gu = (float*)c.take(4 * (size_t)n * 2 * I);
+  p.h = c.take(2 * (size_t)n * I);
+  p.y = (float*)c.take(4 * (size_t)n * H);
+  p.bytes = c.used;
+  return p;
+}
+
+int zero(void* p, size_t bytes, hipStream_t s) {  // (a fill kernel, not a memset node: the call may be captured in a graph)
+  const int64_t n16 = (int64_t)(bytes / 16);
+  int64_t g = (n16 + 255) / 256;
+  if (g > 8192) g = 8192;
+  if (g > 0) hipLaunchKernelGGL(k_zero16, dim3((unsigned)g), dim3(256), 0, s, (u32x4*)p, n16);
+  return check_launch("zero");
+}
+
+}  // namespace
+}  // namespace bp
+
+using namespace bp;
+
+extern "C" size_t bp_moe_layer_workspace_bytes(int64_t T, int64_t H, int64_t I, int64_t E, int64_t k, int act) {
+  if (T < 0 || H <= 0 || I <= 0 || E <= 0 || k <= 0) return 0;
+  return plan(nullptr, T, H, I, E, k, act).bytes;
+}
+
+extern "C" int bp_moe_layer_bf16(void* out, const void* x, const int64_t* experts, const void* weights,
+                                 const uint8_t* const* gate_up_packed, const void* const* gate_up_scale,
+                                 const uint8_t* const* down_packed, const void* const* down_scale, int scale_dtype,
+                                 int n_terms, int64_t T, int64_t H, int64_t I, int64_t E, int64_t k, int64_t group, int fmt,
+                                 int act, void* workspace, size_t workspace_bytes, int32_t* bad, void* stream) {
+  if (T < 0 || H <= 0 || I <= 0 || E <= 0 || E > 65535 || k <= 0 || k > 64 || k > E) return fail(BP_ERR_ARG, "invalid MoE layer dimensions (experts up to 65535, top-k up to 64)");
+  if (T * k > ((int64_t)1 << 31) - 1 - 32 * E) return fail(BP_ERR_ARG, "too many routed rows for one call");
+  if (fmt != BP_TQ1 && fmt != BP_TQ2) return fail(BP_ERR_ARG, "fmt must be 1 (TQ1) or 2 (TQ2)");
+  if (act != BP_BF16 && act != BP_I8) return fail(BP_ERR_ARG, "act must be BP_BF16 or BP_I8");
+  if (scale_dtype != BP_F32 && scale_dtype != BP_F16 && scale_dtype != BP_BF16) return fail(BP_ERR_ARG, "unexpected scale dtype");
+  if (n_terms < 1 || n_terms > BP_MAX_TERMS) return fail(BP_ERR_ARG, "n_terms must be in 1..%d", BP_MAX_TERMS);
+  if (group <= 0 || group > ((int64_t)1 << 24)) return fail(BP_ERR_ARG, "invalid group");
+  if ((H % 8) != 0 || (I % 8) != 0) return fail(BP_ERR_ARG, "hidden and intermediate sizes must be multiples of 8 (16-byte rows)");
+  if (T == 0) return BP_OK;
+  if (!out || !x || !experts || !weights || !gate_up_packed || !gate_up_scale || !down_packed || !down_scale) return fail(BP_ERR_ARG, "null pointer");
+  for (int t = 0; t < n_terms; ++t)
+    if (!gate_up_packed[t] || !gate_up_scale[t] || !down_packed[t] || !down_scale[t]) return fail(BP_ERR_ARG, "null packed or scale pointer in term %d", t);
+  const Plan p = plan(workspace, T, H, I, E, k, act);
+  if (!workspace || workspace_bytes < p.bytes) return fail(BP_ERR_ARG, "the workspace must hold bp_moe_layer_workspace_bytes() = %zu bytes", p.bytes);
+  if (((uintptr_t)workspace & 255) != 0) return fail(BP_ERR_ARG, "the workspace must be 256-byte aligned");
+  hipStream_t s = (hipStream_t)stream;
+  const int64_t n = T * k;
+  const int per = fmt == BP_TQ2 ? 4 : 5;
+
+  int rc = bp_sort_by_expert(p.order, p.offsets, experts, n, E, bp_sort_workspace_ints(n, E) > 0 ? p.sort_ws : nullptr, bad, s);
+  if (rc != BP_OK) return rc;
+  hipLaunchKernelGGL(k_invert, dim3((unsigned)((n + 255) / 256)), dim3(256), 0, s, p.inv, p.order, n);
+  if ((rc = check_launch("invert")) != BP_OK) return rc;
+  if ((rc = bp_gather_rows(p.xg, x, p.order, k, n, T, 2 * H, s)) != BP_OK) return rc;
+
+  auto gemm = [&](float* o, const void* in, const uint8_t* const* packed, const void* const* scale, int64_t N, int64_t K, bool tiles) -> int {
+    GemmArgs a;
+    memset(&a, 0, sizeof(a));
+    a.out = o;
+    a.x = in;
+    a.offsets = p.offsets;
+    a.x_dtype = act;
+    if (act == BP_I8) {
+      if (const int q = bp_quant_act_int8(p.q, p.q_scale, in, BP_BF16, n, K, s)) return q;
+      a.x = p.q;
+      a.x_scale = p.q_scale;
+    }
+    for (int t = 0; t < n_terms; ++t) { a.packed[t] = packed[t]; a.w_scale[t] = scale[t]; }
+    a.scale_dtype = scale_dtype; a.n_terms = n_terms; a.fmt = fmt;
+    a.T = n; a.N = N; a.K = K; a.Kp = (K + per - 1) / per; a.G = (K + group - 1) / group; a.group = group; a.E = E;
+    a.max_rows = T < n ? T : n;  // an expert has at most one row per token
+    if (tiles) {
+      a.tiles = p.tiles; a.tile_count = p.tile_count; a.tile_cap = p.tile_cap;
+      if (kernel_policy() != 1 && gemm_tiles_supported(a)) {
+        a.overwrite = 1;
+        a.max_rows = TILE_ROWS;
+        return run_gemm(a, s);
+      }
+      a.tiles = nullptr;  // no tile kernel for this shape: the launch covers the bound (every expert up to T rows)
+    }
+    if (const int z = zero(o, 4 * (size_t)n * N, s)) return z;
+    return run_gemm(a, s);
+  };
+  const bool tiles = T > 64;
+  if (tiles) {
+    hipLaunchKernelGGL(k_tile_list, dim3(1), dim3(1024), 0, s, p.tiles, p.tile_count, p.offsets, E, n, p.tile_cap);
+    if ((rc = check_launch("tile_list")) != BP_OK) return rc;
+  }
+  if ((rc = gemm(p.gu, p.xg, gate_up_packed, gate_up_scale, 2 * I, H, tiles)) != BP_OK) return rc;
+  if ((rc = bp_swiglu_bf16(p.h, p.gu, p.gu + I, n, I, 2 * I, s)) != BP_OK) return rc;
+  if ((rc = gemm(p.y, p.h, down_packed, down_scale, H, I, tiles)) != BP_OK) return rc;
+  return bp_moe_combine_bf16(out, p.y, p.inv, weights, experts, T, k, H, s);
+}

@@ -192,7 +192,7 @@ __global__ __launch_bounds__(256) void k_combine(uint16_t* __restrict__ out, con
   if (sl < k) {  // position of slot sl in ascending expert order (ties: slot order), as a rank among the k slots
     int rank = 0;
     for (int j = 0; j < k; ++j) rank += (expert_of[j] < my_expert || (expert_of[j] == my_expert && j < sl)) ? 1 : 0;
-    row_of[rank] = inv[t * k + sl];
+    row_of[rank] = clamp_i64(inv[t * k + sl], 0, (int64_t)gridDim.x * k - 1);  // (a position outside y - from a caller's corrupt routing - reads a wrong row, not foreign memory)
     weight_of[rank] = bf16_bits_to_f32(w[t * k + sl]);
   }
   __syncthreads();

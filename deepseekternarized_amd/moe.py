@@ -75,16 +75,57 @@ class TernaryMoE:
         return grouped_ternary_gemm(q, s, self._offsets, [p for p, _ in terms], [sc for _, sc in terms], K, self.group, self.fmt,
                                     max_rows=self._max_rows)
 
-    def __call__(self, x: torch.Tensor, router_logits: torch.Tensor) -> torch.Tensor:
-        shape = x.shape
-        flat = x.reshape(-1, self.hidden).to(torch.bfloat16).contiguous()
-        _need_ext(flat)
-        scores = torch.softmax(router_logits.reshape(flat.size(0), -1).float(), dim=-1)
+    def route(self, router_logits: torch.Tensor, tokens: int):
+        """``softmax`` / ``topk`` of the router logits in torch, as the reference does (engine/standard.py:158-161):
+        routing weights bf16 [T, k], expert ids int64 [T, k]."""
+        scores = torch.softmax(router_logits.reshape(tokens, -1).float(), dim=-1)
         values, indices = torch.topk(scores, self.top_k, dim=-1)
         if self.renorm:
             values = values / values.sum(-1, keepdim=True)
-        values = values.to(torch.bfloat16).contiguous()
-        indices = indices.contiguous()
+        return values.to(torch.bfloat16).contiguous(), indices.contiguous()
+
+    def _workspace(self, tokens: int, device) -> torch.Tensor:
+        e = _need_ext(self.down[0][0])
+        need = int(e.lib.bp_moe_layer_workspace_bytes(tokens, self.hidden, self.inter, self.n_experts, self.top_k,
+                                                      _lib.BP_I8 if self.act == "int8" else _lib.BP_BF16))
+        ws = getattr(self, "_ws", None)
+        if ws is None or ws.numel() < need or ws.device != torch.device(device):
+            self._ws = ws = torch.empty(need, dtype=torch.uint8, device=device)   # (reused by later calls of up to this many tokens)
+        return ws
+
+    def __call__(self, x: torch.Tensor, router_logits: torch.Tensor) -> torch.Tensor:
+        """The layer through ``bp_moe_layer_bf16``: one library call after the router's top-k, no host synchronisation
+        (the grouped launches take the token tiles from a device-side list), intermediates in a cached workspace."""
+        shape = x.shape
+        flat = x.reshape(-1, self.hidden).to(torch.bfloat16).contiguous()
+        e = _need_ext(flat)
+        T = flat.size(0)
+        values, indices = self.route(router_logits, T)
+        out = torch.empty(T, self.hidden, dtype=torch.bfloat16, device=flat.device)
+        if T == 0:
+            return out.view(shape).to(x.dtype)
+        ws = self._workspace(T, flat.device)
+        import ctypes as C
+        n = len(self.down)
+        arr = lambda ts: (C.c_void_p * n)(*[t.data_ptr() for t in ts])
+        gp, gs = arr([p for p, _ in self.gate_up]), arr([s for _, s in self.gate_up])
+        dp, ds = arr([p for p, _ in self.down]), arr([s for _, s in self.down])
+        sdt = {torch.float32: _lib.BP_F32, torch.float16: _lib.BP_F16, torch.bfloat16: _lib.BP_BF16}[self.down[0][1].dtype]
+        with torch.cuda.device(flat.device):
+            _lib.check(e.lib.bp_moe_layer_bf16(
+                out.data_ptr(), flat.data_ptr(), indices.data_ptr(), values.data_ptr(), gp, gs, dp, ds, sdt, n,
+                T, self.hidden, self.inter, self.n_experts, self.top_k, self.group, _fmt_code(self.fmt),
+                _lib.BP_I8 if self.act == "int8" else _lib.BP_BF16, ws.data_ptr(), ws.numel(), None, _lib.stream_ptr(flat.device)))
+        return out.view(shape).to(x.dtype)
+
+    def composed(self, x: torch.Tensor, router_logits: torch.Tensor) -> torch.Tensor:
+        """The same layer as separate library calls (sort, gather, two grouped GEMMs, SwiGLU, combine), sizing the
+        grouped launches the reference's way: beyond 64 tokens the widest expert's row count is read back to the host
+        (boilerplate/kernels/ternary_cuda.py:97). Kept as the check of ``__call__`` and for callers that want the stages."""
+        shape = x.shape
+        flat = x.reshape(-1, self.hidden).to(torch.bfloat16).contiguous()
+        _need_ext(flat)
+        values, indices = self.route(router_logits, flat.size(0))
         order, self._offsets = sort_by_expert(indices.reshape(-1), self.n_experts)
         # Rows of the widest expert: at most one per token (top-k picks distinct experts). For a few tokens that
         # bound costs nothing and keeps the layer free of host synchronisation; for many, the launch would cover
@@ -106,10 +147,10 @@ class TernaryMoE:
         copies its arguments into the graph's input buffers, replays the captured launches and returns the graph's
         output buffer (overwritten by the next replay). With a handful of tokens the layer is a dozen launches of a few
         microseconds each, and issuing them costs more than running them; a replay issues them at once.
-        Only for ``tokens <= 64``: beyond that the layer reads the widest expert's row count back to the host, which
-        cannot be captured."""
-        if not 1 <= tokens <= 64:
-            raise ValueError("graphed() covers 1..64 tokens (larger batches read the routing back to the host)")
+        Any number of tokens: the layer never reads the routing back to the host."""
+        if tokens < 1:
+            raise ValueError("graphed() needs at least one token")
+        self._workspace(tokens, device)
         xs = torch.zeros(tokens, self.hidden, dtype=dtype, device=device)
         ls = torch.zeros(tokens, self.n_experts, dtype=torch.float32, device=device)
         side = torch.cuda.Stream(device=device)

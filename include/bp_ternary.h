@@ -16,6 +16,7 @@
 #ifndef BP_TERNARY_H
 #define BP_TERNARY_H
 
+#include <stddef.h>
 #include <stdint.h>
 
 #ifdef __cplusplus
@@ -160,6 +161,30 @@ int bp_swiglu_bf16(void* h, const float* gate, const float* up, int64_t rows, in
  * w bf16 [T, k], experts i64 [T, k] (to order the slots of one token), out bf16 [T, H]. */
 int bp_moe_combine_bf16(void* out, const float* y, const int64_t* inv, const void* w, const int64_t* experts,
                         int64_t T, int64_t k, int64_t H, void* stream);
+
+/* One routed-expert MoE layer after the router's top-k (the per-expert loop of boilerplate/engine/standard.py:156-176,
+ * whose experts are TernaryLinear triples, engine/standard.py:37-41 and 151-154): for every (token, slot)
+ *   y = down(bf16(bf16(silu(bf16 gate(x))) * bf16 up(x))) * weights[token, slot]       (each linear rounded to bf16)
+ *   out[token] = sum of bf16(y) over the token's slots in ascending expert order, accumulated in bf16,
+ * as one sort of the routing, one row gather, two grouped launches (gate and up stacked along N), SwiGLU and the
+ * combine, all asynchronous on `stream`; nothing is copied to the host and nothing is allocated (capturable in a
+ * HIP graph). Beyond 64 tokens the grouped launches run over a device-side list of the 32-row token tiles that exist
+ * instead of the reference's `int(offsets.diff().max())` read-back (boilerplate/kernels/ternary_cuda.py:97).
+ *   out      device bf16 [T, H]
+ *   x        device bf16 [T, H] (16-byte aligned)
+ *   experts  device i64 [T, k], values in [0, E), distinct per token (torch.topk indices)
+ *   weights  device bf16 [T, k] routing weights
+ *   gate_up_packed[t] device u8 [E, 2 I, Kp(H)], gate_up_scale[t] device [E, 2 I, G(H)]: rows [0, I) gate, [I, 2 I) up
+ *   down_packed[t]    device u8 [E, H, Kp(I)],   down_scale[t]    device [E, H, G(I)];  n_terms stacked terms each
+ *   act      BP_BF16 (activations as they are) or BP_I8 (per-row int8 of every linear's input, boilerplate/ternary/ops.py:20-25)
+ *   workspace device memory, 256-byte aligned, at least bp_moe_layer_workspace_bytes(T, H, I, E, k, act) bytes
+ *   bad      device i32 flag set to 1 if an expert id is out of range (may be NULL) */
+size_t bp_moe_layer_workspace_bytes(int64_t T, int64_t H, int64_t I, int64_t E, int64_t k, int act);
+int bp_moe_layer_bf16(void* out, const void* x, const int64_t* experts, const void* weights,
+                      const uint8_t* const* gate_up_packed, const void* const* gate_up_scale,
+                      const uint8_t* const* down_packed, const void* const* down_scale, int scale_dtype,
+                      int n_terms, int64_t T, int64_t H, int64_t I, int64_t E, int64_t k, int64_t group, int fmt,
+                      int act, void* workspace, size_t workspace_bytes, int32_t* bad, void* stream);
 
 #ifdef __cplusplus
 }

@@ -1,0 +1,152 @@
+"""bp_moe_layer_bf16 (one library call per MoE layer, no host synchronisation, caller's workspace) against the same layer
+composed of separate library calls with the reference's host-side sizing (boilerplate/kernels/ternary_cuda.py:97), and
+against the CPU restatement of boilerplate/engine/standard.py:151-176 (oracle.moe_layer_ref)."""
+
+import ctypes as C
+
+import numpy as np
+import pytest
+import torch
+
+from oracle import ternary_oracle as orc
+
+pytestmark = pytest.mark.gpu
+
+
+def _layer(fmt, act, H, I, E, k, terms=1, seed=0, sdtype=torch.float16):
+    import deepseekternarized_amd as bp
+    from deepseekternarized_amd.moe import TernaryMoE
+
+    g = torch.Generator(device="cuda").manual_seed(seed)
+    mats = []
+    for n, kk in ((I, H), (I, H), (H, I)):
+        ts = []
+        for t in range(terms):
+            u = torch.rand(E, n, kk, device="cuda", generator=g)
+            tr = torch.where(u < 0.3, -1, torch.where(u < 0.6, 1, 0)).to(torch.int8)
+            pk = torch.stack([bp.pack(tr[e], fmt) for e in range(E)])
+            sc = (0.04 * torch.randn(E, n, kk // 128, device="cuda", generator=g).abs() * 0.25 ** t).to(sdtype)
+            ts.append((pk, sc))
+        mats.append(ts)
+    return TernaryMoE(*mats, H, I, k, fmt, 128, act=act), mats
+
+
+def _rel(a, b):
+    return ((a.float() - b.float()).norm() / b.float().norm().clamp(min=1e-9)).item()
+
+
+@pytest.mark.parametrize("act", ["bf16", "int8"])
+@pytest.mark.parametrize("fmt", ["tq1", "tq2"])
+@pytest.mark.parametrize("T", [1, 7, 64])
+def test_layer_call_equals_composed_calls_up_to_64_tokens(fmt, act, T):
+    """Up to 64 tokens both paths size the grouped launches by the same bound: the same kernels, bit-identical outputs."""
+    moe, _ = _layer(fmt, act, 1024, 1024, 8, 2, seed=T)
+    g = torch.Generator(device="cuda").manual_seed(100 + T)
+    x = torch.randn(T, 1024, device="cuda", generator=g).to(torch.bfloat16)
+    logits = torch.randn(T, 8, device="cuda", generator=g)
+    got, want = moe(x, logits), moe.composed(x, logits)
+    assert got.shape == want.shape == (T, 1024) and torch.isfinite(got.float()).all()
+    assert torch.equal(got, want)
+
+
+@pytest.mark.parametrize("act", ["bf16", "int8"])
+@pytest.mark.parametrize("fmt,terms", [("tq1", 1), ("tq2", 2)])
+def test_layer_call_over_the_tile_list_matches_composed_calls(fmt, terms, act):
+    """Beyond 64 tokens the call runs the grouped GEMMs over the device-side tile list. Skewed routing: an expert with no
+    row, experts with 1..31 rows, one with several tiles and a ragged last tile."""
+    from deepseekternarized_amd import ext
+
+    H, I, E, k, T = 1024, 2048, 16, 2, 300
+    moe, _ = _layer(fmt, act, H, I, E, k, terms=terms, seed=3)
+    g = torch.Generator(device="cuda").manual_seed(5)
+    x = torch.randn(T, H, device="cuda", generator=g).to(torch.bfloat16)
+    logits = torch.randn(T, E, device="cuda", generator=g)
+    logits[:, 0] += 4.0    # nearly every token routes to expert 0: 300 rows = 10 tiles, the last one ragged
+    logits[:, 9] = -40.0   # expert 9 gets nothing
+    logits[:, 11] -= 2.5   # a handful of rows
+    got = moe(x, logits)
+    assert ext().last_kernel().startswith("gemm_" + fmt), ext().last_kernel()
+    want = moe.composed(x, logits)
+    assert torch.isfinite(got.float()).all()
+    # the composed path may pick other kernels for the same rows (its bound is exact): same rounding points, float32 sums in another order
+    assert _rel(got, want) <= 2e-3, _rel(got, want)
+    # the same call again: identical (nothing of the previous call is left in the workspace that matters)
+    assert torch.equal(moe(x, logits), got)
+    # fewer tokens through the same (larger) workspace
+    got2 = moe(x[:70], logits[:70])
+    assert _rel(got2, moe.composed(x[:70], logits[:70])) <= 2e-3
+
+
+@pytest.mark.parametrize("act", ["bf16", "int8"])
+@pytest.mark.parametrize("fmt", ["tq1", "tq2"])
+def test_layer_call_matches_the_reference_loop(fmt, act):
+    """Against the per-expert loop of boilerplate/engine/standard.py:151-176 restated on the CPU, 96 tokens (tile-list path)."""
+    H, I, E, k, T, group = 1024, 1024, 8, 2, 96, 128
+    moe, mats = _layer(fmt, act, H, I, E, k, seed=11)
+    rng = np.random.default_rng(12)
+    x = orc.bf16_round(rng.standard_normal((T, H)).astype(np.float32))
+    logits = (rng.standard_normal((T, E)) * 1.5).astype(np.float32)
+    logits[:, 5] = -30.0
+    experts = [tuple([(mats[n][0][0][e].cpu().numpy(), mats[n][0][1][e].cpu().numpy())] for n in range(3)) for e in range(E)]
+    want = orc.moe_layer_ref(x, logits, experts, k, H, I, group, fmt, act=act)
+    got = moe(torch.from_numpy(x).cuda().to(torch.bfloat16), torch.from_numpy(logits).cuda()).float().cpu().numpy()
+    rel = np.linalg.norm(got - want) / np.linalg.norm(want)
+    assert rel <= 5e-3, rel  # bf16 at the same points; float32 summation order flips a few roundings
+
+
+def test_layer_call_as_a_graph_beyond_64_tokens():
+    """No read-back anywhere: 128 tokens captured as one HIP graph, replayed with eager work in between."""
+    moe, _ = _layer("tq2", "bf16", 1024, 1024, 8, 2, seed=21)
+    run = moe.graphed(128)
+    g = torch.Generator(device="cuda").manual_seed(22)
+    for rep in range(3):
+        x = torch.randn(128, 1024, device="cuda", generator=g).to(torch.bfloat16)
+        logits = torch.randn(128, 8, device="cuda", generator=g)
+        want = moe(x, logits).clone()
+        torch.cuda.synchronize()
+        got = run(x, logits).clone()
+        torch.cuda.synchronize()
+        assert torch.equal(got, want), rep
+
+
+def test_layer_call_argument_checks():
+    from deepseekternarized_amd.kernels import _lib
+
+    lib = _lib.load()
+    moe, _ = _layer("tq2", "bf16", 1024, 1024, 8, 2, seed=31)
+    T = 4
+    x = torch.zeros(T, 1024, dtype=torch.bfloat16, device="cuda")
+    out = torch.empty_like(x)
+    idx = torch.zeros(T, 2, dtype=torch.int64, device="cuda")
+    idx[:, 1] = 1
+    w = torch.ones(T, 2, dtype=torch.bfloat16, device="cuda")
+    need = lib.bp_moe_layer_workspace_bytes(T, 1024, 1024, 8, 2, _lib.BP_BF16)
+    assert need > 0 and need % 256 == 0
+    assert lib.bp_moe_layer_workspace_bytes(T, 1024, 1024, 8, 2, _lib.BP_I8) > need
+    ws = torch.empty(need, dtype=torch.uint8, device="cuda")
+    arr = lambda ts: (C.c_void_p * 1)(*[t.data_ptr() for t in ts])
+    gp, gs = arr([moe.gate_up[0][0]]), arr([moe.gate_up[0][1]])
+    dp, ds = arr([moe.down[0][0]]), arr([moe.down[0][1]])
+
+    def call(**kw):
+        a = dict(out=out.data_ptr(), x=x.data_ptr(), idx=idx.data_ptr(), w=w.data_ptr(), T=T, H=1024, I=1024, E=8, k=2, fmt=2,
+                 act=_lib.BP_BF16, ws=ws.data_ptr(), ws_bytes=need)
+        a.update(kw)
+        return lib.bp_moe_layer_bf16(a["out"], a["x"], a["idx"], a["w"], gp, gs, dp, ds, _lib.BP_F16, 1, a["T"], a["H"], a["I"], a["E"],
+                                     a["k"], 128, a["fmt"], a["act"], a["ws"], a["ws_bytes"], None, None)
+
+    assert call() == 0
+    torch.cuda.synchronize()
+    for bad in (dict(ws_bytes=need - 1), dict(ws=None), dict(ws=ws.data_ptr() + 8), dict(k=0), dict(k=9), dict(fmt=3), dict(act=_lib.BP_F32),
+                dict(H=1020), dict(x=None), dict(E=70000)):
+        assert call(**bad) != 0, bad
+        assert lib.bp_last_error()
+    assert call(T=0) == 0
+    # an expert id out of range raises the flag and faults nothing
+    flag = torch.zeros(1, dtype=torch.int32, device="cuda")
+    idx2 = idx.clone()
+    idx2[1, 1] = 99
+    rc = lib.bp_moe_layer_bf16(out.data_ptr(), x.data_ptr(), idx2.data_ptr(), w.data_ptr(), gp, gs, dp, ds, _lib.BP_F16, 1, T, 1024, 1024, 8, 2,
+                               128, 2, _lib.BP_BF16, ws.data_ptr(), need, flag.data_ptr(), None)
+    torch.cuda.synchronize()
+    assert rc == 0 and int(flag) == 1
