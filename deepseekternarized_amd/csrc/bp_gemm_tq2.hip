@@ -175,36 +175,38 @@ __global__ __launch_bounds__(GTHREADS, 2) void k_gemm_tq2(GemmArgs a) {
   const unsigned xlane = (unsigned)(lane * 16);
   const unsigned clane = (unsigned)(XT + 16 * b);
 
-  // first tile
+  // first tile: its loads are issued here, ahead of the first term's weight and scale loads, and stored once those
+  // are on their way too (one memory latency for all of them)
   stage_load(0, 0);
-  stage_store(0, 0);
   stage_load(0, 1);
-  stage_store(0, 1);
-  if (tiles > 1) {
-    stage_load(tile_k0(1), 0);
-    stage_load(tile_k0(1), 1);
-  }
-  __syncthreads();
   int seq = 0;  // tiles consumed so far
   // The whole loop nest is instantiated once per number of token sub-tiles and the choice made outside it: a branch
   // inside would end in a merge of the two paths' registers, and a register that a load in flight is about to write
   // can only be merged after waiting for that load - the weight ring would drain at the end of every tile.
   auto all_terms = [&](auto mtn_c) {
+  u32x4 ring[RD][GR];
+  constexpr int SPRE = 4;  // 16-byte units of the scale tile per thread that are fetched ahead (the rest, if any, at the term's start)
+  u32x4 spre[SPRE];
+  bool ring_filled = false;  // the ring already holds the term's first steps (loaded at the end of the term before)
   for (int term = 0; term < a.n_terms; ++term) {
     const int64_t rows_here = a.N - n0 < 16 * GR ? a.N - n0 : 16 * GR;
     const __amdgpu_buffer_rsrc_t wrs = make_rsrc(a.packed[term] + (e * a.N + n0) * a.Kp, rows_here * a.Kp);
+    // a term's last refills of the ring run on into the next term's first steps (whole tiles only: the ring slot of a
+    // step is its index within the tile)
+    const bool chain = steps % PF == 0 && term + 1 < a.n_terms;
+    const __amdgpu_buffer_rsrc_t wrs_next = make_rsrc(a.packed[chain ? term + 1 : term] + (e * a.N + n0) * a.Kp, rows_here * a.Kp);
     const __amdgpu_buffer_rsrc_t srs = make_rsrc((const unsigned char*)a.w_scale[term] + (e * a.N + n0) * a.G * SB, rows_here * a.G * SB);
     const unsigned woff = (unsigned)r16 * (unsigned)a.Kp + 16u * b;
     const unsigned soff = (unsigned)r16 * (unsigned)a.G * SB;
     const unsigned slane = stile + (unsigned)((wave * 16 * GR + r16) * (int)a.G * SB);
-    u32x4 ring[RD][GR];
     u32x4 sraw[GR][2], snext[GR][2];
     auto fetch_w = [&](int c, u32x4 (&dst)[GR]) {
-      const int cc = c < steps ? c : steps - 1;
+      const bool over = chain && c >= steps;
+      const int cc = over ? c - steps : c < steps ? c : steps - 1;
 #pragma unroll
       for (int r = 0; r < GR; ++r) {
         if (ABL == 5) { asm volatile("" : "+v"(dst[r])); continue; }
-        dst[r] = buf_load16(wrs, woff, (unsigned)(row_shift[r] * a.Kp) + 64u * cc);
+        dst[r] = buf_load16(over ? wrs_next : wrs, woff, (unsigned)(row_shift[r] * a.Kp) + 64u * cc);
       }
     };
     auto fetch_s = [&](int c, u32x4 (&dst)[GR][2]) {  // scales of steps c .. c+3
@@ -221,23 +223,49 @@ __global__ __launch_bounds__(GTHREADS, 2) void k_gemm_tq2(GemmArgs a) {
         }
       }
     };
+    // the workgroup's rows of a term's scales: one contiguous block, copied to LDS in 16-byte units
+    const int64_t wg_row0 = (int64_t)wg_tile * GROWS;
+    const int64_t wg_rows = a.N - wg_row0 < GROWS ? a.N - wg_row0 : GROWS;
+    const int units16 = (int)(wg_rows * a.G * SB / 16);
+    auto scale_prefetch = [&](int t) {
+      const unsigned char* src = (const unsigned char*)a.w_scale[t] + (e * a.N + wg_row0) * a.G * SB;
+#pragma unroll
+      for (int i = 0; i < SPRE; ++i) {
+        const int u = (int)threadIdx.x + i * GTHREADS;
+        if (u < units16) spre[i] = *(const u32x4*)(src + 16 * (int64_t)u);
+      }
+    };
     if (!SL) fetch_s(0, snext);
     __builtin_amdgcn_sched_barrier(0);
+    if (!ring_filled) {
 #pragma unroll
-    for (int i = 0; i < RD; ++i) {
-      fetch_w(i, ring[i]);
-      __builtin_amdgcn_sched_barrier(0);
+      for (int i = 0; i < RD; ++i) {
+        fetch_w(i, ring[i]);
+        __builtin_amdgcn_sched_barrier(0);
+      }
     }
+    ring_filled = chain;
     if (SL) {
-      const int64_t wg_row0 = (int64_t)wg_tile * GROWS;
-      const int64_t wg_rows = a.N - wg_row0 < GROWS ? a.N - wg_row0 : GROWS;
+      if (term == 0) scale_prefetch(0);
+      else __syncthreads();  // the previous term's scales are no longer read
+#pragma unroll
+      for (int i = 0; i < SPRE; ++i) {
+        const int u = (int)threadIdx.x + i * GTHREADS;
+        if (u < units16) *(lds_u32x4*)(stile + 16 * u) = spre[i];
+      }
       const unsigned char* src = (const unsigned char*)a.w_scale[term] + (e * a.N + wg_row0) * a.G * SB;
-      const int units16 = (int)(wg_rows * a.G * SB / 16);
-      if (term > 0) __syncthreads();  // the previous term's scales are no longer read
-      for (int u = threadIdx.x; u < units16; u += GTHREADS) *(lds_u32x4*)(stile + 16 * u) = *(const u32x4*)(src + 16 * (int64_t)u);
-      __syncthreads();
-      fetch_s(0, snext);
+      for (int u = threadIdx.x + SPRE * GTHREADS; u < units16; u += GTHREADS) *(lds_u32x4*)(stile + 16 * u) = *(const u32x4*)(src + 16 * (int64_t)u);
     }
+    if (term == 0) {
+      stage_store(0, 0);
+      stage_store(0, 1);
+      if (tiles > 1) {
+        stage_load(tile_k0(1), 0);
+        stage_load(tile_k0(1), 1);
+      }
+    }
+    if (SL || term == 0) __syncthreads();
+    if (SL) fetch_s(0, snext);
 
     for (int ch = 0; ch < chunks; ++ch) {
       // a tile that holds all of K is staged once and serves every term
@@ -251,6 +279,7 @@ __global__ __launch_bounds__(GTHREADS, 2) void k_gemm_tq2(GemmArgs a) {
       for (int r = 0; r < GR; ++r) { sraw[r][0] = snext[r][0]; sraw[r][1] = snext[r][1]; }
       const int c4 = ch * PF;
       fetch_s(c4 + PF, snext);
+      if (SL && ch == chunks - 1 && term + 1 < a.n_terms) scale_prefetch(term + 1);
 
       // The four steps of the tile, for MTN token sub-tiles (a tile of at most 16 tokens skips the second one).
       auto run_steps = [&](auto mtn_c) {
