@@ -54,7 +54,10 @@ int launch_mfma(const GemmArgs& a, hipStream_t s) {
   // expert) and the bound small: then nearly every expert fits one 16-token tile of the lighter kernel, and the few
   // that do not (or a loose upper bound from a caller that keeps the routing on the device) cost a second tile.
   const bool sparse = a.T <= 8 * a.E && a.max_rows <= 64;
-  if (a.max_rows > 16 && !sparse) return launch_gemm_tq2(a, s);
+  // A launch of few workgroups (one dense linear on a decode batch: 256 rows x 32 tokens per workgroup leaves most CUs
+  // idle) also goes to the 16-token tiles, which make four times as many.
+  const bool few = a.E == 1 && ((a.N + 255) / 256) * ((a.max_rows + 31) / 32) < 64 && a.max_rows <= 128;
+  if (a.max_rows > 16 && !sparse && !few) return launch_gemm_tq2(a, s);
   return launch_mfma_tq2(a, s, R, 1, waves);
 }
 

@@ -408,8 +408,11 @@ int launch_mfma_tq1(const GemmArgs& a, hipStream_t s, int waves) {
       if (rc != BP_ERR_UNSUPPORTED) return rc;
     }
   }
-  {  // more rows per expert: token tiles of 32 on the fp8 x fp4 matrix instruction
-    if (tuning().tq1 != 'm') {  // (development: "mfma" keeps the 16-token kernel below)
+  {  // more rows per expert: token tiles of 32 on the fp8 x fp4 matrix instruction - unless the launch would be a few
+    // dozen workgroups (one dense linear on a decode batch: 512 rows x 32 tokens each): the 16-token kernel below makes
+    // eight times as many and takes half the time there
+    const bool few = a.E == 1 && ((a.N + 511) / 512) * ((a.max_rows + 31) / 32) < 64 && a.max_rows <= 128;
+    if (tuning().tq1 != 'm' && !few) {  // (development: "mfma" keeps the 16-token kernel below)
       const int rc = launch_gemm_tq1(a, s);
       if (rc != BP_ERR_UNSUPPORTED) return rc;
     }

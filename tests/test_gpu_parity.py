@@ -99,7 +99,8 @@ def test_quant_act_int8_keeps_leading_shape(bp):
 
 # --------------------------------------------------------------------------- routing: bit-exact
 @pytest.mark.parametrize("n,E", [(0, 4), (1, 1), (18, 6), (6, 64), (100, 384), (128, 3), (129, 7), (64, 5000), (512, 384), (4096, 64), (12288, 384),
-                                  (70000, 8), (3000, 5000)])  # up to 128 ids: the one-pass kernel
+                                  (70000, 8), (3000, 5000), (2048, 1), (2048, 4096), (2049, 64), (1500, 4097),
+                                  (777, 2500)])  # up to 128 ids: the one-pass kernel
 def test_sort_by_expert_bit_exact(bp, n, E):
     rng = np.random.default_rng(n + E)
     ids = rng.integers(0, E, n).astype(np.int64)

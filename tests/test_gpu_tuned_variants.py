@@ -356,10 +356,22 @@ def test_tq2_gemm_scales_from_global_memory_and_other_scale_dtypes(bp):
     assert kern.startswith("gemm_tq2"), kern
     _check(got, want)
     packed, scales = synth_weights(23, 1, 80, 2048, GROUP, "tq2")
-    x = orc.bf16_round(np.random.default_rng(23).standard_normal((37, 2048)).astype(np.float32))
+    x = orc.bf16_round(np.random.default_rng(23).standard_normal((137, 2048)).astype(np.float32))
     want = c_gemm(x, None, packed[0][0], scales[0][0].astype(np.float32), 2048, GROUP, "tq2")
     got = bp.ternary_gemm_float(dev(x).to(torch.bfloat16), dev(packed[0][0]), dev(scales[0][0]).float(), 2048, GROUP, "tq2")
     assert bp.ext().last_kernel().startswith("gemm_tq2")
+    _check(got.cpu().numpy(), want)
+
+
+@pytest.mark.parametrize("fmt,prefix", [("tq1", "mfma_tq1"), ("tq2", "mfma_tq2")])
+def test_one_dense_linear_on_a_decode_batch_takes_the_16_token_tiles(bp, fmt, prefix):
+    """A single linear (E = 1) with a few dozen rows: the 32-token-tile kernels would launch a handful of workgroups, so the
+    call goes to the 16-token tiles (same contract, more workgroups)."""
+    packed, scales = synth_weights(29, 1, 272, 2048, GROUP, fmt)
+    x = orc.bf16_round(np.random.default_rng(29).standard_normal((64, 2048)).astype(np.float32))
+    want = c_gemm(x, None, packed[0][0], scales[0][0].astype(np.float32), 2048, GROUP, fmt)
+    got = bp.ternary_gemm_float(dev(x).to(torch.bfloat16), dev(packed[0][0]), dev(scales[0][0]), 2048, GROUP, fmt)
+    assert bp.ext().last_kernel().startswith(prefix), bp.ext().last_kernel()
     _check(got.cpu().numpy(), want)
 
 
