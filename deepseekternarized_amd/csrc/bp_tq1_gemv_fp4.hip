@@ -129,11 +129,10 @@ __global__ __launch_bounds__(WAVES * 64, 4) void k_tq1_gemv_fp4(GemmArgs a, int 
   const bool x16 = a.x_dtype == BP_BF16 || a.x_dtype == BP_F16;
   auto widen16 = [&](unsigned h) { return a.x_dtype == BP_BF16 ? bf16_bits_to_f32((uint16_t)h) : f16_bits_to_f32((uint16_t)h); };
 
-  // ---- the byte table: entry v = digits d0..d4 of v as fp4 codes (-1 -> 0xA, 0 -> 0, +1 -> 0x2) in nibbles 0..4;
-  // computed once per value into copy 0, then spread over the other 31 copies.
-  // Alongside: the largest magnitude of every 128-wide group of the token (LDS maximum over the float bits).
-  if (threadIdx.x < 256) {
-    unsigned v = threadIdx.x, ent = 0;
+  // ---- the byte table: entry v = digits d0..d4 of v as fp4 codes (-1 -> 0xA, 0 -> 0, +1 -> 0x2) in nibbles 0..4, one
+  // copy per LDS bank: four threads per entry, eight copies each.
+  for (int idx = threadIdx.x; idx < 256 * 4; idx += THREADS) {
+    unsigned v = (unsigned)idx >> 2, ent = 0;
     if (v < 243) {
 #pragma unroll
       for (int d = 0; d < 5; ++d) {
@@ -142,7 +141,8 @@ __global__ __launch_bounds__(WAVES * 64, 4) void k_tq1_gemv_fp4(GemmArgs a, int 
         v = q;
       }
     }
-    *(lds_u32*)(128 * threadIdx.x) = ent;
+#pragma unroll
+    for (int cpy = 0; cpy < 8; ++cpy) *(lds_u32*)(128 * (idx >> 2) + 4 * (8 * (idx & 3) + cpy)) = ent;
   }
   // A launch covers the chunks first_chunk .. first_chunk + nchunks - 1 of every row (all of them unless the tokens'
   // tiles of all chunks do not fit in LDS: then the host launches once per segment of K, and the output takes the
@@ -152,67 +152,19 @@ __global__ __launch_bounds__(WAVES * 64, 4) void k_tq1_gemv_fp4(GemmArgs a, int 
   // the end of a row that dword meets activations that are 0; at the end of a segment it is needed, so the chunk
   // after a segment that is not the last one is loaded as well.
   const int last_load = NTOK > 1 && cb + nchunks < total_chunks ? nchunks : nchunks - 1;
-  for (int g = threadIdx.x; g < ntok * nchunks * 8; g += THREADS) {
-    const int tt = g / (nchunks * 8), gc = g - tt * nchunks * 8;
-    *(lds_u32*)(tile_at(tt, gc >> 3) + F4_PRE_OFF + 4 * (gc & 7)) = 0u;
-  }
-  __syncthreads();
-  for (int idx = threadIdx.x; idx < 256 * 32; idx += THREADS) *(lds_u32*)(4 * idx) = *(const lds_u32*)(128 * (idx >> 5));
-  const int64_t kbeg = 640 * (int64_t)cb, kend = a.K < 640 * (int64_t)(cb + nchunks) ? a.K : 640 * (int64_t)(cb + nchunks);
-  for (int tt = 0; tt < ntok; ++tt) {
-  const int64_t xrow = (tok + tt) * a.K;
-  if (a.x_dtype != BP_I8) {  // (int8 values fit as they are: prescale 1)
-    for (int64_t k0 = kbeg + 8 * (int64_t)threadIdx.x; k0 < kend; k0 += 8 * THREADS) {  // 8 values of one group per thread
-      unsigned m = 0;
-      if (x16 && k0 + 8 <= a.K) {
-        const u32x4 q = ((const F4Packed16*)((const uint16_t*)a.x + xrow + k0))->v;
-#pragma unroll
-        for (int i = 0; i < 4; ++i) {
-          const unsigned lo = __float_as_uint(widen16(q[i] & 0xffffu)) & 0x7fffffffu, hi = __float_as_uint(widen16(q[i] >> 16)) & 0x7fffffffu;
-          m = m > lo ? m : lo;
-          m = m > hi ? m : hi;
-        }
-      } else {
-        for (int i = 0; i < 8 && k0 + i < a.K; ++i) {
-          const unsigned v = __float_as_uint(load_act_f32(a.x, a.x_dtype, xrow + k0 + i)) & 0x7fffffffu;
-          m = m > v ? m : v;
-        }
-      }
-      const int gg = (int)((k0 - kbeg) >> 7);
-      __hip_atomic_fetch_max((lds_u32*)(tile_at(tt, gg / 5) + F4_PRE_OFF + 4 * (gg % 5)), m, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
-    }
-  }
-  }
-  __syncthreads();
-  // the maxima become prescales 2^sh (sh brings the group's largest magnitude into [128, 256)) and their inverses
-  for (int gt = threadIdx.x; gt < ntok * nchunks * 8; gt += THREADS) {
-    const int tt = gt / (nchunks * 8), g = gt - tt * nchunks * 8;
-    const unsigned at = (unsigned)(tile_at(tt, g >> 3) + 4 * (g & 7));
-    const bool real = (g & 7) < 5 && 128 * (int64_t)(5 * (cb + (g >> 3)) + (g & 7)) < a.K;
-    int sh = 0;
-    bool finite = true;
-    if (real && a.x_dtype != BP_I8) {
-      const int ex = (int)((*(const lds_u32*)(at + F4_PRE_OFF) >> 23) & 255u);
-      finite = ex != 255;  // a NaN or an infinity among the group's activations
-      sh = 134 - ex;
-      sh = sh > 120 ? 120 : sh < -120 ? -120 : sh;
-    }
-    *(lds_u32*)(at + F4_PRE_OFF) = (unsigned)(sh + 127) << 23;
-    // (the inverse prescale multiplies every row's group sum: NaN for a group with a non-finite activation, so the
-    // token's outputs are NaN rather than finite and wrong)
-    *(lds_u32*)(at + F4_INV_OFF) = !real ? 0u : finite ? (unsigned)(127 - sh) << 23 : 0x7fc00000u;
-  }
-  __syncthreads();
 
-  // ---- operand A tile: one item = the 10 activations behind a byte pair -> 3 pieces x (first-group block, second-group block)
-  for (int itt = threadIdx.x; itt < ntok * nchunks * 64; itt += THREADS) {
-    const int tt = itt / (nchunks * 64), it = itt - tt * nchunks * 64;
+  // ---- operand A tiles: a wave builds whole chunks by itself (64 byte pairs = 64 lanes; a chunk holds 5 whole scale
+  // groups), so the activations are read from memory once and nothing waits for another wave until the tiles are
+  // complete. Lane = byte pair: its 10 activations -> the largest magnitude of each of its (one or two) groups by an LDS
+  // maximum over the float bits -> the groups' prescales 2^sh (sh brings the group's largest magnitude into [128, 256))
+  // and their inverses -> 3 pieces x (first-group block, second-group block).
+  for (int item = wave; item < ntok * nchunks; item += WAVES) {
+    const int tt = item / nchunks, c = item - tt * nchunks;
     const int64_t xrow = (tok + tt) * a.K;
-    const int c = it >> 6, blk = it & 63;
+    const int blk = lane;
     const int tt0 = 5 * f4_pair_byte(blk >> 3, (blk >> 1) & 3, blk & 1), glo = tt0 >> 7, ghi = (tt0 + 9) >> 7;
     const unsigned dst = (unsigned)tile_at(tt, c);
-    const float pre_lo = __uint_as_float(*(const lds_u32*)(dst + F4_PRE_OFF + 4 * glo));
-    const float pre_hi = __uint_as_float(*(const lds_u32*)(dst + F4_PRE_OFF + 4 * ghi));
+    if (lane < 8) *(lds_u32*)(dst + F4_PRE_OFF + 4 * lane) = 0u;
     const int64_t k0 = 640 * (int64_t)(cb + c) + tt0;
     float y[10];
     if (x16 && k0 + 10 <= a.K) {  // 20 bytes at an even address
@@ -227,6 +179,42 @@ __global__ __launch_bounds__(WAVES * 64, 4) void k_tq1_gemv_fp4(GemmArgs a, int 
 #pragma unroll
       for (int t = 0; t < 10; ++t) y[t] = k0 + t < a.K ? load_act_f32(a.x, a.x_dtype, xrow + k0 + t) : 0.f;
     }
+    if (a.x_dtype != BP_I8) {  // (int8 values fit as they are: prescale 1)
+      unsigned m_lo = 0, m_hi = 0;
+#pragma unroll
+      for (int t = 0; t < 10; ++t) {
+        const unsigned v = __float_as_uint(y[t]) & 0x7fffffffu;
+        if (((tt0 + t) >> 7) == glo) m_lo = m_lo > v ? m_lo : v;
+        else m_hi = m_hi > v ? m_hi : v;
+      }
+      __hip_atomic_fetch_max((lds_u32*)(dst + F4_PRE_OFF + 4 * glo), m_lo, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WAVEFRONT);
+      if (ghi != glo) __hip_atomic_fetch_max((lds_u32*)(dst + F4_PRE_OFF + 4 * ghi), m_hi, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WAVEFRONT);
+    }
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+    __builtin_amdgcn_wave_barrier();
+    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+    if (lane < 8) {
+      const int g = lane;
+      const unsigned at = dst + 4 * g;
+      const bool real = g < 5 && 128 * (int64_t)(5 * (cb + c) + g) < a.K;
+      int sh = 0;
+      bool finite = true;
+      if (real && a.x_dtype != BP_I8) {
+        const int ex = (int)((*(const lds_u32*)(at + F4_PRE_OFF) >> 23) & 255u);
+        finite = ex != 255;  // a NaN or an infinity among the group's activations
+        sh = 134 - ex;
+        sh = sh > 120 ? 120 : sh < -120 ? -120 : sh;
+      }
+      *(lds_u32*)(at + F4_PRE_OFF) = (unsigned)(sh + 127) << 23;
+      // (the inverse prescale multiplies every row's group sum: NaN for a group with a non-finite activation, so the
+      // token's outputs are NaN rather than finite and wrong)
+      *(lds_u32*)(at + F4_INV_OFF) = !real ? 0u : finite ? (unsigned)(127 - sh) << 23 : 0x7fc00000u;
+    }
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+    __builtin_amdgcn_wave_barrier();
+    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+    const float pre_lo = __uint_as_float(*(const lds_u32*)(dst + F4_PRE_OFF + 4 * glo));
+    const float pre_hi = __uint_as_float(*(const lds_u32*)(dst + F4_PRE_OFF + 4 * ghi));
     u32x4 lo[PC] = {}, hi[PC] = {};
 #pragma unroll
     for (int t = 0; t < 10; t += 2) {  // two activations per conversion
