@@ -228,6 +228,15 @@ __global__ __launch_bounds__(256) void k_combine(uint16_t* __restrict__ out, con
   }
 }
 
+// flag = 1 if an expert has more rows than `max_rows` (offsets clamped to [0, T] as the GEMM kernels clamp them)
+__global__ __launch_bounds__(256) void k_check_rows(int32_t* __restrict__ flag, const int64_t* __restrict__ offsets, int64_t E, int64_t T,
+                                                    int64_t max_rows) {
+  for (int64_t e = (int64_t)blockIdx.x * 256 + threadIdx.x; e < E; e += (int64_t)gridDim.x * 256) {
+    const int64_t o0 = clamp_i64(offsets[e], 0, T), o1 = clamp_i64(offsets[e + 1], 0, T);
+    if (o1 - o0 > max_rows) *flag = 1;
+  }
+}
+
 }  // namespace
 }  // namespace bp
 
@@ -314,4 +323,14 @@ extern "C" int bp_moe_combine_bf16(void* out, const float* y, const int64_t* inv
   hipLaunchKernelGGL(k_combine, dim3((unsigned)T, (unsigned)((H + COMBINE_COLS - 1) / COMBINE_COLS)), dim3(256), 0, (hipStream_t)stream, (uint16_t*)out, y, inv,
                      (const uint16_t*)w, experts, k, H);
   return check_launch("moe_combine");
+}
+
+extern "C" int bp_check_max_rows(int32_t* flag, const int64_t* offsets, int64_t E, int64_t T, int64_t max_rows, void* stream) {
+  if (E < 0 || T < 0 || max_rows < 0) return fail(BP_ERR_ARG, "invalid dimensions");
+  if (E == 0) return BP_OK;
+  if (!flag || !offsets) return fail(BP_ERR_ARG, "null pointer");
+  int64_t g = (E + 255) / 256;
+  if (g > 1024) g = 1024;
+  hipLaunchKernelGGL(k_check_rows, dim3((unsigned)g), dim3(256), 0, (hipStream_t)stream, flag, offsets, E, T, max_rows);
+  return check_launch("check_max_rows");
 }

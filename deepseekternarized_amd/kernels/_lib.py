@@ -31,6 +31,7 @@ SIGNATURES = {
     "bp_sort_workspace_ints": (_l, [_l, _l]),
     "bp_sort_by_expert": (_i, [_p, _p, _p, _l, _l, _p, _p, _p]),
     "bp_sort_by_expert_static": (_i, [_p, _p, _p, _l, _l, _p, _p]),
+    "bp_check_max_rows": (_i, [_p, _p, _l, _l, _l, _p]),
     "bp_gather_rows": (_i, [_p, _p, _p, _l, _l, _l, _l, _p]),
     "bp_swiglu_bf16": (_i, [_p, _p, _p, _l, _l, _l, _p]),
     "bp_moe_combine_bf16": (_i, [_p, _p, _p, _p, _p, _l, _l, _l, _p]),

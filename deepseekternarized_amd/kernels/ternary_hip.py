@@ -179,7 +179,7 @@ def ternary_gemm_ref(x: torch.Tensor, x_scale: torch.Tensor, packed: torch.Tenso
 
 
 def grouped_ternary_gemm(x: torch.Tensor, x_scale, offsets, packed, w_scale, K: int, group: int, fmt: str,
-                         backend: str = "auto", max_rows: int | None = None) -> torch.Tensor:
+                         backend: str = "auto", max_rows: int | None = None, validate: bool = False) -> torch.Tensor:
     """Rows of ``x`` sorted by expert; ``packed`` [E, N, Kp], ``w_scale`` [E, N, G] -> [T, N] float32
     (``boilerplate/kernels/ternary_cuda.py:90-111``).
 
@@ -189,7 +189,9 @@ def grouped_ternary_gemm(x: torch.Tensor, x_scale, offsets, packed, w_scale, K: 
     The launch then covers ``max_rows`` rows per expert - an upper bound the caller knows (the token count,
     when every token picks distinct experts), by default the row count of ``x``; rows of an expert beyond
     ``max_rows`` would not be computed. With host offsets the widest expert is taken from them and ``max_rows``
-    is ignored.
+    is ignored. ``validate=True`` checks a caller's bound against device offsets on the device and raises the
+    reference's error ("max_rows is smaller than the largest expert row count"); it reads one flag back, so it
+    synchronises - a debugging aid, not for the serving path.
     """
     code = _fmt_code(fmt)
     if backend not in _BACKENDS:
@@ -213,6 +215,12 @@ def grouped_ternary_gemm(x: torch.Tensor, x_scale, offsets, packed, w_scale, K: 
         max_rows = x.size(0)
     else:
         max_rows = max(0, min(int(max_rows), x.size(0)))
+    if validate and on_device and E:
+        flag = torch.zeros(1, dtype=torch.int32, device=dev)
+        with torch.cuda.device(dev):
+            _lib.check(e.lib.bp_check_max_rows(flag.data_ptr(), offs_dev.data_ptr(), E, x.size(0), max_rows, _lib.stream_ptr(dev)))
+        if int(flag):
+            raise RuntimeError("max_rows is smaller than the largest expert row count")
     out = torch.zeros(x.size(0), pk[0].size(1), dtype=torch.float32, device=dev)
     xs = None if x_scale is None else x_scale.float().contiguous()
     args = (out, x.contiguous(), xs, offs_dev, [p.contiguous() for p in pk], [s.contiguous() for s in sc], K, group, code, None, max_rows)

@@ -144,6 +144,13 @@ int bp_sort_by_expert(int64_t* order, int64_t* offsets, const int64_t* ids, int6
 int bp_sort_by_expert_static(int64_t* order, int64_t* offsets, const int64_t* ids, int64_t n, int64_t E,
                              int32_t* bad, void* stream);
 
+/* The check the reference makes on the host before a grouped launch ("max_rows is smaller than the largest expert row
+ * count", boilerplate/kernels/csrc/ternary_cuda_kernel.cu:130-139), for callers that keep the offsets on the device:
+ * sets *flag (device i32, cleared by the caller) to 1 if an expert has more than max_rows rows. bp_ternary_grouped_gemm
+ * with device offsets computes at most max_rows rows per expert and leaves the others untouched, without an error;
+ * max_rows = T is always safe. */
+int bp_check_max_rows(int32_t* flag, const int64_t* offsets, int64_t E, int64_t T, int64_t max_rows, void* stream);
+
 /* Row gather dst[i, :] = src[index[i] / divisor, :] (the x[order // k] permute of
  * scripts/eval/ternary_kernel_bench.py:90-93). row_bytes must be a multiple of 2. */
 int bp_gather_rows(void* dst, const void* src, const int64_t* index, int64_t divisor, int64_t rows,

@@ -517,3 +517,18 @@ def test_sort_by_expert_ids_out_of_range(bp):
         bp.sort_by_expert(ids, 8, validate=True)
     order, offsets = bp.sort_by_expert(ids.clamp(0, 7), 8, validate=True)
     assert offsets.cpu().tolist()[-1] == 7 and sorted(order.cpu().tolist()) == list(range(7))
+
+
+def test_max_rows_bound_too_small_is_reported_on_request(bp):
+    """Device offsets with a caller's bound: rows beyond it are left out without an error (documented); `validate=True`
+    raises the reference's message (ternary_cuda_kernel.cu:130-139 checks a host copy on every call)."""
+    E, N, K, group = 3, 16, 256, 128
+    packed, scales = synth_weights(5, E, N, K, group, "tq2")
+    rng = np.random.default_rng(6)
+    x, xs = orc.quant_act_int8(rng.standard_normal((9, K)).astype(np.float32))
+    offsets = torch.tensor([0, 5, 5, 9], device="cuda")
+    full = bp.grouped_ternary_gemm(dev(x), dev(xs), offsets, dev(packed[0]), dev(scales[0]), K, group, "tq2", max_rows=5, validate=True)
+    with pytest.raises(RuntimeError, match="max_rows is smaller"):
+        bp.grouped_ternary_gemm(dev(x), dev(xs), offsets, dev(packed[0]), dev(scales[0]), K, group, "tq2", max_rows=4, validate=True)
+    part = bp.grouped_ternary_gemm(dev(x), dev(xs), offsets, dev(packed[0]), dev(scales[0]), K, group, "tq2", max_rows=4)
+    assert torch.equal(part[:4], full[:4]) and torch.equal(part[5:9], full[5:9]) and not part[4].any()  # expert 0's fifth row is left at zero
