@@ -45,6 +45,7 @@ typedef __bf16 bf16x2 __attribute__((ext_vector_type(2)));
 typedef __attribute__((address_space(3))) u32x2 lds_u32x2;
 typedef __attribute__((address_space(3))) u32x4 lds_u32x4;
 typedef __attribute__((address_space(3))) unsigned lds_u32;
+typedef __attribute__((address_space(3))) unsigned short lds_u16;
 
 // Weights and scales are read with raw buffer loads: a wave-uniform descriptor (base, byte range) in
 // scalar registers, a 32-bit lane offset and a scalar step offset, so a load needs no vector address

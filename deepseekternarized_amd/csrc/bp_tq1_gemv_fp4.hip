@@ -72,6 +72,7 @@ constexpr int F4_LDS_MAX = 160 * 1024;
 // per launch, two tiles with 2 chunks each 638 MB (405 MB are packed bytes and scales). Rows of 1434 bytes share
 // 128-byte lines between consecutive chunks; the sooner a wave returns to a row, the more of those lines it still
 // finds in the L2.
+constexpr int F4_SCALE_SLOT = 16 * 80;           // (SR) per wave: 16 rows x 80 bytes (48 of them a round's scales)
 constexpr int F4_GR = 1;                         // 16-row tiles per wave (more than one share the reads of operand A)
 constexpr int F4_RD = 4;                         // chunks of packed bytes in registers per tile (the ring of loads in flight)
 constexpr int F4_BD = 1;                         // table reads run this many (instruction, tile) pairs ahead of the matrix instructions
@@ -101,8 +102,16 @@ __device__ __forceinline__ int f4_pair_byte(int j, int kbA, int hf) {
 // first window and group 3, 4, 2 (s = 0, 1, 2) in the second, so a lane of the result (rows 4 lg + i) holds both
 // tokens' pieces of one group per window. 8 matrix instructions per chunk and token pair; with two pairs the ring
 // of loads is two chunks (registers; the loads are not what a wave then waits for).
-template <int SDT, int WAVES, int ABL = 0, int NTOK = 1>
+//
+// SR (one token, 2-byte scales): scales by the round. A scale per row and group loaded where it is applied is a wave
+// load per chunk that touches 16 memory lines for 8 bytes each: a third of the kernel's load instructions for 7 % of its
+// bytes. Instead a wave loads, once per round of the ring (4 chunks = 20 groups = 40 bytes of a row's scales), 16 bytes
+// per lane (quarters 0..2 of a row's four lanes cover 48 bytes), a round ahead and unconditionally - so the compiler's
+// count of loads in flight stays exact - parks them in a private 1.25 KiB slot of LDS at the start of the round, and a
+// chunk's two scales per lane are two 2-byte LDS reads.
+template <int SDT, int WAVES, int ABL = 0, int NTOK = 1, int SR = 0>
 __global__ __launch_bounds__(WAVES * 64, 4) void k_tq1_gemv_fp4(GemmArgs a, int total_chunks, int first_chunk, int nchunks, int bpw /* row blocks per workgroup */, int first_row) {
+  static_assert(!SR || (NTOK == 1 && SDT != BP_F32 && F4_GR == 1 && F4_RD == 4), "scales by the round: one token, one tile per wave, 2-byte scales, rounds of 4 chunks");
   constexpr int THREADS = WAVES * 64, GR = F4_GR, RD = NTOK <= 2 ? F4_RD : 2, BD = F4_BD, AD = F4_AD, PAIRS = NTOK <= 2 ? F4_PAIRS : 0;
   static_assert(!PAIRS || RD % 2 == 0, "pairs of chunks need an even ring");
   static_assert(NTOK == 1 || (GR == 1 && AD == 0 && NTOK % 2 == 0), "several tokens: one tile per wave, one operand A buffer, token pairs");
@@ -302,6 +311,9 @@ __global__ __launch_bounds__(WAVES * 64, 4) void k_tq1_gemv_fp4(GemmArgs a, int 
     const unsigned srow = smis + (unsigned)r16 * (unsigned)a.G * SB;
     u32x4 W[RD][GR][2];
     u32x2 SQ[GR];  // the scales of one chunk: refilled for the next chunk as soon as they have been applied
+    // (SR) the wave's scale slot behind the tiles: [16 rows][80 bytes], 48 of them the scales of the round's 20 groups
+    const unsigned sr_at = (unsigned)(AT + nchunks * F4_CHUNK_BYTES + wave * F4_SCALE_SLOT + r16 * 80);
+    u32x4 SN = {0u, 0u, 0u, 0u};  // (SR) the next round's scales of this lane's row: 16 bytes at 16 kb
 
   for (int pass = 0; pass < bpw; ++pass) {
     const int64_t n0 = block_row0(pass), n0_next = pass + 1 < bpw ? block_row0(pass + 1) : n0;
@@ -349,6 +361,13 @@ __global__ __launch_bounds__(WAVES * 64, 4) void k_tq1_gemv_fp4(GemmArgs a, int 
         SQ[s] = f4_load8(srs, at, (unsigned)(row * a.G * SB));
       }
     };
+    auto fetch_round = [&](int c) {  // (SR) the scales of the round that starts with chunk c (a multiple of 4; past the block: of the next one)
+      int64_t row0;
+      int cc;
+      target(c, row0, cc);
+      SN = buf_load16(srs, srow + 16u * kb, (unsigned)(row0 * a.G * SB) + SB * (unsigned)((5 * cc) >> gs));
+    };
+    auto park_round = [&]() { *(lds_u32x4*)(sr_at + 16 * kb) = SN; };
     // (chunk slots and pipeline stages are compile-time constants: every register array below is indexed statically)
     auto step = [&](int c, auto cur_c) {
       constexpr int cur = decltype(cur_c)::value, nxt = (cur + 1) % RD;
@@ -470,6 +489,16 @@ __global__ __launch_bounds__(WAVES * 64, 4) void k_tq1_gemv_fp4(GemmArgs a, int 
       // group 4, whose scale sits next to that of group 3 in the lanes kb = 3. Several tokens: one group per window.
       const int g_first = PC == 3 ? kb : g_w0;
       const unsigned ia = (unsigned)((5 * (cb + c) + g_first) >> gs), ib = (unsigned)((5 * (cb + c) + (PC == 3 ? g_first + 1 : g_w1)) >> gs);
+      if constexpr (SR != 0) {
+        const unsigned ra = *(const lds_u16*)(sr_at + SB * (unsigned)((5 * (c & 3) + kb) >> gs));
+        const unsigned r4 = *(const lds_u16*)(sr_at + SB * (unsigned)((5 * (c & 3) + 4) >> gs));
+        const float sa = SDT == BP_F16 ? f16_bits_to_f32((uint16_t)ra) : __uint_as_float(ra << 16);
+        const float s4 = SDT == BP_F16 ? f16_bits_to_f32((uint16_t)r4) : __uint_as_float(r4 << 16);
+        const float inv_a = __uint_as_float(*(const lds_u32*)(cbase + F4_INV_OFF + 4 * kb));
+        const float inv_4 = __uint_as_float(*(const lds_u32*)(cbase + F4_INV_OFF + 16)) * f4th;
+        total[0] += sa * inv_a * (C[0][0] + C[0][1] + C[0][2] * (1.f / 256.f)) + s4 * inv_4 * C[0][3];
+        return;
+      }
 #pragma unroll
       for (int s = 0; s < GR; ++s) {
         unsigned ra, rb;  // the scale of group g_first, and the one after it (bits as stored)
@@ -510,23 +539,33 @@ __global__ __launch_bounds__(WAVES * 64, 4) void k_tq1_gemv_fp4(GemmArgs a, int 
     // scales last: the waits at the head of the loop are counted along this path too, and here as there the
     // loads of later chunks and of the scales are the ones in flight behind the chunk that is needed.
     if (pass == 0 || !chain) {
+      // (SR: the first round's scales are requested before the ring's loads, as in the loop - where a round's refills lie
+      // between a round's scales and the wait for them - so that the wait at the head of the loop counts those loads on
+      // this path too and does not drain the ring)
+      if (SR) fetch_round(0);
+      __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
       for (int u = 0; u < RD; ++u) {
         fetch_w(u, u, 0);
         fetch_w(u, u, 1);
       }
       __builtin_amdgcn_sched_barrier(0);
-      fetch_s(0);
+      if (SR) park_round();
+      else fetch_s(0);
       __builtin_amdgcn_sched_barrier(0);
     }
     // RD chunks per iteration with no way around any of them: the compiler counts the loads in flight along every
     // path into the head of the loop, and a path on which fewer are in flight would make every iteration wait
     const int full_end = ABL == 1 ? 0 : nchunks - nchunks % RD;
     for (int c0 = 0; c0 < full_end; c0 += RD) {
+      // (SR) the next round's scales are requested at the head of a round and parked in LDS at its end, after the
+      // round's last scale has been read: the round's 8 refills of the ring lie between, in straight-line code
+      if (SR) fetch_round(c0 + RD);
       step(c0, IC<0>{});
       step(c0 + 1, IC<1 % RD>{});
       if (RD > 2) step(c0 + 2, IC<2 % RD>{});
       if (RD > 3) step(c0 + 3, IC<3 % RD>{});
+      if (SR) park_round();
     }
     if (ABL != 1 && nchunks - full_end > 0) step(full_end, IC<0>{});  // uniform
     if (ABL != 1 && nchunks - full_end > 1) step(full_end + 1, IC<1 % RD>{});
@@ -565,9 +604,10 @@ int f4_cus() {  // compute units of the current device (256 if the query fails);
   return known[dev];
 }
 
-template <int SDT, int WAVES, int ABL = 0, int NTOK = 1>
+template <int SDT, int WAVES, int ABL = 0, int NTOK = 1, int SR = 0>
 int launch_f4_k(const GemmArgs& a, hipStream_t s, const char* name, int nchunks, size_t lds, int seg_chunks = 0 /* chunks per launch (0: all) */, int first_row = 0) {
-  if (const int rc = raise_lds_limit<k_tq1_gemv_fp4<SDT, WAVES, ABL, NTOK>>(F4_LDS_MAX)) return rc;
+  if (const int rc = raise_lds_limit<k_tq1_gemv_fp4<SDT, WAVES, ABL, NTOK, SR>>(F4_LDS_MAX)) return rc;
+  if (SR) lds += (size_t)WAVES * F4_SCALE_SLOT;
   const int cus = f4_cus();
   // Every workgroup builds the tables of its expert's token, so a workgroup takes as many row blocks as still leaves
   // every CU its full set of resident workgroups (16 waves): all workgroups resident at once, one build each.
@@ -581,7 +621,7 @@ int launch_f4_k(const GemmArgs& a, hipStream_t s, const char* name, int nchunks,
   note_kernel(name);
   const int per = seg_chunks > 0 ? seg_chunks : nchunks;
   for (int cb = 0; cb < nchunks; cb += per) {
-    hipLaunchKernelGGL((k_tq1_gemv_fp4<SDT, WAVES, ABL, NTOK>), grid, dim3(WAVES * 64), lds, s, a, nchunks, cb, nchunks - cb < per ? nchunks - cb : per, (int)bpw, first_row);
+    hipLaunchKernelGGL((k_tq1_gemv_fp4<SDT, WAVES, ABL, NTOK, SR>), grid, dim3(WAVES * 64), lds, s, a, nchunks, cb, nchunks - cb < per ? nchunks - cb : per, (int)bpw, first_row);
     const int rc = check_launch(name);
     if (rc != BP_OK) return rc;
   }
@@ -619,7 +659,14 @@ int launch_f4(const GemmArgs& a, hipStream_t s, int first_row = 0) {
   // there are row blocks enough for every CU anyway (the tables are then built once per CU instead of twice).
   bool wide = lds > (size_t)F4_LDS_MAX / 2 || ((a.N + 255) / 256) * experts >= 4 * (int64_t)cus;
   if (tuning().f4w) wide = lds > (size_t)F4_LDS_MAX / 2 || tuning().f4w == 16;  // (development)
-  if (!wide) return launch_f4_k<SDT, 8>(a, s, "fp4_tq1_t1_w8", (int)nchunks, lds);
+  // 2-byte scales go by the round through LDS where the slots fit behind the tile and a row's scales start dword-aligned
+  constexpr int SR = SDT != BP_F32 ? 1 : 0;
+  const bool sr_ok = SR && (a.G * 2) % 4 == 0;
+  if (!wide) {
+    if (sr_ok && lds + 8 * F4_SCALE_SLOT <= (size_t)F4_LDS_MAX) return launch_f4_k<SDT, 8, 0, 1, SR>(a, s, "fp4_tq1_t1_w8", (int)nchunks, lds);
+    return launch_f4_k<SDT, 8>(a, s, "fp4_tq1_t1_w8", (int)nchunks, lds);
+  }
+  if (sr_ok && lds + 16 * F4_SCALE_SLOT <= (size_t)F4_LDS_MAX) return launch_f4_k<SDT, 16, 0, 1, SR>(a, s, "fp4_tq1_t1_w16", (int)nchunks, lds);
   return launch_f4_k<SDT, 16>(a, s, "fp4_tq1_t1_w16", (int)nchunks, lds);
 }
 
