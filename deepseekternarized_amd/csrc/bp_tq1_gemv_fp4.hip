@@ -111,7 +111,7 @@ __device__ __forceinline__ int f4_pair_byte(int j, int kbA, int hf) {
 // chunk's two scales per lane are two 2-byte LDS reads.
 template <int SDT, int WAVES, int ABL = 0, int NTOK = 1, int SR = 0>
 __global__ __launch_bounds__(WAVES * 64, 4) void k_tq1_gemv_fp4(GemmArgs a, int total_chunks, int first_chunk, int nchunks, int bpw /* row blocks per workgroup */, int first_row) {
-  static_assert(!SR || (NTOK == 1 && SDT != BP_F32 && F4_GR == 1 && F4_RD == 4), "scales by the round: one token, one tile per wave, 2-byte scales, rounds of 4 chunks");
+  static_assert(!SR || (SDT != BP_F32 && F4_GR == 1), "scales by the round: one tile per wave, 2-byte scales (a round of 2 or 4 chunks is 20 or 40 bytes of a row's scales)");
   constexpr int THREADS = WAVES * 64, GR = F4_GR, RD = NTOK <= 2 ? F4_RD : 2, BD = F4_BD, AD = F4_AD, PAIRS = NTOK <= 2 ? F4_PAIRS : 0;
   static_assert(!PAIRS || RD % 2 == 0, "pairs of chunks need an even ring");
   static_assert(NTOK == 1 || (GR == 1 && AD == 0 && NTOK % 2 == 0), "several tokens: one tile per wave, one operand A buffer, token pairs");
@@ -312,7 +312,7 @@ __global__ __launch_bounds__(WAVES * 64, 4) void k_tq1_gemv_fp4(GemmArgs a, int 
     u32x4 W[RD][GR][2];
     u32x2 SQ[GR];  // the scales of one chunk: refilled for the next chunk as soon as they have been applied
     // (SR) the wave's scale slot behind the tiles: [16 rows][80 bytes], 48 of them the scales of the round's 20 groups
-    const unsigned sr_at = (unsigned)(AT + nchunks * F4_CHUNK_BYTES + wave * F4_SCALE_SLOT + r16 * 80);
+    const unsigned sr_at = (unsigned)(AT + nchunks * NTOK * F4_CHUNK_BYTES + wave * F4_SCALE_SLOT + r16 * 80);
     u32x4 SN = {0u, 0u, 0u, 0u};  // (SR) the next round's scales of this lane's row: 16 bytes at 16 kb
 
   for (int pass = 0; pass < bpw; ++pass) {
@@ -365,7 +365,14 @@ __global__ __launch_bounds__(WAVES * 64, 4) void k_tq1_gemv_fp4(GemmArgs a, int 
       int64_t row0;
       int cc;
       target(c, row0, cc);
-      SN = buf_load16(srs, srow + 16u * kb, (unsigned)(row0 * a.G * SB) + SB * (unsigned)((5 * cc) >> gs));
+      SN = buf_load16(srs, srow + 16u * kb, (unsigned)(row0 * a.G * SB) + ((SB * (unsigned)((5 * (cb + cc)) >> gs)) & ~3u));
+    };
+    // byte offset, within the parked window of its round, of the scale of group g of chunk c
+    auto parked_at = [&](int c, int g) {
+      // (one token: rounds of 4 chunks from chunk 0, so a round starts 20 groups = a whole number of dwords into the row)
+      if (NTOK == 1) return SB * (unsigned)((5 * (c & (RD - 1)) + g) >> gs);
+      const unsigned first = (SB * (unsigned)((5 * (cb + (c & ~(RD - 1)))) >> gs)) & ~3u;
+      return SB * (unsigned)((5 * (cb + c) + g) >> gs) - first;
     };
     auto park_round = [&]() { *(lds_u32x4*)(sr_at + 16 * kb) = SN; };
     // (chunk slots and pipeline stages are compile-time constants: every register array below is indexed statically)
@@ -490,13 +497,26 @@ __global__ __launch_bounds__(WAVES * 64, 4) void k_tq1_gemv_fp4(GemmArgs a, int 
       const int g_first = PC == 3 ? kb : g_w0;
       const unsigned ia = (unsigned)((5 * (cb + c) + g_first) >> gs), ib = (unsigned)((5 * (cb + c) + (PC == 3 ? g_first + 1 : g_w1)) >> gs);
       if constexpr (SR != 0) {
-        const unsigned ra = *(const lds_u16*)(sr_at + SB * (unsigned)((5 * (c & 3) + kb) >> gs));
-        const unsigned r4 = *(const lds_u16*)(sr_at + SB * (unsigned)((5 * (c & 3) + 4) >> gs));
+        // the lane's two scales of the chunk from the round's parked window: group kb and group 4 (one token), or the
+        // groups of its two windows (several tokens)
+        const unsigned ra = *(const lds_u16*)(sr_at + parked_at(c, g_first));
+        const unsigned rb = *(const lds_u16*)(sr_at + parked_at(c, PC == 3 ? 4 : g_w1));
         const float sa = SDT == BP_F16 ? f16_bits_to_f32((uint16_t)ra) : __uint_as_float(ra << 16);
-        const float s4 = SDT == BP_F16 ? f16_bits_to_f32((uint16_t)r4) : __uint_as_float(r4 << 16);
-        const float inv_a = __uint_as_float(*(const lds_u32*)(cbase + F4_INV_OFF + 4 * kb));
-        const float inv_4 = __uint_as_float(*(const lds_u32*)(cbase + F4_INV_OFF + 16)) * f4th;
-        total[0] += sa * inv_a * (C[0][0] + C[0][1] + C[0][2] * (1.f / 256.f)) + s4 * inv_4 * C[0][3];
+        const float sb = SDT == BP_F16 ? f16_bits_to_f32((uint16_t)rb) : __uint_as_float(rb << 16);
+        if (PC == 3) {
+          const float inv_a = __uint_as_float(*(const lds_u32*)(cbase + F4_INV_OFF + 4 * kb));
+          const float inv_4 = __uint_as_float(*(const lds_u32*)(cbase + F4_INV_OFF + 16)) * f4th;
+          total[0] += sa * inv_a * (C[0][0] + C[0][1] + C[0][2] * (1.f / 256.f)) + sb * inv_4 * C[0][3];
+        } else {
+#pragma unroll
+          for (int tt = 0; tt < 2 * NPR; ++tt) {  // rows 4 lg + 2 (tt % 2) + p of the pair's two tiles
+            const unsigned ivb = cbase + (unsigned)(tt * F4_CHUNK_BYTES) + F4_INV_OFF;
+            const float inv_a = __uint_as_float(*(const lds_u32*)(ivb + 4 * g_w0)), inv_b = __uint_as_float(*(const lds_u32*)(ivb + 4 * g_w1));
+            const f32x4 c0 = C[2 * (tt >> 1)], c1 = C[2 * (tt >> 1) + 1];
+            const float s0 = (tt & 1) ? c0[2] + c0[3] : c0[0] + c0[1], s1 = (tt & 1) ? c1[2] + c1[3] : c1[0] + c1[1];
+            total[tt] += sa * inv_a * s0 + sb * inv_b * s1;
+          }
+        }
         return;
       }
 #pragma unroll
@@ -638,10 +658,19 @@ int launch_f4(const GemmArgs& a, hipStream_t s, int first_row = 0) {
   if (lds > (size_t)F4_LDS_MAX || nseg > 4) return BP_ERR_UNSUPPORTED;
   const int cus = f4_cus();
   const int64_t experts = a.E < a.T ? a.E : a.T;
+  // 2-byte scales go by the round through LDS where the slots fit behind the tiles and a row's scales start dword-aligned
+  constexpr int SRV = SDT != BP_F32 && NTOK <= 4 ? 1 : 0;
+  const bool sr_ok = SRV && (a.G * 2) % 4 == 0;
   if (NTOK > 1) {
     const bool wide = lds > (size_t)F4_LDS_MAX / 2 || ((a.N + 255) / 256) * experts >= 4 * (int64_t)cus;
-    if (!wide) return launch_f4_k<SDT, 8, 0, NTOK>(a, s, NTOK == 2 ? "fp4_tq1_m2_w8" : NTOK == 4 ? "fp4_tq1_m4_w8" : NTOK == 6 ? "fp4_tq1_m6_w8" : "fp4_tq1_m8_w8", (int)nchunks, lds, (int)seg, first_row);
-    return launch_f4_k<SDT, 16, 0, NTOK>(a, s, NTOK == 2 ? "fp4_tq1_m2_w16" : NTOK == 4 ? "fp4_tq1_m4_w16" : NTOK == 6 ? "fp4_tq1_m6_w16" : "fp4_tq1_m8_w16", (int)nchunks, lds, (int)seg, first_row);
+    const char* name8 = NTOK == 2 ? "fp4_tq1_m2_w8" : NTOK == 4 ? "fp4_tq1_m4_w8" : NTOK == 6 ? "fp4_tq1_m6_w8" : "fp4_tq1_m8_w8";
+    const char* name16 = NTOK == 2 ? "fp4_tq1_m2_w16" : NTOK == 4 ? "fp4_tq1_m4_w16" : NTOK == 6 ? "fp4_tq1_m6_w16" : "fp4_tq1_m8_w16";
+    if (!wide) {
+      if (sr_ok && lds + 8 * F4_SCALE_SLOT <= (size_t)F4_LDS_MAX) return launch_f4_k<SDT, 8, 0, NTOK, SRV>(a, s, name8, (int)nchunks, lds, (int)seg, first_row);
+      return launch_f4_k<SDT, 8, 0, NTOK>(a, s, name8, (int)nchunks, lds, (int)seg, first_row);
+    }
+    if (sr_ok && lds + 16 * F4_SCALE_SLOT <= (size_t)F4_LDS_MAX) return launch_f4_k<SDT, 16, 0, NTOK, SRV>(a, s, name16, (int)nchunks, lds, (int)seg, first_row);
+    return launch_f4_k<SDT, 16, 0, NTOK>(a, s, name16, (int)nchunks, lds, (int)seg, first_row);
   }
 #ifdef BP_DEV_ABLATIONS  // timing ablations (results are wrong): development builds only
   if (const char* t = getenv("BP_TUNE_F4ABL")) {
@@ -659,9 +688,7 @@ int launch_f4(const GemmArgs& a, hipStream_t s, int first_row = 0) {
   // there are row blocks enough for every CU anyway (the tables are then built once per CU instead of twice).
   bool wide = lds > (size_t)F4_LDS_MAX / 2 || ((a.N + 255) / 256) * experts >= 4 * (int64_t)cus;
   if (tuning().f4w) wide = lds > (size_t)F4_LDS_MAX / 2 || tuning().f4w == 16;  // (development)
-  // 2-byte scales go by the round through LDS where the slots fit behind the tile and a row's scales start dword-aligned
-  constexpr int SR = SDT != BP_F32 ? 1 : 0;
-  const bool sr_ok = SR && (a.G * 2) % 4 == 0;
+  constexpr int SR = SRV;
   if (!wide) {
     if (sr_ok && lds + 8 * F4_SCALE_SLOT <= (size_t)F4_LDS_MAX) return launch_f4_k<SDT, 8, 0, 1, SR>(a, s, "fp4_tq1_t1_w8", (int)nchunks, lds);
     return launch_f4_k<SDT, 8>(a, s, "fp4_tq1_t1_w8", (int)nchunks, lds);
