@@ -132,6 +132,9 @@ __global__ __launch_bounds__(WAVES * 64, 4) void k_tq1_gemv_fp4(GemmArgs a, int 
   if (tok >= o1) return;
   const int ntok = o1 - tok < NTOK ? (int)(o1 - tok) : NTOK;
   const int npairs = (ntok + 1) >> 1;  // token pairs the expert has in this launch: the others' matrix instructions are left out
+  float xsc[NTOK];  // int8 activations: the tokens' scales
+#pragma unroll
+  for (int tt = 0; tt < NTOK; ++tt) xsc[tt] = a.x_dtype == BP_I8 && tt < ntok ? a.x_scale[tok + tt] : 1.f;
   // the tiles of the NTOK tokens are interleaved chunk by chunk (a pair's tiles are a constant apart)
   auto tile_at = [](int tt, int c) { return AT + (c * NTOK + tt) * F4_CHUNK_BYTES; };
   const int gs = a.group == 256 ? 1 : 0;  // scale groups of 256: two 128-wide work groups share a scale
@@ -319,8 +322,20 @@ __global__ __launch_bounds__(WAVES * 64, 4) void k_tq1_gemv_fp4(GemmArgs a, int 
     const int64_t n0 = block_row0(pass), n0_next = pass + 1 < bpw ? block_row0(pass + 1) : n0;
     const bool wave_live = (((int64_t)blockIdx.x * bpw + pass) * WAVES + wave) * (16 * GR) < a.N;
     float total[NTOK > 1 ? NTOK : GR];  // per token (this lane's two groups of every chunk), or (one token) per row tile
+    // The outputs this block is added to are requested now and used when the block ends: read where they are added, the
+    // load would be the youngest one in flight and the wait for it would drain the ring once per block. (Device scope:
+    // with stacked terms the value may be one this wave stored a term ago.)
+    // (up to 4 tokens; beyond, the registers are not there)
+    constexpr bool EARLY = NTOK <= 4;
+    float before[NTOK > 1 ? NTOK : GR];
 #pragma unroll
-    for (int s = 0; s < (NTOK > 1 ? NTOK : GR); ++s) total[s] = 0.f;
+    for (int s = 0; s < (NTOK > 1 ? NTOK : GR); ++s) {
+      total[s] = 0.f;
+      const int tile = NTOK > 1 ? 0 : s, tt = NTOK > 1 ? s : 0;
+      before[s] = 0.f;
+      if (EARLY && kb == 0 && wave_live && n0 + 16 * tile < a.N && tt < ntok)
+        before[s] = __hip_atomic_load(a.out + (tok + tt) * a.N + n0 + 16 * tile + r16, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    }
     // chunk c of this block, or (c >= nchunks, chained) chunk c - nchunks of the next one: row offset (scalar) and chunk
     auto target = [&](int c, int64_t& row0, int& cc) {
       const bool over = chain && c >= nchunks && pass + 1 < bpw;
@@ -599,7 +614,8 @@ __global__ __launch_bounds__(WAVES * 64, 4) void k_tq1_gemv_fp4(GemmArgs a, int 
     const int tile = NTOK > 1 ? 0 : s, tt = NTOK > 1 ? s : 0;
     if (kb == 0 && wave_live && n0 + 16 * tile < a.N && tt < ntok) {
       float* o = a.out + (tok + tt) * a.N + n0 + 16 * tile + r16;
-      *o += a.x_dtype == BP_I8 ? t * a.x_scale[tok + tt] : t;
+      const float was = EARLY ? before[s] : __hip_atomic_load(o, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+      *o = was + (a.x_dtype == BP_I8 ? t * xsc[tt] : t);
     }
   }
   }  // pass
