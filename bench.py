@@ -63,6 +63,8 @@ def arithmetic_of(kernel):
         return "activations as 2 E4M3 pieces under a per-group power-of-two prescale x E2M1 weights (v_mfma_f32_16x16x128_f8f6f4), fp32 accumulate"
     if kernel.startswith("gemm_tq1"):
         return "activations as 2 E4M3 pieces under E8M0 block scales (blocks of 20) x E2M1 weights (v_mfma_scale_f32_16x16x128_f8f6f4), fp32 accumulate, scale per 128-group applied in fp32"
+    if kernel.startswith("gemm_tq2f"):
+        return "activations as 2 E4M3 pieces under E8M0 block scales (blocks of 32), converted once into a workspace, x E2M1 weights (v_mfma_scale_f32_16x16x128_f8f6f4), fp32 accumulate, scale per 128-group applied in fp32"
     if kernel.startswith(("mfma_tq2_bf16", "gemm_tq2_bf16", "mfma_tq1")):
         return "bf16 activations x bf16-decoded trits (v_mfma_f32_16x16x32_bf16), fp32 accumulate, scale per 128-group applied in fp32"
     if kernel.startswith(("mfma_tq2_i8", "gemm_tq2_i8")):

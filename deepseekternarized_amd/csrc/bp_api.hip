@@ -29,13 +29,14 @@ void note_kernel(const char* name) {
 }
 
 namespace {
-Tuning g_tuning = {0, 0, 0, 0, -1, 0};
+Tuning g_tuning = {0, 0, 0, 0, 0, -1, 0};
 std::once_flag g_tuning_once;
 void read_tuning() {
-  Tuning t = {0, 0, 0, 0, -1, 0};
+  Tuning t = {0, 0, 0, 0, 0, -1, 0};
   if (const char* v = getenv("BP_TUNE_R")) t.r = atoi(v);
   if (const char* v = getenv("BP_TUNE_WAVES")) t.waves = atoi(v);
   if (const char* v = getenv("BP_TUNE_TQ1")) t.tq1 = v[0];
+  if (const char* v = getenv("BP_TUNE_TQ2G")) t.tq2g = v[0];
   if (const char* v = getenv("BP_TUNE_F4W")) t.f4w = atoi(v);
   if (const char* v = getenv("BP_TUNE_F4T")) t.f4t = atoi(v);
   if (const char* v = getenv("BP_TUNE_CPT")) t.cpt = atoi(v);
@@ -75,13 +76,10 @@ extern "C" int bp_set_kernel_policy(int policy) {
 static bool valid_scale_dtype(int d) { return d == BP_F32 || d == BP_F16 || d == BP_BF16; }
 static bool valid_act_dtype(int d) { return d == BP_I8 || d == BP_BF16 || d == BP_F16 || d == BP_F32; }
 
-extern "C" int bp_ternary_grouped_gemm(float* out, const void* x, int x_dtype, const float* x_scale,
-                                       const int64_t* offsets, const int64_t* offsets_host,
-                                       const uint8_t* const* packed, const void* const* w_scale, int scale_dtype,
-                                       int n_terms, int64_t T, int64_t N, int64_t K, int64_t Kp, int64_t G,
-                                       int64_t group, int64_t E, int fmt, int64_t max_rows, const int8_t* lut1,
-                                       void* stream) {
-  (void)lut1;  // the kernels carry the table themselves; see bp_tq1_lut for the tensor form
+static int grouped_gemm(float* out, const void* x, int x_dtype, const float* x_scale, const int64_t* offsets,
+                        const int64_t* offsets_host, const uint8_t* const* packed, const void* const* w_scale,
+                        int scale_dtype, int n_terms, int64_t T, int64_t N, int64_t K, int64_t Kp, int64_t G, int64_t group,
+                        int64_t E, int fmt, int64_t max_rows, void* workspace, size_t workspace_bytes, void* stream) {
   g_error[0] = 0;
   g_kernel[0] = 0;
   if (!valid_act_dtype(x_dtype)) return fail(BP_ERR_ARG, "unexpected ternary GEMM activation dtype");
@@ -128,8 +126,40 @@ extern "C" int bp_ternary_grouped_gemm(float* out, const void* x, int x_dtype, c
   }
   a.x_dtype = x_dtype; a.scale_dtype = scale_dtype; a.n_terms = n_terms; a.fmt = fmt;
   a.T = T; a.N = N; a.K = K; a.Kp = Kp; a.G = G; a.group = group; a.E = E; a.max_rows = max_rows;
+  a.stage = (unsigned char*)workspace;
+  a.stage_bytes = workspace ? (int64_t)workspace_bytes : 0;
 
   return run_gemm(a, (hipStream_t)stream);
+}
+
+extern "C" int bp_ternary_grouped_gemm(float* out, const void* x, int x_dtype, const float* x_scale,
+                                       const int64_t* offsets, const int64_t* offsets_host,
+                                       const uint8_t* const* packed, const void* const* w_scale, int scale_dtype,
+                                       int n_terms, int64_t T, int64_t N, int64_t K, int64_t Kp, int64_t G,
+                                       int64_t group, int64_t E, int fmt, int64_t max_rows, const int8_t* lut1,
+                                       void* stream) {
+  (void)lut1;  // the kernels carry the table themselves; see bp_tq1_lut for the tensor form
+  return grouped_gemm(out, x, x_dtype, x_scale, offsets, offsets_host, packed, w_scale, scale_dtype, n_terms, T, N, K, Kp, G,
+                      group, E, fmt, max_rows, nullptr, 0, stream);
+}
+
+extern "C" size_t bp_grouped_gemm_workspace_bytes(int x_dtype, int64_t T, int64_t N, int64_t K, int64_t E, int fmt) {
+  if (fmt != BP_TQ2 || x_dtype != BP_BF16 || (N < 1024 && tuning().tq2g != 'f')) return 0;
+  return gemm_tq2f_workspace_bytes(T, K, E);
+}
+
+extern "C" int bp_ternary_grouped_gemm_ws(float* out, const void* x, int x_dtype, const float* x_scale,
+                                          const int64_t* offsets, const int64_t* offsets_host,
+                                          const uint8_t* const* packed, const void* const* w_scale, int scale_dtype,
+                                          int n_terms, int64_t T, int64_t N, int64_t K, int64_t Kp, int64_t G,
+                                          int64_t group, int64_t E, int fmt, int64_t max_rows, void* workspace,
+                                          size_t workspace_bytes, void* stream) {
+  if (workspace && ((uintptr_t)workspace & 255) != 0) {
+    g_error[0] = 0;
+    return fail(BP_ERR_ARG, "workspace must be 256-byte aligned");
+  }
+  return grouped_gemm(out, x, x_dtype, x_scale, offsets, offsets_host, packed, w_scale, scale_dtype, n_terms, T, N, K, Kp, G,
+                      group, E, fmt, max_rows, workspace, workspace_bytes, stream);
 }
 
 namespace bp {

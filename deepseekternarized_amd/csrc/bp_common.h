@@ -33,6 +33,9 @@ struct GemmArgs {
   const int32_t* tile_count;
   int64_t tile_cap;
   int overwrite;  // tile-list mode: the kernel's result replaces `out` instead of being added to it (one launch covers all of K and all terms)
+  // Workspace of the caller for kernels that convert the activations in a pass of their own (NULL: those kernels are not used).
+  unsigned char* stage;
+  int64_t stage_bytes;
 };
 
 __device__ __forceinline__ int64_t clamp_i64(int64_t v, int64_t lo, int64_t hi) { return v < lo ? lo : (v > hi ? hi : v); }
@@ -65,6 +68,7 @@ struct Tuning {
   int r;       // BP_TUNE_R: 16-row tiles per wave of the TQ2 kernel (1, 2)
   int waves;   // BP_TUNE_WAVES: waves per workgroup (8, 16)
   char tq1;    // BP_TUNE_TQ1: 'l' table-lookup GEMV, 'm' 16-token MFMA kernel (first letter of the value)
+  char tq2g;   // BP_TUNE_TQ2G: 'b' (bf16) never the fp8 x fp4 grouped GEMM over converted activations, 'f' (fp4) wherever it can run
   int f4w;     // BP_TUNE_F4W: waves per workgroup of the fp8 x fp4 GEMV (8, 16)
   int f4t;     // BP_TUNE_F4T: routed rows per expert up to which launches of 8 rows are used (-1 = default)
   int cpt;     // BP_TUNE_CPT: chunks per table pass of the table-lookup GEMV
@@ -91,6 +95,8 @@ int raise_lds_limit(int bytes) {
 int run_gemm(const GemmArgs& a, hipStream_t s);
 // True when a launch in tile-list mode would run on one of the 32-token-tile kernels (which honour tiles / overwrite).
 bool gemm_tiles_supported(const GemmArgs& a);
+// Workspace bytes of the TQ2 grouped GEMM over converted activations (GemmArgs::stage) for T rows in all; 0: not available.
+size_t gemm_tq2f_workspace_bytes(int64_t T, int64_t K, int64_t E);
 int launch_general(const GemmArgs& a, hipStream_t s);
 // Returns BP_ERR_UNSUPPORTED (without setting an error message) when the shape is outside the
 // tuned kernels' preconditions.

@@ -433,6 +433,10 @@ int launch_gemm_sd(const GemmArgs& a, hipStream_t s, const char* name, const cha
 
 // Preconditions (checked by mfma_supports): group 128, K % 256 == 0, K >= 1024, N % 16 == 0, 16-byte aligned x / packed / scales.
 int launch_gemm_tq2(const GemmArgs& a, hipStream_t s) {
+  if (a.stage && tuning().tq2g != 'b') {  // with a workspace: the fp8 x fp4 kernel over converted activations (development: BP_TUNE_TQ2G=bf16 keeps this file's kernel)
+    const int rc = launch_gemm_tq2f(a, s);
+    if (rc != BP_ERR_UNSUPPORTED) return rc;
+  }
 #ifdef BP_DEV_ABLATIONS  // timing ablations (results are wrong): development builds only
   if (const char* t = getenv("BP_TUNE_ABL")) {
     const size_t lds = 2 * gemm_tile_bytes<BP_BF16>() + (size_t)GROWS * a.G * 2;

@@ -1,0 +1,693 @@
+// TQ2 grouped GEMM for bf16 activations and token tiles of 16 or 32 rows on the scaled fp8 x fp4 matrix instruction
+// (v_mfma_scale_f32_16x16x128_f8f6f4), over activations converted beforehand: 2-bit codes become fp4 operands with four
+// vector instructions per 16 weights, and one matrix instruction covers exactly one 128-wide scale group.
+//
+// Contract as everywhere (boilerplate/kernels/ternary_cuda.py:58-63, boilerplate/kernels/csrc/ternary_cuda_kernel.cu:44-99):
+// out[t, n] += sum_g scale[n, g] * sum_{k in g} x[t, k] * trit[n, k], float32 accumulation.
+//
+//  * Weights as fp4. A code u = trit + 1 placed at bits [2:1] of a nibble is the E2M1 number u (0000 = 0, 0010 = 1,
+//    0100 = 2), so a packed dword (16 codes) becomes two operand dwords by (w << 1) & 0x66666666 (even codes) and
+//    (w >> 1) & 0x66666666 (odd codes): no table, no LDS. The products then carry sum x * u; every group's accumulator
+//    starts from -sum x, which leaves sum x * (u - 1). The unused code 3 reads 4 - 1 = +3 (pack never writes it).
+//  * A lane loads 16 bytes of its row per 64-byte window (rows are 16-byte aligned: K % 256 == 0); two
+//    v_permlane32_swap leave every lane with 8 bytes of each of the window's two groups, so the four lanes of a row
+//    supply the 128 weights of ONE group to a matrix instruction: lane quarter kb holds the group's weights
+//    64 (kb % 2) + 32 (kb / 2) .. + 31.
+//  * Activations as two fp8 (E4M3) pieces under a power-of-two block scale that the instruction applies itself: the
+//    32 activations that meet one lane of operand B (32 consecutive k) share one E8M0 scale 2^(e - 7), e the exponent
+//    of the block's largest magnitude; y = x / scale = p0 + p1, p0 = y rounded to E4M3, p1 the rounded remainder.
+//    bf16 activations are exactly p0 + p1 down to 2^-9 of their block's largest magnitude; less than 2^-17 of it is
+//    dropped below. Products fp8 x fp4 are exact. A block that holds a NaN or an infinity makes the token's outputs NaN.
+//  * The conversion is vector-ALU work, about as many cycles per token as a workgroup's matrix instructions, and every
+//    row block of an expert would repeat it. So it runs once, in a kernel of its own (k_stage_tq2f), into a workspace of
+//    the caller: per token tile of 32 and 64-byte window, 17 KiB in exactly the layout the GEMM's LDS buffer has
+//    (operands in operand-A register order, block scales, offset sums). The GEMM copies a window's 17 KiB from there.
+//  * A GEMM workgroup (8 waves) owns 512 output rows x 32 tokens; a wave 64 rows (4 row tiles) x 32 tokens (2 token
+//    tiles): an operand A read from LDS feeds 4 matrix instructions, a decoded weight meets 32 tokens. Weights, scales
+//    and staged activations are requested two windows ahead, one load after each row tile's matrix instructions (all at
+//    once they fill the CU's vector-memory queue and the waves that come last wait thousands of cycles to issue theirs);
+//    every wave issues the same loads in the same order in every window and the stacked terms run as one sequence of
+//    windows, so every wait is for loads at least a window old and counts the younger ones exactly. One barrier per window.
+//
+// Operand layout of the instruction (A = fp8, 8 VGPRs; B = fp4, 4 VGPRs; established by probing on gfx950): B lane
+// (n = lane % 16, kb = lane / 16), VGPR w, nibble q is paired with A lane (m = lane % 16, 2 (kb % 2) + w / 2), VGPR
+// 4 (kb / 2) + 2 (w % 2) + q / 4, byte q % 4; the E8M0 scale of A row m for the 32 slots of B lane kb is byte `opsel`
+// of the scale operand in lane (m, kb); C lane (n, lg) holds rows 4 lg + i.
+#include <type_traits>
+
+#include "bp_mfma.h"
+
+namespace bp {
+namespace {
+
+typedef int i32x8 __attribute__((ext_vector_type(8)));
+template <int V>
+using FC = std::integral_constant<int, V>;
+
+constexpr int F_WAVES = 8;                         // waves per workgroup
+constexpr int F_RT = 4;                            // 16-row tiles per wave
+constexpr int F_THREADS = F_WAVES * 64;
+constexpr int F_ROWS = F_WAVES * 16 * F_RT;        // output rows per workgroup
+constexpr int F_OPS = 2 * 2 * 2 * 2048;            // operands of a window: 2 groups x 2 token tiles x 2 pieces x 2 KiB
+constexpr int F_SCL = 2 * 64 * 4;                  // ... the block scales: per token tile one dword per lane (byte g = group g)
+constexpr int F_SUM = 2 * 32 * 4;                  // ... and the offset sums: [group][token] float
+constexpr int F_TAIL = F_SCL + F_SUM;              // (48 x 16 bytes)
+constexpr int F_FB = 32 * 544;                     // a staged window of a token tile: operands, scales, sums, padding (544 bytes per token: a multiple of 16)
+static_assert(F_OPS + F_TAIL <= F_FB && F_OPS == F_THREADS * 32 && F_TAIL % 16 == 0, "a staged window: two 16-byte pieces per thread and a tail");
+constexpr int F_SC = 2 * F_FB;                     // LDS: two staged windows, then the rows' scales: 2 slots (window parity) of [512 rows][2 groups] as stored
+constexpr int f_lds_bytes(int scale_bytes) { return F_SC + 2 * F_ROWS * 2 * scale_bytes; }  // 38,912 (16-bit scales) / 43,008 (float32)
+
+template <int N, class F>
+__device__ __forceinline__ void static_for(F&& f) {
+  if constexpr (N > 0) {
+    static_for<N - 1>(f);
+    f(FC<N - 1>{});
+  }
+}
+
+__device__ __forceinline__ unsigned moved(unsigned v) {  // v in a register of its own
+  unsigned r;
+  asm("v_mov_b32 %0, %1" : "=&v"(r) : "v"(v));
+  return r;
+}
+
+// Where token tile (expert e, first row tok0) keeps its staged windows: tile z of expert e starts 32 (e + z) + offsets[e]
+// tokens into the workspace, so tiles never overlap whatever the experts' row counts are.
+__device__ __forceinline__ unsigned char* staged_tile(const GemmArgs& a, int64_t e, int64_t tok0) {
+  return a.stage + (tok0 + 32 * e) * (a.K / 256) * (F_FB / 32);
+}
+
+// ---- the conversion: one workgroup per (token tile, window). Wave = (token tile stt, group sg of the window, token half
+// mh); lane = (token m3 of 8, quarter kbA of operand A's lanes, half hi of its registers): the thread converts the 16
+// activations that fill registers 4 hi .. 4 hi + 3 of A lane (m, kbA) for the group's instruction: k = 64 (kbA / 2) +
+// 32 hi + 16 (kbA % 2) .. + 15 of the group. A token's group is the 8 lanes (kbA, hi) of one wave: 256 consecutive bytes.
+__global__ __launch_bounds__(F_THREADS) void k_stage_tq2f(GemmArgs a) {
+  const int wave = __builtin_amdgcn_readfirstlane((int)(threadIdx.x >> 6)), lane = threadIdx.x & 63;
+  const TileRef tr = tile_ref(a, blockIdx.x, blockIdx.z);
+  if (!tr.live) return;  // uniform for the workgroup
+  const int64_t tok0 = tr.tok0;
+  const int ntok = (int)(tr.o1 - tok0 < 32 ? tr.o1 - tok0 : 32);
+  const int s = blockIdx.y;  // the window
+  const int stt = wave & 1, sg = (wave >> 1) & 1, mh = wave >> 2;
+  const int m3 = lane & 7, kbA = (lane >> 3) & 3, hi = lane >> 5;
+  const int sm = 8 * mh + m3;
+  unsigned char* dst = staged_tile(a, tr.e, tok0) + (int64_t)s * F_FB;
+  if (stt == 1 && ntok <= 16) {  // no second token tile: its scales and sums are read all the same (and multiply nothing that is stored)
+    if ((kbA & 1) == 0) dst[F_OPS + (stt * 64 + ((kbA >> 1) + 2 * hi) * 16 + sm) * 4 + sg] = 127;
+    if (kbA == 0 && hi == 0) *(float*)(dst + F_OPS + F_SCL + (sg * 32 + 16 * stt + sm) * 4) = 0.f;
+    return;
+  }
+  int srow = 16 * stt + sm;
+  if (srow >= ntok) srow = ntok - 1;  // rows past the expert's tokens repeat its last one (their results are not stored)
+  const uint16_t* xp = (const uint16_t*)a.x + (tok0 + srow) * a.K + 256 * (int64_t)s + 128 * sg + 64 * (kbA >> 1) + 32 * hi + 16 * (kbA & 1);
+  const u32x4 raw[2] = {*(const u32x4*)xp, *(const u32x4*)(xp + 8)};
+  float y[16];
+#pragma unroll
+  for (int i = 0; i < 8; ++i) {
+    const unsigned v = raw[i >> 2][i & 3];
+    y[2 * i] = __uint_as_float(v << 16);
+    y[2 * i + 1] = __uint_as_float(v & 0xffff0000u);
+  }
+  unsigned mx = 0;
+#pragma unroll
+  for (int i = 0; i < 16; ++i) {
+    const unsigned v = __float_as_uint(y[i]) & 0x7fffffffu;
+    mx = mx > v ? mx : v;
+  }
+  {  // the block of 32 = this lane's 16 and those of the lane with the other kbA % 2
+    const unsigned other = (unsigned)__shfl_xor((int)mx, 8, 64);
+    mx = mx > other ? mx : other;
+  }
+  const int ex = (int)(mx >> 23);
+  int sh = 134 - ex;  // brings the block's largest magnitude into [128, 256)
+  sh = sh > 126 ? 126 : sh;
+  float mult = __uint_as_float((unsigned)(127 + sh) << 23);
+  if (ex == 255) mult = __uint_as_float(0x7fc00000u);  // a NaN or an infinity in the block: every slot becomes NaN
+  // activation j of the 16 goes to register 2 (j % 2) + j / 8, byte (j % 8) / 2: bytes t, t + 1 of a register are
+  // activations j, j + 2
+  u32x4 p0, p1;
+  float used = 0.f;  // sum of what the two pieces represent, in the block's scaled domain
+#pragma unroll
+  for (int d = 0; d < 4; ++d) {
+    const int v1 = d >> 1, v0 = d & 1;
+    int c0 = 0, c1 = 0;
+#pragma unroll
+    for (int h = 0; h < 2; ++h) {
+      const float f0 = y[8 * v0 + 4 * h + v1] * mult, f1 = y[8 * v0 + 4 * h + 2 + v1] * mult;
+      c0 = h == 0 ? __builtin_amdgcn_cvt_pk_fp8_f32(f0, f1, c0, false) : __builtin_amdgcn_cvt_pk_fp8_f32(f0, f1, c0, true);
+      const float b0 = h == 0 ? __builtin_amdgcn_cvt_f32_fp8(c0, 0) : __builtin_amdgcn_cvt_f32_fp8(c0, 2);
+      const float b1 = h == 0 ? __builtin_amdgcn_cvt_f32_fp8(c0, 1) : __builtin_amdgcn_cvt_f32_fp8(c0, 3);
+      const float r0 = f0 - b0, r1 = f1 - b1;
+      c1 = h == 0 ? __builtin_amdgcn_cvt_pk_fp8_f32(r0, r1, c1, false) : __builtin_amdgcn_cvt_pk_fp8_f32(r0, r1, c1, true);
+      const float e0 = h == 0 ? __builtin_amdgcn_cvt_f32_fp8(c1, 0) : __builtin_amdgcn_cvt_f32_fp8(c1, 2);
+      const float e1 = h == 0 ? __builtin_amdgcn_cvt_f32_fp8(c1, 1) : __builtin_amdgcn_cvt_f32_fp8(c1, 3);
+      used += (b0 + e0) + (b1 + e1);
+    }
+    p0[d] = (unsigned)c0;
+    p1[d] = (unsigned)c1;
+  }
+  unsigned char* ob = dst + ((sg * 2 + stt) * 2) * 2048 + (kbA * 2 + hi) * 256 + sm * 16;
+  *(u32x4*)ob = p0;
+  *(u32x4*)(ob + 2048) = p1;
+  // the block's scale: byte sg of the scale operand's dword in lane (m, kb) with kb % 2 = kbA / 2, kb / 2 = hi
+  if ((kbA & 1) == 0) dst[F_OPS + (stt * 64 + ((kbA >> 1) + 2 * hi) * 16 + sm) * 4 + sg] = (unsigned char)(127 - sh);
+  // the group's offset sum: what the pieces represent, back in the activations' units, over the token's 8 lanes
+  float part = used * __uint_as_float((unsigned)(127 - sh) << 23);
+  if (ex == 255) part = __uint_as_float(0x7fc00000u);
+  part += __shfl_xor(part, 8, 64);
+  part += __shfl_xor(part, 16, 64);
+  part += __shfl_xor(part, 32, 64);
+  if (kbA == 0 && hi == 0) *(float*)(dst + F_OPS + F_SCL + (sg * 32 + 16 * stt + sm) * 4) = -part;
+}
+
+template <int SDT>
+__global__ __launch_bounds__(F_THREADS, 2) void k_gemm_tq2f(GemmArgs a) {
+  constexpr int SB = SDT == BP_F32 ? 4 : 2;
+
+  const int wave = __builtin_amdgcn_readfirstlane((int)(threadIdx.x >> 6)), lane = threadIdx.x & 63;
+  const int r16 = lane & 15, kb = lane >> 4;
+  // Workgroups are dealt to the 8 XCDs round-robin by linear index; the row blocks of one expert read the same
+  // activations, so they get linear indices 8 apart (same XCD, one L2).
+  const int row_blocks = (int)((a.N + F_ROWS - 1) / F_ROWS);
+  const int wg_block = (int)((blockIdx.x >> 3) % (unsigned)row_blocks);
+  const TileRef tr = tile_ref(a, (blockIdx.x & 7) + 8 * (int64_t)((blockIdx.x >> 3) / (unsigned)row_blocks), blockIdx.z);
+  if (!tr.live) return;  // uniform for the workgroup
+  const int64_t e = tr.e, tok0 = tr.tok0, o1 = tr.o1;
+  const int ntok = (int)(o1 - tok0 < 32 ? o1 - tok0 : 32);
+  const bool two = ntok > 16;  // the second token tile holds tokens
+  const int64_t n_base = (int64_t)wg_block * F_ROWS;
+  const int64_t n_wave = n_base + wave * (16 * F_RT);
+
+  const int nwin = (int)(a.K / 256);      // 64-byte windows of a row = pairs of 128-wide groups
+  const int NW = nwin * a.n_terms;        // the stacked terms, one after the other
+  const int gs = a.group == 256 ? 1 : 0;  // scale groups of 256: the two groups of a window share a scale
+
+  const unsigned alane = (unsigned)(kb * 512 + r16 * 16);
+  int ones = 0x7f7f7f7f;  // operand B's block scales: 2^0
+  asm volatile("" : "+v"(ones));
+  unsigned m66 = 0x66666666u;
+  asm volatile("" : "+s"(m66));
+
+  // ---- the load stream. Window w of the sequence is window w % nwin of term w / nwin; (lterm, ls) names the next window
+  // to request. Per window every wave issues, in this order: the thread's three pieces of the staged window, the thread's
+  // row's two scales, the wave's four weight loads. Requests past the last window repeat it (never used).
+#if defined(BP_DEV_ABLATION) && (BP_DEV_ABLATION == 32 || BP_DEV_ABLATION == 38)  // timing only (wrong results): quads of lanes read 64 contiguous bytes
+  const unsigned voff = (unsigned)(lane >> 2) * (unsigned)a.Kp + 16u * (lane & 3);
+#else
+  const unsigned voff = (unsigned)r16 * (unsigned)a.Kp + 16u * kb;
+#endif
+  unsigned wrow[F_RT];  // byte offset of the row tile's first row (a tile past N repeats the wave's first tile and is not stored)
+#pragma unroll
+  for (int r = 0; r < F_RT; ++r) {
+    int64_t row = n_wave + 16 * r;
+    if (row >= a.N) row = n_wave < a.N ? n_wave : 0;
+    wrow[r] = (unsigned)(row * a.Kp);
+  }
+  const int64_t my_row = n_base + threadIdx.x;
+  const unsigned my_scales = my_row < a.N ? (unsigned)(my_row * a.G * SB) : 0xfffffff0u;  // rows past N: zeros
+  const __amdgpu_buffer_rsrc_t xrs = make_rsrc(staged_tile(a, e, tok0), (int64_t)nwin * F_FB);
+  const unsigned tail_off = threadIdx.x < F_TAIL / 16 ? (unsigned)(F_OPS + 16 * threadIdx.x) : 0xfffffff0u;  // (past the range: no memory access)
+  int lterm = 0, ls = 0;
+  __amdgpu_buffer_rsrc_t wrs, srs;
+  auto set_term = [&](int term) {
+    const unsigned char* wbeg = a.packed[term];
+    wrs = make_rsrc(wbeg + e * a.N * a.Kp, (a.E - e) * a.N * a.Kp);
+    const unsigned char* sbeg = (const unsigned char*)a.w_scale[term];
+    const unsigned char* expert_scales = sbeg + e * a.N * a.G * SB;
+    srs = make_rsrc(expert_scales, (sbeg + a.E * a.N * a.G * SB) - expert_scales);
+  };
+  set_term(0);
+  u32x4 W[2][F_RT];        // the weights of the windows of either parity
+  u32x4 xa[2][3];          // ... the thread's pieces of their staged activations (two of the operands, one of the tail)
+  unsigned sq[2][SB / 2];  // ... the thread's row's scales: [group 0 | group 1] as stored
+  int sodd[2] = {0, 0};    // ... and, with one scale per window, which of the loaded entries is the window's (uniform)
+  // part 0..3: the weights of row tile `part`; 4: the scales; 5, 6, 7: the staged activations; 8: on to the next window.
+  // Order within a window: 5, 6, 7, 4 (with the first group's matrix instructions), 0 .. 3 (with the second group's), 8.
+  auto request = [&](auto p_c, auto part_c) {
+    constexpr int P = decltype(p_c)::value, PART = decltype(part_c)::value;
+    const unsigned s = (unsigned)ls;
+    if (PART < F_RT) W[P][PART] = buf_load16(wrs, voff, wrow[PART] + 64u * s);
+    if (PART == 4) {
+      // entries (2 s) >> gs and (2 s + 1) >> gs of the row, by one load of the same width either way. gs = 1: 16-bit
+      // scales - the aligned pair that holds entry s (rows are dword-aligned: the launcher requires an even number of
+      // entries); float32 - entry s and the one after it, or the one before it for the row's last entry, so that no
+      // load reaches past the row. The store picks entry s for both groups.
+      unsigned at, pick = 0;
+      if (SB == 2) {
+        at = gs ? (2u * s) & ~3u : 4u * s;
+        pick = s & 1u;
+      } else {
+        pick = gs && s + 1 == (unsigned)nwin ? 1u : 0u;
+        at = gs ? 4u * (s - pick) : 8u * s;
+      }
+      const unsigned so = my_scales == 0xfffffff0u ? my_scales : my_scales + at;
+#if defined(BP_DEV_ABLATION) && BP_DEV_ABLATION == 38
+      if (SB == 2) sq[P][0] = so | 0x3c003c00u;
+#else
+      if (SB == 2) sq[P][0] = (unsigned)__builtin_amdgcn_raw_buffer_load_b32(srs, (int)so, 0, 0);
+#endif
+      else {
+        const u32x2 v = __builtin_bit_cast(u32x2, __builtin_amdgcn_raw_buffer_load_b64(srs, (int)so, 0, 0));
+        sq[P][0] = v.x;
+        sq[P][SB / 2 - 1] = v.y;
+      }
+      sodd[P] = (int)pick;
+    }
+    if (PART == 5 || PART == 6) xa[P][PART - 5] = buf_load16(xrs, 16u * threadIdx.x + 8192u * (PART - 5), (unsigned)F_FB * s);
+    if (PART == 7) xa[P][2] = buf_load16(xrs, tail_off, (unsigned)F_FB * s);
+    if (PART == 8) {
+      if (ls + 1 < nwin) ++ls;
+      else if (lterm + 1 < a.n_terms) {
+        ++lterm;
+        ls = 0;
+        set_term(lterm);
+      }
+    }
+  };
+  auto request_all = [&](auto p_c) {
+    request(p_c, FC<5>{});
+    request(p_c, FC<6>{});
+    request(p_c, FC<7>{});
+    request(p_c, FC<4>{});
+    static_for<F_RT>([&](auto r_c) { request(p_c, r_c); });
+    request(p_c, FC<8>{});
+  };
+  auto staged_store = [&](int buf, const u32x4 (&v)[3]) {
+    const unsigned ab = (unsigned)(buf * F_FB);
+    *(lds_u32x4*)(ab + 16u * threadIdx.x) = v[0];
+    *(lds_u32x4*)(ab + 8192u + 16u * threadIdx.x) = v[1];
+    if (threadIdx.x < F_TAIL / 16) *(lds_u32x4*)(ab + (unsigned)F_OPS + 16u * threadIdx.x) = v[2];
+  };
+  auto scale_store = [&](int slot, const unsigned (&v)[SB / 2], int odd) {
+#pragma unroll
+    for (int i = 0; i < SB / 2; ++i) {
+      unsigned d = v[i];
+      if (gs) d = SB == 2 ? ((v[0] >> (16 * odd)) & 0xffffu) * 0x10001u : v[odd ? SB / 2 - 1 : 0];
+      *(lds_u32*)(unsigned)(F_SC + (slot * F_ROWS + (int)threadIdx.x) * (2 * SB) + 4 * i) = d;
+    }
+  };
+
+#if defined(BP_DEV_ABLATION) && (BP_DEV_ABLATION == 31 || BP_DEV_ABLATION == 35)
+  unsigned st[64];
+  int ns = 0;
+  bool son = BP_DEV_ABLATION == 31;
+#define BP_STAMP() do { if (son && ns < 64) st[ns++] = (unsigned)clock64(); } while (0)
+#if BP_DEV_ABLATION == 35
+#define BP_STAMP2() do { __builtin_amdgcn_sched_barrier(0); BP_STAMP(); __builtin_amdgcn_sched_barrier(0); } while (0)
+#else
+#define BP_STAMP2() do {} while (0)
+#endif
+#else
+#define BP_STAMP() do {} while (0)
+#define BP_STAMP2() do {} while (0)
+#endif
+  auto all_windows = [&](auto tt_c) {
+    constexpr int TT = decltype(tt_c)::value;  // token tiles processed
+    f32x4 total[F_RT][TT];
+#pragma unroll
+    for (int r = 0; r < F_RT; ++r)
+#pragma unroll
+      for (int t = 0; t < TT; ++t) total[r][t] = f32x4{0.f, 0.f, 0.f, 0.f};
+
+#if defined(BP_DEV_ABLATION) && BP_DEV_ABLATION == 36
+    if (wave < 4) __builtin_amdgcn_s_setprio(2);
+#endif
+#if defined(BP_DEV_ABLATION) && BP_DEV_ABLATION == 37
+    if (wave >= 4) __builtin_amdgcn_s_setprio(2);
+#endif
+    // ---- prologue: windows 0 and 1 requested, window 0's operands and scales into LDS
+    request_all(FC<0>{});
+    request_all(FC<1>{});
+    staged_store(0, xa[0]);
+    scale_store(0, sq[0], sodd[0]);
+    __syncthreads();
+
+    if constexpr (TT == 2) {
+      // ---- 32 tokens: the matrix instructions of a wave run on without a gap. A group's 16 go in four batches of
+      // four row tiles - (token tile 0, piece 0), (1, 0), (0, 1), (1, 1) - so that an operand A is free for the next
+      // group's (read from LDS behind its batch) as soon as its batch has issued, an instruction of the second pieces
+      // finds its accumulator finished, and the scaling of token tile 0's sums runs beside batch 3, that of token tile
+      // 1's beside the next group's batch 0. The workgroup's one barrier per window sits between the two groups: before
+      // it a wave writes the next window's staged activations and scales to LDS, after it it reads them.
+      i32x8 A[2][2];
+      f32x4 base[2];
+      int sa[2][2];                    // [window parity][token tile]
+      unsigned sraw[2][F_RT][SB / 2];  // [window parity]: the window's two scales of the lane's row of each row tile, as stored
+      float scp[F_RT];                 // the scales of the group whose token tile 1 is still to be summed
+      f32x4 C[F_RT][2];
+      i32x8 B[F_RT];
+#pragma unroll
+      for (int r = 0; r < F_RT; ++r) {
+        scp[r] = 0.f;
+        C[r][0] = C[r][1] = f32x4{0.f, 0.f, 0.f, 0.f};
+      }
+      auto read_a = [&](unsigned ab, int g, auto t_c, auto p_c) {
+        constexpr int t = decltype(t_c)::value, pp = decltype(p_c)::value;
+        const unsigned at = ab + (unsigned)(((g * 2 + t) * 2 + pp) * 2048) + alane;
+        const u32x4 lo = *(const lds_u32x4*)at, hi4 = *(const lds_u32x4*)(at + 256);
+        A[t][pp] = i32x8{(int)lo.x, (int)lo.y, (int)lo.z, (int)lo.w, (int)hi4.x, (int)hi4.y, (int)hi4.z, (int)hi4.w};
+      };
+      auto read_base = [&](unsigned ab, int g) {
+#pragma unroll
+        for (int t = 0; t < 2; ++t) base[t] = __builtin_bit_cast(f32x4, *(const lds_u32x4*)(ab + F_OPS + F_SCL + (unsigned)((g * 32 + 16 * t + 4 * kb) * 4)));
+      };
+      auto read_window_scales = [&](auto h_c) {  // block scales and row scales of the window of parity H
+        constexpr int H = decltype(h_c)::value;
+        const unsigned ab = (unsigned)(H * F_FB);
+        const unsigned sb = (unsigned)(F_SC + (H * F_ROWS + wave * (16 * F_RT) + r16) * (2 * SB));
+#pragma unroll
+        for (int t = 0; t < 2; ++t) sa[H][t] = (int)*(const lds_u32*)(ab + F_OPS + (unsigned)((t * 64 + lane) * 4));
+#pragma unroll
+        for (int r = 0; r < F_RT; ++r) {
+          if (SB == 2) sraw[H][r][0] = *(const lds_u32*)(sb + (unsigned)(16 * r * 2 * SB));
+          else {
+            const u32x2 v = *(const lds_u32x2*)(sb + (unsigned)(16 * r * 2 * SB));
+            sraw[H][r][0] = v.x;
+            sraw[H][r][SB / 2 - 1] = v.y;
+          }
+        }
+      };
+      read_a(0u, 0, FC<0>{}, FC<0>{});
+      read_a(0u, 0, FC<1>{}, FC<0>{});
+      read_a(0u, 0, FC<0>{}, FC<1>{});
+      read_a(0u, 0, FC<1>{}, FC<1>{});
+      read_base(0u, 0);
+      read_window_scales(FC<0>{});
+
+      unsigned D[F_RT][2][2];  // the window's bytes regrouped: D[r][g] = the lane's 8 bytes (32 weights) of group g
+      auto pgroup = [&](auto h_c, auto g_c) {
+        constexpr int H = decltype(h_c)::value, g = decltype(g_c)::value;
+        const unsigned nb = (unsigned)((g == 0 ? H : H ^ 1) * F_FB);  // where the next group's operands are
+        constexpr int ng = g ^ 1;
+        auto mfma = [&](const i32x8& av, const i32x8& bv, const f32x4& cv, int sav) {
+          return __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(av, bv, cv, 0 /* A: E4M3 */, 4 /* B: E2M1 */, g, sav, 0, ones);
+        };
+        auto row_scale = [&](int r) {
+          if (SDT == BP_F32) return __uint_as_float(sraw[H][r][g == 0 ? 0 : SB / 2 - 1]);
+          const unsigned rawsc = g == 0 ? sraw[H][r][0] & 0xffffu : sraw[H][r][0] >> 16;
+          return SDT == BP_F16 ? f16_bits_to_f32((uint16_t)rawsc) : __uint_as_float(rawsc << 16);
+        };
+        // batch 0: (token tile 0, piece 0). A row tile's operand B is made just before its first use; the previous
+        // group's token tile 1 is summed here.
+        static_for<F_RT>([&](auto r_c) {
+          constexpr int r = decltype(r_c)::value;
+          const unsigned d0 = D[r][g][0], d1 = D[r][g][1];
+          B[r] = i32x8{(int)((d0 << 1) & m66), (int)((d0 >> 1) & m66), (int)((d1 << 1) & m66), (int)((d1 >> 1) & m66), 0, 0, 0, 0};
+#pragma unroll
+          for (int i = 0; i < 4; ++i) total[r][1][i] += scp[r] * C[r][1][i];
+          asm volatile("" : "+v"(total[r][1]));
+          C[r][0] = mfma(A[0][0], B[r], base[0], sa[H][0]);
+          asm volatile("" : "+v"(C[r][0]) : : "memory");
+          __builtin_amdgcn_sched_barrier(0);
+        });
+        read_a(nb, ng, FC<0>{}, FC<0>{});
+        if (g == 0) staged_store(H ^ 1, xa[H ^ 1]);  // (the other buffer: last read before the previous barrier)
+        request(h_c, FC<g == 0 ? 5 : 0>{});
+        __builtin_amdgcn_sched_barrier(0);
+        BP_STAMP2();
+        // batch 1: (1, 0)
+        static_for<F_RT>([&](auto r_c) {
+          constexpr int r = decltype(r_c)::value;
+          C[r][1] = mfma(A[1][0], B[r], base[1], sa[H][1]);
+          asm volatile("" : "+v"(C[r][1]) : : "memory");
+          __builtin_amdgcn_sched_barrier(0);
+        });
+        read_a(nb, ng, FC<1>{}, FC<0>{});
+        if (g == 0) scale_store(H ^ 1, sq[H ^ 1], sodd[H ^ 1]);
+        request(h_c, FC<g == 0 ? 6 : 1>{});
+        __builtin_amdgcn_sched_barrier(0);
+        BP_STAMP2();
+        // batch 2: (0, 1)
+        static_for<F_RT>([&](auto r_c) {
+          constexpr int r = decltype(r_c)::value;
+          C[r][0] = mfma(A[0][1], B[r], C[r][0], sa[H][0]);
+          asm volatile("" : "+v"(C[r][0]) : : "memory");
+          __builtin_amdgcn_sched_barrier(0);
+        });
+        read_a(nb, ng, FC<0>{}, FC<1>{});
+        read_base(nb, ng);  // (the accumulators' starting values were last read by batch 1)
+        if (g == 1) read_window_scales(FC<H ^ 1>{});
+        request(h_c, FC<g == 0 ? 7 : 2>{});
+        __builtin_amdgcn_sched_barrier(0);
+        BP_STAMP2();
+        // batch 3: (1, 1), and token tile 0's sums under the rows' scales
+        static_for<F_RT>([&](auto r_c) {
+          constexpr int r = decltype(r_c)::value;
+          C[r][1] = mfma(A[1][1], B[r], C[r][1], sa[H][1]);
+          asm volatile("" : "+v"(C[r][1]) : : "memory");
+          const float sc = row_scale(r);
+#pragma unroll
+          for (int i = 0; i < 4; ++i) total[r][0][i] += sc * C[r][0][i];
+          asm volatile("" : "+v"(total[r][0]));
+          scp[r] = sc;
+          __builtin_amdgcn_sched_barrier(0);
+        });
+        read_a(nb, ng, FC<1>{}, FC<1>{});
+        request(h_c, FC<g == 0 ? 4 : 3>{});
+        if (g == 1) request(h_c, FC<8>{});
+        __builtin_amdgcn_sched_barrier(0);
+      };
+      auto pwindow = [&](auto h_c) {
+        constexpr int H = decltype(h_c)::value;
+#pragma unroll
+        for (int r = 0; r < F_RT; ++r) {
+          const auto s0 = __builtin_amdgcn_permlane32_swap(W[H][r].x, W[H][r].z, false, false);
+          const auto s1 = __builtin_amdgcn_permlane32_swap(W[H][r].y, W[H][r].w, false, false);
+          D[r][0][0] = moved(s0[0]);
+          D[r][0][1] = moved(s1[0]);
+          D[r][1][0] = moved(s0[1]);
+          D[r][1][1] = moved(s1[1]);
+        }
+        __builtin_amdgcn_sched_barrier(0);
+        BP_STAMP();
+        pgroup(h_c, FC<0>{});
+        BP_STAMP();
+        __syncthreads();
+        BP_STAMP();
+        pgroup(h_c, FC<1>{});
+        BP_STAMP();
+      };
+      int w = 0;
+      for (; w + 1 < NW; w += 2) {
+#if defined(BP_DEV_ABLATION) && BP_DEV_ABLATION == 35
+        son = w == 6 || w == 8;
+#endif
+        pwindow(FC<0>{});
+        pwindow(FC<1>{});
+      }
+      if (w < NW) pwindow(FC<0>{});  // uniform
+      // the last group's token tile 1
+#pragma unroll
+      for (int r = 0; r < F_RT; ++r)
+#pragma unroll
+        for (int i = 0; i < 4; ++i) total[r][1][i] += scp[r] * C[r][1][i];
+    } else {
+      // one window of parity H
+      auto window = [&](auto h_c) {
+        constexpr int H = decltype(h_c)::value;
+        const unsigned ab = (unsigned)(H * F_FB);
+        const unsigned sb = (unsigned)(F_SC + (H * F_ROWS + wave * (16 * F_RT) + r16) * (2 * SB));
+        // this window's bytes regrouped: D[r][g] = the lane's 8 bytes (32 weights) of group g
+        unsigned D[F_RT][2][2];
+  #pragma unroll
+        for (int r = 0; r < F_RT; ++r) {
+          const auto s0 = __builtin_amdgcn_permlane32_swap(W[H][r].x, W[H][r].z, false, false);
+          const auto s1 = __builtin_amdgcn_permlane32_swap(W[H][r].y, W[H][r].w, false, false);
+          // (copies into other registers: the swap works in place, and the registers of W[H] are wanted back at once for
+          // the requests below - otherwise the loop ends with moves that wait for the loads just issued)
+          D[r][0][0] = moved(s0[0]);
+          D[r][0][1] = moved(s1[0]);
+          D[r][1][0] = moved(s0[1]);
+          D[r][1][1] = moved(s1[1]);
+        }
+        // What the previous window of this parity left in registers has been used (its activations and scales went to LDS
+        // during the window before this one): the window two ahead is requested into them, one load after each row
+        // tile's matrix instructions.
+        BP_STAMP();
+        int sa[TT];
+  #pragma unroll
+        for (int t = 0; t < TT; ++t) sa[t] = (int)*(const lds_u32*)(ab + F_OPS + (unsigned)((t * 64 + lane) * 4));
+        unsigned sraw[F_RT][SB / 2];  // the window's two scales of the lane's row of each row tile, as stored
+  #pragma unroll
+        for (int r = 0; r < F_RT; ++r) {
+          if (SB == 2) sraw[r][0] = *(const lds_u32*)(sb + (unsigned)(16 * r * 2 * SB));
+          else {
+            const u32x2 v = *(const lds_u32x2*)(sb + (unsigned)(16 * r * 2 * SB));
+            sraw[r][0] = v.x;
+            sraw[r][SB / 2 - 1] = v.y;
+          }
+        }
+
+        // One group of the window: the group's operands, its matrix instructions, its sums under the rows' scales.
+        auto group = [&](auto g_c) {
+          constexpr int g = decltype(g_c)::value;
+          auto& tot = total;
+          f32x4 base[TT];
+          i32x8 A[TT][2];
+  #pragma unroll
+          for (int t = 0; t < TT; ++t) {
+            base[t] = __builtin_bit_cast(f32x4, *(const lds_u32x4*)(ab + F_OPS + F_SCL + (unsigned)((g * 32 + 16 * t + 4 * kb) * 4)));
+  #pragma unroll
+            for (int p = 0; p < 2; ++p) {
+              const unsigned at = ab + (unsigned)(((g * 2 + t) * 2 + p) * 2048) + alane;
+              const u32x4 lo = *(const lds_u32x4*)at, hi4 = *(const lds_u32x4*)(at + 256);
+              A[t][p] = i32x8{(int)lo.x, (int)lo.y, (int)lo.z, (int)lo.w, (int)hi4.x, (int)hi4.y, (int)hi4.z, (int)hi4.w};
+            }
+          }
+          __builtin_amdgcn_sched_barrier(0);
+  #if defined(BP_DEV_ABLATION) && BP_DEV_ABLATION == 35
+          asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+          BP_STAMP2();
+  #endif
+          f32x4 C[F_RT][TT];
+          // Matrix instructions two chains at a time (the two token tiles of a row tile, or two row tiles when there is
+          // one token tile): the second piece's instruction reads the first one's result, with the other chain's
+          // instruction between them.
+          auto operand_b = [&](int r) {
+            const unsigned d0 = D[r][g][0], d1 = D[r][g][1];
+            return i32x8{(int)((d0 << 1) & m66), (int)((d0 >> 1) & m66), (int)((d1 << 1) & m66), (int)((d1 >> 1) & m66), 0, 0, 0, 0};
+          };
+          static_for<F_RT * TT / 2>([&](auto u_c) {
+            constexpr int u = decltype(u_c)::value;
+            constexpr int ra = TT == 2 ? u : 2 * u, rb = TT == 2 ? u : 2 * u + 1, ta = 0, tb = TT == 2 ? 1 : 0;
+            const i32x8 Ba = operand_b(ra), Bb = TT == 2 ? Ba : operand_b(rb);
+            C[ra][ta] = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(A[ta][0], Ba, base[ta], 0 /* A: E4M3 */, 4 /* B: E2M1 */, g, sa[ta], 0, ones);
+            C[rb][tb] = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(A[tb][0], Bb, base[tb], 0, 4, g, sa[tb], 0, ones);
+            C[ra][ta] = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(A[ta][1], Ba, C[ra][ta], 0, 4, g, sa[ta], 0, ones);
+            C[rb][tb] = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(A[tb][1], Bb, C[rb][tb], 0, 4, g, sa[tb], 0, ones);
+            // (the products named here, so that the matrix instructions stay above the loads)
+            asm volatile("" : "+v"(C[ra][ta]), "+v"(C[rb][tb]) : : "memory");
+            __builtin_amdgcn_sched_barrier(0);
+            if (g == 0) {
+              request(h_c, FC<u == 0 ? 5 : 7>{});
+              request(h_c, FC<u == 0 ? 6 : 4>{});
+            } else {
+              request(h_c, FC<2 * u>{});
+              request(h_c, FC<2 * u + 1>{});
+              if (u == 1) request(h_c, FC<8>{});
+            }
+            __builtin_amdgcn_sched_barrier(0);
+          });
+          BP_STAMP2();
+  #pragma unroll
+          for (int r = 0; r < F_RT; ++r) {
+            float sc;
+            if (SDT == BP_F32) sc = __uint_as_float(sraw[r][g]);
+            else {
+              const unsigned rawsc = g == 0 ? sraw[r][0] & 0xffffu : sraw[r][0] >> 16;
+              sc = SDT == BP_F16 ? f16_bits_to_f32((uint16_t)rawsc) : __uint_as_float(rawsc << 16);
+            }
+  #pragma unroll
+            for (int t = 0; t < TT; ++t) {
+  #pragma unroll
+              for (int i = 0; i < 4; ++i) tot[r][t][i] += sc * C[r][t][i];
+              asm volatile("" : "+v"(tot[r][t]));  // (keeps the matrix instructions from sinking below what follows)
+            }
+          }
+        };
+        __builtin_amdgcn_sched_barrier(0);
+        group(FC<0>{});
+        BP_STAMP();
+        __builtin_amdgcn_sched_barrier(0);
+        staged_store(H ^ 1, xa[H ^ 1]);  // the next window's operands (the other buffer: last read before the previous barrier)
+        BP_STAMP();
+        __builtin_amdgcn_sched_barrier(0);
+        group(FC<1>{});
+        BP_STAMP();
+        __builtin_amdgcn_sched_barrier(0);
+        scale_store(H ^ 1, sq[H ^ 1], sodd[H ^ 1]);
+        BP_STAMP();
+        __builtin_amdgcn_sched_barrier(0);
+        __syncthreads();
+      };
+
+      int w = 0;
+      for (; w + 1 < NW; w += 2) {
+  #if defined(BP_DEV_ABLATION) && BP_DEV_ABLATION == 35
+        son = w == 6 || w == 8;
+  #endif
+        window(FC<0>{});
+        window(FC<1>{});
+      }
+      if (w < NW) window(FC<0>{});  // uniform
+    }
+
+#if defined(BP_DEV_ABLATION) && (BP_DEV_ABLATION == 31 || BP_DEV_ABLATION == 35)
+    if (blockIdx.x == 8 * 4 * 20 && blockIdx.z == 0) {  // expert 160, row block 0: every wave writes its stamps over its own outputs
+      if (lane == 0)
+        for (int i = 0; i < ns; ++i) a.out[(tok0 + i / 32) * a.N + n_wave + i % 32] = (float)(st[i] - st[0]);
+      return;
+    }
+#endif
+    // ---- epilogue: lane holds tokens 4 kb + i of each token tile, output row n_wave + 16 r + r16
+#pragma unroll
+    for (int t = 0; t < TT; ++t) {
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        const int tk = 16 * t + 4 * kb + i;
+        if (tk < ntok) {
+          const int64_t tok = tok0 + tk;
+#pragma unroll
+          for (int r = 0; r < F_RT; ++r) {
+            const int64_t row = n_wave + 16 * r;
+            if (row < a.N) {
+              float* o = a.out + tok * a.N + row + r16;
+              *o = (a.overwrite ? 0.f : *o) + total[r][t][i];
+            }
+          }
+        }
+      }
+    }
+  };
+  if (two) all_windows(FC<2>{});
+  else all_windows(FC<1>{});
+}
+
+template <int SDT>
+int launch_gemm_tq2f_k(const GemmArgs& a, hipStream_t s) {
+  if (const int rc = raise_lds_limit<k_gemm_tq2f<SDT>>(f_lds_bytes(SDT == BP_F32 ? 4 : 2))) return rc;
+  const int64_t row_blocks = (a.N + F_ROWS - 1) / F_ROWS;
+  const int64_t slots = a.tiles ? a.tile_cap : a.E;
+  const unsigned z = a.tiles ? 1u : (unsigned)((a.max_rows + 31) / 32);
+  hipLaunchKernelGGL(k_stage_tq2f, dim3((unsigned)slots, (unsigned)(a.K / 256), z), dim3(F_THREADS), 0, s, a);
+  if (const int rc = check_launch("stage_tq2f")) return rc;
+  const dim3 grid((unsigned)(row_blocks * ((slots + 7) / 8 * 8)), 1, z);
+  note_kernel("gemm_tq2f_bf16");
+  hipLaunchKernelGGL((k_gemm_tq2f<SDT>), grid, dim3(F_THREADS), f_lds_bytes(SDT == BP_F32 ? 4 : 2), s, a);
+  return check_launch("gemm_tq2f_bf16");
+}
+
+}  // namespace
+
+// Bytes of workspace the staged path takes for a call with T rows in all, K columns and E experts (0: no staged path
+// for these arguments): room for every token tile's windows, tiles placed so that they cannot overlap.
+size_t gemm_tq2f_workspace_bytes(int64_t T, int64_t K, int64_t E) {
+  if (T <= 0 || K % 256 != 0 || K < 1024 || E <= 0) return 0;
+  return (size_t)(T + 32 * E + 32) * (size_t)(K / 256) * (F_FB / 32);
+}
+
+// Preconditions (beyond mfma_supports: groups of 128 or 256, K % 256 == 0, K >= 1024, N % 16 == 0, 16-byte aligned x,
+// packed rows and scales): a workspace of gemm_tq2f_workspace_bytes in a.stage (16-byte aligned); an even number of
+// 16-bit scales per row; bf16 activations (int8 ones have a matrix instruction of their own at twice this one's rate
+// per activation: bp_gemm_tq2.hip); offsets into an expert's rows fit 32 bits; a launch whose token tiles mostly exist
+// (the conversion runs one workgroup per tile and window: a loose bound on the rows per expert would launch mostly
+// empty ones). BP_ERR_UNSUPPORTED (no message): the caller falls back to its other kernels.
+int launch_gemm_tq2f(const GemmArgs& a, hipStream_t s) {
+  if (a.x_dtype != BP_BF16 || !a.stage || ((uintptr_t)a.stage & 15) != 0) return BP_ERR_UNSUPPORTED;
+  if ((size_t)a.stage_bytes < gemm_tq2f_workspace_bytes(a.T, a.K, a.E) || gemm_tq2f_workspace_bytes(a.T, a.K, a.E) == 0) return BP_ERR_UNSUPPORTED;
+  if (a.K > ((int64_t)1 << 24) || a.N * a.Kp > ((int64_t)1 << 31) - 4096) return BP_ERR_UNSUPPORTED;
+  if (tuning().tq2g != 'f') {  // (development: BP_TUNE_TQ2G=fp4 runs this kernel wherever it can)
+    if (a.N < 2 * F_ROWS) return BP_ERR_UNSUPPORTED;  // (one or two row blocks: converting first saves nothing)
+    // One workgroup of 8 waves takes a CU: below three rounds of them (a round = 256 workgroups) the last, partly filled
+    // round costs more than the kernel gains over the one that runs two smaller workgroups per CU.
+    if ((a.T + 31) / 32 * ((a.N + F_ROWS - 1) / F_ROWS) < 768) return BP_ERR_UNSUPPORTED;
+  }
+  if (!a.tiles && ((a.max_rows + 31) / 32 > 65535 || (a.max_rows + 31) / 32 * 32 * a.E > 4 * a.T + 32 * a.E)) return BP_ERR_UNSUPPORTED;
+  if (a.K / 256 > 65535) return BP_ERR_UNSUPPORTED;
+  if (a.group == 256 && a.scale_dtype != BP_F32 && a.G % 2 != 0) return BP_ERR_UNSUPPORTED;  // (rows of scales not dword-aligned)
+  if (a.scale_dtype == BP_F16) return launch_gemm_tq2f_k<BP_F16>(a, s);
+  if (a.scale_dtype == BP_BF16) return launch_gemm_tq2f_k<BP_BF16>(a, s);
+  return launch_gemm_tq2f_k<BP_F32>(a, s);
+}
+
+}  // namespace bp

@@ -98,11 +98,13 @@ struct Plan {
   float* gu;      // f32 [T k, 2 I]
   void* h;        // bf16 [T k, I]
   float* y;       // f32 [T k, H]
+  unsigned char* stage;  // converted activations of the GEMM in flight (TQ2, bf16 activations, more than 64 tokens)
+  size_t stage_bytes;
   int64_t tile_cap;
   size_t bytes;
 };
 
-Plan plan(void* workspace, int64_t T, int64_t H, int64_t I, int64_t E, int64_t k, int act) {
+Plan plan(void* workspace, int64_t T, int64_t H, int64_t I, int64_t E, int64_t k, int act, int fmt) {
   Carve c = {(unsigned char*)workspace, 0};
   Plan p;
   const int64_t n = T * k;
@@ -119,6 +121,12 @@ Plan plan(void* workspace, int64_t T, int64_t H, int64_t I, int64_t E, int64_t k
   p.gu = (float*)c.take(4 * (size_t)n * 2 * I);
   p.h = c.take(2 * (size_t)n * I);
   p.y = (float*)c.take(4 * (size_t)n * H);
+  p.stage_bytes = 0;
+  if (fmt == BP_TQ2 && act == BP_BF16 && T > 64) {
+    const size_t a = gemm_tq2f_workspace_bytes(n, H, E), b = gemm_tq2f_workspace_bytes(n, I, E);
+    p.stage_bytes = a > b ? a : b;
+  }
+  p.stage = (unsigned char*)c.take(p.stage_bytes);
   p.bytes = c.used;
   return p;
 }
@@ -136,9 +144,9 @@ int zero(void* p, size_t bytes, hipStream_t s) {  // (a fill kernel, not a memse
 
 using namespace bp;
 
-extern "C" size_t bp_moe_layer_workspace_bytes(int64_t T, int64_t H, int64_t I, int64_t E, int64_t k, int act) {
+extern "C" size_t bp_moe_layer_workspace_bytes(int64_t T, int64_t H, int64_t I, int64_t E, int64_t k, int act, int fmt) {
   if (T < 0 || H <= 0 || I <= 0 || E <= 0 || k <= 0) return 0;
-  return plan(nullptr, T, H, I, E, k, act).bytes;
+  return plan(nullptr, T, H, I, E, k, act, fmt).bytes;
 }
 
 extern "C" int bp_moe_layer_bf16(void* out, const void* x, const int64_t* experts, const void* weights,
@@ -158,7 +166,7 @@ extern "C" int bp_moe_layer_bf16(void* out, const void* x, const int64_t* expert
   if (!out || !x || !experts || !weights || !gate_up_packed || !gate_up_scale || !down_packed || !down_scale) return fail(BP_ERR_ARG, "null pointer");
   for (int t = 0; t < n_terms; ++t)
     if (!gate_up_packed[t] || !gate_up_scale[t] || !down_packed[t] || !down_scale[t]) return fail(BP_ERR_ARG, "null packed or scale pointer in term %d", t);
-  const Plan p = plan(workspace, T, H, I, E, k, act);
+  const Plan p = plan(workspace, T, H, I, E, k, act, fmt);
   if (!workspace || workspace_bytes < p.bytes) return fail(BP_ERR_ARG, "the workspace must hold bp_moe_layer_workspace_bytes() = %zu bytes", p.bytes);
   if (((uintptr_t)workspace & 255) != 0) return fail(BP_ERR_ARG, "the workspace must be 256-byte aligned");
   hipStream_t s = (hipStream_t)stream;
@@ -187,6 +195,10 @@ extern "C" int bp_moe_layer_bf16(void* out, const void* x, const int64_t* expert
     a.scale_dtype = scale_dtype; a.n_terms = n_terms; a.fmt = fmt;
     a.T = n; a.N = N; a.K = K; a.Kp = (K + per - 1) / per; a.G = (K + group - 1) / group; a.group = group; a.E = E;
     a.max_rows = T < n ? T : n;  // an expert has at most one row per token
+    if (p.stage_bytes) {
+      a.stage = p.stage;
+      a.stage_bytes = (int64_t)p.stage_bytes;
+    }
     if (tiles) {
       a.tiles = p.tiles; a.tile_count = p.tile_count; a.tile_cap = p.tile_cap;
       if (kernel_policy() != 1 && gemm_tiles_supported(a)) {

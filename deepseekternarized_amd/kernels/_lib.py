@@ -22,6 +22,8 @@ SIGNATURES = {
     "bp_set_kernel_policy": (_i, [_i]),
     "bp_reload_tuning": (None, []),
     "bp_ternary_grouped_gemm": (_i, [_p, _p, _i, _p, _p, _p, _p, _p, _i, _i, _l, _l, _l, _l, _l, _l, _l, _i, _l, _p, _p]),
+    "bp_grouped_gemm_workspace_bytes": (C.c_size_t, [_i, _l, _l, _l, _l, _i]),
+    "bp_ternary_grouped_gemm_ws": (_i, [_p, _p, _i, _p, _p, _p, _p, _p, _i, _i, _l, _l, _l, _l, _l, _l, _l, _i, _l, _p, C.c_size_t, _p]),
     "bp_unpack_trits": (_i, [_p, _p, _l, _l, _i, _p]),
     "bp_pack_trits": (_i, [_p, _p, _l, _l, _i, _p]),
     "bp_expand_scales": (_i, [_p, _p, _i, _l, _p]),
@@ -35,7 +37,7 @@ SIGNATURES = {
     "bp_gather_rows": (_i, [_p, _p, _p, _l, _l, _l, _l, _p]),
     "bp_swiglu_bf16": (_i, [_p, _p, _p, _l, _l, _l, _p]),
     "bp_moe_combine_bf16": (_i, [_p, _p, _p, _p, _p, _l, _l, _l, _p]),
-    "bp_moe_layer_workspace_bytes": (C.c_size_t, [_l, _l, _l, _l, _l, _i]),
+    "bp_moe_layer_workspace_bytes": (C.c_size_t, [_l, _l, _l, _l, _l, _i, _i]),
     "bp_moe_layer_bf16": (_i, [_p, _p, _p, _p, _p, _p, _p, _p, _i, _i, _l, _l, _l, _l, _l, _l, _i, _i, _p, C.c_size_t, _p, _p]),
 }
 

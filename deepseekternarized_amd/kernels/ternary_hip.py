@@ -80,12 +80,24 @@ class _HipTernary:
         pk = (C.c_void_p * len(packed_l))(*[p.data_ptr() for p in packed_l])
         sc = (C.c_void_p * len(scale_l))(*[s.data_ptr() for s in scale_l])
         with torch.cuda.device(out.device):
-            rc = self.lib.bp_ternary_grouped_gemm(
-                out.data_ptr(), x.data_ptr(), _lib.dtype_code(x.dtype),
-                x_scale.data_ptr() if x_scale is not None else None, offsets.data_ptr(), host,
-                C.cast(pk, C.c_void_p), C.cast(sc, C.c_void_p), _lib.dtype_code(sdt), len(packed_l),
-                T, N, int(K), Kp, G, int(group), E, int(fmt), int(max_rows),
-                lut1.data_ptr() if lut1 is not None else None, _lib.stream_ptr(out.device))
+            # Prefill-sized calls get a workspace (the library allocates nothing itself): with one, the TQ2 kernels for bf16
+            # activations convert the activations once instead of once per block of output rows.
+            need = self.lib.bp_grouped_gemm_workspace_bytes(_lib.dtype_code(x.dtype), T, N, int(K), E, int(fmt)) if max_rows > 16 else 0
+            if need:
+                ws = torch.empty(need, dtype=torch.uint8, device=out.device)
+                rc = self.lib.bp_ternary_grouped_gemm_ws(
+                    out.data_ptr(), x.data_ptr(), _lib.dtype_code(x.dtype),
+                    x_scale.data_ptr() if x_scale is not None else None, offsets.data_ptr(), host,
+                    C.cast(pk, C.c_void_p), C.cast(sc, C.c_void_p), _lib.dtype_code(sdt), len(packed_l),
+                    T, N, int(K), Kp, G, int(group), E, int(fmt), int(max_rows), ws.data_ptr(), need,
+                    _lib.stream_ptr(out.device))
+            else:
+                rc = self.lib.bp_ternary_grouped_gemm(
+                    out.data_ptr(), x.data_ptr(), _lib.dtype_code(x.dtype),
+                    x_scale.data_ptr() if x_scale is not None else None, offsets.data_ptr(), host,
+                    C.cast(pk, C.c_void_p), C.cast(sc, C.c_void_p), _lib.dtype_code(sdt), len(packed_l),
+                    T, N, int(K), Kp, G, int(group), E, int(fmt), int(max_rows),
+                    lut1.data_ptr() if lut1 is not None else None, _lib.stream_ptr(out.device))
         _lib.check(rc)
 
     def last_kernel(self) -> str:

@@ -87,7 +87,7 @@ class TernaryMoE:
     def _workspace(self, tokens: int, device) -> torch.Tensor:
         e = _need_ext(self.down[0][0])
         need = int(e.lib.bp_moe_layer_workspace_bytes(tokens, self.hidden, self.inter, self.n_experts, self.top_k,
-                                                      _lib.BP_I8 if self.act == "int8" else _lib.BP_BF16))
+                                                      _lib.BP_I8 if self.act == "int8" else _lib.BP_BF16, _fmt_code(self.fmt)))
         ws = getattr(self, "_ws", None)
         if ws is None or ws.numel() < need or ws.device != torch.device(device):
             self._ws = ws = torch.empty(need, dtype=torch.uint8, device=device)   # (reused by later calls of up to this many tokens)

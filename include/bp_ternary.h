@@ -80,6 +80,21 @@ int bp_ternary_grouped_gemm(float* out, const void* x, int x_dtype, const float*
                             int64_t group, int64_t E, int fmt, int64_t max_rows, const int8_t* lut1,
                             void* stream);
 
+/* bp_ternary_grouped_gemm with a workspace of the caller's (the library allocates no device memory). It has no
+ * counterpart in the reference. With a workspace of at least bp_grouped_gemm_workspace_bytes(...) bytes (256-byte
+ * aligned device memory; contents undefined before and after the call) the TQ2 kernels for bf16 activations and more
+ * than 16 rows per expert convert the activations to matrix-instruction operands once, in a pass of their own,
+ * instead of once per block of output rows; results agree with bp_ternary_grouped_gemm's to float32 rounding of the
+ * sums. workspace = NULL, or a size of 0 from bp_grouped_gemm_workspace_bytes (no such kernel for these arguments):
+ * identical to bp_ternary_grouped_gemm. T is the row count of x (all experts). */
+size_t bp_grouped_gemm_workspace_bytes(int x_dtype, int64_t T, int64_t N, int64_t K, int64_t E, int fmt);
+int bp_ternary_grouped_gemm_ws(float* out, const void* x, int x_dtype, const float* x_scale,
+                               const int64_t* offsets, const int64_t* offsets_host,
+                               const uint8_t* const* packed, const void* const* w_scale, int scale_dtype,
+                               int n_terms, int64_t T, int64_t N, int64_t K, int64_t Kp, int64_t G,
+                               int64_t group, int64_t E, int fmt, int64_t max_rows, void* workspace,
+                               size_t workspace_bytes, void* stream);
+
 /* Selects the kernel family for bp_ternary_grouped_gemm on the calling thread:
  *   0 = automatic (tuned kernels where the shape allows, general kernel otherwise)
  *   1 = general kernel only (any K, group, format; int8 path bit-identical to
@@ -184,9 +199,9 @@ int bp_moe_combine_bf16(void* out, const float* y, const int64_t* inv, const voi
  *   gate_up_packed[t] device u8 [E, 2 I, Kp(H)], gate_up_scale[t] device [E, 2 I, G(H)]: rows [0, I) gate, [I, 2 I) up
  *   down_packed[t]    device u8 [E, H, Kp(I)],   down_scale[t]    device [E, H, G(I)];  n_terms stacked terms each
  *   act      BP_BF16 (activations as they are) or BP_I8 (per-row int8 of every linear's input, boilerplate/ternary/ops.py:20-25)
- *   workspace device memory, 256-byte aligned, at least bp_moe_layer_workspace_bytes(T, H, I, E, k, act) bytes
+ *   workspace device memory, 256-byte aligned, at least bp_moe_layer_workspace_bytes(T, H, I, E, k, act, fmt) bytes
  *   bad      device i32 flag set to 1 if an expert id is out of range (may be NULL) */
-size_t bp_moe_layer_workspace_bytes(int64_t T, int64_t H, int64_t I, int64_t E, int64_t k, int act);
+size_t bp_moe_layer_workspace_bytes(int64_t T, int64_t H, int64_t I, int64_t E, int64_t k, int act, int fmt);
 int bp_moe_layer_bf16(void* out, const void* x, const int64_t* experts, const void* weights,
                       const uint8_t* const* gate_up_packed, const void* const* gate_up_scale,
                       const uint8_t* const* down_packed, const void* const* down_scale, int scale_dtype,

@@ -77,6 +77,29 @@ def test_layer_call_over_the_tile_list_matches_composed_calls(fmt, terms, act):
     assert _rel(got2, moe.composed(x[:70], logits[:70])) <= 2e-3
 
 
+def test_layer_call_over_the_tile_list_with_converted_activations(tune):
+    """TQ2, bf16 activations, beyond 64 tokens: the workspace has room for the activations converted to fp8 pieces, and the
+    grouped GEMMs over them read the same device-side tile list (forced here: the shape is below that kernel's thresholds)."""
+    from deepseekternarized_amd import ext
+
+    H, I, E, k, T = 1024, 2048, 16, 2, 300
+    moe, _ = _layer("tq2", "bf16", H, I, E, k, terms=2, seed=3)
+    g = torch.Generator(device="cuda").manual_seed(5)
+    x = torch.randn(T, H, device="cuda", generator=g).to(torch.bfloat16)
+    logits = torch.randn(T, E, device="cuda", generator=g)
+    logits[:, 0] += 4.0
+    logits[:, 9] = -40.0
+    logits[:, 11] -= 2.5
+    tune("BP_TUNE_TQ2G", "fp4")
+    got = moe(x, logits).clone()
+    assert ext().last_kernel() == "gemm_tq2f_bf16", ext().last_kernel()
+    assert torch.equal(moe(x, logits), got)
+    tune("BP_TUNE_TQ2G", "bf16")
+    want = moe(x, logits)
+    assert ext().last_kernel().startswith("gemm_tq2_bf16"), ext().last_kernel()
+    assert torch.isfinite(got.float()).all() and _rel(got, want) <= 2e-3, _rel(got, want)
+
+
 @pytest.mark.parametrize("act", ["bf16", "int8"])
 @pytest.mark.parametrize("fmt", ["tq1", "tq2"])
 def test_layer_call_matches_the_reference_loop(fmt, act):
@@ -120,9 +143,11 @@ def test_layer_call_argument_checks():
     idx = torch.zeros(T, 2, dtype=torch.int64, device="cuda")
     idx[:, 1] = 1
     w = torch.ones(T, 2, dtype=torch.bfloat16, device="cuda")
-    need = lib.bp_moe_layer_workspace_bytes(T, 1024, 1024, 8, 2, _lib.BP_BF16)
+    need = lib.bp_moe_layer_workspace_bytes(T, 1024, 1024, 8, 2, _lib.BP_BF16, 2)
     assert need > 0 and need % 256 == 0
-    assert lib.bp_moe_layer_workspace_bytes(T, 1024, 1024, 8, 2, _lib.BP_I8) > need
+    assert lib.bp_moe_layer_workspace_bytes(T, 1024, 1024, 8, 2, _lib.BP_I8, 2) > need
+    # TQ2 with bf16 activations beyond 64 tokens: room for the converted activations of a grouped GEMM as well
+    assert lib.bp_moe_layer_workspace_bytes(128, 1024, 1024, 8, 2, _lib.BP_BF16, 2) > lib.bp_moe_layer_workspace_bytes(128, 1024, 1024, 8, 2, _lib.BP_BF16, 1)
     ws = torch.empty(need, dtype=torch.uint8, device="cuda")
     arr = lambda ts: (C.c_void_p * 1)(*[t.data_ptr() for t in ts])
     gp, gs = arr([moe.gate_up[0][0]]), arr([moe.gate_up[0][1]])

@@ -331,29 +331,115 @@ def test_tq2_bf16_scales_and_f32_scales(bp):
 
 
 # --------------------------------------------------------------------------- TQ2 grouped GEMM (token tiles of 32)
+@pytest.fixture(params=["fp4", "bf16"])
+def tq2_gemm_kernel(request, tune):
+    """More than 16 rows per expert, bf16 activations: the fp8 x fp4 grouped GEMM over activations converted into a
+    workspace (kernel name gemm_tq2f_bf16; BP_TUNE_TQ2G=fp4 runs it on shapes below its thresholds too) and the bf16
+    MFMA kernel (gemm_tq2_bf16*; BP_TUNE_TQ2G=bf16). int8 activations run gemm_tq2_i8* either way."""
+    tune("BP_TUNE_TQ2G", request.param)
+    return "gemm_tq2f_" if request.param == "fp4" else "gemm_tq2_"
+
+
 @pytest.mark.parametrize("act", ["bf16", "int8"])
 @pytest.mark.parametrize(
     "E,N,K,counts,terms",
     [
-        (3, 64, 1024, [17, 0, 40], 2),        # one activation tile for all of K, reused by the second term
-        (5, 272, 2048, [32, 33, 1, 64, 16], 1),  # N not a multiple of the 256 rows of a workgroup; full, 1-row and 16-row tiles
+        (3, 64, 1024, [17, 0, 40], 2),        # the smallest K the tuned kernels take (four windows); two terms
+        (5, 272, 2048, [32, 33, 1, 64, 16], 1),  # N not a multiple of a workgroup's rows; full, 1-row and 16-row tiles
         (11, 48, 3072, [20] * 11, 2),          # more experts than XCDs and not a multiple of 8; odd number of tiles
-        (2, 528, 7168, [48, 31], 1),           # config-3 K, three row tiles
+        (2, 528, 7168, [48, 31], 1),           # config-3 K; a second row block with 16 of its rows
+        (3, 1040, 1280, [100, 9, 31], 1),      # an odd number of windows; three row blocks of the fp8 x fp4 kernel; four token tiles
     ],
 )
-def test_tq2_gemm_tiles(bp, act, E, N, K, counts, terms):
+def test_tq2_gemm_tiles(bp, act, E, N, K, counts, terms, tq2_gemm_kernel):
     got, want, kern = _run(bp, "tq2", E, N, K, counts, act, terms=terms, seed=K + N)
-    assert kern.startswith("gemm_tq2"), kern
+    assert kern.startswith(tq2_gemm_kernel if act == "bf16" else "gemm_tq2_i8"), kern
     _check(got, want)
 
 
-def test_tq2_gemm_scales_from_global_memory_and_other_scale_dtypes(bp):
-    """K = 10240: 256 rows x 80 groups of scales do not fit beside two activation tiles; bf16 scales; float32 scales."""
+def test_tq2_gemm_fp8_pieces_keep_small_activations(bp, tune):
+    """Activations spread over five decades with 1000 x outliers: two E4M3 pieces under a scale per 32 activations."""
+    tune("BP_TUNE_TQ2G", "fp4")
+    rng = np.random.default_rng(77)
+    E, N, K, counts = 2, 64, 2048, [33, 20]
+    packed, scales = synth_weights(78, E, N, K, GROUP, "tq2")
+    x = rng.standard_normal((sum(counts), K)).astype(np.float32) * np.exp(rng.uniform(-6, 6, (sum(counts), K))).astype(np.float32)
+    x[rng.random(x.shape) < 0.01] *= 1000.0
+    x = orc.bf16_round(x)
+    offsets = np.concatenate([[0], np.cumsum(counts)])
+    got = bp.grouped_ternary_gemm(dev(x).to(torch.bfloat16), None, dev(offsets), dev(packed[0]), dev(scales[0]), K, GROUP, "tq2", max_rows=max(counts))
+    assert bp.ext().last_kernel().startswith("gemm_tq2f_"), bp.ext().last_kernel()
+    want = np.concatenate([c_gemm(x[a:b], None, packed[0][e], scales[0][e].astype(np.float32), K, GROUP, "tq2")
+                           for e, (a, b) in enumerate(zip(offsets[:-1], offsets[1:]))])
+    rel = np.linalg.norm(got.cpu().numpy() - want) / np.linalg.norm(want)
+    assert rel <= 1e-4, rel
+
+
+@pytest.mark.parametrize("act", ["bf16", "int8"])
+def test_tq2_gemm_float32_scales(bp, act, tq2_gemm_kernel):
+    """What the reference's wrappers hand the kernel (`w_scale.float()`, boilerplate/kernels/ternary_cuda.py:95-97);
+    also with one scale per 256 weights and an odd number of them per row."""
+    got, want, kern = _run(bp, "tq2", 3, 80, 2304, [21, 0, 50], act, terms=2, seed=31, scale_dtype="f32")
+    assert kern.startswith(tq2_gemm_kernel if act == "bf16" else "gemm_tq2_i8"), kern
+    _check(got, want)
+    got, want, kern = _run(bp, "tq2", 2, 528, 2304, [19, 33], act, terms=2, seed=32, scale_dtype="f32", group=256)
+    assert kern.startswith(tq2_gemm_kernel if act == "bf16" else "gemm_tq2_i8"), kern
+    _check(got, want)
+
+
+def test_tq2_gemm_over_converted_activations_is_the_default_for_large_prefill(bp, tune):
+    """Without a development switch: 8 experts x 800 rows x N = 2048 is above the thresholds; the result agrees with the bf16
+    MFMA kernel's (which the tests above pin against the CPU restatement) to float32 summation order and the 2^-17 the
+    fp8 pieces drop. The mirrored call brings the workspace; the plain C entry point (no workspace) keeps the bf16 kernel."""
+    import ctypes as C
+
+    from deepseekternarized_amd.kernels import _lib
+
+    E, N, K, rows = 8, 2048, 1024, 800
+    packed, scales = synth_weights(91, E, N, K, GROUP, "tq2", terms=2)
+    pk, sc = [dev(p) for p in packed], [dev(s) for s in scales]
+    g = torch.Generator(device="cuda").manual_seed(92)
+    x = torch.randn(E * rows, K, device="cuda", generator=g).to(torch.bfloat16)
+    offsets = torch.arange(0, E * rows + 1, rows, device="cuda", dtype=torch.int64)
+    offsets[3] -= 13  # ragged tiles on both sides
+    got = bp.grouped_ternary_gemm(x, None, offsets, pk, sc, K, GROUP, "tq2", max_rows=rows + 13)
+    assert bp.ext().last_kernel() == "gemm_tq2f_bf16", bp.ext().last_kernel()
+    lib = bp.ext().lib
+    assert lib.bp_grouped_gemm_workspace_bytes(_lib.BP_BF16, E * rows, N, K, E, 2) > 0
+    assert lib.bp_grouped_gemm_workspace_bytes(_lib.BP_I8, E * rows, N, K, E, 2) == 0
+    assert lib.bp_grouped_gemm_workspace_bytes(_lib.BP_BF16, E * rows, N, K, E, 1) == 0
+    tune("BP_TUNE_TQ2G", "bf16")
+    want = bp.grouped_ternary_gemm(x, None, offsets, pk, sc, K, GROUP, "tq2", max_rows=rows + 13)
+    assert bp.ext().last_kernel().startswith("gemm_tq2_bf16"), bp.ext().last_kernel()
+    rel = ((got - want).norm() / want.norm()).item()
+    assert rel <= 2e-5, rel
+    tune("BP_TUNE_TQ2G", None)
+    out = torch.zeros_like(got)
+    pa = (C.c_void_p * 2)(*[p.data_ptr() for p in pk])
+    sa = (C.c_void_p * 2)(*[s.data_ptr() for s in sc])
+    args = (out.data_ptr(), x.data_ptr(), _lib.BP_BF16, None, offsets.data_ptr(), None, C.cast(pa, C.c_void_p), C.cast(sa, C.c_void_p),
+            _lib.BP_F16, 2, E * rows, N, K, K // 4, K // GROUP, GROUP, E, 2, rows + 13)
+    rc = lib.bp_ternary_grouped_gemm(*args, None, None)
+    torch.cuda.synchronize()
+    assert rc == 0 and lib.bp_last_kernel().decode().startswith("gemm_tq2_bf16")
+    assert torch.equal(out, want)
+    # a workspace that is too small: the same kernel as without one; a misaligned one: an error
+    ws = torch.empty(4096, dtype=torch.uint8, device="cuda")
+    out.zero_()
+    rc = lib.bp_ternary_grouped_gemm_ws(*args, ws.data_ptr(), 4096, None)
+    torch.cuda.synchronize()
+    assert rc == 0 and lib.bp_last_kernel().decode().startswith("gemm_tq2_bf16") and torch.equal(out, want)
+    rc = lib.bp_ternary_grouped_gemm_ws(*args, ws.data_ptr() + 8, 4096, None)
+    assert rc != 0 and b"aligned" in lib.bp_last_error()
+
+
+def test_tq2_gemm_scales_from_global_memory_and_other_scale_dtypes(bp, tq2_gemm_kernel):
+    """K = 10240: 256 rows x 80 groups of scales do not fit beside the bf16 kernel's two activation tiles; bf16 scales; float32 scales."""
     got, want, kern = _run(bp, "tq2", 2, 64, 10240, [33, 18], "bf16", seed=21)
-    assert kern == "gemm_tq2_bf16_gs", kern
+    assert kern == ("gemm_tq2_bf16_gs" if tq2_gemm_kernel == "gemm_tq2_" else "gemm_tq2f_bf16"), kern
     _check(got, want)
     got, want, kern = _run(bp, "tq2", 2, 64, 2048, [18, 40], "bf16", seed=22, scale_dtype=np.float32)  # bf16 scales
-    assert kern.startswith("gemm_tq2"), kern
+    assert kern.startswith(tq2_gemm_kernel), kern
     _check(got, want)
     packed, scales = synth_weights(23, 1, 80, 2048, GROUP, "tq2")
     x = orc.bf16_round(np.random.default_rng(23).standard_normal((137, 2048)).astype(np.float32))
@@ -456,14 +542,16 @@ def test_group_256(bp, act, fmt, K, counts, prefix):
 # --------------------------------------------------------------------------- activations that are not finite
 @pytest.mark.parametrize("fmt,counts,prefix", [
     ("tq1", [1, 1], "fp4_tq1_t1"), ("tq1", [4, 3], "fp4_tq1_m4"), ("tq1", [20, 12], "gemm_tq1"),
-    ("tq2", [1, 1], "mfma_tq2"), ("tq2", [9, 16], "mfma_tq2"), ("tq2", [40, 33], "gemm_tq2"),
+    ("tq2", [1, 1], "mfma_tq2"), ("tq2", [9, 16], "mfma_tq2"), ("tq2", [40, 33], "gemm_tq2_"), ("tq2", [40, 33], "gemm_tq2f_"),
 ])
-def test_non_finite_activations_never_give_finite_wrong_values(bp, fmt, counts, prefix):
+def test_non_finite_activations_never_give_finite_wrong_values(bp, tune, fmt, counts, prefix):
     """The reference's CPU kernel skips zero weights (boilerplate/kernels/csrc/boilerplate_cpu.cpp:70-77), so a NaN or an
     infinite activation makes exactly the outputs with a nonzero weight at that k non-finite. The tuned kernels multiply
     zeros too (0 x Inf = NaN) or scale whole blocks: they may make more outputs of that token non-finite, but every
     output the reference makes non-finite must be non-finite here, and tokens without such an activation are untouched."""
     E, N, K = 2, 64, 2048
+    if prefix == "gemm_tq2f_":
+        tune("BP_TUNE_TQ2G", "fp4")
     rng = np.random.default_rng(5)
     packed, scales = synth_weights(17, E, N, K, GROUP, fmt)
     trits = np.stack([orc.unpack(packed[0][e], fmt, K) for e in range(E)])
