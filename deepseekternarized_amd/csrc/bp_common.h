@@ -62,6 +62,31 @@ __device__ __forceinline__ TileRef tile_ref(const GemmArgs& a, int64_t slot, uns
   return r;
 }
 
+// Which token tile and which block of output rows a workgroup of a 32-token-tile kernel takes, from its linear index.
+// Workgroups are dealt to the 8 XCDs round-robin by linear index and each XCD has its own L2. The row blocks of a token
+// tile read the same activations and the token tiles of an expert the same weights, so an XCD takes its experts one after
+// the other, an expert's token tiles one after the other and a tile's row blocks one after the other: the workgroups
+// that run on it at one time share what they stream through its L2. In tile-list mode an expert's tiles are neighbours
+// in the list, and an XCD takes the list in runs of TILE_RUN entries.
+constexpr int TILE_RUN = 4;
+__device__ __forceinline__ TileRef tile_of_workgroup(const GemmArgs& a, unsigned linear, int row_blocks, int& row_block) {
+  const unsigned xcd = linear & 7;
+  unsigned q = linear >> 3;
+  row_block = (int)(q % (unsigned)row_blocks);
+  q /= (unsigned)row_blocks;
+  if (a.tiles) return tile_ref(a, (int64_t)(q / TILE_RUN) * (8 * TILE_RUN) + xcd * TILE_RUN + q % TILE_RUN, 0);
+  const unsigned tiles_per_expert = (unsigned)((a.max_rows + 31) / 32);
+  return tile_ref(a, xcd + 8 * (int64_t)(q / tiles_per_expert), q % tiles_per_expert);
+}
+// Workgroups of such a launch (-1: more than a grid's x extent holds).
+inline int64_t tile_workgroups(const GemmArgs& a, int64_t row_blocks) {
+  const int64_t slots = a.tiles ? a.tile_cap : a.E, per_round = a.tiles ? 8 * TILE_RUN : 8;
+  const int64_t z = a.tiles ? 1 : (a.max_rows + 31) / 32;
+  const int64_t rounds = (slots + per_round - 1) / per_round;
+  if (z > 0x7fffffff / (row_blocks * per_round) || rounds > 0x7fffffff / (row_blocks * per_round * z)) return -1;
+  return row_blocks * per_round * rounds * z;
+}
+
 // Development overrides of the kernel selection (environment variables BP_TUNE_*), read once when the library is first
 // used; bp_reload_tuning() reads them again (the tests switch kernels that way). 0 / unset = automatic.
 struct Tuning {

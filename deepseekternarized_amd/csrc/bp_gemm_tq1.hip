@@ -68,11 +68,9 @@ __global__ __launch_bounds__(Q_THREADS, 2) void k_gemm_tq1(GemmArgs a) {
 
   const int wave = __builtin_amdgcn_readfirstlane((int)(threadIdx.x >> 6)), lane = threadIdx.x & 63;
   const int r16 = lane & 15, kb = lane >> 4;
-  // Workgroups are dealt to the 8 XCDs round-robin by linear index; the row blocks of one expert read the same
-  // activations, so they get linear indices 8 apart (same XCD, one L2).
   const int row_blocks = (int)((a.N + Q_ROWS - 1) / Q_ROWS);
-  const int wg_block = (int)((blockIdx.x >> 3) % (unsigned)row_blocks);
-  const TileRef tr = tile_ref(a, (blockIdx.x & 7) + 8 * (int64_t)((blockIdx.x >> 3) / (unsigned)row_blocks), blockIdx.z);
+  int wg_block;
+  const TileRef tr = tile_of_workgroup(a, blockIdx.x, row_blocks, wg_block);
   if (!tr.live) return;  // uniform for the workgroup
   const int64_t e = tr.e, tok0 = tr.tok0, o1 = tr.o1;
   const int ntok = (int)(o1 - tok0 < 32 ? o1 - tok0 : 32);
@@ -461,8 +459,9 @@ template <int ACT, int SDT>
 int launch_gemm_tq1_k(const GemmArgs& a, hipStream_t s, const char* name) {
   if (const int rc = raise_lds_limit<k_gemm_tq1<ACT, SDT>>(q_lds_bytes(SDT == BP_F32 ? 4 : 2))) return rc;
   const int64_t row_blocks = (a.N + Q_ROWS - 1) / Q_ROWS;
-  const int64_t slots = a.tiles ? a.tile_cap : a.E;
-  const dim3 grid((unsigned)(row_blocks * ((slots + 7) / 8 * 8)), 1, a.tiles ? 1u : (unsigned)((a.max_rows + 31) / 32));
+  const int64_t wgs = tile_workgroups(a, row_blocks);
+  if (wgs < 0) return BP_ERR_UNSUPPORTED;
+  const dim3 grid((unsigned)wgs, 1, 1);
   note_kernel(name);
   hipLaunchKernelGGL((k_gemm_tq1<ACT, SDT>), grid, dim3(Q_THREADS), q_lds_bytes(SDT == BP_F32 ? 4 : 2), s, a);
   return check_launch(name);

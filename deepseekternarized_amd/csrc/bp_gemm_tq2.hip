@@ -50,13 +50,9 @@ __global__ __launch_bounds__(GTHREADS, 2) void k_gemm_tq2(GemmArgs a) {
 
   const int wave = __builtin_amdgcn_readfirstlane((int)(threadIdx.x >> 6)), lane = threadIdx.x & 63;
   const int r16 = lane & 15, b = lane >> 4;
-  // Workgroups are dealt to the 8 XCDs round-robin by linear index; each XCD has its own L2. The row tiles of
-  // one expert read the same activations, so they get linear indices 8 apart (same XCD, consecutive in time):
-  // linear index L -> expert (L % 8) + 8 * (L / 8 / row_tiles), row tile (L / 8) % row_tiles (tile-list mode: list entry
-  // instead of expert).
   const int row_tiles = (int)((a.N + GROWS - 1) / GROWS);
-  const int wg_tile = (int)((blockIdx.x >> 3) % (unsigned)row_tiles);
-  const TileRef tr = tile_ref(a, (blockIdx.x & 7) + 8 * (int64_t)((blockIdx.x >> 3) / (unsigned)row_tiles), blockIdx.z);
+  int wg_tile;
+  const TileRef tr = tile_of_workgroup(a, blockIdx.x, row_tiles, wg_tile);
   if (!tr.live) return;  // uniform for the workgroup
   const int64_t e = tr.e, tok0 = tr.tok0, o1 = tr.o1;
   const int ntok = (int)(o1 - tok0 < 16 * GT ? o1 - tok0 : 16 * GT);
@@ -412,8 +408,10 @@ __global__ __launch_bounds__(GTHREADS, 2) void k_gemm_tq2(GemmArgs a) {
 template <int ACT, int SDT, int SL, int ABL = 0>
 int launch_gemm_k(const GemmArgs& a, hipStream_t s, size_t lds, const char* name) {
   if (const int rc = raise_lds_limit<k_gemm_tq2<ACT, SDT, SL, ABL>>(160 * 1024)) return rc;
-  const int64_t slots = a.tiles ? a.tile_cap : a.E;
-  const dim3 grid((unsigned)((a.N + GROWS - 1) / GROWS * ((slots + 7) / 8 * 8)), 1, a.tiles ? 1u : (unsigned)((a.max_rows + 16 * GT - 1) / (16 * GT)));
+  static_assert(16 * GT == 32, "tile_of_workgroup counts token tiles of 32");
+  const int64_t wgs = tile_workgroups(a, (a.N + GROWS - 1) / GROWS);
+  if (wgs < 0) return BP_ERR_UNSUPPORTED;
+  const dim3 grid((unsigned)wgs, 1, 1);
   note_kernel(name);
   hipLaunchKernelGGL((k_gemm_tq2<ACT, SDT, SL, ABL>), grid, dim3(GTHREADS), lds, s, a);
   return check_launch(name);

@@ -166,11 +166,9 @@ __global__ __launch_bounds__(F_THREADS, 2) void k_gemm_tq2f(GemmArgs a) {
 
   const int wave = __builtin_amdgcn_readfirstlane((int)(threadIdx.x >> 6)), lane = threadIdx.x & 63;
   const int r16 = lane & 15, kb = lane >> 4;
-  // Workgroups are dealt to the 8 XCDs round-robin by linear index; the row blocks of one expert read the same
-  // activations, so they get linear indices 8 apart (same XCD, one L2).
   const int row_blocks = (int)((a.N + F_ROWS - 1) / F_ROWS);
-  const int wg_block = (int)((blockIdx.x >> 3) % (unsigned)row_blocks);
-  const TileRef tr = tile_ref(a, (blockIdx.x & 7) + 8 * (int64_t)((blockIdx.x >> 3) / (unsigned)row_blocks), blockIdx.z);
+  int wg_block;
+  const TileRef tr = tile_of_workgroup(a, blockIdx.x, row_blocks, wg_block);
   if (!tr.live) return;  // uniform for the workgroup
   const int64_t e = tr.e, tok0 = tr.tok0, o1 = tr.o1;
   const int ntok = (int)(o1 - tok0 < 32 ? o1 - tok0 : 32);
@@ -651,7 +649,9 @@ int launch_gemm_tq2f_k(const GemmArgs& a, hipStream_t s) {
   const unsigned z = a.tiles ? 1u : (unsigned)((a.max_rows + 31) / 32);
   hipLaunchKernelGGL(k_stage_tq2f, dim3((unsigned)slots, (unsigned)(a.K / 256), z), dim3(F_THREADS), 0, s, a);
   if (const int rc = check_launch("stage_tq2f")) return rc;
-  const dim3 grid((unsigned)(row_blocks * ((slots + 7) / 8 * 8)), 1, z);
+  const int64_t wgs = tile_workgroups(a, row_blocks);
+  if (wgs < 0) return BP_ERR_UNSUPPORTED;
+  const dim3 grid((unsigned)wgs, 1, 1);
   note_kernel("gemm_tq2f_bf16");
   hipLaunchKernelGGL((k_gemm_tq2f<SDT>), grid, dim3(F_THREADS), f_lds_bytes(SDT == BP_F32 ? 4 : 2), s, a);
   return check_launch("gemm_tq2f_bf16");
