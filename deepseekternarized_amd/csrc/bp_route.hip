@@ -79,24 +79,27 @@ __global__ __launch_bounds__(SORT_THREADS) void k_sort(int64_t* __restrict__ ord
   if (threadIdx.x == 0) offsets[E] = carry;
   __threadfence();
   __syncthreads();
+  // Pass 2, 64 ids at a time: every lane finds the lanes that hold its expert (one ballot per bit of the expert index),
+  // the lowest of them claims the run of output slots with one atomic, and a lane's slot is the run's first plus the
+  // number of lower lanes with the same expert.
+  int nbits = 1;
+  while (((int64_t)1 << nbits) < E) ++nbits;
   for (int64_t i0 = lo; i0 < hi; i0 += 64) {
     const int64_t i = i0 + lane;
     const bool live = i < hi;
     const int64_t id = live ? ids[i] : -1;
-    bool todo = live && id >= 0 && id < E;
-    while (__any(todo)) {
-      const unsigned long long pending = __ballot(todo);
-      const int leader = __ffsll((long long)pending) - 1;
-      const int64_t key = __shfl(id, leader, 64);
-      const bool same = todo && id == key;
-      const unsigned long long m = __ballot(same);
+    const bool todo = live && id >= 0 && id < E;
+    unsigned long long same = __ballot(todo);
+    for (int bit = 0; bit < nbits; ++bit) {
+      const unsigned long long set = __ballot(todo && ((id >> bit) & 1));
+      same &= ((id >> bit) & 1) ? set : ~set;
+    }
+    if (todo) {  // (same holds this lane)
+      const int leader = __ffsll((long long)same) - 1;
       int32_t first = 0;
-      if (lane == leader) first = atomicAdd(&mine[key], (int32_t)__popcll(m));  // claims the run of slots
+      if (lane == leader) first = atomicAdd(&mine[id], (int32_t)__popcll(same));  // claims the run of slots
       first = __shfl(first, leader, 64);
-      if (same) {
-        order[first + __popcll(m & ((1ull << lane) - 1ull))] = i;
-        todo = false;
-      }
+      order[first + __popcll(same & ((1ull << lane) - 1ull))] = i;
     }
   }
 }
