@@ -123,6 +123,21 @@ def test_gather_rows_bit_exact(bp):
         assert torch.equal(got, src[order // 6])
 
 
+@pytest.mark.parametrize("rows,inter", [(37, 2048), (5, 1028), (3, 1030), (70000, 8)])
+def test_swiglu_bit_exact(bp, rows, inter):
+    """h = bf16(bf16(silu(bf16 gate)) * bf16 up), the expert MLP's elementwise stage (boilerplate/engine/standard.py:151-154),
+    against torch on bf16 tensors: four columns per thread where the row length allows it, one otherwise (1030), more
+    rows than a grid's y extent."""
+    from deepseekternarized_amd.moe import swiglu_bf16
+
+    g = torch.Generator(device="cuda").manual_seed(rows + inter)
+    gu = torch.randn(rows, 2 * inter, device="cuda", generator=g) * 3.0
+    got = swiglu_bf16(gu, inter)
+    gate, up = gu[:, :inter].to(torch.bfloat16), gu[:, inter:].to(torch.bfloat16)
+    want = torch.nn.functional.silu(gate) * up
+    assert got.dtype == torch.bfloat16 and torch.equal(got, want)
+
+
 # --------------------------------------------------------------------------- GEMM vs golden fixtures
 def _lin_terms(c):
     return [dev(c[f"packed{t}"]) for t in range(c["terms"])], [dev(c[f"scale{t}"]) for t in range(c["terms"])]
