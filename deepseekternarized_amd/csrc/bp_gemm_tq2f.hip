@@ -189,11 +189,7 @@ __global__ __launch_bounds__(F_THREADS, 2) void k_gemm_tq2f(GemmArgs a) {
   // ---- the load stream. Window w of the sequence is window w % nwin of term w / nwin; (lterm, ls) names the next window
   // to request. Per window every wave issues, in this order: the thread's three pieces of the staged window, the thread's
   // row's two scales, the wave's four weight loads. Requests past the last window repeat it (never used).
-#if defined(BP_DEV_ABLATION) && (BP_DEV_ABLATION == 32 || BP_DEV_ABLATION == 38)  // timing only (wrong results): quads of lanes read 64 contiguous bytes
-  const unsigned voff = (unsigned)(lane >> 2) * (unsigned)a.Kp + 16u * (lane & 3);
-#else
   const unsigned voff = (unsigned)r16 * (unsigned)a.Kp + 16u * kb;
-#endif
   unsigned wrow[F_RT];  // byte offset of the row tile's first row (a tile past N repeats the wave's first tile and is not stored)
 #pragma unroll
   for (int r = 0; r < F_RT; ++r) {
@@ -239,11 +235,7 @@ __global__ __launch_bounds__(F_THREADS, 2) void k_gemm_tq2f(GemmArgs a) {
         at = gs ? 4u * (s - pick) : 8u * s;
       }
       const unsigned so = my_scales == 0xfffffff0u ? my_scales : my_scales + at;
-#if defined(BP_DEV_ABLATION) && BP_DEV_ABLATION == 38
-      if (SB == 2) sq[P][0] = so | 0x3c003c00u;
-#else
       if (SB == 2) sq[P][0] = (unsigned)__builtin_amdgcn_raw_buffer_load_b32(srs, (int)so, 0, 0);
-#endif
       else {
         const u32x2 v = __builtin_bit_cast(u32x2, __builtin_amdgcn_raw_buffer_load_b64(srs, (int)so, 0, 0));
         sq[P][0] = v.x;
@@ -285,20 +277,6 @@ __global__ __launch_bounds__(F_THREADS, 2) void k_gemm_tq2f(GemmArgs a) {
     }
   };
 
-#if defined(BP_DEV_ABLATION) && (BP_DEV_ABLATION == 31 || BP_DEV_ABLATION == 35)
-  unsigned st[64];
-  int ns = 0;
-  bool son = BP_DEV_ABLATION == 31;
-#define BP_STAMP() do { if (son && ns < 64) st[ns++] = (unsigned)clock64(); } while (0)
-#if BP_DEV_ABLATION == 35
-#define BP_STAMP2() do { __builtin_amdgcn_sched_barrier(0); BP_STAMP(); __builtin_amdgcn_sched_barrier(0); } while (0)
-#else
-#define BP_STAMP2() do {} while (0)
-#endif
-#else
-#define BP_STAMP() do {} while (0)
-#define BP_STAMP2() do {} while (0)
-#endif
   auto all_windows = [&](auto tt_c) {
     constexpr int TT = decltype(tt_c)::value;  // token tiles processed
     f32x4 total[F_RT][TT];
@@ -307,12 +285,6 @@ __global__ __launch_bounds__(F_THREADS, 2) void k_gemm_tq2f(GemmArgs a) {
 #pragma unroll
       for (int t = 0; t < TT; ++t) total[r][t] = f32x4{0.f, 0.f, 0.f, 0.f};
 
-#if defined(BP_DEV_ABLATION) && BP_DEV_ABLATION == 36
-    if (wave < 4) __builtin_amdgcn_s_setprio(2);
-#endif
-#if defined(BP_DEV_ABLATION) && BP_DEV_ABLATION == 37
-    if (wave >= 4) __builtin_amdgcn_s_setprio(2);
-#endif
     // ---- prologue: windows 0 and 1 requested, window 0's operands and scales into LDS
     request_all(FC<0>{});
     request_all(FC<1>{});
@@ -402,7 +374,6 @@ __global__ __launch_bounds__(F_THREADS, 2) void k_gemm_tq2f(GemmArgs a) {
         if (g == 0) staged_store(H ^ 1, xa[H ^ 1]);  // (the other buffer: last read before the previous barrier)
         request(h_c, FC<g == 0 ? 5 : 0>{});
         __builtin_amdgcn_sched_barrier(0);
-        BP_STAMP2();
         // batch 1: (1, 0)
         static_for<F_RT>([&](auto r_c) {
           constexpr int r = decltype(r_c)::value;
@@ -414,7 +385,6 @@ __global__ __launch_bounds__(F_THREADS, 2) void k_gemm_tq2f(GemmArgs a) {
         if (g == 0) scale_store(H ^ 1, sq[H ^ 1], sodd[H ^ 1]);
         request(h_c, FC<g == 0 ? 6 : 1>{});
         __builtin_amdgcn_sched_barrier(0);
-        BP_STAMP2();
         // batch 2: (0, 1)
         static_for<F_RT>([&](auto r_c) {
           constexpr int r = decltype(r_c)::value;
@@ -427,7 +397,6 @@ __global__ __launch_bounds__(F_THREADS, 2) void k_gemm_tq2f(GemmArgs a) {
         if (g == 1) read_window_scales(FC<H ^ 1>{});
         request(h_c, FC<g == 0 ? 7 : 2>{});
         __builtin_amdgcn_sched_barrier(0);
-        BP_STAMP2();
         // batch 3: (1, 1), and token tile 0's sums under the rows' scales
         static_for<F_RT>([&](auto r_c) {
           constexpr int r = decltype(r_c)::value;
@@ -457,19 +426,12 @@ __global__ __launch_bounds__(F_THREADS, 2) void k_gemm_tq2f(GemmArgs a) {
           D[r][1][1] = moved(s1[1]);
         }
         __builtin_amdgcn_sched_barrier(0);
-        BP_STAMP();
         pgroup(h_c, FC<0>{});
-        BP_STAMP();
         __syncthreads();
-        BP_STAMP();
         pgroup(h_c, FC<1>{});
-        BP_STAMP();
       };
       int w = 0;
       for (; w + 1 < NW; w += 2) {
-#if defined(BP_DEV_ABLATION) && BP_DEV_ABLATION == 35
-        son = w == 6 || w == 8;
-#endif
         pwindow(FC<0>{});
         pwindow(FC<1>{});
       }
@@ -501,7 +463,6 @@ __global__ __launch_bounds__(F_THREADS, 2) void k_gemm_tq2f(GemmArgs a) {
         // What the previous window of this parity left in registers has been used (its activations and scales went to LDS
         // during the window before this one): the window two ahead is requested into them, one load after each row
         // tile's matrix instructions.
-        BP_STAMP();
         int sa[TT];
   #pragma unroll
         for (int t = 0; t < TT; ++t) sa[t] = (int)*(const lds_u32*)(ab + F_OPS + (unsigned)((t * 64 + lane) * 4));
@@ -533,10 +494,6 @@ __global__ __launch_bounds__(F_THREADS, 2) void k_gemm_tq2f(GemmArgs a) {
             }
           }
           __builtin_amdgcn_sched_barrier(0);
-  #if defined(BP_DEV_ABLATION) && BP_DEV_ABLATION == 35
-          asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
-          BP_STAMP2();
-  #endif
           f32x4 C[F_RT][TT];
           // Matrix instructions two chains at a time (the two token tiles of a row tile, or two row tiles when there is
           // one token tile): the second piece's instruction reads the first one's result, with the other chain's
@@ -566,7 +523,6 @@ __global__ __launch_bounds__(F_THREADS, 2) void k_gemm_tq2f(GemmArgs a) {
             }
             __builtin_amdgcn_sched_barrier(0);
           });
-          BP_STAMP2();
   #pragma unroll
           for (int r = 0; r < F_RT; ++r) {
             float sc;
@@ -585,38 +541,24 @@ __global__ __launch_bounds__(F_THREADS, 2) void k_gemm_tq2f(GemmArgs a) {
         };
         __builtin_amdgcn_sched_barrier(0);
         group(FC<0>{});
-        BP_STAMP();
         __builtin_amdgcn_sched_barrier(0);
         staged_store(H ^ 1, xa[H ^ 1]);  // the next window's operands (the other buffer: last read before the previous barrier)
-        BP_STAMP();
         __builtin_amdgcn_sched_barrier(0);
         group(FC<1>{});
-        BP_STAMP();
         __builtin_amdgcn_sched_barrier(0);
         scale_store(H ^ 1, sq[H ^ 1], sodd[H ^ 1]);
-        BP_STAMP();
         __builtin_amdgcn_sched_barrier(0);
         __syncthreads();
       };
 
       int w = 0;
       for (; w + 1 < NW; w += 2) {
-  #if defined(BP_DEV_ABLATION) && BP_DEV_ABLATION == 35
-        son = w == 6 || w == 8;
-  #endif
         window(FC<0>{});
         window(FC<1>{});
       }
       if (w < NW) window(FC<0>{});  // uniform
     }
 
-#if defined(BP_DEV_ABLATION) && (BP_DEV_ABLATION == 31 || BP_DEV_ABLATION == 35)
-    if (blockIdx.x == 8 * 4 * 20 && blockIdx.z == 0) {  // expert 160, row block 0: every wave writes its stamps over its own outputs
-      if (lane == 0)
-        for (int i = 0; i < ns; ++i) a.out[(tok0 + i / 32) * a.N + n_wave + i % 32] = (float)(st[i] - st[0]);
-      return;
-    }
-#endif
     // ---- epilogue: lane holds tokens 4 kb + i of each token tile, output row n_wave + 16 r + r16
 #pragma unroll
     for (int t = 0; t < TT; ++t) {
