@@ -144,7 +144,11 @@ extern "C" int bp_ternary_grouped_gemm(float* out, const void* x, int x_dtype, c
 }
 
 extern "C" size_t bp_grouped_gemm_workspace_bytes(int x_dtype, int64_t T, int64_t N, int64_t K, int64_t E, int fmt) {
-  if (fmt != BP_TQ2 || x_dtype != BP_BF16 || (N < 1024 && tuning().tq2g != 'f')) return 0;
+  if (fmt != BP_TQ2 || x_dtype != BP_BF16) return 0;
+  // (the launcher's own thresholds, so that a call it would turn down does not make its caller allocate: at least two
+  // blocks of 512 output rows, at least three rounds of one workgroup per CU)
+  if (tuning().tq2g != 'f' && (N < 1024 || (T + 31) / 32 * ((N + 511) / 512) < 768)) return 0;
+  if (tuning().tq2g == 'b') return 0;
   return gemm_tq2f_workspace_bytes(T, K, E);
 }
 

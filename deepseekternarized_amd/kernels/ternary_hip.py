@@ -27,6 +27,9 @@ from . import _lib
 _BACKENDS = ("auto", "cuda", "hip", "torch", "cpp")
 
 
+_WORKSPACE_CAP = 8 << 30  # bytes of workspace the mirrored grouped call allocates at most
+
+
 class _HipTernary:
     """Object returned by :func:`ext`: the native module surface of the reference
     (``boilerplate/kernels/csrc/ternary_cuda.cpp:7-10``) over the C ABI."""
@@ -83,6 +86,8 @@ class _HipTernary:
             # Prefill-sized calls get a workspace (the library allocates nothing itself): with one, the TQ2 kernels for bf16
             # activations convert the activations once instead of once per block of output rows.
             need = self.lib.bp_grouped_gemm_workspace_bytes(_lib.dtype_code(x.dtype), T, N, int(K), E, int(fmt)) if max_rows > 16 else 0
+            if need > _WORKSPACE_CAP:  # (about 2.1 bytes per activation: a call this large keeps its memory and runs the kernels without one)
+                need = 0
             if need:
                 ws = torch.empty(need, dtype=torch.uint8, device=out.device)
                 rc = self.lib.bp_ternary_grouped_gemm_ws(

@@ -85,7 +85,8 @@ int bp_ternary_grouped_gemm(float* out, const void* x, int x_dtype, const float*
  * aligned device memory; contents undefined before and after the call) the TQ2 kernels for bf16 activations and more
  * than 16 rows per expert convert the activations to matrix-instruction operands once, in a pass of their own,
  * instead of once per block of output rows; results agree with bp_ternary_grouped_gemm's to float32 rounding of the
- * sums. workspace = NULL, or a size of 0 from bp_grouped_gemm_workspace_bytes (no such kernel for these arguments):
+ * sums. workspace = NULL, or a size of 0 from bp_grouped_gemm_workspace_bytes (no such kernel for these arguments, or a
+ * launch too small for it to pay: fewer than 1024 output rows, or fewer than 768 blocks of 32 tokens x 512 rows):
  * identical to bp_ternary_grouped_gemm. T is the row count of x (all experts). */
 size_t bp_grouped_gemm_workspace_bytes(int x_dtype, int64_t T, int64_t N, int64_t K, int64_t E, int fmt);
 int bp_ternary_grouped_gemm_ws(float* out, const void* x, int x_dtype, const float* x_scale,
