@@ -54,8 +54,8 @@ constexpr int F_SUM = 2 * 32 * 4;                  // ... and the offset sums: [
 constexpr int F_TAIL = F_SCL + F_SUM;              // (48 x 16 bytes)
 constexpr int F_FB = 32 * 544;                     // a staged window of a token tile: operands, scales, sums, padding (544 bytes per token: a multiple of 16)
 static_assert(F_OPS + F_TAIL <= F_FB && F_OPS == F_THREADS * 32 && F_TAIL % 16 == 0, "a staged window: two 16-byte pieces per thread and a tail");
-constexpr int F_SC = 2 * F_FB;                     // LDS: two staged windows, then the rows' scales: 2 slots (window parity) of [512 rows][2 groups] as stored
-constexpr int f_lds_bytes(int scale_bytes) { return F_SC + 2 * F_ROWS * 2 * scale_bytes; }  // 38,912 (16-bit scales) / 43,008 (float32)
+constexpr int F_SC = 2 * F_FB;                     // LDS: two staged windows, then the rows' scales: 2 slots of [512 rows][8 scales] as stored
+constexpr int f_lds_bytes(int scale_bytes) { return F_SC + 2 * F_ROWS * 8 * scale_bytes; }  // 51,200 (16-bit scales) / 67,584 (float32)
 
 template <int N, class F>
 __device__ __forceinline__ void static_for(F&& f) {
@@ -213,8 +213,16 @@ __global__ __launch_bounds__(F_THREADS, 2) void k_gemm_tq2f(GemmArgs a) {
   set_term(0);
   u32x4 W[2][F_RT];        // the weights of the windows of either parity
   u32x4 xa[2][3];          // ... the thread's pieces of their staged activations (two of the operands, one of the tail)
-  unsigned sq[2][SB / 2];  // ... the thread's row's scales: [group 0 | group 1] as stored
-  int sodd[2] = {0, 0};    // ... and, with one scale per window, which of the loaded entries is the window's (uniform)
+  // The rows' scales travel in blocks of 8 entries (4 windows, or 8 with one scale per 256 weights): thread = row, one
+  // 16- or 32-byte load per block (a load per window of 4 bytes per lane costs the memory pipeline as much as one of 16,
+  // and fetches a 64-byte sector per row each time). A row's last block starts 8 entries before the row's end.
+  u32x4 sq[SB / 2];        // the thread's row's block on its way to LDS
+  auto scale_block = [&](int sw, unsigned& first) {  // the block of window sw of a term and its first entry
+    const unsigned b = (unsigned)((2 * sw) >> gs) >> 3;
+    first = 8u * b + 8u <= (unsigned)a.G ? 8u * b : (unsigned)a.G - 8u;
+    return b;
+  };
+  auto starts_block = [&](int sw) { return ((((unsigned)(2 * sw)) >> gs) & 7u) == 0u; };
   // part 0..3: the weights of row tile `part`; 4: the scales; 5, 6, 7: the staged activations; 8: on to the next window.
   // Order within a window: 5, 6, 7, 4 (with the first group's matrix instructions), 0 .. 3 (with the second group's), 8.
   auto request = [&](auto p_c, auto part_c) {
@@ -222,26 +230,13 @@ __global__ __launch_bounds__(F_THREADS, 2) void k_gemm_tq2f(GemmArgs a) {
     const unsigned s = (unsigned)ls;
     if (PART < F_RT) W[P][PART] = buf_load16(wrs, voff, wrow[PART] + 64u * s);
     if (PART == 4) {
-      // entries (2 s) >> gs and (2 s + 1) >> gs of the row, by one load of the same width either way. gs = 1: 16-bit
-      // scales - the aligned pair that holds entry s (rows are dword-aligned: the launcher requires an even number of
-      // entries); float32 - entry s and the one after it, or the one before it for the row's last entry, so that no
-      // load reaches past the row. The store picks entry s for both groups.
-      unsigned at, pick = 0;
-      if (SB == 2) {
-        at = gs ? (2u * s) & ~3u : 4u * s;
-        pick = s & 1u;
-      } else {
-        pick = gs && s + 1 == (unsigned)nwin ? 1u : 0u;
-        at = gs ? 4u * (s - pick) : 8u * s;
+      if (starts_block((int)s)) {  // uniform
+        unsigned first;
+        scale_block((int)s, first);
+        const unsigned so = my_scales == 0xfffffff0u ? my_scales : my_scales + first * SB;
+#pragma unroll
+        for (int i = 0; i < SB / 2; ++i) sq[i] = buf_load16(srs, so == 0xfffffff0u ? so : so + 16u * i, 0u);
       }
-      const unsigned so = my_scales == 0xfffffff0u ? my_scales : my_scales + at;
-      if (SB == 2) sq[P][0] = (unsigned)__builtin_amdgcn_raw_buffer_load_b32(srs, (int)so, 0, 0);
-      else {
-        const u32x2 v = __builtin_bit_cast(u32x2, __builtin_amdgcn_raw_buffer_load_b64(srs, (int)so, 0, 0));
-        sq[P][0] = v.x;
-        sq[P][SB / 2 - 1] = v.y;
-      }
-      sodd[P] = (int)pick;
     }
     if (PART == 5 || PART == 6) xa[P][PART - 5] = buf_load16(xrs, 16u * threadIdx.x + 8192u * (PART - 5), (unsigned)F_FB * s);
     if (PART == 7) xa[P][2] = buf_load16(xrs, tail_off, (unsigned)F_FB * s);
@@ -268,13 +263,15 @@ __global__ __launch_bounds__(F_THREADS, 2) void k_gemm_tq2f(GemmArgs a) {
     *(lds_u32x4*)(ab + 8192u + 16u * threadIdx.x) = v[1];
     if (threadIdx.x < F_TAIL / 16) *(lds_u32x4*)(ab + (unsigned)F_OPS + 16u * threadIdx.x) = v[2];
   };
-  auto scale_store = [&](int slot, const unsigned (&v)[SB / 2], int odd) {
+  // The two LDS slots alternate block by block (also from a term's last block to the next term's first): the slot
+  // written before a window's barrier was last read two blocks - at least four barriers - earlier.
+  int wslot = 0, rslot = 0, rslot_next = 0;  // (uniform)
+  auto scale_store = [&](int sw) {  // the block that window sw of a term starts, if it starts one
+    if (!starts_block(sw)) return;  // uniform
 #pragma unroll
-    for (int i = 0; i < SB / 2; ++i) {
-      unsigned d = v[i];
-      if (gs) d = SB == 2 ? ((v[0] >> (16 * odd)) & 0xffffu) * 0x10001u : v[odd ? SB / 2 - 1 : 0];
-      *(lds_u32*)(unsigned)(F_SC + (slot * F_ROWS + (int)threadIdx.x) * (2 * SB) + 4 * i) = d;
-    }
+    for (int i = 0; i < SB / 2; ++i) *(lds_u32x4*)(unsigned)(F_SC + (wslot * F_ROWS + (int)threadIdx.x) * (8 * SB) + 16 * i) = sq[i];
+    rslot_next = wslot;
+    wslot ^= 1;
   };
 
   auto all_windows = [&](auto tt_c) {
@@ -289,92 +286,105 @@ __global__ __launch_bounds__(F_THREADS, 2) void k_gemm_tq2f(GemmArgs a) {
     request_all(FC<0>{});
     request_all(FC<1>{});
     staged_store(0, xa[0]);
-    scale_store(0, sq[0], sodd[0]);
+    scale_store(0);
     __syncthreads();
 
-    if constexpr (TT == 2) {
-      // ---- 32 tokens: the matrix instructions of a wave run on without a gap. A group's 16 go in four batches of
-      // four row tiles - (token tile 0, piece 0), (1, 0), (0, 1), (1, 1) - so that an operand A is free for the next
-      // group's (read from LDS behind its batch) as soon as its batch has issued, an instruction of the second pieces
-      // finds its accumulator finished, and the scaling of token tile 0's sums runs beside batch 3, that of token tile
-      // 1's beside the next group's batch 0. The workgroup's one barrier per window sits between the two groups: before
-      // it a wave writes the next window's staged activations and scales to LDS, after it it reads them.
-      i32x8 A[2][2];
-      f32x4 base[2];
-      int sa[2][2];                    // [window parity][token tile]
-      unsigned sraw[2][F_RT][SB / 2];  // [window parity]: the window's two scales of the lane's row of each row tile, as stored
-      float scp[F_RT];                 // the scales of the group whose token tile 1 is still to be summed
-      f32x4 C[F_RT][2];
-      i32x8 B[F_RT];
+    // ---- The matrix instructions of a wave run on without a gap. A group's go in batches of four row tiles - (token
+    // tile 0, piece 0), (1, 0), (0, 1), (1, 1); with one token tile only the first and the third - so that an operand A
+    // is free for the next group's (read from LDS behind its batch) as soon as its batch has issued, an instruction of
+    // the second pieces finds its accumulator finished, and the scaling of token tile 0's sums runs beside batch 3, that
+    // of the last token tile's beside the next group's batch 0. The workgroup's one barrier per window sits between the two groups: before
+    // it a wave writes the next window's staged activations and scales to LDS, after it it reads them.
+    constexpr int DT = TT - 1;       // the token tile whose sums wait for the next group's batch 0
+    i32x8 A[TT][2];
+    f32x4 base[TT];
+    int sa[2][TT];                   // [window parity][token tile]
+    unsigned sraw[2][F_RT][SB / 2];  // [window parity]: the window's two scales of the lane's row of each row tile, as stored
+    float scp[F_RT];                 // the scales of the group whose token tile DT is still to be summed
+    f32x4 C[F_RT][TT];
+    i32x8 B[F_RT];
+#pragma unroll
+    for (int r = 0; r < F_RT; ++r) {
+      scp[r] = 0.f;
+#pragma unroll
+      for (int t = 0; t < TT; ++t) C[r][t] = f32x4{0.f, 0.f, 0.f, 0.f};
+    }
+    auto read_a = [&](unsigned ab, int g, auto t_c, auto p_c) {
+      constexpr int t = decltype(t_c)::value, pp = decltype(p_c)::value;
+      const unsigned at = ab + (unsigned)(((g * 2 + t) * 2 + pp) * 2048) + alane;
+      const u32x4 lo = *(const lds_u32x4*)at, hi4 = *(const lds_u32x4*)(at + 256);
+      A[t][pp] = i32x8{(int)lo.x, (int)lo.y, (int)lo.z, (int)lo.w, (int)hi4.x, (int)hi4.y, (int)hi4.z, (int)hi4.w};
+    };
+    auto read_base = [&](unsigned ab, int g) {
+#pragma unroll
+      for (int t = 0; t < TT; ++t) base[t] = __builtin_bit_cast(f32x4, *(const lds_u32x4*)(ab + F_OPS + F_SCL + (unsigned)((g * 32 + 16 * t + 4 * kb) * 4)));
+    };
+    auto read_window_scales = [&](auto h_c, int sw) {  // block scales and row scales of the window of parity H, window sw of its term
+      constexpr int H = decltype(h_c)::value;
+      const unsigned ab = (unsigned)(H * F_FB);
+      unsigned first;
+      scale_block(sw, first);
+      if (starts_block(sw)) rslot = rslot_next;
+      const unsigned sb = (unsigned)(F_SC + (rslot * F_ROWS + wave * (16 * F_RT) + r16) * (8 * SB)) + ((((unsigned)(2 * sw)) >> gs) - first) * SB;
+#pragma unroll
+      for (int t = 0; t < TT; ++t) sa[H][t] = (int)*(const lds_u32*)(ab + F_OPS + (unsigned)((t * 64 + lane) * 4));
 #pragma unroll
       for (int r = 0; r < F_RT; ++r) {
-        scp[r] = 0.f;
-        C[r][0] = C[r][1] = f32x4{0.f, 0.f, 0.f, 0.f};
-      }
-      auto read_a = [&](unsigned ab, int g, auto t_c, auto p_c) {
-        constexpr int t = decltype(t_c)::value, pp = decltype(p_c)::value;
-        const unsigned at = ab + (unsigned)(((g * 2 + t) * 2 + pp) * 2048) + alane;
-        const u32x4 lo = *(const lds_u32x4*)at, hi4 = *(const lds_u32x4*)(at + 256);
-        A[t][pp] = i32x8{(int)lo.x, (int)lo.y, (int)lo.z, (int)lo.w, (int)hi4.x, (int)hi4.y, (int)hi4.z, (int)hi4.w};
-      };
-      auto read_base = [&](unsigned ab, int g) {
-#pragma unroll
-        for (int t = 0; t < 2; ++t) base[t] = __builtin_bit_cast(f32x4, *(const lds_u32x4*)(ab + F_OPS + F_SCL + (unsigned)((g * 32 + 16 * t + 4 * kb) * 4)));
-      };
-      auto read_window_scales = [&](auto h_c) {  // block scales and row scales of the window of parity H
-        constexpr int H = decltype(h_c)::value;
-        const unsigned ab = (unsigned)(H * F_FB);
-        const unsigned sb = (unsigned)(F_SC + (H * F_ROWS + wave * (16 * F_RT) + r16) * (2 * SB));
-#pragma unroll
-        for (int t = 0; t < 2; ++t) sa[H][t] = (int)*(const lds_u32*)(ab + F_OPS + (unsigned)((t * 64 + lane) * 4));
-#pragma unroll
-        for (int r = 0; r < F_RT; ++r) {
-          if (SB == 2) sraw[H][r][0] = *(const lds_u32*)(sb + (unsigned)(16 * r * 2 * SB));
-          else {
-            const u32x2 v = *(const lds_u32x2*)(sb + (unsigned)(16 * r * 2 * SB));
-            sraw[H][r][0] = v.x;
-            sraw[H][r][SB / 2 - 1] = v.y;
-          }
+        const unsigned at = sb + (unsigned)(16 * r * 8 * SB);
+        if (SB == 2) {
+          if (gs) sraw[H][r][0] = (unsigned)*(const lds_u16*)at * 0x10001u;  // (one scale for both groups)
+          else sraw[H][r][0] = *(const lds_u32*)at;
+        } else if (gs) {
+          sraw[H][r][0] = sraw[H][r][SB / 2 - 1] = *(const lds_u32*)at;
+        } else {
+          const u32x2 v = *(const lds_u32x2*)at;
+          sraw[H][r][0] = v.x;
+          sraw[H][r][SB / 2 - 1] = v.y;
         }
-      };
-      read_a(0u, 0, FC<0>{}, FC<0>{});
+      }
+    };
+    read_a(0u, 0, FC<0>{}, FC<0>{});
+    read_a(0u, 0, FC<0>{}, FC<1>{});
+    if constexpr (TT == 2) {
       read_a(0u, 0, FC<1>{}, FC<0>{});
-      read_a(0u, 0, FC<0>{}, FC<1>{});
       read_a(0u, 0, FC<1>{}, FC<1>{});
-      read_base(0u, 0);
-      read_window_scales(FC<0>{});
+    }
+    read_base(0u, 0);
+    read_window_scales(FC<0>{}, 0);
 
-      unsigned D[F_RT][2][2];  // the window's bytes regrouped: D[r][g] = the lane's 8 bytes (32 weights) of group g
-      auto pgroup = [&](auto h_c, auto g_c) {
-        constexpr int H = decltype(h_c)::value, g = decltype(g_c)::value;
-        const unsigned nb = (unsigned)((g == 0 ? H : H ^ 1) * F_FB);  // where the next group's operands are
-        constexpr int ng = g ^ 1;
-        auto mfma = [&](const i32x8& av, const i32x8& bv, const f32x4& cv, int sav) {
-          return __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(av, bv, cv, 0 /* A: E4M3 */, 4 /* B: E2M1 */, g, sav, 0, ones);
-        };
-        auto row_scale = [&](int r) {
-          if (SDT == BP_F32) return __uint_as_float(sraw[H][r][g == 0 ? 0 : SB / 2 - 1]);
-          const unsigned rawsc = g == 0 ? sraw[H][r][0] & 0xffffu : sraw[H][r][0] >> 16;
-          return SDT == BP_F16 ? f16_bits_to_f32((uint16_t)rawsc) : __uint_as_float(rawsc << 16);
-        };
-        // batch 0: (token tile 0, piece 0). A row tile's operand B is made just before its first use; the previous
-        // group's token tile 1 is summed here.
-        static_for<F_RT>([&](auto r_c) {
-          constexpr int r = decltype(r_c)::value;
-          const unsigned d0 = D[r][g][0], d1 = D[r][g][1];
-          B[r] = i32x8{(int)((d0 << 1) & m66), (int)((d0 >> 1) & m66), (int)((d1 << 1) & m66), (int)((d1 >> 1) & m66), 0, 0, 0, 0};
+    unsigned D[F_RT][2][2];  // the window's bytes regrouped: D[r][g] = the lane's 8 bytes (32 weights) of group g
+    int cs = 0, ns = 0;  // the window's index in its term, and the next window's (uniform)
+    auto pgroup = [&](auto h_c, auto g_c) {
+      constexpr int H = decltype(h_c)::value, g = decltype(g_c)::value;
+      const unsigned nb = (unsigned)((g == 0 ? H : H ^ 1) * F_FB);  // where the next group's operands are
+      constexpr int ng = g ^ 1;
+      auto mfma = [&](const i32x8& av, const i32x8& bv, const f32x4& cv, int sav) {
+        return __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(av, bv, cv, 0 /* A: E4M3 */, 4 /* B: E2M1 */, g, sav, 0, ones);
+      };
+      auto row_scale = [&](int r) {
+        if (SDT == BP_F32) return __uint_as_float(sraw[H][r][g == 0 ? 0 : SB / 2 - 1]);
+        const unsigned rawsc = g == 0 ? sraw[H][r][0] & 0xffffu : sraw[H][r][0] >> 16;
+        return SDT == BP_F16 ? f16_bits_to_f32((uint16_t)rawsc) : __uint_as_float(rawsc << 16);
+      };
+      // batch 0: (token tile 0, piece 0). A row tile's operand B is made just before its first use; the previous
+      // group's token tile 1 is summed here.
+      static_for<F_RT>([&](auto r_c) {
+        constexpr int r = decltype(r_c)::value;
+        const unsigned d0 = D[r][g][0], d1 = D[r][g][1];
+        B[r] = i32x8{(int)((d0 << 1) & m66), (int)((d0 >> 1) & m66), (int)((d1 << 1) & m66), (int)((d1 >> 1) & m66), 0, 0, 0, 0};
 #pragma unroll
-          for (int i = 0; i < 4; ++i) total[r][1][i] += scp[r] * C[r][1][i];
-          asm volatile("" : "+v"(total[r][1]));
-          C[r][0] = mfma(A[0][0], B[r], base[0], sa[H][0]);
-          asm volatile("" : "+v"(C[r][0]) : : "memory");
-          __builtin_amdgcn_sched_barrier(0);
-        });
-        read_a(nb, ng, FC<0>{}, FC<0>{});
-        if (g == 0) staged_store(H ^ 1, xa[H ^ 1]);  // (the other buffer: last read before the previous barrier)
-        request(h_c, FC<g == 0 ? 5 : 0>{});
+        for (int i = 0; i < 4; ++i) total[r][DT][i] += scp[r] * C[r][DT][i];
+        asm volatile("" : "+v"(total[r][DT]));
+        C[r][0] = mfma(A[0][0], B[r], base[0], sa[H][0]);
+        asm volatile("" : "+v"(C[r][0]) : : "memory");
         __builtin_amdgcn_sched_barrier(0);
-        // batch 1: (1, 0)
+      });
+      read_a(nb, ng, FC<0>{}, FC<0>{});
+      if (g == 0) staged_store(H ^ 1, xa[H ^ 1]);  // (the other buffer: last read before the previous barrier)
+      request(h_c, FC<g == 0 ? 5 : 0>{});
+      __builtin_amdgcn_sched_barrier(0);
+      // batch 1: (1, 0)
+      if constexpr (TT == 2) {
         static_for<F_RT>([&](auto r_c) {
           constexpr int r = decltype(r_c)::value;
           C[r][1] = mfma(A[1][0], B[r], base[1], sa[H][1]);
@@ -382,22 +392,24 @@ __global__ __launch_bounds__(F_THREADS, 2) void k_gemm_tq2f(GemmArgs a) {
           __builtin_amdgcn_sched_barrier(0);
         });
         read_a(nb, ng, FC<1>{}, FC<0>{});
-        if (g == 0) scale_store(H ^ 1, sq[H ^ 1], sodd[H ^ 1]);
-        request(h_c, FC<g == 0 ? 6 : 1>{});
+      }
+      if (g == 0) scale_store(ns);
+      request(h_c, FC<g == 0 ? 6 : 1>{});
+      __builtin_amdgcn_sched_barrier(0);
+      // batch 2: (0, 1)
+      static_for<F_RT>([&](auto r_c) {
+        constexpr int r = decltype(r_c)::value;
+        C[r][0] = mfma(A[0][1], B[r], C[r][0], sa[H][0]);
+        asm volatile("" : "+v"(C[r][0]) : : "memory");
         __builtin_amdgcn_sched_barrier(0);
-        // batch 2: (0, 1)
-        static_for<F_RT>([&](auto r_c) {
-          constexpr int r = decltype(r_c)::value;
-          C[r][0] = mfma(A[0][1], B[r], C[r][0], sa[H][0]);
-          asm volatile("" : "+v"(C[r][0]) : : "memory");
-          __builtin_amdgcn_sched_barrier(0);
-        });
-        read_a(nb, ng, FC<0>{}, FC<1>{});
-        read_base(nb, ng);  // (the accumulators' starting values were last read by batch 1)
-        if (g == 1) read_window_scales(FC<H ^ 1>{});
-        request(h_c, FC<g == 0 ? 7 : 2>{});
-        __builtin_amdgcn_sched_barrier(0);
-        // batch 3: (1, 1), and token tile 0's sums under the rows' scales
+      });
+      read_a(nb, ng, FC<0>{}, FC<1>{});
+      read_base(nb, ng);  // (the accumulators' starting values were last read by batch 1)
+      if (g == 1) read_window_scales(FC<H ^ 1>{}, ns);
+      request(h_c, FC<g == 0 ? 7 : 2>{});
+      __builtin_amdgcn_sched_barrier(0);
+      // batch 3: (1, 1), and token tile 0's sums under the rows' scales
+      if constexpr (TT == 2) {
         static_for<F_RT>([&](auto r_c) {
           constexpr int r = decltype(r_c)::value;
           C[r][1] = mfma(A[1][1], B[r], C[r][1], sa[H][1]);
@@ -410,154 +422,43 @@ __global__ __launch_bounds__(F_THREADS, 2) void k_gemm_tq2f(GemmArgs a) {
           __builtin_amdgcn_sched_barrier(0);
         });
         read_a(nb, ng, FC<1>{}, FC<1>{});
-        request(h_c, FC<g == 0 ? 4 : 3>{});
-        if (g == 1) request(h_c, FC<8>{});
-        __builtin_amdgcn_sched_barrier(0);
-      };
-      auto pwindow = [&](auto h_c) {
-        constexpr int H = decltype(h_c)::value;
+      } else {
 #pragma unroll
-        for (int r = 0; r < F_RT; ++r) {
-          const auto s0 = __builtin_amdgcn_permlane32_swap(W[H][r].x, W[H][r].z, false, false);
-          const auto s1 = __builtin_amdgcn_permlane32_swap(W[H][r].y, W[H][r].w, false, false);
-          D[r][0][0] = moved(s0[0]);
-          D[r][0][1] = moved(s1[0]);
-          D[r][1][0] = moved(s0[1]);
-          D[r][1][1] = moved(s1[1]);
-        }
-        __builtin_amdgcn_sched_barrier(0);
-        pgroup(h_c, FC<0>{});
-        __syncthreads();
-        pgroup(h_c, FC<1>{});
-      };
-      int w = 0;
-      for (; w + 1 < NW; w += 2) {
-        pwindow(FC<0>{});
-        pwindow(FC<1>{});
+        for (int r = 0; r < F_RT; ++r) scp[r] = row_scale(r);
       }
-      if (w < NW) pwindow(FC<0>{});  // uniform
-      // the last group's token tile 1
+      request(h_c, FC<g == 0 ? 4 : 3>{});
+      if (g == 1) request(h_c, FC<8>{});
+      __builtin_amdgcn_sched_barrier(0);
+    };
+    auto pwindow = [&](auto h_c) {
+      constexpr int H = decltype(h_c)::value;
 #pragma unroll
-      for (int r = 0; r < F_RT; ++r)
-#pragma unroll
-        for (int i = 0; i < 4; ++i) total[r][1][i] += scp[r] * C[r][1][i];
-    } else {
-      // one window of parity H
-      auto window = [&](auto h_c) {
-        constexpr int H = decltype(h_c)::value;
-        const unsigned ab = (unsigned)(H * F_FB);
-        const unsigned sb = (unsigned)(F_SC + (H * F_ROWS + wave * (16 * F_RT) + r16) * (2 * SB));
-        // this window's bytes regrouped: D[r][g] = the lane's 8 bytes (32 weights) of group g
-        unsigned D[F_RT][2][2];
-  #pragma unroll
-        for (int r = 0; r < F_RT; ++r) {
-          const auto s0 = __builtin_amdgcn_permlane32_swap(W[H][r].x, W[H][r].z, false, false);
-          const auto s1 = __builtin_amdgcn_permlane32_swap(W[H][r].y, W[H][r].w, false, false);
-          // (copies into other registers: the swap works in place, and the registers of W[H] are wanted back at once for
-          // the requests below - otherwise the loop ends with moves that wait for the loads just issued)
-          D[r][0][0] = moved(s0[0]);
-          D[r][0][1] = moved(s1[0]);
-          D[r][1][0] = moved(s0[1]);
-          D[r][1][1] = moved(s1[1]);
-        }
-        // What the previous window of this parity left in registers has been used (its activations and scales went to LDS
-        // during the window before this one): the window two ahead is requested into them, one load after each row
-        // tile's matrix instructions.
-        int sa[TT];
-  #pragma unroll
-        for (int t = 0; t < TT; ++t) sa[t] = (int)*(const lds_u32*)(ab + F_OPS + (unsigned)((t * 64 + lane) * 4));
-        unsigned sraw[F_RT][SB / 2];  // the window's two scales of the lane's row of each row tile, as stored
-  #pragma unroll
-        for (int r = 0; r < F_RT; ++r) {
-          if (SB == 2) sraw[r][0] = *(const lds_u32*)(sb + (unsigned)(16 * r * 2 * SB));
-          else {
-            const u32x2 v = *(const lds_u32x2*)(sb + (unsigned)(16 * r * 2 * SB));
-            sraw[r][0] = v.x;
-            sraw[r][SB / 2 - 1] = v.y;
-          }
-        }
-
-        // One group of the window: the group's operands, its matrix instructions, its sums under the rows' scales.
-        auto group = [&](auto g_c) {
-          constexpr int g = decltype(g_c)::value;
-          auto& tot = total;
-          f32x4 base[TT];
-          i32x8 A[TT][2];
-  #pragma unroll
-          for (int t = 0; t < TT; ++t) {
-            base[t] = __builtin_bit_cast(f32x4, *(const lds_u32x4*)(ab + F_OPS + F_SCL + (unsigned)((g * 32 + 16 * t + 4 * kb) * 4)));
-  #pragma unroll
-            for (int p = 0; p < 2; ++p) {
-              const unsigned at = ab + (unsigned)(((g * 2 + t) * 2 + p) * 2048) + alane;
-              const u32x4 lo = *(const lds_u32x4*)at, hi4 = *(const lds_u32x4*)(at + 256);
-              A[t][p] = i32x8{(int)lo.x, (int)lo.y, (int)lo.z, (int)lo.w, (int)hi4.x, (int)hi4.y, (int)hi4.z, (int)hi4.w};
-            }
-          }
-          __builtin_amdgcn_sched_barrier(0);
-          f32x4 C[F_RT][TT];
-          // Matrix instructions two chains at a time (the two token tiles of a row tile, or two row tiles when there is
-          // one token tile): the second piece's instruction reads the first one's result, with the other chain's
-          // instruction between them.
-          auto operand_b = [&](int r) {
-            const unsigned d0 = D[r][g][0], d1 = D[r][g][1];
-            return i32x8{(int)((d0 << 1) & m66), (int)((d0 >> 1) & m66), (int)((d1 << 1) & m66), (int)((d1 >> 1) & m66), 0, 0, 0, 0};
-          };
-          static_for<F_RT * TT / 2>([&](auto u_c) {
-            constexpr int u = decltype(u_c)::value;
-            constexpr int ra = TT == 2 ? u : 2 * u, rb = TT == 2 ? u : 2 * u + 1, ta = 0, tb = TT == 2 ? 1 : 0;
-            const i32x8 Ba = operand_b(ra), Bb = TT == 2 ? Ba : operand_b(rb);
-            C[ra][ta] = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(A[ta][0], Ba, base[ta], 0 /* A: E4M3 */, 4 /* B: E2M1 */, g, sa[ta], 0, ones);
-            C[rb][tb] = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(A[tb][0], Bb, base[tb], 0, 4, g, sa[tb], 0, ones);
-            C[ra][ta] = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(A[ta][1], Ba, C[ra][ta], 0, 4, g, sa[ta], 0, ones);
-            C[rb][tb] = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(A[tb][1], Bb, C[rb][tb], 0, 4, g, sa[tb], 0, ones);
-            // (the products named here, so that the matrix instructions stay above the loads)
-            asm volatile("" : "+v"(C[ra][ta]), "+v"(C[rb][tb]) : : "memory");
-            __builtin_amdgcn_sched_barrier(0);
-            if (g == 0) {
-              request(h_c, FC<u == 0 ? 5 : 7>{});
-              request(h_c, FC<u == 0 ? 6 : 4>{});
-            } else {
-              request(h_c, FC<2 * u>{});
-              request(h_c, FC<2 * u + 1>{});
-              if (u == 1) request(h_c, FC<8>{});
-            }
-            __builtin_amdgcn_sched_barrier(0);
-          });
-  #pragma unroll
-          for (int r = 0; r < F_RT; ++r) {
-            float sc;
-            if (SDT == BP_F32) sc = __uint_as_float(sraw[r][g]);
-            else {
-              const unsigned rawsc = g == 0 ? sraw[r][0] & 0xffffu : sraw[r][0] >> 16;
-              sc = SDT == BP_F16 ? f16_bits_to_f32((uint16_t)rawsc) : __uint_as_float(rawsc << 16);
-            }
-  #pragma unroll
-            for (int t = 0; t < TT; ++t) {
-  #pragma unroll
-              for (int i = 0; i < 4; ++i) tot[r][t][i] += sc * C[r][t][i];
-              asm volatile("" : "+v"(tot[r][t]));  // (keeps the matrix instructions from sinking below what follows)
-            }
-          }
-        };
-        __builtin_amdgcn_sched_barrier(0);
-        group(FC<0>{});
-        __builtin_amdgcn_sched_barrier(0);
-        staged_store(H ^ 1, xa[H ^ 1]);  // the next window's operands (the other buffer: last read before the previous barrier)
-        __builtin_amdgcn_sched_barrier(0);
-        group(FC<1>{});
-        __builtin_amdgcn_sched_barrier(0);
-        scale_store(H ^ 1, sq[H ^ 1], sodd[H ^ 1]);
-        __builtin_amdgcn_sched_barrier(0);
-        __syncthreads();
-      };
-
-      int w = 0;
-      for (; w + 1 < NW; w += 2) {
-        window(FC<0>{});
-        window(FC<1>{});
+      for (int r = 0; r < F_RT; ++r) {
+        const auto s0 = __builtin_amdgcn_permlane32_swap(W[H][r].x, W[H][r].z, false, false);
+        const auto s1 = __builtin_amdgcn_permlane32_swap(W[H][r].y, W[H][r].w, false, false);
+        D[r][0][0] = moved(s0[0]);
+        D[r][0][1] = moved(s1[0]);
+        D[r][1][0] = moved(s0[1]);
+        D[r][1][1] = moved(s1[1]);
       }
-      if (w < NW) window(FC<0>{});  // uniform
+      __builtin_amdgcn_sched_barrier(0);
+      ns = cs + 1 < nwin ? cs + 1 : 0;  // the next window's index in its term
+      pgroup(h_c, FC<0>{});
+      __syncthreads();
+      pgroup(h_c, FC<1>{});
+      cs = ns;
+    };
+    int w = 0;
+    for (; w + 1 < NW; w += 2) {
+      pwindow(FC<0>{});
+      pwindow(FC<1>{});
     }
+    if (w < NW) pwindow(FC<0>{});  // uniform
+    // the last group's token tile DT
+#pragma unroll
+    for (int r = 0; r < F_RT; ++r)
+#pragma unroll
+      for (int i = 0; i < 4; ++i) total[r][DT][i] += scp[r] * C[r][DT][i];
 
     // ---- epilogue: lane holds tokens 4 kb + i of each token tile, output row n_wave + 16 r + r16
 #pragma unroll
