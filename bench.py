@@ -3,7 +3,7 @@
     python bench.py [--gpus 1] [--steps K] [--warmup W] [--spin-up SECONDS] [--workload NAME] [--no-extras] [--no-cpu]
 
 A step is one pass of the hot path over one batch of synthetic input. For the decode workloads (the default is
-BASELINE config 1: TQ1, K = 7168, N = 2048, one token, bf16) it is one grouped launch that streams L distinct packed
+the headline configuration: TQ1, K = 7168, N = 2048, one token, bf16) it is one grouped launch that streams L distinct packed
 linears of the named configuration (L chosen so the packed weights exceed the 256 MB Infinity Cache, i.e. every step
 reads its weights from HBM). `--workload cfg3_grouped` times the grouped-expert GEMM of config 3 (value in TFLOP/s,
 roofline against the bf16 MFMA peak), `--workload cfg2_moe_T{1,32,256}` one routed-expert layer of config 2; these

@@ -1,4 +1,4 @@
-"""BASELINE configs 2, 3 and 4 at their full shapes on the device. The whole oracle product at these sizes would take
+"""The benchmark configurations 2, 3 and 4 at their full shapes on the device. The whole oracle product at these sizes would take
 minutes on the host, so every launch is checked on samples against the float64 dense evaluation (weights decoded by the
 bit-exact unpack kernel and evaluated on the host) and through size-independent properties (linearity on integer
 inputs, unit-vector read-out)."""
