@@ -65,12 +65,6 @@ __device__ __forceinline__ void static_for(F&& f) {
   }
 }
 
-__device__ __forceinline__ unsigned moved(unsigned v) {  // v in a register of its own
-  unsigned r;
-  asm("v_mov_b32 %0, %1" : "=&v"(r) : "v"(v));
-  return r;
-}
-
 // Where token tile (expert e, first row tok0) keeps its staged windows: tile z of expert e starts 32 (e + z) + offsets[e]
 // tokens into the workspace, so tiles never overlap whatever the experts' row counts are.
 __device__ __forceinline__ unsigned char* staged_tile(const GemmArgs& a, int64_t e, int64_t tok0) {
@@ -433,13 +427,13 @@ __global__ __launch_bounds__(F_THREADS, 2) void k_gemm_tq2f(GemmArgs a) {
     auto pwindow = [&](auto h_c) {
       constexpr int H = decltype(h_c)::value;
 #pragma unroll
-      for (int r = 0; r < F_RT; ++r) {
+      for (int r = 0; r < F_RT; ++r) {  // (in place: the registers of W[H] are requested again only in this window's second group, after D's last use)
         const auto s0 = __builtin_amdgcn_permlane32_swap(W[H][r].x, W[H][r].z, false, false);
         const auto s1 = __builtin_amdgcn_permlane32_swap(W[H][r].y, W[H][r].w, false, false);
-        D[r][0][0] = moved(s0[0]);
-        D[r][0][1] = moved(s1[0]);
-        D[r][1][0] = moved(s0[1]);
-        D[r][1][1] = moved(s1[1]);
+        D[r][0][0] = s0[0];
+        D[r][0][1] = s1[0];
+        D[r][1][0] = s0[1];
+        D[r][1][1] = s1[1];
       }
       __builtin_amdgcn_sched_barrier(0);
       ns = cs + 1 < nwin ? cs + 1 : 0;  // the next window's index in its term
