@@ -88,61 +88,17 @@ __device__ __forceinline__ int f4_pair_byte(int j, int kbA, int hf) {
   return 64 * (j >> 2) + 16 * (2 * hf + (kbA >> 1)) + 4 * (j & 3) + 2 * (kbA & 1);
 }
 
-// ABL (development): timing ablations - 1 no chunk loop, 2 no table reads, 3 no operand A reads, 4 no matrix instructions, 5 no byte extraction (and the loads are not waited for),
-// 6 bytes extracted from registers that are not loaded (no loads at all), 7 = 2 + 3 + 4 (loads and byte extraction only),
-// 8 = 7 without the byte extraction (loads and their realignment only)
-//
-// NTOK > 1: up to NTOK token rows per expert (small decode batches). Every token has its own operand A tile; the
-// packed bytes and the table reads are shared. To fit 4 tiles beside the table, an activation is then split into
-// TWO fp8 pieces (PC = 2: exact for bf16 / int8 values down to 2^-9 of their group's largest magnitude, at most
-// 2^-17 of it dropped below), and one matrix instruction serves TWO tokens: the 64-byte window (half a chunk, 320
-// digits) that instructions 0..3, and the one that instructions 4..7 multiply holds digits of only 3 groups
-// (0, 1, 2 and 2, 3, 4), so a token needs 3 group slots x 2 pieces = 6 rows instead of 10 if each window has its
-// own accumulator tile. Row 4 s + 2 t + p = piece p of token t (of the pair) in slot s; slot s is group s in the
-// first window and group 3, 4, 2 (s = 0, 1, 2) in the second, so a lane of the result (rows 4 lg + i) holds both
-// tokens' pieces of one group per window. 8 matrix instructions per chunk and token pair; with two pairs the ring
-// of loads is two chunks (registers; the loads are not what a wave then waits for).
-//
-// SR (one token, 2-byte scales): scales by the round. A scale per row and group loaded where it is applied is a wave
-// load per chunk that touches 16 memory lines for 8 bytes each: a third of the kernel's load instructions for 7 % of its
-// bytes. Instead a wave loads, once per round of the ring (4 chunks = 20 groups = 40 bytes of a row's scales), 16 bytes
-// per lane (quarters 0..2 of a row's four lanes cover 48 bytes), a round ahead and unconditionally - so the compiler's
-// count of loads in flight stays exact - parks them in a private 1.25 KiB slot of LDS at the start of the round, and a
-// chunk's two scales per lane are two 2-byte LDS reads.
-template <int SDT, int WAVES, int ABL = 0, int NTOK = 1, int SR = 0>
-__global__ __launch_bounds__(WAVES * 64, 4) void k_tq1_gemv_fp4(GemmArgs a, int total_chunks, int first_chunk, int nchunks, int bpw /* row blocks per workgroup */, int first_row) {
-  static_assert(!SR || (SDT != BP_F32 && F4_GR == 1), "scales by the round: one tile per wave, 2-byte scales (a round of 2 or 4 chunks is 20 or 40 bytes of a row's scales)");
-  constexpr int THREADS = WAVES * 64, GR = F4_GR, RD = NTOK <= 2 ? F4_RD : 2, BD = F4_BD, AD = F4_AD, PAIRS = NTOK <= 2 ? F4_PAIRS : 0;
-  static_assert(!PAIRS || RD % 2 == 0, "pairs of chunks need an even ring");
-  static_assert(NTOK == 1 || (GR == 1 && AD == 0 && NTOK % 2 == 0), "several tokens: one tile per wave, one operand A buffer, token pairs");
-  constexpr int NP = NTOK / 2;               // token pairs
-  constexpr int PC = f4_pieces(NTOK);        // fp8 pieces per activation
-  constexpr int F4_HI_OFF = 64 * PC * 16, F4_ZERO_OFF = F4_HI_OFF + 4 * PC * 16, F4_PRE_OFF = F4_ZERO_OFF + 16;
-  constexpr int F4_INV_OFF = F4_PRE_OFF + 32, F4_CHUNK_BYTES = f4_chunk_bytes(NTOK);
-  constexpr int AT = F4_LUT_BYTES;           // the operand A tiles (one per token) start after the table
-  constexpr int SB = SDT == BP_F32 ? 4 : 2;  // bytes per scale
+// Layout of one chunk of an operand A tile for PC pieces per activation (byte offsets within the chunk's part).
+template <int PC>
+struct F4Tile {
+  static constexpr int HI_OFF = 64 * PC * 16, ZERO_OFF = HI_OFF + 4 * PC * 16, PRE_OFF = ZERO_OFF + 16;
+  static constexpr int INV_OFF = PRE_OFF + 32, CHUNK_BYTES = (64 + 4) * PC * 16 + 16 + 32 + 32;
+};
 
-  const int wave = __builtin_amdgcn_readfirstlane((int)(threadIdx.x >> 6)), lane = threadIdx.x & 63;
-  const int r16 = lane & 15, kb = lane >> 4;
-  const int64_t e = blockIdx.y;
-  const int64_t o0 = clamp_i64(a.offsets[e], 0, a.T), o1 = clamp_i64(a.offsets[e + 1], 0, a.T);
-  // A launch takes the expert's token rows first_row .. first_row + NTOK - 1 (one token: its first row); an expert with
-  // more rows than that gets further launches, one without any in this range is done at once (uniform).
-  const int64_t tok = o0 + (NTOK == 1 ? 0 : first_row);
-  if (tok >= o1) return;
-  const int ntok = o1 - tok < NTOK ? (int)(o1 - tok) : NTOK;
-  const int npairs = (ntok + 1) >> 1;  // token pairs the expert has in this launch: the others' matrix instructions are left out
-  float xsc[NTOK];  // int8 activations: the tokens' scales
-#pragma unroll
-  for (int tt = 0; tt < NTOK; ++tt) xsc[tt] = a.x_dtype == BP_I8 && tt < ntok ? a.x_scale[tok + tt] : 1.f;
-  // the tiles of the NTOK tokens are interleaved chunk by chunk (a pair's tiles are a constant apart)
-  auto tile_at = [](int tt, int c) { return AT + (c * NTOK + tt) * F4_CHUNK_BYTES; };
-  const int gs = a.group == 256 ? 1 : 0;  // scale groups of 256: two 128-wide work groups share a scale
-  const bool x16 = a.x_dtype == BP_BF16 || a.x_dtype == BP_F16;
-  auto widen16 = [&](unsigned h) { return a.x_dtype == BP_BF16 ? bf16_bits_to_f32((uint16_t)h) : f16_bits_to_f32((uint16_t)h); };
-
-  // ---- the byte table: entry v = digits d0..d4 of v as fp4 codes (-1 -> 0xA, 0 -> 0, +1 -> 0x2) in nibbles 0..4, one
-  // copy per LDS bank: four threads per entry, eight copies each.
+// ---- the byte table: entry v = digits d0..d4 of v as fp4 codes (-1 -> 0xA, 0 -> 0, +1 -> 0x2) in nibbles 0..4, one
+// copy per LDS bank: four threads per entry, eight copies each.
+template <int THREADS>
+__device__ __forceinline__ void f4_build_table() {
   for (int idx = threadIdx.x; idx < 256 * 4; idx += THREADS) {
     unsigned v = (unsigned)idx >> 2, ent = 0;
     if (v < 243) {
@@ -156,15 +112,18 @@ __global__ __launch_bounds__(WAVES * 64, 4) void k_tq1_gemv_fp4(GemmArgs a, int 
 #pragma unroll
     for (int cpy = 0; cpy < 8; ++cpy) *(lds_u32*)(128 * (idx >> 2) + 4 * (8 * (idx & 3) + cpy)) = ent;
   }
-  // A launch covers the chunks first_chunk .. first_chunk + nchunks - 1 of every row (all of them unless the tokens'
-  // tiles of all chunks do not fit in LDS: then the host launches once per segment of K, and the output takes the
-  // segments' partial sums one launch after the other). Chunk c below is chunk cb + c of the rows.
-  const int cb = NTOK == 1 ? 0 : first_chunk;
-  // The last bytes of a chunk are completed from the first dword of the chunk after it (rows start at any byte). At
-  // the end of a row that dword meets activations that are 0; at the end of a segment it is needed, so the chunk
-  // after a segment that is not the last one is loaded as well.
-  const int last_load = NTOK > 1 && cb + nchunks < total_chunks ? nchunks : nchunks - 1;
+}
 
+// The operand A tiles of the launch's `ntok` tokens (rows tok, tok + 1, ... of x) for chunks cb .. cb + nchunks - 1, built
+// behind the table (from LDS byte AT) by the workgroup's WAVES waves (the caller synchronises afterwards).
+template <int NTOK, int WAVES, int AT = F4_LUT_BYTES>
+__device__ __forceinline__ void f4_build_tiles(const GemmArgs& a, int64_t tok, int ntok, int nchunks, int cb, int wave, int lane) {
+  constexpr int PC = f4_pieces(NTOK);
+  constexpr int F4_HI_OFF = F4Tile<PC>::HI_OFF, F4_ZERO_OFF = F4Tile<PC>::ZERO_OFF, F4_PRE_OFF = F4Tile<PC>::PRE_OFF;
+  constexpr int F4_INV_OFF = F4Tile<PC>::INV_OFF, F4_CHUNK_BYTES = F4Tile<PC>::CHUNK_BYTES;
+  auto tile_at = [](int tt, int c) { return AT + (c * NTOK + tt) * F4_CHUNK_BYTES; };
+  const bool x16 = a.x_dtype == BP_BF16 || a.x_dtype == BP_F16;
+  auto widen16 = [&](unsigned h) { return a.x_dtype == BP_BF16 ? bf16_bits_to_f32((uint16_t)h) : f16_bits_to_f32((uint16_t)h); };
   // ---- operand A tiles: a wave builds whole chunks by itself (64 byte pairs = 64 lanes; a chunk holds 5 whole scale
   // groups), so the activations are read from memory once and nothing waits for another wave until the tiles are
   // complete. Lane = byte pair: its 10 activations -> the largest magnitude of each of its (one or two) groups by an LDS
@@ -255,14 +214,16 @@ __global__ __launch_bounds__(WAVES * 64, 4) void k_tq1_gemv_fp4(GemmArgs a, int 
     }
     if (blk == 0) *(lds_u32x4*)(dst + F4_ZERO_OFF) = u32x4{0u, 0u, 0u, 0u};
   }
-  __syncthreads();
+}
 
-  // ---- this lane as a row of operand A: rows 4 g + p = piece p of group g < 4; rows 3, 7, 11 = pieces of group 4; row 15 unused
-  // (several tokens: row 4 s + 2 t + p = piece p of the pair's token t in group slot s < 3, rows 12..15 unused)
+// A lane as a row of operand A (rows 4 g + p = piece p of group g < 4; rows 3, 7, 11 = pieces of group 4; row 15 unused;
+// several tokens: row 4 s + 2 t + p = piece p of the pair's token t in group slot s < 3, rows 12..15 unused): the 16-byte
+// block (index within the chunk's part of the tile) of instruction j, half hf, in byte 2 (j % 2) + hf of aoff[j / 2].
+template <int PC>
+__device__ __forceinline__ void f4_block_offsets(int r16, int kb, unsigned (&aoff)[4]) {
+  constexpr int F4_HI_OFF = F4Tile<PC>::HI_OFF, F4_ZERO_OFF = F4Tile<PC>::ZERO_OFF;
   const int am_g = PC == 2 ? r16 >> 2 : (r16 & 3) < 3 ? r16 >> 2 : 4, am_p = PC == 2 ? r16 & 1 : (r16 & 3) < 3 ? r16 & 3 : r16 >> 2;
   const bool am_used = PC == 2 ? r16 < 12 : r16 < 15;
-  const unsigned lane_tok = PC == 2 ? (unsigned)(((r16 >> 1) & 1) * F4_CHUNK_BYTES) : 0u;  // the lane's token of a pair: its tile
-  unsigned aoff[4];  // 16-byte block (index within the chunk's part of the tile) of instruction j, half hf: byte 2 (j % 2) + hf of aoff[j / 2]
 #pragma unroll
   for (int j = 0; j < 8; ++j) {
     unsigned both = 0;
@@ -280,6 +241,74 @@ __global__ __launch_bounds__(WAVES * 64, 4) void k_tq1_gemv_fp4(GemmArgs a, int 
     if (j & 1) aoff[j >> 1] |= both << 16;
     else aoff[j >> 1] = both;
   }
+}
+
+// ABL (development): timing ablations - 1 no chunk loop, 2 no table reads, 3 no operand A reads, 4 no matrix instructions, 5 no byte extraction (and the loads are not waited for),
+// 6 bytes extracted from registers that are not loaded (no loads at all), 7 = 2 + 3 + 4 (loads and byte extraction only),
+// 8 = 7 without the byte extraction (loads and their realignment only)
+//
+// NTOK > 1: up to NTOK token rows per expert (small decode batches). Every token has its own operand A tile; the
+// packed bytes and the table reads are shared. To fit 4 tiles beside the table, an activation is then split into
+// TWO fp8 pieces (PC = 2: exact for bf16 / int8 values down to 2^-9 of their group's largest magnitude, at most
+// 2^-17 of it dropped below), and one matrix instruction serves TWO tokens: the 64-byte window (half a chunk, 320
+// digits) that instructions 0..3, and the one that instructions 4..7 multiply holds digits of only 3 groups
+// (0, 1, 2 and 2, 3, 4), so a token needs 3 group slots x 2 pieces = 6 rows instead of 10 if each window has its
+// own accumulator tile. Row 4 s + 2 t + p = piece p of token t (of the pair) in slot s; slot s is group s in the
+// first window and group 3, 4, 2 (s = 0, 1, 2) in the second, so a lane of the result (rows 4 lg + i) holds both
+// tokens' pieces of one group per window. 8 matrix instructions per chunk and token pair; with two pairs the ring
+// of loads is two chunks (registers; the loads are not what a wave then waits for).
+//
+// SR (one token, 2-byte scales): scales by the round. A scale per row and group loaded where it is applied is a wave
+// load per chunk that touches 16 memory lines for 8 bytes each: a third of the kernel's load instructions for 7 % of its
+// bytes. Instead a wave loads, once per round of the ring (4 chunks = 20 groups = 40 bytes of a row's scales), 16 bytes
+// per lane (quarters 0..2 of a row's four lanes cover 48 bytes), a round ahead and unconditionally - so the compiler's
+// count of loads in flight stays exact - parks them in a private 1.25 KiB slot of LDS at the start of the round, and a
+// chunk's two scales per lane are two 2-byte LDS reads.
+template <int SDT, int WAVES, int ABL = 0, int NTOK = 1, int SR = 0>
+__global__ __launch_bounds__(WAVES * 64, 4) void k_tq1_gemv_fp4(GemmArgs a, int total_chunks, int first_chunk, int nchunks, int bpw /* row blocks per workgroup */, int first_row) {
+  static_assert(!SR || (SDT != BP_F32 && F4_GR == 1), "scales by the round: one tile per wave, 2-byte scales (a round of 2 or 4 chunks is 20 or 40 bytes of a row's scales)");
+  constexpr int THREADS = WAVES * 64, GR = F4_GR, RD = NTOK <= 2 ? F4_RD : 2, BD = F4_BD, AD = F4_AD, PAIRS = NTOK <= 2 ? F4_PAIRS : 0;
+  static_assert(!PAIRS || RD % 2 == 0, "pairs of chunks need an even ring");
+  static_assert(NTOK == 1 || (GR == 1 && AD == 0 && NTOK % 2 == 0), "several tokens: one tile per wave, one operand A buffer, token pairs");
+  constexpr int NP = NTOK / 2;               // token pairs
+  constexpr int PC = f4_pieces(NTOK);        // fp8 pieces per activation
+  constexpr int F4_INV_OFF = F4Tile<PC>::INV_OFF, F4_CHUNK_BYTES = F4Tile<PC>::CHUNK_BYTES;
+  constexpr int AT = F4_LUT_BYTES;           // the operand A tiles (one per token) start after the table
+  constexpr int SB = SDT == BP_F32 ? 4 : 2;  // bytes per scale
+
+  const int wave = __builtin_amdgcn_readfirstlane((int)(threadIdx.x >> 6)), lane = threadIdx.x & 63;
+  const int r16 = lane & 15, kb = lane >> 4;
+  const int64_t e = blockIdx.y;
+  const int64_t o0 = clamp_i64(a.offsets[e], 0, a.T), o1 = clamp_i64(a.offsets[e + 1], 0, a.T);
+  // A launch takes the expert's token rows first_row .. first_row + NTOK - 1 (one token: its first row); an expert with
+  // more rows than that gets further launches, one without any in this range is done at once (uniform).
+  const int64_t tok = o0 + (NTOK == 1 ? 0 : first_row);
+  if (tok >= o1) return;
+  const int ntok = o1 - tok < NTOK ? (int)(o1 - tok) : NTOK;
+  const int npairs = (ntok + 1) >> 1;  // token pairs the expert has in this launch: the others' matrix instructions are left out
+  float xsc[NTOK];  // int8 activations: the tokens' scales
+#pragma unroll
+  for (int tt = 0; tt < NTOK; ++tt) xsc[tt] = a.x_dtype == BP_I8 && tt < ntok ? a.x_scale[tok + tt] : 1.f;
+  // the tiles of the NTOK tokens are interleaved chunk by chunk (a pair's tiles are a constant apart)
+  auto tile_at = [](int tt, int c) { return AT + (c * NTOK + tt) * F4_CHUNK_BYTES; };
+  const int gs = a.group == 256 ? 1 : 0;  // scale groups of 256: two 128-wide work groups share a scale
+
+  f4_build_table<THREADS>();
+  // A launch covers the chunks first_chunk .. first_chunk + nchunks - 1 of every row (all of them unless the tokens'
+  // tiles of all chunks do not fit in LDS: then the host launches once per segment of K, and the output takes the
+  // segments' partial sums one launch after the other). Chunk c below is chunk cb + c of the rows.
+  const int cb = NTOK == 1 ? 0 : first_chunk;
+  // The last bytes of a chunk are completed from the first dword of the chunk after it (rows start at any byte). At
+  // the end of a row that dword meets activations that are 0; at the end of a segment it is needed, so the chunk
+  // after a segment that is not the last one is loaded as well.
+  const int last_load = NTOK > 1 && cb + nchunks < total_chunks ? nchunks : nchunks - 1;
+
+  f4_build_tiles<NTOK, WAVES>(a, tok, ntok, nchunks, cb, wave, lane);
+  __syncthreads();
+
+  const unsigned lane_tok = PC == 2 ? (unsigned)(((r16 >> 1) & 1) * F4_CHUNK_BYTES) : 0u;  // the lane's token of a pair: its tile
+  unsigned aoff[4];  // 16-byte block (index within the chunk's part of the tile) of instruction j, half hf: byte 2 (j % 2) + hf of aoff[j / 2]
+  f4_block_offsets<PC>(r16, kb, aoff);
   // ---- this lane as a column of the result: rows 4 kb + i of C: pieces 0..2 of group kb, and piece kb of group 4
   const float f4th = kb == 3 ? 0.f : kb == 2 ? 1.f / 256.f : 1.f;
   const unsigned lane4 = (unsigned)(lane & 31) << 2;
@@ -626,6 +655,285 @@ __global__ __launch_bounds__(WAVES * 64, 4) void k_tq1_gemv_fp4(GemmArgs a, int 
   else if (NP >= 4 && npairs == 3) all_terms(IC<(NP >= 4 ? 3 : NP)>{});
   else all_terms(IC<NP>{});
 }
+// ---- One token row per expert, the rows streamed through LDS tile by tile: "a chunk per wave" -------------------------
+//
+// The kernel above lets every wave walk along its own 16 rows: a wave load is 16 rows x 64 bytes (rows of Kp bytes start
+// at any byte, so each of the 16 pieces straddles memory lines that the wave comes back to chunks later), and operand A
+// is read from LDS once per matrix instruction - 8 x the packed bytes. Here a workgroup of 16 waves walks over tiles of
+// 16 rows together, with two kinds of waves:
+//  * loaders request a tile's 16 x Kp bytes as 4 rows x 256 bytes per wave load (a lane takes 16 bytes at a dword-aligned
+//    address; LPW loads per loader and tile, the tile's scales - 16 x G x 2 bytes, contiguous - among them), two tiles
+//    ahead, and park them in tile buffers in LDS (row n at n x pitch, shifted by the row's misalignment of 0..3 bytes);
+//  * multipliers read a tile back as the matrix instruction wants it (row n = lane % 16, the 16-byte quarters of a 64-byte
+//    window across lanes / 16, plus the dword that follows for the realignment). Wave c of a group keeps chunk c of the
+//    token's operand A in registers (8 instructions x 8 registers) and multiplies chunk c of every tile: no operand A
+//    reads in the loop. A group is nchunks multipliers and its loaders; groups walk over their own tiles (tile index =
+//    group mod groups);
+//  * a multiplier's 16 partial sums of a tile (one per row) go to LDS, and the group's first loader adds the chunks' sums
+//    in a fixed order and adds the result to the output with one atomic per row (nothing else writes the row in this
+//    launch, so the result does not depend on timing).
+// A barrier hands over two tiles (the loaders' waits for memory and the multipliers' work vary from tile to tile: the
+// fewer the meeting points, the less is waited), so there are four tile buffers: the pair that the loaders fill was
+// multiplied before the previous barrier. The tile buffers take the place of the operand A tiles once those are in
+// registers.
+constexpr int CW_WAVES = 16;
+constexpr int CW_LUT_BYTES = 256 * 256;  // byte -> 5 fp4 codes, 64 copies: entry v copy c at 256 v + 4 c
+constexpr int cw_pitch(int colblks) { return colblks * 256 + 16; }  // (+ 16: rows 4 banks apart, and room for the dword after the last window)
+constexpr int cw_colblks(int64_t Kp) { return (int)((Kp + 3 + 255) / 256); }
+constexpr int64_t cw_buffer_bytes(int64_t Kp, int64_t G) { return 16 * (int64_t)cw_pitch(cw_colblks(Kp)) + 16 * G * 2; }
+
+// LPW: wave loads of packed bytes per loader and tile; TPB: tiles per barrier
+template <int SDT, int LPW, int TPB>
+__global__ __launch_bounds__(CW_WAVES * 64) void k_tq1_gemv_cw(GemmArgs a, int nchunks, int groups, int tiles_per_wg) {
+  static_assert(SDT == BP_F16 || SDT == BP_BF16, "2-byte scales");
+  constexpr int WAVES = CW_WAVES, THREADS = WAVES * 64, NB = 2 * TPB, PC = 3, SB = 2;
+  constexpr int F4_INV_OFF = F4Tile<PC>::INV_OFF, F4_CHUNK_BYTES = F4Tile<PC>::CHUNK_BYTES, AT = CW_LUT_BYTES;
+  const int wave = __builtin_amdgcn_readfirstlane((int)(threadIdx.x >> 6)), lane = threadIdx.x & 63;
+  const int r16 = lane & 15, kb = lane >> 4;
+  const int64_t e = blockIdx.y;
+  const int64_t o0 = clamp_i64(a.offsets[e], 0, a.T), o1 = clamp_i64(a.offsets[e + 1], 0, a.T);
+  const int64_t tok = o0;
+  if (tok >= o1) return;  // (uniform: an expert without a token)
+  const float xsc = a.x_dtype == BP_I8 ? a.x_scale[tok] : 1.f;
+  const int gs = a.group == 256 ? 1 : 0;
+
+  // ---- roles (wave-uniform): multiplier of chunk c in group grp, or loader number lidx of the group's lpg loaders
+  const int active = groups * nchunks, extra = wave - active, lpg = (WAVES - active) / groups;
+  const bool multiplier = wave < active, loader = !multiplier && extra < lpg * groups;
+  const int grp = multiplier ? wave / nchunks : extra % groups;
+  const int c = multiplier ? wave - grp * nchunks : 0;
+  const int lidx = multiplier ? 0 : extra / groups;
+
+  // ---- LDS behind the table: per group NB tile buffers (16 rows at `pitch`, then the tile's scales), then the partial sums
+  const int colblks = cw_colblks(a.Kp), pitch = cw_pitch(colblks);
+  const int scb = (int)(16 * a.G * SB);  // a tile's scales: 16 rows x G entries, contiguous
+  const int buf_bytes = 16 * pitch + scb;
+  const unsigned gbase = (unsigned)(AT + grp * NB * buf_bytes);
+  const unsigned red = (unsigned)(AT + groups * NB * buf_bytes + grp * NB * nchunks * 64);  // [tile % NB][chunk][row]
+  const int nl = 4 * colblks, ns = (scb + 1023) >> 10;  // wave loads of a tile: packed bytes, scales
+  const int64_t tiles = a.N / 16;
+  const int64_t tile0 = (int64_t)blockIdx.x * tiles_per_wg;
+  const int64_t tile_end = tile0 + tiles_per_wg < tiles ? tile0 + tiles_per_wg : tiles;
+  const int n_iter = (tiles_per_wg + groups - 1) / groups;  // tiles of a group
+  const int n_int = (n_iter + TPB - 1) / TPB;                 // barriers: TPB tiles each
+  auto tile_of = [&](int t) -> int64_t { return tile0 + (int64_t)t * groups + grp; };
+
+  // ---- loaders: state of the current term (the expert's rows and scales as buffers of their own: a tile past N reads
+  // zeros) and the wave's loads of a tile: LPW of the nl wave loads of packed bytes (li = i * lpg + lidx: rows
+  // 4 (li % 4) .. + 3, bytes 256 (li / 4) .. + 255 of the rows' LDS images) and one of the ns wave loads of the scales
+  __amdgpu_buffer_rsrc_t wrs = make_rsrc(a.packed[0], 0), srs = wrs;
+  unsigned voff[LPW + 1], dst[LPW + 1];
+  bool put[LPW + 1];
+  u32x4 ring[2][LPW + 1];
+  auto setup_term = [&](int term) {
+    const unsigned char* expert_rows = a.packed[term] + e * a.N * a.Kp;
+    const unsigned mis = (unsigned)((uintptr_t)expert_rows & 3);
+    wrs = make_rsrc(expert_rows - mis, a.N * a.Kp + mis);
+    srs = make_rsrc((const unsigned char*)a.w_scale[term] + e * a.N * a.G * SB, a.N * a.G * SB);  // (dword-aligned: checked by the host)
+#pragma unroll
+    for (int i = 0; i <= LPW; ++i) {
+      voff[i] = 0x7ffffff0u;  // (past the buffer, also with a tile's offset added: zeros, no memory access)
+      dst[i] = 0u;
+      put[i] = false;
+    }
+#pragma unroll
+    for (int i = 0; i < LPW; ++i) {
+      const int li = i * lpg + lidx;
+      if (loader && li < nl) {
+        const int row = 4 * (li & 3) + kb, col = 256 * (li >> 2) + 16 * r16;
+        const unsigned ro = mis + (unsigned)row * (unsigned)a.Kp;
+        if (col < (int)(ro & 3u) + (int)a.Kp) voff[i] = (ro & ~3u) + (unsigned)col;
+        dst[i] = (unsigned)(row * pitch + col);
+        put[i] = true;
+      }
+    }
+    if (loader && lidx < ns && 16 * (lidx * 64 + lane) < scb) {
+      voff[LPW] = (unsigned)(16 * (lidx * 64 + lane));
+      dst[LPW] = (unsigned)(16 * pitch) + voff[LPW];
+      put[LPW] = true;
+    }
+  };
+  const unsigned step_w = (unsigned)(16 * a.Kp), step_s = (unsigned)scb;  // a tile's bytes
+  auto request = [&](int t, auto slot_c) {  // the loads of the tile of iteration t
+    constexpr int slot = decltype(slot_c)::value;
+    const int64_t tile = tile_of(t);
+    const unsigned so_w = tile < tiles ? (unsigned)tile * step_w : 0x7ffffff0u, so_s = tile < tiles ? (unsigned)tile * step_s : 0x7ffffff0u;
+#pragma unroll
+    for (int i = 0; i < LPW; ++i) ring[slot][i] = buf_load16(wrs, voff[i], so_w);
+    ring[slot][LPW] = buf_load16(srs, voff[LPW], so_s);
+  };
+  auto park = [&](int t, auto slot_c) {  // ... into the buffer of iteration t
+    constexpr int slot = decltype(slot_c)::value;
+    const unsigned wb = gbase + (unsigned)((t % NB) * buf_bytes);
+#pragma unroll
+    for (int i = 0; i <= LPW; ++i)
+      if (put[i]) *(lds_u32x4*)(wb + dst[i]) = ring[slot][i];
+  };
+  // A loader has few instructions per tile and everything waits for them: they go before those of the multipliers on
+  // its SIMD. The first term's first two tiles are requested before the table and the token's tile are built.
+  if (!multiplier) {
+    __builtin_amdgcn_s_setprio(3);
+    setup_term(0);
+    request(0, IC<0>{});
+    request(1, IC<1>{});
+  } else {
+    f4_build_tiles<1, WAVES, AT>(a, tok, 1, nchunks, 0, wave, lane);  // (chunk by chunk by the waves 0 .. nchunks - 1: multipliers)
+  }
+
+  // ---- the byte table, one copy per lane (64 banks: no two lanes of a wave share one): entry v = digits d0..d4 of v as
+  // fp4 codes in nibbles 0..4, at 256 v + 4 lane - an address that one byte permute makes from a packed byte and 4 lane
+  for (int idx = threadIdx.x; idx < 256 * 16; idx += THREADS) {
+    unsigned v = (unsigned)idx >> 4, ent = 0;
+    if (v < 243) {
+#pragma unroll
+      for (int d = 0; d < 5; ++d) {
+        const unsigned q = v / 3, dig = v - 3 * q;
+        ent |= (dig == 0 ? 0xAu : dig == 2 ? 0x2u : 0u) << (4 * d);
+        v = q;
+      }
+    }
+    *(lds_u32x4*)(16 * idx) = u32x4{ent, ent, ent, ent};
+  }
+  __syncthreads();
+
+  if (multiplier) {
+    // ---- the wave's chunk of operand A, and the inverse prescales of the lane's two groups (group kb; group 4, of which
+    // the lane holds piece kb)
+    i32x8 A[8];
+    float inv_a, inv_4;
+    {
+      unsigned aoff[4];
+      f4_block_offsets<PC>(r16, kb, aoff);
+      const unsigned cbase = (unsigned)(AT + c * F4_CHUNK_BYTES);
+#pragma unroll
+      for (int j = 0; j < 8; ++j) {
+        const u32x4 lo = *(const lds_u32x4*)((((aoff[j >> 1] >> (16 * (j & 1))) & 0xffu) << 4) + cbase);
+        const u32x4 hi = *(const lds_u32x4*)((((aoff[j >> 1] >> (16 * (j & 1) + 8)) & 0xffu) << 4) + cbase);
+        A[j] = i32x8{(int)lo.x, (int)lo.y, (int)lo.z, (int)lo.w, (int)hi.x, (int)hi.y, (int)hi.z, (int)hi.w};
+      }
+      const float f4th = kb == 3 ? 0.f : kb == 2 ? 1.f / 256.f : 1.f;
+      inv_a = __uint_as_float(*(const lds_u32*)(cbase + F4_INV_OFF + 4 * kb));
+      inv_4 = __uint_as_float(*(const lds_u32*)(cbase + F4_INV_OFF + 16)) * f4th;
+    }
+    const unsigned lane4 = (unsigned)lane << 2;
+    // the lane's reads of a tile: its row's window of chunk c, and the scales of its two groups (an index past the row's
+    // last group - the last chunk of a row - meets sums that are 0 and takes the last group's scale)
+    const unsigned rd_w = (unsigned)(r16 * pitch + 128 * c + 16 * kb);
+    const int64_t g_last = a.G - 1;
+    const int64_t ga = (5 * (int64_t)c + kb) >> gs, gb = (5 * (int64_t)c + 4) >> gs;
+    const unsigned rd_sa = (unsigned)(16 * pitch + r16 * (int)(a.G * SB) + SB * (int)(ga < g_last ? ga : g_last));
+    const unsigned rd_sb = (unsigned)(16 * pitch + r16 * (int)(a.G * SB) + SB * (int)(gb < g_last ? gb : g_last));
+    __syncthreads();  // (every multiplier has its operand A: the tile buffers may overwrite the tiles)
+
+    for (int term = 0; term < a.n_terms; ++term) {
+      const unsigned mis = (unsigned)((uintptr_t)(a.packed[term] + e * a.N * a.Kp) & 3);
+      const unsigned dlt = (mis + (unsigned)r16 * (unsigned)a.Kp) & 3u;  // the lane's row starts dlt bytes into its LDS row
+      auto multiply = [&](int t) {
+        const unsigned rb = gbase + (unsigned)((t % NB) * buf_bytes);
+        const u32x4 W0 = *(const lds_u32x4*)(rb + rd_w), W1 = *(const lds_u32x4*)(rb + rd_w + 64);
+        const unsigned x0 = *(const lds_u32*)(rb + rd_w + 16), x1 = *(const lds_u32*)(rb + rd_w + 80);
+        const unsigned ra = *(const lds_u16*)(rb + rd_sa), rbits = *(const lds_u16*)(rb + rd_sb);
+        // the table reads run BD instructions ahead of the matrix instructions (the scheduling barriers keep the compiler
+        // from sinking them back to their uses: a wave would wait out an LDS round trip per instruction)
+        constexpr int BD = 2;
+        u32x4 Bq[BD + 1];
+        auto lookup = [&](auto j_c) {
+          constexpr int j = decltype(j_c)::value, i = j & 3;
+          const u32x4& W = j < 4 ? W0 : W1;
+          const unsigned d = __builtin_amdgcn_alignbyte(i < 3 ? W[i < 3 ? i + 1 : 0] : (j < 4 ? x0 : x1), W[i], dlt);
+#pragma unroll
+          for (int w = 0; w < 4; ++w)  // (byte 1 of the address: byte w of d; byte 0: 4 lane)
+            Bq[j % (BD + 1)][w] = *(const lds_u32*)__builtin_amdgcn_perm(d, lane4, 0x0c0c0400u + ((unsigned)w << 8));
+        };
+        f32x4 C = {0.f, 0.f, 0.f, 0.f};
+        lookup(IC<0>{});
+        lookup(IC<1>{});
+        auto stage = [&](auto j_c) {
+          constexpr int j = decltype(j_c)::value;
+          __builtin_amdgcn_sched_barrier(0);
+          if (j + BD < 8) lookup(IC<(j + BD < 8 ? j + BD : 0)>{});
+          __builtin_amdgcn_sched_barrier(0);
+          const u32x4 bq = Bq[j % (BD + 1)];
+          const i32x8 B8 = {(int)bq.x, (int)bq.y, (int)bq.z, (int)bq.w, 0, 0, 0, 0};
+          C = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(A[j], B8, C, 0 /* A: E4M3 */, 4 /* B: E2M1 */, 0, 0, 0, 0);
+        };
+        stage(IC<0>{}); stage(IC<1>{}); stage(IC<2>{}); stage(IC<3>{}); stage(IC<4>{}); stage(IC<5>{}); stage(IC<6>{}); stage(IC<7>{});
+        __builtin_amdgcn_sched_barrier(0);
+        const float sa = SDT == BP_F16 ? f16_bits_to_f32((uint16_t)ra) : __uint_as_float(ra << 16);
+        const float sb = SDT == BP_F16 ? f16_bits_to_f32((uint16_t)rbits) : __uint_as_float(rbits << 16);
+        // the row's sum over its four lanes (one per quarter): row n ends up in every lane n + 16 q
+        float v = sa * inv_a * (C[0] + C[1] + C[2] * (1.f / 256.f)) + sb * inv_4 * C[3];
+        const auto h32 = __builtin_amdgcn_permlane32_swap(__float_as_uint(v), __float_as_uint(v), false, false);
+        v = __uint_as_float(h32[0]) + __uint_as_float(h32[1]);
+        const auto h16 = __builtin_amdgcn_permlane16_swap(__float_as_uint(v), __float_as_uint(v), false, false);
+        v = __uint_as_float(h16[0]) + __uint_as_float(h16[1]);
+        if (kb == 0) *(lds_u32*)(red + (unsigned)(((t % NB) * nchunks + c) * 64 + 4 * r16)) = __float_as_uint(v);
+      };
+      __syncthreads();  // (the previous term's last tiles have been added)
+      for (int i = 0; i < n_int; ++i) {
+        __syncthreads();  // (the tiles TPB i .. TPB i + TPB - 1 are in their buffers)
+#pragma unroll
+        for (int u = 0; u < TPB; ++u) multiply(TPB * i + u);
+      }
+      __syncthreads();
+    }
+    return;
+  }
+
+  // ---- loaders (and waves without a role, which only keep the barriers' count)
+  __syncthreads();  // (the multipliers have their operand A)
+  for (int term = 0; term < a.n_terms; ++term) {
+    if (term > 0) setup_term(term);
+    // The sums of the tile of iteration t, by the group's first loader: lane (row n, quarter q) adds chunks q, q + 4, ...
+    // in that order, the row's four lanes are added in a fixed order too, and the output takes one addition per row.
+    auto reduce = [&](int t) {
+      if (!loader || lidx != 0) return;  // (uniform)
+      const int64_t tile = tile_of(t);
+      float v = 0.f;
+#pragma unroll
+      for (int q = 0; q < CW_WAVES / 4; ++q) {
+        const int ch = 4 * q + kb;
+        const unsigned at = red + (unsigned)(((t % NB) * nchunks + (ch < nchunks ? ch : 0)) * 64 + 4 * r16);
+        const float part = __uint_as_float(*(const lds_u32*)at);
+        v += ch < nchunks ? part : 0.f;
+      }
+      const auto h32 = __builtin_amdgcn_permlane32_swap(__float_as_uint(v), __float_as_uint(v), false, false);
+      v = __uint_as_float(h32[0]) + __uint_as_float(h32[1]);
+      const auto h16 = __builtin_amdgcn_permlane16_swap(__float_as_uint(v), __float_as_uint(v), false, false);
+      v = __uint_as_float(h16[0]) + __uint_as_float(h16[1]);
+      if (lane < 16 && tile < tile_end) unsafeAtomicAdd(a.out + tok * a.N + tile * 16 + lane, a.x_dtype == BP_I8 ? v * xsc : v);
+    };
+    // Two tiles are in flight per loader: the tile parked before a barrier was requested two tiles ago.
+    static_assert(TPB == 1 || TPB == 2, "tiles per barrier");
+    __syncthreads();  // (the previous term's last tiles have been multiplied)
+    if (term > 0) {
+      request(0, IC<0>{});
+      request(1, IC<1>{});
+    }
+    for (int t = 0; t < TPB * n_int; t += 2) {
+      park(t, IC<0>{});
+      request(t + 2, IC<0>{});
+      if constexpr (TPB == 1) {
+        __syncthreads();
+        if (t > 0) reduce(t - 1);  // (multiplied before this barrier)
+        if (t + 1 >= n_int) break;  // (uniform)
+      }
+      park(t + 1, IC<1>{});
+      request(t + 3, IC<1>{});
+      __syncthreads();
+      if constexpr (TPB == 1) {
+        reduce(t);
+      } else if (t > 0) {
+        reduce(t - 2);
+        reduce(t - 1);
+      }
+    }
+    __syncthreads();
+    if constexpr (TPB == 2) reduce(TPB * n_int - 2);
+    reduce(TPB * n_int - 1);
+  }
+}
+
 int f4_cus() {  // compute units of the current device (256 if the query fails); looked up once per device
   static std::mutex m;
   static int known[64] = {};
@@ -664,6 +972,64 @@ int launch_f4_k(const GemmArgs& a, hipStream_t s, const char* name, int nchunks,
   return BP_OK;
 }
 
+// Launch of the chunk-per-wave kernel, or BP_ERR_UNSUPPORTED (no message) where it does not apply: more than 15 chunks
+// per row, scales that are not dword-aligned, an expert whose rows or scales exceed a buffer descriptor, tile buffers
+// that do not fit, or a call too small for it (each workgroup builds the table and the token's tile before it streams).
+template <int SDT>
+int launch_cw(const GemmArgs& a, hipStream_t s, int64_t nchunks, int cus) {
+  const char force = tuning().tq1;
+  if (force == 'r') return BP_ERR_UNSUPPORTED;
+  for (int t = 0; t < a.n_terms; ++t)
+    if (((uintptr_t)a.w_scale[t] & 3) != 0) return BP_ERR_UNSUPPORTED;
+  if (a.N * a.Kp >= 0x7fffffe0 || a.N * a.G * 2 >= 0x7fffffe0) return BP_ERR_UNSUPPORTED;
+  const int64_t experts = a.E < a.T ? a.E : a.T, tiles = a.N / 16;
+  if (force != 'c' && experts * tiles < 16 * (int64_t)cus) return BP_ERR_UNSUPPORTED;
+  int64_t wpe = cus / experts;  // workgroups per expert: one workgroup per CU is resident
+  wpe = wpe < 1 ? 1 : wpe > tiles ? tiles : wpe;
+  int64_t per = (tiles + wpe - 1) / wpe;  // tiles per workgroup
+  const int64_t buf = cw_buffer_bytes(a.Kp, a.G);
+  const int64_t nl = 4 * cw_colblks(a.Kp), ns = (16 * a.G * 2 + 1023) / 1024;  // wave loads per tile: packed bytes, scales
+  // A group: nchunks multipliers and its loaders, which take up to 8 wave loads of packed bytes each and one of the
+  // scales. As many groups as fit the 16 waves, the tiles of a workgroup and LDS (two tiles per barrier if those fit too).
+  auto loaders_of = [&](int g) { return (CW_WAVES - g * nchunks) / g; };
+  auto lds_of = [&](int g, int tpb) {
+    const int64_t stream = (int64_t)g * 2 * tpb * (buf + nchunks * 64), build = nchunks * f4_chunk_bytes(1);
+    return (int64_t)CW_LUT_BYTES + (stream > build ? stream : build);
+  };
+  auto fits = [&](int g, int tpb) {
+    const int64_t l = loaders_of(g);
+    return l >= 1 && l >= ns && (nl + l - 1) / l <= 8 && lds_of(g, tpb) <= F4_LDS_MAX;
+  };
+  int groups = (int)(CW_WAVES / (nchunks + 1));
+  if (groups > per) groups = (int)per;
+  while (groups > 1 && !fits(groups, 1)) --groups;
+  if (groups < 1 || !fits(groups, 1)) return BP_ERR_UNSUPPORTED;
+  const int tpb = fits(groups, 2) ? 2 : 1;
+  const int64_t loaders = loaders_of(groups), lpw = (nl + loaders - 1) / loaders;
+  per = (per + groups - 1) / groups * groups;
+  // Measured against the kernel above (E x N x K from 64 x 4096 x 2048 to 256 x 2048 x 7168): ahead by 3 - 12 % with 10 or
+  // more multipliers and 48 or more tiles per group, behind with fewer of either (7 multipliers at K = 4096; 21 tiles).
+  if (force != 'c' && (groups * nchunks < 10 || per / groups < 48)) return BP_ERR_UNSUPPORTED;
+  const dim3 grid((unsigned)((tiles + per - 1) / per), (unsigned)a.E, 1u);
+  const size_t lds = (size_t)lds_of(groups, tpb);
+  note_kernel("fp4_tq1_t1_cw");
+#define BP_CW_LAUNCH(L, P)                                                                                                \
+  {                                                                                                                       \
+    if (const int rc = raise_lds_limit<k_tq1_gemv_cw<SDT, L, P>>(F4_LDS_MAX)) return rc;                                  \
+    hipLaunchKernelGGL((k_tq1_gemv_cw<SDT, L, P>), grid, dim3(CW_WAVES * 64), lds, s, a, (int)nchunks, groups, (int)per); \
+    return check_launch("fp4_tq1_t1_cw");                                                                                 \
+  }
+#define BP_CW_LPW(L)        \
+  if (lpw == L) {           \
+    if (tpb == 2) BP_CW_LAUNCH(L, 2) \
+    BP_CW_LAUNCH(L, 1)      \
+  }
+  BP_CW_LPW(1) BP_CW_LPW(2) BP_CW_LPW(3) BP_CW_LPW(4) BP_CW_LPW(5) BP_CW_LPW(6) BP_CW_LPW(7) BP_CW_LPW(8)
+#undef BP_CW_LPW
+#undef BP_CW_LAUNCH
+  return BP_ERR_UNSUPPORTED;
+}
+
 template <int SDT, int NTOK>
 int launch_f4(const GemmArgs& a, hipStream_t s, int first_row = 0) {
   const int64_t nchunks = (a.K + 639) / 640;
@@ -687,6 +1053,10 @@ int launch_f4(const GemmArgs& a, hipStream_t s, int first_row = 0) {
     }
     if (sr_ok && lds + 16 * F4_SCALE_SLOT <= (size_t)F4_LDS_MAX) return launch_f4_k<SDT, 16, 0, NTOK, SRV>(a, s, name16, (int)nchunks, lds, (int)seg, first_row);
     return launch_f4_k<SDT, 16, 0, NTOK>(a, s, name16, (int)nchunks, lds, (int)seg, first_row);
+  }
+  if constexpr (SDT != BP_F32) {
+    const int rc = launch_cw<SDT>(a, s, nchunks, cus);
+    if (rc != BP_ERR_UNSUPPORTED) return rc;
   }
 #ifdef BP_DEV_ABLATIONS  // timing ablations (results are wrong): development builds only
   if (const char* t = getenv("BP_TUNE_F4ABL")) {

@@ -1,4 +1,4 @@
-"""The benchmark configurations 2, 3 and 4 at their full shapes on the device. The whole oracle product at these sizes would take
+"""The benchmark configurations 1 (the decode launch), 2, 3 and 4 at their full shapes on the device. The whole oracle product at these sizes would take
 minutes on the host, so every launch is checked on samples against the float64 dense evaluation (weights decoded by the
 bit-exact unpack kernel and evaluated on the host) and through size-independent properties (linearity on integer
 inputs, unit-vector read-out)."""
@@ -50,6 +50,33 @@ def _dense_rows(bp, packed, scales, e, rows, K, fmt):
         d = t * np.repeat(s[e][idx].cpu().numpy().astype(np.float64), GROUP, axis=1)
         w = d if w is None else w + d
     return w
+
+
+def test_config1_decode_gemv_full_size():
+    """E = 256 experts, N = 2048, K = 7168, TQ1, one token per expert: the launch bench.py times by default, on the kernel
+    chosen without a switch (rows streamed through LDS tile by tile). Sampled experts against the oracle, all rows; a
+    second call adds to the first one's output (the contract: out += ...)."""
+    import deepseekternarized_amd as bp
+    from _util import c_gemm
+
+    E, N, K, fmt = 256, 2048, 7168, "tq1"
+    packed, scales = _weights(bp, E, N, K, fmt, 1, seed=11)
+    g = torch.Generator(device="cuda").manual_seed(12)
+    x = torch.randn(E, K, device="cuda", generator=g).to(torch.bfloat16)
+    offsets = torch.arange(E + 1, device="cuda", dtype=torch.int64)
+    got = bp.grouped_ternary_gemm(x, None, offsets, packed, scales, K, GROUP, fmt, max_rows=1)
+    assert bp.ext().last_kernel() == "fp4_tq1_t1_cw", bp.ext().last_kernel()
+    assert torch.isfinite(got).all()
+    xh = x.float().cpu().numpy()
+    rng = np.random.default_rng(13)
+    for e in sorted({0, 1, 127, 128, 254, 255, *rng.choice(E, 6, replace=False).tolist()}):
+        want = np.zeros((1, N), np.float32)
+        c_gemm(xh[e:e + 1], None, packed[0][e].cpu().numpy(), scales[0][e].float().cpu().numpy(), K, GROUP, fmt, out=want)
+        assert rel_l2(got[e:e + 1].cpu().numpy(), want) <= REL_L2, (e, rel_l2(got[e:e + 1].cpu().numpy(), want))
+    ext = bp.ext()
+    twice = got.clone()
+    ext.ternary_grouped_gemm(twice, x, None, offsets, packed, scales, K, GROUP, 1, None, 1)
+    assert torch.equal(twice, got + got)  # (x + x is exact)
 
 
 def test_config3_grouped_gemm_full_size():

@@ -93,12 +93,15 @@ def _check(got, want):
 
 
 # --------------------------------------------------------------------------- TQ1 decode GEMV
-# Two kernels: fp8 x fp4 matrix instructions (16-bit and int8 activations, tables that fit in LDS) and the table
-# lookup of partial sums (everything else; BP_TUNE_TQ1=lut selects it for every call; the `tune` fixture makes the library read the switch again).
-@pytest.fixture(params=["fp4", "lut"])
+# Three kernels: fp8 x fp4 matrix instructions with every wave walking along its own rows (16-bit and int8 activations,
+# tables that fit in LDS), the same instructions with the rows streamed through LDS tile by tile and a chunk of the
+# token's operand per wave (large calls; BP_TUNE_TQ1=chunk selects it wherever it can run, =rows never), and the table
+# lookup of partial sums (everything else; BP_TUNE_TQ1=lut selects it for every call; the `tune` fixture makes the
+# library read the switch again).
+@pytest.fixture(params=["fp4", "chunk", "lut"])
 def gemv_kernel(request, tune):
-    tune("BP_TUNE_TQ1", "lut" if request.param == "lut" else None)
-    return request.param + "_tq1"
+    tune("BP_TUNE_TQ1", {"fp4": "rows", "chunk": "chunk", "lut": "lut"}[request.param])
+    return "lut_tq1" if request.param == "lut" else "fp4_tq1"
 
 
 @pytest.mark.parametrize("K", [1024, 1280, 2048, 4352, 7168])  # Kp = 205 (odd: rows at every byte alignment), 256, 410, 871, 1434
@@ -120,6 +123,41 @@ def test_tq1_gemv_many_rows_two_terms_bf16_scales(bp, gemv_kernel):
     """N spans several workgroups and is not a multiple of their rows; two stacked terms; bf16 scales."""
     got, want, kern = _run(bp, "tq1", 2, 2048 + 48, 2304, [1, 1], "bf16", terms=2, seed=5, scale_dtype=np.float32)
     assert kern.startswith(gemv_kernel), kern
+    _check(got, want)
+
+
+@pytest.mark.parametrize("K,counts,act,N", [(1024, [1, 0, 1], "bf16", 48),      # Kp = 205: rows at every byte alignment; 2 chunks, 5 groups of waves
+                                           (1280, [1, 1], "int8", 2048 + 16),   # Kp = 256; N not a multiple of a workgroup's tiles
+                                           (4352, [0, 1, 1], "f16", 80),        # 7 chunks: one group, 9 loaders
+                                           (7168, [1, 1, 1], "bf16", 2048),     # 12 chunks, 4 loaders: the decode shape
+                                           (7680, [1, 1], "int8", 96)])         # 12 chunks of rows of 1536 bytes: 7 wave loads per loader
+def test_tq1_gemv_chunk_per_wave(bp, tune, K, counts, act, N):
+    """The kernel that streams the rows through LDS tile by tile: every split of the 16 waves into groups, multipliers
+    and loaders; odd and even row lengths; empty experts; the token's tile aliasing the tile buffers."""
+    tune("BP_TUNE_TQ1", "chunk")
+    got, want, kern = _run(bp, "tq1", len(counts), N, K, counts, act, seed=K + 1)
+    assert kern == "fp4_tq1_t1_cw", kern
+    _check(got, want)
+
+
+def test_tq1_gemv_chunk_per_wave_terms_scales_groups(bp, tune):
+    """Two stacked terms with bf16 scales (the second term adds to the first one's output), scale groups of 256, and
+    the calls it leaves to the other kernels: float32 scales, scales that are not dword-aligned, 16 chunks or more."""
+    tune("BP_TUNE_TQ1", "chunk")
+    got, want, kern = _run(bp, "tq1", 2, 2048 + 48, 2304, [1, 1], "bf16", terms=2, seed=5, scale_dtype=np.float32)
+    assert kern == "fp4_tq1_t1_cw", kern
+    _check(got, want)
+    got, want, kern = _run(bp, "tq1", 3, 272, 2560, [1, 1, 1], "bf16", terms=2, seed=9, group=256)
+    assert kern == "fp4_tq1_t1_cw", kern
+    _check(got, want)
+    got, want, kern = _run(bp, "tq1", 2, 64, 2048, [1, 1], "bf16", seed=10, scale_dtype="f32")
+    assert kern.startswith("fp4_tq1_t1_w"), kern
+    _check(got, want)
+    got, want, kern = _run(bp, "tq1", 1, 272, 10240, [1], "bf16", seed=12)  # 16 chunks: no wave left for the loads
+    assert kern.startswith("fp4_tq1_t1_w"), kern
+    _check(got, want)
+    got, want, kern = _run(bp, "tq1", 2, 96, 9472, [1, 1], "int8", seed=13)  # 15 chunks: one loader, three wave loads of scales
+    assert kern.startswith("fp4_tq1_t1_w"), kern
     _check(got, want)
 
 
