@@ -670,8 +670,7 @@ __global__ __launch_bounds__(WAVES * 64, 4) void k_tq1_gemv_fp4(GemmArgs a, int 
 //    reads in the loop. A group is nchunks multipliers and its loaders; groups walk over their own tiles (tile index =
 //    group mod groups);
 //  * a multiplier's 16 partial sums of a tile (one per row) go to LDS, and the group's first loader adds the chunks' sums
-//    in a fixed order and adds the result to the output with one atomic per row (nothing else writes the row in this
-//    launch, so the result does not depend on timing).
+//    in a fixed order and adds the result to the output (read a barrier earlier).
 // A barrier hands over two tiles (the loaders' waits for memory and the multipliers' work vary from tile to tile: the
 // fewer the meeting points, the less is waited), so there are four tile buffers: the pair that the loaders fill was
 // multiplied before the previous barrier. The tile buffers take the place of the operand A tiles once those are in
@@ -720,54 +719,47 @@ __global__ __launch_bounds__(CW_WAVES * 64) void k_tq1_gemv_cw(GemmArgs a, int n
 
   // ---- loaders: state of the current term (the expert's rows and scales as buffers of their own: a tile past N reads
   // zeros) and the wave's loads of a tile: LPW of the nl wave loads of packed bytes (li = i * lpg + lidx: rows
-  // 4 (li % 4) .. + 3, bytes 256 (li / 4) .. + 255 of the rows' LDS images) and one of the ns wave loads of the scales
+  // 4 (li % 4) .. + 3, bytes 256 (li / 4) .. + 255 of the rows' LDS images; what depends on li is uniform and goes into
+  // the loads' scalar offsets, so one lane offset serves all of them) and one of the ns wave loads of the scales
   __amdgpu_buffer_rsrc_t wrs = make_rsrc(a.packed[0], 0), srs = wrs;
-  unsigned voff[LPW + 1], dst[LPW + 1];
-  bool put[LPW + 1];
+  unsigned w_lane = 0, w_last = 0, s_lane = 0x7ffffff0u;  // lane offsets of the loads (past the buffer: zeros, no memory access)
+  const unsigned d_lane = (unsigned)(kb * pitch + 16 * r16), ds_lane = (unsigned)(16 * pitch + 16 * (lidx * 64 + lane));
+  const bool put_s = loader && lidx < ns && 16 * (lidx * 64 + lane) < scb;
   u32x4 ring[2][LPW + 1];
+  auto slot_li = [&](int i) { return i * lpg + lidx; };
   auto setup_term = [&](int term) {
     const unsigned char* expert_rows = a.packed[term] + e * a.N * a.Kp;
     const unsigned mis = (unsigned)((uintptr_t)expert_rows & 3);
     wrs = make_rsrc(expert_rows - mis, a.N * a.Kp + mis);
     srs = make_rsrc((const unsigned char*)a.w_scale[term] + e * a.N * a.G * SB, a.N * a.G * SB);  // (dword-aligned: checked by the host)
-#pragma unroll
-    for (int i = 0; i <= LPW; ++i) {
-      voff[i] = 0x7ffffff0u;  // (past the buffer, also with a tile's offset added: zeros, no memory access)
-      dst[i] = 0u;
-      put[i] = false;
-    }
-#pragma unroll
-    for (int i = 0; i < LPW; ++i) {
-      const int li = i * lpg + lidx;
-      if (loader && li < nl) {
-        const int row = 4 * (li & 3) + kb, col = 256 * (li >> 2) + 16 * r16;
-        const unsigned ro = mis + (unsigned)row * (unsigned)a.Kp;
-        if (col < (int)(ro & 3u) + (int)a.Kp) voff[i] = (ro & ~3u) + (unsigned)col;
-        dst[i] = (unsigned)(row * pitch + col);
-        put[i] = true;
-      }
-    }
-    if (loader && lidx < ns && 16 * (lidx * 64 + lane) < scb) {
-      voff[LPW] = (unsigned)(16 * (lidx * 64 + lane));
-      dst[LPW] = (unsigned)(16 * pitch) + voff[LPW];
-      put[LPW] = true;
-    }
+    const unsigned ro = mis + (unsigned)kb * (unsigned)a.Kp;
+    w_lane = (ro & ~3u) + 16u * (unsigned)r16;  // (rows 4 apart are a multiple of 4 bytes apart)
+    // (the last block of 256 bytes: only the pieces that hold bytes of the row)
+    w_last = 256 * (colblks - 1) + 16 * r16 < (int)(ro & 3u) + (int)a.Kp ? w_lane : 0x7ffffff0u;
+    s_lane = put_s ? (unsigned)(16 * (lidx * 64 + lane)) : 0x7ffffff0u;
   };
   const unsigned step_w = (unsigned)(16 * a.Kp), step_s = (unsigned)scb;  // a tile's bytes
   auto request = [&](int t, auto slot_c) {  // the loads of the tile of iteration t
     constexpr int slot = decltype(slot_c)::value;
     const int64_t tile = tile_of(t);
-    const unsigned so_w = tile < tiles ? (unsigned)tile * step_w : 0x7ffffff0u, so_s = tile < tiles ? (unsigned)tile * step_s : 0x7ffffff0u;
+    const bool live = loader && tile < tiles;
 #pragma unroll
-    for (int i = 0; i < LPW; ++i) ring[slot][i] = buf_load16(wrs, voff[i], so_w);
-    ring[slot][LPW] = buf_load16(srs, voff[LPW], so_s);
+    for (int i = 0; i < LPW; ++i) {
+      const int li = slot_li(i);
+      const unsigned so = (unsigned)tile * step_w + (unsigned)(4 * (li & 3)) * (unsigned)a.Kp + 256u * (unsigned)(li >> 2);
+      ring[slot][i] = buf_load16(wrs, (li >> 2) == colblks - 1 ? w_last : w_lane, live && li < nl ? so : 0x7ffffff0u);
+    }
+    ring[slot][LPW] = buf_load16(srs, s_lane, live ? (unsigned)tile * step_s : 0x7ffffff0u);
   };
   auto park = [&](int t, auto slot_c) {  // ... into the buffer of iteration t
     constexpr int slot = decltype(slot_c)::value;
     const unsigned wb = gbase + (unsigned)((t % NB) * buf_bytes);
 #pragma unroll
-    for (int i = 0; i <= LPW; ++i)
-      if (put[i]) *(lds_u32x4*)(wb + dst[i]) = ring[slot][i];
+    for (int i = 0; i < LPW; ++i) {
+      const int li = slot_li(i);
+      if (loader && li < nl) *(lds_u32x4*)(wb + (unsigned)(4 * (li & 3) * pitch + 256 * (li >> 2)) + d_lane) = ring[slot][i];  // (uniform)
+    }
+    if (put_s) *(lds_u32x4*)(wb + ds_lane) = ring[slot][LPW];
   };
   // A loader has few instructions per tile and everything waits for them: they go before those of the multipliers on
   // its SIMD. The first term's first two tiles are requested before the table and the token's tile are built.
@@ -886,7 +878,19 @@ __global__ __launch_bounds__(CW_WAVES * 64) void k_tq1_gemv_cw(GemmArgs a, int n
     if (term > 0) setup_term(term);
     // The sums of the tile of iteration t, by the group's first loader: lane (row n, quarter q) adds chunks q, q + 4, ...
     // in that order, the row's four lanes are added in a fixed order too, and the output takes one addition per row.
-    auto reduce = [&](int t) {
+    // The outputs that a tile is added to are requested a barrier before they are used (device scope: with stacked terms
+    // the value may be one this wave stored a term ago), by every loader in the same place of its instruction stream
+    // (past the buffer for all but the 16 lanes that use them), so that the waits on the loads of the tiles stay exact.
+    const __amdgpu_buffer_rsrc_t ors = make_rsrc(a.out + tok * a.N, a.N * 4);
+    float before[2] = {0.f, 0.f};
+    auto request_out = [&](int t, auto slot_c) {
+      constexpr int slot = decltype(slot_c)::value;
+      const int64_t tile = tile_of(t);
+      const bool mine = loader && lidx == 0 && lane < 16 && tile < tile_end;
+      before[slot] = __uint_as_float((unsigned)__builtin_amdgcn_raw_buffer_load_b32(ors, (int)(mine ? (unsigned)(tile * 64 + 4 * lane) : 0x7ffffff0u), 0, 1 /* glc */));
+    };
+    auto reduce = [&](int t, auto slot_c) {
+      constexpr int slot = decltype(slot_c)::value;
       if (!loader || lidx != 0) return;  // (uniform)
       const int64_t tile = tile_of(t);
       float v = 0.f;
@@ -901,7 +905,7 @@ __global__ __launch_bounds__(CW_WAVES * 64) void k_tq1_gemv_cw(GemmArgs a, int n
       v = __uint_as_float(h32[0]) + __uint_as_float(h32[1]);
       const auto h16 = __builtin_amdgcn_permlane16_swap(__float_as_uint(v), __float_as_uint(v), false, false);
       v = __uint_as_float(h16[0]) + __uint_as_float(h16[1]);
-      if (lane < 16 && tile < tile_end) unsafeAtomicAdd(a.out + tok * a.N + tile * 16 + lane, a.x_dtype == BP_I8 ? v * xsc : v);
+      if (lane < 16 && tile < tile_end) a.out[tok * a.N + tile * 16 + lane] = before[slot] + (a.x_dtype == BP_I8 ? v * xsc : v);
     };
     // Two tiles are in flight per loader: the tile parked before a barrier was requested two tiles ago.
     static_assert(TPB == 1 || TPB == 2, "tiles per barrier");
@@ -915,22 +919,29 @@ __global__ __launch_bounds__(CW_WAVES * 64) void k_tq1_gemv_cw(GemmArgs a, int n
       request(t + 2, IC<0>{});
       if constexpr (TPB == 1) {
         __syncthreads();
-        if (t > 0) reduce(t - 1);  // (multiplied before this barrier)
+        if (t > 0) reduce(t - 1, IC<1>{});  // (multiplied before this barrier)
+        request_out(t, IC<0>{});
         if (t + 1 >= n_int) break;  // (uniform)
       }
       park(t + 1, IC<1>{});
       request(t + 3, IC<1>{});
       __syncthreads();
       if constexpr (TPB == 1) {
-        reduce(t);
-      } else if (t > 0) {
-        reduce(t - 2);
-        reduce(t - 1);
+        reduce(t, IC<0>{});
+        request_out(t + 1, IC<1>{});
+      } else {
+        if (t > 0) {
+          reduce(t - 2, IC<0>{});
+          reduce(t - 1, IC<1>{});
+        }
+        request_out(t, IC<0>{});
+        request_out(t + 1, IC<1>{});
       }
     }
     __syncthreads();
-    if constexpr (TPB == 2) reduce(TPB * n_int - 2);
-    reduce(TPB * n_int - 1);
+    if constexpr (TPB == 2) reduce(TPB * n_int - 2, IC<0>{});
+    if (TPB == 2 || (n_int & 1) == 0) reduce(TPB * n_int - 1, IC<1>{});
+    else reduce(n_int - 1, IC<0>{});
   }
 }
 
