@@ -222,7 +222,7 @@ __global__ __launch_bounds__(F_THREADS, 2) void k_gemm_tq2f(GemmArgs a) {
   auto request = [&](auto p_c, auto part_c) {
     constexpr int P = decltype(p_c)::value, PART = decltype(part_c)::value;
     const unsigned s = (unsigned)ls;
-    if (PART < F_RT) W[P][PART] = buf_load16(wrs, voff, wrow[PART] + 64u * s);
+    if constexpr (PART < F_RT) W[P][PART] = buf_load16(wrs, voff, wrow[PART] + 64u * s);
     if (PART == 4) {
       if (starts_block((int)s)) {  // uniform
         unsigned first;
@@ -232,7 +232,7 @@ __global__ __launch_bounds__(F_THREADS, 2) void k_gemm_tq2f(GemmArgs a) {
         for (int i = 0; i < SB / 2; ++i) sq[i] = buf_load16(srs, so == 0xfffffff0u ? so : so + 16u * i, 0u);
       }
     }
-    if (PART == 5 || PART == 6) xa[P][PART - 5] = buf_load16(xrs, 16u * threadIdx.x + 8192u * (PART - 5), (unsigned)F_FB * s);
+    if constexpr (PART == 5 || PART == 6) xa[P][PART - 5] = buf_load16(xrs, 16u * threadIdx.x + 8192u * (PART - 5), (unsigned)F_FB * s);
     if (PART == 7) xa[P][2] = buf_load16(xrs, tail_off, (unsigned)F_FB * s);
     if (PART == 8) {
       if (ls + 1 < nwin) ++ls;

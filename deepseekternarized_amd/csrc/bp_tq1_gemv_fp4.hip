@@ -115,9 +115,9 @@ __device__ __forceinline__ void f4_build_table() {
 }
 
 // The operand A tiles of the launch's `ntok` tokens (rows tok, tok + 1, ... of x) for chunks cb .. cb + nchunks - 1, built
-// behind the table (from LDS byte AT) by the workgroup's WAVES waves (the caller synchronises afterwards).
+// behind the table (from LDS byte AT) by the workgroup's first `builders` waves (the caller synchronises afterwards).
 template <int NTOK, int WAVES, int AT = F4_LUT_BYTES>
-__device__ __forceinline__ void f4_build_tiles(const GemmArgs& a, int64_t tok, int ntok, int nchunks, int cb, int wave, int lane) {
+__device__ __forceinline__ void f4_build_tiles(const GemmArgs& a, int64_t tok, int ntok, int nchunks, int cb, int wave, int lane, int builders = WAVES) {
   constexpr int PC = f4_pieces(NTOK);
   constexpr int F4_HI_OFF = F4Tile<PC>::HI_OFF, F4_ZERO_OFF = F4Tile<PC>::ZERO_OFF, F4_PRE_OFF = F4Tile<PC>::PRE_OFF;
   constexpr int F4_INV_OFF = F4Tile<PC>::INV_OFF, F4_CHUNK_BYTES = F4Tile<PC>::CHUNK_BYTES;
@@ -129,7 +129,7 @@ __device__ __forceinline__ void f4_build_tiles(const GemmArgs& a, int64_t tok, i
   // complete. Lane = byte pair: its 10 activations -> the largest magnitude of each of its (one or two) groups by an LDS
   // maximum over the float bits -> the groups' prescales 2^sh (sh brings the group's largest magnitude into [128, 256))
   // and their inverses -> 3 pieces x (first-group block, second-group block).
-  for (int item = wave; item < ntok * nchunks; item += WAVES) {
+  for (int item = wave; item < ntok * nchunks; item += builders) {  // (the waves 0 .. builders - 1 call this)
     const int tt = item / nchunks, c = item - tt * nchunks;
     const int64_t xrow = (tok + tt) * a.K;
     const int blk = lane;
@@ -681,19 +681,26 @@ constexpr int cw_pitch(int colblks) { return colblks * 256 + 16; }  // (+ 16: ro
 constexpr int cw_colblks(int64_t Kp) { return (int)((Kp + 3 + 255) / 256); }
 constexpr int64_t cw_buffer_bytes(int64_t Kp, int64_t G) { return 16 * (int64_t)cw_pitch(cw_colblks(Kp)) + 16 * G * 2; }
 
-// LPW: wave loads of packed bytes per loader and tile; TPB: tiles per barrier
-template <int SDT, int LPW, int TPB>
-__global__ __launch_bounds__(CW_WAVES * 64) void k_tq1_gemv_cw(GemmArgs a, int nchunks, int groups, int tiles_per_wg) {
+// LPW: wave loads of packed bytes per loader and tile; TPB: tiles per barrier. NTOK = 2: a pair of token rows per expert
+// (rows first_row, first_row + 1), as in the kernel above: two fp8 pieces per activation, one matrix instruction serves
+// both tokens (row 4 s + 2 t + p of operand A = piece p of token t in group slot s), an accumulator tile per 64-byte window,
+// and a multiplier's registers hold the pair's chunk (the same 8 x 8 registers).
+template <int SDT, int LPW, int TPB, int NTOK = 1>
+__global__ __launch_bounds__(CW_WAVES * 64) void k_tq1_gemv_cw(GemmArgs a, int nchunks, int groups, int tiles_per_wg, int first_row) {
   static_assert(SDT == BP_F16 || SDT == BP_BF16, "2-byte scales");
-  constexpr int WAVES = CW_WAVES, THREADS = WAVES * 64, NB = 2 * TPB, PC = 3, SB = 2;
+  static_assert(NTOK == 1 || NTOK == 2, "one token row per expert, or a pair");
+  constexpr int WAVES = CW_WAVES, THREADS = WAVES * 64, NB = 2 * TPB, PC = f4_pieces(NTOK), SB = 2;
   constexpr int F4_INV_OFF = F4Tile<PC>::INV_OFF, F4_CHUNK_BYTES = F4Tile<PC>::CHUNK_BYTES, AT = CW_LUT_BYTES;
   const int wave = __builtin_amdgcn_readfirstlane((int)(threadIdx.x >> 6)), lane = threadIdx.x & 63;
   const int r16 = lane & 15, kb = lane >> 4;
   const int64_t e = blockIdx.y;
   const int64_t o0 = clamp_i64(a.offsets[e], 0, a.T), o1 = clamp_i64(a.offsets[e + 1], 0, a.T);
-  const int64_t tok = o0;
-  if (tok >= o1) return;  // (uniform: an expert without a token)
-  const float xsc = a.x_dtype == BP_I8 ? a.x_scale[tok] : 1.f;
+  const int64_t tok = o0 + first_row;
+  if (tok >= o1) return;  // (uniform: an expert without a token row in this launch)
+  const int ntok = o1 - tok < NTOK ? (int)(o1 - tok) : NTOK;
+  float xsc[NTOK];
+#pragma unroll
+  for (int tt = 0; tt < NTOK; ++tt) xsc[tt] = a.x_dtype == BP_I8 && tt < ntok ? a.x_scale[tok + tt] : 1.f;
   const int gs = a.group == 256 ? 1 : 0;
 
   // ---- roles (wave-uniform): multiplier of chunk c in group grp, or loader number lidx of the group's lpg loaders
@@ -708,7 +715,7 @@ __global__ __launch_bounds__(CW_WAVES * 64) void k_tq1_gemv_cw(GemmArgs a, int n
   const int scb = (int)(16 * a.G * SB);  // a tile's scales: 16 rows x G entries, contiguous
   const int buf_bytes = 16 * pitch + scb;
   const unsigned gbase = (unsigned)(AT + grp * NB * buf_bytes);
-  const unsigned red = (unsigned)(AT + groups * NB * buf_bytes + grp * NB * nchunks * 64);  // [tile % NB][chunk][row]
+  const unsigned red = (unsigned)(AT + groups * NB * buf_bytes + grp * NB * nchunks * 64 * NTOK);  // [tile % NB][chunk][token][row]
   const int nl = 4 * colblks, ns = (scb + 1023) >> 10;  // wave loads of a tile: packed bytes, scales
   const int64_t tiles = a.N / 16;
   const int64_t tile0 = (int64_t)blockIdx.x * tiles_per_wg;
@@ -769,7 +776,7 @@ __global__ __launch_bounds__(CW_WAVES * 64) void k_tq1_gemv_cw(GemmArgs a, int n
     request(0, IC<0>{});
     request(1, IC<1>{});
   } else {
-    f4_build_tiles<1, WAVES, AT>(a, tok, 1, nchunks, 0, wave, lane);  // (chunk by chunk by the waves 0 .. nchunks - 1: multipliers)
+    f4_build_tiles<NTOK, WAVES, AT>(a, tok, ntok, nchunks, 0, wave, lane, active);  // (chunk by chunk, by the multipliers)
   }
 
   // ---- the byte table, one copy per lane (64 banks: no two lanes of a wave share one): entry v = digits d0..d4 of v as
@@ -789,30 +796,36 @@ __global__ __launch_bounds__(CW_WAVES * 64) void k_tq1_gemv_cw(GemmArgs a, int n
   __syncthreads();
 
   if (multiplier) {
-    // ---- the wave's chunk of operand A, and the inverse prescales of the lane's two groups (group kb; group 4, of which
-    // the lane holds piece kb)
+    // ---- the wave's chunk of operand A (a pair: the lane's token's tile), and the inverse prescales of the lane's two
+    // groups: one token: group kb and group 4, of which the lane holds piece kb; a pair: the lane's group of the first
+    // window and of the second (kb and 3, 4, 2, 2 for kb = 0..3; the lanes kb = 3 hold unused rows: their sums are 0)
     i32x8 A[8];
-    float inv_a, inv_4;
+    float inv_a[NTOK], inv_b[NTOK];
+    const int g_w0 = NTOK == 1 ? kb : kb < 3 ? kb : 2, g_w1 = NTOK == 1 ? 4 : kb == 0 ? 3 : kb == 1 ? 4 : 2;
     {
       unsigned aoff[4];
       f4_block_offsets<PC>(r16, kb, aoff);
-      const unsigned cbase = (unsigned)(AT + c * F4_CHUNK_BYTES);
+      const unsigned cbase = (unsigned)(AT + c * NTOK * F4_CHUNK_BYTES);
+      const unsigned mine = cbase + (NTOK == 2 ? (unsigned)(((r16 >> 1) & 1) * F4_CHUNK_BYTES) : 0u);
 #pragma unroll
       for (int j = 0; j < 8; ++j) {
-        const u32x4 lo = *(const lds_u32x4*)((((aoff[j >> 1] >> (16 * (j & 1))) & 0xffu) << 4) + cbase);
-        const u32x4 hi = *(const lds_u32x4*)((((aoff[j >> 1] >> (16 * (j & 1) + 8)) & 0xffu) << 4) + cbase);
+        const u32x4 lo = *(const lds_u32x4*)((((aoff[j >> 1] >> (16 * (j & 1))) & 0xffu) << 4) + mine);
+        const u32x4 hi = *(const lds_u32x4*)((((aoff[j >> 1] >> (16 * (j & 1) + 8)) & 0xffu) << 4) + mine);
         A[j] = i32x8{(int)lo.x, (int)lo.y, (int)lo.z, (int)lo.w, (int)hi.x, (int)hi.y, (int)hi.z, (int)hi.w};
       }
       const float f4th = kb == 3 ? 0.f : kb == 2 ? 1.f / 256.f : 1.f;
-      inv_a = __uint_as_float(*(const lds_u32*)(cbase + F4_INV_OFF + 4 * kb));
-      inv_4 = __uint_as_float(*(const lds_u32*)(cbase + F4_INV_OFF + 16)) * f4th;
+#pragma unroll
+      for (int tt = 0; tt < NTOK; ++tt) {
+        inv_a[tt] = __uint_as_float(*(const lds_u32*)(cbase + tt * F4_CHUNK_BYTES + F4_INV_OFF + 4 * g_w0));
+        inv_b[tt] = __uint_as_float(*(const lds_u32*)(cbase + tt * F4_CHUNK_BYTES + F4_INV_OFF + 4 * g_w1)) * (NTOK == 1 ? f4th : 1.f);
+      }
     }
     const unsigned lane4 = (unsigned)lane << 2;
     // the lane's reads of a tile: its row's window of chunk c, and the scales of its two groups (an index past the row's
     // last group - the last chunk of a row - meets sums that are 0 and takes the last group's scale)
     const unsigned rd_w = (unsigned)(r16 * pitch + 128 * c + 16 * kb);
     const int64_t g_last = a.G - 1;
-    const int64_t ga = (5 * (int64_t)c + kb) >> gs, gb = (5 * (int64_t)c + 4) >> gs;
+    const int64_t ga = (5 * (int64_t)c + g_w0) >> gs, gb = (5 * (int64_t)c + g_w1) >> gs;
     const unsigned rd_sa = (unsigned)(16 * pitch + r16 * (int)(a.G * SB) + SB * (int)(ga < g_last ? ga : g_last));
     const unsigned rd_sb = (unsigned)(16 * pitch + r16 * (int)(a.G * SB) + SB * (int)(gb < g_last ? gb : g_last));
     __syncthreads();  // (every multiplier has its operand A: the tile buffers may overwrite the tiles)
@@ -837,29 +850,40 @@ __global__ __launch_bounds__(CW_WAVES * 64) void k_tq1_gemv_cw(GemmArgs a, int n
           for (int w = 0; w < 4; ++w)  // (byte 1 of the address: byte w of d; byte 0: 4 lane)
             Bq[j % (BD + 1)][w] = *(const lds_u32*)__builtin_amdgcn_perm(d, lane4, 0x0c0c0400u + ((unsigned)w << 8));
         };
-        f32x4 C = {0.f, 0.f, 0.f, 0.f};
+        f32x4 C[NTOK];  // (a pair: one accumulator tile per window)
+#pragma unroll
+        for (int q = 0; q < NTOK; ++q) C[q] = f32x4{0.f, 0.f, 0.f, 0.f};
         lookup(IC<0>{});
         lookup(IC<1>{});
         auto stage = [&](auto j_c) {
-          constexpr int j = decltype(j_c)::value;
+          constexpr int j = decltype(j_c)::value, ci = NTOK == 1 ? 0 : j >> 2;
           __builtin_amdgcn_sched_barrier(0);
           if (j + BD < 8) lookup(IC<(j + BD < 8 ? j + BD : 0)>{});
           __builtin_amdgcn_sched_barrier(0);
           const u32x4 bq = Bq[j % (BD + 1)];
           const i32x8 B8 = {(int)bq.x, (int)bq.y, (int)bq.z, (int)bq.w, 0, 0, 0, 0};
-          C = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(A[j], B8, C, 0 /* A: E4M3 */, 4 /* B: E2M1 */, 0, 0, 0, 0);
+          C[ci] = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(A[j], B8, C[ci], 0 /* A: E4M3 */, 4 /* B: E2M1 */, 0, 0, 0, 0);
         };
         stage(IC<0>{}); stage(IC<1>{}); stage(IC<2>{}); stage(IC<3>{}); stage(IC<4>{}); stage(IC<5>{}); stage(IC<6>{}); stage(IC<7>{});
         __builtin_amdgcn_sched_barrier(0);
         const float sa = SDT == BP_F16 ? f16_bits_to_f32((uint16_t)ra) : __uint_as_float(ra << 16);
         const float sb = SDT == BP_F16 ? f16_bits_to_f32((uint16_t)rbits) : __uint_as_float(rbits << 16);
         // the row's sum over its four lanes (one per quarter): row n ends up in every lane n + 16 q
-        float v = sa * inv_a * (C[0] + C[1] + C[2] * (1.f / 256.f)) + sb * inv_4 * C[3];
-        const auto h32 = __builtin_amdgcn_permlane32_swap(__float_as_uint(v), __float_as_uint(v), false, false);
-        v = __uint_as_float(h32[0]) + __uint_as_float(h32[1]);
-        const auto h16 = __builtin_amdgcn_permlane16_swap(__float_as_uint(v), __float_as_uint(v), false, false);
-        v = __uint_as_float(h16[0]) + __uint_as_float(h16[1]);
-        if (kb == 0) *(lds_u32*)(red + (unsigned)(((t % NB) * nchunks + c) * 64 + 4 * r16)) = __float_as_uint(v);
+#pragma unroll
+        for (int tt = 0; tt < NTOK; ++tt) {
+          float v;
+          if (NTOK == 1) {
+            v = sa * inv_a[0] * (C[0][0] + C[0][1] + C[0][2] * (1.f / 256.f)) + sb * inv_b[0] * C[0][3];
+          } else {  // rows 4 kb + 2 tt + p of the two windows' tiles
+            const f32x4 c0 = C[0], c1 = C[NTOK - 1];
+            v = sa * inv_a[tt] * (tt ? c0[2] + c0[3] : c0[0] + c0[1]) + sb * inv_b[tt] * (tt ? c1[2] + c1[3] : c1[0] + c1[1]);
+          }
+          const auto h32 = __builtin_amdgcn_permlane32_swap(__float_as_uint(v), __float_as_uint(v), false, false);
+          v = __uint_as_float(h32[0]) + __uint_as_float(h32[1]);
+          const auto h16 = __builtin_amdgcn_permlane16_swap(__float_as_uint(v), __float_as_uint(v), false, false);
+          v = __uint_as_float(h16[0]) + __uint_as_float(h16[1]);
+          if (kb == 0) *(lds_u32*)(red + (unsigned)((((t % NB) * nchunks + c) * NTOK + tt) * 64 + 4 * r16)) = __float_as_uint(v);
+        }
       };
       __syncthreads();  // (the previous term's last tiles have been added)
       for (int i = 0; i < n_int; ++i) {
@@ -881,31 +905,36 @@ __global__ __launch_bounds__(CW_WAVES * 64) void k_tq1_gemv_cw(GemmArgs a, int n
     // The outputs that a tile is added to are requested a barrier before they are used (device scope: with stacked terms
     // the value may be one this wave stored a term ago), by every loader in the same place of its instruction stream
     // (past the buffer for all but the 16 lanes that use them), so that the waits on the loads of the tiles stay exact.
-    const __amdgpu_buffer_rsrc_t ors = make_rsrc(a.out + tok * a.N, a.N * 4);
-    float before[2] = {0.f, 0.f};
+    const __amdgpu_buffer_rsrc_t ors = make_rsrc(a.out + tok * a.N, (int64_t)ntok * a.N * 4);  // (the launch's token rows)
+    float before[2][NTOK];
     auto request_out = [&](int t, auto slot_c) {
       constexpr int slot = decltype(slot_c)::value;
       const int64_t tile = tile_of(t);
       const bool mine = loader && lidx == 0 && lane < 16 && tile < tile_end;
-      before[slot] = __uint_as_float((unsigned)__builtin_amdgcn_raw_buffer_load_b32(ors, (int)(mine ? (unsigned)(tile * 64 + 4 * lane) : 0x7ffffff0u), 0, 1 /* glc */));
+#pragma unroll
+      for (int tt = 0; tt < NTOK; ++tt)  // (a token row the expert does not have lies past the buffer)
+        before[slot][tt] = __uint_as_float((unsigned)__builtin_amdgcn_raw_buffer_load_b32(ors, (int)(mine ? (unsigned)(tile * 64 + 4 * lane) : 0x7ffffff0u), (int)((unsigned)tt * (unsigned)a.N * 4u), 1 /* glc */));
     };
     auto reduce = [&](int t, auto slot_c) {
       constexpr int slot = decltype(slot_c)::value;
       if (!loader || lidx != 0) return;  // (uniform)
       const int64_t tile = tile_of(t);
-      float v = 0.f;
 #pragma unroll
-      for (int q = 0; q < CW_WAVES / 4; ++q) {
-        const int ch = 4 * q + kb;
-        const unsigned at = red + (unsigned)(((t % NB) * nchunks + (ch < nchunks ? ch : 0)) * 64 + 4 * r16);
-        const float part = __uint_as_float(*(const lds_u32*)at);
-        v += ch < nchunks ? part : 0.f;
+      for (int tt = 0; tt < NTOK; ++tt) {
+        float v = 0.f;
+#pragma unroll
+        for (int q = 0; q < CW_WAVES / 4; ++q) {
+          const int ch = 4 * q + kb;
+          const unsigned at = red + (unsigned)((((t % NB) * nchunks + (ch < nchunks ? ch : 0)) * NTOK + tt) * 64 + 4 * r16);
+          const float part = __uint_as_float(*(const lds_u32*)at);
+          v += ch < nchunks ? part : 0.f;
+        }
+        const auto h32 = __builtin_amdgcn_permlane32_swap(__float_as_uint(v), __float_as_uint(v), false, false);
+        v = __uint_as_float(h32[0]) + __uint_as_float(h32[1]);
+        const auto h16 = __builtin_amdgcn_permlane16_swap(__float_as_uint(v), __float_as_uint(v), false, false);
+        v = __uint_as_float(h16[0]) + __uint_as_float(h16[1]);
+        if (lane < 16 && tile < tile_end && tt < ntok) a.out[(tok + tt) * a.N + tile * 16 + lane] = before[slot][tt] + (a.x_dtype == BP_I8 ? v * xsc[tt] : v);
       }
-      const auto h32 = __builtin_amdgcn_permlane32_swap(__float_as_uint(v), __float_as_uint(v), false, false);
-      v = __uint_as_float(h32[0]) + __uint_as_float(h32[1]);
-      const auto h16 = __builtin_amdgcn_permlane16_swap(__float_as_uint(v), __float_as_uint(v), false, false);
-      v = __uint_as_float(h16[0]) + __uint_as_float(h16[1]);
-      if (lane < 16 && tile < tile_end) a.out[tok * a.N + tile * 16 + lane] = before[slot] + (a.x_dtype == BP_I8 ? v * xsc : v);
     };
     // Two tiles are in flight per loader: the tile parked before a barrier was requested two tiles ago.
     static_assert(TPB == 1 || TPB == 2, "tiles per barrier");
@@ -986,8 +1015,8 @@ int launch_f4_k(const GemmArgs& a, hipStream_t s, const char* name, int nchunks,
 // Launch of the chunk-per-wave kernel, or BP_ERR_UNSUPPORTED (no message) where it does not apply: more than 15 chunks
 // per row, scales that are not dword-aligned, an expert whose rows or scales exceed a buffer descriptor, tile buffers
 // that do not fit, or a call too small for it (each workgroup builds the table and the token's tile before it streams).
-template <int SDT>
-int launch_cw(const GemmArgs& a, hipStream_t s, int64_t nchunks, int cus) {
+template <int SDT, int NTOK>
+int launch_cw(const GemmArgs& a, hipStream_t s, int64_t nchunks, int cus, int first_row) {
   const char force = tuning().tq1;
   if (force == 'r') return BP_ERR_UNSUPPORTED;
   for (int t = 0; t < a.n_terms; ++t)
@@ -1004,7 +1033,7 @@ int launch_cw(const GemmArgs& a, hipStream_t s, int64_t nchunks, int cus) {
   // scales. As many groups as fit the 16 waves, the tiles of a workgroup and LDS (two tiles per barrier if those fit too).
   auto loaders_of = [&](int g) { return (CW_WAVES - g * nchunks) / g; };
   auto lds_of = [&](int g, int tpb) {
-    const int64_t stream = (int64_t)g * 2 * tpb * (buf + nchunks * 64), build = nchunks * f4_chunk_bytes(1);
+    const int64_t stream = (int64_t)g * 2 * tpb * (buf + nchunks * 64 * NTOK), build = nchunks * NTOK * f4_chunk_bytes(NTOK);
     return (int64_t)CW_LUT_BYTES + (stream > build ? stream : build);
   };
   auto fits = [&](int g, int tpb) {
@@ -1023,12 +1052,12 @@ int launch_cw(const GemmArgs& a, hipStream_t s, int64_t nchunks, int cus) {
   if (force != 'c' && (groups * nchunks < 10 || per / groups < 48)) return BP_ERR_UNSUPPORTED;
   const dim3 grid((unsigned)((tiles + per - 1) / per), (unsigned)a.E, 1u);
   const size_t lds = (size_t)lds_of(groups, tpb);
-  note_kernel("fp4_tq1_t1_cw");
-#define BP_CW_LAUNCH(L, P)                                                                                                \
-  {                                                                                                                       \
-    if (const int rc = raise_lds_limit<k_tq1_gemv_cw<SDT, L, P>>(F4_LDS_MAX)) return rc;                                  \
-    hipLaunchKernelGGL((k_tq1_gemv_cw<SDT, L, P>), grid, dim3(CW_WAVES * 64), lds, s, a, (int)nchunks, groups, (int)per); \
-    return check_launch("fp4_tq1_t1_cw");                                                                                 \
+  note_kernel(NTOK == 1 ? "fp4_tq1_t1_cw" : "fp4_tq1_m2_cw");
+#define BP_CW_LAUNCH(L, P)                                                                                                                  \
+  {                                                                                                                                         \
+    if (const int rc = raise_lds_limit<k_tq1_gemv_cw<SDT, L, P, NTOK>>(F4_LDS_MAX)) return rc;                                              \
+    hipLaunchKernelGGL((k_tq1_gemv_cw<SDT, L, P, NTOK>), grid, dim3(CW_WAVES * 64), lds, s, a, (int)nchunks, groups, (int)per, first_row); \
+    return check_launch(NTOK == 1 ? "fp4_tq1_t1_cw" : "fp4_tq1_m2_cw");                                                                     \
   }
 #define BP_CW_LPW(L)        \
   if (lpw == L) {           \
@@ -1054,6 +1083,12 @@ int launch_f4(const GemmArgs& a, hipStream_t s, int first_row = 0) {
   // 2-byte scales go by the round through LDS where the slots fit behind the tiles and a row's scales start dword-aligned
   constexpr int SRV = SDT != BP_F32 && NTOK <= 4 ? 1 : 0;
   const bool sr_ok = SRV && (a.G * 2) % 4 == 0;
+  if constexpr (NTOK == 2 && SDT != BP_F32) {  // (a pair of rows per expert in a large call: the rows through LDS tile by tile)
+    if (nseg == 1) {
+      const int rc = launch_cw<SDT, 2>(a, s, nchunks, cus, first_row);
+      if (rc != BP_ERR_UNSUPPORTED) return rc;
+    }
+  }
   if (NTOK > 1) {
     const bool wide = lds > (size_t)F4_LDS_MAX / 2 || ((a.N + 255) / 256) * experts >= 4 * (int64_t)cus;
     const char* name8 = NTOK == 2 ? "fp4_tq1_m2_w8" : NTOK == 4 ? "fp4_tq1_m4_w8" : NTOK == 6 ? "fp4_tq1_m6_w8" : "fp4_tq1_m8_w8";
@@ -1066,7 +1101,7 @@ int launch_f4(const GemmArgs& a, hipStream_t s, int first_row = 0) {
     return launch_f4_k<SDT, 16, 0, NTOK>(a, s, name16, (int)nchunks, lds, (int)seg, first_row);
   }
   if constexpr (SDT != BP_F32) {
-    const int rc = launch_cw<SDT>(a, s, nchunks, cus);
+    const int rc = launch_cw<SDT, 1>(a, s, nchunks, cus, 0);
     if (rc != BP_ERR_UNSUPPORTED) return rc;
   }
 #ifdef BP_DEV_ABLATIONS  // timing ablations (results are wrong): development builds only

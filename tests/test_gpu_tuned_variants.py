@@ -161,6 +161,24 @@ def test_tq1_gemv_chunk_per_wave_terms_scales_groups(bp, tune):
     _check(got, want)
 
 
+@pytest.mark.parametrize("K,counts,act", [(1024, [2, 0, 1], "bf16"), (7168, [2, 2, 1], "int8"), (2304, [1, 2], "bf16"), (4352, [2, 2], "int8")])
+def test_tq1_gemv_chunk_per_wave_token_pairs(bp, tune, K, counts, act):
+    """The same kernel with a pair of token rows per expert (two fp8 pieces per activation, one matrix instruction for both
+    tokens): experts with two rows, one row and none; two stacked terms; N not a multiple of a workgroup's tiles."""
+    tune("BP_TUNE_TQ1", "chunk")
+    got, want, kern = _run(bp, "tq1", len(counts), 2048 + 48, K, counts, act, terms=2, seed=K + 2)
+    assert kern == "fp4_tq1_m2_cw", kern
+    _check(got, want)
+
+
+def test_tq1_gemv_chunk_per_wave_pair_after_launches_of_eight(bp, tune):
+    """Up to 10 rows per expert where most experts have few: a launch of 8 rows, then the rows 8 and 9 as a pair."""
+    tune("BP_TUNE_TQ1", "chunk")
+    got, want, kern = _run(bp, "tq1", 8, 272, 2048, [10, 1, 0, 2, 1, 0, 9, 1], "bf16", seed=17)
+    assert kern == "fp4_tq1_m2_cw", kern
+    _check(got, want)
+
+
 def test_tq1_fp4_small_batches_many_rows_bf16_scales(bp):
     """The small-batch variants over several workgroups and row blocks (N not a multiple of their rows), bf16 scales,
     int8 activations with their per-row scales."""
