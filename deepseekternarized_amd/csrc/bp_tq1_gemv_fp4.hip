@@ -671,10 +671,10 @@ __global__ __launch_bounds__(WAVES * 64, 4) void k_tq1_gemv_fp4(GemmArgs a, int 
 //    group mod groups);
 //  * a multiplier's 16 partial sums of a tile (one per row) go to LDS, and the group's first loader adds the chunks' sums
 //    in a fixed order and adds the result to the output (read a barrier earlier).
-// A barrier hands over two tiles (the loaders' waits for memory and the multipliers' work vary from tile to tile: the
-// fewer the meeting points, the less is waited), so there are four tile buffers: the pair that the loaders fill was
-// multiplied before the previous barrier. The tile buffers take the place of the operand A tiles once those are in
-// registers.
+// A barrier hands over TPB tiles: two where four tile buffers fit beside the table (the loaders' waits for memory and
+// the multipliers' work vary from tile to tile: the fewer the meeting points, the less is waited), else one with two
+// buffers. The buffers that the loaders fill were multiplied before the previous barrier. The tile buffers take the
+// place of the operand A tiles once those are in registers.
 constexpr int CW_WAVES = 16;
 constexpr int CW_LUT_BYTES = 256 * 256;  // byte -> 5 fp4 codes, 64 copies: entry v copy c at 256 v + 4 c
 constexpr int cw_pitch(int colblks) { return colblks * 256 + 16; }  // (+ 16: rows 4 banks apart, and room for the dword after the last window)
