@@ -597,7 +597,7 @@ def test_group_256(bp, act, fmt, K, counts, prefix):
 
 # --------------------------------------------------------------------------- activations that are not finite
 @pytest.mark.parametrize("fmt,counts,prefix", [
-    ("tq1", [1, 1], "fp4_tq1_t1"), ("tq1", [4, 3], "fp4_tq1_m4"), ("tq1", [20, 12], "gemm_tq1"),
+    ("tq1", [1, 1], "fp4_tq1_t1"), ("tq1", [1, 1], "fp4_tq1_t1_cw"), ("tq1", [2, 2], "fp4_tq1_m2_cw"), ("tq1", [4, 3], "fp4_tq1_m4"), ("tq1", [20, 12], "gemm_tq1"),
     ("tq2", [1, 1], "mfma_tq2"), ("tq2", [9, 16], "mfma_tq2"), ("tq2", [40, 33], "gemm_tq2_"), ("tq2", [40, 33], "gemm_tq2f_"),
 ])
 def test_non_finite_activations_never_give_finite_wrong_values(bp, tune, fmt, counts, prefix):
@@ -608,6 +608,8 @@ def test_non_finite_activations_never_give_finite_wrong_values(bp, tune, fmt, co
     E, N, K = 2, 64, 2048
     if prefix == "gemm_tq2f_":
         tune("BP_TUNE_TQ2G", "fp4")
+    if prefix.endswith("_cw"):
+        tune("BP_TUNE_TQ1", "chunk")
     rng = np.random.default_rng(5)
     packed, scales = synth_weights(17, E, N, K, GROUP, fmt)
     trits = np.stack([orc.unpack(packed[0][e], fmt, K) for e in range(E)])
