@@ -179,6 +179,26 @@ def test_tq1_gemv_chunk_per_wave_pair_after_launches_of_eight(bp, tune):
     _check(got, want)
 
 
+def test_tq1_gemv_chunk_per_wave_random_shapes(bp, tune):
+    """30 seeded random calls with one or two rows per expert (experts, rows, K, activation type, terms, scale type and
+    group size drawn at random, some experts empty): whatever kernel takes them, the oracle decides; most land on the
+    kernel under test."""
+    tune("BP_TUNE_TQ1", "chunk")
+    rng = np.random.default_rng(123)
+    on_it = 0
+    for it in range(30):
+        E, N, K = int(rng.integers(1, 7)), 16 * int(rng.integers(1, 40)), 256 * int(rng.integers(1, 31))
+        M, act, terms = int(rng.integers(1, 3)), ["bf16", "int8"][int(rng.integers(0, 2))], int(rng.integers(1, 3))
+        group = 128 if K % 512 or rng.integers(0, 2) else 256
+        counts = [int(rng.integers(0, M + 1)) for _ in range(E)]
+        counts[-1] = M
+        got, want, kern = _run(bp, "tq1", E, N, K, counts, act, terms=terms, seed=1000 + it, group=group,
+                               scale_dtype=[np.float16, np.float32][int(rng.integers(0, 2))])
+        on_it += kern.endswith("_cw")
+        assert np.isfinite(got).all() and rel_l2(got, want) <= REL_L2, (it, E, N, K, counts, act, terms, group, kern, rel_l2(got, want))
+    assert on_it >= 20, on_it
+
+
 def test_tq1_fp4_small_batches_many_rows_bf16_scales(bp):
     """The small-batch variants over several workgroups and row blocks (N not a multiple of their rows), bf16 scales,
     int8 activations with their per-row scales."""
