@@ -677,9 +677,16 @@ __global__ __launch_bounds__(WAVES * 64, 4) void k_tq1_gemv_fp4(GemmArgs a, int 
 // place of the operand A tiles once those are in registers.
 constexpr int CW_WAVES = 16;
 constexpr int CW_LUT_BYTES = 256 * 256;  // byte -> 5 fp4 codes, 64 copies: entry v copy c at 256 v + 4 c
-constexpr int cw_pitch(int colblks) { return colblks * 256 + 16; }  // (+ 16: rows 4 banks apart, and room for the dword after the last window)
-constexpr int cw_colblks(int64_t Kp) { return (int)((Kp + 3 + 255) / 256); }
-constexpr int64_t cw_buffer_bytes(int64_t Kp, int64_t G) { return 16 * (int64_t)cw_pitch(cw_colblks(Kp)) + 16 * G * 2; }
+// A row's image in a tile buffer: up to 3 bytes of misalignment, the row's Kp bytes and the dword after them, in whole
+// 16-byte pieces, at a pitch that is an odd number of pieces (16 rows: 16 different groups of 4 banks). What a
+// multiplier reads past a row's image in its last chunk (the next row's bytes, or what follows the buffer) meets
+// activations that are 0.
+constexpr int cw_pitch(int64_t Kp) {
+  const int pieces = (int)((Kp + 3 + 4 + 15) / 16);
+  return 16 * (pieces | 1);
+}
+constexpr int cw_colblks(int64_t Kp) { return (int)((Kp + 3 + 255) / 256); }  // wave loads of 4 rows x 256 bytes per 4 rows
+constexpr int64_t cw_buffer_bytes(int64_t Kp, int64_t G) { return 16 * (int64_t)cw_pitch(Kp) + 16 * G * 2; }
 
 // LPW: wave loads of packed bytes per loader and tile; TPB: tiles per barrier. NTOK = 2: a pair of token rows per expert
 // (rows first_row, first_row + 1), as in the kernel above: two fp8 pieces per activation, one matrix instruction serves
@@ -711,7 +718,7 @@ __global__ __launch_bounds__(CW_WAVES * 64) void k_tq1_gemv_cw(GemmArgs a, int n
   const int lidx = multiplier ? 0 : extra / groups;
 
   // ---- LDS behind the table: per group NB tile buffers (16 rows at `pitch`, then the tile's scales), then the partial sums
-  const int colblks = cw_colblks(a.Kp), pitch = cw_pitch(colblks);
+  const int colblks = cw_colblks(a.Kp), pitch = cw_pitch(a.Kp);
   const int scb = (int)(16 * a.G * SB);  // a tile's scales: 16 rows x G entries, contiguous
   const int buf_bytes = 16 * pitch + scb;
   const unsigned gbase = (unsigned)(AT + grp * NB * buf_bytes);
@@ -764,7 +771,9 @@ __global__ __launch_bounds__(CW_WAVES * 64) void k_tq1_gemv_cw(GemmArgs a, int n
 #pragma unroll
     for (int i = 0; i < LPW; ++i) {
       const int li = slot_li(i);
-      if (loader && li < nl) *(lds_u32x4*)(wb + (unsigned)(4 * (li & 3) * pitch + 256 * (li >> 2)) + d_lane) = ring[slot][i];  // (uniform)
+      if (loader && li < nl) {  // (uniform; in a row's last block of 256 bytes only the pieces that hold bytes of the row: the next row's image follows)
+        if ((li >> 2) < colblks - 1 || w_last != 0x7ffffff0u) *(lds_u32x4*)(wb + (unsigned)(4 * (li & 3) * pitch + 256 * (li >> 2)) + d_lane) = ring[slot][i];
+      }
     }
     if (put_s) *(lds_u32x4*)(wb + ds_lane) = ring[slot][LPW];
   };
