@@ -149,11 +149,14 @@ extern "C" size_t bp_moe_layer_workspace_bytes(int64_t T, int64_t H, int64_t I, 
   return plan(nullptr, T, H, I, E, k, act, fmt).bytes;
 }
 
-extern "C" int bp_moe_layer_bf16(void* out, const void* x, const int64_t* experts, const void* weights,
-                                 const uint8_t* const* gate_up_packed, const void* const* gate_up_scale,
-                                 const uint8_t* const* down_packed, const void* const* down_scale, int scale_dtype,
-                                 int n_terms, int64_t T, int64_t H, int64_t I, int64_t E, int64_t k, int64_t group, int fmt,
-                                 int act, void* workspace, size_t workspace_bytes, int32_t* bad, void* stream) {
+// `v4`: the rounding points of the V4 engine (boilerplate/engine/model.py:376-387, 407-422) instead of the standard
+// decoder's: float32 routing weights applied to the float32 SwiGLU product before the down projection, `limit` clamps,
+// float32 accumulation over a token's experts, output float32 or cast once to bf16 (out_dtype).
+static int moe_layer(bool v4, void* out, int out_dtype, float limit, const void* x, const int64_t* experts, const void* weights,
+                     const uint8_t* const* gate_up_packed, const void* const* gate_up_scale,
+                     const uint8_t* const* down_packed, const void* const* down_scale, int scale_dtype,
+                     int n_terms, int64_t T, int64_t H, int64_t I, int64_t E, int64_t k, int64_t group, int fmt,
+                     int act, void* workspace, size_t workspace_bytes, int32_t* bad, void* stream) {
   if (T < 0 || H <= 0 || I <= 0 || E <= 0 || E > 65535 || k <= 0 || k > 64 || k > E) return fail(BP_ERR_ARG, "invalid MoE layer dimensions (experts up to 65535, top-k up to 64)");
   if (T * k > ((int64_t)1 << 31) - 1 - 32 * E) return fail(BP_ERR_ARG, "too many routed rows for one call");
   if (fmt != BP_TQ1 && fmt != BP_TQ2) return fail(BP_ERR_ARG, "fmt must be 1 (TQ1) or 2 (TQ2)");
@@ -217,7 +220,30 @@ extern "C" int bp_moe_layer_bf16(void* out, const void* x, const int64_t* expert
     if ((rc = check_launch("tile_list")) != BP_OK) return rc;
   }
   if ((rc = gemm(p.gu, p.xg, gate_up_packed, gate_up_scale, 2 * I, H, tiles)) != BP_OK) return rc;
-  if ((rc = bp_swiglu_bf16(p.h, p.gu, p.gu + I, n, I, 2 * I, s)) != BP_OK) return rc;
+  if (v4) rc = bp_swiglu_v4(p.h, p.gu, p.gu + I, (const float*)weights, p.order, n, limit, n, I, 2 * I, s);
+  else rc = bp_swiglu_bf16(p.h, p.gu, p.gu + I, n, I, 2 * I, s);
+  if (rc != BP_OK) return rc;
   if ((rc = gemm(p.y, p.h, down_packed, down_scale, H, I, tiles)) != BP_OK) return rc;
+  if (v4) return bp_moe_combine_v4(out, out_dtype, p.y, p.inv, experts, T, k, H, s);
   return bp_moe_combine_bf16(out, p.y, p.inv, weights, experts, T, k, H, s);
+}
+
+extern "C" int bp_moe_layer_bf16(void* out, const void* x, const int64_t* experts, const void* weights,
+                                 const uint8_t* const* gate_up_packed, const void* const* gate_up_scale,
+                                 const uint8_t* const* down_packed, const void* const* down_scale, int scale_dtype,
+                                 int n_terms, int64_t T, int64_t H, int64_t I, int64_t E, int64_t k, int64_t group, int fmt,
+                                 int act, void* workspace, size_t workspace_bytes, int32_t* bad, void* stream) {
+  return moe_layer(false, out, BP_BF16, 0.f, x, experts, weights, gate_up_packed, gate_up_scale, down_packed, down_scale, scale_dtype,
+                   n_terms, T, H, I, E, k, group, fmt, act, workspace, workspace_bytes, bad, stream);
+}
+
+extern "C" int bp_moe_layer_v4(void* out, int out_dtype, const void* x, const int64_t* experts, const float* weights, float swiglu_limit,
+                               const uint8_t* const* gate_up_packed, const void* const* gate_up_scale,
+                               const uint8_t* const* down_packed, const void* const* down_scale, int scale_dtype,
+                               int n_terms, int64_t T, int64_t H, int64_t I, int64_t E, int64_t k, int64_t group, int fmt,
+                               int act, void* workspace, size_t workspace_bytes, int32_t* bad, void* stream) {
+  if (out_dtype != BP_F32 && out_dtype != BP_BF16) return fail(BP_ERR_ARG, "the layer's output is float32 or bf16");
+  if (!(swiglu_limit == swiglu_limit) || swiglu_limit < 0.f) return fail(BP_ERR_ARG, "swiglu_limit must be 0 (no clamp) or positive");
+  return moe_layer(true, out, out_dtype, swiglu_limit, x, experts, weights, gate_up_packed, gate_up_scale, down_packed, down_scale, scale_dtype,
+                   n_terms, T, H, I, E, k, group, fmt, act, workspace, workspace_bytes, bad, stream);
 }

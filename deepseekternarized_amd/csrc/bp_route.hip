@@ -251,6 +251,70 @@ __global__ __launch_bounds__(256) void k_combine(uint16_t* __restrict__ out, con
   }
 }
 
+// SwiGLU of the V4 engine's experts (boilerplate/engine/model.py:376-387): the two linears return bf16, everything after
+// them is float32 - up clamped to [-limit, limit] and gate to at most limit when limit > 0, silu(gate) * up, times the
+// routing weight of the row's (token, slot) pair - and the product is rounded to bf16 once, as w2's input.
+// Row r of the expert-ordered tensors belongs to pair order[r]; weights f32 [pairs] (NULL: no weighting, a shared expert).
+__global__ __launch_bounds__(256) void k_swiglu_v4(uint16_t* __restrict__ h, const float* __restrict__ gate, const float* __restrict__ up,
+                                                    const float* __restrict__ weights, const int64_t* __restrict__ order, int64_t pairs,
+                                                    float limit, int64_t rows, int64_t I, int64_t ld) {
+  const int64_t c = ((int64_t)blockIdx.x * 256 + threadIdx.x) * 4;
+  if (c >= I) return;
+  for (int64_t r = blockIdx.y; r < rows; r += gridDim.y) {
+    float w = 1.0f;
+    if (weights) w = weights[order ? clamp_i64(order[r], 0, pairs - 1) : r];
+    float gs[4], us[4];
+    if ((I & 3) == 0 && (ld & 3) == 0 && (((uintptr_t)gate | (uintptr_t)up) & 15) == 0) {
+      const float4 g4 = *(const float4*)(gate + r * ld + c), u4 = *(const float4*)(up + r * ld + c);
+      gs[0] = g4.x; gs[1] = g4.y; gs[2] = g4.z; gs[3] = g4.w;
+      us[0] = u4.x; us[1] = u4.y; us[2] = u4.z; us[3] = u4.w;
+    } else {
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        gs[i] = c + i < I ? gate[r * ld + c + i] : 0.f;
+        us[i] = c + i < I ? up[r * ld + c + i] : 0.f;
+      }
+    }
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      float g = round_bf16(gs[i]), u = round_bf16(us[i]);
+      if (limit > 0.f) {  // torch.clamp: a NaN stays a NaN
+        u = u < -limit ? -limit : (u > limit ? limit : u);
+        g = g > limit ? limit : g;
+      }
+      float v = (g / (1.0f + expf(-g))) * u;
+      if (weights) v = w * v;
+      if (c + i < I) h[r * I + c + i] = f32_to_bf16_bits(v);
+    }
+  }
+}
+
+// Combine of the V4 engine (boilerplate/engine/model.py:407-422): y = zeros float32; for each expert in ascending
+// order y[token] += its bf16 output (already weighted before w2). out[t] = that float32 sum (OUT_BF16: cast once).
+template <bool OUT_BF16>
+__global__ __launch_bounds__(256) void k_combine_v4(void* __restrict__ out, const float* __restrict__ y, const int64_t* __restrict__ inv,
+                                                     const int64_t* __restrict__ experts, int64_t k, int64_t H) {
+  const int64_t t = blockIdx.x;
+  __shared__ int64_t expert_of[64];
+  __shared__ int64_t row_of[64];
+  const int sl = threadIdx.x;
+  int64_t my_expert = 0;
+  if (sl < k) expert_of[sl] = my_expert = experts[t * k + sl];
+  __syncthreads();
+  if (sl < k) {
+    int rank = 0;
+    for (int j = 0; j < k; ++j) rank += (expert_of[j] < my_expert || (expert_of[j] == my_expert && j < sl)) ? 1 : 0;
+    row_of[rank] = clamp_i64(inv[t * k + sl], 0, (int64_t)gridDim.x * k - 1);
+  }
+  __syncthreads();
+  for (int64_t c = (int64_t)blockIdx.y * COMBINE_COLS + threadIdx.x; c < H && c < ((int64_t)blockIdx.y + 1) * COMBINE_COLS; c += 256) {
+    float acc = 0.f;
+    for (int s = 0; s < k; ++s) acc += round_bf16(y[row_of[s] * H + c]);
+    if (OUT_BF16) ((uint16_t*)out)[t * H + c] = f32_to_bf16_bits(acc);
+    else ((float*)out)[t * H + c] = acc;
+  }
+}
+
 // flag = 1 if an expert has more rows than `max_rows` (offsets clamped to [0, T] as the GEMM kernels clamp them)
 __global__ __launch_bounds__(256) void k_check_rows(int32_t* __restrict__ flag, const int64_t* __restrict__ offsets, int64_t E, int64_t T,
                                                     int64_t max_rows) {
@@ -351,6 +415,30 @@ extern "C" int bp_moe_combine_bf16(void* out, const float* y, const int64_t* inv
   hipLaunchKernelGGL(k_combine, dim3((unsigned)T, (unsigned)((H + COMBINE_COLS - 1) / COMBINE_COLS)), dim3(256), 0, (hipStream_t)stream, (uint16_t*)out, y, inv,
                      (const uint16_t*)w, experts, k, H);
   return check_launch("moe_combine");
+}
+
+extern "C" int bp_swiglu_v4(void* h, const float* gate, const float* up, const float* weights, const int64_t* order, int64_t pairs,
+                            float limit, int64_t rows, int64_t I, int64_t ld_in, void* stream) {
+  if (rows < 0 || I <= 0 || ld_in < I || pairs < 0) return fail(BP_ERR_ARG, "invalid SwiGLU dimensions");
+  if (rows == 0) return BP_OK;
+  if (!h || !gate || !up) return fail(BP_ERR_ARG, "null pointer");
+  if (weights && pairs == 0) return fail(BP_ERR_ARG, "routing weights without (token, slot) pairs");
+  if (!(limit == limit)) return fail(BP_ERR_ARG, "swiglu_limit is NaN");
+  const dim3 grid((unsigned)((I + 1023) / 1024), (unsigned)(rows < 65535 ? rows : 65535));
+  hipLaunchKernelGGL(k_swiglu_v4, grid, dim3(256), 0, (hipStream_t)stream, (uint16_t*)h, gate, up, weights, order, pairs, limit, rows, I, ld_in);
+  return check_launch("swiglu_v4");
+}
+
+extern "C" int bp_moe_combine_v4(void* out, int out_dtype, const float* y, const int64_t* inv, const int64_t* experts,
+                                 int64_t T, int64_t k, int64_t H, void* stream) {
+  if (T < 0 || k <= 0 || k > 64 || H <= 0 || T > 0x7fffffff) return fail(BP_ERR_ARG, "invalid combine dimensions (top-k up to 64)");
+  if (out_dtype != BP_F32 && out_dtype != BP_BF16) return fail(BP_ERR_ARG, "the combined output is float32 or bf16");
+  if (T == 0) return BP_OK;
+  if (!out || !y || !inv || !experts) return fail(BP_ERR_ARG, "null pointer");
+  const dim3 grid((unsigned)T, (unsigned)((H + COMBINE_COLS - 1) / COMBINE_COLS));
+  if (out_dtype == BP_BF16) hipLaunchKernelGGL(k_combine_v4<true>, grid, dim3(256), 0, (hipStream_t)stream, out, y, inv, experts, k, H);
+  else hipLaunchKernelGGL(k_combine_v4<false>, grid, dim3(256), 0, (hipStream_t)stream, out, y, inv, experts, k, H);
+  return check_launch("moe_combine_v4");
 }
 
 extern "C" int bp_check_max_rows(int32_t* flag, const int64_t* offsets, int64_t E, int64_t T, int64_t max_rows, void* stream) {

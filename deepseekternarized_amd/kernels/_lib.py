@@ -37,6 +37,9 @@ SIGNATURES = {
     "bp_gather_rows": (_i, [_p, _p, _p, _l, _l, _l, _l, _p]),
     "bp_swiglu_bf16": (_i, [_p, _p, _p, _l, _l, _l, _p]),
     "bp_moe_combine_bf16": (_i, [_p, _p, _p, _p, _p, _l, _l, _l, _p]),
+    "bp_swiglu_v4": (_i, [_p, _p, _p, _p, _p, _l, C.c_float, _l, _l, _l, _p]),
+    "bp_moe_combine_v4": (_i, [_p, _i, _p, _p, _p, _l, _l, _l, _p]),
+    "bp_moe_layer_v4": (_i, [_p, _i, _p, _p, _p, C.c_float, _p, _p, _p, _p, _i, _i, _l, _l, _l, _l, _l, _l, _i, _i, _p, C.c_size_t, _p, _p]),
     "bp_moe_layer_workspace_bytes": (C.c_size_t, [_l, _l, _l, _l, _l, _i, _i]),
     "bp_moe_layer_bf16": (_i, [_p, _p, _p, _p, _p, _p, _p, _p, _i, _i, _l, _l, _l, _l, _l, _l, _i, _i, _p, C.c_size_t, _p, _p]),
 }

@@ -12,6 +12,11 @@ weight):
 
 softmax / topk are torch ops (as in the reference); everything touching packed weights runs in the HIP
 kernels. bf16 activations (``act="bf16"``) or per-row int8 (``act="int8"``, Mode D default).
+
+``pattern="v4"`` runs the rounding points of the V4 engine instead (``boilerplate/engine/model.py:376-387`` ``swiglu``,
+``:407-422`` ``moe``): the caller's router hands over float32 weights and expert ids, gate / up are rounded to bf16 and
+widened again, clamped by ``swiglu_limit``, ``weights * (silu(gate) * up)`` is float32 and rounded once as the input of
+the down projection, and a token's experts are added in float32 in ascending expert order.
 """
 
 from __future__ import annotations
@@ -54,10 +59,15 @@ class TernaryMoE:
     ``gate`` / ``up`` with N = inter, K = hidden; ``down`` with N = hidden, K = inter."""
 
     def __init__(self, gate, up, down, hidden: int, inter: int, top_k: int, fmt: str, group: int,
-                 act: str = "bf16", renorm: bool = False):
+                 act: str = "bf16", renorm: bool = False, pattern: str = "standard", swiglu_limit: float = 0.0):
         _fmt_code(fmt)
         if act not in ("bf16", "int8"):
             raise ValueError(f"unknown activation mode {act!r}")
+        if pattern not in ("standard", "v4"):
+            raise ValueError(f"unknown MoE call pattern {pattern!r}")
+        if not swiglu_limit >= 0.0:
+            raise ValueError("swiglu_limit must be 0 (no clamp) or positive")
+        self.pattern, self.swiglu_limit = pattern, float(swiglu_limit)
         if not (len(gate) == len(up) == len(down)):
             raise ValueError("gate, up and down must hold the same number of stacked terms")
         self.hidden, self.inter, self.top_k, self.fmt, self.group, self.act, self.renorm = hidden, inter, top_k, fmt, group, act, renorm
@@ -88,8 +98,16 @@ class TernaryMoE:
         e = _need_ext(self.down[0][0])
         need = int(e.lib.bp_moe_layer_workspace_bytes(tokens, self.hidden, self.inter, self.n_experts, self.top_k,
                                                       _lib.BP_I8 if self.act == "int8" else _lib.BP_BF16, _fmt_code(self.fmt)))
+        device = torch.device(device)
+        if device.index is None:  # torch.device("cuda") != torch.device("cuda:0"): compare devices with their index
+            device = torch.device(device.type, torch.cuda.current_device())
         ws = getattr(self, "_ws", None)
-        if ws is None or ws.numel() < need or ws.device != torch.device(device):
+        if ws is None or ws.numel() < need or ws.device != device:
+            # A HIP graph captured by graphed() holds the address of the workspace it ran in: a workspace that is
+            # replaced stays referenced (self._ws_captured) instead of going back to the allocator under that graph.
+            if ws is not None and getattr(self, "_ws_in_graph", False):
+                self.__dict__.setdefault("_ws_captured", []).append(ws)
+                self._ws_in_graph = False
             self._ws = ws = torch.empty(need, dtype=torch.uint8, device=device)   # (reused by later calls of up to this many tokens)
         return ws
 
@@ -100,28 +118,61 @@ class TernaryMoE:
         flat = x.reshape(-1, self.hidden).to(torch.bfloat16).contiguous()
         e = _need_ext(flat)
         T = flat.size(0)
+        if self.pattern == "v4":
+            raise RuntimeError('a pattern="v4" layer takes the router\'s output: call routed(x, weights, indices)')
         values, indices = self.route(router_logits, T)
         out = torch.empty(T, self.hidden, dtype=torch.bfloat16, device=flat.device)
         if T == 0:
             return out.view(shape).to(x.dtype)
-        ws = self._workspace(T, flat.device)
+        self._launch(e, out, flat, values, indices, T)
+        return out.view(shape).to(x.dtype)
+
+    def _launch(self, e, out, flat, values, indices, T, out_dtype=None):
         import ctypes as C
+
+        ws = self._workspace(T, flat.device)
+        if torch.cuda.is_current_stream_capturing():
+            self._ws_in_graph = True
         n = len(self.down)
         arr = lambda ts: (C.c_void_p * n)(*[t.data_ptr() for t in ts])
         gp, gs = arr([p for p, _ in self.gate_up]), arr([s for _, s in self.gate_up])
         dp, ds = arr([p for p, _ in self.down]), arr([s for _, s in self.down])
         sdt = {torch.float32: _lib.BP_F32, torch.float16: _lib.BP_F16, torch.bfloat16: _lib.BP_BF16}[self.down[0][1].dtype]
+        tail = (gp, gs, dp, ds, sdt, n, T, self.hidden, self.inter, self.n_experts, self.top_k, self.group, _fmt_code(self.fmt),
+                _lib.BP_I8 if self.act == "int8" else _lib.BP_BF16, ws.data_ptr(), ws.numel(), None, _lib.stream_ptr(flat.device))
         with torch.cuda.device(flat.device):
-            _lib.check(e.lib.bp_moe_layer_bf16(
-                out.data_ptr(), flat.data_ptr(), indices.data_ptr(), values.data_ptr(), gp, gs, dp, ds, sdt, n,
-                T, self.hidden, self.inter, self.n_experts, self.top_k, self.group, _fmt_code(self.fmt),
-                _lib.BP_I8 if self.act == "int8" else _lib.BP_BF16, ws.data_ptr(), ws.numel(), None, _lib.stream_ptr(flat.device)))
-        return out.view(shape).to(x.dtype)
+            if self.pattern == "v4":
+                _lib.check(e.lib.bp_moe_layer_v4(out.data_ptr(), out_dtype, flat.data_ptr(), indices.data_ptr(), values.data_ptr(),
+                                                 self.swiglu_limit, *tail))
+            else:
+                _lib.check(e.lib.bp_moe_layer_bf16(out.data_ptr(), flat.data_ptr(), indices.data_ptr(), values.data_ptr(), *tail))
+
+    def routed(self, x: torch.Tensor, weights: torch.Tensor, indices: torch.Tensor, out_dtype: torch.dtype = torch.float32) -> torch.Tensor:
+        """The routed experts of a V4 layer (``pattern="v4"``) through ``bp_moe_layer_v4``: ``weights`` float32 [T, k] and
+        ``indices`` int64 [T, k] are the router's output (boilerplate/engine/model.py:389-405 stays with the caller, as do the
+        shared experts). Returns the float32 sum ``y`` of model.py:411-420 (``out_dtype=torch.float32``: the caller adds
+        its shared experts and casts, :421-422) or that sum cast once to bf16."""
+        if self.pattern != "v4":
+            raise RuntimeError('routed() is the entry of pattern="v4" layers')
+        if out_dtype not in (torch.float32, torch.bfloat16):
+            raise ValueError("out_dtype must be torch.float32 or torch.bfloat16")
+        shape = x.shape
+        flat = x.reshape(-1, self.hidden).to(torch.bfloat16).contiguous()
+        e = _need_ext(flat)
+        T = flat.size(0)
+        w = weights.reshape(T, self.top_k).to(torch.float32).contiguous()
+        idx = indices.reshape(T, self.top_k).to(torch.int64).contiguous()
+        out = torch.empty(T, self.hidden, dtype=out_dtype, device=flat.device)
+        if T:
+            self._launch(e, out, flat, w, idx, T, _lib.dtype_code(out_dtype))
+        return out.view(shape)
 
     def composed(self, x: torch.Tensor, router_logits: torch.Tensor) -> torch.Tensor:
         """The same layer as separate library calls (sort, gather, two grouped GEMMs, SwiGLU, combine), sizing the
         grouped launches the reference's way: beyond 64 tokens the widest expert's row count is read back to the host
         (boilerplate/kernels/ternary_cuda.py:97). Kept as the check of ``__call__`` and for callers that want the stages."""
+        if self.pattern != "standard":
+            raise RuntimeError("composed() restates the standard decoder's layer only")
         shape = x.shape
         flat = x.reshape(-1, self.hidden).to(torch.bfloat16).contiguous()
         _need_ext(flat)
@@ -150,6 +201,8 @@ class TernaryMoE:
         Any number of tokens: the layer never reads the routing back to the host."""
         if tokens < 1:
             raise ValueError("graphed() needs at least one token")
+        if self.pattern != "standard":
+            raise RuntimeError("graphed() captures the standard decoder's layer")
         self._workspace(tokens, device)
         xs = torch.zeros(tokens, self.hidden, dtype=dtype, device=device)
         ls = torch.zeros(tokens, self.n_experts, dtype=torch.float32, device=device)
@@ -171,5 +224,6 @@ class TernaryMoE:
             return out
 
         run.graph = graph  # keeps the graph (and its memory pool) alive with the callable
+        run.workspace = self._ws  # ... and the workspace whose address the captured launches hold
         return run
 

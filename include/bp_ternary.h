@@ -185,6 +185,23 @@ int bp_swiglu_bf16(void* h, const float* gate, const float* up, int64_t rows, in
 int bp_moe_combine_bf16(void* out, const float* y, const int64_t* inv, const void* w, const int64_t* experts,
                         int64_t T, int64_t k, int64_t H, void* stream);
 
+/* SwiGLU of the V4 engine's expert MLP (boilerplate/engine/model.py:376-387, `swiglu`): the two linears return bf16,
+ * then everything is float32: up clamped to [-limit, limit] and gate to at most limit (limit > 0; 0 = no clamp),
+ * silu(gate) * up, times the routing weight when there is one, rounded to bf16 once (the input of w2).
+ *   h        device bf16 [rows, I]
+ *   gate, up device f32 GEMM outputs, row stride ld_in
+ *   weights  device f32 [pairs] routing weights of the (token, slot) pairs, or NULL (a shared expert: no weighting)
+ *   order    device i64 [rows]: row r belongs to pair order[r] (bp_sort_by_expert's order), or NULL (row r = pair r) */
+int bp_swiglu_v4(void* h, const float* gate, const float* up, const float* weights, const int64_t* order, int64_t pairs,
+                 float limit, int64_t rows, int64_t I, int64_t ld_in, void* stream);
+
+/* Combine of the V4 engine's routed experts (boilerplate/engine/model.py:411-420: `y = zeros(float32)`, then for each
+ * expert in ascending order `y[idx] += swiglu(...)`, whose results are bf16 and already weighted):
+ * out[token, :] = float32 sum over the token's slots, in ascending expert order, of bf16(y[pos, :]);
+ * out f32 [T, H] (the caller adds its shared experts and casts, model.py:421-422) or bf16 [T, H] (cast once here). */
+int bp_moe_combine_v4(void* out, int out_dtype, const float* y, const int64_t* inv, const int64_t* experts,
+                      int64_t T, int64_t k, int64_t H, void* stream);
+
 /* One routed-expert MoE layer after the router's top-k (the per-expert loop of boilerplate/engine/standard.py:156-176,
  * whose experts are TernaryLinear triples, engine/standard.py:37-41 and 151-154): for every (token, slot)
  *   y = down(bf16(bf16(silu(bf16 gate(x))) * bf16 up(x))) * weights[token, slot]       (each linear rounded to bf16)
@@ -208,6 +225,19 @@ int bp_moe_layer_bf16(void* out, const void* x, const int64_t* experts, const vo
                       const uint8_t* const* down_packed, const void* const* down_scale, int scale_dtype,
                       int n_terms, int64_t T, int64_t H, int64_t I, int64_t E, int64_t k, int64_t group, int fmt,
                       int act, void* workspace, size_t workspace_bytes, int32_t* bad, void* stream);
+
+/* The same layer with the rounding points of the V4 engine (boilerplate/engine/model.py:376-387 `swiglu`, 407-422 `moe`):
+ *   h = bf16(weights[token, slot] * (silu(clamp(float(bf16 gate(x)))) * clamp(float(bf16 up(x)))))   (float32 until the cast)
+ *   out[token] = float32 sum of bf16(down(h)) over the token's slots in ascending expert order
+ * weights device f32 [T, k] (the router's `weights`, model.py:389-405); swiglu_limit as in the model's config (0: no
+ * clamp); out device f32 [T, H] (out_dtype BP_F32: the caller adds the shared experts, which are two more
+ * TernaryLinear-style calls, and casts) or bf16 [T, H] (BP_BF16: cast once). Everything else - arguments, workspace
+ * (bp_moe_layer_workspace_bytes), no read-back, no allocation - as bp_moe_layer_bf16. */
+int bp_moe_layer_v4(void* out, int out_dtype, const void* x, const int64_t* experts, const float* weights, float swiglu_limit,
+                    const uint8_t* const* gate_up_packed, const void* const* gate_up_scale,
+                    const uint8_t* const* down_packed, const void* const* down_scale, int scale_dtype,
+                    int n_terms, int64_t T, int64_t H, int64_t I, int64_t E, int64_t k, int64_t group, int fmt,
+                    int act, void* workspace, size_t workspace_bytes, int32_t* bad, void* stream);
 
 #ifdef __cplusplus
 }

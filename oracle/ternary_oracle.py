@@ -336,3 +336,39 @@ def moe_layer_ref(x_bf16, router_logits, experts, top_k: int, K_hidden: int, K_i
         for i, tok in enumerate(token):  # index_add_ in bf16, one (token, slot) pair at a time
             out[tok] = bf16_round(out[tok] + r[i])
     return out
+
+
+def moe_layer_v4_ref(x_bf16, weights, indices, experts, K_hidden: int, K_inter: int, group: int, fmt: str,
+                     act: str = "bf16", swiglu_limit: float = 0.0) -> np.ndarray:
+    """boilerplate/engine/model.py:376-387 (``swiglu``) and :407-420 (``moe``, the routed experts; the shared experts
+    of :421 are further ``swiglu`` calls without weights and stay with the caller). Returns the float32 ``y``.
+
+    ``weights`` float32 [T, k] and ``indices`` int [T, k] are the router's output (:389-405).
+    Rounding points: ``w1(x)`` / ``w3(x)`` return bf16 (TernaryLinear's ``out_dtype``, boilerplate/ternary/ops.py:60) and are
+    widened to float32; ``up`` is clamped to [-limit, limit] and ``gate`` to at most limit when limit > 0; ``silu(gate) * up``
+    and the product with the routing weight are float32; that is rounded to bf16 once (``x.to(dtype)``) as ``w2``'s input;
+    ``w2`` returns bf16; ``y[idx] +=`` accumulates in float32, experts in ascending order.
+    """
+    x = bf16_round(np.asarray(x_bf16, dtype=np.float32))
+    weights = np.asarray(weights, dtype=np.float32)
+    indices = np.asarray(indices)
+    y = np.zeros_like(x, dtype=np.float32)
+    lim = np.float32(swiglu_limit)
+    for e in range(len(experts)):
+        token, slot = np.nonzero(indices == e)
+        if token.size == 0:
+            continue
+        gate_t, up_t, down_t = experts[e]
+        xe = x[token]
+        g = bf16_round(ternary_linear_ref(xe, gate_t, K_hidden, group, fmt, act).astype(np.float32))
+        u = bf16_round(ternary_linear_ref(xe, up_t, K_hidden, group, fmt, act).astype(np.float32))
+        if lim > 0:
+            u = np.clip(u, -lim, lim)
+            g = np.minimum(g, lim)
+        sg = (g.astype(np.float64) / (1.0 + np.exp(-g.astype(np.float64)))).astype(np.float32)  # float32 silu, correctly rounded
+        h = (sg * u).astype(np.float32)
+        h = (weights[token, slot, None] * h).astype(np.float32)
+        d = bf16_round(ternary_linear_ref(bf16_round(h), down_t, K_inter, group, fmt, act).astype(np.float32))
+        for i, tok in enumerate(token):
+            y[tok] = (y[tok] + d[i]).astype(np.float32)
+    return y

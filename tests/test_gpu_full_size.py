@@ -144,6 +144,41 @@ def test_config2_moe_layer_full_size(T):
     assert np.abs(got[sample] - want).max() <= 2e-2 * max(1.0, np.abs(want).max())
 
 
+def test_config3_moe_layer_v4_full_size():
+    """Config 3's layer (E = 384, H = 4096, I = 2048, two stacked TQ2 terms, 2048 tokens top-6) through the V4 engine's call
+    pattern (boilerplate/engine/model.py:376-387, 407-420): sampled tokens against oracle.moe_layer_v4_ref."""
+    import deepseekternarized_amd as bp
+    from deepseekternarized_amd.moe import TernaryMoE
+
+    H, I, E, k, T, fmt = 4096, 2048, 384, 6, 2048, "tq2"
+    mats = {}
+    for name, (n, kk), seed in (("gate", (I, H), 3), ("up", (I, H), 4), ("down", (H, I), 5)):
+        p, s = _weights(bp, E, n, kk, fmt, 2, seed)
+        mats[name] = list(zip(p, s))
+    moe = TernaryMoE(mats["gate"], mats["up"], mats["down"], H, I, k, fmt, GROUP, act="bf16", pattern="v4", swiglu_limit=7.0)
+    g = torch.Generator(device="cuda").manual_seed(9)
+    x = torch.randn(T, H, device="cuda", generator=g).to(torch.bfloat16)
+    scores = torch.softmax(torch.randn(T, E, device="cuda", generator=g) * 1.5, -1)
+    weights, indices = torch.topk(scores, k, -1)
+    weights = weights / (weights.sum(-1, keepdim=True) + 1e-20) * 2.5  # (norm_topk_prob and route_scale, model.py:401-404)
+    got = moe.routed(x, weights, indices)
+    assert bp.ext().last_kernel().startswith("gemm_tq2"), bp.ext().last_kernel()
+    assert got.dtype == torch.float32 and torch.isfinite(got).all()
+    sample = sorted({0, T - 1, *np.random.default_rng(3).choice(T, 3, replace=False).tolist()})
+    used = sorted(set(indices[sample].reshape(-1).tolist()))
+    experts = [None] * E
+    for e in used:
+        experts[e] = tuple([(pk[e].cpu().numpy(), sc[e].cpu().numpy()) for pk, sc in mats[n]] for n in ("gate", "up", "down"))
+    for e in range(E):
+        if experts[e] is None:
+            experts[e] = experts[used[0]]  # (never selected by the sampled tokens)
+    want = orc.moe_layer_v4_ref(x[sample].float().cpu().numpy(), weights[sample].cpu().numpy(), indices[sample].cpu().numpy(), experts,
+                                H, I, GROUP, fmt, act="bf16", swiglu_limit=7.0)
+    gs = got[sample].cpu().numpy()
+    assert rel_l2(gs, want) <= 5e-3, rel_l2(gs, want)
+    assert np.abs(gs - want).max() <= 2e-2 * max(1.0, np.abs(want).max())
+
+
 def test_config4_decoder_full_size():
     """The OLMoE-shaped Mode D decoder at its full shape (16 layers, hidden 2048, 16 heads, 64 experts top-8,
     intermediate 1024, vocabulary 50304, TQ2, int8 activations): a prefill and two greedy decode steps, every ternary

@@ -175,3 +175,111 @@ def test_layer_call_argument_checks():
                                128, 2, _lib.BP_BF16, ws.data_ptr(), need, flag.data_ptr(), None)
     torch.cuda.synchronize()
     assert rc == 0 and int(flag) == 1
+
+
+# --------------------------------------------------------------------------- the V4 engine's call pattern
+def _v4_inputs(T, H, E, k, seed):
+    rng = np.random.default_rng(seed)
+    x = orc.bf16_round(rng.standard_normal((T, H)).astype(np.float32))
+    scores = orc.softmax_f32((rng.standard_normal((T, E)) * 1.5).astype(np.float32))
+    _, indices = orc.topk_desc(scores, k)
+    weights = (np.take_along_axis(scores, indices, -1) * np.float32(2.5)).astype(np.float32)
+    return x, weights, indices
+
+
+@pytest.mark.parametrize("limit", [0.0, 0.5])
+@pytest.mark.parametrize("fmt,terms,act,T", [("tq1", 1, "bf16", 96), ("tq2", 2, "bf16", 96), ("tq2", 1, "int8", 40), ("tq1", 1, "int8", 5)])
+def test_v4_layer_matches_the_reference_lines(fmt, terms, act, T, limit):
+    """bp_moe_layer_v4 against boilerplate/engine/model.py:376-387 / :407-420 restated on the CPU (oracle.moe_layer_v4_ref):
+    float32 routing weights before w2, the clamps, float32 accumulation over a token's experts."""
+    from deepseekternarized_amd.moe import TernaryMoE
+
+    H, I, E, k, group = 1024, 1024, 8, 2, 128
+    _, mats = _layer(fmt, act, H, I, E, k, terms=terms, seed=41)
+    moe = TernaryMoE(*mats, H, I, k, fmt, group, act=act, pattern="v4", swiglu_limit=limit)
+    x, weights, indices = _v4_inputs(T, H, E, k, seed=42 + T)
+    experts = [tuple([(mats[n][t][0][e].cpu().numpy(), mats[n][t][1][e].cpu().numpy()) for t in range(terms)] for n in range(3)) for e in range(E)]
+    want = orc.moe_layer_v4_ref(x, weights, indices, experts, H, I, group, fmt, act=act, swiglu_limit=limit)
+    xd = torch.from_numpy(x).cuda().to(torch.bfloat16)
+    got = moe.routed(xd, torch.from_numpy(weights).cuda(), torch.from_numpy(indices).cuda())
+    assert got.dtype == torch.float32 and got.shape == (T, H)
+    rel = np.linalg.norm(got.cpu().numpy() - want) / np.linalg.norm(want)
+    assert rel <= 5e-3, rel  # the same rounding points; float32 sums in another order flip a few bf16 roundings
+    # the bf16 form is the float32 one cast once
+    got16 = moe.routed(xd, torch.from_numpy(weights).cuda(), torch.from_numpy(indices).cuda(), out_dtype=torch.bfloat16)
+    assert torch.equal(got16, got.to(torch.bfloat16))
+    if limit > 0:  # the clamp changes the result (it is exercised), and a different pattern is a different number
+        free = TernaryMoE(*mats, H, I, k, fmt, group, act=act, pattern="v4").routed(xd, torch.from_numpy(weights).cuda(), torch.from_numpy(indices).cuda())
+        assert not torch.equal(free, got)
+    with pytest.raises(RuntimeError):
+        moe(xd, torch.zeros(T, E, device="cuda"))
+
+
+def test_v4_stages_bit_exact():
+    """bp_swiglu_v4 and bp_moe_combine_v4 alone, against their definitions evaluated with torch on the device
+    (float32 throughout; expf may differ from torch's by an ulp, which the bf16 rounding rarely sees)."""
+    import torch.nn.functional as F
+
+    from deepseekternarized_amd.kernels import _lib
+
+    lib = _lib.load()
+    g = torch.Generator(device="cuda").manual_seed(7)
+    rows, I, pairs = 37, 520, 37
+    gu = torch.randn(rows, 2 * I, device="cuda", generator=g) * 2
+    w = torch.rand(pairs, device="cuda", generator=g) * 3
+    order = torch.randperm(pairs, device="cuda", generator=g)
+    h = torch.empty(rows, I, dtype=torch.bfloat16, device="cuda")
+    for limit in (0.0, 1.25):
+        rc = lib.bp_swiglu_v4(h.data_ptr(), gu.data_ptr(), gu[:, I:].data_ptr(), w.data_ptr(), order.data_ptr(), pairs, limit, rows, I, 2 * I, None)
+        assert rc == 0, lib.bp_last_error()
+        gate, up = gu[:, :I].to(torch.bfloat16).float(), gu[:, I:].to(torch.bfloat16).float()
+        if limit > 0:
+            up, gate = torch.clamp(up, min=-limit, max=limit), torch.clamp(gate, max=limit)
+        want = (w[order][:, None] * (F.silu(gate) * up)).to(torch.bfloat16)
+        same = (h == want).float().mean().item()
+        assert same >= 0.999, same
+        assert ((h.float() - want.float()).abs() <= want.float().abs() * 2.0 ** -7 + 1e-30).all()
+    # no weights: a shared expert
+    rc = lib.bp_swiglu_v4(h.data_ptr(), gu.data_ptr(), gu[:, I:].data_ptr(), None, None, 0, 0.0, rows, I, 2 * I, None)
+    assert rc == 0
+    want = (F.silu(gu[:, :I].to(torch.bfloat16).float()) * gu[:, I:].to(torch.bfloat16).float()).to(torch.bfloat16)
+    assert (h == want).float().mean().item() >= 0.999
+    # combine: float32 sums in ascending expert order of the bf16-rounded rows
+    T, k, H = 9, 4, 300
+    experts = torch.stack([torch.randperm(16, device="cuda", generator=g)[:k] for _ in range(T)])
+    flat_order = torch.argsort(experts.reshape(-1), stable=True)
+    inv = torch.empty_like(flat_order)
+    inv[flat_order] = torch.arange(T * k, device="cuda")
+    y = torch.randn(T * k, H, device="cuda", generator=g) * 100
+    out = torch.empty(T, H, device="cuda")
+    assert lib.bp_moe_combine_v4(out.data_ptr(), _lib.BP_F32, y.data_ptr(), inv.data_ptr(), experts.data_ptr(), T, k, H, None) == 0
+    want = torch.zeros(T, H, device="cuda")
+    yb = y.to(torch.bfloat16).float()
+    for e in range(16):
+        tok, slot = torch.where(experts == e)
+        if tok.numel():
+            want[tok] += yb[inv[tok * k + slot]]
+    assert torch.equal(out, want)
+    assert lib.bp_moe_combine_v4(out.data_ptr(), _lib.BP_I8, y.data_ptr(), inv.data_ptr(), experts.data_ptr(), T, k, H, None) != 0
+
+
+def test_graphs_of_one_layer_keep_their_workspaces():
+    """Two graphed callables of one layer and a larger eager call in between: every graph replays into the workspace it
+    captured, which the layer keeps alive when a later call needs a bigger one."""
+    moe, _ = _layer("tq2", "bf16", 1024, 1024, 8, 2, seed=51)
+    g = torch.Generator(device="cuda").manual_seed(52)
+    g1 = moe.graphed(8)
+    g2 = moe.graphed(40)
+    x300 = torch.randn(300, 1024, device="cuda", generator=g).to(torch.bfloat16)
+    l300 = torch.randn(300, 8, device="cuda", generator=g)
+    big = moe(x300, l300).clone()
+    filler = [torch.randn(1 << 20, device="cuda") for _ in range(8)]  # takes freed blocks, if any were freed
+    for run, T in ((g1, 8), (g2, 40), (g1, 8)):
+        x = torch.randn(T, 1024, device="cuda", generator=g).to(torch.bfloat16)
+        lg = torch.randn(T, 8, device="cuda", generator=g)
+        want = moe(x, lg).clone()
+        got = run(x, lg).clone()
+        torch.cuda.synchronize()
+        assert torch.equal(got, want), T
+    assert torch.equal(moe(x300, l300), big)
+    del filler

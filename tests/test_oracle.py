@@ -218,3 +218,138 @@ def test_absmean_ternary_known_answers():
         orc.absmean_ternary(np.zeros((2, 0), np.float32), 3)
     with pytest.raises(ValueError):
         orc.absmean_ternary(np.zeros((2, 4), np.float32), 0)
+
+
+# --------------------------------------------------------------------------- MoE oracles against torch CPU restatements
+def _tiny_experts(rng, H, I, E, group, fmt, terms=1):
+    experts = []
+    for e in range(E):
+        mats = []
+        for (n, kk) in ((I, H), (I, H), (H, I)):
+            ts = []
+            for t in range(terms):
+                tr = rng.integers(-1, 2, (n, kk)).astype(np.int8)
+                sc = (0.1 * 0.25 ** t * np.abs(rng.standard_normal((n, kk // group)))).astype(np.float16)
+                ts.append((orc.pack(tr, fmt), sc))
+            mats.append(ts)
+        experts.append(tuple(mats))
+    return experts
+
+
+def _torch_linear_bf16(x, terms, K, group, fmt):
+    """A float-activation TernaryLinear on dequantized weights (boilerplate/ternary/ops.py:51-58, 81-86), the product in
+    float64 so that its value is the exact one up to 2^-53, rounded to bf16 as ``out_dtype=x.dtype`` does."""
+    import torch
+
+    w = torch.from_numpy(orc.dequantize(terms, K, group, fmt).astype(np.float64))
+    return (x.double() @ w.t()).float().to(torch.bfloat16)
+
+
+def _bf16_ulps(a, b):
+    """Distance in bf16 steps between two bf16-valued float32 arrays of one sign pattern (0 where equal)."""
+    ia = (np.asarray(a, np.float32).view(np.uint32) >> 16).astype(np.int64)
+    ib = (np.asarray(b, np.float32).view(np.uint32) >> 16).astype(np.int64)
+    ia = np.where(ia & 0x8000, 0x8000 - ia, ia)
+    ib = np.where(ib & 0x8000, 0x8000 - ib, ib)
+    return np.abs(ia - ib)
+
+
+@pytest.mark.parametrize("renorm", [False, True])
+def test_moe_layer_ref_against_the_reference_lines_in_torch(renorm):
+    """moe_layer_ref against boilerplate/engine/standard.py:151-176 restated line by line with torch CPU ops on bf16
+    tensors (softmax, topk, F.silu, bf16 products, index_add_), the linears on dequantized weights. Every rounding
+    point and the accumulation order are pinned: agreement within one bf16 step per element, nearly all equal."""
+    import torch
+    import torch.nn.functional as F
+
+    rng = np.random.default_rng(21)
+    H, I, E, k, T, group, fmt = 64, 32, 6, 3, 40, 32, "tq1"
+    experts = _tiny_experts(rng, H, I, E, group, fmt)
+    x = orc.bf16_round(rng.standard_normal((T, H)).astype(np.float32))
+    logits = (rng.standard_normal((T, E)) * 1.5).astype(np.float32)
+    got = orc.moe_layer_ref(x, logits, experts, k, H, I, group, fmt, act="bf16", renorm=renorm)
+
+    flat = torch.from_numpy(x).to(torch.bfloat16)
+    scores = torch.softmax(torch.from_numpy(logits).float(), dim=-1)
+    values, indices = torch.topk(scores, k, dim=-1)
+    if renorm:
+        values = values / values.sum(-1, keepdim=True)
+    values = values.to(flat.dtype)
+    output = torch.zeros_like(flat)
+    for e in range(E):
+        token, slot = torch.where(indices == e)
+        if not token.numel():
+            continue
+        gate_t, up_t, down_t = experts[e]
+        xe = flat[token]
+        h = F.silu(_torch_linear_bf16(xe, gate_t, H, group, fmt)) * _torch_linear_bf16(xe, up_t, H, group, fmt)
+        result = _torch_linear_bf16(h, down_t, I, group, fmt) * values[token, slot, None]
+        output.index_add_(0, token, result.to(output.dtype))
+    want = output.float().numpy()
+    ulps = _bf16_ulps(got, want)
+    assert ulps.max() <= 1, ulps.max()
+    assert (ulps == 0).mean() >= 0.995, (ulps == 0).mean()
+
+
+def test_topk_desc_matches_torch_topk():
+    """The routing's top-k: values and indices equal torch.topk's on rows without ties (softmax scores of random logits), and
+    on rows with ties the same VALUES; which of two equal scores torch.topk returns first is not specified by torch,
+    the oracle takes the lower index (a stable sort)."""
+    import torch
+
+    rng = np.random.default_rng(5)
+    scores = orc.softmax_f32((rng.standard_normal((200, 64)) * 1.5).astype(np.float32))
+    assert all(np.unique(r).size == r.size for r in scores)
+    v, i = orc.topk_desc(scores, 6)
+    tv, ti = torch.topk(torch.from_numpy(scores), 6, dim=-1)
+    assert np.array_equal(v, tv.numpy()) and np.array_equal(i, ti.numpy())
+    tied = np.array([[0.25, 0.5, 0.25, 0.5, 0.125]], np.float32)
+    v, i = orc.topk_desc(tied, 3)
+    assert v.tolist() == [[0.5, 0.5, 0.25]] and i.tolist() == [[1, 3, 0]]
+    assert torch.topk(torch.from_numpy(tied), 3).values.tolist() == v.tolist()
+
+
+@pytest.mark.parametrize("limit", [0.0, 0.75])
+def test_moe_layer_v4_ref_against_the_reference_lines_in_torch(limit):
+    """moe_layer_v4_ref against boilerplate/engine/model.py:376-387 and :407-420 restated with torch CPU ops: bf16 linears
+    widened to float32, the clamps, F.silu in float32, the routing weight before w2, one cast to bf16, float32 `y[idx] +=`.
+    float32 silu differs from the oracle's correctly rounded one by an ulp now and then, which a bf16 rounding of the
+    product rarely sees: within one bf16 step of w2's output scale, nearly all sums equal to the last float32 bit."""
+    import torch
+    import torch.nn.functional as F
+
+    rng = np.random.default_rng(22)
+    H, I, E, k, T, group, fmt = 64, 32, 6, 3, 40, 32, "tq2"
+    experts = _tiny_experts(rng, H, I, E, group, fmt, terms=2)
+    x = orc.bf16_round(rng.standard_normal((T, H)).astype(np.float32))
+    scores = orc.softmax_f32((rng.standard_normal((T, E)) * 1.5).astype(np.float32))
+    _, indices = orc.topk_desc(scores, k)
+    weights = (np.take_along_axis(scores, indices, -1) * np.float32(2.5)).astype(np.float32)  # (route_scale, model.py:404)
+    got = orc.moe_layer_v4_ref(x, weights, indices, experts, H, I, group, fmt, act="bf16", swiglu_limit=limit)
+
+    xt = torch.from_numpy(x).to(torch.bfloat16)
+    wt, it = torch.from_numpy(weights), torch.from_numpy(indices)
+    y = torch.zeros_like(xt, dtype=torch.float32)
+    clamped = 0
+    for e in range(E):
+        idx, top = torch.where(it == e)
+        if not idx.numel():
+            continue
+        w1, w3, w2 = experts[e]
+        xe = xt[idx]
+        gate, up = _torch_linear_bf16(xe, w1, H, group, fmt).float(), _torch_linear_bf16(xe, w3, H, group, fmt).float()
+        if limit > 0:
+            clamped += int((up.abs() > limit).sum() + (gate > limit).sum())
+            up = torch.clamp(up, min=-limit, max=limit)
+            gate = torch.clamp(gate, max=limit)
+        h = F.silu(gate) * up
+        h = wt[idx, top, None] * h
+        y[idx] += _torch_linear_bf16(h.to(torch.bfloat16), w2, I, group, fmt)
+    want = y.numpy()
+    assert limit == 0 or clamped > 50  # the clamp is exercised
+    scale = np.abs(want).max()
+    assert np.abs(got - want).max() <= scale * 2.0 ** -7
+    assert (got == want).mean() >= 0.98, (got == want).mean()
+    # a dropped routing weight, a clamp on the wrong operand or bf16 accumulation would not pass:
+    wrong = orc.moe_layer_v4_ref(x, np.ones_like(weights), indices, experts, H, I, group, fmt, swiglu_limit=limit)
+    assert (wrong == want).mean() < 0.5
