@@ -1,6 +1,7 @@
 // C entry point of the grouped ternary GEMM: argument validation (the checks of the reference
 // launcher, boilerplate/kernels/csrc/ternary_cuda_kernel.cu:109-141, done without any
 // device-to-host copy), kernel selection, and the thread-local error/kernel-name plumbing.
+#include <atomic>
 #include <cstdarg>
 #include <cstdio>
 #include <cstdlib>
@@ -29,24 +30,27 @@ void note_kernel(const char* name) {
 }
 
 namespace {
-Tuning g_tuning = {0, 0, 0, 0, 0, -1, 0};
+// The overrides in force: an immutable snapshot behind an atomic pointer, so that a launch path on one thread reads a
+// consistent set while bp_reload_tuning() on another publishes a new one (old snapshots are never freed: a reader may
+// still hold one, and there are only as many as there were reloads).
+std::atomic<const Tuning*> g_tuning{nullptr};
 std::once_flag g_tuning_once;
 void read_tuning() {
-  Tuning t = {0, 0, 0, 0, 0, -1, 0};
-  if (const char* v = getenv("BP_TUNE_R")) t.r = atoi(v);
-  if (const char* v = getenv("BP_TUNE_WAVES")) t.waves = atoi(v);
-  if (const char* v = getenv("BP_TUNE_TQ1")) t.tq1 = v[0];
-  if (const char* v = getenv("BP_TUNE_TQ2G")) t.tq2g = v[0];
-  if (const char* v = getenv("BP_TUNE_F4W")) t.f4w = atoi(v);
-  if (const char* v = getenv("BP_TUNE_F4T")) t.f4t = atoi(v);
-  if (const char* v = getenv("BP_TUNE_CPT")) t.cpt = atoi(v);
-  g_tuning = t;
+  Tuning* t = new Tuning{0, 0, 0, 0, 0, -1, 0};
+  if (const char* v = getenv("BP_TUNE_R")) t->r = atoi(v);
+  if (const char* v = getenv("BP_TUNE_WAVES")) t->waves = atoi(v);
+  if (const char* v = getenv("BP_TUNE_TQ1")) t->tq1 = v[0];
+  if (const char* v = getenv("BP_TUNE_TQ2G")) t->tq2g = v[0];
+  if (const char* v = getenv("BP_TUNE_F4W")) t->f4w = atoi(v);
+  if (const char* v = getenv("BP_TUNE_F4T")) t->f4t = atoi(v);
+  if (const char* v = getenv("BP_TUNE_CPT")) t->cpt = atoi(v);
+  g_tuning.store(t, std::memory_order_release);
 }
 }  // namespace
 
 const Tuning& tuning() {
   std::call_once(g_tuning_once, read_tuning);
-  return g_tuning;
+  return *g_tuning.load(std::memory_order_acquire);
 }
 
 int check_launch(const char* what) {

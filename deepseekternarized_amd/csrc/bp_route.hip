@@ -358,6 +358,7 @@ extern "C" int bp_sort_by_expert(int64_t* order, int64_t* offsets, const int64_t
 
 extern "C" int bp_sort_by_expert_static(int64_t* order, int64_t* offsets, const int64_t* ids, int64_t n, int64_t E,
                                         int32_t* bad, void* stream) {
+  fail(BP_OK, "%s", "");  // (an earlier call's message does not outlive this one)
   if (n < 0 || E < 0 || n > ((int64_t)1 << 31) - 1) return fail(BP_ERR_ARG, "invalid n or E");
   if (E > SORT_STATIC_MAX_E)
     return fail(BP_ERR_ARG, "bp_sort_by_expert_static takes at most %lld experts (its histograms live in a fixed device array); "

@@ -106,7 +106,9 @@ int bp_set_kernel_policy(int policy);
 
 /* The kernel selection has development overrides (environment variables BP_TUNE_*), read once when the library is first
  * used. This reads them again; it is for tests and tuning sweeps that switch kernels inside one process, and has no
- * counterpart in the reference. */
+ * counterpart in the reference. Development only: the variables steer which kernel a call runs on (never its result
+ * beyond the documented tolerances) and the answer of bp_grouped_gemm_workspace_bytes; a deployment leaves them unset.
+ * Safe against launches on other threads: they read either the old or the new set, whole. */
 void bp_reload_tuning(void);
 
 /* Name of the kernel the last bp_ternary_grouped_gemm on this thread launched ("" if none). */
@@ -155,7 +157,9 @@ int bp_sort_by_expert(int64_t* order, int64_t* offsets, const int64_t* ids, int6
  * live in a fixed 4 MiB device array inside the library (one per GPU, held until the process ends), so E is limited
  * to BP_SORT_STATIC_MAX_EXPERTS (more: BP_ERR_ARG). Results are identical to bp_sort_by_expert's. All calls on
  * one GPU share that array: calls that overlap in time on one GPU (different streams) race; calls on one
- * stream are ordered and each clears the counters it uses itself. */
+ * stream are ordered and each clears the counters it uses itself. The first call on a device looks up the array's
+ * address and sets a kernel attribute (host-side runtime calls): make it outside any stream capture; later calls
+ * on that device are plain kernel launches and can be captured. */
 #define BP_SORT_STATIC_MAX_EXPERTS 65536
 int bp_sort_by_expert_static(int64_t* order, int64_t* offsets, const int64_t* ids, int64_t n, int64_t E,
                              int32_t* bad, void* stream);

@@ -1,5 +1,7 @@
 """The Mode C / D checkpoint reader against directories written here in the reference's on-disk layout
-(docs/architecture/format.md:87-134): manifest checks, shapes, SHA-256, stacking of per-expert weights."""
+(docs/architecture/format.md:87-134): manifest checks, shapes, SHA-256, stacking of per-expert weights; and against
+tests/golden/export_tiny, two checkpoints written by the reference's own exporter (boilerplate/format/export.py:115-300,
+run by tests/golden/make_export_fixture.py)."""
 
 import json
 
@@ -184,3 +186,101 @@ def test_symlinked_shard_outside_the_directory_is_refused(tmp_path):
     shard.symlink_to(moved)
     with pytest.raises(ValueError, match="escapes"):
         TernaryCheckpoint(root).terms(next(iter(w)))
+
+
+# --------------------------------------------------------------------------- checkpoints written by the reference's exporter
+from pathlib import Path  # noqa: E402
+
+EXPORTS = Path(__file__).resolve().parent / "golden" / "export_tiny"
+EXPERT_BASES = [f"layers.0.ffn.experts.{e}.{w}" for e in range(2) for w in ("w1", "w2", "w3")]
+
+
+def _source():
+    from safetensors import safe_open
+
+    with safe_open(str(EXPORTS / "source" / "weights.safetensors"), framework="pt", device="cpu") as f:
+        return {n: f.get_tensor(n) for n in f.keys()}
+
+
+@pytest.mark.parametrize("name,mode,fmt,terms,group,sdt,act", [("mode_c_tq1", "C", "tq1", 2, 128, torch.float16, "int8"),
+                                                                ("mode_d_tq2", "D", "tq2", 1, 64, torch.bfloat16, "bf16")])
+def test_reads_what_the_reference_exporter_wrote(name, mode, fmt, terms, group, sdt, act):
+    """Names, `terms`, `group`, `scale_dtype`, `act`, shapes and SHA-256 of every stored tensor as the reference's exporter
+    recorded them (boilerplate/format/export.py:204-234); the dense weight no rule matched stays Mode A and is refused."""
+    ck = TernaryCheckpoint(EXPORTS / name, verify=True)
+    assert ck.bases() == sorted(EXPERT_BASES)
+    src = _source()
+    for base in EXPERT_BASES:
+        tm, m = ck.terms(base)
+        N, K = src[base + ".weight"].shape
+        assert (m["mode"], m["packing"], m["terms"], m["group"], m["act"], tuple(m["shape"])) == (mode, fmt, terms, group, act, (N, K))
+        assert len(tm) == terms
+        for i, t in enumerate(tm):
+            assert t.packed.dtype == torch.uint8 and tuple(t.packed.shape) == (N, -(-K // (5 if fmt == "tq1" else 4)))
+            assert t.scale.dtype == sdt and tuple(t.scale.shape) == (N, -(-K // group))
+            rec = m["stored"][f"{base}.tq{i}.packed"]
+            assert tensor_sha256(t.packed) == rec["sha256"] and rec["file"] == "model-00001-of-00001.safetensors"
+        lin = ck.linear(base)
+        assert (lin.K, lin.fmt, lin.group, lin.act, lin.out_features) == (K, fmt, group, act, N)
+    with pytest.raises(ValueError, match="mode 'A'"):
+        ck.entry("layers.0.attn.wq")
+    stacks, meta = ck.stack([f"layers.0.ffn.experts.{e}.w1" for e in range(2)], "cpu")
+    assert meta == {"N": 16, "K": 200, "fmt": fmt, "group": group, "act": act, "terms": terms}
+    assert len(stacks) == terms and tuple(stacks[0][0].shape) == (2, 16, 50 if fmt == "tq2" else 40)
+
+
+def test_exported_terms_decode_to_the_source_weights():
+    """What the stored bytes mean: the oracle's unpack x scales of the reference-written terms reconstruct the source weight
+    to the error the reference's own test allows (tests/test_format.py:230-231: k = 2 on Gaussians < 0.3), padding included
+    (K = 200: the last TQ1 byte holds no pad digits, the last TQ2 byte none either, the last scale group is 72 / 8 wide)."""
+    src = _source()
+    for name, fmt, group, bound in (("mode_c_tq1", "tq1", 128, 0.3), ("mode_d_tq2", "tq2", 64, 0.55)):
+        ck = TernaryCheckpoint(EXPORTS / name)
+        for base in EXPERT_BASES:
+            tm, m = ck.terms(base)
+            K = m["shape"][1]
+            W = src[base + ".weight"].float().numpy()
+            R = orc.dequantize([(t.packed.numpy(), t.scale.float().numpy()) for t in tm], K, group, fmt)
+            err = np.linalg.norm(W - R) / np.linalg.norm(W)
+            assert err < bound, (name, base, err)
+            trits = orc.unpack(tm[0].packed.numpy(), fmt, K)
+            assert set(np.unique(trits).tolist()) <= {-1, 0, 1}
+
+
+def test_mode_d_export_equals_the_oracle_quantizer():
+    """The reference's Mode D producer on general (Gaussian bf16) weights against oracle.absmean_ternary + pack: the stored
+    scales and packed bytes are the oracle's, bit for bit - which pins the oracle's float32 summation order against
+    torch's `abs().sum(-1)` on these rows (groups of 64 and a last group of 8)."""
+    src = _source()
+    ck = TernaryCheckpoint(EXPORTS / "mode_d_tq2")
+    for base in EXPERT_BASES:
+        tm, m = ck.terms(base)
+        trits, scale = orc.absmean_ternary(src[base + ".weight"].float().numpy(), 64, "bf16")
+        assert np.array_equal(tm[0].scale.float().numpy(), scale), base
+        assert np.array_equal(tm[0].packed.numpy(), orc.pack(trits, "tq2")), base
+
+
+@pytest.mark.gpu
+def test_reference_written_checkpoints_run_on_the_gpu():
+    """Both exports through `linear` on the device against the oracle on the decoded terms, and the Mode D export
+    reproduced on the device from the source weights by bp_absmean_pack."""
+    import deepseekternarized_amd as bp
+    from deepseekternarized_amd.ternary.fit import packed_term
+
+    src = _source()
+    rng = np.random.default_rng(1)
+    for name, fmt, group in (("mode_c_tq1", "tq1", 128), ("mode_d_tq2", "tq2", 64)):
+        ck = TernaryCheckpoint(EXPORTS / name, verify=True)
+        for base in EXPERT_BASES[:3]:
+            lin = ck.linear(base)
+            tm, m = ck.terms(base)
+            K = m["shape"][1]
+            x = orc.bf16_round(rng.standard_normal((3, K)).astype(np.float32))
+            got = lin(torch.from_numpy(x).cuda().to(torch.bfloat16), out_dtype=torch.float32).cpu().numpy()
+            want = orc.ternary_linear_ref(x, [(t.packed.numpy(), t.scale.float().numpy()) for t in tm], K, group, fmt, act=m["act"])
+            assert np.linalg.norm(got - want) <= 1e-3 * np.linalg.norm(want), (name, base)
+    ck = TernaryCheckpoint(EXPORTS / "mode_d_tq2")
+    for base in EXPERT_BASES:
+        tm, _ = ck.terms(base)
+        term = packed_term(src[base + ".weight"].cuda(), 64, "tq2", scale_dtype=torch.bfloat16)
+        assert torch.equal(term.packed.cpu(), tm[0].packed) and torch.equal(term.scale.cpu(), tm[0].scale), base

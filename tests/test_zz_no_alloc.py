@@ -54,3 +54,32 @@ def test_static_sort_rejects_more_experts_than_its_array_holds():
     offs = torch.zeros(65538, dtype=torch.int64, device="cuda")
     assert lib.bp_sort_by_expert_static(out.data_ptr(), offs.data_ptr(), ids.data_ptr(), 200, 65537, None, None) == 1
     assert b"at most 65536" in lib.bp_last_error()
+
+
+def test_static_sort_captured_in_a_graph_after_a_first_eager_call():
+    """The first call per device resolves the array's address outside any capture; a later call is plain launches and
+    can be captured: replayed three times with eager work in between, each replay equal to bp_sort_by_expert."""
+    from deepseekternarized_amd.kernels import _lib
+
+    lib = _lib.load()
+    n, E = 9000, 3000
+    g = torch.Generator(device="cuda").manual_seed(3)
+    ids = torch.randint(0, E, (n,), device="cuda", generator=g)
+    order = torch.empty(n, dtype=torch.int64, device="cuda")
+    offsets = torch.empty(E + 1, dtype=torch.int64, device="cuda")
+    _lib.check(lib.bp_sort_by_expert_static(order.data_ptr(), offsets.data_ptr(), ids.data_ptr(), n, E, None, _lib.stream_ptr(ids.device)))
+    torch.cuda.synchronize()
+    assert lib.bp_last_error() == b""
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        _lib.check(lib.bp_sort_by_expert_static(order.data_ptr(), offsets.data_ptr(), ids.data_ptr(), n, E, None, _lib.stream_ptr(ids.device)))
+    ws = torch.empty(lib.bp_sort_workspace_ints(n, E), dtype=torch.int32, device="cuda")
+    want_order, want_offsets = torch.empty_like(order), torch.empty_like(offsets)
+    for rep in range(3):
+        ids.copy_(torch.randint(0, E, (n,), device="cuda", generator=g))
+        order.fill_(-1)
+        graph.replay()
+        _lib.check(lib.bp_sort_by_expert(want_order.data_ptr(), want_offsets.data_ptr(), ids.data_ptr(), n, E, ws.data_ptr(), None,
+                                         _lib.stream_ptr(ids.device)))
+        torch.cuda.synchronize()
+        assert torch.equal(order, want_order) and torch.equal(offsets, want_offsets), rep
