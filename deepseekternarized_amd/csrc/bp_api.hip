@@ -147,12 +147,14 @@ extern "C" int bp_ternary_grouped_gemm(float* out, const void* x, int x_dtype, c
                       group, E, fmt, max_rows, nullptr, 0, stream);
 }
 
-extern "C" size_t bp_grouped_gemm_workspace_bytes(int x_dtype, int64_t T, int64_t N, int64_t K, int64_t E, int fmt) {
-  if (fmt != BP_TQ2 || x_dtype != BP_BF16) return 0;
-  // (the launcher's own thresholds, so that a call it would turn down does not make its caller allocate: at least two
-  // blocks of 512 output rows, at least three rounds of one workgroup per CU)
-  if (tuning().tq2g != 'f' && (N < 1024 || (T + 31) / 32 * ((N + 511) / 512) < 768)) return 0;
+extern "C" size_t bp_grouped_gemm_workspace_bytes(int x_dtype, int64_t T, int64_t N, int64_t K, int64_t E, int fmt, int64_t max_rows) {
+  if ((fmt != BP_TQ2 && fmt != BP_TQ1) || x_dtype != BP_BF16 || T <= 0 || E <= 0 || N <= 0) return 0;
   if (tuning().tq2g == 'b') return 0;
+  if (max_rows > T) max_rows = T;
+  // (the launcher's own thresholds, so that a call it would turn down does not make its caller allocate)
+  if (fmt == BP_TQ2 && tuning().tq2g != 'f' && (N < 1024 || (T + 31) / 32 * ((N + 511) / 512) < 768)) return 0;  // at least two blocks of 512 output rows, three rounds of one workgroup per CU
+  if (fmt == BP_TQ1 && max_rows <= 8 && tuning().tq2g != 'f') return 0;  // (the small-batch kernels take these)
+  if (max_rows <= 0 || (max_rows + 31) / 32 * 32 * E > 4 * T + 32 * E) return 0;  // a loose bound on the rows per expert: mostly token tiles that do not exist
   return gemm_tq2f_workspace_bytes(T, K, E);
 }
 

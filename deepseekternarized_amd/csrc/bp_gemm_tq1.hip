@@ -473,6 +473,10 @@ int launch_gemm_tq1_k(const GemmArgs& a, hipStream_t s, const char* name) {
 // bf16 or int8 activations; 4-byte aligned scale rows; K small enough for 32-bit offsets into a 32-token activation tile.
 // BP_ERR_UNSUPPORTED (no message): the caller falls back to its other kernels.
 int launch_gemm_tq1(const GemmArgs& a, hipStream_t s) {
+  if (a.stage && tuning().tq2g != 'b') {  // with a workspace: one matrix instruction per scale group over converted activations (bp_gemm_tq2f.hip; development: BP_TUNE_TQ2G=bf16 keeps this file's kernel)
+    const int rc = launch_gemm_tq2f(a, s);
+    if (rc != BP_ERR_UNSUPPORTED) return rc;
+  }
   if (a.x_dtype != BP_BF16 && a.x_dtype != BP_I8) return BP_ERR_UNSUPPORTED;
   if (a.K > ((int64_t)1 << 24) || a.N * a.Kp > ((int64_t)1 << 31) - 4096) return BP_ERR_UNSUPPORTED;
   if ((a.max_rows + 31) / 32 > 65535) return BP_ERR_UNSUPPORTED;

@@ -122,7 +122,7 @@ Plan plan(void* workspace, int64_t T, int64_t H, int64_t I, int64_t E, int64_t k
   p.h = c.take(2 * (size_t)n * I);
   p.y = (float*)c.take(4 * (size_t)n * H);
   p.stage_bytes = 0;
-  if (fmt == BP_TQ2 && act == BP_BF16 && T > 64) {
+  if (act == BP_BF16 && T > 64) {
     const size_t a = gemm_tq2f_workspace_bytes(n, H, E), b = gemm_tq2f_workspace_bytes(n, I, E);
     p.stage_bytes = a > b ? a : b;
   }

@@ -22,7 +22,7 @@ SIGNATURES = {
     "bp_set_kernel_policy": (_i, [_i]),
     "bp_reload_tuning": (None, []),
     "bp_ternary_grouped_gemm": (_i, [_p, _p, _i, _p, _p, _p, _p, _p, _i, _i, _l, _l, _l, _l, _l, _l, _l, _i, _l, _p, _p]),
-    "bp_grouped_gemm_workspace_bytes": (C.c_size_t, [_i, _l, _l, _l, _l, _i]),
+    "bp_grouped_gemm_workspace_bytes": (C.c_size_t, [_i, _l, _l, _l, _l, _i, _l]),
     "bp_ternary_grouped_gemm_ws": (_i, [_p, _p, _i, _p, _p, _p, _p, _p, _i, _i, _l, _l, _l, _l, _l, _l, _l, _i, _l, _p, C.c_size_t, _p]),
     "bp_unpack_trits": (_i, [_p, _p, _l, _l, _i, _p]),
     "bp_pack_trits": (_i, [_p, _p, _l, _l, _i, _p]),

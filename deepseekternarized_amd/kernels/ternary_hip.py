@@ -83,9 +83,10 @@ class _HipTernary:
         pk = (C.c_void_p * len(packed_l))(*[p.data_ptr() for p in packed_l])
         sc = (C.c_void_p * len(scale_l))(*[s.data_ptr() for s in scale_l])
         with torch.cuda.device(out.device):
-            # Prefill-sized calls get a workspace (the library allocates nothing itself): with one, the TQ2 kernels for bf16
-            # activations convert the activations once instead of once per block of output rows.
-            need = self.lib.bp_grouped_gemm_workspace_bytes(_lib.dtype_code(x.dtype), T, N, int(K), E, int(fmt)) if max_rows > 16 else 0
+            # Prefill-sized calls get a workspace (the library allocates nothing itself): with one, the grouped GEMM kernels
+            # for bf16 activations convert the activations once instead of once per block of output rows. The size query
+            # answers 0 where the launch would not use one (small calls, a loose max_rows).
+            need = self.lib.bp_grouped_gemm_workspace_bytes(_lib.dtype_code(x.dtype), T, N, int(K), E, int(fmt), int(max_rows))
             if need > _WORKSPACE_CAP:  # (about 2.1 bytes per activation: a call this large keeps its memory and runs the kernels without one)
                 need = 0
             if need:

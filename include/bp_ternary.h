@@ -82,13 +82,15 @@ int bp_ternary_grouped_gemm(float* out, const void* x, int x_dtype, const float*
 
 /* bp_ternary_grouped_gemm with a workspace of the caller's (the library allocates no device memory). It has no
  * counterpart in the reference. With a workspace of at least bp_grouped_gemm_workspace_bytes(...) bytes (256-byte
- * aligned device memory; contents undefined before and after the call) the TQ2 kernels for bf16 activations and more
- * than 16 rows per expert convert the activations to matrix-instruction operands once, in a pass of their own,
- * instead of once per block of output rows; results agree with bp_ternary_grouped_gemm's to float32 rounding of the
- * sums. workspace = NULL, or a size of 0 from bp_grouped_gemm_workspace_bytes (no such kernel for these arguments, or a
- * launch too small for it to pay: fewer than 1024 output rows, or fewer than 768 blocks of 32 tokens x 512 rows):
- * identical to bp_ternary_grouped_gemm. T is the row count of x (all experts). */
-size_t bp_grouped_gemm_workspace_bytes(int x_dtype, int64_t T, int64_t N, int64_t K, int64_t E, int fmt);
+ * aligned device memory; contents undefined before and after the call) the grouped GEMM kernels for bf16 activations
+ * (TQ2: more than 16 rows per expert; TQ1: more than 8) convert the activations to matrix-instruction operands once, in
+ * a pass of their own, instead of once per block of output rows; results agree with bp_ternary_grouped_gemm's to
+ * float32 rounding of the sums. workspace = NULL, or a size of 0 from bp_grouped_gemm_workspace_bytes (no such kernel
+ * for these arguments; a launch too small for it to pay - TQ2: fewer than 1024 output rows, or fewer than 768 blocks
+ * of 32 tokens x 512 rows; or max_rows so loose a bound that most of the launch's token tiles would not exist:
+ * ceil(max_rows / 32) * 32 * E > 4 T + 32 E, e.g. the default max_rows = T with more than a few experts):
+ * identical to bp_ternary_grouped_gemm. T is the row count of x (all experts), max_rows the bound the call will pass. */
+size_t bp_grouped_gemm_workspace_bytes(int x_dtype, int64_t T, int64_t N, int64_t K, int64_t E, int fmt, int64_t max_rows);
 int bp_ternary_grouped_gemm_ws(float* out, const void* x, int x_dtype, const float* x_scale,
                                const int64_t* offsets, const int64_t* offsets_host,
                                const uint8_t* const* packed, const void* const* w_scale, int scale_dtype,

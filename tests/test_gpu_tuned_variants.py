@@ -267,6 +267,16 @@ def test_tq1_mfma_tiles(bp, K, counts, act, tq1_rows_kernel):
     _check(got, want)
 
 
+@pytest.fixture(params=["staged", "inline"])
+def tq1_gemm_kernel(request, tune):
+    """More than 8 rows per expert, bf16 activations: the grouped GEMM over activations converted into a workspace, one
+    matrix instruction per scale group (kernel name gemm_tq1f_bf16; the default with a workspace, which the mirrored call
+    brings), and the kernel that converts them itself (gemm_tq1_bf16; BP_TUNE_TQ2G=bf16 or no workspace). int8 activations
+    run gemm_tq1_i8 either way."""
+    tune("BP_TUNE_TQ2G", "fp4" if request.param == "staged" else "bf16")
+    return "gemm_tq1f_bf16" if request.param == "staged" else "gemm_tq1_bf16"
+
+
 @pytest.mark.parametrize("act", ["bf16", "int8"])
 @pytest.mark.parametrize(
     "E,N,K,counts,terms",
@@ -278,14 +288,29 @@ def test_tq1_mfma_tiles(bp, K, counts, act, tq1_rows_kernel):
         (3, 64, 1024, [9, 100, 15], 2),          # the smallest K the tuned kernels take; four token tiles in one expert
     ],
 )
-def test_tq1_gemm_tiles(bp, act, E, N, K, counts, terms):
+def test_tq1_gemm_tiles(bp, act, E, N, K, counts, terms, tq1_gemm_kernel):
     got, want, kern = _run(bp, "tq1", E, N, K, counts, act, terms=terms, seed=K + N)
-    assert kern.startswith("gemm_tq1"), kern
+    assert kern == (tq1_gemm_kernel if act == "bf16" else "gemm_tq1_i8"), kern
     _check(got, want)
 
 
+@pytest.mark.parametrize("K", [1024, 1280, 1536, 1792, 2048])  # K % 5 = 4, 0, 1, 2, 3: Kp = 205, 256, 308, 359, 410
+@pytest.mark.parametrize("scale_dtype", [np.float16, "f32", "bf16"])
+def test_tq1_gemm_over_converted_activations_reads_the_last_bytes_of_the_tensor(bp, tune, K, scale_dtype):
+    """The last slice of the last row of the last expert ends at the tensor's last byte, or its 8-byte load one byte
+    past it - and the hardware zeroes a dword that straddles the end of the buffer, valid bytes included, so that wave
+    loads the window byte by byte. Every remainder of K / 5 (= every byte alignment of the rows); N = 48 leaves row tiles
+    of the wave past N, N = 528 a second row block of 16 rows."""
+    tune("BP_TUNE_TQ2G", "fp4")
+    for E, N, counts in ((2, 48, [20, 33]), (2, 528, [1, 40])):
+        got, want, kern = _run(bp, "tq1", E, N, K, counts, "bf16", seed=K, scale_dtype=scale_dtype)
+        # (float32 scales: their ring does not fit in LDS beside the table and the transit area; the other kernel takes the call)
+        assert kern == ("gemm_tq1_bf16" if scale_dtype == "f32" else "gemm_tq1f_bf16"), kern
+        _check(got, want)
+
+
 @pytest.mark.parametrize("ntok", [9, 16, 32])
-def test_tq1_gemm_fp8_pieces_keep_small_activations(bp, ntok):
+def test_tq1_gemm_fp8_pieces_keep_small_activations(bp, ntok, tq1_gemm_kernel):
     """The grouped GEMM splits an activation into two E4M3 pieces under a power-of-two scale per block of 20: exact for
     bf16 values down to 2^-9 of the block's largest magnitude. Activations spread over 5 decades with outliers 1000 x
     the typical value must still come out far inside the general tolerance."""
@@ -300,7 +325,7 @@ def test_tq1_gemm_fp8_pieces_keep_small_activations(bp, ntok):
     for e in range(E):
         c_gemm(x[e * ntok:(e + 1) * ntok], None, packed[0][e], scales[0][e].astype(np.float32), K, GROUP, "tq1", out=want[e * ntok:(e + 1) * ntok])
     got = bp.grouped_ternary_gemm(dev(x).to(torch.bfloat16), None, [0, ntok, 2 * ntok], [dev(packed[0])], [dev(scales[0])], K, GROUP, "tq1").cpu().numpy()
-    assert bp.ext().last_kernel().startswith("gemm_tq1")
+    assert bp.ext().last_kernel() == tq1_gemm_kernel, bp.ext().last_kernel()
     assert rel_l2(got, want) <= 2e-4, rel_l2(got, want)
     z = np.zeros_like(x)  # all-zero activations: the block scale has nothing to go by
     got = bp.grouped_ternary_gemm(dev(z).to(torch.bfloat16), None, [0, ntok, 2 * ntok], [dev(packed[0])], [dev(scales[0])], K, GROUP, "tq1")
@@ -481,9 +506,12 @@ def test_tq2_gemm_over_converted_activations_is_the_default_for_large_prefill(bp
     got = bp.grouped_ternary_gemm(x, None, offsets, pk, sc, K, GROUP, "tq2", max_rows=rows + 13)
     assert bp.ext().last_kernel() == "gemm_tq2f_bf16", bp.ext().last_kernel()
     lib = bp.ext().lib
-    assert lib.bp_grouped_gemm_workspace_bytes(_lib.BP_BF16, E * rows, N, K, E, 2) > 0
-    assert lib.bp_grouped_gemm_workspace_bytes(_lib.BP_I8, E * rows, N, K, E, 2) == 0
-    assert lib.bp_grouped_gemm_workspace_bytes(_lib.BP_BF16, E * rows, N, K, E, 1) == 0
+    assert lib.bp_grouped_gemm_workspace_bytes(_lib.BP_BF16, E * rows, N, K, E, 2, rows + 13) > 0
+    assert lib.bp_grouped_gemm_workspace_bytes(_lib.BP_I8, E * rows, N, K, E, 2, rows + 13) == 0
+    assert lib.bp_grouped_gemm_workspace_bytes(_lib.BP_BF16, E * rows, N, K, E, 1, rows + 13) > 0  # (TQ1: the same kernel with the byte-table decode)
+    assert lib.bp_grouped_gemm_workspace_bytes(_lib.BP_BF16, E * rows, N, K, E, 1, 8) == 0          # (the small-batch kernels take these)
+    # a bound on the rows per expert so loose that most token tiles of the launch would not exist: no staged kernel, no workspace
+    assert lib.bp_grouped_gemm_workspace_bytes(_lib.BP_BF16, E * rows, N, K, E, 2, E * rows) == 0
     tune("BP_TUNE_TQ2G", "bf16")
     want = bp.grouped_ternary_gemm(x, None, offsets, pk, sc, K, GROUP, "tq2", max_rows=rows + 13)
     assert bp.ext().last_kernel().startswith("gemm_tq2_bf16"), bp.ext().last_kernel()
