@@ -98,7 +98,7 @@ struct Plan {
   float* gu;      // f32 [T k, 2 I]
   void* h;        // bf16 [T k, I]
   float* y;       // f32 [T k, H]
-  unsigned char* stage;  // converted activations of the GEMM in flight (TQ2, bf16 activations, more than 64 tokens)
+  unsigned char* stage;  // converted activations of the GEMM in flight (bf16 activations)
   size_t stage_bytes;
   int64_t tile_cap;
   size_t bytes;
@@ -122,7 +122,7 @@ Plan plan(void* workspace, int64_t T, int64_t H, int64_t I, int64_t E, int64_t k
   p.h = c.take(2 * (size_t)n * I);
   p.y = (float*)c.take(4 * (size_t)n * H);
   p.stage_bytes = 0;
-  if (act == BP_BF16 && T > 64) {
+  if (act == BP_BF16) {
     const size_t a = gemm_tq2f_workspace_bytes(n, H, E), b = gemm_tq2f_workspace_bytes(n, I, E);
     p.stage_bytes = a > b ? a : b;
   }
