@@ -147,10 +147,22 @@ extern "C" int bp_ternary_grouped_gemm(float* out, const void* x, int x_dtype, c
                       group, E, fmt, max_rows, nullptr, 0, stream);
 }
 
+static size_t staged_workspace_bytes(int64_t T, int64_t N, int64_t K, int64_t E, int fmt, int64_t max_rows);
+
 extern "C" size_t bp_grouped_gemm_workspace_bytes(int x_dtype, int64_t T, int64_t N, int64_t K, int64_t E, int fmt, int64_t max_rows) {
-  if ((fmt != BP_TQ2 && fmt != BP_TQ1) || x_dtype != BP_BF16 || T <= 0 || E <= 0 || N <= 0) return 0;
-  if (tuning().tq2g == 'b') return 0;
+  if ((fmt != BP_TQ2 && fmt != BP_TQ1) || T <= 0 || E <= 0 || N <= 0 || K <= 0) return 0;
   if (max_rows > T) max_rows = T;
+  if (x_dtype == BP_F32 || x_dtype == BP_F16) {  // split into a bf16 pair where only bf16 activations have tuned kernels
+    if (K % 256 != 0 || K < 1024 || N % 16 != 0 || (fmt == BP_TQ1 && max_rows == 1)) return 0;
+    const size_t pair = 2 * ((((size_t)T * (size_t)K * 2) + 255) & ~(size_t)255);
+    return pair + staged_workspace_bytes(T, N, K, E, fmt, max_rows);
+  }
+  if (x_dtype != BP_BF16) return 0;
+  return staged_workspace_bytes(T, N, K, E, fmt, max_rows);
+}
+
+static size_t staged_workspace_bytes(int64_t T, int64_t N, int64_t K, int64_t E, int fmt, int64_t max_rows) {
+  if (tuning().tq2g == 'b') return 0;
   // (the launcher's own thresholds, so that a call it would turn down does not make its caller allocate)
   if (fmt == BP_TQ2 && tuning().tq2g != 'f' && (N < 1024 || (T + 31) / 32 * ((N + 511) / 512) < 768)) return 0;  // at least two blocks of 512 output rows, three rounds of one workgroup per CU
   if (fmt == BP_TQ1 && max_rows <= 8 && tuning().tq2g != 'f') return 0;  // (the small-batch kernels take these)
@@ -175,7 +187,73 @@ extern "C" int bp_ternary_grouped_gemm_ws(float* out, const void* x, int x_dtype
 namespace bp {
 int kernel_policy() { return g_policy; }
 
+namespace {
+// x = hi + lo + e with hi = bf16(x), lo = bf16(x - hi): |e| <= 2^-17 |x| for float32 x; exact for fp16 x (11 significant
+// bits: 8 in hi, the other 3 in lo). 8 activations per thread.
+template <int XDT>
+__global__ __launch_bounds__(256) void k_split_bf16(uint16_t* __restrict__ hi, uint16_t* __restrict__ lo, const void* __restrict__ x, int64_t n8) {
+  for (int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x; i < n8; i += (int64_t)gridDim.x * 256) {
+    float v[8];
+    if (XDT == BP_F32) {
+      const float4 a0 = ((const float4*)x)[2 * i], a1 = ((const float4*)x)[2 * i + 1];
+      v[0] = a0.x; v[1] = a0.y; v[2] = a0.z; v[3] = a0.w; v[4] = a1.x; v[5] = a1.y; v[6] = a1.z; v[7] = a1.w;
+    } else {
+      const uint4 raw = ((const uint4*)x)[i];
+      const uint32_t w[4] = {raw.x, raw.y, raw.z, raw.w};
+#pragma unroll
+      for (int j = 0; j < 4; ++j) {
+        v[2 * j] = f16_bits_to_f32((uint16_t)(w[j] & 0xffffu));
+        v[2 * j + 1] = f16_bits_to_f32((uint16_t)(w[j] >> 16));
+      }
+    }
+    uint32_t h[4], l[4];
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      const uint16_t h0 = f32_to_bf16_bits(v[2 * j]), h1 = f32_to_bf16_bits(v[2 * j + 1]);
+      const uint16_t l0 = f32_to_bf16_bits(v[2 * j] - bf16_bits_to_f32(h0)), l1 = f32_to_bf16_bits(v[2 * j + 1] - bf16_bits_to_f32(h1));
+      h[j] = (uint32_t)h0 | ((uint32_t)h1 << 16);
+      l[j] = (uint32_t)l0 | ((uint32_t)l1 << 16);
+    }
+    ((uint4*)hi)[i] = make_uint4(h[0], h[1], h[2], h[3]);
+    ((uint4*)lo)[i] = make_uint4(l[0], l[1], l[2], l[3]);
+  }
+}
+
+// float32 / fp16 activations where only bf16 ones have tuned kernels (TQ2, and TQ1 with more than one token row per
+// expert): with a workspace they are split into a bf16 pair and the call runs twice, adding both products into `out`
+// (the kernels accumulate). The weights stream twice - against the general kernel's 0.1 TB/s.
+bool split_applies(const GemmArgs& a) {
+  if (a.x_dtype != BP_F32 && a.x_dtype != BP_F16) return false;
+  if (a.fmt == BP_TQ1 && a.max_rows == 1) return false;  // (the single-token TQ1 kernels take these dtypes as they are)
+  if (a.tiles || ((uintptr_t)a.x & 15) != 0 || a.K % 8 != 0) return false;
+  GemmArgs b = a;
+  b.x_dtype = BP_BF16;
+  return mfma_supports(b);
+}
+size_t split_bytes(int64_t T, int64_t K) { return ((size_t)T * (size_t)K * 2 + 255) & ~(size_t)255; }
+}  // namespace
+
 int run_gemm(const GemmArgs& a, hipStream_t s) {
+  if (g_policy != 1 && a.stage && split_applies(a) && (size_t)a.stage_bytes >= 2 * split_bytes(a.T, a.K)) {
+    const size_t part = split_bytes(a.T, a.K);
+    uint16_t* hi = (uint16_t*)a.stage;
+    uint16_t* lo = (uint16_t*)(a.stage + part);
+    const int64_t n8 = a.T * a.K / 8;
+    int64_t g = (n8 + 255) / 256;
+    if (g > 16384) g = 16384;
+    if (a.x_dtype == BP_F32) hipLaunchKernelGGL(k_split_bf16<BP_F32>, dim3((unsigned)g), dim3(256), 0, s, hi, lo, a.x, n8);
+    else hipLaunchKernelGGL(k_split_bf16<BP_F16>, dim3((unsigned)g), dim3(256), 0, s, hi, lo, a.x, n8);
+    if (const int rc = check_launch("split_bf16")) return rc;
+    GemmArgs b = a;
+    b.x_dtype = BP_BF16;
+    b.stage = a.stage + 2 * part;  // (what is left of the workspace serves the bf16 calls)
+    b.stage_bytes = a.stage_bytes - (int64_t)(2 * part);
+    if (b.stage_bytes <= 0) { b.stage = nullptr; b.stage_bytes = 0; }
+    b.x = hi;
+    if (const int rc = run_gemm(b, s)) return rc;
+    b.x = lo;
+    return run_gemm(b, s);
+  }
   if (g_policy != 1 && mfma_supports(a)) {
     const int rc = launch_mfma(a, s);
     if (rc != BP_ERR_UNSUPPORTED) return rc;  // (a tuned variant may turn a launch down, e.g. when its LDS tiles do not fit)

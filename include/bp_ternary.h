@@ -89,7 +89,11 @@ int bp_ternary_grouped_gemm(float* out, const void* x, int x_dtype, const float*
  * for these arguments; a launch too small for it to pay - TQ2: fewer than 1024 output rows, or fewer than 768 blocks
  * of 32 tokens x 512 rows; or max_rows so loose a bound that most of the launch's token tiles would not exist:
  * ceil(max_rows / 32) * 32 * E > 4 T + 32 E, e.g. the default max_rows = T with more than a few experts):
- * identical to bp_ternary_grouped_gemm. T is the row count of x (all experts), max_rows the bound the call will pass. */
+ * identical to bp_ternary_grouped_gemm. T is the row count of x (all experts), max_rows the bound the call will pass.
+ * float32 and fp16 activations (the reference CPU kernel's float path, boilerplate/kernels/csrc/boilerplate_cpu.cpp:70-77,
+ * 114-124) have tuned kernels only for single-token TQ1 calls; with a workspace every other shape the bf16 kernels cover
+ * runs on them as well: the activations are split into a bf16 pair x = hi + lo (exact for fp16, to 2^-17 |x| for float32)
+ * and both products are added into out. Without one they run on the general kernel. */
 size_t bp_grouped_gemm_workspace_bytes(int x_dtype, int64_t T, int64_t N, int64_t K, int64_t E, int fmt, int64_t max_rows);
 int bp_ternary_grouped_gemm_ws(float* out, const void* x, int x_dtype, const float* x_scale,
                                const int64_t* offsets, const int64_t* offsets_host,

@@ -371,12 +371,14 @@ def test_tq1_fp4_upper_bound_max_rows(bp):
 
 
 def test_tq1_small_batches_other_kernels(bp, tune):
-    """fp16 activations (11 significant bits: more than two fp8 pieces hold) and K that would take more than 4 segments
-    go to the kernels they went to before; the development switch keeps the multi-row MFMA kernel. K = 16384 with 4
+    """fp16 activations (11 significant bits: more than two fp8 pieces hold) run as a pair of bf16 halves (8 + 3 bits) on
+    the same kernel when the call brings a workspace (the mirrored call does); K that would take more than 4 segments
+    goes to the kernels it went to before; the development switch keeps the multi-row MFMA kernel. K = 16384 with 4
     tokens runs as two segments of 13 chunks, with 8 tokens as four of 7 (the last one 5)."""
     got, want, kern = _run(bp, "tq1", 3, 80, 2048, [2, 4, 1], "f16", seed=21)
-    assert not kern.startswith("fp4_tq1"), kern
+    assert kern.startswith("fp4_tq1_m4"), kern
     _check(got, want)
+    assert rel_l2(got, want) <= 1e-5, rel_l2(got, want)  # (the halves are exact; what is left is the pieces' 2^-17)
     got, want, kern = _run(bp, "tq1", 2, 32, 16384, [4, 2], "bf16", seed=22)
     assert kern.startswith("fp4_tq1_m4"), kern
     _check(got, want)
@@ -683,3 +685,38 @@ def test_non_finite_activations_never_give_finite_wrong_values(bp, tune, fmt, co
     ref = bp.grouped_ternary_gemm(dev(x), None, offsets.tolist(), [dev(packed[0])], [dev(scales[0])], K, GROUP, fmt, backend="torch").cpu().numpy()
     assert np.array_equal(~np.isfinite(ref[0]), trits[0][:, 777] != 0)
     assert np.array_equal(~np.isfinite(ref[T - 1]), trits[1][:, 130] != 0)
+
+
+# --------------------------------------------------------------------------- float32 / fp16 activations beyond the single-token TQ1 kernels
+@pytest.mark.parametrize("act", ["f32", "f16"])
+@pytest.mark.parametrize("fmt,M", [("tq2", 1), ("tq2", 8), ("tq1", 8), ("tq2", 40)])
+def test_float_activations_run_on_the_bf16_kernels_as_a_pair(bp, fmt, M, act):
+    """Config 0's inputs (TQ2, K = 4096, N = 2048, M in {1, 8}, float32 activations; the reference runs them on its CPU
+    kernel's float path, boilerplate/kernels/csrc/boilerplate_cpu.cpp:70-77, 114-124) and their fp16 / TQ1 / prefill
+    relatives: split into hi + lo bf16 halves and multiplied by the bf16 kernels, both products added into the output.
+    Held to the reference's own float-path tolerance (tests/test_ternary.py:98: rtol 1e-4, atol 1e-3)."""
+    N, K = 2048, 4096
+    rng = np.random.default_rng(M)
+    packed, scales = synth_weights(5, 1, N, K, GROUP, fmt)
+    x = rng.standard_normal((M, K)).astype(np.float32)
+    if act == "f16":
+        x = x.astype(np.float16).astype(np.float32)
+    xd = dev(x).half() if act == "f16" else dev(x)
+    got = bp.ternary_gemm_float(xd, dev(packed[0][0]), dev(scales[0][0]), K, GROUP, fmt)
+    kern = bp.ext().last_kernel()
+    assert kern.startswith(("mfma_" + fmt, "gemm_" + fmt, "fp4_" + fmt)) and "general" not in kern, kern
+    want = c_gemm(x, None, packed[0][0], scales[0][0].astype(np.float32), K, GROUP, fmt)
+    np.testing.assert_allclose(got.cpu().numpy(), want, rtol=1e-4, atol=1e-3)
+    # without a workspace (the plain C entry point): the general kernel, same numbers
+    out = torch.zeros(M, N, device="cuda")
+    offs = torch.tensor([0, M], device="cuda")
+    bp.ext().lib.bp_set_kernel_policy(0)
+    import ctypes as C
+    from deepseekternarized_amd.kernels import _lib
+    pk, sc = dev(packed[0]), dev(scales[0])
+    pa, sa = (C.c_void_p * 1)(pk.data_ptr()), (C.c_void_p * 1)(sc.data_ptr())
+    rc = bp.ext().lib.bp_ternary_grouped_gemm(out.data_ptr(), xd.data_ptr(), _lib.dtype_code(xd.dtype), None, offs.data_ptr(), None, C.cast(pa, C.c_void_p),
+                                              C.cast(sa, C.c_void_p), _lib.BP_F16, 1, M, N, K, packed[0].shape[-1], K // GROUP, GROUP, 1, 2 if fmt == "tq2" else 1, M, None, None)
+    torch.cuda.synchronize()
+    assert rc == 0 and bp.ext().last_kernel().startswith("general"), bp.ext().last_kernel()
+    np.testing.assert_allclose(out.cpu().numpy(), want, rtol=1e-4, atol=1e-3)
