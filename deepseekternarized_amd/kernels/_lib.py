@@ -12,6 +12,7 @@ BP_I8, BP_BF16, BP_F16, BP_F32 = 0, 1, 2, 3
 BP_TQ1, BP_TQ2 = 1, 2
 BP_ERR_OFFSETS = 2
 BP_MAX_TERMS = 4
+BP_GGUF_TQ1_0, BP_GGUF_TQ2_0 = 34, 35
 
 _p, _i, _l = C.c_void_p, C.c_int, C.c_int64
 
@@ -40,6 +41,9 @@ SIGNATURES = {
     "bp_swiglu_v4": (_i, [_p, _p, _p, _p, _p, _l, C.c_float, _l, _l, _l, _p]),
     "bp_moe_combine_v4": (_i, [_p, _i, _p, _p, _p, _l, _l, _l, _p]),
     "bp_moe_layer_v4": (_i, [_p, _i, _p, _p, _p, C.c_float, _p, _p, _p, _p, _i, _i, _l, _l, _l, _l, _l, _l, _i, _i, _p, C.c_size_t, _p, _p]),
+    "bp_gguf_block_bytes": (_l, [_i]),
+    "bp_gguf_from_ternary": (_i, [_p, _i, _p, _p, _l, _l, _i, _p]),
+    "bp_gguf_to_trits": (_i, [_p, _p, _p, _i, _l, _l, _p]),
     "bp_moe_layer_workspace_bytes": (C.c_size_t, [_l, _l, _l, _l, _l, _i, _i]),
     "bp_moe_layer_bf16": (_i, [_p, _p, _p, _p, _p, _p, _p, _p, _i, _i, _l, _l, _l, _l, _l, _l, _i, _i, _p, C.c_size_t, _p, _p]),
 }

@@ -249,6 +249,22 @@ int bp_moe_layer_v4(void* out, int out_dtype, const void* x, const int64_t* expe
                     int n_terms, int64_t T, int64_t H, int64_t I, int64_t E, int64_t k, int64_t group, int fmt,
                     int act, void* workspace, size_t workspace_bytes, int32_t* bad, void* stream);
 
+/* llama.cpp's TQ1_0 / TQ2_0 blocks (256 weights and one fp16 scale per block; ggml type numbers 34 / 35) from a
+ * single-term ternary weight with group 256 and fp16 scales - what the reference makes by dequantizing the weight and
+ * calling gguf.quants.quantize on the values (boilerplate/format/gguf_export.py:45-58, 103-114): bit-identical blocks,
+ * straight from the packed rows. K must be a multiple of 256, N at most 65535 rows per call.
+ *   blocks  device u8 [N, K / 256, bp_gguf_block_bytes(qtype)] (54 bytes for TQ1_0, 66 for TQ2_0)
+ *   packed  device u8 [N, Kp] in the layout of bp_pack_trits (fmt), scale device fp16 [N, K / 256] */
+#define BP_GGUF_TQ1_0 34
+#define BP_GGUF_TQ2_0 35
+int64_t bp_gguf_block_bytes(int qtype);
+int bp_gguf_from_ternary(uint8_t* blocks, int qtype, const uint8_t* packed, const void* scale, int64_t N, int64_t K,
+                         int fmt, void* stream);
+/* The other way: such blocks decoded to trits i8 [N, K] (digit - 1) and their scales fp16 [N, K / 256]; bp_pack_trits
+ * then gives the packed rows of either format. trit * scale equals gguf.quants.dequantize of the blocks bit for bit
+ * (the check of boilerplate/format/gguf_export.py:109-113 and tests/test_gguf_export.py:54-75). */
+int bp_gguf_to_trits(int8_t* trits, void* scale, const uint8_t* blocks, int qtype, int64_t N, int64_t K, void* stream);
+
 #ifdef __cplusplus
 }
 #endif

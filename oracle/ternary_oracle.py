@@ -372,3 +372,90 @@ def moe_layer_v4_ref(x_bf16, weights, indices, experts, K_hidden: int, K_inter: 
         for i, tok in enumerate(token):
             y[tok] = (y[tok] + d[i]).astype(np.float32)
     return y
+
+
+# --------------------------------------------------------------------------- ggml TQ1_0 / TQ2_0 blocks (GGUF interop)
+# boilerplate/format/gguf_export.py:103-114 (`quantize_exact`) hands the dequantized values of a single-term, group-256,
+# fp16-scale ternary weight to `gguf.quants.quantize(arr, TQ1_0 | TQ2_0)` of the `gguf` Python package (llama.cpp's
+# gguf-py; the reference asks for `pip install gguf` without a version) and checks that `gguf.quants.dequantize` gives
+# the values back bit for bit. That package is not vendored in the reference and is absent here, so the functions
+# below restate the published block layout and algorithm of llama.cpp (ggml/src/ggml-common.h `block_tq1_0` /
+# `block_tq2_0`, ggml/src/ggml-quants.c `quantize_row_tq{1,2}_0_ref` / `dequantize_row_tq{1,2}_0`), which gguf-py's
+# quants.py mirrors. PARITY UNPINNED against the package itself: pinned by hand-worked blocks from those formulas, the
+# exhaustive digit round trip and the exact value round trip the reference's own test asks for
+# (tests/test_gguf_export.py:54-75), nothing more.
+GGUF_QK = 256
+GGUF_TQ1_0_BYTES = 54  # qs[48] (5 trits per byte) + qh[4] (4 trits per byte) + fp16 d
+GGUF_TQ2_0_BYTES = 66  # qs[64] (4 trits per byte) + fp16 d
+
+
+def _gguf_digits(values: np.ndarray) -> tuple[np.ndarray, np.ndarray]:
+    """Per block of 256: d = fp16(max |x|), digits xi = lroundf(x * (1 / d)) + 1 in 0..2 (d = 0: all 1)."""
+    v = np.asarray(values, np.float32)
+    if v.ndim != 2 or v.shape[1] % GGUF_QK:
+        raise ValueError("values must be [N, K] with K a multiple of 256")
+    blk = v.reshape(v.shape[0], -1, GGUF_QK)
+    d = np.abs(blk).max(-1).astype(np.float32)
+    with np.errstate(divide="ignore"):
+        inv = np.where(d > 0, np.float32(1.0) / d, np.float32(0.0)).astype(np.float32)
+    t = (blk * inv[..., None]).astype(np.float32)
+    xi = (np.sign(t) * np.floor(np.abs(t) + np.float32(0.5))).astype(np.int64) + 1  # lroundf: halves away from zero
+    return d.astype(np.float16), xi
+
+
+def _tq1_byte(digits: np.ndarray) -> np.ndarray:
+    """digits [..., n] most significant first -> ceil(q * 256 / 243) with q = sum digit * 3^(4 - i) (n = 4: times 3)."""
+    q = np.zeros(digits.shape[:-1], np.int64)
+    for i in range(digits.shape[-1]):
+        q = q * 3 + digits[..., i]
+    if digits.shape[-1] == 4:
+        q = q * 3
+    return ((q * 256 + 242) // 243).astype(np.uint8)
+
+
+def gguf_quantize(values: np.ndarray, qtype: str) -> np.ndarray:
+    """[N, K] float32 -> uint8 [N, K / 256 * block bytes] of TQ1_0 / TQ2_0 blocks (quantize_row_tq{1,2}_0_ref)."""
+    d, xi = _gguf_digits(values)
+    N, nb = d.shape
+    dbytes = d.view(np.uint8).reshape(N, nb, 2)
+    if qtype == "tq2_0":
+        # two chunks of 128 elements: byte m of a chunk holds elements m, m + 32, m + 64, m + 96 at bits 0, 2, 4, 6
+        c = xi.reshape(N, nb, 2, 4, 32)
+        qs = (c[:, :, :, 0] | (c[:, :, :, 1] << 2) | (c[:, :, :, 2] << 4) | (c[:, :, :, 3] << 6)).astype(np.uint8).reshape(N, nb, 64)
+        return np.concatenate([qs, dbytes], -1).reshape(N, nb * GGUF_TQ2_0_BYTES)
+    if qtype == "tq1_0":
+        a = xi[:, :, :160].reshape(N, nb, 5, 32)          # element m + 32 n -> byte m, digit n
+        b = xi[:, :, 160:240].reshape(N, nb, 5, 16)       # element 160 + m + 16 n -> byte 32 + m, digit n
+        h = xi[:, :, 240:].reshape(N, nb, 4, 4)           # element 240 + j + 4 m -> qh[j], digit m
+        qs = np.concatenate([_tq1_byte(np.moveaxis(a, 2, -1)), _tq1_byte(np.moveaxis(b, 2, -1))], -1)
+        qh = _tq1_byte(np.moveaxis(h, 2, -1))
+        return np.concatenate([qs, qh, dbytes], -1).reshape(N, nb * GGUF_TQ1_0_BYTES)
+    raise ValueError(f"unknown ggml type {qtype!r}")
+
+
+def gguf_dequantize(blocks: np.ndarray, qtype: str, K: int) -> np.ndarray:
+    """uint8 blocks [N, ...] -> float32 [N, K] (dequantize_row_tq{1,2}_0): (digit - 1) * d."""
+    blocks = np.asarray(blocks, np.uint8)
+    N = blocks.shape[0]
+    nb = K // GGUF_QK
+    if qtype == "tq2_0":
+        b = blocks.reshape(N, nb, GGUF_TQ2_0_BYTES)
+        qs = b[:, :, :64].reshape(N, nb, 2, 1, 32).astype(np.int64)
+        dig = (qs >> (2 * np.arange(4)).reshape(1, 1, 1, 4, 1)) & 3
+        d = np.ascontiguousarray(b[:, :, 64:]).view(np.float16).reshape(N, nb).astype(np.float32)
+        return ((dig.reshape(N, nb, GGUF_QK) - 1).astype(np.float32) * d[..., None]).reshape(N, K)
+    if qtype == "tq1_0":
+        b = blocks.reshape(N, nb, GGUF_TQ1_0_BYTES)
+        pow3 = np.array([1, 3, 9, 27, 81], np.int64)
+
+        def digits(q, n):  # digit i (most significant first) of each byte: ((q * 3^i mod 256) * 3) >> 8
+            qq = (q.astype(np.int64)[..., None, :] * pow3[:n].reshape(-1, 1)) & 0xFF
+            return (qq * 3) >> 8
+
+        a = digits(b[:, :, :32], 5).reshape(N, nb, 160)
+        c = digits(b[:, :, 32:48], 5).reshape(N, nb, 80)
+        h = digits(b[:, :, 48:52], 4).reshape(N, nb, 16)
+        d = np.ascontiguousarray(b[:, :, 52:]).view(np.float16).reshape(N, nb).astype(np.float32)
+        dig = np.concatenate([a, c, h], -1)
+        return ((dig - 1).astype(np.float32) * d[..., None]).reshape(N, K)
+    raise ValueError(f"unknown ggml type {qtype!r}")
