@@ -61,6 +61,8 @@ def arithmetic_of(kernel):
         return "activations as 3 E4M3 pieces under a per-group power-of-two prescale x E2M1 weights (v_mfma_f32_16x16x128_f8f6f4), fp32 accumulate, fp16 scale per 128-group applied in fp32"
     if kernel.startswith("fp4_tq1_m"):
         return "activations as 2 E4M3 pieces under a per-group power-of-two prescale x E2M1 weights (v_mfma_f32_16x16x128_f8f6f4), fp32 accumulate"
+    if kernel.startswith("gemm_tq1f"):
+        return "activations as 2 E4M3 pieces under E8M0 block scales (blocks of 32), converted once into a workspace, x E2M1 weights strung together from a byte table, one v_mfma_scale_f32_16x16x128_f8f6f4 per 128-group, fp32 accumulate, scale per group applied in fp32"
     if kernel.startswith("gemm_tq1"):
         return "activations as 2 E4M3 pieces under E8M0 block scales (blocks of 20) x E2M1 weights (v_mfma_scale_f32_16x16x128_f8f6f4), fp32 accumulate, scale per 128-group applied in fp32"
     if kernel.startswith("gemm_tq2f"):
@@ -142,8 +144,9 @@ class Launch:
             self()
         # The boxes show an occasional stall of ~30 ms in the middle of back-to-back launches (about one per several
         # seconds, whatever the kernel). A timed sequence in which one launch took more than 20 x the median launch
-        # is taken again, once; `self.retimed` says so.
-        self.retimed = 0
+        # is taken again, once; `self.retimed` says so and `self.stalled` keeps what the discarded sequence measured
+        # (its mean and its slowest launch, in microseconds).
+        self.retimed, self.stalled = 0, None
         for attempt in range(2):
             ev = [(torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)) for _ in range(steps)]
             torch.cuda.synchronize()
@@ -157,9 +160,13 @@ class Launch:
             each = sorted(a.elapsed_time(b) for a, b in ev)
             if attempt == 0 and steps >= 5 and each[-1] > 20.0 * each[len(each) // 2]:
                 self.retimed = 1
+                self.stalled = {"mean_us": round(sum(each) / steps * 1e3, 2), "slowest_launch_us": round(each[-1] * 1e3, 1),
+                                "median_us": round(each[len(each) // 2] * 1e3, 2), "wall_us_per_step": round(wall * 1e6, 2)}
                 continue
             break
         kern = sum(each) / steps / 1e3
+        # the spread of the per-launch times (HIP events around each launch, microseconds)
+        self.spread = {"median": round(each[len(each) // 2] * 1e3, 2), "min": round(each[0] * 1e3, 2), "max": round(each[-1] * 1e3, 2)}
         return wall, kern, self.e.last_kernel()
 
 
@@ -291,7 +298,8 @@ def run_cfg3_grouped(bp, torch, a) -> int:
                    "retimed_after_stall": launch.retimed, "weight_GBps": round(wbytes / kern / 1e9, 1)},
         "roofline": {"bound": "mfma", "achieved": round(flops / kern / 1e12, 1), "peak": MFMA_BF16_PEAK_TFLOPS, "unit": "TFLOP/s",
                      "frac": round(flops / kern / 1e12 / MFMA_BF16_PEAK_TFLOPS, 4), "traffic": measured_traffic("cfg3_grouped", kname),
-                     "kernel_us": round(kern * 1e6, 2)},
+                     "kernel_us": round(kern * 1e6, 2), "kernel_us_median": launch.spread["median"], "kernel_us_min": launch.spread["min"],
+                     "kernel_us_max": launch.spread["max"]},
         "cpu_baseline": None, "also": {}})
 
 
@@ -323,6 +331,31 @@ def run_cfg2_moe(bp, torch, a, T2) -> int:
         "cpu_baseline": None, "also": {}})
 
 
+def run_cfg4_decoder(bp, torch, a, graph: bool) -> int:
+    """Config 4: the OLMoE-shaped Mode D decoder harness, batch 64, 128 prompt + 128 greedy decode tokens (one HIP graph
+    per decode step with `graph`); value = decode tokens per second."""
+    from deepseekternarized_amd.decoder_harness import DecoderConfig, TernaryDecoder, bench_decoder
+
+    cfg = DecoderConfig()
+    model = TernaryDecoder(cfg)
+    r = bench_decoder(model, 64, 128, 128, graph=graph)
+    weight_bytes_per_step = cfg.layers * (4 * (cfg.hidden * cfg.hidden // 4 + 2 * cfg.hidden * cfg.hidden // GROUP)
+                                          + cfg.experts * 3 * (cfg.inter * cfg.hidden // 4 + 2 * cfg.inter * cfg.hidden // GROUP))
+    step_s = 64.0 / r["decode_tok_s"]
+    return emit({
+        "metric": "ternary GEMV HBM GB/s (% peak); grouped-expert GEMM TFLOP/s (% MFMA peak)",
+        "value": round(r["decode_tok_s"], 1), "unit": "tok/s", "n_gpus": 1, "steps": 128, "warmup": 0,
+        "ms_per_step": round(step_s * 1e3, 4), "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+        "dtype": cfg.act, "data": "synthetic",
+        "config": {"workload": f"cfg4_decode{'_graph' if graph else ''}: {cfg.layers} layers, hidden {cfg.hidden}, {cfg.experts} experts top-{cfg.top_k}, inter {cfg.inter}, "
+                               f"{cfg.fmt.upper()}, {cfg.act} activations, random weights; batch 64, prompt 128, 128 greedy decode steps",
+                   "prefill_tok_s": r["prefill_tok_s"], "peak_vram_bytes": r["peak_vram_bytes"], "finite": r["finite"]},
+        "roofline": {"bound": "hbm", "achieved": round(weight_bytes_per_step / step_s / 1e9, 1), "peak": HBM_PEAK_GBPS, "unit": "GB/s",
+                     "frac": round(weight_bytes_per_step / step_s / 1e9 / HBM_PEAK_GBPS, 4), "traffic": None,
+                     "note": "all ternary weights of the model (every expert is active at batch 64) per decode step by wall clock; not one kernel"},
+        "cpu_baseline": None, "also": {}})
+
+
 def main() -> int:
     global SPIN_UP_S
     ap = argparse.ArgumentParser(description=__doc__.split("\n\n")[0])
@@ -330,7 +363,7 @@ def main() -> int:
     ap.add_argument("--steps", type=int, default=200)
     ap.add_argument("--warmup", type=int, default=20)
     ap.add_argument("--spin-up", type=float, default=SPIN_UP_S, help="seconds of untimed launches before warm-up and timed steps (0: none, for counter runs)")
-    ap.add_argument("--workload", default="cfg1a_tq1_gemv", choices=sorted(WORKLOADS) + ["cfg3_grouped", "cfg2_moe_T1", "cfg2_moe_T32", "cfg2_moe_T256"])
+    ap.add_argument("--workload", default="cfg1a_tq1_gemv", choices=sorted(WORKLOADS) + ["cfg3_grouped", "cfg2_moe_T1", "cfg2_moe_T32", "cfg2_moe_T256", "cfg4_decode", "cfg4_decode_graph"])
     ap.add_argument("--no-extras", action="store_true", help="skip the secondary measurements")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline")
     ap.add_argument("--calibrate-copy", action="store_true",
@@ -361,10 +394,12 @@ def main() -> int:
         return run_cfg3_grouped(bp, torch, a)
     if a.workload.startswith("cfg2_moe_T"):
         return run_cfg2_moe(bp, torch, a, int(a.workload[len("cfg2_moe_T"):]))
+    if a.workload.startswith("cfg4_decode"):
+        return run_cfg4_decoder(bp, torch, a, a.workload.endswith("_graph"))
     fmt, N, K, M, act, terms, L = WORKLOADS[a.workload]
     launch, wbytes = uniform_launch(bp, torch, fmt, N, K, M, act, terms, L)
     wall, kern, kname = launch.time(a.steps, a.warmup)
-    retimed = launch.retimed
+    retimed, stalled, spread = launch.retimed, launch.stalled, launch.spread
     act_bytes = L * M * K * 2 + L * M * N * 4 * 2  # bf16 activations read, f32 output read-modify-write
 
     also = {}
@@ -376,6 +411,7 @@ def main() -> int:
             _, k2, kn2 = l2.time(max(5, a.steps // 2), 2)
             also[f"M{m}_weight_GBps"] = round(wb2 / k2 / 1e9, 1)
             also[f"M{m}_kernel"] = kn2
+            also[f"M{m}_us"] = round(k2 * 1e6, 1)
             del l2
             torch.cuda.empty_cache()
         for name in ("cfg1a_tq2_gemv", "cfg1a_tq2_i8_gemv", "cfg1b_tq1_gemv"):  # the same GEMV in the other formats / shapes
@@ -464,11 +500,14 @@ def main() -> int:
         "config": {"workload": f"{a.workload}: {fmt.upper()} decode GEMV N={N} K={K} M={M} {act} activations, group 128, "
                                f"fp16 scales, {L} distinct linears per launch ({wbytes / 1e6:.0f} MB of weights, > Infinity Cache)",
                    "kernel": kname, "arithmetic": arithmetic_of(kname), "bytes_counted": "packed + fp16 scales as stored", "device_spin_up_s": SPIN_UP_S, "retimed_after_stall": retimed,
+                   "discarded_sequence_with_stall": stalled,
                    "packed_only_GBps": round(wbytes * (1.0 - 2.0 * (K // GROUP) / (bp.packed_cols(fmt, K) + 2.0 * (K // GROUP))) / kern / 1e9, 1),
                    "activation_and_output_bytes_per_step": act_bytes},
         "roofline": {"bound": "hbm", "achieved": round(wbytes / kern / 1e9, 1), "peak": HBM_PEAK_GBPS, "unit": "GB/s",
                      "frac": round(wbytes / kern / 1e9 / HBM_PEAK_GBPS, 4), "traffic": measured_traffic(a.workload, kname),
-                     "kernel_us": round(kern * 1e6, 2)},
+                     "kernel_us": round(kern * 1e6, 2), "kernel_us_median": spread["median"], "kernel_us_min": spread["min"],
+                     "kernel_us_max": spread["max"],
+                     "note": "achieved / frac use the MEAN launch duration over the timed steps (HIP events on the launch stream)"},
         "cpu_baseline": None if a.no_cpu else cpu_baseline(fmt, N, K, M),
         "also": also,
     }

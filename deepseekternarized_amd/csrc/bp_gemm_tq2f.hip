@@ -173,7 +173,8 @@ __global__ __launch_bounds__(F_THREADS) void k_stage_tq2f(GemmArgs a) {
   if (kbA == 0 && hi == 0) *(float*)(dst + F_OPS + F_SCL + (sg * 32 + 16 * stt + sm) * 4) = -part;
 }
 
-template <int SDT, int FMT>
+// GS = 1: scale groups of 256 (the two groups of a window share a scale); 0: of 128.
+template <int SDT, int FMT, int GS>
 __global__ __launch_bounds__(F_THREADS, 2) void k_gemm_tq2f(GemmArgs a) {
   constexpr int SB = SDT == BP_F32 ? 4 : 2;
   constexpr bool Q1 = FMT == BP_TQ1;
@@ -193,7 +194,7 @@ __global__ __launch_bounds__(F_THREADS, 2) void k_gemm_tq2f(GemmArgs a) {
 
   const int nwin = (int)(a.K / 256);      // 64-byte windows of a row = pairs of 128-wide groups
   const int NW = nwin * a.n_terms;        // the stacked terms, one after the other
-  const int gs = a.group == 256 ? 1 : 0;  // scale groups of 256: the two groups of a window share a scale
+  constexpr int gs = GS;
 
   const unsigned alane = LB + (unsigned)(kb * 512 + r16 * 16);
   if constexpr (Q1) {  // the byte table: two threads per byte value, 32 copies each
@@ -639,12 +640,12 @@ __global__ __launch_bounds__(F_THREADS, 2) void k_gemm_tq2f(GemmArgs a) {
   else all_windows(FC<1>{});
 }
 
-template <int SDT, int FMT>
-int launch_gemm_tq2f_k(const GemmArgs& a, hipStream_t s) {
+template <int SDT, int FMT, int GS>
+int launch_gemm_tq2f_g(const GemmArgs& a, hipStream_t s) {
   constexpr int LDS = f_lds_bytes(SDT == BP_F32 ? 4 : 2) + (FMT == BP_TQ1 ? F_LUT + F_WAVES * F_RT * F_TR : 0);
   static_assert(LDS <= 160 * 1024, "LDS of a workgroup");
   const char* name = FMT == BP_TQ1 ? "gemm_tq1f_bf16" : "gemm_tq2f_bf16";
-  if (const int rc = raise_lds_limit<k_gemm_tq2f<SDT, FMT>>(LDS)) return rc;
+  if (const int rc = raise_lds_limit<k_gemm_tq2f<SDT, FMT, GS>>(LDS)) return rc;
   const int64_t row_blocks = (a.N + F_ROWS - 1) / F_ROWS;
   const int64_t wgs = tile_workgroups(a, row_blocks);
   if (wgs < 0) return BP_ERR_UNSUPPORTED;
@@ -654,8 +655,13 @@ int launch_gemm_tq2f_k(const GemmArgs& a, hipStream_t s) {
   if (const int rc = check_launch("stage_tq2f")) return rc;
   const dim3 grid((unsigned)wgs, 1, 1);
   note_kernel(name);
-  hipLaunchKernelGGL((k_gemm_tq2f<SDT, FMT>), grid, dim3(F_THREADS), LDS, s, a);
+  hipLaunchKernelGGL((k_gemm_tq2f<SDT, FMT, GS>), grid, dim3(F_THREADS), LDS, s, a);
   return check_launch(name);
+}
+
+template <int SDT, int FMT>
+int launch_gemm_tq2f_k(const GemmArgs& a, hipStream_t s) {
+  return a.group == 256 ? launch_gemm_tq2f_g<SDT, FMT, 1>(a, s) : launch_gemm_tq2f_g<SDT, FMT, 0>(a, s);
 }
 
 }  // namespace
