@@ -44,6 +44,7 @@ SIGNATURES = {
     "bp_gguf_block_bytes": (_l, [_i]),
     "bp_gguf_from_ternary": (_i, [_p, _i, _p, _p, _l, _l, _i, _p]),
     "bp_gguf_to_trits": (_i, [_p, _p, _p, _i, _l, _l, _p]),
+    "bp_huff_decode": (_i, [_p, _l, _p, _l, _p, _p, _l, _l, _p, _p, _l, _p, _l, _p, _p]),
     "bp_moe_layer_workspace_bytes": (C.c_size_t, [_l, _l, _l, _l, _l, _i, _i]),
     "bp_moe_layer_bf16": (_i, [_p, _p, _p, _p, _p, _p, _p, _p, _i, _i, _l, _l, _l, _l, _l, _l, _i, _i, _p, C.c_size_t, _p, _p]),
 }

@@ -265,6 +265,22 @@ int bp_gguf_from_ternary(uint8_t* blocks, int qtype, const uint8_t* packed, cons
  * (the check of boilerplate/format/gguf_export.py:109-113 and tests/test_gguf_export.py:54-75). */
 int bp_gguf_to_trits(int8_t* trits, void* scale, const uint8_t* blocks, int qtype, int64_t N, int64_t K, void* stream);
 
+/* Mode B: canonical-Huffman decode of weight bytes on the device (the device decoder of
+ * boilerplate/kernels/csrc/huffman_cuda_kernel.cu:12-79 `huff_decode_into_cuda`; stream layout
+ * boilerplate/format/entropy.py:13-18): symbols in blocks of `block`, codes MSB-first back to back, offsets[b] = bit
+ * where block b starts (offsets[blocks] = total bits), every block decoded independently through the 2^maxlen-entry
+ * table lut[prefix] = (symbol << 8) | length. raw_bytes = 0: out[i] = symbol i (1-byte formats); else out[2 i] =
+ * raw[i], out[2 i + 1] = symbol i (2-byte formats: the coded high byte next to the stored low byte).
+ *   out, stream, offsets (i64 [blocks + 1]), lut (i32 [2^maxlen]), raw: device memory; stream_bytes >= 4 (padding)
+ *   offsets_host / lut_host: optional host copies; when given they are validated exactly as the reference validates
+ *       them (huffman_validation.h:16-41), without any device-to-host copy; NULL skips those checks
+ *   error   device i32, cleared by the caller: set to 1 when a block's bits are invalid or truncated (where the
+ *       reference raises "invalid or truncated Huffman bitstream"); no memory outside the stream, the table and the
+ *       output is touched whatever the stream holds. */
+int bp_huff_decode(uint8_t* out, int64_t out_bytes, const uint8_t* stream, int64_t stream_bytes, const int64_t* offsets,
+                   const int64_t* offsets_host, int64_t n, int64_t block, const int32_t* lut, const int32_t* lut_host,
+                   int64_t maxlen, const uint8_t* raw, int64_t raw_bytes, int32_t* error, void* stream_handle);
+
 #ifdef __cplusplus
 }
 #endif
