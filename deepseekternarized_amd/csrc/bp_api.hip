@@ -36,7 +36,7 @@ namespace {
 std::atomic<const Tuning*> g_tuning{nullptr};
 std::once_flag g_tuning_once;
 void read_tuning() {
-  Tuning* t = new Tuning{0, 0, 0, 0, 0, -1, 0};
+  Tuning* t = new Tuning{0, 0, 0, 0, 0, -1, 0, -1};
   if (const char* v = getenv("BP_TUNE_R")) t->r = atoi(v);
   if (const char* v = getenv("BP_TUNE_WAVES")) t->waves = atoi(v);
   if (const char* v = getenv("BP_TUNE_TQ1")) t->tq1 = v[0];
@@ -44,6 +44,7 @@ void read_tuning() {
   if (const char* v = getenv("BP_TUNE_F4W")) t->f4w = atoi(v);
   if (const char* v = getenv("BP_TUNE_F4T")) t->f4t = atoi(v);
   if (const char* v = getenv("BP_TUNE_CPT")) t->cpt = atoi(v);
+  if (const char* v = getenv("BP_TUNE_TILES")) t->tiles = atoi(v);
   g_tuning.store(t, std::memory_order_release);
 }
 }  // namespace

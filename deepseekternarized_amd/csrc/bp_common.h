@@ -97,6 +97,7 @@ struct Tuning {
   int f4w;     // BP_TUNE_F4W: waves per workgroup of the fp8 x fp4 GEMV (8, 16)
   int f4t;     // BP_TUNE_F4T: routed rows per expert up to which launches of 8 rows are used (-1 = default)
   int cpt;     // BP_TUNE_CPT: chunks per table pass of the table-lookup GEMV
+  int tiles;   // BP_TUNE_TILES: tokens from which bp_moe_layer_* runs its GEMMs over the device-side list of token tiles (-1 = default)
 };
 const Tuning& tuning();
 

@@ -75,6 +75,61 @@ __global__ __launch_bounds__(256) void k_zero16(u32x4* __restrict__ p, int64_t n
   for (int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x; i < n16; i += (int64_t)gridDim.x * 256) p[i] = u32x4{0u, 0u, 0u, 0u};
 }
 
+// A few routed rows (n <= ROUTE_SMALL_N): the layer's whole preparation in one launch instead of five - stable sort of
+// the expert ids (every workgroup ranks the ids for itself in LDS: element i goes to slot #(ids below id_i) + #(equal
+// ids before i); workgroup 0 writes order, offsets and the inverse permutation), the row gather xg[r] = x[order[r] / k],
+// and the zero-fill of the two float32 outputs that the small-batch kernels accumulate into.
+constexpr int ROUTE_SMALL_N = 256, ROUTE_SMALL_THREADS = 256;
+__global__ __launch_bounds__(ROUTE_SMALL_THREADS) void k_route_small(int64_t* __restrict__ order, int64_t* __restrict__ offsets, int64_t* __restrict__ inv,
+                                                                     const int64_t* __restrict__ ids, int n, int64_t E, int32_t* __restrict__ bad,
+                                                                     u32x4* __restrict__ xg, const u32x4* __restrict__ x, int k, int64_t T, int64_t row16,
+                                                                     u32x4* __restrict__ z0, int64_t z0_16, u32x4* __restrict__ z1, int64_t z1_16) {
+  __shared__ int32_t sid[ROUTE_SMALL_N];
+  __shared__ int32_t ord[ROUTE_SMALL_N];
+  const int i = threadIdx.x;
+  int32_t mine = 0x7fffffff;  // an id outside [0, E) is left out of the order, as in bp_sort_by_expert
+  if (i < n) {
+    const int64_t id = ids[i];
+    if (id >= 0 && id < E) mine = (int32_t)id;
+    else if (bad && blockIdx.x == 0) *bad = 1;
+  }
+  sid[i] = mine;
+  ord[i] = -1;
+  __syncthreads();
+  if (i < n && mine != 0x7fffffff) {
+    int rank = 0;
+    for (int j = 0; j < n; ++j) {
+      const int32_t v = sid[j];
+      rank += (v < mine || (v == mine && j < i)) ? 1 : 0;
+    }
+    ord[rank] = i;
+    if (blockIdx.x == 0) {
+      order[rank] = i;
+      inv[i] = rank;
+    }
+  }
+  if (blockIdx.x == 0) {
+    for (int64_t e = i; e <= E; e += ROUTE_SMALL_THREADS) {
+      int cnt = 0;
+      for (int j = 0; j < n; ++j) cnt += sid[j] < e ? 1 : 0;
+      offsets[e] = cnt;
+    }
+  }
+  __syncthreads();
+  const int64_t gtid = (int64_t)blockIdx.x * ROUTE_SMALL_THREADS + i, gsz = (int64_t)gridDim.x * ROUTE_SMALL_THREADS;
+  for (int64_t w = gtid; w < (int64_t)n * row16; w += gsz) {  // 16 bytes of a gathered row
+    const int64_t r = w / row16, c = w - r * row16;
+    const int o = ord[r];
+    if (o >= 0) {
+      int64_t src = o / k;
+      src = src < T ? src : T - 1;
+      xg[r * row16 + c] = x[src * row16 + c];
+    }
+  }
+  for (int64_t w = gtid; w < z0_16; w += gsz) z0[w] = u32x4{0u, 0u, 0u, 0u};
+  for (int64_t w = gtid; w < z1_16; w += gsz) z1[w] = u32x4{0u, 0u, 0u, 0u};
+}
+
 struct Carve {
   unsigned char* base;
   size_t used;
@@ -176,11 +231,30 @@ static int moe_layer(bool v4, void* out, int out_dtype, float limit, const void*
   const int64_t n = T * k;
   const int per = fmt == BP_TQ2 ? 4 : 5;
 
-  int rc = bp_sort_by_expert(p.order, p.offsets, experts, n, E, bp_sort_workspace_ints(n, E) > 0 ? p.sort_ws : nullptr, bad, s);
-  if (rc != BP_OK) return rc;
-  hipLaunchKernelGGL(k_invert, dim3((unsigned)((n + 255) / 256)), dim3(256), 0, s, p.inv, p.order, n);
-  if ((rc = check_launch("invert")) != BP_OK) return rc;
-  if ((rc = bp_gather_rows(p.xg, x, p.order, k, n, T, 2 * H, s)) != BP_OK) return rc;
+  int rc = BP_OK;
+  // (the outputs' zero-fill rides along only where both GEMMs are going to accumulate: no tile list, and a policy that
+  // lets them run; rows of 16-byte multiples: H % 8 == 0 is checked above)
+  // Tokens beyond which the GEMMs run over the tile list. Up to 64 no expert can have more than 64 rows and the small-batch
+  // kernels take the launch by that bound; TQ1 with bf16 activations changes over at 24 already: the launches of 8 rows
+  // cost what their widest expert costs (an expert with 9 rows means a second pass over few CUs), the tile kernel a flat
+  // 0.23 ms from 24 to 64 tokens on config 2's layer, where the small-batch kernels take 0.25 - 0.26 (and 0.18 - 0.21 below).
+  const int64_t tiles_from = tuning().tiles >= 0 ? tuning().tiles : (fmt == BP_TQ1 && act == BP_BF16 ? 24 : 64);
+  const bool tiles = T > tiles_from;
+  const bool small = n <= ROUTE_SMALL_N && !tiles && (((uintptr_t)x | (uintptr_t)p.xg) & 15) == 0;
+  if (small) {
+    const int64_t z0 = (int64_t)(4 * (size_t)n * 2 * I / 16), z1 = (int64_t)(4 * (size_t)n * H / 16);
+    int64_t g = (z0 + z1 + (int64_t)n * (H / 8) + ROUTE_SMALL_THREADS - 1) / ROUTE_SMALL_THREADS;
+    g = g < 1 ? 1 : (g > 256 ? 256 : g);
+    hipLaunchKernelGGL(k_route_small, dim3((unsigned)g), dim3(ROUTE_SMALL_THREADS), 0, s, p.order, p.offsets, p.inv, experts, (int)n, E, bad,
+                       (u32x4*)p.xg, (const u32x4*)x, (int)k, T, H / 8, (u32x4*)p.gu, z0, (u32x4*)p.y, z1);
+    if ((rc = check_launch("route_small")) != BP_OK) return rc;
+  } else {
+    rc = bp_sort_by_expert(p.order, p.offsets, experts, n, E, bp_sort_workspace_ints(n, E) > 0 ? p.sort_ws : nullptr, bad, s);
+    if (rc != BP_OK) return rc;
+    hipLaunchKernelGGL(k_invert, dim3((unsigned)((n + 255) / 256)), dim3(256), 0, s, p.inv, p.order, n);
+    if ((rc = check_launch("invert")) != BP_OK) return rc;
+    if ((rc = bp_gather_rows(p.xg, x, p.order, k, n, T, 2 * H, s)) != BP_OK) return rc;
+  }
 
   auto gemm = [&](float* o, const void* in, const uint8_t* const* packed, const void* const* scale, int64_t N, int64_t K, bool tiles) -> int {
     GemmArgs a;
@@ -211,10 +285,10 @@ static int moe_layer(bool v4, void* out, int out_dtype, float limit, const void*
       }
       a.tiles = nullptr;  // no tile kernel for this shape: the launch covers the bound (every expert up to T rows)
     }
-    if (const int z = zero(o, 4 * (size_t)n * N, s)) return z;
+    if (!small)
+      if (const int z = zero(o, 4 * (size_t)n * N, s)) return z;
     return run_gemm(a, s);
   };
-  const bool tiles = T > 64;
   if (tiles) {
     hipLaunchKernelGGL(k_tile_list, dim3(1), dim3(1024), 0, s, p.tiles, p.tile_count, p.offsets, E, n, p.tile_cap);
     if ((rc = check_launch("tile_list")) != BP_OK) return rc;

@@ -82,29 +82,36 @@ class _HipTernary:
             host = host_t.data_ptr()
         pk = (C.c_void_p * len(packed_l))(*[p.data_ptr() for p in packed_l])
         sc = (C.c_void_p * len(scale_l))(*[s.data_ptr() for s in scale_l])
-        with torch.cuda.device(out.device):
+        dev = out.device
+        xdt, index = _lib.dtype_code(x.dtype), dev.index if dev.index is not None else torch.cuda.current_device()
+        switch = torch.cuda.current_device() != index  # (entering a device context costs microseconds: only when it changes anything)
+        if switch:
+            prev = torch.cuda.current_device()
+            torch.cuda.set_device(index)
+        try:
+            stream = torch._C._cuda_getCurrentRawStream(index)
             # Prefill-sized calls get a workspace (the library allocates nothing itself): with one, the grouped GEMM kernels
-            # for bf16 activations convert the activations once instead of once per block of output rows. The size query
-            # answers 0 where the launch would not use one (small calls, a loose max_rows).
-            need = self.lib.bp_grouped_gemm_workspace_bytes(_lib.dtype_code(x.dtype), T, N, int(K), E, int(fmt), int(max_rows))
-            if need > _WORKSPACE_CAP:  # (about 2.1 bytes per activation: a call this large keeps its memory and runs the kernels without one)
-                need = 0
+            # for bf16 activations convert the activations once instead of once per block of output rows, and float32 /
+            # fp16 activations run on the bf16 kernels as a pair. The size query answers 0 where the launch would not use
+            # one (small calls, a loose max_rows); decode-sized bf16 / int8 calls never do and skip the query.
+            need = 0
+            if max_rows > 8 or xdt in (_lib.BP_F16, _lib.BP_F32):
+                need = self.lib.bp_grouped_gemm_workspace_bytes(xdt, T, N, int(K), E, int(fmt), int(max_rows))
+                if need > _WORKSPACE_CAP:  # (about 2.1 bytes per activation: a call this large keeps its memory and runs the kernels without one)
+                    need = 0
+            head = (out.data_ptr(), x.data_ptr(), xdt, x_scale.data_ptr() if x_scale is not None else None, offsets.data_ptr(), host,
+                    C.cast(pk, C.c_void_p), C.cast(sc, C.c_void_p), _lib.dtype_code(sdt), len(packed_l),
+                    T, N, int(K), Kp, G, int(group), E, int(fmt), int(max_rows))
             if need:
-                ws = torch.empty(need, dtype=torch.uint8, device=out.device)
-                rc = self.lib.bp_ternary_grouped_gemm_ws(
-                    out.data_ptr(), x.data_ptr(), _lib.dtype_code(x.dtype),
-                    x_scale.data_ptr() if x_scale is not None else None, offsets.data_ptr(), host,
-                    C.cast(pk, C.c_void_p), C.cast(sc, C.c_void_p), _lib.dtype_code(sdt), len(packed_l),
-                    T, N, int(K), Kp, G, int(group), E, int(fmt), int(max_rows), ws.data_ptr(), need,
-                    _lib.stream_ptr(out.device))
+                ws = torch.empty(need, dtype=torch.uint8, device=dev)
+                rc = self.lib.bp_ternary_grouped_gemm_ws(*head, ws.data_ptr(), need, stream)
             else:
-                rc = self.lib.bp_ternary_grouped_gemm(
-                    out.data_ptr(), x.data_ptr(), _lib.dtype_code(x.dtype),
-                    x_scale.data_ptr() if x_scale is not None else None, offsets.data_ptr(), host,
-                    C.cast(pk, C.c_void_p), C.cast(sc, C.c_void_p), _lib.dtype_code(sdt), len(packed_l),
-                    T, N, int(K), Kp, G, int(group), E, int(fmt), int(max_rows),
-                    lut1.data_ptr() if lut1 is not None else None, _lib.stream_ptr(out.device))
-        _lib.check(rc)
+                rc = self.lib.bp_ternary_grouped_gemm(*head, lut1.data_ptr() if lut1 is not None else None, stream)
+        finally:
+            if switch:
+                torch.cuda.set_device(prev)
+        if rc:
+            _lib.check(rc)
 
     def last_kernel(self) -> str:
         return self.lib.bp_last_kernel().decode()
