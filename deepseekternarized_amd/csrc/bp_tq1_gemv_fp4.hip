@@ -1131,6 +1131,17 @@ int launch_f4(const GemmArgs& a, hipStream_t s, int first_row = 0) {
   if (tuning().f4w) wide = lds > (size_t)F4_LDS_MAX / 2 || tuning().f4w == 16;  // (development)
   constexpr int SR = SRV;
   if (!wide) {
+    if constexpr (SDT != BP_F32) {
+      // A call with few row tiles (one linear of a decode step) is mostly set-up, table and token tile, which every
+      // workgroup repeats: workgroups of 4 waves put the tiles on twice as many CUs (measured, N = 2048, K = 7168, one
+      // expert: 16.7 us per call against 17.3; workgroups of 2 waves 19.8, of 1 wave 27.3: fewer threads build longer).
+      const int64_t tiles = ((a.N + 15) / 16) * experts;
+      const bool four = tuning().f4w ? tuning().f4w == 4 : tiles <= 2 * (int64_t)cus;
+      if (four) {
+        if (sr_ok && lds + 4 * F4_SCALE_SLOT <= (size_t)F4_LDS_MAX) return launch_f4_k<SDT, 4, 0, 1, SR>(a, s, "fp4_tq1_t1_w4", (int)nchunks, lds);
+        return launch_f4_k<SDT, 4>(a, s, "fp4_tq1_t1_w4", (int)nchunks, lds);
+      }
+    }
     if (sr_ok && lds + 8 * F4_SCALE_SLOT <= (size_t)F4_LDS_MAX) return launch_f4_k<SDT, 8, 0, 1, SR>(a, s, "fp4_tq1_t1_w8", (int)nchunks, lds);
     return launch_f4_k<SDT, 8>(a, s, "fp4_tq1_t1_w8", (int)nchunks, lds);
   }
