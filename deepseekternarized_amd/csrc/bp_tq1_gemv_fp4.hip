@@ -264,9 +264,13 @@ __device__ __forceinline__ void f4_block_offsets(int r16, int kb, unsigned (&aof
 // per lane (quarters 0..2 of a row's four lanes cover 48 bytes), a round ahead and unconditionally - so the compiler's
 // count of loads in flight stays exact - parks them in a private 1.25 KiB slot of LDS at the start of the round, and a
 // chunk's two scales per lane are two 2-byte LDS reads.
-template <int SDT, int WAVES, int ABL = 0, int NTOK = 1, int SR = 0>
+// KS (one token, a call with few row tiles): the waves of a workgroup share one row tile and split its chunks - wave w
+// takes chunks w cpw .. w cpw + cpw - 1 - and their partial sums are added through LDS in wave order. A call with 128
+// row tiles then runs on 128 CUs for a sixth of the chunks each, where whole rows per wave keep 16 CUs busy.
+template <int SDT, int WAVES, int ABL = 0, int NTOK = 1, int SR = 0, int KS = 0>
 __global__ __launch_bounds__(WAVES * 64, 4) void k_tq1_gemv_fp4(GemmArgs a, int total_chunks, int first_chunk, int nchunks, int bpw /* row blocks per workgroup */, int first_row) {
   static_assert(!SR || (SDT != BP_F32 && F4_GR == 1), "scales by the round: one tile per wave, 2-byte scales (a round of 2 or 4 chunks is 20 or 40 bytes of a row's scales)");
+  static_assert(!KS || (NTOK == 1 && F4_GR == 1 && ABL == 0), "chunks split over the waves: one token, one tile per workgroup");
   constexpr int THREADS = WAVES * 64, GR = F4_GR, RD = NTOK <= 2 ? F4_RD : 2, BD = F4_BD, AD = F4_AD, PAIRS = NTOK <= 2 ? F4_PAIRS : 0;
   static_assert(!PAIRS || RD % 2 == 0, "pairs of chunks need an even ring");
   static_assert(NTOK == 1 || (GR == 1 && AD == 0 && NTOK % 2 == 0), "several tokens: one tile per wave, one operand A buffer, token pairs");
@@ -297,14 +301,18 @@ __global__ __launch_bounds__(WAVES * 64, 4) void k_tq1_gemv_fp4(GemmArgs a, int 
   // A launch covers the chunks first_chunk .. first_chunk + nchunks - 1 of every row (all of them unless the tokens'
   // tiles of all chunks do not fit in LDS: then the host launches once per segment of K, and the output takes the
   // segments' partial sums one launch after the other). Chunk c below is chunk cb + c of the rows.
-  const int cb = NTOK == 1 ? 0 : first_chunk;
+  // (KS: this wave's chunks; a wave past the row's last chunk has none and only meets the others at the barriers)
+  const int cpw = KS ? (nchunks + WAVES - 1) / WAVES : nchunks;
+  const int cb = KS ? (wave * cpw < nchunks ? wave * cpw : nchunks) : NTOK == 1 ? 0 : first_chunk;
+  const int nch = KS ? (nchunks - cb < cpw ? nchunks - cb : cpw) : nchunks;  // chunks this wave multiplies
   // The last bytes of a chunk are completed from the first dword of the chunk after it (rows start at any byte). At
   // the end of a row that dword meets activations that are 0; at the end of a segment it is needed, so the chunk
   // after a segment that is not the last one is loaded as well.
-  const int last_load = NTOK > 1 && cb + nchunks < total_chunks ? nchunks : nchunks - 1;
+  const int last_load = (NTOK > 1 || KS) && cb + nch < total_chunks ? nch : nch - 1;
 
-  f4_build_tiles<NTOK, WAVES>(a, tok, ntok, nchunks, cb, wave, lane);
+  f4_build_tiles<NTOK, WAVES>(a, tok, ntok, nchunks, KS ? 0 : cb, wave, lane);  // (KS: the tiles of all chunks, tile index = chunk)
   __syncthreads();
+  const int tb = KS ? cb : 0;  // tile index of the wave's chunk 0
 
   const unsigned lane_tok = PC == 2 ? (unsigned)(((r16 >> 1) & 1) * F4_CHUNK_BYTES) : 0u;  // the lane's token of a pair: its tile
   unsigned aoff[4];  // 16-byte block (index within the chunk's part of the tile) of instruction j, half hf: byte 2 (j % 2) + hf of aoff[j / 2]
@@ -317,9 +325,13 @@ __global__ __launch_bounds__(WAVES * 64, 4) void k_tq1_gemv_fp4(GemmArgs a, int 
   // The tables serve `bpw` blocks of WAVES x GR x 16 rows, one after the other (the build is paid once per workgroup),
   // term by term: a term's blocks form one stream of chunks, and when the chunks of a row fill the ring a whole
   // number of times the refills run on into the next block, so the loads do not drain between blocks.
-  const bool chain = nchunks % RD == 0 && last_load == nchunks - 1;
-  auto block_row0 = [&](int pass) -> int64_t {  // first row of this wave's tile(s) in block `pass`; 0 (valid, not stored) past N
-    const int64_t r = (((int64_t)blockIdx.x * bpw + pass) * WAVES + wave) * (16 * GR);
+  const bool chain = !KS && nchunks % RD == 0 && last_load == nchunks - 1;
+  auto block_row = [&](int pass) -> int64_t {  // first row of this wave's tile(s) in block `pass`
+    if (KS) return ((int64_t)blockIdx.x * bpw + pass) * (16 * GR);
+    return (((int64_t)blockIdx.x * bpw + pass) * WAVES + wave) * (16 * GR);
+  };
+  auto block_row0 = [&](int pass) -> int64_t {  // ... or 0 (valid, not stored) past N
+    const int64_t r = block_row(pass);
     return r < a.N ? r : 0;
   };
   // (the whole loop nest once per number of token pairs the expert has in this launch, chosen outside it: a branch
@@ -349,7 +361,7 @@ __global__ __launch_bounds__(WAVES * 64, 4) void k_tq1_gemv_fp4(GemmArgs a, int 
 
   for (int pass = 0; pass < bpw; ++pass) {
     const int64_t n0 = block_row0(pass), n0_next = pass + 1 < bpw ? block_row0(pass + 1) : n0;
-    const bool wave_live = (((int64_t)blockIdx.x * bpw + pass) * WAVES + wave) * (16 * GR) < a.N;
+    const bool wave_live = block_row(pass) < a.N;
     float total[NTOK > 1 ? NTOK : GR];  // per token (this lane's two groups of every chunk), or (one token) per row tile
     // The outputs this block is added to are requested now and used when the block ends: read where they are added, the
     // load would be the youngest one in flight and the wait for it would drain the ring once per block. (Device scope:
@@ -362,14 +374,14 @@ __global__ __launch_bounds__(WAVES * 64, 4) void k_tq1_gemv_fp4(GemmArgs a, int 
       total[s] = 0.f;
       const int tile = NTOK > 1 ? 0 : s, tt = NTOK > 1 ? s : 0;
       before[s] = 0.f;
-      if (EARLY && kb == 0 && wave_live && n0 + 16 * tile < a.N && tt < ntok)
+      if (EARLY && kb == 0 && wave_live && n0 + 16 * tile < a.N && tt < ntok && (!KS || wave == 0))
         before[s] = __hip_atomic_load(a.out + (tok + tt) * a.N + n0 + 16 * tile + r16, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
     }
     // chunk c of this block, or (c >= nchunks, chained) chunk c - nchunks of the next one: row offset (scalar) and chunk
     auto target = [&](int c, int64_t& row0, int& cc) {
-      const bool over = chain && c >= nchunks && pass + 1 < bpw;
+      const bool over = chain && c >= nch && pass + 1 < bpw;
       row0 = over ? n0_next : n0;
-      cc = over ? c - nchunks : (c < last_load ? c : last_load);
+      cc = over ? c - nch : (c < last_load ? c : last_load);
     };
 
     // RD chunks in registers per tile; a chunk's registers are refilled (RD chunks on) as soon as its last byte has
@@ -414,7 +426,7 @@ __global__ __launch_bounds__(WAVES * 64, 4) void k_tq1_gemv_fp4(GemmArgs a, int 
     // byte offset, within the parked window of its round, of the scale of group g of chunk c
     auto parked_at = [&](int c, int g) {
       // (one token: rounds of 4 chunks from chunk 0, so a round starts 20 groups = a whole number of dwords into the row)
-      if (NTOK == 1) return SB * (unsigned)((5 * (c & (RD - 1)) + g) >> gs);
+      if (NTOK == 1 && !KS) return SB * (unsigned)((5 * (c & (RD - 1)) + g) >> gs);
       const unsigned first = (SB * (unsigned)((5 * (cb + (c & ~(RD - 1)))) >> gs)) & ~3u;
       return SB * (unsigned)((5 * (cb + c) + g) >> gs) - first;
     };
@@ -426,7 +438,7 @@ __global__ __launch_bounds__(WAVES * 64, 4) void k_tq1_gemv_fp4(GemmArgs a, int 
       f32x4 C[NC];
 #pragma unroll
       for (int s = 0; s < NC; ++s) C[s] = f32x4{0.f, 0.f, 0.f, 0.f};
-      const unsigned cbase = (unsigned)tile_at(0, c);
+      const unsigned cbase = (unsigned)tile_at(0, tb + c);
       // packed bytes of (instruction j, tile s) = dword j % 4 of the lane's window j / 4, shifted to the row's alignment;
       // the dword after a window is the first one of the next quarter's window (for the last quarter: of the first
       // quarter's next window, which for the second window is the next chunk's)
@@ -620,7 +632,7 @@ __global__ __launch_bounds__(WAVES * 64, 4) void k_tq1_gemv_fp4(GemmArgs a, int 
     }
     // RD chunks per iteration with no way around any of them: the compiler counts the loads in flight along every
     // path into the head of the loop, and a path on which fewer are in flight would make every iteration wait
-    const int full_end = ABL == 1 ? 0 : nchunks - nchunks % RD;
+    const int full_end = ABL == 1 ? 0 : nch - nch % RD;
     for (int c0 = 0; c0 < full_end; c0 += RD) {
       // (SR) the next round's scales are requested at the head of a round and parked in LDS at its end, after the
       // round's last scale has been read: the round's 8 refills of the ring lie between, in straight-line code
@@ -631,9 +643,9 @@ __global__ __launch_bounds__(WAVES * 64, 4) void k_tq1_gemv_fp4(GemmArgs a, int 
       if (RD > 3) step(c0 + 3, IC<3 % RD>{});
       if (SR) park_round();
     }
-    if (ABL != 1 && nchunks - full_end > 0) step(full_end, IC<0>{});  // uniform
-    if (ABL != 1 && nchunks - full_end > 1) step(full_end + 1, IC<1 % RD>{});
-    if (ABL != 1 && nchunks - full_end > 2) step(full_end + 2, IC<2 % RD>{});
+    if (ABL != 1 && nch - full_end > 0) step(full_end, IC<0>{});  // uniform
+    if (ABL != 1 && nch - full_end > 1) step(full_end + 1, IC<1 % RD>{});
+    if (ABL != 1 && nch - full_end > 2) step(full_end + 2, IC<2 % RD>{});
   // ---- the four quarter lanes of a row hold its partial sums (of this term: the output is added to)
 #pragma unroll
   for (int s = 0; s < (NTOK > 1 ? NTOK : GR); ++s) {
@@ -641,6 +653,18 @@ __global__ __launch_bounds__(WAVES * 64, 4) void k_tq1_gemv_fp4(GemmArgs a, int 
     t += __shfl_xor(t, 16);
     t += __shfl_xor(t, 32);
     const int tile = NTOK > 1 ? 0 : s, tt = NTOK > 1 ? s : 0;
+    if constexpr (KS != 0) {  // the waves' partial sums of the tile's 16 rows, added in wave order by wave 0
+      const unsigned red = (unsigned)(AT + nchunks * NTOK * F4_CHUNK_BYTES + (SR ? WAVES * F4_SCALE_SLOT : 0));
+      if (kb == 0) *(lds_u32*)(red + (unsigned)((wave * 16 + r16) * 4)) = __float_as_uint(t);
+      __syncthreads();
+      if (wave == 0) {
+        t = 0.f;
+#pragma unroll
+        for (int w = 0; w < WAVES; ++w) t += __uint_as_float(*(const lds_u32*)(red + (unsigned)((w * 16 + r16) * 4)));
+      }
+      __syncthreads();  // (the next term writes the same slots)
+      if (wave != 0) continue;
+    }
     if (kb == 0 && wave_live && n0 + 16 * tile < a.N && tt < ntok) {
       float* o = a.out + (tok + tt) * a.N + n0 + 16 * tile + r16;
       const float was = EARLY ? before[s] : __hip_atomic_load(o, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
@@ -997,24 +1021,25 @@ int f4_cus() {  // compute units of the current device (256 if the query fails);
   return known[dev];
 }
 
-template <int SDT, int WAVES, int ABL = 0, int NTOK = 1, int SR = 0>
+template <int SDT, int WAVES, int ABL = 0, int NTOK = 1, int SR = 0, int KS = 0>
 int launch_f4_k(const GemmArgs& a, hipStream_t s, const char* name, int nchunks, size_t lds, int seg_chunks = 0 /* chunks per launch (0: all) */, int first_row = 0) {
-  if (const int rc = raise_lds_limit<k_tq1_gemv_fp4<SDT, WAVES, ABL, NTOK, SR>>(F4_LDS_MAX)) return rc;
+  if (const int rc = raise_lds_limit<k_tq1_gemv_fp4<SDT, WAVES, ABL, NTOK, SR, KS>>(F4_LDS_MAX)) return rc;
   if (SR) lds += (size_t)WAVES * F4_SCALE_SLOT;
+  if (KS) lds += (size_t)WAVES * 64;  // the waves' partial sums
   const int cus = f4_cus();
   // Every workgroup builds the tables of its expert's token, so a workgroup takes as many row blocks as still leaves
   // every CU its full set of resident workgroups (16 waves): all workgroups resident at once, one build each.
-  const int64_t rows_per_block = (int64_t)WAVES * 16 * F4_GR;
+  const int64_t rows_per_block = (int64_t)(KS ? 1 : WAVES) * 16 * F4_GR;
   const int64_t blocks = (a.N + rows_per_block - 1) / rows_per_block;  // per expert
   const int64_t resident = (int64_t)cus * (16 / WAVES);
   const int64_t experts = a.E < a.T ? a.E : a.T;  // (an expert without a token returns at once)
   int64_t bpw = blocks * experts / resident;
-  bpw = bpw < 1 ? 1 : bpw > blocks ? blocks : bpw;
+  bpw = bpw < 1 || KS ? 1 : bpw > blocks ? blocks : bpw;
   const dim3 grid((unsigned)((blocks + bpw - 1) / bpw), (unsigned)a.E, 1u);
   note_kernel(name);
   const int per = seg_chunks > 0 ? seg_chunks : nchunks;
   for (int cb = 0; cb < nchunks; cb += per) {
-    hipLaunchKernelGGL((k_tq1_gemv_fp4<SDT, WAVES, ABL, NTOK, SR>), grid, dim3(WAVES * 64), lds, s, a, nchunks, cb, nchunks - cb < per ? nchunks - cb : per, (int)bpw, first_row);
+    hipLaunchKernelGGL((k_tq1_gemv_fp4<SDT, WAVES, ABL, NTOK, SR, KS>), grid, dim3(WAVES * 64), lds, s, a, nchunks, cb, nchunks - cb < per ? nchunks - cb : per, (int)bpw, first_row);
     const int rc = check_launch(name);
     if (rc != BP_OK) return rc;
   }
@@ -1136,6 +1161,12 @@ int launch_f4(const GemmArgs& a, hipStream_t s, int first_row = 0) {
       // workgroup repeats: workgroups of 4 waves put the tiles on twice as many CUs (measured, N = 2048, K = 7168, one
       // expert: 16.7 us per call against 17.3; workgroups of 2 waves 19.8, of 1 wave 27.3: fewer threads build longer).
       const int64_t tiles = ((a.N + 15) / 16) * experts;
+      // ... and with no more row tiles than CUs, a tile per workgroup with its chunks split over the 8 waves
+      const bool split = tuning().f4w ? tuning().f4w == 1 : tiles <= (int64_t)cus && nchunks >= 2;
+      if (split && lds + 8 * F4_SCALE_SLOT + 512 <= (size_t)F4_LDS_MAX) {
+        if (sr_ok) return launch_f4_k<SDT, 8, 0, 1, SR, 1>(a, s, "fp4_tq1_t1_ks", (int)nchunks, lds);
+        return launch_f4_k<SDT, 8, 0, 1, 0, 1>(a, s, "fp4_tq1_t1_ks", (int)nchunks, lds);
+      }
       const bool four = tuning().f4w ? tuning().f4w == 4 : tiles <= 2 * (int64_t)cus;
       if (four) {
         if (sr_ok && lds + 4 * F4_SCALE_SLOT <= (size_t)F4_LDS_MAX) return launch_f4_k<SDT, 4, 0, 1, SR>(a, s, "fp4_tq1_t1_w4", (int)nchunks, lds);

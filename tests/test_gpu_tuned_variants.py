@@ -126,6 +126,30 @@ def test_tq1_gemv_many_rows_two_terms_bf16_scales(bp, gemv_kernel):
     _check(got, want)
 
 
+@pytest.mark.parametrize("act", ["bf16", "int8", "f16"])
+@pytest.mark.parametrize("K,N,counts,terms,scale_dtype,group,misalign", [
+    (1024, 48, [1, 0, 1], 1, np.float16, 128, False),    # 2 chunks: six of the eight waves have none
+    (5376, 2048, [1], 2, "bf16", 128, False),            # 9 chunks: 2, 2, 2, 2, 1, 0, 0, 0 per wave; two terms = two rounds of the sum through LDS
+    (7168, 2048, [0, 1], 2, np.float16, 256, False),     # 12 chunks, one scale per 256
+    (2304, 528, [1, 1, 1], 1, np.float16, 128, True),    # scales from global memory (misaligned rows of scales); N not a multiple of 128
+    (4608, 4096, [1], 1, "f32", 128, False),             # float32 scales: not this variant
+])
+def test_tq1_single_token_call_with_few_row_tiles_splits_the_chunks_over_the_waves(bp, act, K, N, counts, terms, scale_dtype, group, misalign):
+    """One token and no more row tiles than CUs (a dense linear of a decode step): a row tile per workgroup, its chunks
+    split over the 8 waves, partial sums added in wave order (kernel name fp4_tq1_t1_ks)."""
+    got, want, kern = _run(bp, "tq1", len(counts), N, K, counts, act, terms=terms, seed=K + N, scale_dtype=scale_dtype, group=group,
+                           misalign_scales=misalign)
+    if scale_dtype != "f32":
+        assert kern == "fp4_tq1_t1_ks", kern
+    else:
+        assert kern.startswith("fp4_tq1_t1_w"), kern
+    _check(got, want)
+    if act != "f16":  # the same call twice gives the same bits (fixed order of the waves' sums)
+        again, _, _ = _run(bp, "tq1", len(counts), N, K, counts, act, terms=terms, seed=K + N, scale_dtype=scale_dtype, group=group,
+                           misalign_scales=misalign)
+        assert np.array_equal(got, again)
+
+
 @pytest.mark.parametrize("K,counts,act,N", [(1024, [1, 0, 1], "bf16", 48),      # Kp = 205: rows at every byte alignment; 2 chunks, 5 groups of waves
                                            (1280, [1, 1], "int8", 2048 + 16),   # Kp = 256; N not a multiple of a workgroup's tiles
                                            (4352, [0, 1, 1], "f16", 80),        # 7 chunks: one group, 9 loaders
