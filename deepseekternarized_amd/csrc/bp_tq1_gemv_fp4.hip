@@ -129,19 +129,32 @@ __device__ __forceinline__ void f4_build_tiles(const GemmArgs& a, int64_t tok, i
   // complete. Lane = byte pair: its 10 activations -> the largest magnitude of each of its (one or two) groups by an LDS
   // maximum over the float bits -> the groups' prescales 2^sh (sh brings the group's largest magnitude into [128, 256))
   // and their inverses -> 3 pieces x (first-group block, second-group block).
+  const int blk = lane;
+  const int tt0 = 5 * f4_pair_byte(blk >> 3, (blk >> 1) & 3, blk & 1), glo = tt0 >> 7, ghi = (tt0 + 9) >> 7;
+  // (a wave with several items requests the next item's activations before it works on the current one's)
+  u32x4 qn = {0u, 0u, 0u, 0u};
+  unsigned q4n = 0u;
+  auto request_x = [&](int item) {  // the lane's 20 bytes of a 16-bit item, if they lie inside the row
+    const int tt = item / nchunks, c = item - tt * nchunks;
+    const int64_t k0 = 640 * (int64_t)(cb + c) + tt0;
+    if (x16 && item < ntok * nchunks && k0 + 10 <= a.K) {  // 20 bytes at an even address
+      const uint16_t* src = (const uint16_t*)a.x + (tok + tt) * a.K + k0;
+      qn = ((const F4Packed16*)src)->v;
+      q4n = ((const F4Packed4*)(src + 8))->v;
+    }
+  };
+  request_x(wave);
   for (int item = wave; item < ntok * nchunks; item += builders) {  // (the waves 0 .. builders - 1 call this)
     const int tt = item / nchunks, c = item - tt * nchunks;
     const int64_t xrow = (tok + tt) * a.K;
-    const int blk = lane;
-    const int tt0 = 5 * f4_pair_byte(blk >> 3, (blk >> 1) & 3, blk & 1), glo = tt0 >> 7, ghi = (tt0 + 9) >> 7;
     const unsigned dst = (unsigned)tile_at(tt, c);
     if (lane < 8) *(lds_u32*)(dst + F4_PRE_OFF + 4 * lane) = 0u;
     const int64_t k0 = 640 * (int64_t)(cb + c) + tt0;
     float y[10];
-    if (x16 && k0 + 10 <= a.K) {  // 20 bytes at an even address
-      const uint16_t* src = (const uint16_t*)a.x + xrow + k0;
-      const u32x4 q = ((const F4Packed16*)src)->v;
-      const unsigned q4 = ((const F4Packed4*)(src + 8))->v;
+    const u32x4 q = qn;
+    const unsigned q4 = q4n;
+    request_x(item + builders);
+    if (x16 && k0 + 10 <= a.K) {
 #pragma unroll
       for (int i = 0; i < 4; ++i) { y[2 * i] = widen16(q[i] & 0xffffu); y[2 * i + 1] = widen16(q[i] >> 16); }
       y[8] = widen16(q4 & 0xffffu);
@@ -268,7 +281,7 @@ __device__ __forceinline__ void f4_block_offsets(int r16, int kb, unsigned (&aof
 // takes chunks w cpw .. w cpw + cpw - 1 - and their partial sums are added through LDS in wave order. A call with 128
 // row tiles then runs on 128 CUs for a sixth of the chunks each, where whole rows per wave keep 16 CUs busy.
 template <int SDT, int WAVES, int ABL = 0, int NTOK = 1, int SR = 0, int KS = 0>
-__global__ __launch_bounds__(WAVES * 64, 4) void k_tq1_gemv_fp4(GemmArgs a, int total_chunks, int first_chunk, int nchunks, int bpw /* row blocks per workgroup */, int first_row) {
+__global__ __launch_bounds__(WAVES * 64, KS ? 2 : 4) void k_tq1_gemv_fp4(GemmArgs a, int total_chunks, int first_chunk, int nchunks, int bpw /* row blocks per workgroup */, int first_row) {
   static_assert(!SR || (SDT != BP_F32 && F4_GR == 1), "scales by the round: one tile per wave, 2-byte scales (a round of 2 or 4 chunks is 20 or 40 bytes of a row's scales)");
   static_assert(!KS || (NTOK == 1 && F4_GR == 1 && ABL == 0), "chunks split over the waves: one token, one tile per workgroup");
   constexpr int THREADS = WAVES * 64, GR = F4_GR, RD = NTOK <= 2 ? F4_RD : 2, BD = F4_BD, AD = F4_AD, PAIRS = NTOK <= 2 ? F4_PAIRS : 0;
@@ -287,17 +300,22 @@ __global__ __launch_bounds__(WAVES * 64, 4) void k_tq1_gemv_fp4(GemmArgs a, int 
   // A launch takes the expert's token rows first_row .. first_row + NTOK - 1 (one token: its first row); an expert with
   // more rows than that gets further launches, one without any in this range is done at once (uniform).
   const int64_t tok = o0 + (NTOK == 1 ? 0 : first_row);
-  if (tok >= o1) return;
+  // (KS: the offsets are waited for behind the first loads of packed bytes, which do not depend on them)
+  if (!KS && tok >= o1) return;
   const int ntok = o1 - tok < NTOK ? (int)(o1 - tok) : NTOK;
   const int npairs = (ntok + 1) >> 1;  // token pairs the expert has in this launch: the others' matrix instructions are left out
   float xsc[NTOK];  // int8 activations: the tokens' scales
 #pragma unroll
-  for (int tt = 0; tt < NTOK; ++tt) xsc[tt] = a.x_dtype == BP_I8 && tt < ntok ? a.x_scale[tok + tt] : 1.f;
+  for (int tt = 0; tt < NTOK; ++tt) xsc[tt] = !KS && a.x_dtype == BP_I8 && tt < ntok ? a.x_scale[tok + tt] : 1.f;  // (KS: read behind the first loads, below)
   // the tiles of the NTOK tokens are interleaved chunk by chunk (a pair's tiles are a constant apart)
   auto tile_at = [](int tt, int c) { return AT + (c * NTOK + tt) * F4_CHUNK_BYTES; };
   const int gs = a.group == 256 ? 1 : 0;  // scale groups of 256: two 128-wide work groups share a scale
 
-  f4_build_table<THREADS>();
+  // KS: the table and the token's tiles are built behind the first loads of packed bytes (in all_terms below), whose
+  // latency then passes while the workgroup builds (such a call is mostly latencies in a row; the registers that the
+  // loads in flight hold during the build are there with one workgroup per CU).
+  constexpr bool LATE = KS != 0;
+  if (!LATE) f4_build_table<THREADS>();
   // A launch covers the chunks first_chunk .. first_chunk + nchunks - 1 of every row (all of them unless the tokens'
   // tiles of all chunks do not fit in LDS: then the host launches once per segment of K, and the output takes the
   // segments' partial sums one launch after the other). Chunk c below is chunk cb + c of the rows.
@@ -310,8 +328,10 @@ __global__ __launch_bounds__(WAVES * 64, 4) void k_tq1_gemv_fp4(GemmArgs a, int 
   // after a segment that is not the last one is loaded as well.
   const int last_load = (NTOK > 1 || KS) && cb + nch < total_chunks ? nch : nch - 1;
 
-  f4_build_tiles<NTOK, WAVES>(a, tok, ntok, nchunks, KS ? 0 : cb, wave, lane);  // (KS: the tiles of all chunks, tile index = chunk)
-  __syncthreads();
+  if (!LATE) {
+    f4_build_tiles<NTOK, WAVES>(a, tok, ntok, nchunks, KS ? 0 : cb, wave, lane);  // (KS: the tiles of all chunks, tile index = chunk)
+    __syncthreads();
+  }
   const int tb = KS ? cb : 0;  // tile index of the wave's chunk 0
 
   const unsigned lane_tok = PC == 2 ? (unsigned)(((r16 >> 1) & 1) * F4_CHUNK_BYTES) : 0u;  // the lane's token of a pair: its tile
@@ -624,6 +644,14 @@ __global__ __launch_bounds__(WAVES * 64, 4) void k_tq1_gemv_fp4(GemmArgs a, int 
       for (int u = 0; u < RD; ++u) {
         fetch_w(u, u, 0);
         fetch_w(u, u, 1);
+      }
+      __builtin_amdgcn_sched_barrier(0);
+      if (LATE && term == 0 && pass == 0) {  // (uniform)
+        if (tok >= o1) return;  // (uniform for the workgroup and before its first barrier: this ends the kernel - all_terms is its last statement)
+        if (a.x_dtype == BP_I8) xsc[0] = a.x_scale[tok];
+        f4_build_table<THREADS>();
+        f4_build_tiles<NTOK, WAVES>(a, tok, ntok, nchunks, KS ? 0 : cb, wave, lane);
+        __syncthreads();
       }
       __builtin_amdgcn_sched_barrier(0);
       if (SR) park_round();
