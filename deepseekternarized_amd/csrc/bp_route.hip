@@ -324,6 +324,70 @@ __global__ __launch_bounds__(256) void k_check_rows(int32_t* __restrict__ flag, 
   }
 }
 
+
+// ---- the router's softmax and top-k (boilerplate/engine/standard.py:160-165): one wave per token, lane L holds the
+// scores of experts L, L + 64, ... (up to ROUTE_PER_LANE of them). Softmax in float32 - the largest logit by a wave
+// maximum, exp(x - max), the sum lane by lane in expert order and then across the wave in a fixed butterfly - then k
+// rounds of a wave arg-max over (score, expert) with ties to the lower expert, the winner's entry taken out after each:
+// the slots come out in descending score like torch.topk's. `renorm`: the k scores are divided by their sum
+// (norm_topk_prob) before they are rounded to the output dtype.
+constexpr int ROUTE_PER_LANE = 16;  // experts per lane: up to 1024 experts
+template <int LDT, bool W_BF16>
+__global__ __launch_bounds__(256) void k_route_topk(void* __restrict__ weights, int64_t* __restrict__ experts, const void* __restrict__ logits,
+                                                     int64_t T, int E, int k, int renorm) {
+  const int lane = threadIdx.x & 63;
+  const int64_t t = (int64_t)blockIdx.x * 4 + (threadIdx.x >> 6);
+  if (t >= T) return;  // (uniform for the wave; no barrier below)
+  float sc[ROUTE_PER_LANE];
+  float mx = -INFINITY;
+#pragma unroll
+  for (int j = 0; j < ROUTE_PER_LANE; ++j) {
+    const int e = lane + 64 * j;
+    sc[j] = e < E ? load_act_f32(logits, LDT, t * E + e) : -INFINITY;
+    mx = fmaxf(mx, sc[j]);
+  }
+#pragma unroll
+  for (int off = 32; off > 0; off >>= 1) mx = fmaxf(mx, __shfl_xor(mx, off, 64));
+  float sum = 0.f;
+#pragma unroll
+  for (int j = 0; j < ROUTE_PER_LANE; ++j) {
+    sc[j] = lane + 64 * j < E ? expf(sc[j] - mx) : 0.f;
+    sum += sc[j];
+  }
+#pragma unroll
+  for (int off = 32; off > 0; off >>= 1) sum += __shfl_xor(sum, off, 64);
+#pragma unroll
+  for (int j = 0; j < ROUTE_PER_LANE; ++j) sc[j] = lane + 64 * j < E ? sc[j] / sum : -1.f;  // (scores are >= 0: -1 marks "no expert")
+  float mine = 0.f;  // lane s keeps the score of slot s
+  int mine_e = 0;
+  float ksum = 0.f;
+  for (int s = 0; s < k; ++s) {
+    float best = -1.f;
+    int best_e = 0x7fffffff;
+#pragma unroll
+    for (int j = 0; j < ROUTE_PER_LANE; ++j)  // (ascending expert: a later equal score does not replace an earlier one)
+      if (sc[j] > best) { best = sc[j]; best_e = lane + 64 * j; }
+#pragma unroll
+    for (int off = 32; off > 0; off >>= 1) {
+      const float ov = __shfl_xor(best, off, 64);
+      const int oe = __shfl_xor(best_e, off, 64);
+      if (ov > best || (ov == best && oe < best_e)) { best = ov; best_e = oe; }
+    }
+    if ((best_e & 63) == lane) {  // the winner leaves its lane's list
+#pragma unroll
+      for (int j = 0; j < ROUTE_PER_LANE; ++j)
+        if (j == (best_e >> 6)) sc[j] = -1.f;
+    }
+    if (lane == s) { mine = best; mine_e = best_e; }
+    ksum += best;
+  }
+  if (lane < k) {
+    const float v = renorm ? mine / ksum : mine;
+    if (W_BF16) ((uint16_t*)weights)[t * k + lane] = f32_to_bf16_bits(v);
+    else ((float*)weights)[t * k + lane] = v;
+    experts[t * k + lane] = mine_e;
+  }
+}
 }  // namespace
 }  // namespace bp
 
@@ -440,6 +504,26 @@ extern "C" int bp_moe_combine_v4(void* out, int out_dtype, const float* y, const
   if (out_dtype == BP_BF16) hipLaunchKernelGGL(k_combine_v4<true>, grid, dim3(256), 0, (hipStream_t)stream, out, y, inv, experts, k, H);
   else hipLaunchKernelGGL(k_combine_v4<false>, grid, dim3(256), 0, (hipStream_t)stream, out, y, inv, experts, k, H);
   return check_launch("moe_combine_v4");
+}
+
+extern "C" int bp_route_topk(void* weights, int weights_dtype, int64_t* experts, const void* logits, int logits_dtype, int64_t T, int64_t E,
+                             int64_t k, int renorm, void* stream) {
+  if (T < 0 || E <= 0 || E > 64 * ROUTE_PER_LANE || k <= 0 || k > 64 || k > E) return fail(BP_ERR_ARG, "invalid routing dimensions (up to 1024 experts, top-k up to 64)");
+  if (weights_dtype != BP_BF16 && weights_dtype != BP_F32) return fail(BP_ERR_ARG, "routing weights are bf16 or float32");
+  if (logits_dtype != BP_BF16 && logits_dtype != BP_F16 && logits_dtype != BP_F32) return fail(BP_ERR_ARG, "router logits are bf16, fp16 or float32");
+  if (T == 0) return BP_OK;
+  if (!weights || !experts || !logits) return fail(BP_ERR_ARG, "null pointer");
+  if ((T + 3) / 4 > 0x7fffffff) return fail(BP_ERR_ARG, "too many tokens");
+  const dim3 grid((unsigned)((T + 3) / 4)), block(256);
+  const hipStream_t s = (hipStream_t)stream;
+#define BP_ROUTE(LDT)                                                                                                                          \
+  if (logits_dtype == LDT) {                                                                                                                   \
+    if (weights_dtype == BP_BF16) hipLaunchKernelGGL((k_route_topk<LDT, true>), grid, block, 0, s, weights, experts, logits, T, (int)E, (int)k, renorm); \
+    else hipLaunchKernelGGL((k_route_topk<LDT, false>), grid, block, 0, s, weights, experts, logits, T, (int)E, (int)k, renorm);                \
+  }
+  BP_ROUTE(BP_BF16) BP_ROUTE(BP_F16) BP_ROUTE(BP_F32)
+#undef BP_ROUTE
+  return check_launch("route_topk");
 }
 
 extern "C" int bp_check_max_rows(int32_t* flag, const int64_t* offsets, int64_t E, int64_t T, int64_t max_rows, void* stream) {

@@ -70,9 +70,11 @@ class TernaryDecoder:
             L = _Layer()
             L.input_norm = torch.ones(H, device="cuda", dtype=dtype)
             L.post_norm = torch.ones(H, device="cuda", dtype=dtype)
-            for name in ("q", "k", "v", "o"):
-                p, sc = random_ternary(1, H, H, cfg.fmt, cfg.group, g, wscale)
-                setattr(L, name, TernaryLinear([PackedTerm(p[0], sc[0])], H, cfg.fmt, cfg.group, act=cfg.act))
+            # q | k | v stacked along N like the experts' gate | up: one activation quantisation and one launch for the three
+            qkv = [random_ternary(1, H, H, cfg.fmt, cfg.group, g, wscale) for _ in range(3)]
+            L.qkv = TernaryLinear([PackedTerm(torch.cat([p[0] for p, _ in qkv]), torch.cat([sc[0] for _, sc in qkv]))], H, cfg.fmt, cfg.group, act=cfg.act)
+            p, sc = random_ternary(1, H, H, cfg.fmt, cfg.group, g, wscale)
+            L.o = TernaryLinear([PackedTerm(p[0], sc[0])], H, cfg.fmt, cfg.group, act=cfg.act)
             L.router = (torch.randn(cfg.experts, H, device="cuda", generator=g) * s).to(dtype)
             gate = random_ternary(cfg.experts, cfg.inter, H, cfg.fmt, cfg.group, g, wscale)
             up = random_ternary(cfg.experts, cfg.inter, H, cfg.fmt, cfg.group, g, wscale)
@@ -113,7 +115,7 @@ class TernaryDecoder:
         for index, layer in enumerate(self.layers):
             residual = x
             z = self._norm(x, layer.input_norm)
-            q, k, v = self.linear(layer.q, z), self.linear(layer.k, z), self.linear(layer.v, z)
+            q, k, v = self.linear(layer.qkv, z).split(self.cfg.hidden, dim=-1)
             b, s, _ = q.shape
             q = q.view(b, s, self.cfg.heads, self.head_dim).transpose(1, 2)
             k = k.view(b, s, self.cfg.heads, self.head_dim).transpose(1, 2)
@@ -201,7 +203,7 @@ class GraphedDecode:
         for index, layer in enumerate(m.layers):
             residual = x
             z = m._norm(x, layer.input_norm)
-            q, k, v = m.linear(layer.q, z), m.linear(layer.k, z), m.linear(layer.v, z)
+            q, k, v = m.linear(layer.qkv, z).split(m.cfg.hidden, dim=-1)
             b = q.size(0)
             q = q.view(b, 1, cfg.heads, m.head_dim).transpose(1, 2)
             k = k.view(b, 1, cfg.heads, m.head_dim).transpose(1, 2)

@@ -40,6 +40,7 @@ SIGNATURES = {
     "bp_moe_combine_bf16": (_i, [_p, _p, _p, _p, _p, _l, _l, _l, _p]),
     "bp_swiglu_v4": (_i, [_p, _p, _p, _p, _p, _l, C.c_float, _l, _l, _l, _p]),
     "bp_moe_combine_v4": (_i, [_p, _i, _p, _p, _p, _l, _l, _l, _p]),
+    "bp_route_topk": (_i, [_p, _i, _p, _p, _i, _l, _l, _l, _i, _p]),
     "bp_moe_layer_v4": (_i, [_p, _i, _p, _p, _p, C.c_float, _p, _p, _p, _p, _i, _i, _l, _l, _l, _l, _l, _l, _i, _i, _p, C.c_size_t, _p, _p]),
     "bp_gguf_block_bytes": (_l, [_i]),
     "bp_gguf_from_ternary": (_i, [_p, _i, _p, _p, _l, _l, _i, _p]),

@@ -86,9 +86,21 @@ class TernaryMoE:
                                     max_rows=self._max_rows)
 
     def route(self, router_logits: torch.Tensor, tokens: int):
-        """``softmax`` / ``topk`` of the router logits in torch, as the reference does (engine/standard.py:158-161):
-        routing weights bf16 [T, k], expert ids int64 [T, k]."""
-        scores = torch.softmax(router_logits.reshape(tokens, -1).float(), dim=-1)
+        """``softmax`` / ``topk`` of the router logits (engine/standard.py:160-165): routing weights bf16 [T, k], expert
+        ids int64 [T, k], slots in descending score. One launch (``bp_route_topk``: float32 softmax, ties to the lower
+        expert id) for up to 1024 experts; beyond, the same torch ops the reference uses."""
+        logits = router_logits.reshape(tokens, -1)
+        E = logits.size(-1)
+        if E <= 1024 and self.top_k <= min(E, 64) and logits.dtype in (torch.bfloat16, torch.float16, torch.float32):
+            e = _need_ext(logits)
+            logits = logits.contiguous()
+            values = torch.empty(tokens, self.top_k, dtype=torch.bfloat16, device=logits.device)
+            indices = torch.empty(tokens, self.top_k, dtype=torch.int64, device=logits.device)
+            with torch.cuda.device(logits.device):
+                _lib.check(e.lib.bp_route_topk(values.data_ptr(), _lib.BP_BF16, indices.data_ptr(), logits.data_ptr(), _lib.dtype_code(logits.dtype),
+                                               tokens, E, self.top_k, int(self.renorm), _lib.stream_ptr(logits.device)))
+            return values, indices
+        scores = torch.softmax(logits.float(), dim=-1)
         values, indices = torch.topk(scores, self.top_k, dim=-1)
         if self.renorm:
             values = values / values.sum(-1, keepdim=True)

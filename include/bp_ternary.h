@@ -195,6 +195,16 @@ int bp_swiglu_bf16(void* h, const float* gate, const float* up, int64_t rows, in
 int bp_moe_combine_bf16(void* out, const float* y, const int64_t* inv, const void* w, const int64_t* experts,
                         int64_t T, int64_t k, int64_t H, void* stream);
 
+/* The router's softmax and top-k (boilerplate/engine/standard.py:160-165: `scores = softmax(logits.float())`,
+ * `values, indices = topk(scores, k)`, `values / values.sum()` under norm_topk_prob, `values.to(x.dtype)`), one launch:
+ * float32 softmax, the k largest scores per token in descending order with ties to the lower expert id.
+ *   weights  device bf16 or f32 [T, k] (weights_dtype BP_BF16 / BP_F32)
+ *   experts  device i64 [T, k]
+ *   logits   device bf16 / fp16 / f32 [T, E], E <= 1024, k <= 64
+ *   renorm   nonzero: the k scores are divided by their sum before rounding */
+int bp_route_topk(void* weights, int weights_dtype, int64_t* experts, const void* logits, int logits_dtype, int64_t T, int64_t E,
+                  int64_t k, int renorm, void* stream);
+
 /* SwiGLU of the V4 engine's expert MLP (boilerplate/engine/model.py:376-387, `swiglu`): the two linears return bf16,
  * then everything is float32: up clamped to [-limit, limit] and gate to at most limit (limit > 0; 0 = no clamp),
  * silu(gate) * up, times the routing weight when there is one, rounded to bf16 once (the input of w2).

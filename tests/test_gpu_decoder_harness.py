@@ -39,7 +39,7 @@ def test_decoder_matches_dense_torch_model(act):
     m = TernaryDecoder(cfg, seed=1)
     dense = []
     for L in m.layers:
-        d = {n: _dense(getattr(L, n).terms[0].packed, getattr(L, n).terms[0].scale, cfg.hidden, cfg.fmt, cfg.group) for n in "qkvo"}
+        d = {n: _dense(getattr(L, n).terms[0].packed, getattr(L, n).terms[0].scale, cfg.hidden, cfg.fmt, cfg.group) for n in ("qkv", "o")}  # (q | k | v are one stacked linear)
         (gp, gs), (up, us), (dp, ds) = L.experts
         d["gate"] = [_dense(gp[e], gs[e], cfg.hidden, cfg.fmt, cfg.group) for e in range(cfg.experts)]
         d["up"] = [_dense(up[e], us[e], cfg.hidden, cfg.fmt, cfg.group) for e in range(cfg.experts)]
@@ -66,7 +66,7 @@ def test_decoder_matches_dense_torch_model(act):
     assert got.shape == (2, 6, cfg.vocab) and torch.isfinite(got).all()
     # Second pass with every ternary op checked in place against its dense torch equivalent on the SAME input
     # (comparing whole forwards would also compare routing decisions, which flip on near-tied router scores).
-    index = {id(getattr(L, n)): (i, n) for i, L in enumerate(m.layers) for n in "qkvo"}
+    index = {id(getattr(L, n)): (i, n) for i, L in enumerate(m.layers) for n in ("qkv", "o")}
     hip_linear, hip_moe, worst = m.linear, m.moe, [0.0]
 
     def rel(a, b):

@@ -283,3 +283,61 @@ def test_graphs_of_one_layer_keep_their_workspaces():
         assert torch.equal(got, want), T
     assert torch.equal(moe(x300, l300), big)
     del filler
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16, torch.float16])
+@pytest.mark.parametrize("T,E,k,renorm", [(1, 64, 6, False), (37, 64, 8, True), (300, 384, 6, False), (5, 1024, 16, True), (9, 7, 7, False), (4, 130, 1, True)])
+def test_router_softmax_and_topk_in_one_launch(T, E, k, renorm, dtype):
+    """bp_route_topk against the oracle's float32 softmax and stable top-k (boilerplate/engine/standard.py:160-165) and
+    against torch's own ops on the device: the same experts in the same slots wherever the scores involved are further
+    apart than float32 rounding, weights equal to within one bf16 step."""
+    from deepseekternarized_amd.kernels import _lib
+
+    lib = _lib.load()
+    g = torch.Generator(device="cuda").manual_seed(T * 1000 + E)
+    logits = (torch.randn(T, E, device="cuda", generator=g) * 1.5).to(dtype)
+    for wdt, code in ((torch.bfloat16, _lib.BP_BF16), (torch.float32, _lib.BP_F32)):
+        w = torch.full((T, k), -1.0, dtype=wdt, device="cuda")
+        ids = torch.full((T, k), -1, dtype=torch.int64, device="cuda")
+        _lib.check(lib.bp_route_topk(w.data_ptr(), code, ids.data_ptr(), logits.data_ptr(), _lib.dtype_code(dtype), T, E, k, int(renorm),
+                                     _lib.stream_ptr(logits.device)))
+        torch.cuda.synchronize()
+        scores = orc.softmax_f32(logits.float().cpu().numpy())
+        want_v, want_i = orc.topk_desc(scores, k)
+        srt = -np.sort(-scores, axis=-1)
+        # tokens whose k + 1 largest scores are equal (equal logits: the lower expert wins, here as in the oracle) or
+        # further apart than the rounding of a float32 softmax; `strict`: no equal ones either (torch.topk's choice
+        # among equal scores is its own)
+        gaps = np.abs(np.diff(srt[:, : min(k + 1, E)], axis=-1))
+        clear = ((gaps == 0) | (gaps > 4e-6 * srt[:, :1])).all(-1)
+        strict = (gaps > 4e-6 * srt[:, :1]).all(-1)
+        assert clear.mean() > 0.5
+        got_i = ids.cpu().numpy()
+        assert np.array_equal(got_i[clear], want_i[clear])
+        assert ((got_i >= 0) & (got_i < E)).all() and all(len(set(r)) == k for r in got_i.tolist())
+        if renorm:
+            want_v = want_v / want_v.sum(-1, keepdims=True, dtype=np.float32)
+        got_v = w.float().cpu().numpy()
+        tol = 2.0 ** -8 if wdt == torch.bfloat16 else 2e-6
+        assert np.all(np.abs(got_v[clear] - want_v[clear]) <= tol * np.abs(want_v[clear]) + 1e-30)
+        # torch on the device, as the reference computes it
+        tv, ti = torch.topk(torch.softmax(logits.float(), -1), k, dim=-1)
+        assert np.array_equal(ti.cpu().numpy()[strict], got_i[strict])
+
+
+def test_router_kernel_ties_go_to_the_lower_expert_and_bad_arguments_are_rejected():
+    from deepseekternarized_amd.kernels import _lib
+
+    lib = _lib.load()
+    logits = torch.zeros(3, 200, device="cuda")
+    logits[1, 150] = logits[1, 20] = 2.0  # two equal maxima, then all the zeros
+    w = torch.empty(3, 4, device="cuda")
+    ids = torch.empty(3, 4, dtype=torch.int64, device="cuda")
+    _lib.check(lib.bp_route_topk(w.data_ptr(), _lib.BP_F32, ids.data_ptr(), logits.data_ptr(), _lib.BP_F32, 3, 200, 4, 0, _lib.stream_ptr(logits.device)))
+    torch.cuda.synchronize()
+    assert ids.cpu().tolist() == [[0, 1, 2, 3], [20, 150, 0, 1], [0, 1, 2, 3]]
+    assert torch.allclose(w[0].cpu(), torch.full((4,), 1 / 200))
+    assert lib.bp_route_topk(w.data_ptr(), _lib.BP_F32, ids.data_ptr(), logits.data_ptr(), _lib.BP_F32, 3, 2000, 4, 0, None) == 1
+    assert b"1024 experts" in lib.bp_last_error()
+    assert lib.bp_route_topk(w.data_ptr(), _lib.BP_I8, ids.data_ptr(), logits.data_ptr(), _lib.BP_F32, 3, 200, 4, 0, None) == 1
+    assert lib.bp_route_topk(w.data_ptr(), _lib.BP_F32, ids.data_ptr(), logits.data_ptr(), _lib.BP_F32, 3, 3, 4, 0, None) == 1
