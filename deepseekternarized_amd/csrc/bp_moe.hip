@@ -78,14 +78,18 @@ __global__ __launch_bounds__(256) void k_zero16(u32x4* __restrict__ p, int64_t n
 // A few routed rows (n <= ROUTE_SMALL_N): the layer's whole preparation in one launch instead of five - stable sort of
 // the expert ids (every workgroup ranks the ids for itself in LDS: element i goes to slot #(ids below id_i) + #(equal
 // ids before i); workgroup 0 writes order, offsets and the inverse permutation), the row gather xg[r] = x[order[r] / k],
-// and the zero-fill of the two float32 outputs that the small-batch kernels accumulate into.
+// and the zero-fill of the two float32 outputs that the small-batch kernels accumulate into - or, where the GEMMs run
+// over the list of token tiles, that list (position r of the order starts a tile when it is a multiple of 32 rows into
+// its expert; the tiles come out in expert order) instead of the zero-fill.
 constexpr int ROUTE_SMALL_N = 256, ROUTE_SMALL_THREADS = 256;
 __global__ __launch_bounds__(ROUTE_SMALL_THREADS) void k_route_small(int64_t* __restrict__ order, int64_t* __restrict__ offsets, int64_t* __restrict__ inv,
                                                                      const int64_t* __restrict__ ids, int n, int64_t E, int32_t* __restrict__ bad,
                                                                      u32x4* __restrict__ xg, const u32x4* __restrict__ x, int k, int64_t T, int64_t row16,
-                                                                     u32x4* __restrict__ z0, int64_t z0_16, u32x4* __restrict__ z1, int64_t z1_16) {
+                                                                     u32x4* __restrict__ z0, int64_t z0_16, u32x4* __restrict__ z1, int64_t z1_16,
+                                                                     int32_t* __restrict__ tiles, int32_t* __restrict__ tile_count, int64_t tile_cap) {
   __shared__ int32_t sid[ROUTE_SMALL_N];
   __shared__ int32_t ord[ROUTE_SMALL_N];
+  __shared__ int32_t tstart[ROUTE_SMALL_N];  // position r of the order starts a token tile
   const int i = threadIdx.x;
   int32_t mine = 0x7fffffff;  // an id outside [0, E) is left out of the order, as in bp_sort_by_expert
   if (i < n) {
@@ -95,14 +99,18 @@ __global__ __launch_bounds__(ROUTE_SMALL_THREADS) void k_route_small(int64_t* __
   }
   sid[i] = mine;
   ord[i] = -1;
+  tstart[i] = 0;
   __syncthreads();
+  int rank = 0;
   if (i < n && mine != 0x7fffffff) {
-    int rank = 0;
+    int lower = 0;  // rows of the experts before this one
     for (int j = 0; j < n; ++j) {
       const int32_t v = sid[j];
       rank += (v < mine || (v == mine && j < i)) ? 1 : 0;
+      lower += v < mine ? 1 : 0;
     }
     ord[rank] = i;
+    if (((rank - lower) & (TILE_ROWS - 1)) == 0) tstart[rank] = 1;
     if (blockIdx.x == 0) {
       order[rank] = i;
       inv[i] = rank;
@@ -116,6 +124,21 @@ __global__ __launch_bounds__(ROUTE_SMALL_THREADS) void k_route_small(int64_t* __
     }
   }
   __syncthreads();
+  if (tiles && blockIdx.x == 0) {
+    if (i < n && mine != 0x7fffffff && tstart[rank]) {
+      int at = 0;  // tiles that start before this one
+      for (int q = 0; q < rank; ++q) at += tstart[q];
+      if (at < tile_cap) {
+        tiles[2 * at] = mine;
+        tiles[2 * at + 1] = rank;
+      }
+    }
+    if (i == ROUTE_SMALL_THREADS - 1) {
+      int total = 0;
+      for (int q = 0; q < n; ++q) total += tstart[q];
+      tile_count[0] = total < tile_cap ? total : (int)tile_cap;
+    }
+  }
   const int64_t gtid = (int64_t)blockIdx.x * ROUTE_SMALL_THREADS + i, gsz = (int64_t)gridDim.x * ROUTE_SMALL_THREADS;
   for (int64_t w = gtid; w < (int64_t)n * row16; w += gsz) {  // 16 bytes of a gathered row
     const int64_t r = w / row16, c = w - r * row16;
@@ -240,13 +263,15 @@ static int moe_layer(bool v4, void* out, int out_dtype, float limit, const void*
   // 0.23 ms from 24 to 64 tokens on config 2's layer, where the small-batch kernels take 0.25 - 0.26 (and 0.18 - 0.21 below).
   const int64_t tiles_from = tuning().tiles >= 0 ? tuning().tiles : (fmt == BP_TQ1 && act == BP_BF16 ? 24 : 64);
   const bool tiles = T > tiles_from;
-  const bool small = n <= ROUTE_SMALL_N && !tiles && (((uintptr_t)x | (uintptr_t)p.xg) & 15) == 0;
+  const bool small = n <= ROUTE_SMALL_N && (((uintptr_t)x | (uintptr_t)p.xg) & 15) == 0;
+  const bool prezeroed = small && !tiles;  // (the GEMMs over the tile list write instead of accumulate)
   if (small) {
-    const int64_t z0 = (int64_t)(4 * (size_t)n * 2 * I / 16), z1 = (int64_t)(4 * (size_t)n * H / 16);
+    const int64_t z0 = prezeroed ? (int64_t)(4 * (size_t)n * 2 * I / 16) : 0, z1 = prezeroed ? (int64_t)(4 * (size_t)n * H / 16) : 0;
     int64_t g = (z0 + z1 + (int64_t)n * (H / 8) + ROUTE_SMALL_THREADS - 1) / ROUTE_SMALL_THREADS;
     g = g < 1 ? 1 : (g > 256 ? 256 : g);
     hipLaunchKernelGGL(k_route_small, dim3((unsigned)g), dim3(ROUTE_SMALL_THREADS), 0, s, p.order, p.offsets, p.inv, experts, (int)n, E, bad,
-                       (u32x4*)p.xg, (const u32x4*)x, (int)k, T, H / 8, (u32x4*)p.gu, z0, (u32x4*)p.y, z1);
+                       (u32x4*)p.xg, (const u32x4*)x, (int)k, T, H / 8, (u32x4*)p.gu, z0, (u32x4*)p.y, z1, tiles ? p.tiles : nullptr, p.tile_count,
+                       p.tile_cap);
     if ((rc = check_launch("route_small")) != BP_OK) return rc;
   } else {
     rc = bp_sort_by_expert(p.order, p.offsets, experts, n, E, bp_sort_workspace_ints(n, E) > 0 ? p.sort_ws : nullptr, bad, s);
@@ -285,11 +310,11 @@ static int moe_layer(bool v4, void* out, int out_dtype, float limit, const void*
       }
       a.tiles = nullptr;  // no tile kernel for this shape: the launch covers the bound (every expert up to T rows)
     }
-    if (!small)
+    if (!prezeroed)
       if (const int z = zero(o, 4 * (size_t)n * N, s)) return z;
     return run_gemm(a, s);
   };
-  if (tiles) {
+  if (tiles && !small) {
     hipLaunchKernelGGL(k_tile_list, dim3(1), dim3(1024), 0, s, p.tiles, p.tile_count, p.offsets, E, n, p.tile_cap);
     if ((rc = check_launch("tile_list")) != BP_OK) return rc;
   }
