@@ -87,9 +87,9 @@ __global__ __launch_bounds__(ROUTE_SMALL_THREADS) void k_route_small(int64_t* __
                                                                      u32x4* __restrict__ xg, const u32x4* __restrict__ x, int k, int64_t T, int64_t row16,
                                                                      u32x4* __restrict__ z0, int64_t z0_16, u32x4* __restrict__ z1, int64_t z1_16,
                                                                      int32_t* __restrict__ tiles, int32_t* __restrict__ tile_count, int64_t tile_cap) {
-  __shared__ int32_t sid[ROUTE_SMALL_N];
+  __shared__ __attribute__((aligned(16))) int32_t sid[ROUTE_SMALL_N];  // (entries from n on: 0x7fffffff, "no expert")
   __shared__ int32_t ord[ROUTE_SMALL_N];
-  __shared__ int32_t tstart[ROUTE_SMALL_N];  // position r of the order starts a token tile
+  __shared__ __attribute__((aligned(16))) int32_t tstart[ROUTE_SMALL_N];  // position r of the order starts a token tile
   const int i = threadIdx.x;
   int32_t mine = 0x7fffffff;  // an id outside [0, E) is left out of the order, as in bp_sort_by_expert
   if (i < n) {
@@ -104,11 +104,12 @@ __global__ __launch_bounds__(ROUTE_SMALL_THREADS) void k_route_small(int64_t* __
   int rank = 0;
   if (i < n && mine != 0x7fffffff) {
     int lower = 0;  // rows of the experts before this one
-    for (int j = 0; j < n; ++j) {
-      const int32_t v = sid[j];
-      rank += (v < mine || (v == mine && j < i)) ? 1 : 0;
-      lower += v < mine ? 1 : 0;
+    for (int j = 0; j < n; j += 4) {  // (four ids per LDS read; the padding compares as "after every expert")
+      const int4 v = *(const int4*)&sid[j];
+      lower += (v.x < mine ? 1 : 0) + (v.y < mine ? 1 : 0) + (v.z < mine ? 1 : 0) + (v.w < mine ? 1 : 0);
+      rank += (v.x == mine && j < i ? 1 : 0) + (v.y == mine && j + 1 < i ? 1 : 0) + (v.z == mine && j + 2 < i ? 1 : 0) + (v.w == mine && j + 3 < i ? 1 : 0);
     }
+    rank += lower;
     ord[rank] = i;
     if (((rank - lower) & (TILE_ROWS - 1)) == 0) tstart[rank] = 1;
     if (blockIdx.x == 0) {
@@ -119,7 +120,10 @@ __global__ __launch_bounds__(ROUTE_SMALL_THREADS) void k_route_small(int64_t* __
   if (blockIdx.x == 0) {
     for (int64_t e = i; e <= E; e += ROUTE_SMALL_THREADS) {
       int cnt = 0;
-      for (int j = 0; j < n; ++j) cnt += sid[j] < e ? 1 : 0;
+      for (int j = 0; j < n; j += 4) {
+        const int4 v = *(const int4*)&sid[j];
+        cnt += (v.x < e ? 1 : 0) + (v.y < e ? 1 : 0) + (v.z < e ? 1 : 0) + (v.w < e ? 1 : 0);
+      }
       offsets[e] = cnt;
     }
   }
@@ -127,7 +131,10 @@ __global__ __launch_bounds__(ROUTE_SMALL_THREADS) void k_route_small(int64_t* __
   if (tiles && blockIdx.x == 0) {
     if (i < n && mine != 0x7fffffff && tstart[rank]) {
       int at = 0;  // tiles that start before this one
-      for (int q = 0; q < rank; ++q) at += tstart[q];
+      for (int q = 0; q < rank; q += 4) {
+        const int4 v = *(const int4*)&tstart[q];
+        at += v.x + (q + 1 < rank ? v.y : 0) + (q + 2 < rank ? v.z : 0) + (q + 3 < rank ? v.w : 0);
+      }
       if (at < tile_cap) {
         tiles[2 * at] = mine;
         tiles[2 * at + 1] = rank;
@@ -135,7 +142,10 @@ __global__ __launch_bounds__(ROUTE_SMALL_THREADS) void k_route_small(int64_t* __
     }
     if (i == ROUTE_SMALL_THREADS - 1) {
       int total = 0;
-      for (int q = 0; q < n; ++q) total += tstart[q];
+      for (int q = 0; q < n; q += 4) {  // (entries from n on are 0)
+        const int4 v = *(const int4*)&tstart[q];
+        total += v.x + v.y + v.z + v.w;
+      }
       tile_count[0] = total < tile_cap ? total : (int)tile_cap;
     }
   }

@@ -331,17 +331,17 @@ __global__ __launch_bounds__(256) void k_check_rows(int32_t* __restrict__ flag, 
 // rounds of a wave arg-max over (score, expert) with ties to the lower expert, the winner's entry taken out after each:
 // the slots come out in descending score like torch.topk's. `renorm`: the k scores are divided by their sum
 // (norm_topk_prob) before they are rounded to the output dtype.
-constexpr int ROUTE_PER_LANE = 16;  // experts per lane: up to 1024 experts
-template <int LDT, bool W_BF16>
+constexpr int ROUTE_PER_LANE = 16;  // experts per lane at most: up to 1024 experts
+template <int LDT, bool W_BF16, int PER /* experts per lane: E <= 64 PER */>
 __global__ __launch_bounds__(256) void k_route_topk(void* __restrict__ weights, int64_t* __restrict__ experts, const void* __restrict__ logits,
                                                      int64_t T, int E, int k, int renorm) {
   const int lane = threadIdx.x & 63;
   const int64_t t = (int64_t)blockIdx.x * 4 + (threadIdx.x >> 6);
   if (t >= T) return;  // (uniform for the wave; no barrier below)
-  float sc[ROUTE_PER_LANE];
+  float sc[PER];
   float mx = -INFINITY;
 #pragma unroll
-  for (int j = 0; j < ROUTE_PER_LANE; ++j) {
+  for (int j = 0; j < PER; ++j) {
     const int e = lane + 64 * j;
     sc[j] = e < E ? load_act_f32(logits, LDT, t * E + e) : -INFINITY;
     mx = fmaxf(mx, sc[j]);
@@ -350,14 +350,14 @@ __global__ __launch_bounds__(256) void k_route_topk(void* __restrict__ weights, 
   for (int off = 32; off > 0; off >>= 1) mx = fmaxf(mx, __shfl_xor(mx, off, 64));
   float sum = 0.f;
 #pragma unroll
-  for (int j = 0; j < ROUTE_PER_LANE; ++j) {
+  for (int j = 0; j < PER; ++j) {
     sc[j] = lane + 64 * j < E ? expf(sc[j] - mx) : 0.f;
     sum += sc[j];
   }
 #pragma unroll
   for (int off = 32; off > 0; off >>= 1) sum += __shfl_xor(sum, off, 64);
 #pragma unroll
-  for (int j = 0; j < ROUTE_PER_LANE; ++j) sc[j] = lane + 64 * j < E ? sc[j] / sum : -1.f;  // (scores are >= 0: -1 marks "no expert")
+  for (int j = 0; j < PER; ++j) sc[j] = lane + 64 * j < E ? sc[j] / sum : -1.f;  // (scores are >= 0: -1 marks "no expert")
   float mine = 0.f;  // lane s keeps the score of slot s
   int mine_e = 0;
   float ksum = 0.f;
@@ -365,7 +365,7 @@ __global__ __launch_bounds__(256) void k_route_topk(void* __restrict__ weights, 
     float best = -1.f;
     int best_e = 0x7fffffff;
 #pragma unroll
-    for (int j = 0; j < ROUTE_PER_LANE; ++j)  // (ascending expert: a later equal score does not replace an earlier one)
+    for (int j = 0; j < PER; ++j)  // (ascending expert: a later equal score does not replace an earlier one)
       if (sc[j] > best) { best = sc[j]; best_e = lane + 64 * j; }
 #pragma unroll
     for (int off = 32; off > 0; off >>= 1) {
@@ -375,7 +375,7 @@ __global__ __launch_bounds__(256) void k_route_topk(void* __restrict__ weights, 
     }
     if ((best_e & 63) == lane) {  // the winner leaves its lane's list
 #pragma unroll
-      for (int j = 0; j < ROUTE_PER_LANE; ++j)
+      for (int j = 0; j < PER; ++j)
         if (j == (best_e >> 6)) sc[j] = -1.f;
     }
     if (lane == s) { mine = best; mine_e = best_e; }
@@ -516,13 +516,22 @@ extern "C" int bp_route_topk(void* weights, int weights_dtype, int64_t* experts,
   if ((T + 3) / 4 > 0x7fffffff) return fail(BP_ERR_ARG, "too many tokens");
   const dim3 grid((unsigned)((T + 3) / 4)), block(256);
   const hipStream_t s = (hipStream_t)stream;
-#define BP_ROUTE(LDT)                                                                                                                          \
-  if (logits_dtype == LDT) {                                                                                                                   \
-    if (weights_dtype == BP_BF16) hipLaunchKernelGGL((k_route_topk<LDT, true>), grid, block, 0, s, weights, experts, logits, T, (int)E, (int)k, renorm); \
-    else hipLaunchKernelGGL((k_route_topk<LDT, false>), grid, block, 0, s, weights, experts, logits, T, (int)E, (int)k, renorm);                \
+#define BP_ROUTE_P(LDT, PER)                                                                                                                        \
+  {                                                                                                                                                 \
+    if (weights_dtype == BP_BF16) hipLaunchKernelGGL((k_route_topk<LDT, true, PER>), grid, block, 0, s, weights, experts, logits, T, (int)E, (int)k, renorm); \
+    else hipLaunchKernelGGL((k_route_topk<LDT, false, PER>), grid, block, 0, s, weights, experts, logits, T, (int)E, (int)k, renorm);               \
+  }
+#define BP_ROUTE(LDT)                                 \
+  if (logits_dtype == LDT) {                          \
+    if (E <= 64) BP_ROUTE_P(LDT, 1)                   \
+    else if (E <= 128) BP_ROUTE_P(LDT, 2)             \
+    else if (E <= 256) BP_ROUTE_P(LDT, 4)             \
+    else if (E <= 512) BP_ROUTE_P(LDT, 8)             \
+    else BP_ROUTE_P(LDT, ROUTE_PER_LANE)              \
   }
   BP_ROUTE(BP_BF16) BP_ROUTE(BP_F16) BP_ROUTE(BP_F32)
 #undef BP_ROUTE
+#undef BP_ROUTE_P
   return check_launch("route_topk");
 }
 
