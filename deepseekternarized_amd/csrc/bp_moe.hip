@@ -16,6 +16,8 @@
 
 namespace bp {
 int kernel_policy();  // bp_api.hip
+int sort_with_inverse(int64_t* order, int64_t* offsets, int64_t* inv, const int64_t* ids, int64_t n, int64_t E, int32_t* workspace,
+                      int32_t* bad, hipStream_t stream);  // bp_route.hip
 namespace {
 
 constexpr int TILE_ROWS = 32;  // token tile of k_gemm_tq1 / k_gemm_tq2
@@ -60,15 +62,6 @@ __global__ __launch_bounds__(1024) void k_tile_list(int32_t* __restrict__ tiles,
     __syncthreads();
   }
   if (threadIdx.x == 0) count[0] = carry < cap ? carry : (int)cap;
-}
-
-// inv[order[i]] = i: where pair (token, slot) sits in expert order
-__global__ __launch_bounds__(256) void k_invert(int64_t* __restrict__ inv, const int64_t* __restrict__ order, int64_t n) {
-  const int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x;
-  if (i < n) {
-    const int64_t o = order[i];
-    if (o >= 0 && o < n) inv[o] = i;
-  }
 }
 
 __global__ __launch_bounds__(256) void k_zero16(u32x4* __restrict__ p, int64_t n16) {
@@ -284,10 +277,7 @@ static int moe_layer(bool v4, void* out, int out_dtype, float limit, const void*
                        p.tile_cap);
     if ((rc = check_launch("route_small")) != BP_OK) return rc;
   } else {
-    rc = bp_sort_by_expert(p.order, p.offsets, experts, n, E, bp_sort_workspace_ints(n, E) > 0 ? p.sort_ws : nullptr, bad, s);
-    if (rc != BP_OK) return rc;
-    hipLaunchKernelGGL(k_invert, dim3((unsigned)((n + 255) / 256)), dim3(256), 0, s, p.inv, p.order, n);
-    if ((rc = check_launch("invert")) != BP_OK) return rc;
+    if ((rc = sort_with_inverse(p.order, p.offsets, p.inv, experts, n, E, p.sort_ws, bad, s)) != BP_OK) return rc;
     if ((rc = bp_gather_rows(p.xg, x, p.order, k, n, T, 2 * H, s)) != BP_OK) return rc;
   }
 

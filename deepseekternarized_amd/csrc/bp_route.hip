@@ -26,10 +26,11 @@ constexpr int64_t SORT_LDS_INTS = 32768;  // 128 KiB of per-wave histograms in L
 // One workgroup. Wave w owns the contiguous segment [w*seg, (w+1)*seg) of ids.
 // Pass 1: per-wave histograms. Scan: offsets and, per wave, the first output slot of each expert.
 // Pass 2: every wave walks its segment in order, 64 ids at a time; lanes holding the same expert are
-// ranked by lane index (ballot + popcount), so equal ids keep their input order (stable).
+// ranked by lane index (ballot + popcount), so equal ids keep their input order (stable). `inv` (or NULL): the inverse
+// permutation, inv[i] = the slot of id i in the order (ids outside [0, E) have none and keep what inv held).
 __global__ __launch_bounds__(SORT_THREADS) void k_sort(int64_t* __restrict__ order, int64_t* __restrict__ offsets,
                                                         const int64_t* __restrict__ ids, int64_t n, int64_t E,
-                                                        int32_t* __restrict__ ws, int32_t* __restrict__ bad) {
+                                                        int32_t* __restrict__ ws, int32_t* __restrict__ bad, int64_t* __restrict__ inv) {
   extern __shared__ int32_t lds_hist[];
   int32_t* hist = ws ? ws : lds_hist;  // [SORT_WAVES][E]
   __shared__ int64_t carry;
@@ -47,22 +48,28 @@ __global__ __launch_bounds__(SORT_THREADS) void k_sort(int64_t* __restrict__ ord
   }
   __threadfence();
   __syncthreads();
-  // exclusive scan over experts of the column sums; chunks of SORT_THREADS experts at a time
-  __shared__ int64_t scan[SORT_THREADS];
+  // exclusive scan over experts of the column sums; chunks of SORT_THREADS experts at a time: a scan inside every wave
+  // (shuffles), then the waves' totals through LDS
+  __shared__ int64_t wave_total[SORT_WAVES];
   for (int64_t e0 = 0; e0 < E; e0 += SORT_THREADS) {
     const int64_t e = e0 + threadIdx.x;
     int64_t cnt = 0;
     if (e < E)
       for (int w = 0; w < SORT_WAVES; ++w) cnt += hist[w * E + e];
-    scan[threadIdx.x] = cnt;
-    __syncthreads();
-    for (int off = 1; off < SORT_THREADS; off <<= 1) {
-      const int64_t v = threadIdx.x >= off ? scan[threadIdx.x - off] : 0;
-      __syncthreads();
-      scan[threadIdx.x] += v;
-      __syncthreads();
+    int64_t incl = cnt;
+#pragma unroll
+    for (int d = 1; d < 64; d <<= 1) {
+      const int64_t up = __shfl_up(incl, d, 64);
+      if (lane >= d) incl += up;
     }
-    const int64_t base = carry + scan[threadIdx.x] - cnt;  // exclusive prefix for expert e
+    if (lane == 63) wave_total[wave] = incl;
+    __syncthreads();
+    int64_t chunk_total = 0;
+    for (int w = 0; w < SORT_WAVES; ++w) {
+      if (w < wave) incl += wave_total[w];
+      chunk_total += wave_total[w];
+    }
+    const int64_t base = carry + incl - cnt;  // exclusive prefix for expert e
     if (e < E) {
       offsets[e] = base;
       int64_t run = base;
@@ -72,8 +79,8 @@ __global__ __launch_bounds__(SORT_THREADS) void k_sort(int64_t* __restrict__ ord
         run += c;
       }
     }
-    __syncthreads();
-    if (threadIdx.x == SORT_THREADS - 1) carry += scan[SORT_THREADS - 1];
+    __syncthreads();  // (every thread has read carry and the waves' totals)
+    if (threadIdx.x == 0) carry += chunk_total;
     __syncthreads();
   }
   if (threadIdx.x == 0) offsets[E] = carry;
@@ -99,7 +106,9 @@ __global__ __launch_bounds__(SORT_THREADS) void k_sort(int64_t* __restrict__ ord
       int32_t first = 0;
       if (lane == leader) first = atomicAdd(&mine[id], (int32_t)__popcll(same));  // claims the run of slots
       first = __shfl(first, leader, 64);
-      order[first + __popcll(same & ((1ull << lane) - 1ull))] = i;
+      const int64_t slot = first + __popcll(same & ((1ull << lane) - 1ull));
+      order[slot] = i;
+      if (inv) inv[i] = slot;
     }
   }
 }
@@ -400,16 +409,24 @@ extern "C" int64_t bp_sort_workspace_ints(int64_t n, int64_t E) {
 }
 
 static int launch_sort(int64_t* order, int64_t* offsets, const int64_t* ids, int64_t n, int64_t E, int32_t* hist_mem,
-                       int32_t* bad, hipStream_t stream) {
-  if (n <= SORT_SMALL_N && E < ((int64_t)1 << 24)) {
+                       int32_t* bad, hipStream_t stream, int64_t* inv = nullptr) {
+  if (!inv && n <= SORT_SMALL_N && E < ((int64_t)1 << 24)) {
     hipLaunchKernelGGL(k_sort_small, dim3(1), dim3(SORT_SMALL_THREADS), 0, stream, order, offsets, ids, (int)n, E, bad);
     return check_launch("sort_by_expert");
   }
   const size_t lds = hist_mem ? 0 : (size_t)(SORT_WAVES * (E > 0 ? E : 1)) * sizeof(int32_t);
   if (const int rc = raise_lds_limit<k_sort>((int)(SORT_LDS_INTS * 4))) return rc;
-  hipLaunchKernelGGL(k_sort, dim3(1), dim3(SORT_THREADS), lds, stream, order, offsets, ids, n, E, hist_mem, bad);
+  hipLaunchKernelGGL(k_sort, dim3(1), dim3(SORT_THREADS), lds, stream, order, offsets, ids, n, E, hist_mem, bad, inv);
   return check_launch("sort_by_expert");
 }
+
+namespace bp {
+// bp_sort_by_expert that also writes the inverse permutation (the MoE layer's preparation; arguments checked by its caller)
+int sort_with_inverse(int64_t* order, int64_t* offsets, int64_t* inv, const int64_t* ids, int64_t n, int64_t E, int32_t* workspace,
+                      int32_t* bad, hipStream_t stream) {
+  return launch_sort(order, offsets, ids, n, E, bp_sort_workspace_ints(n, E) > 0 ? workspace : (int32_t*)nullptr, bad, stream, inv);
+}
+}  // namespace bp
 
 extern "C" int bp_sort_by_expert(int64_t* order, int64_t* offsets, const int64_t* ids, int64_t n, int64_t E,
                                  int32_t* workspace, int32_t* bad, void* stream) {
