@@ -46,7 +46,7 @@ __global__ __launch_bounds__(SORT_THREADS) void k_sort(int64_t* __restrict__ ord
     if (id >= 0 && id < E) atomicAdd(&mine[id], 1);
     else if (bad) *bad = 1;
   }
-  __threadfence();
+  if (ws) __threadfence();  // (histograms in device memory; in LDS the barrier orders them)
   __syncthreads();
   // exclusive scan over experts of the column sums; chunks of SORT_THREADS experts at a time: a scan inside every wave
   // (shuffles), then the waves' totals through LDS
@@ -84,7 +84,7 @@ __global__ __launch_bounds__(SORT_THREADS) void k_sort(int64_t* __restrict__ ord
     __syncthreads();
   }
   if (threadIdx.x == 0) offsets[E] = carry;
-  __threadfence();
+  if (ws) __threadfence();  // (histograms in device memory; in LDS the barrier orders them)
   __syncthreads();
   // Pass 2, 64 ids at a time: every lane finds the lanes that hold its expert (one ballot per bit of the expert index),
   // the lowest of them claims the run of output slots with one atomic, and a lane's slot is the run's first plus the
