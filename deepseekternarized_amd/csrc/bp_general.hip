@@ -172,6 +172,63 @@ __global__ __launch_bounds__(256) void k_quant(int8_t* __restrict__ q, float* __
   }
 }
 
+// The same for 16-bit activations in rows of whole 16-byte pieces (K % 8 == 0, K <= 8192, aligned pointers): a thread keeps
+// its up to four pieces of the row in registers between the two passes, so the row is read once, in 16-byte loads, and
+// written in 8-byte stores. Same arithmetic as k_quant, operation for operation.
+constexpr int QUANT_VPT = 4;
+typedef unsigned u32x2 __attribute__((ext_vector_type(2)));
+typedef unsigned u32x4 __attribute__((ext_vector_type(4)));
+template <int DT>
+__global__ __launch_bounds__(256) void k_quant16(int8_t* __restrict__ q, float* __restrict__ s, const uint16_t* __restrict__ x, int64_t K) {
+  __shared__ float part[4];
+  const int64_t m = blockIdx.x;
+  const int pieces = (int)(K / 8);
+  u32x4 raw[QUANT_VPT];
+  float amax = 0.f;
+  bool nan = false;
+#pragma unroll
+  for (int i = 0; i < QUANT_VPT; ++i) {
+    const int pc = threadIdx.x + 256 * i;
+    raw[i] = u32x4{0u, 0u, 0u, 0u};
+    if (pc < pieces) raw[i] = *(const u32x4*)(x + m * K + 8 * (int64_t)pc);
+#pragma unroll
+    for (int j = 0; j < 8; ++j) {
+      const uint16_t h = (uint16_t)(raw[i][j >> 1] >> (16 * (j & 1)));
+      const float v = DT == BP_BF16 ? bf16_bits_to_f32(h) : f16_bits_to_f32(h);
+      nan |= v != v;
+      amax = fmaxf(amax, fabsf(v));
+    }
+  }
+  if (nan) amax = __builtin_nanf("");
+  float w = amax;
+#pragma unroll
+  for (int off = 32; off > 0; off >>= 1) {
+    const float o = __shfl_xor(w, off, 64);
+    w = (w != w || o != o) ? __builtin_nanf("") : fmaxf(w, o);
+  }
+  if ((threadIdx.x & 63) == 0) part[threadIdx.x >> 6] = w;
+  __syncthreads();
+  float a = part[0];
+  for (int i = 1; i < 4; ++i) a = (a != a || part[i] != part[i]) ? __builtin_nanf("") : fmaxf(a, part[i]);
+  float sc = __fdiv_rn(a, 127.0f);
+  sc = sc != sc ? sc : fmaxf(sc, 1e-8f);  // clamp(min=1e-8) keeps NaN
+  if (threadIdx.x == 0) s[m] = sc;
+#pragma unroll
+  for (int i = 0; i < QUANT_VPT; ++i) {
+    const int pc = threadIdx.x + 256 * i;
+    unsigned out[2] = {0u, 0u};
+#pragma unroll
+    for (int j = 0; j < 8; ++j) {
+      const uint16_t h = (uint16_t)(raw[i][j >> 1] >> (16 * (j & 1)));
+      const float v = DT == BP_BF16 ? bf16_bits_to_f32(h) : f16_bits_to_f32(h);
+      float r = rintf(__fdiv_rn(v, sc));  // round half to even, like torch.round
+      r = fminf(fmaxf(r, -127.f), 127.f);
+      out[j >> 2] |= ((unsigned)(r != r ? 0 : (int)r) & 0xffu) << (8 * (j & 3));
+    }
+    if (pc < pieces) *(u32x2*)(q + m * K + 8 * (int64_t)pc) = u32x2{out[0], out[1]};
+  }
+}
+
 int grid_for(int64_t n) {
   int64_t g = (n + 255) / 256;
   return (int)(g < 1 ? 1 : (g > 65535 ? 65535 : g));
@@ -296,7 +353,10 @@ extern "C" int bp_quant_act_int8(int8_t* q, float* s, const void* x, int x_dtype
   if (M < 0 || K <= 0 || M > 0x7fffffff) return fail(BP_ERR_ARG, "invalid M or K");
   if (M == 0) return BP_OK;
   if (!q || !s || !x) return fail(BP_ERR_ARG, "null pointer");
-  hipLaunchKernelGGL(k_quant, dim3((unsigned)M), dim3(256), 0, (hipStream_t)stream, q, s, x, x_dtype, K);
+  const bool pieces = x_dtype != BP_F32 && K % 8 == 0 && K <= 8 * 256 * QUANT_VPT && ((uintptr_t)x & 15) == 0 && ((uintptr_t)q & 7) == 0;
+  if (pieces && x_dtype == BP_BF16) hipLaunchKernelGGL(k_quant16<BP_BF16>, dim3((unsigned)M), dim3(256), 0, (hipStream_t)stream, q, s, (const uint16_t*)x, K);
+  else if (pieces) hipLaunchKernelGGL(k_quant16<BP_F16>, dim3((unsigned)M), dim3(256), 0, (hipStream_t)stream, q, s, (const uint16_t*)x, K);
+  else hipLaunchKernelGGL(k_quant, dim3((unsigned)M), dim3(256), 0, (hipStream_t)stream, q, s, x, x_dtype, K);
   return check_launch("quant_act_int8");
 }
 

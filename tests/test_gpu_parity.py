@@ -78,10 +78,11 @@ def test_scale_expansion_bit_exact(bp, dtype):
     assert bool(got[want.isnan()].isnan().all())
 
 
+@pytest.mark.parametrize("K", [300, 64, 2048, 8192, 8200])  # rows of whole 16-byte pieces up to 8192 take the one-read kernel (16-bit inputs)
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16, torch.float16])
-def test_quant_act_int8_bit_exact(bp, dtype):
-    rng = np.random.default_rng(0)
-    x = torch.from_numpy((rng.standard_normal((37, 300)) * 3).astype(np.float32)).to(dtype)
+def test_quant_act_int8_bit_exact(bp, dtype, K):
+    rng = np.random.default_rng(K)
+    x = torch.from_numpy((rng.standard_normal((37, K)) * 3).astype(np.float32)).to(dtype)
     x[3] = 0  # scale clamps at 1e-8
     x[4, :5] = torch.tensor([254.0, -127.0, 1.0, 3.0, 5.0]).to(dtype)
     q, s = bp.quant_act_int8(x.cuda())
@@ -89,6 +90,15 @@ def test_quant_act_int8_bit_exact(bp, dtype):
     assert q.dtype == torch.int8 and s.dtype == torch.float32 and tuple(s.shape) == (37,)
     assert np.array_equal(s.cpu().numpy(), ws) and np.array_equal(q.cpu().numpy(), wq)
     assert ((q.float() * s[:, None] - x.cuda().float()).abs() <= s[:, None] / 2 + 1e-6).all()
+    # A NaN makes its row's scale NaN, an infinity makes it infinite (the int8 values of such a row are a cast of NaN in
+    # the reference, boilerplate/ternary/ops.py:22: unspecified); the other rows are not touched by it.
+    y = x.clone()
+    y[1, K // 2] = float("nan")
+    y[2, K - 1] = float("inf")
+    q2, s2 = bp.quant_act_int8(y.cuda())
+    keep = np.array([r not in (1, 2) for r in range(37)])
+    assert np.array_equal(q2.cpu().numpy()[keep], wq[keep]) and np.array_equal(s2.cpu().numpy()[keep], ws[keep])
+    assert np.isnan(s2[1].item()) and np.isinf(s2[2].item())
 
 
 def test_quant_act_int8_keeps_leading_shape(bp):
