@@ -64,6 +64,21 @@ __global__ __launch_bounds__(1024) void k_tile_list(int32_t* __restrict__ tiles,
   if (threadIdx.x == 0) count[0] = carry < cap ? carry : (int)cap;
 }
 
+// The row gather xg[r] = x[order[r] / k] (rows of 16-byte pieces) and, in the same launch, the zero-fill of the two float32
+// outputs that the GEMMs accumulate into (z0_16 = z1_16 = 0 where they write instead).
+__global__ __launch_bounds__(256) void k_gather_zero(u32x4* __restrict__ xg, const u32x4* __restrict__ x, const int64_t* __restrict__ order, int64_t n,
+                                                     int64_t k, int64_t T, int64_t row16, u32x4* __restrict__ z0, int64_t z0_16, u32x4* __restrict__ z1,
+                                                     int64_t z1_16) {
+  const int64_t gtid = (int64_t)blockIdx.x * 256 + threadIdx.x, gsz = (int64_t)gridDim.x * 256;
+  for (int64_t w = gtid; w < n * row16; w += gsz) {
+    const int64_t r = w / row16, c = w - r * row16;
+    const int64_t src = clamp_i64(order[r] / k, 0, T - 1);
+    xg[r * row16 + c] = x[src * row16 + c];
+  }
+  for (int64_t w = gtid; w < z0_16; w += gsz) z0[w] = u32x4{0u, 0u, 0u, 0u};
+  for (int64_t w = gtid; w < z1_16; w += gsz) z1[w] = u32x4{0u, 0u, 0u, 0u};
+}
+
 __global__ __launch_bounds__(256) void k_zero16(u32x4* __restrict__ p, int64_t n16) {
   for (int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x; i < n16; i += (int64_t)gridDim.x * 256) p[i] = u32x4{0u, 0u, 0u, 0u};
 }
@@ -267,7 +282,8 @@ static int moe_layer(bool v4, void* out, int out_dtype, float limit, const void*
   const int64_t tiles_from = tuning().tiles >= 0 ? tuning().tiles : (fmt == BP_TQ1 && act == BP_BF16 ? 24 : 64);
   const bool tiles = T > tiles_from;
   const bool small = n <= ROUTE_SMALL_N && (((uintptr_t)x | (uintptr_t)p.xg) & 15) == 0;
-  const bool prezeroed = small && !tiles;  // (the GEMMs over the tile list write instead of accumulate)
+  const bool aligned16 = (((uintptr_t)x | (uintptr_t)p.xg) & 15) == 0;
+  const bool prezeroed = aligned16 && !tiles;  // the zero-fill rides along with the gather (the GEMMs over the tile list write instead of accumulate)
   if (small) {
     const int64_t z0 = prezeroed ? (int64_t)(4 * (size_t)n * 2 * I / 16) : 0, z1 = prezeroed ? (int64_t)(4 * (size_t)n * H / 16) : 0;
     int64_t g = (z0 + z1 + (int64_t)n * (H / 8) + ROUTE_SMALL_THREADS - 1) / ROUTE_SMALL_THREADS;
@@ -278,7 +294,14 @@ static int moe_layer(bool v4, void* out, int out_dtype, float limit, const void*
     if ((rc = check_launch("route_small")) != BP_OK) return rc;
   } else {
     if ((rc = sort_with_inverse(p.order, p.offsets, p.inv, experts, n, E, p.sort_ws, bad, s)) != BP_OK) return rc;
-    if ((rc = bp_gather_rows(p.xg, x, p.order, k, n, T, 2 * H, s)) != BP_OK) return rc;
+    if (aligned16) {
+      const int64_t z0 = prezeroed ? (int64_t)(4 * (size_t)n * 2 * I / 16) : 0, z1 = prezeroed ? (int64_t)(4 * (size_t)n * H / 16) : 0;
+      int64_t g = (z0 + z1 + n * (H / 8) + 255) / 256;
+      g = g < 1 ? 1 : (g > 4096 ? 4096 : g);
+      hipLaunchKernelGGL(k_gather_zero, dim3((unsigned)g), dim3(256), 0, s, (u32x4*)p.xg, (const u32x4*)x, p.order, n, k, T, H / 8, (u32x4*)p.gu, z0,
+                         (u32x4*)p.y, z1);
+      if ((rc = check_launch("gather_zero")) != BP_OK) return rc;
+    } else if ((rc = bp_gather_rows(p.xg, x, p.order, k, n, T, 2 * H, s)) != BP_OK) return rc;
   }
 
   auto gemm = [&](float* o, const void* in, const uint8_t* const* packed, const void* const* scale, int64_t N, int64_t K, bool tiles) -> int {
