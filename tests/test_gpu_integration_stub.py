@@ -1,5 +1,5 @@
-"""The binding that INTEGRATION.md proposes for the reference (Option B), executed verbatim: the stub text is cut out of
-the document, exec'd, and called exactly as boilerplate/kernels/ternary_cuda.py:98-103 calls its native module
+"""The binding that the integration guide at the repository root proposes for the reference (its option B), executed
+verbatim: the stub text is cut out of the document, exec'd, and called exactly as boilerplate/kernels/ternary_cuda.py:98-103 calls its native module
 (11 positional arguments, float32 scales from `w_scale.float()`, a real `lut1` tensor, device offsets)."""
 
 import re
