@@ -341,3 +341,23 @@ def test_router_kernel_ties_go_to_the_lower_expert_and_bad_arguments_are_rejecte
     assert b"1024 experts" in lib.bp_last_error()
     assert lib.bp_route_topk(w.data_ptr(), _lib.BP_I8, ids.data_ptr(), logits.data_ptr(), _lib.BP_F32, 3, 200, 4, 0, None) == 1
     assert lib.bp_route_topk(w.data_ptr(), _lib.BP_F32, ids.data_ptr(), logits.data_ptr(), _lib.BP_F32, 3, 3, 4, 0, None) == 1
+
+
+@pytest.mark.parametrize("T,E,k", [(25, 8, 2), (40, 4, 2), (42, 16, 6), (33, 3, 3)])
+def test_small_batch_preparation_kernel_writes_the_tile_list(T, E, k):
+    """Between 24 tokens (TQ1, bf16: the tile list takes over) and 256 routed rows the preparation kernel also writes the
+    list of token tiles - experts without rows, experts with more than one tile of 32 rows - and the layer equals the
+    composed calls bit for bit (the same GEMM kernel, sized by the bound instead of the list)."""
+    from deepseekternarized_amd import ext
+
+    moe, _ = _layer("tq1", "bf16", 1024, 1024, E, k, seed=T)
+    g = torch.Generator(device="cuda").manual_seed(7 * T)
+    x = torch.randn(T, 1024, device="cuda", generator=g).to(torch.bfloat16)
+    logits = torch.randn(T, E, device="cuda", generator=g) * 2.0
+    logits[:, 0] -= 30.0  # expert 0 gets no row
+    if E == 4:
+        logits[:, 1] += 6.0  # expert 1 is in every token's top-2: more than one tile
+    got = moe(x, logits)
+    assert ext().last_kernel() == "gemm_tq1f_bf16", ext().last_kernel()
+    want = moe.composed(x, logits)
+    assert torch.isfinite(got.float()).all() and torch.equal(got, want)
