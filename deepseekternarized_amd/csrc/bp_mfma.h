@@ -55,6 +55,11 @@ __device__ __forceinline__ __amdgpu_buffer_rsrc_t make_rsrc(const void* base, in
   const int n = bytes > 0x7fffffff ? 0x7fffffff : (int)bytes;
   return __builtin_amdgcn_make_buffer_rsrc(const_cast<void*>(base), (short)0, n, 0x00020000);
 }
+// A buffer load returns zero for a dword that straddles the end of its range, valid bytes included. Ranges over tensors
+// that may start at any byte (the base is aligned down to a dword by the caller) therefore end with the dword that holds
+// the tensor's last byte: up to 3 bytes behind the tensor are read with it - inside a dword of which the tensor owns a
+// byte - and never used.
+__device__ __forceinline__ int64_t whole_dwords(int64_t bytes) { return (bytes + 3) & ~(int64_t)3; }
 __device__ __forceinline__ u32x4 buf_load16(__amdgpu_buffer_rsrc_t r, unsigned lane_off, unsigned wave_off) {
   return __builtin_bit_cast(u32x4, __builtin_amdgcn_raw_buffer_load_b128(r, (int)lane_off, (int)wave_off, 0));
 }

@@ -150,7 +150,7 @@ __global__ __launch_bounds__(WAVES * 64, 4) void k_tq1_gemv(GemmArgs a, int CPT 
     const unsigned char* wbeg = a.packed[term];
     const unsigned char* wave_rows = wbeg + (e * a.N + n0) * a.Kp;
     const unsigned mis = (unsigned)((uintptr_t)wave_rows & 3);
-    const __amdgpu_buffer_rsrc_t wrs = make_rsrc(wave_rows - mis, (wbeg + a.E * a.N * a.Kp) - (wave_rows - mis));
+    const __amdgpu_buffer_rsrc_t wrs = make_rsrc(wave_rows - mis, whole_dwords((wbeg + a.E * a.N * a.Kp) - (wave_rows - mis)));
     const unsigned ro = mis + (unsigned)r16 * (unsigned)a.Kp;
     const unsigned dlt = ro & 3u;            // chunk byte j of this lane's row sits at offset j + dlt of its buffer row
     const unsigned voff_row = ro & ~3u, voff = voff_row + 16u * b;

@@ -364,14 +364,14 @@ __global__ __launch_bounds__(WAVES * 64, KS ? 2 : 4) void k_tq1_gemv_fp4(GemmArg
     const unsigned char* wbeg = a.packed[term];
     const unsigned char* expert_rows = wbeg + e * a.N * a.Kp;
     const unsigned mis = (unsigned)((uintptr_t)expert_rows & 3);
-    const __amdgpu_buffer_rsrc_t wrs = make_rsrc(expert_rows - mis, (wbeg + a.E * a.N * a.Kp) - (expert_rows - mis));
+    const __amdgpu_buffer_rsrc_t wrs = make_rsrc(expert_rows - mis, whole_dwords((wbeg + a.E * a.N * a.Kp) - (expert_rows - mis)));
     const unsigned ro = mis + (unsigned)r16 * (unsigned)a.Kp;
     const unsigned dlt = ro & 3u;  // the lane's window starts dlt bytes before its bytes of the row
     const unsigned voff = (ro & ~3u) + 16u * kb;
     const unsigned char* sbeg = (const unsigned char*)a.w_scale[term];
     const unsigned char* expert_scales = sbeg + e * a.N * a.G * SB;
     const unsigned smis = (unsigned)((uintptr_t)expert_scales & 3);
-    const __amdgpu_buffer_rsrc_t srs = make_rsrc(expert_scales - smis, (sbeg + a.E * a.N * a.G * SB) - (expert_scales - smis));
+    const __amdgpu_buffer_rsrc_t srs = make_rsrc(expert_scales - smis, whole_dwords((sbeg + a.E * a.N * a.G * SB) - (expert_scales - smis)));
     const unsigned srow = smis + (unsigned)r16 * (unsigned)a.G * SB;
     u32x4 W[RD][GR][2];
     u32x2 SQ[GR];  // the scales of one chunk: refilled for the next chunk as soon as they have been applied
@@ -796,7 +796,7 @@ __global__ __launch_bounds__(CW_WAVES * 64) void k_tq1_gemv_cw(GemmArgs a, int n
   auto setup_term = [&](int term) {
     const unsigned char* expert_rows = a.packed[term] + e * a.N * a.Kp;
     const unsigned mis = (unsigned)((uintptr_t)expert_rows & 3);
-    wrs = make_rsrc(expert_rows - mis, a.N * a.Kp + mis);
+    wrs = make_rsrc(expert_rows - mis, whole_dwords(a.N * a.Kp + mis));
     srs = make_rsrc((const unsigned char*)a.w_scale[term] + e * a.N * a.G * SB, a.N * a.G * SB);  // (dword-aligned: checked by the host)
     const unsigned ro = mis + (unsigned)kb * (unsigned)a.Kp;
     w_lane = (ro & ~3u) + 16u * (unsigned)r16;  // (rows 4 apart are a multiple of 4 bytes apart)

@@ -744,3 +744,41 @@ def test_float_activations_run_on_the_bf16_kernels_as_a_pair(bp, fmt, M, act):
     torch.cuda.synchronize()
     assert rc == 0 and bp.ext().last_kernel().startswith("general"), bp.ext().last_kernel()
     np.testing.assert_allclose(out.cpu().numpy(), want, rtol=1e-4, atol=1e-3)
+
+
+# --------------------------------------------------------------------------- packed tensors that start at any byte
+@pytest.mark.parametrize("counts,act,switch,prefix", [
+    ([1, 1], "bf16", None, "fp4_tq1_t1_ks"), ([1, 1], "int8", None, "fp4_tq1_t1_ks"), ([3, 2], "bf16", None, "fp4_tq1_m4"),
+    ([1, 1], "bf16", ("BP_TUNE_TQ1", "chunk"), "fp4_tq1_t1_cw"), ([2, 1], "bf16", ("BP_TUNE_TQ1", "chunk"), "fp4_tq1_m2_cw"),
+    ([1, 1], "bf16", ("BP_TUNE_TQ1", "lut"), "lut_tq1"), ([12, 3], "bf16", ("BP_TUNE_TQ1", "mfma"), "mfma_tq1"),
+    ([9, 20], "bf16", None, "gemm_tq1f"), ([9, 20], "bf16", ("BP_TUNE_TQ2G", "bf16"), "gemm_tq1_"), ([9, 20], "int8", None, "gemm_tq1_"),
+])
+def test_tq1_packed_tensor_at_every_byte_alignment(bp, tune, counts, act, switch, prefix):
+    """TQ1 rows start at any byte, and so may the tensor: a view 1, 2 or 3 bytes into an allocation, with other bytes
+    behind it. The kernels read the rows through a buffer whose base is aligned down to a dword; its range has to end
+    with the dword that holds the tensor's last byte (a dword that straddles the end of a range reads as zero, and the
+    last row's last bytes with it). Every offset gives the bits of offset 0."""
+    if switch:
+        tune(*switch)
+    E, N, K = len(counts), 48 if "cw" not in prefix else 2064, 2048 if "cw" not in prefix else 1024
+    rng = np.random.default_rng(5)
+    packed, scales = synth_weights(5, E, N, K, GROUP, "tq1", terms=1)
+    offsets = np.concatenate([[0], np.cumsum(counts)]).astype(np.int64)
+    T = int(offsets[-1])
+    x, xs, xd, xsd = _activations(rng, T, K, act)
+    want = np.zeros((T, N), np.float32)
+    for e in range(E):
+        a, b = int(offsets[e]), int(offsets[e + 1])
+        c_gemm(x[a:b], None if xs is None else xs[a:b], packed[0][e], scales[0][e].astype(np.float32), K, GROUP, "tq1", out=want[a:b])
+    p, first = packed[0], None
+    for off in (0, 1, 2, 3):
+        buf = torch.full((p.size + 64,), 77, dtype=torch.uint8, device="cuda")  # (what lies behind the tensor must not matter)
+        base = (16 - buf.data_ptr() % 16) % 16 + off
+        buf[base:base + p.size] = dev(p).reshape(-1)
+        view = buf[base:base + p.size].view(p.shape)
+        assert view.data_ptr() % 4 == off
+        got = bp.grouped_ternary_gemm(xd, xsd, offsets.tolist(), [view], [dev(scales[0])], K, GROUP, "tq1").cpu().numpy()
+        assert bp.ext().last_kernel().startswith(prefix), bp.ext().last_kernel()
+        _check(got, want)
+        first = got if first is None else first
+        assert np.array_equal(got, first), off
