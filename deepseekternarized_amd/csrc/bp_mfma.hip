@@ -11,6 +11,9 @@ bool mfma_supports(const GemmArgs& a) {
   if (a.fmt == BP_TQ2) {
     if (a.x_dtype != BP_BF16 && a.x_dtype != BP_I8) return false;
     if (a.K % 256 != 0 || a.K < 1024) return false;  // whole steps of 64 packed bytes
+    // (an odd number of 2-byte scales per row: every other row of scales starts in the middle of a dword, and the kernels
+    // read a row's scales in dword-aligned pieces)
+    if (a.group == 256 && a.K % 512 != 0 && a.scale_dtype != BP_F32) return false;
     for (int t = 0; t < a.n_terms; ++t) {
       if (((uintptr_t)a.packed[t] & 15) != 0) return false;
       if (((uintptr_t)a.w_scale[t] & 15) != 0) return false;

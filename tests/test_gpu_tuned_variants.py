@@ -782,3 +782,15 @@ def test_tq1_packed_tensor_at_every_byte_alignment(bp, tune, counts, act, switch
         _check(got, want)
         first = got if first is None else first
         assert np.array_equal(got, first), off
+
+
+@pytest.mark.parametrize("act", ["bf16", "int8"])
+@pytest.mark.parametrize("K,counts", [(2304, [8]), (5376, [1, 0, 1]), (4352, [1, 24]), (9472, [2])])
+@pytest.mark.parametrize("scale_dtype", [np.float16, "f32"])
+def test_tq2_group_256_with_an_odd_number_of_scales_per_row(bp, act, K, counts, scale_dtype):
+    """K / 256 odd with one scale per 256 weights: every other row of 2-byte scales starts in the middle of a dword. The
+    tuned TQ2 kernels read a row's scales in dword-aligned pieces and leave such calls to the general kernel (float32
+    scales keep their rows aligned and stay on the tuned kernels)."""
+    got, want, kern = _run(bp, "tq2", len(counts), 144, K, counts, act, seed=K, scale_dtype=scale_dtype, group=256)
+    assert kern.startswith("general") == (scale_dtype is np.float16), kern
+    _check(got, want)
