@@ -326,7 +326,10 @@ __global__ __launch_bounds__(WAVES * 64, KS ? 2 : 4) void k_tq1_gemv_fp4(GemmArg
   // The last bytes of a chunk are completed from the first dword of the chunk after it (rows start at any byte). At
   // the end of a row that dword meets activations that are 0; at the end of a segment it is needed, so the chunk
   // after a segment that is not the last one is loaded as well.
-  const int last_load = (NTOK > 1 || KS) && cb + nch < total_chunks ? nch : nch - 1;
+  // (Rows of whole chunks - Kp a multiple of 128 - at an address that is not a multiple of 4 end up to 3 bytes into the
+  // chunk after their last one, with bytes that count: that chunk is loaded too; the term sets last_load below.)
+  const int last_load_aligned = (NTOK > 1 || KS) && cb + nch < total_chunks ? nch : nch - 1;
+  int last_load = last_load_aligned;
 
   if (!LATE) {
     f4_build_tiles<NTOK, WAVES>(a, tok, ntok, nchunks, KS ? 0 : cb, wave, lane);  // (KS: the tiles of all chunks, tile index = chunk)
@@ -345,7 +348,7 @@ __global__ __launch_bounds__(WAVES * 64, KS ? 2 : 4) void k_tq1_gemv_fp4(GemmArg
   // The tables serve `bpw` blocks of WAVES x GR x 16 rows, one after the other (the build is paid once per workgroup),
   // term by term: a term's blocks form one stream of chunks, and when the chunks of a row fill the ring a whole
   // number of times the refills run on into the next block, so the loads do not drain between blocks.
-  const bool chain = !KS && nchunks % RD == 0 && last_load == nchunks - 1;
+  bool chain = false;  // (set by the term)
   auto block_row = [&](int pass) -> int64_t {  // first row of this wave's tile(s) in block `pass`
     if (KS) return ((int64_t)blockIdx.x * bpw + pass) * (16 * GR);
     return (((int64_t)blockIdx.x * bpw + pass) * WAVES + wave) * (16 * GR);
@@ -364,6 +367,8 @@ __global__ __launch_bounds__(WAVES * 64, KS ? 2 : 4) void k_tq1_gemv_fp4(GemmArg
     const unsigned char* wbeg = a.packed[term];
     const unsigned char* expert_rows = wbeg + e * a.N * a.Kp;
     const unsigned mis = (unsigned)((uintptr_t)expert_rows & 3);
+    last_load = mis != 0 && a.Kp == 128 * (int64_t)total_chunks && cb + nch == total_chunks ? nch : last_load_aligned;
+    chain = !KS && nchunks % RD == 0 && last_load == nchunks - 1;
     const __amdgpu_buffer_rsrc_t wrs = make_rsrc(expert_rows - mis, whole_dwords((wbeg + a.E * a.N * a.Kp) - (expert_rows - mis)));
     const unsigned ro = mis + (unsigned)r16 * (unsigned)a.Kp;
     const unsigned dlt = ro & 3u;  // the lane's window starts dlt bytes before its bytes of the row
