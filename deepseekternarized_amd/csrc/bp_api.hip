@@ -36,11 +36,12 @@ namespace {
 std::atomic<const Tuning*> g_tuning{nullptr};
 std::once_flag g_tuning_once;
 void read_tuning() {
-  Tuning* t = new Tuning{0, 0, 0, 0, 0, -1, 0, -1};
+  Tuning* t = new Tuning{0, 0, 0, 0, 0, 0, -1, 0, -1};
   if (const char* v = getenv("BP_TUNE_R")) t->r = atoi(v);
   if (const char* v = getenv("BP_TUNE_WAVES")) t->waves = atoi(v);
   if (const char* v = getenv("BP_TUNE_TQ1")) t->tq1 = v[0];
   if (const char* v = getenv("BP_TUNE_TQ2G")) t->tq2g = v[0];
+  if (const char* v = getenv("BP_TUNE_TQ2V")) t->tq2v = v[0];
   if (const char* v = getenv("BP_TUNE_F4W")) t->f4w = atoi(v);
   if (const char* v = getenv("BP_TUNE_F4T")) t->f4t = atoi(v);
   if (const char* v = getenv("BP_TUNE_CPT")) t->cpt = atoi(v);

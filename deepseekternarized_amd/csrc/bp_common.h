@@ -94,6 +94,7 @@ struct Tuning {
   int waves;   // BP_TUNE_WAVES: waves per workgroup (8, 16)
   char tq1;    // BP_TUNE_TQ1: 'l' table-lookup GEMV, 'm' 16-token MFMA kernel, 'c' the chunk-per-wave GEMV wherever it can run, 'r' never (first letter of the value)
   char tq2g;   // BP_TUNE_TQ2G: 'b' (bf16) never the fp8 x fp4 grouped GEMM over converted activations, 'f' (fp4) wherever it can run
+  char tq2v;   // BP_TUNE_TQ2V: 'k' the K-split fp8 x fp4 TQ2 GEMV wherever it can run, 'n' never
   int f4w;     // BP_TUNE_F4W: waves per workgroup of the fp8 x fp4 GEMV (8, 16)
   int f4t;     // BP_TUNE_F4T: routed rows per expert up to which launches of 8 rows are used (-1 = default)
   int cpt;     // BP_TUNE_CPT: chunks per table pass of the table-lookup GEMV

@@ -53,6 +53,10 @@ int launch_mfma(const GemmArgs& a, hipStream_t s) {
   if (tuning().r == 1 || tuning().r == 2) R = tuning().r;
   if (tuning().waves == 8 || tuning().waves == 16) waves = tuning().waves;
   if (a.fmt == BP_TQ1) return launch_mfma_tq1(a, s, waves);
+  if (a.max_rows == 1) {  // decode GEMV of a large call: K split over the waves, weights as fp4
+    const int rc = launch_tq2_gemv_fp4(a, s);
+    if (rc != BP_ERR_UNSUPPORTED) return rc;
+  }
   // Experts with more than 16 rows get token tiles of 32 - unless the batch is sparse (on average at most 8 rows per
   // expert) and the bound small: then nearly every expert fits one 16-token tile of the lighter kernel, and the few
   // that do not (or a loose upper bound from a caller that keeps the routing on the device) cost a second tile.

@@ -1,4 +1,4 @@
-"""Every code path of the tuned kernels (bp_mfma_tq2.hip, bp_gemm_tq2.hip, bp_mfma_tq1.hip, bp_gemm_tq1.hip, bp_tq1_gemv.hip, bp_tq1_gemv_fp4.hip) against the CPU oracle.
+"""Every code path of the tuned kernels (bp_mfma_tq2.hip, bp_tq2_gemv_fp4.hip, bp_gemm_tq2.hip, bp_mfma_tq1.hip, bp_gemm_tq1.hip, bp_tq1_gemv.hip, bp_tq1_gemv_fp4.hip) against the CPU oracle.
 
 The shapes are chosen by what they select inside the launchers, not by size: odd / even packed row
 lengths (row starts at every byte alignment), K that fits one activation / table tile or needs several,
@@ -434,6 +434,114 @@ def test_tq1_mfma_scales_from_global_memory(bp, tune):
     _check(got, want)
 
 
+# --------------------------------------------------------------------------- TQ2 decode GEMV with K split over the waves
+# One token row per expert on the fp8 x fp4 matrix instruction (bp_tq2_gemv_fp4.hip; kernel names fp4_tq2_t1_ks and
+# fp4_tq2_i8_t1_ks): the default for large single-token calls from K = 2048; BP_TUNE_TQ2V=k selects it wherever it can
+# run, =n never.
+@pytest.mark.parametrize("act", ["bf16", "int8"])
+@pytest.mark.parametrize("E,N,K,group,terms,sdt", [
+    (3, 64, 1024, 128, 1, np.float16),      # 2 waves, a workgroup of one round
+    (2, 144, 1280, 128, 2, "bf16"),         # an odd number of steps: the last wave's second step lies past the row
+    (3, 1040, 4096, 256, 2, np.float16),    # a scale per 256 weights, stacked terms, 65 tiles (a last round of one tile)
+    (2, 2064, 7168, 128, 1, np.float16),    # the headline K: 14 waves
+    (1, 272, 8192, 128, 1, "bf16"),         # 16 waves
+    (5, 48, 768, 128, 1, np.float16),       # below the kernel's K: the other kernels
+])
+def test_tq2_single_token_gemv_with_k_split_over_the_waves(bp, tune, act, E, N, K, group, terms, sdt):
+    tune("BP_TUNE_TQ2V", "k")
+    counts = [1] * E
+    if E > 2:
+        counts[1] = 0  # an expert without a token row
+    got, want, kern = _run(bp, "tq2", E, N, K, counts, act, terms=terms, seed=K + N, scale_dtype=sdt, group=group, max_rows=1)
+    if K >= 1024:
+        assert kern == ("fp4_tq2_i8_t1_ks" if act == "int8" else "fp4_tq2_t1_ks"), kern
+    else:
+        assert not kern.startswith("fp4_tq2"), kern
+    _check(got, want)
+    if act == "int8":  # fp8 pieces hold int8 values exactly and the sums are integers: only the order of the float32 scale products differs
+        assert rel_l2(got, want) <= 1e-6, rel_l2(got, want)
+
+
+def test_tq2_k_split_gemv_is_the_default_for_large_single_token_calls(bp):
+    """64 experts x 64 row tiles at K = 2048 (16 tiles per CU): both activation dtypes take the kernel without a switch;
+    the same call with two rows for one expert does not."""
+    for act in ("bf16", "int8"):
+        got, want, kern = _run(bp, "tq2", 64, 1024, 2048, [1] * 64, act, seed=5, max_rows=1)
+        assert kern == ("fp4_tq2_i8_t1_ks" if act == "int8" else "fp4_tq2_t1_ks"), kern
+        _check(got, want)
+    got, want, kern = _run(bp, "tq2", 64, 1024, 2048, [1] * 63 + [2], "bf16", seed=6, max_rows=2)
+    assert kern.startswith("mfma_tq2"), kern
+    _check(got, want)
+
+
+def test_tq2_k_split_gemv_adds_to_the_output_and_keeps_other_rows(bp, tune):
+    """The C-ABI call accumulates (include/bp_ternary.h): the kernel reads what it adds to when a workgroup starts and
+    writes once at its end; rows of experts without a token and rows past N / 16 tiles of a workgroup stay as they were."""
+    from deepseekternarized_amd.kernels import _lib
+    tune("BP_TUNE_TQ2V", "k")
+    lib = _lib.load()
+    E, N, K = 3, 400, 2048
+    packed, scales = synth_weights(3, E, N, K, GROUP, "tq2")
+    rng = np.random.default_rng(3)
+    x = orc.bf16_round(rng.standard_normal((2, K)).astype(np.float32))
+    offsets = np.array([0, 1, 1, 2], np.int64)
+    base = rng.standard_normal((2, N)).astype(np.float32)
+    out = dev(base.copy())
+    xd, pk, sc, od = dev(x).to(torch.bfloat16), dev(packed[0]), dev(scales[0]), dev(offsets)
+    import ctypes
+    pa = (ctypes.c_void_p * 1)(pk.data_ptr())
+    sa = (ctypes.c_void_p * 1)(sc.data_ptr())
+    rc = lib.bp_ternary_grouped_gemm(out.data_ptr(), xd.data_ptr(), _lib.BP_BF16, None, od.data_ptr(), None, pa, sa, _lib.BP_F16,
+                                     1, 2, N, K, K // 4, K // GROUP, GROUP, E, _lib.BP_TQ2, 1, None, None)
+    assert rc == 0, lib.bp_last_error()
+    assert lib.bp_last_kernel().decode() == "fp4_tq2_t1_ks"
+    want = base.copy()
+    c_gemm(x[0:1], None, packed[0][0], scales[0][0].astype(np.float32), K, GROUP, "tq2", out=want[0:1])
+    c_gemm(x[1:2], None, packed[0][2], scales[0][2].astype(np.float32), K, GROUP, "tq2", out=want[1:2])
+    assert rel_l2(out.cpu().numpy(), want) <= 1e-5
+
+
+def test_tq2_k_split_gemv_keeps_small_activations_next_to_outliers(bp, tune):
+    """Three fp8 pieces under a power-of-two prescale per 128 activations represent bf16 values to 2^-20 of the group's
+    largest magnitude; the matrix instruction's aligned sum of 128 products is what limits the result when a group
+    holds values many decades apart: held to 5e-4 here (measured 1-2e-4; the general tolerance is 1e-3), and to 2e-5 on
+    normally distributed activations (measured 1e-7 to 4e-6)."""
+    tune("BP_TUNE_TQ2V", "k")
+    rng = np.random.default_rng(21)
+    E, N, K = 2, 64, 4096
+    packed, scales = synth_weights(21, E, N, K, GROUP, "tq2")
+    for spread, bound in ((0.0, 2e-5), (6.0, 5e-4)):
+        x = rng.standard_normal((E, K)).astype(np.float32) * np.exp(rng.uniform(-spread, spread, (E, K))).astype(np.float32)
+        if spread:
+            x[:, ::97] *= 1000.0
+        x = orc.bf16_round(x)
+        want = np.zeros((E, N), np.float32)
+        for e in range(E):
+            c_gemm(x[e:e + 1], None, packed[0][e], scales[0][e].astype(np.float32), K, GROUP, "tq2", out=want[e:e + 1])
+        got = bp.grouped_ternary_gemm(dev(x).to(torch.bfloat16), None, dev(np.array([0, 1, 2], np.int64)), [dev(packed[0])], [dev(scales[0])], K, GROUP, "tq2", max_rows=1).cpu().numpy()
+        assert bp.ext().last_kernel() == "fp4_tq2_t1_ks"
+        assert np.isfinite(got).all() and rel_l2(got, want) <= bound, (spread, rel_l2(got, want))
+
+
+def test_tq2_k_split_gemv_counts_the_unused_code_as_unpack_does(bp, tune):
+    """pack never writes the 2-bit code 3. unpack reads it as +2 (boilerplate/ternary/pack.py:47-60: code - 1) and so does
+    this kernel (E2M1 1.5 = 3 / 2, minus the offset); the reference's CPU kernel adds or subtracts by the trit's sign
+    only (boilerplate/kernels/csrc/boilerplate_cpu.cpp:70-77), which makes such a weight +1 there."""
+    tune("BP_TUNE_TQ2V", "k")
+    rng = np.random.default_rng(8)
+    E, N, K = 1, 32, 2048
+    packed = rng.integers(0, 256, (E, N, K // 4), dtype=np.uint8)  # every code, 3 included
+    scales = (rng.uniform(0.01, 0.1, (E, N, K // GROUP))).astype(np.float16)
+    x = orc.bf16_round(rng.standard_normal((1, K)).astype(np.float32))
+    trits = orc.unpack(packed[0], "tq2", K).astype(np.float64)
+    assert trits.max() == 2
+    sums = (trits.reshape(N, K // GROUP, GROUP) * x.astype(np.float64).reshape(1, K // GROUP, GROUP)).sum(-1)
+    want = (sums * scales[0].astype(np.float64)).sum(-1)[None].astype(np.float32)
+    got = bp.grouped_ternary_gemm(dev(x).to(torch.bfloat16), None, dev(np.array([0, 1], np.int64)), [dev(packed)], [dev(scales)], K, GROUP, "tq2", max_rows=1).cpu().numpy()
+    assert bp.ext().last_kernel() == "fp4_tq2_t1_ks"
+    assert rel_l2(got, want) <= 1e-5, rel_l2(got, want)
+
+
 # --------------------------------------------------------------------------- TQ2 MFMA kernel
 @pytest.mark.parametrize("act", ["bf16", "int8"])
 @pytest.mark.parametrize("K,counts", [(1024, [1, 0, 1]), (2048, [1, 1, 1]), (7168, [3, 0, 16]), (4096, [33, 1, 20]), (32768, [1, 2, 0])])
@@ -672,7 +780,7 @@ def test_group_256(bp, act, fmt, K, counts, prefix):
 # --------------------------------------------------------------------------- activations that are not finite
 @pytest.mark.parametrize("fmt,counts,prefix", [
     ("tq1", [1, 1], "fp4_tq1_t1"), ("tq1", [1, 1], "fp4_tq1_t1_cw"), ("tq1", [2, 2], "fp4_tq1_m2_cw"), ("tq1", [4, 3], "fp4_tq1_m4"), ("tq1", [20, 12], "gemm_tq1"),
-    ("tq2", [1, 1], "mfma_tq2"), ("tq2", [9, 16], "mfma_tq2"), ("tq2", [40, 33], "gemm_tq2_"), ("tq2", [40, 33], "gemm_tq2f_"),
+    ("tq2", [1, 1], "mfma_tq2"), ("tq2", [1, 1], "fp4_tq2_t1_ks"), ("tq2", [9, 16], "mfma_tq2"), ("tq2", [40, 33], "gemm_tq2_"), ("tq2", [40, 33], "gemm_tq2f_"),
 ])
 def test_non_finite_activations_never_give_finite_wrong_values(bp, tune, fmt, counts, prefix):
     """The reference's CPU kernel skips zero weights (boilerplate/kernels/csrc/boilerplate_cpu.cpp:70-77), so a NaN or an
@@ -684,6 +792,8 @@ def test_non_finite_activations_never_give_finite_wrong_values(bp, tune, fmt, co
         tune("BP_TUNE_TQ2G", "fp4")
     if prefix.endswith("_cw"):
         tune("BP_TUNE_TQ1", "chunk")
+    if prefix.startswith("fp4_tq2"):
+        tune("BP_TUNE_TQ2V", "k")
     rng = np.random.default_rng(5)
     packed, scales = synth_weights(17, E, N, K, GROUP, fmt)
     trits = np.stack([orc.unpack(packed[0][e], fmt, K) for e in range(E)])
