@@ -734,6 +734,7 @@ __global__ __launch_bounds__(WAVES * 64, KS ? 2 : 4) void k_tq1_gemv_fp4(GemmArg
 // place of the operand A tiles once those are in registers.
 constexpr int CW_WAVES = 16;
 constexpr int CW_LUT_BYTES = 256 * 256;  // byte -> 5 fp4 codes, 64 copies: entry v copy c at 256 v + 4 c
+constexpr int CW_STAGE_PER_THREAD = 4;    // outputs of a workgroup per thread at most (they wait in LDS from the first barrier to the end)
 // A row's image in a tile buffer: up to 3 bytes of misalignment, the row's Kp bytes and the dword after them, in whole
 // 16-byte pieces, at a pitch that is an odd number of pieces (16 rows: 16 different groups of 4 banks). What a
 // multiplier reads past a row's image in its last chunk (the next row's bytes, or what follows the buffer) meets
@@ -787,6 +788,19 @@ __global__ __launch_bounds__(CW_WAVES * 64) void k_tq1_gemv_cw(GemmArgs a, int n
   const int n_iter = (tiles_per_wg + groups - 1) / groups;  // tiles of a group
   const int n_int = (n_iter + TPB - 1) / TPB;                 // barriers: TPB tiles each
   auto tile_of = [&](int t) -> int64_t { return tile0 + (int64_t)t * groups + grp; };
+  // ---- the workgroup's outputs, [tile of the workgroup][token][row] float32, behind the buffers and sums (and behind the
+  // operand A tiles, which are built in the buffers' place): read from memory now, parked in LDS before the first
+  // barrier, added to there tile by tile, and written back once after the last term - no access to the outputs in the loop.
+  const int stream_bytes = groups * NB * (buf_bytes + nchunks * 64 * NTOK), build_bytes = nchunks * NTOK * F4_CHUNK_BYTES;
+  const unsigned stage = (unsigned)(AT + (stream_bytes > build_bytes ? stream_bytes : build_bytes));
+  const int n_stage = (int)(tile_end - tile0) * 16 * NTOK;  // (at most CW_STAGE_PER_THREAD x the workgroup's threads: the launcher's bound)
+  auto out_index = [&](int o) -> int64_t { return (tok + ((o >> 4) % NTOK)) * a.N + (tile0 + (o >> 4) / NTOK) * 16 + (o & 15); };
+  float was[CW_STAGE_PER_THREAD];
+#pragma unroll
+  for (int u = 0; u < CW_STAGE_PER_THREAD; ++u) {
+    const int o = (int)threadIdx.x + u * THREADS;
+    was[u] = o < n_stage && ((o >> 4) % NTOK) < ntok ? a.out[out_index(o)] : 0.f;
+  }
 
   // ---- loaders: state of the current term (the expert's rows and scales as buffers of their own: a tile past N reads
   // zeros) and the wave's loads of a tile: LPW of the nl wave loads of packed bytes (li = i * lpg + lidx: rows
@@ -858,6 +872,11 @@ __global__ __launch_bounds__(CW_WAVES * 64) void k_tq1_gemv_cw(GemmArgs a, int n
       }
     }
     *(lds_u32x4*)(16 * idx) = u32x4{ent, ent, ent, ent};
+  }
+#pragma unroll
+  for (int u = 0; u < CW_STAGE_PER_THREAD; ++u) {
+    const int o = (int)threadIdx.x + u * THREADS;
+    if (o < n_stage) *(lds_u32*)(stage + 4u * (unsigned)o) = __float_as_uint(was[u]);
   }
   __syncthreads();
 
@@ -967,20 +986,8 @@ __global__ __launch_bounds__(CW_WAVES * 64) void k_tq1_gemv_cw(GemmArgs a, int n
   for (int term = 0; term < a.n_terms; ++term) {
     if (term > 0) setup_term(term);
     // The sums of the tile of iteration t, by the group's first loader: lane (row n, quarter q) adds chunks q, q + 4, ...
-    // in that order, the row's four lanes are added in a fixed order too, and the output takes one addition per row.
-    // The outputs that a tile is added to are requested a barrier before they are used (device scope: with stacked terms
-    // the value may be one this wave stored a term ago), by every loader in the same place of its instruction stream
-    // (past the buffer for all but the 16 lanes that use them), so that the waits on the loads of the tiles stay exact.
-    const __amdgpu_buffer_rsrc_t ors = make_rsrc(a.out + tok * a.N, (int64_t)ntok * a.N * 4);  // (the launch's token rows)
-    float before[2][NTOK];
-    auto request_out = [&](int t, auto slot_c) {
-      constexpr int slot = decltype(slot_c)::value;
-      const int64_t tile = tile_of(t);
-      const bool mine = loader && lidx == 0 && lane < 16 && tile < tile_end;
-#pragma unroll
-      for (int tt = 0; tt < NTOK; ++tt)  // (a token row the expert does not have lies past the buffer)
-        before[slot][tt] = __uint_as_float((unsigned)__builtin_amdgcn_raw_buffer_load_b32(ors, (int)(mine ? (unsigned)(tile * 64 + 4 * lane) : 0x7ffffff0u), (int)((unsigned)tt * (unsigned)a.N * 4u), 1 /* glc */));
-    };
+    // in that order, the row's four lanes are added in a fixed order too, and the row's entry of the output stage takes
+    // one addition (this wave is the only one that touches its group's entries between the first barrier and the end).
     auto reduce = [&](int t, auto slot_c) {
       constexpr int slot = decltype(slot_c)::value;
       if (!loader || lidx != 0) return;  // (uniform)
@@ -999,7 +1006,10 @@ __global__ __launch_bounds__(CW_WAVES * 64) void k_tq1_gemv_cw(GemmArgs a, int n
         v = __uint_as_float(h32[0]) + __uint_as_float(h32[1]);
         const auto h16 = __builtin_amdgcn_permlane16_swap(__float_as_uint(v), __float_as_uint(v), false, false);
         v = __uint_as_float(h16[0]) + __uint_as_float(h16[1]);
-        if (lane < 16 && tile < tile_end && tt < ntok) a.out[(tok + tt) * a.N + tile * 16 + lane] = before[slot][tt] + (a.x_dtype == BP_I8 ? v * xsc[tt] : v);
+        if (lane < 16 && tile < tile_end && tt < ntok) {
+          const unsigned at_out = stage + (unsigned)((((int)(tile - tile0) * NTOK + tt) * 16 + lane) * 4);
+          *(lds_u32*)at_out = __float_as_uint(__uint_as_float(*(const lds_u32*)at_out) + (a.x_dtype == BP_I8 ? v * xsc[tt] : v));
+        }
       }
     };
     // Two tiles are in flight per loader: the tile parked before a barrier was requested two tiles ago.
@@ -1015,7 +1025,6 @@ __global__ __launch_bounds__(CW_WAVES * 64) void k_tq1_gemv_cw(GemmArgs a, int n
       if constexpr (TPB == 1) {
         __syncthreads();
         if (t > 0) reduce(t - 1, IC<1>{});  // (multiplied before this barrier)
-        request_out(t, IC<0>{});
         if (t + 1 >= n_int) break;  // (uniform)
       }
       park(t + 1, IC<1>{});
@@ -1023,20 +1032,29 @@ __global__ __launch_bounds__(CW_WAVES * 64) void k_tq1_gemv_cw(GemmArgs a, int n
       __syncthreads();
       if constexpr (TPB == 1) {
         reduce(t, IC<0>{});
-        request_out(t + 1, IC<1>{});
       } else {
         if (t > 0) {
           reduce(t - 2, IC<0>{});
           reduce(t - 1, IC<1>{});
         }
-        request_out(t, IC<0>{});
-        request_out(t + 1, IC<1>{});
       }
     }
     __syncthreads();
     if constexpr (TPB == 2) reduce(TPB * n_int - 2, IC<0>{});
     if (TPB == 2 || (n_int & 1) == 0) reduce(TPB * n_int - 1, IC<1>{});
     else reduce(n_int - 1, IC<0>{});
+  }
+  // ---- the group's first loader writes its tiles' outputs back: the entries it has added to itself (no barrier), four
+  // tiles per wave store
+  if (loader && lidx == 0) {
+    for (int t = kb; t < n_iter; t += 4) {
+      const int64_t tile = tile_of(t);
+#pragma unroll
+      for (int tt = 0; tt < NTOK; ++tt) {
+        if (tile < tile_end && tt < ntok)
+          a.out[(tok + tt) * a.N + tile * 16 + r16] = __uint_as_float(*(const lds_u32*)(stage + (unsigned)((((int)(tile - tile0) * NTOK + tt) * 16 + r16) * 4)));
+      }
+    }
   }
 }
 
@@ -1099,9 +1117,13 @@ int launch_cw(const GemmArgs& a, hipStream_t s, int64_t nchunks, int cus, int fi
   // A group: nchunks multipliers and its loaders, which take up to 8 wave loads of packed bytes each and one of the
   // scales. As many groups as fit the 16 waves, the tiles of a workgroup and LDS (two tiles per barrier if those fit too).
   auto loaders_of = [&](int g) { return (CW_WAVES - g * nchunks) / g; };
+  // (a workgroup keeps its outputs in LDS: at most CW_STAGE_PER_THREAD per thread, 64 bytes per tile and token)
+  const int64_t per_cap = CW_STAGE_PER_THREAD * CW_WAVES * 64 / (16 * NTOK);
+  if (per > per_cap) per = per_cap;
   auto lds_of = [&](int g, int tpb) {
     const int64_t stream = (int64_t)g * 2 * tpb * (buf + nchunks * 64 * NTOK), build = nchunks * NTOK * f4_chunk_bytes(NTOK);
-    return (int64_t)CW_LUT_BYTES + (stream > build ? stream : build);
+    const int64_t mine = (per + g - 1) / g * g;  // tiles per workgroup with g groups
+    return (int64_t)CW_LUT_BYTES + (stream > build ? stream : build) + mine * 64 * NTOK;
   };
   auto fits = [&](int g, int tpb) {
     const int64_t l = loaders_of(g);
@@ -1114,6 +1136,7 @@ int launch_cw(const GemmArgs& a, hipStream_t s, int64_t nchunks, int cus, int fi
   const int tpb = fits(groups, 2) ? 2 : 1;
   const int64_t loaders = loaders_of(groups), lpw = (nl + loaders - 1) / loaders;
   per = (per + groups - 1) / groups * groups;
+  if (per > per_cap) per = per_cap / groups * groups;
   // Measured against the kernel above (E x N x K from 64 x 4096 x 2048 to 256 x 2048 x 7168): ahead by 3 - 12 % with 10 or
   // more multipliers and 48 or more tiles per group, behind with fewer of either (7 multipliers at K = 4096; 21 tiles).
   if (force != 'c' && (groups * nchunks < 10 || per / groups < 48)) return BP_ERR_UNSUPPORTED;
