@@ -257,3 +257,52 @@ def test_config4_decoder_full_size():
     assert checked[0] == 3 * cfg.layers * 3  # per forward and layer: q|k|v (one stacked linear), o, the MoE
     assert worst[0] <= 5e-3, worst[0]  # single linears, bf16 outputs: a few roundings flip on float32 summation order
     assert worst_moe[0] <= 1.25 and worst_moe[1] <= 1.5e-2, worst_moe
+
+
+def test_config4_decode_step_at_the_benchmark_batch():
+    """The decode step `bench.py` times (64 sequences, 128-token prompt): one eager step with every ternary linear
+    checked in place against dequantized dense torch evaluation on sampled rows, and the same step replayed as a HIP
+    graph against the eager logits."""
+    import deepseekternarized_amd as bp
+    from deepseekternarized_amd.decoder_harness import DecoderConfig, GraphedDecode, TernaryDecoder
+
+    cfg = DecoderConfig()
+    m = TernaryDecoder(cfg, seed=5)
+
+    def dense(packed, scale, K):
+        return bp.unpack(packed, cfg.fmt, K).float() * scale.float().repeat_interleave(cfg.group, -1)[:, :K]
+
+    def quant(x):  # boilerplate/ternary/ops.py:20-25 in torch
+        xf = x.float()
+        s = (xf.abs().amax(-1, keepdim=True) / 127.0).clamp(min=1e-8)
+        return torch.round(xf / s).clamp(-127, 127) * s
+
+    hip_linear, worst, checked, on = m.linear, [0.0], [0], [False]
+
+    def checked_linear(l, x):
+        y = hip_linear(l, x)
+        if on[0]:
+            flat, yf = x.reshape(-1, x.shape[-1])[::7], y.reshape(-1, y.shape[-1])[::7]
+            want = (quant(flat) @ dense(l.terms[0].packed, l.terms[0].scale, cfg.hidden).t()).to(y.dtype)
+            worst[0] = max(worst[0], ((yf.float() - want.float()).norm() / want.float().norm().clamp(min=1e-6)).item())
+            checked[0] += 1
+        return y
+
+    m.linear = checked_linear
+    ids = torch.randint(0, cfg.vocab, (64, 128), generator=torch.Generator().manual_seed(6))
+    logits, cache = m.forward(ids)
+    assert torch.isfinite(logits[:, -1]).all()
+    nxt = logits[:, -1].argmax(-1)
+    del logits
+    dec = GraphedDecode(m, cache, max_len=128 + 4)
+    on[0] = True
+    want, cache = m.forward(nxt[:, None].cpu(), cache)
+    on[0] = False
+    torch.cuda.synchronize()
+    assert checked[0] == 2 * cfg.layers and worst[0] <= 5e-3, (checked[0], worst[0])
+    got = dec.step(nxt).clone()
+    torch.cuda.synchronize()
+    assert torch.isfinite(got).all()
+    rel = ((got.float() - want[:, 0].float()).norm() / want[:, 0].float().norm()).item()
+    assert rel <= 2e-2, rel
+    assert (got.argmax(-1) == want[:, 0].argmax(-1)).float().mean().item() >= 0.9
