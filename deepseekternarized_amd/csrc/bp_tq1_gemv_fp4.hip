@@ -116,8 +116,10 @@ __device__ __forceinline__ void f4_build_table() {
 
 // The operand A tiles of the launch's `ntok` tokens (rows tok, tok + 1, ... of x) for chunks cb .. cb + nchunks - 1, built
 // behind the table (from LDS byte AT) by the workgroup's first `builders` waves (the caller synchronises afterwards).
-template <int NTOK, int WAVES, int AT = F4_LUT_BYTES>
-__device__ __forceinline__ void f4_build_tiles(const GemmArgs& a, int64_t tok, int ntok, int nchunks, int cb, int wave, int lane, int builders = WAVES) {
+struct F4Nothing { __device__ __forceinline__ void operator()() const {} };
+// `meanwhile` runs after the wave's first activations are requested and before they are used.
+template <int NTOK, int WAVES, int AT = F4_LUT_BYTES, typename Meanwhile = F4Nothing>
+__device__ __forceinline__ void f4_build_tiles(const GemmArgs& a, int64_t tok, int ntok, int nchunks, int cb, int wave, int lane, int builders = WAVES, Meanwhile meanwhile = Meanwhile()) {
   constexpr int PC = f4_pieces(NTOK);
   constexpr int F4_HI_OFF = F4Tile<PC>::HI_OFF, F4_ZERO_OFF = F4Tile<PC>::ZERO_OFF, F4_PRE_OFF = F4Tile<PC>::PRE_OFF;
   constexpr int F4_INV_OFF = F4Tile<PC>::INV_OFF, F4_CHUNK_BYTES = F4Tile<PC>::CHUNK_BYTES;
@@ -132,18 +134,30 @@ __device__ __forceinline__ void f4_build_tiles(const GemmArgs& a, int64_t tok, i
   const int blk = lane;
   const int tt0 = 5 * f4_pair_byte(blk >> 3, (blk >> 1) & 3, blk & 1), glo = tt0 >> 7, ghi = (tt0 + 9) >> 7;
   // (a wave with several items requests the next item's activations before it works on the current one's)
+  // The lane's 10 activations come as one 20-byte piece (16-bit) or as the three dwords around their 10 bytes (int8)
+  // through a buffer over the whole tensor: what lies past it reads as zero, what lies past the row is masked below.
+  const int esz = x16 ? 2 : 1;
+  const bool vec = a.x_dtype != BP_F32 && ((uintptr_t)a.x & 3) == 0 && a.T * a.K * esz < 0x7ffffff0 && (!x16 || (a.K & 1) == 0);
+  const __amdgpu_buffer_rsrc_t xrs = make_rsrc(a.x, whole_dwords(a.T * a.K * esz));
   u32x4 qn = {0u, 0u, 0u, 0u};
-  unsigned q4n = 0u;
-  auto request_x = [&](int item) {  // the lane's 20 bytes of a 16-bit item, if they lie inside the row
+  unsigned q4n = 0u, xsn = 0u;
+  auto request_x = [&](int item) {
     const int tt = item / nchunks, c = item - tt * nchunks;
     const int64_t k0 = 640 * (int64_t)(cb + c) + tt0;
-    if (x16 && item < ntok * nchunks && k0 + 10 <= a.K) {  // 20 bytes at an even address
-      const uint16_t* src = (const uint16_t*)a.x + (tok + tt) * a.K + k0;
-      qn = ((const F4Packed16*)src)->v;
-      q4n = ((const F4Packed4*)(src + 8))->v;
+    if (vec && item < ntok * nchunks) {
+      const unsigned bo = (unsigned)(((tok + tt) * a.K + k0) * esz);
+      if (x16) {
+        qn = buf_load16(xrs, bo, 0u);
+        q4n = (unsigned)__builtin_amdgcn_raw_buffer_load_b32(xrs, (int)(bo + 16u), 0, 0);
+      } else {
+        const u32x2 lo = f4_load8(xrs, bo & ~3u, 0u);
+        qn = u32x4{lo.x, lo.y, (unsigned)__builtin_amdgcn_raw_buffer_load_b32(xrs, (int)((bo & ~3u) + 8u), 0, 0), 0u};
+        xsn = bo & 3u;
+      }
     }
   };
   request_x(wave);
+  meanwhile();
   for (int item = wave; item < ntok * nchunks; item += builders) {  // (the waves 0 .. builders - 1 call this)
     const int tt = item / nchunks, c = item - tt * nchunks;
     const int64_t xrow = (tok + tt) * a.K;
@@ -152,13 +166,23 @@ __device__ __forceinline__ void f4_build_tiles(const GemmArgs& a, int64_t tok, i
     const int64_t k0 = 640 * (int64_t)(cb + c) + tt0;
     float y[10];
     const u32x4 q = qn;
-    const unsigned q4 = q4n;
+    const unsigned q4 = q4n, xs = xsn;
     request_x(item + builders);
-    if (x16 && k0 + 10 <= a.K) {
+    if (vec && x16) {
 #pragma unroll
       for (int i = 0; i < 4; ++i) { y[2 * i] = widen16(q[i] & 0xffffu); y[2 * i + 1] = widen16(q[i] >> 16); }
       y[8] = widen16(q4 & 0xffffu);
       y[9] = widen16(q4 >> 16);
+    } else if (vec) {
+      const unsigned d[3] = {__builtin_amdgcn_alignbyte(q.y, q.x, xs), __builtin_amdgcn_alignbyte(q.z, q.y, xs), __builtin_amdgcn_alignbyte(0u, q.z, xs)};
+#pragma unroll
+      for (int t = 0; t < 10; ++t) y[t] = (float)(int)(int8_t)((d[t >> 2] >> (8 * (t & 3))) & 0xffu);
+    }
+    if (vec) {
+      if (640 * (int64_t)(cb + c + 1) > a.K) {  // (uniform: the row's last chunk)
+#pragma unroll
+        for (int t = 0; t < 10; ++t) y[t] = k0 + t < a.K ? y[t] : 0.f;
+      }
     } else {
 #pragma unroll
       for (int t = 0; t < 10; ++t) y[t] = k0 + t < a.K ? load_act_f32(a.x, a.x_dtype, xrow + k0 + t) : 0.f;
@@ -848,19 +872,9 @@ __global__ __launch_bounds__(CW_WAVES * 64) void k_tq1_gemv_cw(GemmArgs a, int n
     }
     if (put_s) *(lds_u32x4*)(wb + ds_lane) = ring[slot][LPW];
   };
-  // A loader has few instructions per tile and everything waits for them: they go before those of the multipliers on
-  // its SIMD. The first term's first two tiles are requested before the table and the token's tile are built.
-  if (!multiplier) {
-    __builtin_amdgcn_s_setprio(3);
-    setup_term(0);
-    request(0, IC<0>{});
-    request(1, IC<1>{});
-  } else {
-    f4_build_tiles<NTOK, WAVES, AT>(a, tok, ntok, nchunks, 0, wave, lane, active);  // (chunk by chunk, by the multipliers)
-  }
-
   // ---- the byte table, one copy per lane (64 banks: no two lanes of a wave share one): entry v = digits d0..d4 of v as
   // fp4 codes in nibbles 0..4, at 256 v + 4 lane - an address that one byte permute makes from a packed byte and 4 lane
+  auto build_table = [&] {
   for (int idx = threadIdx.x; idx < 256 * 16; idx += THREADS) {
     unsigned v = (unsigned)idx >> 4, ent = 0;
     if (v < 243) {
@@ -873,6 +887,19 @@ __global__ __launch_bounds__(CW_WAVES * 64) void k_tq1_gemv_cw(GemmArgs a, int n
     }
     *(lds_u32x4*)(16 * idx) = u32x4{ent, ent, ent, ent};
   }
+  };
+  // A loader has few instructions per tile and everything waits for them: they go before those of the multipliers on
+  // its SIMD. The first term's first two tiles are requested before the table and the token's tile are built.
+  if (!multiplier) {
+    __builtin_amdgcn_s_setprio(3);
+    setup_term(0);
+    request(0, IC<0>{});
+    request(1, IC<1>{});
+    build_table();
+  } else {  // (chunk by chunk, by the multipliers; their part of the table while the activations are on their way)
+    f4_build_tiles<NTOK, WAVES, AT>(a, tok, ntok, nchunks, 0, wave, lane, active, build_table);
+  }
+
 #pragma unroll
   for (int u = 0; u < CW_STAGE_PER_THREAD; ++u) {
     const int o = (int)threadIdx.x + u * THREADS;
@@ -970,7 +997,7 @@ __global__ __launch_bounds__(CW_WAVES * 64) void k_tq1_gemv_cw(GemmArgs a, int n
           if (kb == 0) *(lds_u32*)(red + (unsigned)((((t % NB) * nchunks + c) * NTOK + tt) * 64 + 4 * r16)) = __float_as_uint(v);
         }
       };
-      __syncthreads();  // (the previous term's last tiles have been added)
+      if (term > 0) __syncthreads();  // (the previous term's last tiles have been added)
       for (int i = 0; i < n_int; ++i) {
         __syncthreads();  // (the tiles TPB i .. TPB i + TPB - 1 are in their buffers)
 #pragma unroll
@@ -988,8 +1015,7 @@ __global__ __launch_bounds__(CW_WAVES * 64) void k_tq1_gemv_cw(GemmArgs a, int n
     // The sums of the tile of iteration t, by the group's first loader: lane (row n, quarter q) adds chunks q, q + 4, ...
     // in that order, the row's four lanes are added in a fixed order too, and the row's entry of the output stage takes
     // one addition (this wave is the only one that touches its group's entries between the first barrier and the end).
-    auto reduce = [&](int t, auto slot_c) {
-      constexpr int slot = decltype(slot_c)::value;
+    auto reduce = [&](int t, auto) {
       if (!loader || lidx != 0) return;  // (uniform)
       const int64_t tile = tile_of(t);
 #pragma unroll
@@ -1014,7 +1040,7 @@ __global__ __launch_bounds__(CW_WAVES * 64) void k_tq1_gemv_cw(GemmArgs a, int n
     };
     // Two tiles are in flight per loader: the tile parked before a barrier was requested two tiles ago.
     static_assert(TPB == 1 || TPB == 2, "tiles per barrier");
-    __syncthreads();  // (the previous term's last tiles have been multiplied)
+    if (term > 0) __syncthreads();  // (the previous term's last tiles have been multiplied)
     if (term > 0) {
       request(0, IC<0>{});
       request(1, IC<1>{});
