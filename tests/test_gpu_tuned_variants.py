@@ -523,6 +523,36 @@ def test_tq2_k_split_gemv_keeps_small_activations_next_to_outliers(bp, tune):
         assert np.isfinite(got).all() and rel_l2(got, want) <= bound, (spread, rel_l2(got, want))
 
 
+def test_tq2_k_split_gemv_replays_in_a_hip_graph(bp, tune):
+    """The call captured into a HIP graph (the output's zero-fill is torch's fill kernel, the launch reads what it adds
+    to and writes once): several replays with eager launches in between, every replay against the eager result."""
+    tune("BP_TUNE_TQ2V", "k")
+    E, N, K = 4, 528, 4096
+    packed, scales = synth_weights(44, E, N, K, GROUP, "tq2", terms=2)
+    rng = np.random.default_rng(44)
+    pk, sc = [dev(p) for p in packed], [dev(s) for s in scales]
+    off = dev(np.arange(E + 1, dtype=np.int64))
+    x = dev(orc.bf16_round(rng.standard_normal((E, K)).astype(np.float32))).to(torch.bfloat16)
+    want = bp.grouped_ternary_gemm(x, None, off, pk, sc, K, GROUP, "tq2", max_rows=1).clone()
+    assert bp.ext().last_kernel() == "fp4_tq2_t1_ks"
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):
+        bp.grouped_ternary_gemm(x, None, off, pk, sc, K, GROUP, "tq2", max_rows=1)
+    torch.cuda.current_stream().wait_stream(side)
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        got = bp.grouped_ternary_gemm(x, None, off, pk, sc, K, GROUP, "tq2", max_rows=1)
+    for i in range(4):
+        got.fill_(float("nan"))
+        graph.replay()
+        torch.cuda.synchronize()
+        assert torch.equal(got, want), i
+        x2 = dev(orc.bf16_round(rng.standard_normal((E, K)).astype(np.float32))).to(torch.bfloat16)
+        bp.grouped_ternary_gemm(x2, None, off, pk, sc, K, GROUP, "tq2", max_rows=1)  # eager work between the replays
+        torch.cuda.synchronize()
+
+
 def test_tq2_k_split_gemv_counts_the_unused_code_as_unpack_does(bp, tune):
     """pack never writes the 2-bit code 3. unpack reads it as +2 (boilerplate/ternary/pack.py:47-60: code - 1) and so does
     this kernel (E2M1 1.5 = 3 / 2, minus the offset); the reference's CPU kernel adds or subtracts by the trit's sign
