@@ -751,7 +751,8 @@ __global__ __launch_bounds__(WAVES * 64, KS ? 2 : 4) void k_tq1_gemv_fp4(GemmArg
 //    reads in the loop. A group is nchunks multipliers and its loaders; groups walk over their own tiles (tile index =
 //    group mod groups);
 //  * a multiplier's 16 partial sums of a tile (one per row) go to LDS, and the group's first loader adds the chunks' sums
-//    in a fixed order and adds the result to the output (read a barrier earlier).
+//    in a fixed order and adds the result to the row's entry of the workgroup's outputs, which wait in LDS too: read
+//    from memory when the workgroup starts, written back once after the last term.
 // A barrier hands over TPB tiles: two where four tile buffers fit beside the table (the loaders' waits for memory and
 // the multipliers' work vary from tile to tile: the fewer the meeting points, the less is waited), else one with two
 // buffers. The buffers that the loaders fill were multiplied before the previous barrier. The tile buffers take the
