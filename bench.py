@@ -59,6 +59,8 @@ def arithmetic_of(kernel):
     """What the kernel named by bp_last_kernel() multiplies in (the `dtype` field of the line is the activation type)."""
     if kernel.startswith("fp4_tq1_t1"):
         return "activations as 3 E4M3 pieces under a per-group power-of-two prescale x E2M1 weights (v_mfma_f32_16x16x128_f8f6f4), fp32 accumulate, fp16 scale per 128-group applied in fp32"
+    if kernel.startswith("fp4_tq2"):
+        return "activations as 3 E4M3 pieces under a per-group power-of-two prescale (int8 activations: exact) x 2-bit codes read as E2M1 halves with the offset in the accumulator (v_mfma_f32_16x16x128_f8f6f4), fp32 accumulate, fp16 scale per 128-group applied in fp32"
     if kernel.startswith("fp4_tq1_m"):
         return "activations as 2 E4M3 pieces under a per-group power-of-two prescale x E2M1 weights (v_mfma_f32_16x16x128_f8f6f4), fp32 accumulate"
     if kernel.startswith("gemm_tq1f"):
