@@ -769,7 +769,7 @@ constexpr int cw_pitch(int64_t Kp) {
   return 16 * (pieces | 1);
 }
 constexpr int cw_colblks(int64_t Kp) { return (int)((Kp + 3 + 255) / 256); }  // wave loads of 4 rows x 256 bytes per 4 rows
-constexpr int64_t cw_buffer_bytes(int64_t Kp, int64_t G) { return 16 * (int64_t)cw_pitch(Kp) + 16 * G * 2; }
+constexpr int64_t cw_buffer_bytes(int64_t Kp, int64_t G, int64_t scale_bytes) { return 16 * (int64_t)cw_pitch(Kp) + 16 * G * scale_bytes; }
 
 // LPW: wave loads of packed bytes per loader and tile; TPB: tiles per barrier. NTOK = 2: a pair of token rows per expert
 // (rows first_row, first_row + 1), as in the kernel above: two fp8 pieces per activation, one matrix instruction serves
@@ -777,9 +777,8 @@ constexpr int64_t cw_buffer_bytes(int64_t Kp, int64_t G) { return 16 * (int64_t)
 // and a multiplier's registers hold the pair's chunk (the same 8 x 8 registers).
 template <int SDT, int LPW, int TPB, int NTOK = 1>
 __global__ __launch_bounds__(CW_WAVES * 64) void k_tq1_gemv_cw(GemmArgs a, int nchunks, int groups, int tiles_per_wg, int first_row) {
-  static_assert(SDT == BP_F16 || SDT == BP_BF16, "2-byte scales");
   static_assert(NTOK == 1 || NTOK == 2, "one token row per expert, or a pair");
-  constexpr int WAVES = CW_WAVES, THREADS = WAVES * 64, NB = 2 * TPB, PC = f4_pieces(NTOK), SB = 2;
+  constexpr int WAVES = CW_WAVES, THREADS = WAVES * 64, NB = 2 * TPB, PC = f4_pieces(NTOK), SB = SDT == BP_F32 ? 4 : 2;
   constexpr int F4_INV_OFF = F4Tile<PC>::INV_OFF, F4_CHUNK_BYTES = F4Tile<PC>::CHUNK_BYTES, AT = CW_LUT_BYTES;
   const int wave = __builtin_amdgcn_readfirstlane((int)(threadIdx.x >> 6)), lane = threadIdx.x & 63;
   const int r16 = lane & 15, kb = lane >> 4;
@@ -950,7 +949,8 @@ __global__ __launch_bounds__(CW_WAVES * 64) void k_tq1_gemv_cw(GemmArgs a, int n
         const unsigned rb = gbase + (unsigned)((t % NB) * buf_bytes);
         const u32x4 W0 = *(const lds_u32x4*)(rb + rd_w), W1 = *(const lds_u32x4*)(rb + rd_w + 64);
         const unsigned x0 = *(const lds_u32*)(rb + rd_w + 16), x1 = *(const lds_u32*)(rb + rd_w + 80);
-        const unsigned ra = *(const lds_u16*)(rb + rd_sa), rbits = *(const lds_u16*)(rb + rd_sb);
+        const unsigned ra = SB == 4 ? *(const lds_u32*)(rb + rd_sa) : (unsigned)*(const lds_u16*)(rb + rd_sa);
+        const unsigned rbits = SB == 4 ? *(const lds_u32*)(rb + rd_sb) : (unsigned)*(const lds_u16*)(rb + rd_sb);
         // the table reads run BD instructions ahead of the matrix instructions (the scheduling barriers keep the compiler
         // from sinking them back to their uses: a wave would wait out an LDS round trip per instruction)
         constexpr int BD = 2;
@@ -979,8 +979,8 @@ __global__ __launch_bounds__(CW_WAVES * 64) void k_tq1_gemv_cw(GemmArgs a, int n
         };
         stage(IC<0>{}); stage(IC<1>{}); stage(IC<2>{}); stage(IC<3>{}); stage(IC<4>{}); stage(IC<5>{}); stage(IC<6>{}); stage(IC<7>{});
         __builtin_amdgcn_sched_barrier(0);
-        const float sa = SDT == BP_F16 ? f16_bits_to_f32((uint16_t)ra) : __uint_as_float(ra << 16);
-        const float sb = SDT == BP_F16 ? f16_bits_to_f32((uint16_t)rbits) : __uint_as_float(rbits << 16);
+        const float sa = SDT == BP_F32 ? __uint_as_float(ra) : SDT == BP_F16 ? f16_bits_to_f32((uint16_t)ra) : __uint_as_float(ra << 16);
+        const float sb = SDT == BP_F32 ? __uint_as_float(rbits) : SDT == BP_F16 ? f16_bits_to_f32((uint16_t)rbits) : __uint_as_float(rbits << 16);
         // the row's sum over its four lanes (one per quarter): row n ends up in every lane n + 16 q
 #pragma unroll
         for (int tt = 0; tt < NTOK; ++tt) {
@@ -1133,14 +1133,15 @@ int launch_cw(const GemmArgs& a, hipStream_t s, int64_t nchunks, int cus, int fi
   if (force == 'r') return BP_ERR_UNSUPPORTED;
   for (int t = 0; t < a.n_terms; ++t)
     if (((uintptr_t)a.w_scale[t] & 3) != 0) return BP_ERR_UNSUPPORTED;
-  if (a.N * a.Kp >= 0x7fffffe0 || a.N * a.G * 2 >= 0x7fffffe0) return BP_ERR_UNSUPPORTED;
+  constexpr int64_t SB = SDT == BP_F32 ? 4 : 2;
+  if (a.N * a.Kp >= 0x7fffffe0 || a.N * a.G * SB >= 0x7fffffe0) return BP_ERR_UNSUPPORTED;
   const int64_t experts = a.E < a.T ? a.E : a.T, tiles = a.N / 16;
   if (force != 'c' && experts * tiles < 16 * (int64_t)cus) return BP_ERR_UNSUPPORTED;
   int64_t wpe = cus / experts;  // workgroups per expert: one workgroup per CU is resident
   wpe = wpe < 1 ? 1 : wpe > tiles ? tiles : wpe;
   int64_t per = (tiles + wpe - 1) / wpe;  // tiles per workgroup
-  const int64_t buf = cw_buffer_bytes(a.Kp, a.G);
-  const int64_t nl = 4 * cw_colblks(a.Kp), ns = (16 * a.G * 2 + 1023) / 1024;  // wave loads per tile: packed bytes, scales
+  const int64_t buf = cw_buffer_bytes(a.Kp, a.G, SB);
+  const int64_t nl = 4 * cw_colblks(a.Kp), ns = (16 * a.G * SB + 1023) / 1024;  // wave loads per tile: packed bytes, scales
   // A group: nchunks multipliers and its loaders, which take up to 8 wave loads of packed bytes each and one of the
   // scales. As many groups as fit the 16 waves, the tiles of a workgroup and LDS (two tiles per barrier if those fit too).
   auto loaders_of = [&](int g) { return (CW_WAVES - g * nchunks) / g; };
@@ -1200,7 +1201,7 @@ int launch_f4(const GemmArgs& a, hipStream_t s, int first_row = 0) {
   // 2-byte scales go by the round through LDS where the slots fit behind the tiles and a row's scales start dword-aligned
   constexpr int SRV = SDT != BP_F32 && NTOK <= 4 ? 1 : 0;
   const bool sr_ok = SRV && (a.G * 2) % 4 == 0;
-  if constexpr (NTOK == 2 && SDT != BP_F32) {  // (a pair of rows per expert in a large call: the rows through LDS tile by tile)
+  if constexpr (NTOK == 2) {  // (a pair of rows per expert in a large call: the rows through LDS tile by tile)
     if (nseg == 1) {
       const int rc = launch_cw<SDT, 2>(a, s, nchunks, cus, first_row);
       if (rc != BP_ERR_UNSUPPORTED) return rc;
@@ -1217,7 +1218,7 @@ int launch_f4(const GemmArgs& a, hipStream_t s, int first_row = 0) {
     if (sr_ok && lds + 16 * F4_SCALE_SLOT <= (size_t)F4_LDS_MAX) return launch_f4_k<SDT, 16, 0, NTOK, SRV>(a, s, name16, (int)nchunks, lds, (int)seg, first_row);
     return launch_f4_k<SDT, 16, 0, NTOK>(a, s, name16, (int)nchunks, lds, (int)seg, first_row);
   }
-  if constexpr (SDT != BP_F32) {
+  {
     const int rc = launch_cw<SDT, 1>(a, s, nchunks, cus, 0);
     if (rc != BP_ERR_UNSUPPORTED) return rc;
   }

@@ -94,7 +94,7 @@ __device__ __forceinline__ void kv_widen_run(const GemmArgs& a, const KvRun& r, 
 
 template <int SDT>
 __global__ __launch_bounds__(1024) void k_tq2_gemv_ks(GemmArgs a, int nw, int tiles_per_wg) {
-  static_assert(SDT == BP_F16 || SDT == BP_BF16, "2-byte scales");
+  constexpr int SB = SDT == BP_F32 ? 4 : 2, NSL = SB / 2;  // bytes per scale; a wave's 16-byte loads of a round's scales
   const int wave = __builtin_amdgcn_readfirstlane((int)(threadIdx.x >> 6)), lane = threadIdx.x & 63;
   const int n = lane & 15, kb = lane >> 4;
   const int64_t e = blockIdx.y;
@@ -108,14 +108,13 @@ __global__ __launch_bounds__(1024) void k_tq2_gemv_ks(GemmArgs a, int nw, int ti
   const int nrounds = (int)((tile_end - tile0 + KV_R - 1) / KV_R);
 
   // ---- LDS: two slots of a round's scales, then two of a round's partial sums [tile][wave][row]
-  const unsigned row_sb = (unsigned)(a.G * 2), tile_sb = 16 * row_sb, slot_bytes = KV_R * tile_sb;
+  const unsigned row_sb = (unsigned)(a.G * SB), tile_sb = 16 * row_sb, slot_bytes = KV_R * tile_sb;
   const unsigned RED = 2 * slot_bytes;  // [tile of the workgroup][wave][row]
   const int64_t g128 = 2 * KV_S * (int64_t)wave + kb;  // the lane's group of 128 as a column of the result
   const bool g_real = 128 * g128 < a.K;
-  const unsigned rd_s = (unsigned)n * row_sb + 2u * (unsigned)(g_real ? g128 >> gs : 0);
+  const unsigned rd_s = (unsigned)n * row_sb + (unsigned)SB * (unsigned)(g_real ? g128 >> gs : 0);
   const unsigned w_lane = (unsigned)n * (unsigned)a.Kp + 16u * (unsigned)kb + 64u * KV_S * (unsigned)wave;
-  const unsigned s_off = 16u * (unsigned)(64 * wave + lane);
-  const unsigned s_lane = s_off < slot_bytes ? s_off : KV_PAST;
+  const unsigned s_off = 16u * (unsigned)(64 * wave + lane), s_step = 1024u * (unsigned)nw;  // (load j of a wave: + j s_step)
 
   // The lane as a row of operand A: piece p of the wave's group gl (p = 3: unused); its 2 x 16 activations are requested
   // first, the first tiles next, and operand A is built while those are on their way.
@@ -136,8 +135,8 @@ __global__ __launch_bounds__(1024) void k_tq2_gemv_ks(GemmArgs a, int nw, int ti
 
   // (the expert's rows and scales of a term as buffers of their own: what lies past them reads as zeros)
   __amdgpu_buffer_rsrc_t wrs = make_rsrc(a.packed[0] + e * a.N * a.Kp, a.N * a.Kp);
-  __amdgpu_buffer_rsrc_t srs = make_rsrc((const unsigned char*)a.w_scale[0] + e * a.N * a.G * 2, a.N * a.G * 2);
-  u32x4 ring[KV_D][KV_S], sc_next;
+  __amdgpu_buffer_rsrc_t srs = make_rsrc((const unsigned char*)a.w_scale[0] + e * a.N * a.G * SB, a.N * a.G * SB);
+  u32x4 ring[KV_D][KV_S], sc_next[NSL];
   auto request = [&](int t, auto slot_c) {  // the wave's bytes of the workgroup's tile t
     constexpr int slot = decltype(slot_c)::value;
     const int64_t tile = tile0 + t;
@@ -145,16 +144,20 @@ __global__ __launch_bounds__(1024) void k_tq2_gemv_ks(GemmArgs a, int nw, int ti
 #pragma unroll
     for (int s = 0; s < KV_S; ++s) ring[slot][s] = buf_load16(wrs, w_lane, so + (tile < tile_end ? 64u * s : 0u));
   };
-  auto request_scales = [&](int r) {  // the wave's 1024 bytes of round r's scales
+  auto request_scales = [&](int r) {  // the wave's 1024-byte pieces of round r's scales
     const int64_t tile = tile0 + (int64_t)KV_R * r;
-    return buf_load16(srs, s_lane, r < nrounds ? (unsigned)tile * tile_sb : KV_PAST);
+#pragma unroll
+    for (int j = 0; j < NSL; ++j) sc_next[j] = buf_load16(srs, s_off + j * s_step < slot_bytes ? s_off + j * s_step : KV_PAST, r < nrounds ? (unsigned)tile * tile_sb : KV_PAST);
   };
-  auto park_scales = [&](int r, const u32x4& v) {
-    if (s_off < slot_bytes) *(lds_u32x4*)((unsigned)(r & 1) * slot_bytes + s_off) = v;
+  auto park_scales = [&](int r) {
+#pragma unroll
+    for (int j = 0; j < NSL; ++j)
+      if (s_off + j * s_step < slot_bytes) *(lds_u32x4*)((unsigned)(r & 1) * slot_bytes + s_off + j * s_step) = sc_next[j];
   };
   auto multiply = [&](int r, auto i_c) {  // tile i of round r: multiply, request the tile KV_D further on, scale, park the sums
     constexpr int i = decltype(i_c)::value, slot = i % KV_D;
-    const unsigned raw = *(const lds_u16*)((unsigned)(r & 1) * slot_bytes + (unsigned)i * tile_sb + rd_s);
+    const unsigned sat = (unsigned)(r & 1) * slot_bytes + (unsigned)i * tile_sb + rd_s;
+    const unsigned raw = SB == 4 ? *(const lds_u32*)sat : (unsigned)*(const lds_u16*)sat;
     f32x4 C = {cinit[0], cinit[1], cinit[2], 0.f};
 #pragma unroll
     for (int s = 0; s < KV_S; ++s) {
@@ -167,14 +170,14 @@ __global__ __launch_bounds__(1024) void k_tq2_gemv_ks(GemmArgs a, int nw, int ti
       }
     }
     request(KV_R * r + i + KV_D, IC<slot>{});
-    const float sc = SDT == BP_F16 ? f16_bits_to_f32((uint16_t)raw) : __uint_as_float(raw << 16);
+    const float sc = SDT == BP_F32 ? __uint_as_float(raw) : SDT == BP_F16 ? f16_bits_to_f32((uint16_t)raw) : __uint_as_float(raw << 16);
     float v = g_real ? sc * inv2 * (C[0] + C[1] + C[2] * (1.f / 256.f)) : 0.f;
     v = kv_quad_sum(v);
     if (kb == 0) *(lds_u32*)(RED + (unsigned)(((KV_R * r + i) * nw + wave) * 64 + 4 * n)) = __float_as_uint(v);
   };
 
   auto first_requests = [&] {  // a term's first loads: the scales of round 0, the ring's tiles
-    sc_next = request_scales(0);
+    request_scales(0);
     request(0, IC<0>{});
     request(1, IC<1>{});
     request(2, IC<2>{});
@@ -253,17 +256,17 @@ __global__ __launch_bounds__(1024) void k_tq2_gemv_ks(GemmArgs a, int nw, int ti
   for (int term = 0; term < a.n_terms; ++term) {
     if (term > 0) {
       wrs = make_rsrc(a.packed[term] + e * a.N * a.Kp, a.N * a.Kp);
-      srs = make_rsrc((const unsigned char*)a.w_scale[term] + e * a.N * a.G * 2, a.N * a.G * 2);
+      srs = make_rsrc((const unsigned char*)a.w_scale[term] + e * a.N * a.G * SB, a.N * a.G * SB);
       first_requests();
     }
-    park_scales(0, sc_next);
+    park_scales(0);
     for (int r = 0; r < nrounds; ++r) {
       __syncthreads();  // (round r's scales are parked, round r - 1 is multiplied)
-      sc_next = request_scales(r + 1);
+      request_scales(r + 1);
       multiply(r, IC<0>{}); multiply(r, IC<1>{}); multiply(r, IC<2>{}); multiply(r, IC<3>{});
       multiply(r, IC<4>{}); multiply(r, IC<5>{}); multiply(r, IC<6>{}); multiply(r, IC<7>{});
       // (requested at the round's start, older than the loads of the ring: no wait; the slot was read a round ago)
-      park_scales(r + 1, sc_next);
+      park_scales(r + 1);
     }
     __syncthreads();
     // the term's sums: thread o adds the waves' partial sums of output o in wave order
@@ -315,15 +318,16 @@ int launch_tq2_gemv_fp4(const GemmArgs& a, hipStream_t s) {
   if (force == 'n') return BP_ERR_UNSUPPORTED;
   if (a.fmt != BP_TQ2 || a.max_rows != 1 || a.tiles) return BP_ERR_UNSUPPORTED;
   if (a.x_dtype != BP_BF16 && a.x_dtype != BP_I8) return BP_ERR_UNSUPPORTED;
-  if (a.scale_dtype != BP_F16 && a.scale_dtype != BP_BF16) return BP_ERR_UNSUPPORTED;
+  if (a.scale_dtype != BP_F16 && a.scale_dtype != BP_BF16 && a.scale_dtype != BP_F32) return BP_ERR_UNSUPPORTED;
+  const int64_t sb = a.scale_dtype == BP_F32 ? 4 : 2;
   if (a.K % 256 != 0 || a.N % 16 != 0 || (a.group != 128 && a.group != 256) || a.G != a.K / a.group || a.Kp != a.K / 4) return BP_ERR_UNSUPPORTED;
   const int64_t nsteps = a.K / 256, nw = (nsteps + KV_S - 1) / KV_S;
   if (nw < 2 || nw > 16) return BP_ERR_UNSUPPORTED;
-  if (a.N * a.Kp >= 0x7fffffe0 - 64 * KV_S * 16 || a.N * a.G * 2 >= 0x7fffffe0 || a.N * 4 >= 0x7fffffe0) return BP_ERR_UNSUPPORTED;
+  if (a.N * a.Kp >= 0x7fffffe0 - 64 * KV_S * 16 || a.N * a.G * sb >= 0x7fffffe0 || a.N * 4 >= 0x7fffffe0) return BP_ERR_UNSUPPORTED;
   if (((uintptr_t)a.x & 15) != 0) return BP_ERR_UNSUPPORTED;
   for (int t = 0; t < a.n_terms; ++t)
     if (((uintptr_t)a.packed[t] & 15) != 0 || ((uintptr_t)a.w_scale[t] & 15) != 0) return BP_ERR_UNSUPPORTED;
-  const int64_t slots = 2 * KV_R * 16 * a.G * 2;  // LDS: the scales of two rounds, then 64 bytes per tile and wave
+  const int64_t slots = 2 * KV_R * 16 * a.G * sb;  // LDS: the scales of two rounds, then 64 bytes per tile and wave
   const int cus = kv_cus();
   const int64_t per_cu = 16 / nw;  // workgroups that a CU holds: 16 waves of up to 128 registers
   const int64_t resident = (int64_t)cus * per_cu;
@@ -338,6 +342,8 @@ int launch_tq2_gemv_fp4(const GemmArgs& a, hipStream_t s) {
   // Measured against k_mfma_tq2 (N x K from 2048 x 1024 to 7168 x 2048 and 512 x 8192, 1 to 256 experts): ahead or
   // level from two row tiles per CU on with bf16 activations (K = 7168: 1.10 x at 128 experts; K = 4096: 1.33 x at 64;
   // K = 2048: 1.28 x at 128), with int8 ones from 16 tiles per CU (below, 14.2 against 15.7 us); behind at K = 1024.
+  // (int8 activations with float32 scales: 105 against 101.7 us for k_mfma_tq2 on the 128 x 2048 x 7168 launch)
+  if (force != 'k' && a.x_dtype == BP_I8 && a.scale_dtype == BP_F32) return BP_ERR_UNSUPPORTED;
   if (force != 'k' && (a.K < 2048 || experts * tiles < (a.x_dtype == BP_I8 ? 16 : 2) * (int64_t)cus)) return BP_ERR_UNSUPPORTED;
   // (a thread owns up to KV_OPT outputs; the partial sums of a workgroup's tiles stay in LDS until the term's end)
   const int64_t lds_cap = 160 * 1024 / per_cu;
@@ -348,6 +354,7 @@ int launch_tq2_gemv_fp4(const GemmArgs& a, hipStream_t s) {
   const size_t lds = (size_t)(slots + per * nw * 64);
   const dim3 grid((unsigned)((tiles + per - 1) / per), (unsigned)a.E, 1u);
   if (a.E > 65535) return BP_ERR_UNSUPPORTED;
+  if (a.scale_dtype == BP_F32) return launch_kv<BP_F32>(a, s, (int)nw, per, grid, lds);
   return a.scale_dtype == BP_F16 ? launch_kv<BP_F16>(a, s, (int)nw, per, grid, lds) : launch_kv<BP_BF16>(a, s, (int)nw, per, grid, lds);
 }
 

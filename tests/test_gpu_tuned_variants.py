@@ -165,8 +165,9 @@ def test_tq1_gemv_chunk_per_wave(bp, tune, K, counts, act, N):
 
 
 def test_tq1_gemv_chunk_per_wave_terms_scales_groups(bp, tune):
-    """Two stacked terms with bf16 scales (the second term adds to the first one's output), scale groups of 256, and
-    the calls it leaves to the other kernels: float32 scales, scales that are not dword-aligned, 16 chunks or more."""
+    """Two stacked terms with bf16 scales (the second term adds to the first one's output), scale groups of 256, float32
+    scales (what the reference's wrappers pass: boilerplate/kernels/ternary_cuda.py:95-97), and the calls it leaves to
+    the other kernels: 15 chunks or more."""
     tune("BP_TUNE_TQ1", "chunk")
     got, want, kern = _run(bp, "tq1", 2, 2048 + 48, 2304, [1, 1], "bf16", terms=2, seed=5, scale_dtype=np.float32)
     assert kern == "fp4_tq1_t1_cw", kern
@@ -175,7 +176,13 @@ def test_tq1_gemv_chunk_per_wave_terms_scales_groups(bp, tune):
     assert kern == "fp4_tq1_t1_cw", kern
     _check(got, want)
     got, want, kern = _run(bp, "tq1", 2, 64, 2048, [1, 1], "bf16", seed=10, scale_dtype="f32")
-    assert kern.startswith("fp4_tq1_t1_w"), kern
+    assert kern == "fp4_tq1_t1_cw", kern
+    _check(got, want)
+    got, want, kern = _run(bp, "tq1", 3, 2048 + 16, 7168, [1, 0, 1], "int8", terms=2, seed=11, scale_dtype="f32")  # four wave loads of scales per tile
+    assert kern == "fp4_tq1_t1_cw", kern
+    _check(got, want)
+    got, want, kern = _run(bp, "tq1", 2, 272, 4608, [2, 1], "bf16", seed=14, scale_dtype="f32", group=256)  # a pair of rows
+    assert kern == "fp4_tq1_m2_cw", kern
     _check(got, want)
     got, want, kern = _run(bp, "tq1", 1, 272, 10240, [1], "bf16", seed=12)  # 16 chunks: no wave left for the loads
     assert kern.startswith("fp4_tq1_t1_w"), kern
@@ -445,6 +452,8 @@ def test_tq1_mfma_scales_from_global_memory(bp, tune):
     (3, 1040, 4096, 256, 2, np.float16),    # a scale per 256 weights, stacked terms, 65 tiles (a last round of one tile)
     (2, 2064, 7168, 128, 1, np.float16),    # the headline K: 14 waves
     (1, 272, 8192, 128, 1, "bf16"),         # 16 waves
+    (3, 528, 7168, 128, 2, "f32"),          # float32 scales (what the reference's wrappers pass): two 16-byte loads per wave and round
+    (2, 272, 2304, 256, 1, "f32"),
     (5, 48, 768, 128, 1, np.float16),       # below the kernel's K: the other kernels
 ])
 def test_tq2_single_token_gemv_with_k_split_over_the_waves(bp, tune, act, E, N, K, group, terms, sdt):
