@@ -16,7 +16,7 @@ from pathlib import Path
 HERE = Path(__file__).resolve().parent
 CSRC = HERE / "csrc"
 LIB = HERE / "libbp_ternary_hip.so"
-SOURCES = ["bp_api.hip", "bp_general.hip", "bp_route.hip", "bp_gguf.hip", "bp_huffman.hip", "bp_moe.hip", "bp_mfma.hip", "bp_mfma_tq2.hip", "bp_gemm_tq2.hip", "bp_gemm_tq2f.hip", "bp_mfma_tq1.hip", "bp_gemm_tq1.hip", "bp_tq1_gemv.hip", "bp_tq1_gemv_fp4.hip", "bp_tq2_gemv_fp4.hip"]
+SOURCES = ["bp_api.hip", "bp_general.hip", "bp_route.hip", "bp_gguf.hip", "bp_huffman.hip", "bp_moe.hip", "bp_mfma.hip", "bp_mfma_tq2.hip", "bp_gemm_tq2.hip", "bp_gemm_tq2f.hip", "bp_mfma_tq1.hip", "bp_gemm_tq1.hip", "bp_tq1_gemv.hip", "bp_tq1_gemv_fp4.hip", "bp_tq1_gemv_cw.hip", "bp_tq2_gemv_fp4.hip"]
 # packed FP32 VALU ops are disabled for every device object of this library
 FLAGS = ["--offload-arch=gfx950", "-O3", "-fPIC", "-std=c++17", "-Wall", "-Wno-unused-function", "-Wno-int-to-pointer-cast",
          "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops"]
@@ -25,7 +25,7 @@ FLAGS = ["--offload-arch=gfx950", "-O3", "-fPIC", "-std=c++17", "-Wall", "-Wno-u
 # These kernels address LDS absolutely (their dynamic allocation must start at LDS address 0): a kernel of theirs
 # with static LDS - e.g. a register array the compiler moved there because it was indexed dynamically - would
 # compute on the wrong bytes, so the build refuses it.
-NO_STATIC_LDS = {"bp_mfma_tq2.hip", "bp_gemm_tq2.hip", "bp_gemm_tq2f.hip", "bp_mfma_tq1.hip", "bp_gemm_tq1.hip", "bp_gemm_tq1.hip", "bp_tq1_gemv.hip", "bp_tq1_gemv_fp4.hip", "bp_tq2_gemv_fp4.hip"}
+NO_STATIC_LDS = {"bp_mfma_tq2.hip", "bp_gemm_tq2.hip", "bp_gemm_tq2f.hip", "bp_mfma_tq1.hip", "bp_gemm_tq1.hip", "bp_gemm_tq1.hip", "bp_tq1_gemv.hip", "bp_tq1_gemv_fp4.hip", "bp_tq1_gemv_cw.hip", "bp_tq2_gemv_fp4.hip"}
 _REMARK = "[-Rpass-analysis=kernel-resource-usage]"
 
 

@@ -48,237 +48,10 @@
 // Operand layout of the instruction with A = fp8 (8 VGPRs), B = fp4 (4 VGPRs), established by one-hot probing
 // on gfx950: B lane (n = lane % 16, kb = lane / 16), VGPR w, nibble q is paired with A lane (m = lane % 16,
 // kbA = 2 (kb % 2) + w / 2), VGPR 4 (kb / 2) + 2 (w % 2) + q / 4, byte q % 4; C lane (n, lg) holds rows 4 lg + i.
-#include <type_traits>
-
-#include "bp_mfma.h"
+#include "bp_tq1_fp4.h"
 
 namespace bp {
 namespace {
-
-typedef int i32x8 __attribute__((ext_vector_type(8)));
-template <int V>
-using IC = std::integral_constant<int, V>;
-struct __attribute__((packed, aligned(2))) F4Packed16 { u32x4 v; };
-struct __attribute__((packed, aligned(2))) F4Packed4 { unsigned v; };
-
-constexpr int F4_LUT_BYTES = 256 * 128;          // byte -> 5 fp4 codes, one copy per bank
-// Operand A tile, per chunk: 64 byte pairs x PC pieces x 16 bytes, then 4 group boundaries x PC pieces x 16 bytes, a
-// block of zeros, 8 words = the prescales of the chunk's 5 groups (3 unused), 8 floats = their inverses (the unused
-// ones are 0): 3344 bytes with 3 pieces, 2256 with 2.
-constexpr int f4_pieces(int ntok) { return ntok == 1 ? 3 : 2; }
-constexpr int f4_chunk_bytes(int ntok) { return (64 + 4) * f4_pieces(ntok) * 16 + 16 + 32 + 32; }
-constexpr int F4_LDS_MAX = 160 * 1024;
-// Measured on E = 128, N = 2048, K = 7168: one 16-row tile per wave with 4 chunks in flight reads 504 MB from memory
-// per launch, two tiles with 2 chunks each 638 MB (405 MB are packed bytes and scales). Rows of 1434 bytes share
-// 128-byte lines between consecutive chunks; the sooner a wave returns to a row, the more of those lines it still
-// finds in the L2.
-constexpr int F4_SCALE_SLOT = 16 * 80;           // (SR) per wave: 16 rows x 80 bytes (48 of them a round's scales)
-constexpr int F4_GR = 1;                         // 16-row tiles per wave (more than one share the reads of operand A)
-constexpr int F4_RD = 4;                         // chunks of packed bytes in registers per tile (the ring of loads in flight)
-constexpr int F4_BD = 1;                         // table reads run this many (instruction, tile) pairs ahead of the matrix instructions
-constexpr int F4_PAIRS = 1;                      // 1: chunks are refilled two at a time (RD even)
-constexpr int F4_AD = 0;                         // 1: operand A is read one instruction ahead into a second set of registers
-
-__device__ __forceinline__ u32x2 f4_load8(__amdgpu_buffer_rsrc_t r, unsigned lane_off, unsigned wave_off) {
-  return __builtin_bit_cast(u32x2, __builtin_amdgcn_raw_buffer_load_b64(r, (int)lane_off, (int)wave_off, 0));
-}
-
-// first packed byte (of the chunk's 128) of the byte pair behind half `hf` of A lane quarter `kbA` in instruction j
-__device__ __forceinline__ int f4_pair_byte(int j, int kbA, int hf) {
-  return 64 * (j >> 2) + 16 * (2 * hf + (kbA >> 1)) + 4 * (j & 3) + 2 * (kbA & 1);
-}
-
-// Layout of one chunk of an operand A tile for PC pieces per activation (byte offsets within the chunk's part).
-template <int PC>
-struct F4Tile {
-  static constexpr int HI_OFF = 64 * PC * 16, ZERO_OFF = HI_OFF + 4 * PC * 16, PRE_OFF = ZERO_OFF + 16;
-  static constexpr int INV_OFF = PRE_OFF + 32, CHUNK_BYTES = (64 + 4) * PC * 16 + 16 + 32 + 32;
-};
-
-// ---- the byte table: entry v = digits d0..d4 of v as fp4 codes (-1 -> 0xA, 0 -> 0, +1 -> 0x2) in nibbles 0..4, one
-// copy per LDS bank: four threads per entry, eight copies each.
-template <int THREADS>
-__device__ __forceinline__ void f4_build_table() {
-  for (int idx = threadIdx.x; idx < 256 * 4; idx += THREADS) {
-    unsigned v = (unsigned)idx >> 2, ent = 0;
-    if (v < 243) {
-#pragma unroll
-      for (int d = 0; d < 5; ++d) {
-        const unsigned q = v / 3, dig = v - 3 * q;
-        ent |= (dig == 0 ? 0xAu : dig == 2 ? 0x2u : 0u) << (4 * d);
-        v = q;
-      }
-    }
-#pragma unroll
-    for (int cpy = 0; cpy < 8; ++cpy) *(lds_u32*)(128 * (idx >> 2) + 4 * (8 * (idx & 3) + cpy)) = ent;
-  }
-}
-
-// The operand A tiles of the launch's `ntok` tokens (rows tok, tok + 1, ... of x) for chunks cb .. cb + nchunks - 1, built
-// behind the table (from LDS byte AT) by the workgroup's first `builders` waves (the caller synchronises afterwards).
-struct F4Nothing { __device__ __forceinline__ void operator()() const {} };
-// `meanwhile` runs after the wave's first activations are requested and before they are used.
-template <int NTOK, int WAVES, int AT = F4_LUT_BYTES, typename Meanwhile = F4Nothing>
-__device__ __forceinline__ void f4_build_tiles(const GemmArgs& a, int64_t tok, int ntok, int nchunks, int cb, int wave, int lane, int builders = WAVES, Meanwhile meanwhile = Meanwhile()) {
-  constexpr int PC = f4_pieces(NTOK);
-  constexpr int F4_HI_OFF = F4Tile<PC>::HI_OFF, F4_ZERO_OFF = F4Tile<PC>::ZERO_OFF, F4_PRE_OFF = F4Tile<PC>::PRE_OFF;
-  constexpr int F4_INV_OFF = F4Tile<PC>::INV_OFF, F4_CHUNK_BYTES = F4Tile<PC>::CHUNK_BYTES;
-  auto tile_at = [](int tt, int c) { return AT + (c * NTOK + tt) * F4_CHUNK_BYTES; };
-  const bool x16 = a.x_dtype == BP_BF16 || a.x_dtype == BP_F16;
-  auto widen16 = [&](unsigned h) { return a.x_dtype == BP_BF16 ? bf16_bits_to_f32((uint16_t)h) : f16_bits_to_f32((uint16_t)h); };
-  // ---- operand A tiles: a wave builds whole chunks by itself (64 byte pairs = 64 lanes; a chunk holds 5 whole scale
-  // groups), so the activations are read from memory once and nothing waits for another wave until the tiles are
-  // complete. Lane = byte pair: its 10 activations -> the largest magnitude of each of its (one or two) groups by an LDS
-  // maximum over the float bits -> the groups' prescales 2^sh (sh brings the group's largest magnitude into [128, 256))
-  // and their inverses -> 3 pieces x (first-group block, second-group block).
-  const int blk = lane;
-  const int tt0 = 5 * f4_pair_byte(blk >> 3, (blk >> 1) & 3, blk & 1), glo = tt0 >> 7, ghi = (tt0 + 9) >> 7;
-  // (a wave with several items requests the next item's activations before it works on the current one's)
-  // The lane's 10 activations come as one 20-byte piece (16-bit) or as the three dwords around their 10 bytes (int8)
-  // through a buffer over the whole tensor: what lies past it reads as zero, what lies past the row is masked below.
-  const int esz = x16 ? 2 : 1;
-  const bool vec = a.x_dtype != BP_F32 && ((uintptr_t)a.x & 3) == 0 && a.T * a.K * esz < 0x7ffffff0 && (!x16 || (a.K & 1) == 0);
-  const __amdgpu_buffer_rsrc_t xrs = make_rsrc(a.x, whole_dwords(a.T * a.K * esz));
-  u32x4 qn = {0u, 0u, 0u, 0u};
-  unsigned q4n = 0u, xsn = 0u;
-  auto request_x = [&](int item) {
-    const int tt = item / nchunks, c = item - tt * nchunks;
-    const int64_t k0 = 640 * (int64_t)(cb + c) + tt0;
-    if (vec && item < ntok * nchunks) {
-      const unsigned bo = (unsigned)(((tok + tt) * a.K + k0) * esz);
-      if (x16) {
-        qn = buf_load16(xrs, bo, 0u);
-        q4n = (unsigned)__builtin_amdgcn_raw_buffer_load_b32(xrs, (int)(bo + 16u), 0, 0);
-      } else {
-        const u32x2 lo = f4_load8(xrs, bo & ~3u, 0u);
-        qn = u32x4{lo.x, lo.y, (unsigned)__builtin_amdgcn_raw_buffer_load_b32(xrs, (int)((bo & ~3u) + 8u), 0, 0), 0u};
-        xsn = bo & 3u;
-      }
-    }
-  };
-  request_x(wave);
-  meanwhile();
-  for (int item = wave; item < ntok * nchunks; item += builders) {  // (the waves 0 .. builders - 1 call this)
-    const int tt = item / nchunks, c = item - tt * nchunks;
-    const int64_t xrow = (tok + tt) * a.K;
-    const unsigned dst = (unsigned)tile_at(tt, c);
-    if (lane < 8) *(lds_u32*)(dst + F4_PRE_OFF + 4 * lane) = 0u;
-    const int64_t k0 = 640 * (int64_t)(cb + c) + tt0;
-    float y[10];
-    const u32x4 q = qn;
-    const unsigned q4 = q4n, xs = xsn;
-    request_x(item + builders);
-    if (vec && x16) {
-#pragma unroll
-      for (int i = 0; i < 4; ++i) { y[2 * i] = widen16(q[i] & 0xffffu); y[2 * i + 1] = widen16(q[i] >> 16); }
-      y[8] = widen16(q4 & 0xffffu);
-      y[9] = widen16(q4 >> 16);
-    } else if (vec) {
-      const unsigned d[3] = {__builtin_amdgcn_alignbyte(q.y, q.x, xs), __builtin_amdgcn_alignbyte(q.z, q.y, xs), __builtin_amdgcn_alignbyte(0u, q.z, xs)};
-#pragma unroll
-      for (int t = 0; t < 10; ++t) y[t] = (float)(int)(int8_t)((d[t >> 2] >> (8 * (t & 3))) & 0xffu);
-    }
-    if (vec) {
-      if (640 * (int64_t)(cb + c + 1) > a.K) {  // (uniform: the row's last chunk)
-#pragma unroll
-        for (int t = 0; t < 10; ++t) y[t] = k0 + t < a.K ? y[t] : 0.f;
-      }
-    } else {
-#pragma unroll
-      for (int t = 0; t < 10; ++t) y[t] = k0 + t < a.K ? load_act_f32(a.x, a.x_dtype, xrow + k0 + t) : 0.f;
-    }
-    if (a.x_dtype != BP_I8) {  // (int8 values fit as they are: prescale 1)
-      unsigned m_lo = 0, m_hi = 0;
-#pragma unroll
-      for (int t = 0; t < 10; ++t) {
-        const unsigned v = __float_as_uint(y[t]) & 0x7fffffffu;
-        if (((tt0 + t) >> 7) == glo) m_lo = m_lo > v ? m_lo : v;
-        else m_hi = m_hi > v ? m_hi : v;
-      }
-      __hip_atomic_fetch_max((lds_u32*)(dst + F4_PRE_OFF + 4 * glo), m_lo, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WAVEFRONT);
-      if (ghi != glo) __hip_atomic_fetch_max((lds_u32*)(dst + F4_PRE_OFF + 4 * ghi), m_hi, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WAVEFRONT);
-    }
-    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
-    __builtin_amdgcn_wave_barrier();
-    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
-    if (lane < 8) {
-      const int g = lane;
-      const unsigned at = dst + 4 * g;
-      const bool real = g < 5 && 128 * (int64_t)(5 * (cb + c) + g) < a.K;
-      int sh = 0;
-      bool finite = true;
-      if (real && a.x_dtype != BP_I8) {
-        const int ex = (int)((*(const lds_u32*)(at + F4_PRE_OFF) >> 23) & 255u);
-        finite = ex != 255;  // a NaN or an infinity among the group's activations
-        sh = 134 - ex;
-        sh = sh > 120 ? 120 : sh < -120 ? -120 : sh;
-      }
-      *(lds_u32*)(at + F4_PRE_OFF) = (unsigned)(sh + 127) << 23;
-      // (the inverse prescale multiplies every row's group sum: NaN for a group with a non-finite activation, so the
-      // token's outputs are NaN rather than finite and wrong)
-      *(lds_u32*)(at + F4_INV_OFF) = !real ? 0u : finite ? (unsigned)(127 - sh) << 23 : 0x7fc00000u;
-    }
-    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
-    __builtin_amdgcn_wave_barrier();
-    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
-    const float pre_lo = __uint_as_float(*(const lds_u32*)(dst + F4_PRE_OFF + 4 * glo));
-    const float pre_hi = __uint_as_float(*(const lds_u32*)(dst + F4_PRE_OFF + 4 * ghi));
-    u32x4 lo[PC] = {}, hi[PC] = {};
-#pragma unroll
-    for (int t = 0; t < 10; t += 2) {  // two activations per conversion
-      const bool in0 = ((tt0 + t) >> 7) == glo, in1 = ((tt0 + t + 1) >> 7) == glo;
-      float r0 = y[t] * (in0 ? pre_lo : pre_hi), r1 = y[t + 1] * (in1 ? pre_lo : pre_hi);
-      const int pos0 = 8 * (t / 5) + t % 5, pos1 = 8 * ((t + 1) / 5) + (t + 1) % 5;  // digit slots of the block
-#pragma unroll
-      for (int p = 0; p < PC; ++p) {
-        const int w = __builtin_amdgcn_cvt_pk_fp8_f32(p == 2 ? r0 * 256.f : r0, p == 2 ? r1 * 256.f : r1, 0, false);
-        if (p + 1 < PC) {
-          r0 -= __builtin_amdgcn_cvt_f32_fp8(w, 0);
-          r1 -= __builtin_amdgcn_cvt_f32_fp8(w, 1);
-        }
-        const unsigned c0 = (unsigned)w & 0xffu, c1 = ((unsigned)w >> 8) & 0xffu;
-        lo[p][pos0 >> 2] |= (in0 ? c0 : 0u) << (8 * (pos0 & 3));
-        hi[p][pos0 >> 2] |= (in0 ? 0u : c0) << (8 * (pos0 & 3));
-        lo[p][pos1 >> 2] |= (in1 ? c1 : 0u) << (8 * (pos1 & 3));
-        hi[p][pos1 >> 2] |= (in1 ? 0u : c1) << (8 * (pos1 & 3));
-      }
-    }
-#pragma unroll
-    for (int p = 0; p < PC; ++p) *(lds_u32x4*)(dst + 16 * (PC * blk + p)) = lo[p];
-    if (ghi != glo) {
-#pragma unroll
-      for (int p = 0; p < PC; ++p) *(lds_u32x4*)(dst + F4_HI_OFF + 16 * (PC * (ghi - 1) + p)) = hi[p];
-    }
-    if (blk == 0) *(lds_u32x4*)(dst + F4_ZERO_OFF) = u32x4{0u, 0u, 0u, 0u};
-  }
-}
-
-// A lane as a row of operand A (rows 4 g + p = piece p of group g < 4; rows 3, 7, 11 = pieces of group 4; row 15 unused;
-// several tokens: row 4 s + 2 t + p = piece p of the pair's token t in group slot s < 3, rows 12..15 unused): the 16-byte
-// block (index within the chunk's part of the tile) of instruction j, half hf, in byte 2 (j % 2) + hf of aoff[j / 2].
-template <int PC>
-__device__ __forceinline__ void f4_block_offsets(int r16, int kb, unsigned (&aoff)[4]) {
-  constexpr int F4_HI_OFF = F4Tile<PC>::HI_OFF, F4_ZERO_OFF = F4Tile<PC>::ZERO_OFF;
-  const int am_g = PC == 2 ? r16 >> 2 : (r16 & 3) < 3 ? r16 >> 2 : 4, am_p = PC == 2 ? r16 & 1 : (r16 & 3) < 3 ? r16 & 3 : r16 >> 2;
-  const bool am_used = PC == 2 ? r16 < 12 : r16 < 15;
-#pragma unroll
-  for (int j = 0; j < 8; ++j) {
-    unsigned both = 0;
-#pragma unroll
-    for (int hf = 0; hf < 2; ++hf) {
-      const int blk = j * 8 + kb * 2 + hf;
-      const int tt0 = 5 * f4_pair_byte(j, kb, hf), glo = tt0 >> 7, ghi = (tt0 + 9) >> 7;
-      // (several tokens: the group behind the lane's slot in this instruction's window)
-      const int g = PC == 3 || j < 4 ? am_g : am_g == 0 ? 3 : am_g == 1 ? 4 : 2;
-      unsigned o = F4_ZERO_OFF / 16;
-      if (am_used && g == glo) o = PC * blk + am_p;
-      else if (am_used && g == ghi) o = F4_HI_OFF / 16 + PC * (ghi - 1) + am_p;
-      both |= o << (8 * hf);
-    }
-    if (j & 1) aoff[j >> 1] |= both << 16;
-    else aoff[j >> 1] = both;
-  }
-}
 
 // ABL (development): timing ablations - 1 no chunk loop, 2 no table reads, 3 no operand A reads, 4 no matrix instructions, 5 no byte extraction (and the loads are not waited for),
 // 6 bytes extracted from registers that are not loaded (no loads at all), 7 = 2 + 3 + 4 (loads and byte extraction only),
@@ -736,369 +509,6 @@ __global__ __launch_bounds__(WAVES * 64, KS ? 2 : 4) void k_tq1_gemv_fp4(GemmArg
   else if (NP >= 4 && npairs == 3) all_terms(IC<(NP >= 4 ? 3 : NP)>{});
   else all_terms(IC<NP>{});
 }
-// ---- One token row per expert, the rows streamed through LDS tile by tile: "a chunk per wave" -------------------------
-//
-// The kernel above lets every wave walk along its own 16 rows: a wave load is 16 rows x 64 bytes (rows of Kp bytes start
-// at any byte, so each of the 16 pieces straddles memory lines that the wave comes back to chunks later), and operand A
-// is read from LDS once per matrix instruction - 8 x the packed bytes. Here a workgroup of 16 waves walks over tiles of
-// 16 rows together, with two kinds of waves:
-//  * loaders request a tile's 16 x Kp bytes as 4 rows x 256 bytes per wave load (a lane takes 16 bytes at a dword-aligned
-//    address; LPW loads per loader and tile, the tile's scales - 16 x G x 2 bytes, contiguous - among them), two tiles
-//    ahead, and park them in tile buffers in LDS (row n at n x pitch, shifted by the row's misalignment of 0..3 bytes);
-//  * multipliers read a tile back as the matrix instruction wants it (row n = lane % 16, the 16-byte quarters of a 64-byte
-//    window across lanes / 16, plus the dword that follows for the realignment). Wave c of a group keeps chunk c of the
-//    token's operand A in registers (8 instructions x 8 registers) and multiplies chunk c of every tile: no operand A
-//    reads in the loop. A group is nchunks multipliers and its loaders; groups walk over their own tiles (tile index =
-//    group mod groups);
-//  * a multiplier's 16 partial sums of a tile (one per row) go to LDS, and the group's first loader adds the chunks' sums
-//    in a fixed order and adds the result to the row's entry of the workgroup's outputs, which wait in LDS too: read
-//    from memory when the workgroup starts, written back once after the last term.
-// A barrier hands over TPB tiles: two where four tile buffers fit beside the table (the loaders' waits for memory and
-// the multipliers' work vary from tile to tile: the fewer the meeting points, the less is waited), else one with two
-// buffers. The buffers that the loaders fill were multiplied before the previous barrier. The tile buffers take the
-// place of the operand A tiles once those are in registers.
-constexpr int CW_WAVES = 16;
-constexpr int CW_LUT_BYTES = 256 * 256;  // byte -> 5 fp4 codes, 64 copies: entry v copy c at 256 v + 4 c
-constexpr int CW_STAGE_PER_THREAD = 4;    // outputs of a workgroup per thread at most (they wait in LDS from the first barrier to the end)
-// A row's image in a tile buffer: up to 3 bytes of misalignment, the row's Kp bytes and the dword after them, in whole
-// 16-byte pieces, at a pitch that is an odd number of pieces (16 rows: 16 different groups of 4 banks). What a
-// multiplier reads past a row's image in its last chunk (the next row's bytes, or what follows the buffer) meets
-// activations that are 0.
-constexpr int cw_pitch(int64_t Kp) {
-  const int pieces = (int)((Kp + 3 + 4 + 15) / 16);
-  return 16 * (pieces | 1);
-}
-constexpr int cw_colblks(int64_t Kp) { return (int)((Kp + 3 + 255) / 256); }  // wave loads of 4 rows x 256 bytes per 4 rows
-constexpr int64_t cw_buffer_bytes(int64_t Kp, int64_t G, int64_t scale_bytes) { return 16 * (int64_t)cw_pitch(Kp) + 16 * G * scale_bytes; }
-
-// LPW: wave loads of packed bytes per loader and tile; TPB: tiles per barrier. NTOK = 2: a pair of token rows per expert
-// (rows first_row, first_row + 1), as in the kernel above: two fp8 pieces per activation, one matrix instruction serves
-// both tokens (row 4 s + 2 t + p of operand A = piece p of token t in group slot s), an accumulator tile per 64-byte window,
-// and a multiplier's registers hold the pair's chunk (the same 8 x 8 registers).
-template <int SDT, int LPW, int TPB, int NTOK = 1>
-__global__ __launch_bounds__(CW_WAVES * 64) void k_tq1_gemv_cw(GemmArgs a, int nchunks, int groups, int tiles_per_wg, int first_row) {
-  static_assert(NTOK == 1 || NTOK == 2, "one token row per expert, or a pair");
-  constexpr int WAVES = CW_WAVES, THREADS = WAVES * 64, NB = 2 * TPB, PC = f4_pieces(NTOK), SB = SDT == BP_F32 ? 4 : 2;
-  constexpr int F4_INV_OFF = F4Tile<PC>::INV_OFF, F4_CHUNK_BYTES = F4Tile<PC>::CHUNK_BYTES, AT = CW_LUT_BYTES;
-  const int wave = __builtin_amdgcn_readfirstlane((int)(threadIdx.x >> 6)), lane = threadIdx.x & 63;
-  const int r16 = lane & 15, kb = lane >> 4;
-  const int64_t e = blockIdx.y;
-  const int64_t o0 = clamp_i64(a.offsets[e], 0, a.T), o1 = clamp_i64(a.offsets[e + 1], 0, a.T);
-  const int64_t tok = o0 + first_row;
-  if (tok >= o1) return;  // (uniform: an expert without a token row in this launch)
-  const int ntok = o1 - tok < NTOK ? (int)(o1 - tok) : NTOK;
-  float xsc[NTOK];
-#pragma unroll
-  for (int tt = 0; tt < NTOK; ++tt) xsc[tt] = a.x_dtype == BP_I8 && tt < ntok ? a.x_scale[tok + tt] : 1.f;
-  const int gs = a.group == 256 ? 1 : 0;
-
-  // ---- roles (wave-uniform): multiplier of chunk c in group grp, or loader number lidx of the group's lpg loaders
-  const int active = groups * nchunks, extra = wave - active, lpg = (WAVES - active) / groups;
-  const bool multiplier = wave < active, loader = !multiplier && extra < lpg * groups;
-  const int grp = multiplier ? wave / nchunks : extra % groups;
-  const int c = multiplier ? wave - grp * nchunks : 0;
-  const int lidx = multiplier ? 0 : extra / groups;
-
-  // ---- LDS behind the table: per group NB tile buffers (16 rows at `pitch`, then the tile's scales), then the partial sums
-  const int colblks = cw_colblks(a.Kp), pitch = cw_pitch(a.Kp);
-  const int scb = (int)(16 * a.G * SB);  // a tile's scales: 16 rows x G entries, contiguous
-  const int buf_bytes = 16 * pitch + scb;
-  const unsigned gbase = (unsigned)(AT + grp * NB * buf_bytes);
-  const unsigned red = (unsigned)(AT + groups * NB * buf_bytes + grp * NB * nchunks * 64 * NTOK);  // [tile % NB][chunk][token][row]
-  const int nl = 4 * colblks, ns = (scb + 1023) >> 10;  // wave loads of a tile: packed bytes, scales
-  const int64_t tiles = a.N / 16;
-  const int64_t tile0 = (int64_t)blockIdx.x * tiles_per_wg;
-  const int64_t tile_end = tile0 + tiles_per_wg < tiles ? tile0 + tiles_per_wg : tiles;
-  const int n_iter = (tiles_per_wg + groups - 1) / groups;  // tiles of a group
-  const int n_int = (n_iter + TPB - 1) / TPB;                 // barriers: TPB tiles each
-  auto tile_of = [&](int t) -> int64_t { return tile0 + (int64_t)t * groups + grp; };
-  // ---- the workgroup's outputs, [tile of the workgroup][token][row] float32, behind the buffers and sums (and behind the
-  // operand A tiles, which are built in the buffers' place): read from memory now, parked in LDS before the first
-  // barrier, added to there tile by tile, and written back once after the last term - no access to the outputs in the loop.
-  const int stream_bytes = groups * NB * (buf_bytes + nchunks * 64 * NTOK), build_bytes = nchunks * NTOK * F4_CHUNK_BYTES;
-  const unsigned stage = (unsigned)(AT + (stream_bytes > build_bytes ? stream_bytes : build_bytes));
-  const int n_stage = (int)(tile_end - tile0) * 16 * NTOK;  // (at most CW_STAGE_PER_THREAD x the workgroup's threads: the launcher's bound)
-  auto out_index = [&](int o) -> int64_t { return (tok + ((o >> 4) % NTOK)) * a.N + (tile0 + (o >> 4) / NTOK) * 16 + (o & 15); };
-  float was[CW_STAGE_PER_THREAD];
-#pragma unroll
-  for (int u = 0; u < CW_STAGE_PER_THREAD; ++u) {
-    const int o = (int)threadIdx.x + u * THREADS;
-    was[u] = o < n_stage && ((o >> 4) % NTOK) < ntok ? a.out[out_index(o)] : 0.f;
-  }
-
-  // ---- loaders: state of the current term (the expert's rows and scales as buffers of their own: a tile past N reads
-  // zeros) and the wave's loads of a tile: LPW of the nl wave loads of packed bytes (li = i * lpg + lidx: rows
-  // 4 (li % 4) .. + 3, bytes 256 (li / 4) .. + 255 of the rows' LDS images; what depends on li is uniform and goes into
-  // the loads' scalar offsets, so one lane offset serves all of them) and one of the ns wave loads of the scales
-  __amdgpu_buffer_rsrc_t wrs = make_rsrc(a.packed[0], 0), srs = wrs;
-  unsigned w_lane = 0, w_last = 0, s_lane = 0x7ffffff0u;  // lane offsets of the loads (past the buffer: zeros, no memory access)
-  const unsigned d_lane = (unsigned)(kb * pitch + 16 * r16), ds_lane = (unsigned)(16 * pitch + 16 * (lidx * 64 + lane));
-  const bool put_s = loader && lidx < ns && 16 * (lidx * 64 + lane) < scb;
-  u32x4 ring[2][LPW + 1];
-  auto slot_li = [&](int i) { return i * lpg + lidx; };
-  auto setup_term = [&](int term) {
-    const unsigned char* expert_rows = a.packed[term] + e * a.N * a.Kp;
-    const unsigned mis = (unsigned)((uintptr_t)expert_rows & 3);
-    wrs = make_rsrc(expert_rows - mis, whole_dwords(a.N * a.Kp + mis));
-    srs = make_rsrc((const unsigned char*)a.w_scale[term] + e * a.N * a.G * SB, a.N * a.G * SB);  // (dword-aligned: checked by the host)
-    const unsigned ro = mis + (unsigned)kb * (unsigned)a.Kp;
-    w_lane = (ro & ~3u) + 16u * (unsigned)r16;  // (rows 4 apart are a multiple of 4 bytes apart)
-    // (the last block of 256 bytes: only the pieces that hold bytes of the row)
-    w_last = 256 * (colblks - 1) + 16 * r16 < (int)(ro & 3u) + (int)a.Kp ? w_lane : 0x7ffffff0u;
-    s_lane = put_s ? (unsigned)(16 * (lidx * 64 + lane)) : 0x7ffffff0u;
-  };
-  const unsigned step_w = (unsigned)(16 * a.Kp), step_s = (unsigned)scb;  // a tile's bytes
-  auto request = [&](int t, auto slot_c) {  // the loads of the tile of iteration t
-    constexpr int slot = decltype(slot_c)::value;
-    const int64_t tile = tile_of(t);
-    const bool live = loader && tile < tiles;
-#pragma unroll
-    for (int i = 0; i < LPW; ++i) {
-      const int li = slot_li(i);
-      const unsigned so = (unsigned)tile * step_w + (unsigned)(4 * (li & 3)) * (unsigned)a.Kp + 256u * (unsigned)(li >> 2);
-      ring[slot][i] = buf_load16(wrs, (li >> 2) == colblks - 1 ? w_last : w_lane, live && li < nl ? so : 0x7ffffff0u);
-    }
-    ring[slot][LPW] = buf_load16(srs, s_lane, live ? (unsigned)tile * step_s : 0x7ffffff0u);
-  };
-  auto park = [&](int t, auto slot_c) {  // ... into the buffer of iteration t
-    constexpr int slot = decltype(slot_c)::value;
-    const unsigned wb = gbase + (unsigned)((t % NB) * buf_bytes);
-#pragma unroll
-    for (int i = 0; i < LPW; ++i) {
-      const int li = slot_li(i);
-      if (loader && li < nl) {  // (uniform; in a row's last block of 256 bytes only the pieces that hold bytes of the row: the next row's image follows)
-        if ((li >> 2) < colblks - 1 || w_last != 0x7ffffff0u) *(lds_u32x4*)(wb + (unsigned)(4 * (li & 3) * pitch + 256 * (li >> 2)) + d_lane) = ring[slot][i];
-      }
-    }
-    if (put_s) *(lds_u32x4*)(wb + ds_lane) = ring[slot][LPW];
-  };
-  // ---- the byte table, one copy per lane (64 banks: no two lanes of a wave share one): entry v = digits d0..d4 of v as
-  // fp4 codes in nibbles 0..4, at 256 v + 4 lane - an address that one byte permute makes from a packed byte and 4 lane
-  auto build_table = [&] {
-  for (int idx = threadIdx.x; idx < 256 * 16; idx += THREADS) {
-    unsigned v = (unsigned)idx >> 4, ent = 0;
-    if (v < 243) {
-#pragma unroll
-      for (int d = 0; d < 5; ++d) {
-        const unsigned q = v / 3, dig = v - 3 * q;
-        ent |= (dig == 0 ? 0xAu : dig == 2 ? 0x2u : 0u) << (4 * d);
-        v = q;
-      }
-    }
-    *(lds_u32x4*)(16 * idx) = u32x4{ent, ent, ent, ent};
-  }
-  };
-  // A loader has few instructions per tile and everything waits for them: they go before those of the multipliers on
-  // its SIMD. The first term's first two tiles are requested before the table and the token's tile are built.
-  if (!multiplier) {
-    __builtin_amdgcn_s_setprio(3);
-    setup_term(0);
-    request(0, IC<0>{});
-    request(1, IC<1>{});
-    build_table();
-  } else {  // (chunk by chunk, by the multipliers; their part of the table while the activations are on their way)
-    f4_build_tiles<NTOK, WAVES, AT>(a, tok, ntok, nchunks, 0, wave, lane, active, build_table);
-  }
-
-#pragma unroll
-  for (int u = 0; u < CW_STAGE_PER_THREAD; ++u) {
-    const int o = (int)threadIdx.x + u * THREADS;
-    if (o < n_stage) *(lds_u32*)(stage + 4u * (unsigned)o) = __float_as_uint(was[u]);
-  }
-  __syncthreads();
-
-  if (multiplier) {
-    // ---- the wave's chunk of operand A (a pair: the lane's token's tile), and the inverse prescales of the lane's two
-    // groups: one token: group kb and group 4, of which the lane holds piece kb; a pair: the lane's group of the first
-    // window and of the second (kb and 3, 4, 2, 2 for kb = 0..3; the lanes kb = 3 hold unused rows: their sums are 0)
-    i32x8 A[8];
-    float inv_a[NTOK], inv_b[NTOK];
-    const int g_w0 = NTOK == 1 ? kb : kb < 3 ? kb : 2, g_w1 = NTOK == 1 ? 4 : kb == 0 ? 3 : kb == 1 ? 4 : 2;
-    {
-      unsigned aoff[4];
-      f4_block_offsets<PC>(r16, kb, aoff);
-      const unsigned cbase = (unsigned)(AT + c * NTOK * F4_CHUNK_BYTES);
-      const unsigned mine = cbase + (NTOK == 2 ? (unsigned)(((r16 >> 1) & 1) * F4_CHUNK_BYTES) : 0u);
-#pragma unroll
-      for (int j = 0; j < 8; ++j) {
-        const u32x4 lo = *(const lds_u32x4*)((((aoff[j >> 1] >> (16 * (j & 1))) & 0xffu) << 4) + mine);
-        const u32x4 hi = *(const lds_u32x4*)((((aoff[j >> 1] >> (16 * (j & 1) + 8)) & 0xffu) << 4) + mine);
-        A[j] = i32x8{(int)lo.x, (int)lo.y, (int)lo.z, (int)lo.w, (int)hi.x, (int)hi.y, (int)hi.z, (int)hi.w};
-      }
-      const float f4th = kb == 3 ? 0.f : kb == 2 ? 1.f / 256.f : 1.f;
-#pragma unroll
-      for (int tt = 0; tt < NTOK; ++tt) {
-        inv_a[tt] = __uint_as_float(*(const lds_u32*)(cbase + tt * F4_CHUNK_BYTES + F4_INV_OFF + 4 * g_w0));
-        inv_b[tt] = __uint_as_float(*(const lds_u32*)(cbase + tt * F4_CHUNK_BYTES + F4_INV_OFF + 4 * g_w1)) * (NTOK == 1 ? f4th : 1.f);
-      }
-    }
-    const unsigned lane4 = (unsigned)lane << 2;
-    // the lane's reads of a tile: its row's window of chunk c, and the scales of its two groups (an index past the row's
-    // last group - the last chunk of a row - meets sums that are 0 and takes the last group's scale)
-    const unsigned rd_w = (unsigned)(r16 * pitch + 128 * c + 16 * kb);
-    const int64_t g_last = a.G - 1;
-    const int64_t ga = (5 * (int64_t)c + g_w0) >> gs, gb = (5 * (int64_t)c + g_w1) >> gs;
-    const unsigned rd_sa = (unsigned)(16 * pitch + r16 * (int)(a.G * SB) + SB * (int)(ga < g_last ? ga : g_last));
-    const unsigned rd_sb = (unsigned)(16 * pitch + r16 * (int)(a.G * SB) + SB * (int)(gb < g_last ? gb : g_last));
-    __syncthreads();  // (every multiplier has its operand A: the tile buffers may overwrite the tiles)
-
-    for (int term = 0; term < a.n_terms; ++term) {
-      const unsigned mis = (unsigned)((uintptr_t)(a.packed[term] + e * a.N * a.Kp) & 3);
-      const unsigned dlt = (mis + (unsigned)r16 * (unsigned)a.Kp) & 3u;  // the lane's row starts dlt bytes into its LDS row
-      auto multiply = [&](int t) {
-        const unsigned rb = gbase + (unsigned)((t % NB) * buf_bytes);
-        const u32x4 W0 = *(const lds_u32x4*)(rb + rd_w), W1 = *(const lds_u32x4*)(rb + rd_w + 64);
-        const unsigned x0 = *(const lds_u32*)(rb + rd_w + 16), x1 = *(const lds_u32*)(rb + rd_w + 80);
-        const unsigned ra = SB == 4 ? *(const lds_u32*)(rb + rd_sa) : (unsigned)*(const lds_u16*)(rb + rd_sa);
-        const unsigned rbits = SB == 4 ? *(const lds_u32*)(rb + rd_sb) : (unsigned)*(const lds_u16*)(rb + rd_sb);
-        // the table reads run BD instructions ahead of the matrix instructions (the scheduling barriers keep the compiler
-        // from sinking them back to their uses: a wave would wait out an LDS round trip per instruction)
-        constexpr int BD = 2;
-        u32x4 Bq[BD + 1];
-        auto lookup = [&](auto j_c) {
-          constexpr int j = decltype(j_c)::value, i = j & 3;
-          const u32x4& W = j < 4 ? W0 : W1;
-          const unsigned d = __builtin_amdgcn_alignbyte(i < 3 ? W[i < 3 ? i + 1 : 0] : (j < 4 ? x0 : x1), W[i], dlt);
-#pragma unroll
-          for (int w = 0; w < 4; ++w)  // (byte 1 of the address: byte w of d; byte 0: 4 lane)
-            Bq[j % (BD + 1)][w] = *(const lds_u32*)__builtin_amdgcn_perm(d, lane4, 0x0c0c0400u + ((unsigned)w << 8));
-        };
-        f32x4 C[NTOK];  // (a pair: one accumulator tile per window)
-#pragma unroll
-        for (int q = 0; q < NTOK; ++q) C[q] = f32x4{0.f, 0.f, 0.f, 0.f};
-        lookup(IC<0>{});
-        lookup(IC<1>{});
-        auto stage = [&](auto j_c) {
-          constexpr int j = decltype(j_c)::value, ci = NTOK == 1 ? 0 : j >> 2;
-          __builtin_amdgcn_sched_barrier(0);
-          if (j + BD < 8) lookup(IC<(j + BD < 8 ? j + BD : 0)>{});
-          __builtin_amdgcn_sched_barrier(0);
-          const u32x4 bq = Bq[j % (BD + 1)];
-          const i32x8 B8 = {(int)bq.x, (int)bq.y, (int)bq.z, (int)bq.w, 0, 0, 0, 0};
-          C[ci] = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(A[j], B8, C[ci], 0 /* A: E4M3 */, 4 /* B: E2M1 */, 0, 0, 0, 0);
-        };
-        stage(IC<0>{}); stage(IC<1>{}); stage(IC<2>{}); stage(IC<3>{}); stage(IC<4>{}); stage(IC<5>{}); stage(IC<6>{}); stage(IC<7>{});
-        __builtin_amdgcn_sched_barrier(0);
-        const float sa = SDT == BP_F32 ? __uint_as_float(ra) : SDT == BP_F16 ? f16_bits_to_f32((uint16_t)ra) : __uint_as_float(ra << 16);
-        const float sb = SDT == BP_F32 ? __uint_as_float(rbits) : SDT == BP_F16 ? f16_bits_to_f32((uint16_t)rbits) : __uint_as_float(rbits << 16);
-        // the row's sum over its four lanes (one per quarter): row n ends up in every lane n + 16 q
-#pragma unroll
-        for (int tt = 0; tt < NTOK; ++tt) {
-          float v;
-          if (NTOK == 1) {
-            v = sa * inv_a[0] * (C[0][0] + C[0][1] + C[0][2] * (1.f / 256.f)) + sb * inv_b[0] * C[0][3];
-          } else {  // rows 4 kb + 2 tt + p of the two windows' tiles
-            const f32x4 c0 = C[0], c1 = C[NTOK - 1];
-            v = sa * inv_a[tt] * (tt ? c0[2] + c0[3] : c0[0] + c0[1]) + sb * inv_b[tt] * (tt ? c1[2] + c1[3] : c1[0] + c1[1]);
-          }
-          const auto h32 = __builtin_amdgcn_permlane32_swap(__float_as_uint(v), __float_as_uint(v), false, false);
-          v = __uint_as_float(h32[0]) + __uint_as_float(h32[1]);
-          const auto h16 = __builtin_amdgcn_permlane16_swap(__float_as_uint(v), __float_as_uint(v), false, false);
-          v = __uint_as_float(h16[0]) + __uint_as_float(h16[1]);
-          if (kb == 0) *(lds_u32*)(red + (unsigned)((((t % NB) * nchunks + c) * NTOK + tt) * 64 + 4 * r16)) = __float_as_uint(v);
-        }
-      };
-      if (term > 0) __syncthreads();  // (the previous term's last tiles have been added)
-      for (int i = 0; i < n_int; ++i) {
-        __syncthreads();  // (the tiles TPB i .. TPB i + TPB - 1 are in their buffers)
-#pragma unroll
-        for (int u = 0; u < TPB; ++u) multiply(TPB * i + u);
-      }
-      __syncthreads();
-    }
-    return;
-  }
-
-  // ---- loaders (and waves without a role, which only keep the barriers' count)
-  __syncthreads();  // (the multipliers have their operand A)
-  for (int term = 0; term < a.n_terms; ++term) {
-    if (term > 0) setup_term(term);
-    // The sums of the tile of iteration t, by the group's first loader: lane (row n, quarter q) adds chunks q, q + 4, ...
-    // in that order, the row's four lanes are added in a fixed order too, and the row's entry of the output stage takes
-    // one addition (this wave is the only one that touches its group's entries between the first barrier and the end).
-    auto reduce = [&](int t, auto) {
-      if (!loader || lidx != 0) return;  // (uniform)
-      const int64_t tile = tile_of(t);
-#pragma unroll
-      for (int tt = 0; tt < NTOK; ++tt) {
-        float v = 0.f;
-#pragma unroll
-        for (int q = 0; q < CW_WAVES / 4; ++q) {
-          const int ch = 4 * q + kb;
-          const unsigned at = red + (unsigned)((((t % NB) * nchunks + (ch < nchunks ? ch : 0)) * NTOK + tt) * 64 + 4 * r16);
-          const float part = __uint_as_float(*(const lds_u32*)at);
-          v += ch < nchunks ? part : 0.f;
-        }
-        const auto h32 = __builtin_amdgcn_permlane32_swap(__float_as_uint(v), __float_as_uint(v), false, false);
-        v = __uint_as_float(h32[0]) + __uint_as_float(h32[1]);
-        const auto h16 = __builtin_amdgcn_permlane16_swap(__float_as_uint(v), __float_as_uint(v), false, false);
-        v = __uint_as_float(h16[0]) + __uint_as_float(h16[1]);
-        if (lane < 16 && tile < tile_end && tt < ntok) {
-          const unsigned at_out = stage + (unsigned)((((int)(tile - tile0) * NTOK + tt) * 16 + lane) * 4);
-          *(lds_u32*)at_out = __float_as_uint(__uint_as_float(*(const lds_u32*)at_out) + (a.x_dtype == BP_I8 ? v * xsc[tt] : v));
-        }
-      }
-    };
-    // Two tiles are in flight per loader: the tile parked before a barrier was requested two tiles ago.
-    static_assert(TPB == 1 || TPB == 2, "tiles per barrier");
-    if (term > 0) __syncthreads();  // (the previous term's last tiles have been multiplied)
-    if (term > 0) {
-      request(0, IC<0>{});
-      request(1, IC<1>{});
-    }
-    for (int t = 0; t < TPB * n_int; t += 2) {
-      park(t, IC<0>{});
-      request(t + 2, IC<0>{});
-      if constexpr (TPB == 1) {
-        __syncthreads();
-        if (t > 0) reduce(t - 1, IC<1>{});  // (multiplied before this barrier)
-        if (t + 1 >= n_int) break;  // (uniform)
-      }
-      park(t + 1, IC<1>{});
-      request(t + 3, IC<1>{});
-      __syncthreads();
-      if constexpr (TPB == 1) {
-        reduce(t, IC<0>{});
-      } else {
-        if (t > 0) {
-          reduce(t - 2, IC<0>{});
-          reduce(t - 1, IC<1>{});
-        }
-      }
-    }
-    __syncthreads();
-    if constexpr (TPB == 2) reduce(TPB * n_int - 2, IC<0>{});
-    if (TPB == 2 || (n_int & 1) == 0) reduce(TPB * n_int - 1, IC<1>{});
-    else reduce(n_int - 1, IC<0>{});
-  }
-  // ---- the group's first loader writes its tiles' outputs back: the entries it has added to itself (no barrier), four
-  // tiles per wave store
-  if (loader && lidx == 0) {
-    for (int t = kb; t < n_iter; t += 4) {
-      const int64_t tile = tile_of(t);
-#pragma unroll
-      for (int tt = 0; tt < NTOK; ++tt) {
-        if (tile < tile_end && tt < ntok)
-          a.out[(tok + tt) * a.N + tile * 16 + r16] = __uint_as_float(*(const lds_u32*)(stage + (unsigned)((((int)(tile - tile0) * NTOK + tt) * 16 + r16) * 4)));
-      }
-    }
-  }
-}
-
-int f4_cus() {  // compute units of the current device (256 if the query fails); looked up once per device
-  static std::mutex m;
-  static int known[64] = {};
-  int dev = 0;
-  if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64) return 256;
-  std::lock_guard<std::mutex> lock(m);
-  if (known[dev] == 0) {
-    int cus = 0;
-    if (hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || cus < 1) cus = 256;
-    known[dev] = cus;
-  }
-  return known[dev];
-}
-
 template <int SDT, int WAVES, int ABL = 0, int NTOK = 1, int SR = 0, int KS = 0>
 int launch_f4_k(const GemmArgs& a, hipStream_t s, const char* name, int nchunks, size_t lds, int seg_chunks = 0 /* chunks per launch (0: all) */, int first_row = 0) {
   if (const int rc = raise_lds_limit<k_tq1_gemv_fp4<SDT, WAVES, ABL, NTOK, SR, KS>>(F4_LDS_MAX)) return rc;
@@ -1124,70 +534,6 @@ int launch_f4_k(const GemmArgs& a, hipStream_t s, const char* name, int nchunks,
   return BP_OK;
 }
 
-// Launch of the chunk-per-wave kernel, or BP_ERR_UNSUPPORTED (no message) where it does not apply: more than 15 chunks
-// per row, scales that are not dword-aligned, an expert whose rows or scales exceed a buffer descriptor, tile buffers
-// that do not fit, or a call too small for it (each workgroup builds the table and the token's tile before it streams).
-template <int SDT, int NTOK>
-int launch_cw(const GemmArgs& a, hipStream_t s, int64_t nchunks, int cus, int first_row) {
-  const char force = tuning().tq1;
-  if (force == 'r') return BP_ERR_UNSUPPORTED;
-  for (int t = 0; t < a.n_terms; ++t)
-    if (((uintptr_t)a.w_scale[t] & 3) != 0) return BP_ERR_UNSUPPORTED;
-  constexpr int64_t SB = SDT == BP_F32 ? 4 : 2;
-  if (a.N * a.Kp >= 0x7fffffe0 || a.N * a.G * SB >= 0x7fffffe0) return BP_ERR_UNSUPPORTED;
-  const int64_t experts = a.E < a.T ? a.E : a.T, tiles = a.N / 16;
-  if (force != 'c' && experts * tiles < 16 * (int64_t)cus) return BP_ERR_UNSUPPORTED;
-  int64_t wpe = cus / experts;  // workgroups per expert: one workgroup per CU is resident
-  wpe = wpe < 1 ? 1 : wpe > tiles ? tiles : wpe;
-  int64_t per = (tiles + wpe - 1) / wpe;  // tiles per workgroup
-  const int64_t buf = cw_buffer_bytes(a.Kp, a.G, SB);
-  const int64_t nl = 4 * cw_colblks(a.Kp), ns = (16 * a.G * SB + 1023) / 1024;  // wave loads per tile: packed bytes, scales
-  // A group: nchunks multipliers and its loaders, which take up to 8 wave loads of packed bytes each and one of the
-  // scales. As many groups as fit the 16 waves, the tiles of a workgroup and LDS (two tiles per barrier if those fit too).
-  auto loaders_of = [&](int g) { return (CW_WAVES - g * nchunks) / g; };
-  // (a workgroup keeps its outputs in LDS: at most CW_STAGE_PER_THREAD per thread, 64 bytes per tile and token)
-  const int64_t per_cap = CW_STAGE_PER_THREAD * CW_WAVES * 64 / (16 * NTOK);
-  if (per > per_cap) per = per_cap;
-  auto lds_of = [&](int g, int tpb) {
-    const int64_t stream = (int64_t)g * 2 * tpb * (buf + nchunks * 64 * NTOK), build = nchunks * NTOK * f4_chunk_bytes(NTOK);
-    const int64_t mine = (per + g - 1) / g * g;  // tiles per workgroup with g groups
-    return (int64_t)CW_LUT_BYTES + (stream > build ? stream : build) + mine * 64 * NTOK;
-  };
-  auto fits = [&](int g, int tpb) {
-    const int64_t l = loaders_of(g);
-    return l >= 1 && l >= ns && (nl + l - 1) / l <= 8 && lds_of(g, tpb) <= F4_LDS_MAX;
-  };
-  int groups = (int)(CW_WAVES / (nchunks + 1));
-  if (groups > per) groups = (int)per;
-  while (groups > 1 && !fits(groups, 1)) --groups;
-  if (groups < 1 || !fits(groups, 1)) return BP_ERR_UNSUPPORTED;
-  const int tpb = fits(groups, 2) ? 2 : 1;
-  const int64_t loaders = loaders_of(groups), lpw = (nl + loaders - 1) / loaders;
-  per = (per + groups - 1) / groups * groups;
-  if (per > per_cap) per = per_cap / groups * groups;
-  // Measured against the kernel above (E x N x K from 64 x 4096 x 2048 to 256 x 2048 x 7168): ahead by 3 - 12 % with 10 or
-  // more multipliers and 48 or more tiles per group, behind with fewer of either (7 multipliers at K = 4096; 21 tiles).
-  if (force != 'c' && (groups * nchunks < 10 || per / groups < 48)) return BP_ERR_UNSUPPORTED;
-  const dim3 grid((unsigned)((tiles + per - 1) / per), (unsigned)a.E, 1u);
-  const size_t lds = (size_t)lds_of(groups, tpb);
-  note_kernel(NTOK == 1 ? "fp4_tq1_t1_cw" : "fp4_tq1_m2_cw");
-#define BP_CW_LAUNCH(L, P)                                                                                                                  \
-  {                                                                                                                                         \
-    if (const int rc = raise_lds_limit<k_tq1_gemv_cw<SDT, L, P, NTOK>>(F4_LDS_MAX)) return rc;                                              \
-    hipLaunchKernelGGL((k_tq1_gemv_cw<SDT, L, P, NTOK>), grid, dim3(CW_WAVES * 64), lds, s, a, (int)nchunks, groups, (int)per, first_row); \
-    return check_launch(NTOK == 1 ? "fp4_tq1_t1_cw" : "fp4_tq1_m2_cw");                                                                     \
-  }
-#define BP_CW_LPW(L)        \
-  if (lpw == L) {           \
-    if (tpb == 2) BP_CW_LAUNCH(L, 2) \
-    BP_CW_LAUNCH(L, 1)      \
-  }
-  BP_CW_LPW(1) BP_CW_LPW(2) BP_CW_LPW(3) BP_CW_LPW(4) BP_CW_LPW(5) BP_CW_LPW(6) BP_CW_LPW(7) BP_CW_LPW(8)
-#undef BP_CW_LPW
-#undef BP_CW_LAUNCH
-  return BP_ERR_UNSUPPORTED;
-}
-
 template <int SDT, int NTOK>
 int launch_f4(const GemmArgs& a, hipStream_t s, int first_row = 0) {
   const int64_t nchunks = (a.K + 639) / 640;
@@ -1203,7 +549,7 @@ int launch_f4(const GemmArgs& a, hipStream_t s, int first_row = 0) {
   const bool sr_ok = SRV && (a.G * 2) % 4 == 0;
   if constexpr (NTOK == 2) {  // (a pair of rows per expert in a large call: the rows through LDS tile by tile)
     if (nseg == 1) {
-      const int rc = launch_cw<SDT, 2>(a, s, nchunks, cus, first_row);
+      const int rc = launch_tq1_gemv_cw(a, s, 2, nchunks, cus, first_row);
       if (rc != BP_ERR_UNSUPPORTED) return rc;
     }
   }
@@ -1219,7 +565,7 @@ int launch_f4(const GemmArgs& a, hipStream_t s, int first_row = 0) {
     return launch_f4_k<SDT, 16, 0, NTOK>(a, s, name16, (int)nchunks, lds, (int)seg, first_row);
   }
   {
-    const int rc = launch_cw<SDT, 1>(a, s, nchunks, cus, 0);
+    const int rc = launch_tq1_gemv_cw(a, s, 1, nchunks, cus, 0);
     if (rc != BP_ERR_UNSUPPORTED) return rc;
   }
 #ifdef BP_DEV_ABLATIONS  // timing ablations (results are wrong): development builds only

@@ -363,6 +363,35 @@ def test_tq1_gemm_fp8_pieces_keep_small_activations(bp, ntok, tq1_gemm_kernel):
     assert torch.equal(got, torch.zeros_like(got))
 
 
+@pytest.mark.parametrize("ntok,chunk,want_kernel", [(2, False, "fp4_tq1_m2"), (2, True, "fp4_tq1_m2_cw"), (4, False, "fp4_tq1_m4"),
+                                                    (6, False, "fp4_tq1_m6"), (8, False, "fp4_tq1_m8")])
+def test_tq1_small_batches_fp8_pieces_keep_small_activations(bp, tune, ntok, chunk, want_kernel):
+    """The small-batch variants (2 to 8 token rows per expert) keep two E4M3 pieces per activation under the group's
+    power-of-two prescale: exact for bf16 values down to 2^-9 of the group's largest magnitude, at most 2^-17 of it
+    dropped below. Activations spread over 5 decades with outliers 1000 x the typical value must still come out far
+    inside the general tolerance, on the kernels that walk along their rows and on the one that streams them through LDS."""
+    if chunk:
+        tune("BP_TUNE_TQ1", "chunk")
+    rng = np.random.default_rng(17 + ntok)
+    E, N, K = 2, 272, 4352
+    packed, scales = synth_weights(17, E, N, K, GROUP, "tq1")
+    T = E * ntok
+    x = rng.standard_normal((T, K)).astype(np.float32) * np.exp(rng.uniform(-6, 6, (T, K))).astype(np.float32)
+    x[:, ::97] *= 1000.0
+    x = orc.bf16_round(x)
+    want = np.zeros((T, N), np.float32)
+    for e in range(E):
+        c_gemm(x[e * ntok:(e + 1) * ntok], None, packed[0][e], scales[0][e].astype(np.float32), K, GROUP, "tq1", out=want[e * ntok:(e + 1) * ntok])
+    got = bp.grouped_ternary_gemm(dev(x).to(torch.bfloat16), None, [0, ntok, 2 * ntok], [dev(packed[0])], [dev(scales[0])], K, GROUP, "tq1").cpu().numpy()
+    kern = bp.ext().last_kernel()
+    assert kern == want_kernel if chunk else kern.startswith(want_kernel) and not kern.endswith("_cw"), kern
+    print("rel_l2", want_kernel, rel_l2(got, want))
+    assert rel_l2(got, want) <= 2e-4, rel_l2(got, want)
+    z = np.zeros_like(x)  # all-zero activations: the prescale has nothing to go by
+    got = bp.grouped_ternary_gemm(dev(z).to(torch.bfloat16), None, [0, ntok, 2 * ntok], [dev(packed[0])], [dev(scales[0])], K, GROUP, "tq1")
+    assert torch.equal(got, torch.zeros_like(got))
+
+
 @pytest.mark.parametrize("act", ["bf16", "int8"])
 @pytest.mark.parametrize("K", [1024, 2048, 5120, 7168])
 @pytest.mark.parametrize("counts", [[2, 0, 1], [2, 2, 2], [4, 3, 1], [3, 0, 0], [8, 5, 1], [1, 6, 7], [5, 6, 0]])
