@@ -29,6 +29,11 @@ void note_kernel(const char* name) {
   g_kernel[sizeof(g_kernel) - 1] = 0;
 }
 
+void note_kernel_suffix(const char* suffix) {
+  const size_t len = strlen(g_kernel);
+  if (len + strlen(suffix) + 1 <= sizeof(g_kernel)) strcpy(g_kernel + len, suffix);
+}
+
 namespace {
 // The overrides in force: an immutable snapshot behind an atomic pointer, so that a launch path on one thread reads a
 // consistent set while bp_reload_tuning() on another publishes a new one (old snapshots are never freed: a reader may
@@ -36,7 +41,7 @@ namespace {
 std::atomic<const Tuning*> g_tuning{nullptr};
 std::once_flag g_tuning_once;
 void read_tuning() {
-  Tuning* t = new Tuning{0, 0, 0, 0, 0, 0, -1, 0, -1};
+  Tuning* t = new Tuning{0, 0, 0, 0, 0, 0, -1, 0, -1, 0};
   if (const char* v = getenv("BP_TUNE_R")) t->r = atoi(v);
   if (const char* v = getenv("BP_TUNE_WAVES")) t->waves = atoi(v);
   if (const char* v = getenv("BP_TUNE_TQ1")) t->tq1 = v[0];
@@ -46,6 +51,7 @@ void read_tuning() {
   if (const char* v = getenv("BP_TUNE_F4T")) t->f4t = atoi(v);
   if (const char* v = getenv("BP_TUNE_CPT")) t->cpt = atoi(v);
   if (const char* v = getenv("BP_TUNE_TILES")) t->tiles = atoi(v);
+  if (const char* v = getenv("BP_TUNE_GLU")) t->glu = v[0];
   g_tuning.store(t, std::memory_order_release);
 }
 }  // namespace

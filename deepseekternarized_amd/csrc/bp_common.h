@@ -13,6 +13,7 @@ namespace bp {
 // ---- host-side error plumbing (thread local, surfaced through bp_last_error) ----
 int fail(int code, const char* fmt, ...);
 void note_kernel(const char* name);
+void note_kernel_suffix(const char* suffix);  // ... appended to the name noted last
 int check_launch(const char* what);
 
 // ---- argument block of one grouped GEMM call (validated by the C entry point) ----
@@ -36,6 +37,16 @@ struct GemmArgs {
   // Workspace of the caller for kernels that convert the activations in a pass of their own (NULL: those kernels are not used).
   unsigned char* stage;
   int64_t stage_bytes;
+  // SwiGLU in the epilogue of the grouped GEMM over converted activations (glu_h != NULL; tile-list mode with overwrite):
+  // the N output rows are N / 2 gate rows followed by N / 2 up rows, and the kernel writes bf16 glu_h[T, N / 2] instead
+  // of `out`, with the rounding points of bp_swiglu_bf16 (glu_v4 = 0) or of bp_swiglu_v4 (glu_v4 = 1: clamp by glu_limit
+  // when positive, float32 product times glu_weights[glu_order[row]] when glu_weights is set, one rounding to bf16).
+  uint16_t* glu_h;
+  int glu_v4;
+  float glu_limit;
+  const float* glu_weights;
+  const int64_t* glu_order;
+  int64_t glu_pairs;
 };
 
 __device__ __forceinline__ int64_t clamp_i64(int64_t v, int64_t lo, int64_t hi) { return v < lo ? lo : (v > hi ? hi : v); }
@@ -99,6 +110,7 @@ struct Tuning {
   int f4t;     // BP_TUNE_F4T: routed rows per expert up to which launches of 8 rows are used (-1 = default)
   int cpt;     // BP_TUNE_CPT: chunks per table pass of the table-lookup GEMV
   int tiles;   // BP_TUNE_TILES: tokens from which bp_moe_layer_* runs its GEMMs over the device-side list of token tiles (-1 = default)
+  char glu;    // BP_TUNE_GLU: 'n' bp_moe_layer_* never lets the gate | up GEMM apply SwiGLU itself (a launch of its own instead)
 };
 const Tuning& tuning();
 

@@ -182,15 +182,26 @@ __global__ __launch_bounds__(F_THREADS, 2) void k_gemm_tq2f(GemmArgs a) {
 
   const int wave = __builtin_amdgcn_readfirstlane((int)(threadIdx.x >> 6)), lane = threadIdx.x & 63;
   const int r16 = lane & 15, kb = lane >> 4;
-  const int row_blocks = (int)((a.N + F_ROWS - 1) / F_ROWS);
+  // SwiGLU in the epilogue: the launch's rows are NH gate rows followed by NH up rows, and a wave's four row tiles are two
+  // of the gate (r = 0, 1) and the same two of the up projection (r = 2, 3): a row block covers F_ROWS / 2 of either
+  const bool glu = a.glu_h != nullptr;
+  const int64_t NH = glu ? a.N / 2 : a.N;
+  const int row_blocks = glu ? (int)((NH + F_ROWS / 2 - 1) / (F_ROWS / 2)) : (int)((a.N + F_ROWS - 1) / F_ROWS);
   int wg_block;
   const TileRef tr = tile_of_workgroup(a, blockIdx.x, row_blocks, wg_block);
   if (!tr.live) return;  // uniform for the workgroup
   const int64_t e = tr.e, tok0 = tr.tok0, o1 = tr.o1;
   const int ntok = (int)(o1 - tok0 < 32 ? o1 - tok0 : 32);
   const bool two = ntok > 16;  // the second token tile holds tokens
-  const int64_t n_base = (int64_t)wg_block * F_ROWS;
-  const int64_t n_wave = n_base + wave * (16 * F_RT);
+  // first row of row tile r of wave wv (-1: past the rows)
+  auto tile_row = [&](int wv, int r) -> int64_t {
+    if (glu) {
+      const int64_t c = (int64_t)wg_block * (F_ROWS / 2) + wv * (8 * F_RT) + 16 * (r & 1);
+      return c < NH ? (r >> 1) * NH + c : -1;
+    }
+    const int64_t row = (int64_t)wg_block * F_ROWS + wv * (16 * F_RT) + 16 * r;
+    return row < a.N ? row : -1;
+  };
 
   const int nwin = (int)(a.K / 256);      // 64-byte windows of a row = pairs of 128-wide groups
   const int NW = nwin * a.n_terms;        // the stacked terms, one after the other
@@ -231,8 +242,8 @@ __global__ __launch_bounds__(F_THREADS, 2) void k_gemm_tq2f(GemmArgs a) {
   unsigned wrow[F_RT];  // byte offset of the row tile's first row (a tile past N repeats the wave's first tile and is not stored)
 #pragma unroll
   for (int r = 0; r < F_RT; ++r) {
-    int64_t row = n_wave + 16 * r;
-    if (row >= a.N) row = n_wave < a.N ? n_wave : 0;
+    int64_t row = tile_row(wave, r);
+    if (row < 0) row = tile_row(wave, 0) < 0 ? 0 : tile_row(wave, 0);
     wrow[r] = (unsigned)(row * a.Kp);
   }
   // TQ1: the expert's rows as a buffer with a dword-aligned base (mis = what the rows' first byte is past it; the same
@@ -248,8 +259,8 @@ __global__ __launch_bounds__(F_THREADS, 2) void k_gemm_tq2f(GemmArgs a) {
   }
   unsigned lq = 0;  // first byte of the window to request: floor(256 ls / 5)
   const unsigned TRW = LB + (unsigned)f_lds_bytes(SB) + (unsigned)(wave * F_RT * F_TR);  // the wave's transit area
-  const int64_t my_row = n_base + threadIdx.x;
-  const unsigned my_scales = my_row < a.N ? (unsigned)(my_row * a.G * SB) : 0xfffffff0u;  // rows past N: zeros
+  const int64_t my_tile = tile_row((int)(threadIdx.x >> 6), (int)((threadIdx.x >> 4) & 3));  // thread = row, in the order the waves hold their row tiles
+  const unsigned my_scales = my_tile >= 0 ? (unsigned)((my_tile + (threadIdx.x & 15)) * a.G * SB) : 0xfffffff0u;  // rows past N: zeros
   const __amdgpu_buffer_rsrc_t xrs = make_rsrc(staged_tile(a, e, tok0), (int64_t)nwin * F_FB);
   const unsigned tail_off = threadIdx.x < F_TAIL / 16 ? (unsigned)(F_OPS + 16 * threadIdx.x) : 0xfffffff0u;  // (past the range: no memory access)
   int lterm = 0, ls = 0;
@@ -616,7 +627,40 @@ __global__ __launch_bounds__(F_THREADS, 2) void k_gemm_tq2f(GemmArgs a) {
 #pragma unroll
       for (int i = 0; i < 4; ++i) total[r][DT][i] += scp[r] * C[r][DT][i];
 
-    // ---- epilogue: lane holds tokens 4 kb + i of each token tile, output row n_wave + 16 r + r16
+    // ---- epilogue: lane holds tokens 4 kb + i of each token tile, output row tile_row(wave, r) + r16
+    if (glu) {  // (uniform) h = SwiGLU of the lane's gate and up sums, bf16
+#pragma unroll
+      for (int t = 0; t < TT; ++t) {
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+          const int tk = 16 * t + 4 * kb + i;
+          if (tk >= ntok) continue;
+          const int64_t tok = tok0 + tk;
+          float w = 1.f;
+          if (a.glu_v4 && a.glu_weights) w = a.glu_weights[a.glu_order ? clamp_i64(a.glu_order[tok], 0, a.glu_pairs - 1) : tok];
+#pragma unroll
+          for (int q = 0; q < 2; ++q) {
+            const int64_t col = tile_row(wave, q);
+            if (col < 0) continue;
+            float g = bf16_bits_to_f32(f32_to_bf16_bits(total[q][t][i])), u = bf16_bits_to_f32(f32_to_bf16_bits(total[q + 2][t][i]));
+            float v;
+            if (a.glu_v4) {
+              if (a.glu_limit > 0.f) {  // torch.clamp: a NaN stays a NaN
+                u = u < -a.glu_limit ? -a.glu_limit : (u > a.glu_limit ? a.glu_limit : u);
+                g = g > a.glu_limit ? a.glu_limit : g;
+              }
+              v = (g / (1.0f + expf(-g))) * u;
+              if (a.glu_weights) v = w * v;
+            } else {
+              const float sg = bf16_bits_to_f32(f32_to_bf16_bits(g / (1.0f + expf(-g))));
+              v = sg * u;
+            }
+            a.glu_h[tok * NH + col + r16] = f32_to_bf16_bits(v);
+          }
+        }
+      }
+      return;
+    }
 #pragma unroll
     for (int t = 0; t < TT; ++t) {
 #pragma unroll
@@ -626,8 +670,8 @@ __global__ __launch_bounds__(F_THREADS, 2) void k_gemm_tq2f(GemmArgs a) {
           const int64_t tok = tok0 + tk;
 #pragma unroll
           for (int r = 0; r < F_RT; ++r) {
-            const int64_t row = n_wave + 16 * r;
-            if (row < a.N) {
+            const int64_t row = tile_row(wave, r);
+            if (row >= 0) {
               float* o = a.out + tok * a.N + row + r16;
               *o = (a.overwrite ? 0.f : *o) + total[r][t][i];
             }
@@ -646,7 +690,7 @@ int launch_gemm_tq2f_g(const GemmArgs& a, hipStream_t s) {
   static_assert(LDS <= 160 * 1024, "LDS of a workgroup");
   const char* name = FMT == BP_TQ1 ? "gemm_tq1f_bf16" : "gemm_tq2f_bf16";
   if (const int rc = raise_lds_limit<k_gemm_tq2f<SDT, FMT, GS>>(LDS)) return rc;
-  const int64_t row_blocks = (a.N + F_ROWS - 1) / F_ROWS;
+  const int64_t row_blocks = a.glu_h ? (a.N / 2 + F_ROWS / 2 - 1) / (F_ROWS / 2) : (a.N + F_ROWS - 1) / F_ROWS;
   const int64_t wgs = tile_workgroups(a, row_blocks);
   if (wgs < 0) return BP_ERR_UNSUPPORTED;
   const int64_t slots = a.tiles ? a.tile_cap : a.E;
@@ -681,6 +725,7 @@ size_t gemm_tq2f_workspace_bytes(int64_t T, int64_t K, int64_t E) {
 // empty ones). BP_ERR_UNSUPPORTED (no message): the caller falls back to its other kernels.
 int launch_gemm_tq2f(const GemmArgs& a, hipStream_t s) {
   if (a.x_dtype != BP_BF16 || !a.stage || ((uintptr_t)a.stage & 15) != 0) return BP_ERR_UNSUPPORTED;
+  if (a.glu_h && (!a.tiles || !a.overwrite || a.N % 32 != 0)) return BP_ERR_UNSUPPORTED;  // (whole row tiles of either half, one launch for all of K)
   if ((size_t)a.stage_bytes < gemm_tq2f_workspace_bytes(a.T, a.K, a.E) || gemm_tq2f_workspace_bytes(a.T, a.K, a.E) == 0) return BP_ERR_UNSUPPORTED;
   if (a.K > ((int64_t)1 << 24) || a.N * a.Kp > ((int64_t)1 << 31) - 4096) return BP_ERR_UNSUPPORTED;
   if (a.fmt == BP_TQ2 && tuning().tq2g != 'f') {  // (development: BP_TUNE_TQ2G=fp4 runs this kernel wherever it can)

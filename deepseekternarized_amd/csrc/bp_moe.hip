@@ -304,9 +304,21 @@ static int moe_layer(bool v4, void* out, int out_dtype, float limit, const void*
     } else if ((rc = bp_gather_rows(p.xg, x, p.order, k, n, T, 2 * H, s)) != BP_OK) return rc;
   }
 
-  auto gemm = [&](float* o, const void* in, const uint8_t* const* packed, const void* const* scale, int64_t N, int64_t K, bool tiles) -> int {
+  // `glu`: the gate | up projection with SwiGLU in its epilogue (the grouped GEMM over converted activations writes bf16 h
+  // and no float32 gate | up rows); BP_ERR_UNSUPPORTED without a message, and nothing launched, where that kernel does
+  // not take the call.
+  auto gemm = [&](float* o, const void* in, const uint8_t* const* packed, const void* const* scale, int64_t N, int64_t K, bool tiles, bool glu) -> int {
     GemmArgs a;
     memset(&a, 0, sizeof(a));
+    if (glu) {
+      if (!tiles || act != BP_BF16 || !p.stage_bytes || kernel_policy() == 1 || tuning().glu == 'n' || tuning().tq2g == 'b') return BP_ERR_UNSUPPORTED;
+      a.glu_h = (uint16_t*)p.h;
+      a.glu_v4 = v4 ? 1 : 0;
+      a.glu_limit = limit;
+      a.glu_weights = v4 ? (const float*)weights : nullptr;
+      a.glu_order = p.order;
+      a.glu_pairs = n;
+    }
     a.out = o;
     a.x = in;
     a.offsets = p.offsets;
@@ -329,8 +341,10 @@ static int moe_layer(bool v4, void* out, int out_dtype, float limit, const void*
       if (kernel_policy() != 1 && gemm_tiles_supported(a)) {
         a.overwrite = 1;
         a.max_rows = TILE_ROWS;
+        if (glu) return launch_gemm_tq2f(a, s);
         return run_gemm(a, s);
       }
+      if (glu) return BP_ERR_UNSUPPORTED;
       a.tiles = nullptr;  // no tile kernel for this shape: the launch covers the bound (every expert up to T rows)
     }
     if (!prezeroed)
@@ -341,11 +355,16 @@ static int moe_layer(bool v4, void* out, int out_dtype, float limit, const void*
     hipLaunchKernelGGL(k_tile_list, dim3(1), dim3(1024), 0, s, p.tiles, p.tile_count, p.offsets, E, n, p.tile_cap);
     if ((rc = check_launch("tile_list")) != BP_OK) return rc;
   }
-  if ((rc = gemm(p.gu, p.xg, gate_up_packed, gate_up_scale, 2 * I, H, tiles)) != BP_OK) return rc;
-  if (v4) rc = bp_swiglu_v4(p.h, p.gu, p.gu + I, (const float*)weights, p.order, n, limit, n, I, 2 * I, s);
-  else rc = bp_swiglu_bf16(p.h, p.gu, p.gu + I, n, I, 2 * I, s);
+  rc = gemm(p.gu, p.xg, gate_up_packed, gate_up_scale, 2 * I, H, tiles, true);
+  const bool fused = rc == BP_OK;
+  if (rc == BP_ERR_UNSUPPORTED) {
+    if ((rc = gemm(p.gu, p.xg, gate_up_packed, gate_up_scale, 2 * I, H, tiles, false)) != BP_OK) return rc;
+    if (v4) rc = bp_swiglu_v4(p.h, p.gu, p.gu + I, (const float*)weights, p.order, n, limit, n, I, 2 * I, s);
+    else rc = bp_swiglu_bf16(p.h, p.gu, p.gu + I, n, I, 2 * I, s);
+  }
   if (rc != BP_OK) return rc;
-  if ((rc = gemm(p.y, p.h, down_packed, down_scale, H, I, tiles)) != BP_OK) return rc;
+  if ((rc = gemm(p.y, p.h, down_packed, down_scale, H, I, tiles, false)) != BP_OK) return rc;
+  if (fused) note_kernel_suffix("+glu");  // (bp_last_kernel: the down projection's kernel, and that the gate | up one applied SwiGLU)
   if (v4) return bp_moe_combine_v4(out, out_dtype, p.y, p.inv, experts, T, k, H, s);
   return bp_moe_combine_bf16(out, p.y, p.inv, weights, experts, T, k, H, s);
 }

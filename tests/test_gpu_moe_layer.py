@@ -92,7 +92,7 @@ def test_layer_call_over_the_tile_list_with_converted_activations(tune):
     logits[:, 11] -= 2.5
     tune("BP_TUNE_TQ2G", "fp4")
     got = moe(x, logits).clone()
-    assert ext().last_kernel() == "gemm_tq2f_bf16", ext().last_kernel()
+    assert ext().last_kernel() == "gemm_tq2f_bf16+glu", ext().last_kernel()  # (the gate | up launch applied SwiGLU itself)
     assert torch.equal(moe(x, logits), got)
     tune("BP_TUNE_TQ2G", "bf16")
     want = moe(x, logits)
@@ -213,6 +213,41 @@ def test_v4_layer_matches_the_reference_lines(fmt, terms, act, T, limit):
         assert not torch.equal(free, got)
     with pytest.raises(RuntimeError):
         moe(xd, torch.zeros(T, E, device="cuda"))
+
+
+@pytest.mark.parametrize("pattern,limit", [("standard", 0.0), ("v4", 0.0), ("v4", 0.75)])
+@pytest.mark.parametrize("fmt,terms,I", [("tq1", 1, 1024), ("tq2", 2, 1280), ("tq1", 2, 768 + 512)])
+def test_swiglu_in_the_gate_up_epilogue_equals_the_separate_launch(tune, fmt, terms, I, pattern, limit):
+    """Over the tile list with converted activations the gate | up launch applies SwiGLU to its own float32 sums and writes
+    bf16 h (boilerplate/engine/standard.py:151-176, boilerplate/engine/model.py:376-387): the same sums, the same
+    rounding points - bit-identical to the layer with the separate SwiGLU launch (BP_TUNE_GLU=n), for both call patterns.
+    Skewed routing: an expert without rows, ragged last tiles, tiles of at most 16 rows."""
+    from deepseekternarized_amd import ext
+    from deepseekternarized_amd.moe import TernaryMoE
+
+    H, E, k, T = 1024, 16, 2, 200
+    _, mats = _layer(fmt, "bf16", H, I, E, k, terms=terms, seed=I + terms)
+    moe = TernaryMoE(*mats, H, I, k, fmt, 128, act="bf16", pattern=pattern, **({"swiglu_limit": limit} if pattern == "v4" else {}))
+    g = torch.Generator(device="cuda").manual_seed(9)
+    x = torch.randn(T, H, device="cuda", generator=g).to(torch.bfloat16)
+    logits = torch.randn(T, E, device="cuda", generator=g)
+    logits[:, 0] += 4.0
+    logits[:, 9] = -40.0
+    logits[:, 11] -= 2.5
+    if pattern == "v4":
+        scores = torch.softmax(logits.float(), -1)
+        w, idx = torch.topk(scores, k, dim=-1)
+        run = lambda: moe.routed(x, w * 2.5, idx).clone()
+    else:
+        run = lambda: moe(x, logits).clone()
+    if fmt == "tq2":
+        tune("BP_TUNE_TQ2G", "fp4")  # (the shape is below the thresholds of the kernel over converted activations)
+    fused = run()
+    assert ext().last_kernel() == "gemm_%sf_bf16+glu" % fmt, ext().last_kernel()
+    tune("BP_TUNE_GLU", "n")
+    apart = run()
+    assert ext().last_kernel() == "gemm_%sf_bf16" % fmt, ext().last_kernel()
+    assert torch.isfinite(fused.float()).all() and torch.equal(fused, apart)
 
 
 def test_v4_stages_bit_exact():
@@ -358,6 +393,6 @@ def test_small_batch_preparation_kernel_writes_the_tile_list(T, E, k):
     if E == 4:
         logits[:, 1] += 6.0  # expert 1 is in every token's top-2: more than one tile
     got = moe(x, logits)
-    assert ext().last_kernel() == "gemm_tq1f_bf16", ext().last_kernel()
+    assert ext().last_kernel() == "gemm_tq1f_bf16+glu", ext().last_kernel()
     want = moe.composed(x, logits)
     assert torch.isfinite(got.float()).all() and torch.equal(got, want)
