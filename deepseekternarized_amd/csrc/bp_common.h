@@ -41,6 +41,10 @@ struct GemmArgs {
   // the N output rows are N / 2 gate rows followed by N / 2 up rows, and the kernel writes bf16 glu_h[T, N / 2] instead
   // of `out`, with the rounding points of bp_swiglu_bf16 (glu_v4 = 0) or of bp_swiglu_v4 (glu_v4 = 1: clamp by glu_limit
   // when positive, float32 product times glu_weights[glu_order[row]] when glu_weights is set, one rounding to bf16).
+  // Row gather in the conversion pass of that kernel (x_index != NULL): row r of the launch is row
+  // x_index[r] / x_div of x, which has x_rows rows (the routed copy of the activations is never materialised).
+  const int64_t* x_index;
+  int64_t x_div, x_rows;
   uint16_t* glu_h;
   int glu_v4;
   float glu_limit;
@@ -110,7 +114,7 @@ struct Tuning {
   int f4t;     // BP_TUNE_F4T: routed rows per expert up to which launches of 8 rows are used (-1 = default)
   int cpt;     // BP_TUNE_CPT: chunks per table pass of the table-lookup GEMV
   int tiles;   // BP_TUNE_TILES: tokens from which bp_moe_layer_* runs its GEMMs over the device-side list of token tiles (-1 = default)
-  char glu;    // BP_TUNE_GLU: 'n' bp_moe_layer_* never lets the gate | up GEMM apply SwiGLU itself (a launch of its own instead)
+  char glu;    // BP_TUNE_GLU: 'n' bp_moe_layer_* never lets the gate | up GEMM apply SwiGLU itself (a launch of its own instead), 'g' it does but the row gather stays a launch of its own
 };
 const Tuning& tuning();
 

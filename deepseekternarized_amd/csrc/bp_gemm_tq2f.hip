@@ -114,7 +114,9 @@ __global__ __launch_bounds__(F_THREADS) void k_stage_tq2f(GemmArgs a) {
   }
   int srow = 16 * stt + sm;
   if (srow >= ntok) srow = ntok - 1;  // rows past the expert's tokens repeat its last one (their results are not stored)
-  const uint16_t* xp = (const uint16_t*)a.x + (tok0 + srow) * a.K + 256 * (int64_t)s + 128 * sg + 64 * (kbA >> 1) + 32 * hi + 16 * (kbA & 1);
+  int64_t xrow = tok0 + srow;
+  if (a.x_index) xrow = clamp_i64(a.x_index[xrow] / a.x_div, 0, a.x_rows - 1);  // (the routed row's token)
+  const uint16_t* xp = (const uint16_t*)a.x + xrow * a.K + 256 * (int64_t)s + 128 * sg + 64 * (kbA >> 1) + 32 * hi + 16 * (kbA & 1);
   const u32x4 raw[2] = {*(const u32x4*)xp, *(const u32x4*)(xp + 8)};
   float y[16];
 #pragma unroll
@@ -723,7 +725,7 @@ size_t gemm_tq2f_workspace_bytes(int64_t T, int64_t K, int64_t E) {
 // per activation: bp_gemm_tq2.hip); offsets into an expert's rows fit 32 bits; a launch whose token tiles mostly exist
 // (the conversion runs one workgroup per tile and window: a loose bound on the rows per expert would launch mostly
 // empty ones). BP_ERR_UNSUPPORTED (no message): the caller falls back to its other kernels.
-int launch_gemm_tq2f(const GemmArgs& a, hipStream_t s) {
+int gemm_tq2f_applies(const GemmArgs& a) {
   if (a.x_dtype != BP_BF16 || !a.stage || ((uintptr_t)a.stage & 15) != 0) return BP_ERR_UNSUPPORTED;
   if (a.glu_h && (!a.tiles || !a.overwrite || a.N % 32 != 0)) return BP_ERR_UNSUPPORTED;  // (whole row tiles of either half, one launch for all of K)
   if ((size_t)a.stage_bytes < gemm_tq2f_workspace_bytes(a.T, a.K, a.E) || gemm_tq2f_workspace_bytes(a.T, a.K, a.E) == 0) return BP_ERR_UNSUPPORTED;
@@ -741,6 +743,15 @@ int launch_gemm_tq2f(const GemmArgs& a, hipStream_t s) {
     if (a.Kp != (a.K + 4) / 5 || a.scale_dtype == BP_F32) return BP_ERR_UNSUPPORTED;
     for (int t = 1; t < a.n_terms; ++t)  // (one byte alignment of the rows for all terms)
       if ((((uintptr_t)a.packed[t] ^ (uintptr_t)a.packed[0]) & 3) != 0) return BP_ERR_UNSUPPORTED;
+  }
+  const int64_t row_blocks = a.glu_h ? (a.N / 2 + F_ROWS / 2 - 1) / (F_ROWS / 2) : (a.N + F_ROWS - 1) / F_ROWS;
+  if (tile_workgroups(a, row_blocks) < 0) return BP_ERR_UNSUPPORTED;
+  return BP_OK;
+}
+
+int launch_gemm_tq2f(const GemmArgs& a, hipStream_t s) {
+  if (const int rc = gemm_tq2f_applies(a)) return rc;
+  if (a.fmt == BP_TQ1) {
     if (a.scale_dtype == BP_F16) return launch_gemm_tq2f_k<BP_F16, BP_TQ1>(a, s);
     return launch_gemm_tq2f_k<BP_BF16, BP_TQ1>(a, s);  // (float32 scales: the table, the transit area and their ring do not fit in LDS together)
   }

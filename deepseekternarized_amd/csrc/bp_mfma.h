@@ -25,6 +25,7 @@ int launch_mfma_tq1(const GemmArgs& a, hipStream_t s, int waves);
 // bp_gemm_tq2.hip: TQ2 with token tiles of 32 (experts with more than 16 token rows)
 int launch_gemm_tq2(const GemmArgs& a, hipStream_t s);
 int launch_gemm_tq2f(const GemmArgs& a, hipStream_t s);
+int gemm_tq2f_applies(const GemmArgs& a);  // BP_OK where launch_gemm_tq2f takes the call (nothing is launched)
 // bp_gemm_tq1.hip: TQ1 with token tiles of 32 on the fp8 x fp4 matrix instruction (experts with more than 8 token rows);
 // BP_ERR_UNSUPPORTED without a message when the call is outside its preconditions
 int launch_gemm_tq1(const GemmArgs& a, hipStream_t s);

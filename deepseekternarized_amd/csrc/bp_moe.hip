@@ -284,6 +284,29 @@ static int moe_layer(bool v4, void* out, int out_dtype, float limit, const void*
   const bool small = n <= ROUTE_SMALL_N && (((uintptr_t)x | (uintptr_t)p.xg) & 15) == 0;
   const bool aligned16 = (((uintptr_t)x | (uintptr_t)p.xg) & 15) == 0;
   const bool prezeroed = aligned16 && !tiles;  // the zero-fill rides along with the gather (the GEMMs over the tile list write instead of accumulate)
+  // The gate | up projection as the grouped GEMM over converted activations with SwiGLU in its epilogue (bf16 h written,
+  // no float32 gate | up rows), where that kernel takes the call: over the tile list, bf16 activations. Its conversion
+  // pass then also does the row gather (rows read through `order`), unless the preparation kernel of small batches has
+  // done it anyway.
+  GemmArgs fused;
+  memset(&fused, 0, sizeof(fused));
+  bool fuse = false;
+  if (tiles && act == BP_BF16 && p.stage_bytes && kernel_policy() != 1 && tuning().glu != 'n' && tuning().tq2g != 'b') {
+    GemmArgs& a = fused;
+    a.out = p.gu; a.x = p.xg; a.offsets = p.offsets; a.x_dtype = act;
+    for (int t = 0; t < n_terms; ++t) { a.packed[t] = gate_up_packed[t]; a.w_scale[t] = gate_up_scale[t]; }
+    a.scale_dtype = scale_dtype; a.n_terms = n_terms; a.fmt = fmt;
+    a.T = n; a.N = 2 * I; a.K = H; a.Kp = (H + per - 1) / per; a.G = (H + group - 1) / group; a.group = group; a.E = E;
+    a.stage = p.stage; a.stage_bytes = (int64_t)p.stage_bytes;
+    a.tiles = p.tiles; a.tile_count = p.tile_count; a.tile_cap = p.tile_cap;
+    a.overwrite = 1; a.max_rows = TILE_ROWS;
+    a.glu_h = (uint16_t*)p.h; a.glu_v4 = v4 ? 1 : 0; a.glu_limit = limit;
+    a.glu_weights = v4 ? (const float*)weights : nullptr; a.glu_order = p.order; a.glu_pairs = n;
+    if (!small && aligned16 && tuning().glu != 'g') {  // (development: BP_TUNE_GLU=g keeps the gather a launch of its own)
+      a.x = x; a.x_index = p.order; a.x_div = k; a.x_rows = T;
+    }
+    fuse = gemm_tiles_supported(a) && gemm_tq2f_applies(a) == BP_OK;
+  }
   if (small) {
     const int64_t z0 = prezeroed ? (int64_t)(4 * (size_t)n * 2 * I / 16) : 0, z1 = prezeroed ? (int64_t)(4 * (size_t)n * H / 16) : 0;
     int64_t g = (z0 + z1 + (int64_t)n * (H / 8) + ROUTE_SMALL_THREADS - 1) / ROUTE_SMALL_THREADS;
@@ -294,7 +317,9 @@ static int moe_layer(bool v4, void* out, int out_dtype, float limit, const void*
     if ((rc = check_launch("route_small")) != BP_OK) return rc;
   } else {
     if ((rc = sort_with_inverse(p.order, p.offsets, p.inv, experts, n, E, p.sort_ws, bad, s)) != BP_OK) return rc;
-    if (aligned16) {
+    if (fuse && fused.x_index) {
+      // (no routed copy of the activations: the gate | up launch's conversion pass reads them through `order`)
+    } else if (aligned16) {
       const int64_t z0 = prezeroed ? (int64_t)(4 * (size_t)n * 2 * I / 16) : 0, z1 = prezeroed ? (int64_t)(4 * (size_t)n * H / 16) : 0;
       int64_t g = (z0 + z1 + n * (H / 8) + 255) / 256;
       g = g < 1 ? 1 : (g > 4096 ? 4096 : g);
@@ -304,21 +329,9 @@ static int moe_layer(bool v4, void* out, int out_dtype, float limit, const void*
     } else if ((rc = bp_gather_rows(p.xg, x, p.order, k, n, T, 2 * H, s)) != BP_OK) return rc;
   }
 
-  // `glu`: the gate | up projection with SwiGLU in its epilogue (the grouped GEMM over converted activations writes bf16 h
-  // and no float32 gate | up rows); BP_ERR_UNSUPPORTED without a message, and nothing launched, where that kernel does
-  // not take the call.
-  auto gemm = [&](float* o, const void* in, const uint8_t* const* packed, const void* const* scale, int64_t N, int64_t K, bool tiles, bool glu) -> int {
+  auto gemm = [&](float* o, const void* in, const uint8_t* const* packed, const void* const* scale, int64_t N, int64_t K, bool tiles) -> int {
     GemmArgs a;
     memset(&a, 0, sizeof(a));
-    if (glu) {
-      if (!tiles || act != BP_BF16 || !p.stage_bytes || kernel_policy() == 1 || tuning().glu == 'n' || tuning().tq2g == 'b') return BP_ERR_UNSUPPORTED;
-      a.glu_h = (uint16_t*)p.h;
-      a.glu_v4 = v4 ? 1 : 0;
-      a.glu_limit = limit;
-      a.glu_weights = v4 ? (const float*)weights : nullptr;
-      a.glu_order = p.order;
-      a.glu_pairs = n;
-    }
     a.out = o;
     a.x = in;
     a.offsets = p.offsets;
@@ -341,10 +354,8 @@ static int moe_layer(bool v4, void* out, int out_dtype, float limit, const void*
       if (kernel_policy() != 1 && gemm_tiles_supported(a)) {
         a.overwrite = 1;
         a.max_rows = TILE_ROWS;
-        if (glu) return launch_gemm_tq2f(a, s);
         return run_gemm(a, s);
       }
-      if (glu) return BP_ERR_UNSUPPORTED;
       a.tiles = nullptr;  // no tile kernel for this shape: the launch covers the bound (every expert up to T rows)
     }
     if (!prezeroed)
@@ -355,16 +366,16 @@ static int moe_layer(bool v4, void* out, int out_dtype, float limit, const void*
     hipLaunchKernelGGL(k_tile_list, dim3(1), dim3(1024), 0, s, p.tiles, p.tile_count, p.offsets, E, n, p.tile_cap);
     if ((rc = check_launch("tile_list")) != BP_OK) return rc;
   }
-  rc = gemm(p.gu, p.xg, gate_up_packed, gate_up_scale, 2 * I, H, tiles, true);
-  const bool fused = rc == BP_OK;
-  if (rc == BP_ERR_UNSUPPORTED) {
-    if ((rc = gemm(p.gu, p.xg, gate_up_packed, gate_up_scale, 2 * I, H, tiles, false)) != BP_OK) return rc;
+  if (fuse) {
+    rc = launch_gemm_tq2f(fused, s);
+  } else {
+    if ((rc = gemm(p.gu, p.xg, gate_up_packed, gate_up_scale, 2 * I, H, tiles)) != BP_OK) return rc;
     if (v4) rc = bp_swiglu_v4(p.h, p.gu, p.gu + I, (const float*)weights, p.order, n, limit, n, I, 2 * I, s);
     else rc = bp_swiglu_bf16(p.h, p.gu, p.gu + I, n, I, 2 * I, s);
   }
   if (rc != BP_OK) return rc;
-  if ((rc = gemm(p.y, p.h, down_packed, down_scale, H, I, tiles, false)) != BP_OK) return rc;
-  if (fused) note_kernel_suffix("+glu");  // (bp_last_kernel: the down projection's kernel, and that the gate | up one applied SwiGLU)
+  if ((rc = gemm(p.y, p.h, down_packed, down_scale, H, I, tiles)) != BP_OK) return rc;
+  if (fuse) note_kernel_suffix(fused.x_index ? "+glu+gather" : "+glu");  // (bp_last_kernel: the down projection's kernel, and that the gate | up one applied SwiGLU)
   if (v4) return bp_moe_combine_v4(out, out_dtype, p.y, p.inv, experts, T, k, H, s);
   return bp_moe_combine_bf16(out, p.y, p.inv, weights, experts, T, k, H, s);
 }

@@ -92,7 +92,7 @@ def test_layer_call_over_the_tile_list_with_converted_activations(tune):
     logits[:, 11] -= 2.5
     tune("BP_TUNE_TQ2G", "fp4")
     got = moe(x, logits).clone()
-    assert ext().last_kernel() == "gemm_tq2f_bf16+glu", ext().last_kernel()  # (the gate | up launch applied SwiGLU itself)
+    assert ext().last_kernel() == "gemm_tq2f_bf16+glu+gather", ext().last_kernel()  # (the gate | up launch gathered its rows and applied SwiGLU itself)
     assert torch.equal(moe(x, logits), got)
     tune("BP_TUNE_TQ2G", "bf16")
     want = moe(x, logits)
@@ -218,8 +218,8 @@ def test_v4_layer_matches_the_reference_lines(fmt, terms, act, T, limit):
 @pytest.mark.parametrize("pattern,limit", [("standard", 0.0), ("v4", 0.0), ("v4", 0.75)])
 @pytest.mark.parametrize("fmt,terms,I", [("tq1", 1, 1024), ("tq2", 2, 1280), ("tq1", 2, 768 + 512)])
 def test_swiglu_in_the_gate_up_epilogue_equals_the_separate_launch(tune, fmt, terms, I, pattern, limit):
-    """Over the tile list with converted activations the gate | up launch applies SwiGLU to its own float32 sums and writes
-    bf16 h (boilerplate/engine/standard.py:151-176, boilerplate/engine/model.py:376-387): the same sums, the same
+    """Over the tile list with converted activations the gate | up launch reads its rows through the sort order (no routed
+    copy of the activations), applies SwiGLU to its own float32 sums and writes bf16 h (boilerplate/engine/standard.py:151-176, boilerplate/engine/model.py:376-387): the same sums, the same
     rounding points - bit-identical to the layer with the separate SwiGLU launch (BP_TUNE_GLU=n), for both call patterns.
     Skewed routing: an expert without rows, ragged last tiles, tiles of at most 16 rows."""
     from deepseekternarized_amd import ext
@@ -243,6 +243,9 @@ def test_swiglu_in_the_gate_up_epilogue_equals_the_separate_launch(tune, fmt, te
     if fmt == "tq2":
         tune("BP_TUNE_TQ2G", "fp4")  # (the shape is below the thresholds of the kernel over converted activations)
     fused = run()
+    assert ext().last_kernel() == "gemm_%sf_bf16+glu+gather" % fmt, ext().last_kernel()
+    tune("BP_TUNE_GLU", "g")  # the routed copy of the activations written by a launch of its own
+    assert torch.equal(run(), fused)
     assert ext().last_kernel() == "gemm_%sf_bf16+glu" % fmt, ext().last_kernel()
     tune("BP_TUNE_GLU", "n")
     apart = run()
