@@ -299,6 +299,46 @@ def cfg2_moe(bp, torch):
     return moe, layer_bytes, (H2, I2, E2, k2)
 
 
+def cfg3_moe(bp, torch, gate=None):
+    """One routed-expert layer of config 3 (TQ2, two stacked terms, H=4096, I=2048, 384 experts, top-6, bf16 activations)
+    as a TernaryMoE with 2048 tokens of input; `gate`: (packed, scales) of the gate projection if the caller has them."""
+    from deepseekternarized_amd.moe import TernaryMoE
+
+    E3, I3, H3, T3, k3 = 384, 2048, 4096, 2048, 6
+    packed, scales = gate if gate is not None else synth(bp, torch, E3, I3, H3, "tq2", 2, seed=3)
+    up3 = synth(bp, torch, E3, I3, H3, "tq2", 2, seed=4)
+    down3 = synth(bp, torch, E3, H3, I3, "tq2", 2, seed=5)
+    moe3 = TernaryMoE(list(zip(packed, scales)), list(zip(*up3)), list(zip(*down3)), H3, I3, k3, "tq2", GROUP, act="bf16")
+    g3 = torch.Generator(device="cuda").manual_seed(9)
+    x3 = torch.randn(T3, H3, device="cuda", generator=g3).to(torch.bfloat16)
+    lg3 = torch.randn(T3, E3, device="cuda", generator=g3) * 1.5
+    fl3 = 2.0 * T3 * k3 * 3 * H3 * I3 * 2  # per-term count, three projections
+    desc = (f"TQ2 k=2 MoE layer H={H3} I={I3} E={E3} top-{k3}, {T3} tokens, bf16 activations: softmax/top-k, "
+            "sort, gate|up grouped GEMM (row gather in its conversion pass, SwiGLU in its epilogue), down grouped GEMM, weighted combine")
+    return moe3, x3, lg3, fl3, desc
+
+
+def run_cfg3_moe(bp, torch, a) -> int:
+    moe3, x3, lg3, fl3, desc = cfg3_moe(bp, torch)
+    t_end = time.perf_counter() + SPIN_UP_S
+    while time.perf_counter() < t_end:
+        moe3(x3, lg3)
+        torch.cuda.synchronize()
+    dt = wall_per_call(torch, lambda: moe3(x3, lg3), a.steps, a.warmup)
+    kname = bp.ext().last_kernel()
+    return emit({
+        "metric": "ternary GEMV HBM GB/s (% peak); grouped-expert GEMM TFLOP/s (% MFMA peak)",
+        "value": round(fl3 / dt / 1e12, 1), "unit": "TFLOP/s", "n_gpus": 1, "steps": a.steps, "warmup": a.warmup,
+        "ms_per_step": round(dt * 1e3, 5), "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+        "dtype": "bf16", "data": "synthetic",
+        "config": {"workload": "cfg3_moe: " + desc, "kernel": kname, "arithmetic": arithmetic_of(kname.split("+")[0]),
+                   "flops_counted": "2 x routed rows x N x K per term (two terms), three projections", "device_spin_up_s": SPIN_UP_S},
+        "roofline": {"bound": "mfma", "achieved": round(fl3 / dt / 1e12, 1), "peak": MFMA_BF16_PEAK_TFLOPS, "unit": "TFLOP/s",
+                     "frac": round(fl3 / dt / 1e12 / MFMA_BF16_PEAK_TFLOPS, 4), "traffic": None, "layer_us": round(dt * 1e6, 2),
+                     "note": "whole layer (seven launches) by wall clock, not one kernel"},
+        "cpu_baseline": None, "also": {}})
+
+
 def emit(line) -> int:
     print(json.dumps(line))
     return 0
@@ -341,7 +381,7 @@ def run_cfg2_moe(bp, torch, a, T2) -> int:
         "ms_per_step": round(dt * 1e3, 5), "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
         "dtype": "bf16", "data": "synthetic",
         "config": {"workload": f"cfg2_moe_T{T2}: TQ1 MoE layer H={H2} I={I2} E={E2} top-{k2}, {T2} tokens, bf16 activations: softmax/top-k, sort, "
-                               f"gather, gate|up grouped GEMM, SwiGLU, down grouped GEMM, weighted combine; {active} active experts",
+                               f"gather, gate|up grouped GEMM, SwiGLU, down grouped GEMM, weighted combine (beyond 24 tokens the gate|up launch gathers its rows and applies SwiGLU itself); {active} active experts",
                    "kernel": kname, "arithmetic": arithmetic_of(kname), "bytes_counted": "packed + fp16 scales of the active experts",
                    "device_spin_up_s": SPIN_UP_S},
         "roofline": {"bound": "hbm", "achieved": round(abytes / dt / 1e9, 1), "peak": HBM_PEAK_GBPS, "unit": "GB/s",
@@ -382,7 +422,7 @@ def main() -> int:
     ap.add_argument("--steps", type=int, default=200)
     ap.add_argument("--warmup", type=int, default=20)
     ap.add_argument("--spin-up", type=float, default=SPIN_UP_S, help="seconds of untimed launches before warm-up and timed steps (0: none, for counter runs)")
-    ap.add_argument("--workload", default="cfg1a_tq1_gemv", choices=sorted(WORKLOADS) + ["cfg3_grouped", "cfg2_moe_T1", "cfg2_moe_T32", "cfg2_moe_T256", "cfg4_decode", "cfg4_decode_graph"])
+    ap.add_argument("--workload", default="cfg1a_tq1_gemv", choices=sorted(WORKLOADS) + ["cfg3_grouped", "cfg3_moe", "cfg2_moe_T1", "cfg2_moe_T32", "cfg2_moe_T256", "cfg4_decode", "cfg4_decode_graph"])
     ap.add_argument("--no-extras", action="store_true", help="skip the secondary measurements")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline")
     ap.add_argument("--calibrate-copy", action="store_true",
@@ -411,6 +451,8 @@ def main() -> int:
     SPIN_UP_S = max(0.0, a.spin_up)
     if a.workload == "cfg3_grouped":
         return run_cfg3_grouped(bp, torch, a)
+    if a.workload == "cfg3_moe":
+        return run_cfg3_moe(bp, torch, a)
     if a.workload.startswith("cfg2_moe_T"):
         return run_cfg2_moe(bp, torch, a, int(a.workload[len("cfg2_moe_T"):]))
     if a.workload.startswith("cfg4_decode"):
@@ -480,20 +522,10 @@ def main() -> int:
                                 "weight_GBps": round(wb3 / k3t / 1e9, 1), "kernel": kn3, "us": round(k3t * 1e6, 1), "us_median": l3.spread["median"]}
         del l3
         # ... and the whole routed-expert layer of config 3 (gate | up, SwiGLU, down, combine) on the same gate stack
-        from deepseekternarized_amd.moe import TernaryMoE
-
-        H3, I3 = K3, N3
-        up3 = synth(bp, torch, E3, I3, H3, "tq2", 2, seed=4)
-        down3 = synth(bp, torch, E3, H3, I3, "tq2", 2, seed=5)
-        moe3 = TernaryMoE(list(zip(packed, scales)), list(zip(*up3)), list(zip(*down3)), H3, I3, k3, "tq2", GROUP, act="bf16")
-        del packed, scales, up3, down3
-        g3 = torch.Generator(device="cuda").manual_seed(9)
-        x3 = torch.randn(T3, H3, device="cuda", generator=g3).to(torch.bfloat16)
-        lg3 = torch.randn(T3, E3, device="cuda", generator=g3) * 1.5
-        dt3 = wall_per_call(torch, lambda: moe3(x3, lg3), 5, 2)
-        fl3 = 2.0 * T3 * k3 * 3 * H3 * I3 * 2  # per-term count, three projections
-        also["cfg3_moe_layer"] = {"workload": f"TQ2 k=2 MoE layer H={H3} I={I3} E={E3} top-{k3}, {T3} tokens, bf16 activations: softmax/top-k, "
-                                              "sort, gather, gate|up grouped GEMM, SwiGLU, down grouped GEMM, weighted combine",
+        moe3, x3, lg3, fl3, desc3m = cfg3_moe(bp, torch, gate=(packed, scales))
+        del packed, scales
+        dt3 = wall_per_call(torch, lambda: moe3(x3, lg3), 10, 3)
+        also["cfg3_moe_layer"] = {"workload": desc3m, "kernel": bp.ext().last_kernel(),
                                   "ms_per_layer": round(dt3 * 1e3, 3), "TFLOPs_per_term_count": round(fl3 / dt3 / 1e12, 1),
                                   "frac_of_bf16_mfma_peak": round(fl3 / dt3 / 1e12 / MFMA_BF16_PEAK_TFLOPS, 4)}
         del moe3, x3, lg3
