@@ -45,6 +45,7 @@ struct GemmArgs {
   // x_index[r] / x_div of x, which has x_rows rows (the routed copy of the activations is never materialised).
   const int64_t* x_index;
   int64_t x_div, x_rows;
+  uint16_t* out16;  // (the same kernel, tile-list mode with overwrite) bf16 out16[T, N] is written instead of float32 `out`
   uint16_t* glu_h;
   int glu_v4;
   float glu_limit;

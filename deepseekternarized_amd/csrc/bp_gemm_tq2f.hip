@@ -674,8 +674,12 @@ __global__ __launch_bounds__(F_THREADS, 2) void k_gemm_tq2f(GemmArgs a) {
           for (int r = 0; r < F_RT; ++r) {
             const int64_t row = tile_row(wave, r);
             if (row >= 0) {
-              float* o = a.out + tok * a.N + row + r16;
-              *o = (a.overwrite ? 0.f : *o) + total[r][t][i];
+              if (a.out16) {
+                a.out16[tok * a.N + row + r16] = f32_to_bf16_bits(total[r][t][i]);
+              } else {
+                float* o = a.out + tok * a.N + row + r16;
+                *o = (a.overwrite ? 0.f : *o) + total[r][t][i];
+              }
             }
           }
         }
@@ -728,6 +732,7 @@ size_t gemm_tq2f_workspace_bytes(int64_t T, int64_t K, int64_t E) {
 int gemm_tq2f_applies(const GemmArgs& a) {
   if (a.x_dtype != BP_BF16 || !a.stage || ((uintptr_t)a.stage & 15) != 0) return BP_ERR_UNSUPPORTED;
   if (a.glu_h && (!a.tiles || !a.overwrite || a.N % 32 != 0)) return BP_ERR_UNSUPPORTED;  // (whole row tiles of either half, one launch for all of K)
+  if (a.out16 && (!a.tiles || !a.overwrite)) return BP_ERR_UNSUPPORTED;
   if ((size_t)a.stage_bytes < gemm_tq2f_workspace_bytes(a.T, a.K, a.E) || gemm_tq2f_workspace_bytes(a.T, a.K, a.E) == 0) return BP_ERR_UNSUPPORTED;
   if (a.K > ((int64_t)1 << 24) || a.N * a.Kp > ((int64_t)1 << 31) - 4096) return BP_ERR_UNSUPPORTED;
   if (a.fmt == BP_TQ2 && tuning().tq2g != 'f') {  // (development: BP_TUNE_TQ2G=fp4 runs this kernel wherever it can)

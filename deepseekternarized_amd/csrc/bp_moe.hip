@@ -18,6 +18,10 @@ namespace bp {
 int kernel_policy();  // bp_api.hip
 int sort_with_inverse(int64_t* order, int64_t* offsets, int64_t* inv, const int64_t* ids, int64_t n, int64_t E, int32_t* workspace,
                       int32_t* bad, hipStream_t stream);  // bp_route.hip
+int moe_combine(void* out, const void* y, bool y16, const int64_t* inv, const void* w, const int64_t* experts, int64_t T, int64_t k, int64_t H,
+                void* stream);  // bp_route.hip
+int moe_combine_v4(void* out, int out_dtype, const void* y, bool y16, const int64_t* inv, const int64_t* experts, int64_t T, int64_t k, int64_t H,
+                   void* stream);
 namespace {
 
 constexpr int TILE_ROWS = 32;  // token tile of k_gemm_tq1 / k_gemm_tq2
@@ -329,7 +333,11 @@ static int moe_layer(bool v4, void* out, int out_dtype, float limit, const void*
     } else if ((rc = bp_gather_rows(p.xg, x, p.order, k, n, T, 2 * H, s)) != BP_OK) return rc;
   }
 
-  auto gemm = [&](float* o, const void* in, const uint8_t* const* packed, const void* const* scale, int64_t N, int64_t K, bool tiles) -> int {
+  // `o16`: the caller takes bf16 rows (the combine rounds the down projection's rows to bf16 first); set to whether
+  // the launch wrote them - the grouped GEMM over converted activations does, into the same buffer.
+  auto gemm = [&](float* o, const void* in, const uint8_t* const* packed, const void* const* scale, int64_t N, int64_t K, bool tiles, bool* o16) -> int {
+    const bool want16 = o16 && *o16;
+    if (o16) *o16 = false;
     GemmArgs a;
     memset(&a, 0, sizeof(a));
     a.out = o;
@@ -354,6 +362,14 @@ static int moe_layer(bool v4, void* out, int out_dtype, float limit, const void*
       if (kernel_policy() != 1 && gemm_tiles_supported(a)) {
         a.overwrite = 1;
         a.max_rows = TILE_ROWS;
+        if (want16 && tuning().glu != 'n' && tuning().tq2g != 'b') {
+          a.out16 = (uint16_t*)o;
+          if (gemm_tq2f_applies(a) == BP_OK) {
+            *o16 = true;
+            return launch_gemm_tq2f(a, s);
+          }
+          a.out16 = nullptr;
+        }
         return run_gemm(a, s);
       }
       a.tiles = nullptr;  // no tile kernel for this shape: the launch covers the bound (every expert up to T rows)
@@ -369,15 +385,17 @@ static int moe_layer(bool v4, void* out, int out_dtype, float limit, const void*
   if (fuse) {
     rc = launch_gemm_tq2f(fused, s);
   } else {
-    if ((rc = gemm(p.gu, p.xg, gate_up_packed, gate_up_scale, 2 * I, H, tiles)) != BP_OK) return rc;
+    if ((rc = gemm(p.gu, p.xg, gate_up_packed, gate_up_scale, 2 * I, H, tiles, nullptr)) != BP_OK) return rc;
     if (v4) rc = bp_swiglu_v4(p.h, p.gu, p.gu + I, (const float*)weights, p.order, n, limit, n, I, 2 * I, s);
     else rc = bp_swiglu_bf16(p.h, p.gu, p.gu + I, n, I, 2 * I, s);
   }
   if (rc != BP_OK) return rc;
-  if ((rc = gemm(p.y, p.h, down_packed, down_scale, H, I, tiles)) != BP_OK) return rc;
+  bool y16 = true;
+  if ((rc = gemm(p.y, p.h, down_packed, down_scale, H, I, tiles, &y16)) != BP_OK) return rc;
   if (fuse) note_kernel_suffix(fused.x_index ? "+glu+gather" : "+glu");  // (bp_last_kernel: the down projection's kernel, and that the gate | up one applied SwiGLU)
-  if (v4) return bp_moe_combine_v4(out, out_dtype, p.y, p.inv, experts, T, k, H, s);
-  return bp_moe_combine_bf16(out, p.y, p.inv, weights, experts, T, k, H, s);
+  if (y16) note_kernel_suffix("+y16");  // (... and that the down projection wrote bf16 rows)
+  if (v4) return moe_combine_v4(out, out_dtype, p.y, y16, p.inv, experts, T, k, H, s);
+  return moe_combine(out, p.y, y16, p.inv, weights, experts, T, k, H, s);
 }
 
 extern "C" int bp_moe_layer_bf16(void* out, const void* x, const int64_t* experts, const void* weights,

@@ -209,7 +209,9 @@ __global__ __launch_bounds__(256) void k_swiglu4(uint16_t* __restrict__ h, const
 // out[t, :] = bf16-accumulated sum over the token's slots in ascending expert order.
 // One workgroup per (token, 1024 columns): the slots' rows and weights are looked up once, in expert order, then
 // every thread reads its 4 columns of all k rows (independent loads) and accumulates them in that order.
+// Y16: the rows of y are bf16 already (the down projection rounded them itself: the rounding the sum starts with).
 constexpr int COMBINE_COLS = 1024;
+template <bool Y16>
 __global__ __launch_bounds__(256) void k_combine(uint16_t* __restrict__ out, const float* __restrict__ y,
                                                  const int64_t* __restrict__ inv, const uint16_t* __restrict__ w,
                                                  const int64_t* __restrict__ experts, int64_t k, int64_t H) {
@@ -236,8 +238,16 @@ __global__ __launch_bounds__(256) void k_combine(uint16_t* __restrict__ out, con
       float4 v[8];
       const int ns = k - s0 < 8 ? (int)(k - s0) : 8;
 #pragma unroll
-      for (int s = 0; s < 8; ++s)
-        if (s < ns) v[s] = *(const float4*)(y + row_of[s0 + s] * H + c0);
+      for (int s = 0; s < 8; ++s) {
+        if (s < ns) {
+          if (Y16) {
+            const uint2 b = *(const uint2*)((const uint16_t*)y + row_of[s0 + s] * H + c0);
+            v[s] = make_float4(__uint_as_float(b.x << 16), __uint_as_float(b.x & 0xffff0000u), __uint_as_float(b.y << 16), __uint_as_float(b.y & 0xffff0000u));
+          } else {
+            v[s] = *(const float4*)(y + row_of[s0 + s] * H + c0);
+          }
+        }
+      }
 #pragma unroll
       for (int s = 0; s < 8; ++s) {
         if (s < ns) {
@@ -255,7 +265,10 @@ __global__ __launch_bounds__(256) void k_combine(uint16_t* __restrict__ out, con
   }
   for (int64_t c = c0; c < H && c < c0 + 4; ++c) {
     float acc = 0.f;
-    for (int s = 0; s < k; ++s) acc = round_bf16(acc + round_bf16(round_bf16(y[row_of[s] * H + c]) * weight_of[s]));
+    for (int s = 0; s < k; ++s) {
+      const float v = Y16 ? bf16_bits_to_f32(((const uint16_t*)y)[row_of[s] * H + c]) : round_bf16(y[row_of[s] * H + c]);
+      acc = round_bf16(acc + round_bf16(v * weight_of[s]));
+    }
     out[t * H + c] = f32_to_bf16_bits(acc);
   }
 }
@@ -300,7 +313,7 @@ __global__ __launch_bounds__(256) void k_swiglu_v4(uint16_t* __restrict__ h, con
 
 // Combine of the V4 engine (boilerplate/engine/model.py:407-422): y = zeros float32; for each expert in ascending
 // order y[token] += its bf16 output (already weighted before w2). out[t] = that float32 sum (OUT_BF16: cast once).
-template <bool OUT_BF16>
+template <bool OUT_BF16, bool Y16>
 __global__ __launch_bounds__(256) void k_combine_v4(void* __restrict__ out, const float* __restrict__ y, const int64_t* __restrict__ inv,
                                                      const int64_t* __restrict__ experts, int64_t k, int64_t H) {
   const int64_t t = blockIdx.x;
@@ -318,7 +331,7 @@ __global__ __launch_bounds__(256) void k_combine_v4(void* __restrict__ out, cons
   __syncthreads();
   for (int64_t c = (int64_t)blockIdx.y * COMBINE_COLS + threadIdx.x; c < H && c < ((int64_t)blockIdx.y + 1) * COMBINE_COLS; c += 256) {
     float acc = 0.f;
-    for (int s = 0; s < k; ++s) acc += round_bf16(y[row_of[s] * H + c]);
+    for (int s = 0; s < k; ++s) acc += Y16 ? bf16_bits_to_f32(((const uint16_t*)y)[row_of[s] * H + c]) : round_bf16(y[row_of[s] * H + c]);
     if (OUT_BF16) ((uint16_t*)out)[t * H + c] = f32_to_bf16_bits(acc);
     else ((float*)out)[t * H + c] = acc;
   }
@@ -489,14 +502,43 @@ extern "C" int bp_swiglu_bf16(void* h, const float* gate, const float* up, int64
   return check_launch("swiglu");
 }
 
-extern "C" int bp_moe_combine_bf16(void* out, const float* y, const int64_t* inv, const void* w, const int64_t* experts,
-                                   int64_t T, int64_t k, int64_t H, void* stream) {
+namespace bp {
+// the two combines with rows of y that are float32 (the entry points) or bf16 already (y16: bp_moe_layer_* after a down
+// projection that wrote bf16)
+int moe_combine(void* out, const void* y, bool y16, const int64_t* inv, const void* w, const int64_t* experts, int64_t T, int64_t k, int64_t H,
+                void* stream) {
   if (T < 0 || k <= 0 || k > 64 || H <= 0 || T > 0x7fffffff) return fail(BP_ERR_ARG, "invalid combine dimensions (top-k up to 64)");
   if (T == 0) return BP_OK;
   if (!out || !y || !inv || !w || !experts) return fail(BP_ERR_ARG, "null pointer");
-  hipLaunchKernelGGL(k_combine, dim3((unsigned)T, (unsigned)((H + COMBINE_COLS - 1) / COMBINE_COLS)), dim3(256), 0, (hipStream_t)stream, (uint16_t*)out, y, inv,
-                     (const uint16_t*)w, experts, k, H);
+  const dim3 grid((unsigned)T, (unsigned)((H + COMBINE_COLS - 1) / COMBINE_COLS));
+  if (y16) hipLaunchKernelGGL(k_combine<true>, grid, dim3(256), 0, (hipStream_t)stream, (uint16_t*)out, (const float*)y, inv, (const uint16_t*)w, experts, k, H);
+  else hipLaunchKernelGGL(k_combine<false>, grid, dim3(256), 0, (hipStream_t)stream, (uint16_t*)out, (const float*)y, inv, (const uint16_t*)w, experts, k, H);
   return check_launch("moe_combine");
+}
+
+int moe_combine_v4(void* out, int out_dtype, const void* y, bool y16, const int64_t* inv, const int64_t* experts, int64_t T, int64_t k, int64_t H,
+                   void* stream) {
+  if (T < 0 || k <= 0 || k > 64 || H <= 0 || T > 0x7fffffff) return fail(BP_ERR_ARG, "invalid combine dimensions (top-k up to 64)");
+  if (out_dtype != BP_F32 && out_dtype != BP_BF16) return fail(BP_ERR_ARG, "the combined output is float32 or bf16");
+  if (T == 0) return BP_OK;
+  if (!out || !y || !inv || !experts) return fail(BP_ERR_ARG, "null pointer");
+  const dim3 grid((unsigned)T, (unsigned)((H + COMBINE_COLS - 1) / COMBINE_COLS));
+  const float* yf = (const float*)y;
+  const hipStream_t s = (hipStream_t)stream;
+  if (out_dtype == BP_BF16) {
+    if (y16) hipLaunchKernelGGL((k_combine_v4<true, true>), grid, dim3(256), 0, s, out, yf, inv, experts, k, H);
+    else hipLaunchKernelGGL((k_combine_v4<true, false>), grid, dim3(256), 0, s, out, yf, inv, experts, k, H);
+  } else {
+    if (y16) hipLaunchKernelGGL((k_combine_v4<false, true>), grid, dim3(256), 0, s, out, yf, inv, experts, k, H);
+    else hipLaunchKernelGGL((k_combine_v4<false, false>), grid, dim3(256), 0, s, out, yf, inv, experts, k, H);
+  }
+  return check_launch("moe_combine_v4");
+}
+}  // namespace bp
+
+extern "C" int bp_moe_combine_bf16(void* out, const float* y, const int64_t* inv, const void* w, const int64_t* experts,
+                                   int64_t T, int64_t k, int64_t H, void* stream) {
+  return bp::moe_combine(out, y, false, inv, w, experts, T, k, H, stream);
 }
 
 extern "C" int bp_swiglu_v4(void* h, const float* gate, const float* up, const float* weights, const int64_t* order, int64_t pairs,
@@ -513,14 +555,7 @@ extern "C" int bp_swiglu_v4(void* h, const float* gate, const float* up, const f
 
 extern "C" int bp_moe_combine_v4(void* out, int out_dtype, const float* y, const int64_t* inv, const int64_t* experts,
                                  int64_t T, int64_t k, int64_t H, void* stream) {
-  if (T < 0 || k <= 0 || k > 64 || H <= 0 || T > 0x7fffffff) return fail(BP_ERR_ARG, "invalid combine dimensions (top-k up to 64)");
-  if (out_dtype != BP_F32 && out_dtype != BP_BF16) return fail(BP_ERR_ARG, "the combined output is float32 or bf16");
-  if (T == 0) return BP_OK;
-  if (!out || !y || !inv || !experts) return fail(BP_ERR_ARG, "null pointer");
-  const dim3 grid((unsigned)T, (unsigned)((H + COMBINE_COLS - 1) / COMBINE_COLS));
-  if (out_dtype == BP_BF16) hipLaunchKernelGGL(k_combine_v4<true>, grid, dim3(256), 0, (hipStream_t)stream, out, y, inv, experts, k, H);
-  else hipLaunchKernelGGL(k_combine_v4<false>, grid, dim3(256), 0, (hipStream_t)stream, out, y, inv, experts, k, H);
-  return check_launch("moe_combine_v4");
+  return bp::moe_combine_v4(out, out_dtype, y, false, inv, experts, T, k, H, stream);
 }
 
 extern "C" int bp_route_topk(void* weights, int weights_dtype, int64_t* experts, const void* logits, int logits_dtype, int64_t T, int64_t E,

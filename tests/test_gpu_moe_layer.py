@@ -92,7 +92,7 @@ def test_layer_call_over_the_tile_list_with_converted_activations(tune):
     logits[:, 11] -= 2.5
     tune("BP_TUNE_TQ2G", "fp4")
     got = moe(x, logits).clone()
-    assert ext().last_kernel() == "gemm_tq2f_bf16+glu+gather", ext().last_kernel()  # (the gate | up launch gathered its rows and applied SwiGLU itself)
+    assert ext().last_kernel() == "gemm_tq2f_bf16+glu+gather+y16", ext().last_kernel()  # (the gate | up launch gathered its rows and applied SwiGLU itself)
     assert torch.equal(moe(x, logits), got)
     tune("BP_TUNE_TQ2G", "bf16")
     want = moe(x, logits)
@@ -243,10 +243,10 @@ def test_swiglu_in_the_gate_up_epilogue_equals_the_separate_launch(tune, fmt, te
     if fmt == "tq2":
         tune("BP_TUNE_TQ2G", "fp4")  # (the shape is below the thresholds of the kernel over converted activations)
     fused = run()
-    assert ext().last_kernel() == "gemm_%sf_bf16+glu+gather" % fmt, ext().last_kernel()
+    assert ext().last_kernel() == "gemm_%sf_bf16+glu+gather+y16" % fmt, ext().last_kernel()
     tune("BP_TUNE_GLU", "g")  # the routed copy of the activations written by a launch of its own
     assert torch.equal(run(), fused)
-    assert ext().last_kernel() == "gemm_%sf_bf16+glu" % fmt, ext().last_kernel()
+    assert ext().last_kernel() == "gemm_%sf_bf16+glu+y16" % fmt, ext().last_kernel()
     tune("BP_TUNE_GLU", "n")
     apart = run()
     assert ext().last_kernel() == "gemm_%sf_bf16" % fmt, ext().last_kernel()
@@ -396,6 +396,6 @@ def test_small_batch_preparation_kernel_writes_the_tile_list(T, E, k):
     if E == 4:
         logits[:, 1] += 6.0  # expert 1 is in every token's top-2: more than one tile
     got = moe(x, logits)
-    assert ext().last_kernel() == "gemm_tq1f_bf16+glu", ext().last_kernel()
+    assert ext().last_kernel() == "gemm_tq1f_bf16+glu+y16", ext().last_kernel()
     want = moe.composed(x, logits)
     assert torch.isfinite(got.float()).all() and torch.equal(got, want)
