@@ -339,6 +339,147 @@ def run_cfg3_moe(bp, torch, a) -> int:
         "cpu_baseline": None, "also": {}})
 
 
+def huffman_stream(torch, n, seed=0, repeat=1):
+    """A Mode B stream of n symbols made here with numpy (the package has the decoder only): a skewed byte distribution
+    under a canonical code of lengths 2 / 4 / 6 / 8 / 12, MSB first, codes back to back, a bit offset per block of 4096
+    symbols (boilerplate/kernels/csrc/boilerplate_cpu.cpp:133-167)."""
+    import numpy as np
+
+    from deepseekternarized_amd import entropy
+
+    lens = np.full(256, 12, np.uint8)
+    lens[:2], lens[2:6], lens[6:14], lens[14:30] = 2, 4, 6, 8
+    codes = entropy.canonical_codes(torch.from_numpy(lens)).numpy().astype(np.int64)
+    p = 2.0 ** -lens.astype(np.float64)
+    rng = np.random.default_rng(seed)
+    sym = rng.choice(256, size=n, p=p / p.sum()).astype(np.uint8)
+    L = lens[sym].astype(np.int64)
+    if repeat > 1:  # whole bytes and whole blocks, so that the stream can be laid end to end: a few 2-bit codes become 4-bit ones
+        assert n % entropy.BLOCK == 0
+        short = np.flatnonzero(L == 2)[-3:]
+        fix = short[: ((8 - int(L.sum()) % 8) % 8) // 2]
+        sym[fix] = 2
+        L[fix] = 4
+    block = entropy.BLOCK
+    nb = -(-n // block)
+    starts = np.concatenate([[0], np.cumsum(L)]).astype(np.int64)  # first bit of every symbol's code: codes back to back
+    offsets = np.concatenate([starts[:-1][::block][:nb], [starts[-1]]]).astype(np.int64)  # bit where a block starts; last: the total
+    bits = np.zeros(int(starts[-1]), np.uint8)
+    c = codes[sym]
+    for j in range(12):
+        m = L > j
+        bits[starts[:-1][m] + j] = (c[m] >> (L[m] - 1 - j)) & 1
+    packed = np.packbits(bits)
+    if repeat > 1:
+        offsets = np.concatenate([offsets[:-1] + r * int(starts[-1]) for r in range(repeat)] + [[repeat * int(starts[-1])]]).astype(np.int64)
+        packed, sym = np.tile(packed, repeat), np.tile(sym, repeat)
+    stream = np.zeros(packed.size + 8, np.uint8)  # (zero padding behind the last code, as the reference's encoder leaves it)
+    stream[: packed.size] = packed
+    return {"stream": torch.from_numpy(stream).cuda(), "offsets": torch.from_numpy(offsets), "lens": torch.from_numpy(lens)}, sym
+
+
+def huff_case(bp, torch, entropy, timed, res, n_sym, repeat, name):
+    parts, sym = huffman_stream(torch, n_sym // repeat, repeat=repeat)
+    sym_d = torch.from_numpy(sym).cuda()
+    buf = torch.empty(n_sym, dtype=torch.uint8, device="cuda")
+    assert torch.equal(entropy.decode(parts, n_sym, out=buf), sym_d)
+    # (timed through the C entry point with the tables made once: the Python wrapper builds the decode table on the host
+    # and reads the error flag back, about a millisecond per call)
+    from deepseekternarized_amd.kernels import _lib
+    lut_host = entropy.decode_table(parts["lens"], entropy.MAXLEN)
+    lut, off_d, flag = lut_host.cuda(), parts["offsets"].cuda(), torch.zeros(1, dtype=torch.int32, device="cuda")
+    lib = bp.ext().lib
+
+    def huff():
+        _lib.check(lib.bp_huff_decode(buf.data_ptr(), buf.numel(), parts["stream"].data_ptr(), parts["stream"].numel(), off_d.data_ptr(),
+                                      parts["offsets"].data_ptr(), n_sym, entropy.BLOCK, lut.data_ptr(), lut_host.data_ptr(), entropy.MAXLEN,
+                                      None, 0, flag.data_ptr(), _lib.stream_ptr(buf.device)))
+        return buf
+
+    timed(name, huff, parts["stream"].numel() + n_sym, check=lambda o: torch.equal(o, sym_d) and int(flag.item()) == 0)
+    res[name]["bits_per_symbol"] = round(8 * parts["stream"].numel() / n_sym, 2)
+    del parts, sym_d, buf, lut, off_d
+
+
+def run_aux_kernels(bp, torch, a) -> int:
+    """The kernels either side of the GEMMs - pack / unpack, the scale and activation conversions, the absmean producer,
+    GGUF blocks, Mode B's decode, routing - each timed alone on a tensor of config 1's size (16 linears of 2048 x 7168),
+    bytes counted as what the operation has to read and write once."""
+    import numpy as np
+
+    from deepseekternarized_amd import entropy, gguf_blocks
+    from deepseekternarized_amd.kernels.ternary_hip import gather_rows
+    from deepseekternarized_amd.ternary import fit
+    from deepseekternarized_amd.ternary.ops import PackedTerm
+    from deepseekternarized_amd.ternary.pack import expand_scales
+
+    N, K = 16 * 2048, 7168
+    g = torch.Generator(device="cuda").manual_seed(1)
+    w = torch.randn(N, K, device="cuda", generator=g) * 0.02
+    trits = torch.randint(-1, 2, (N, K), device="cuda", generator=g, dtype=torch.int8)
+    res = {}
+
+    def timed(name, f, nbytes, check=None):
+        out = f()
+        torch.cuda.synchronize()
+        if check is not None:
+            assert check(out), name
+        reps = max(5, min(a.steps, 30))
+        ev = [(torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)) for _ in range(reps)]
+        for e0, e1 in ev:
+            e0.record()
+            f()
+            e1.record()
+        torch.cuda.synchronize()
+        t = sorted(e0.elapsed_time(e1) for e0, e1 in ev)[reps // 2] * 1e-3
+        res[name] = {"us": round(t * 1e6, 1), "GBps": round(nbytes / t / 1e9, 1), "frac_of_hbm_peak": round(nbytes / t / 1e9 / HBM_PEAK_GBPS, 4),
+                     "bytes": int(nbytes)}
+        return out
+
+    for fmt in ("tq1", "tq2"):
+        kp = bp.packed_cols(fmt, K)
+        pk = timed(f"pack_{fmt}", lambda: bp.pack(trits, fmt), N * K + N * kp)
+        timed(f"unpack_{fmt}", lambda: bp.unpack(pk, fmt, K), N * kp + N * K, check=lambda o: torch.equal(o, trits))
+        timed(f"absmean_pack_{fmt}_f32", lambda: fit.packed_term(w, 128, fmt), 4 * N * K + N * kp + 2 * N * K // 128)
+    wb = w.to(torch.bfloat16)
+    timed("absmean_pack_tq2_bf16", lambda: fit.packed_term(wb, 128, "tq2"), 2 * N * K + N * K // 4 + 2 * N * K // 128)
+    sc = (torch.rand(N, K // 128, device="cuda", generator=g) + 0.5).half()
+    timed("expand_scales_f16", lambda: expand_scales(sc), 6 * sc.numel())
+    x = torch.randn(4096, K, device="cuda", generator=g).to(torch.bfloat16)
+    timed("quant_act_int8_bf16", lambda: bp.quant_act_int8(x), x.numel() * 3 + 4 * x.size(0))
+    # GGUF blocks: single-term, group-256, fp16 scales
+    sc256 = (torch.rand(N, K // 256, device="cuda", generator=g) + 0.5).half()
+    for fmt, q in (("tq1", "tq1"), ("tq2", "tq2")):
+        kp = bp.packed_cols(fmt, K)
+        term = PackedTerm(bp.pack(trits, fmt), sc256)
+        bs = 54 if q == "tq1" else 66
+        blocks = timed(f"gguf_{q}_0_from_{fmt}", lambda: gguf_blocks.to_gguf_blocks(term, K, fmt, 256, q), N * kp + 2 * sc256.numel() + N * K // 256 * bs)
+        timed(f"gguf_{q}_0_to_{fmt}", lambda: gguf_blocks.from_gguf_blocks(blocks, K, fmt, q), N * K // 256 * bs + N * kp + 2 * sc256.numel(),
+              check=lambda o: torch.equal(o.packed, term.packed) and torch.equal(o.scale, sc256))
+        del term, blocks
+    # Mode B decode, one-byte format: 64 Mi symbols (16,384 blocks: one lane each, one wave per CU) and 1 Gi symbols
+    for n_sym, rep_, name in ((64 << 20, 1, "huff_decode_u8_64Mi"), (1 << 30, 16, "huff_decode_u8_1Gi")):
+        huff_case(bp, torch, entropy, timed, res, n_sym, rep_, name)
+    # routing: config 3's 12,288 ids over 384 experts, and a million ids
+    for n_ids, E in ((12288, 384), (1 << 20, 384)):
+        ids = torch.randint(0, E, (n_ids,), device="cuda", generator=g)
+        timed(f"sort_by_expert_{n_ids}", lambda: bp.sort_by_expert(ids, E), 8 * n_ids * 2 + 8 * E)
+    xs = torch.randn(2048, 4096, device="cuda", generator=g).to(torch.bfloat16)
+    order, _ = bp.sort_by_expert(torch.randint(0, 384, (12288,), device="cuda", generator=g), 384)
+    timed("gather_rows_12288x4096_bf16", lambda: gather_rows(xs, order, 6), 2 * 12288 * 4096 * 2)
+    worst = min(res, key=lambda k: res[k]["frac_of_hbm_peak"] if res[k]["bytes"] > (64 << 20) else 9.0)
+    return emit({
+        "metric": "ternary GEMV HBM GB/s (% peak); grouped-expert GEMM TFLOP/s (% MFMA peak)",
+        "value": res[worst]["GBps"], "unit": "GB/s", "n_gpus": 1, "steps": a.steps, "warmup": a.warmup,
+        "ms_per_step": round(res[worst]["us"] * 1e-3, 5), "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+        "dtype": "u8", "data": "synthetic",
+        "config": {"workload": f"aux_kernels: producer, format and routing kernels alone on {N} x {K} weights (value: the slowest large one, {worst})",
+                   "bytes_counted": "inputs read once + outputs written once; median of the timed calls by HIP events, Python wrapper and output allocation included"},
+        "roofline": {"bound": "hbm", "achieved": res[worst]["GBps"], "peak": HBM_PEAK_GBPS, "unit": "GB/s", "frac": res[worst]["frac_of_hbm_peak"],
+                     "traffic": None, "kernel": worst},
+        "cpu_baseline": None, "also": res})
+
+
 def emit(line) -> int:
     print(json.dumps(line))
     return 0
@@ -422,7 +563,7 @@ def main() -> int:
     ap.add_argument("--steps", type=int, default=200)
     ap.add_argument("--warmup", type=int, default=20)
     ap.add_argument("--spin-up", type=float, default=SPIN_UP_S, help="seconds of untimed launches before warm-up and timed steps (0: none, for counter runs)")
-    ap.add_argument("--workload", default="cfg1a_tq1_gemv", choices=sorted(WORKLOADS) + ["cfg3_grouped", "cfg3_moe", "cfg2_moe_T1", "cfg2_moe_T32", "cfg2_moe_T256", "cfg4_decode", "cfg4_decode_graph"])
+    ap.add_argument("--workload", default="cfg1a_tq1_gemv", choices=sorted(WORKLOADS) + ["aux_kernels", "cfg3_grouped", "cfg3_moe", "cfg2_moe_T1", "cfg2_moe_T32", "cfg2_moe_T256", "cfg4_decode", "cfg4_decode_graph"])
     ap.add_argument("--no-extras", action="store_true", help="skip the secondary measurements")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline")
     ap.add_argument("--calibrate-copy", action="store_true",
@@ -453,6 +594,8 @@ def main() -> int:
         return run_cfg3_grouped(bp, torch, a)
     if a.workload == "cfg3_moe":
         return run_cfg3_moe(bp, torch, a)
+    if a.workload == "aux_kernels":
+        return run_aux_kernels(bp, torch, a)
     if a.workload.startswith("cfg2_moe_T"):
         return run_cfg2_moe(bp, torch, a, int(a.workload[len("cfg2_moe_T"):]))
     if a.workload.startswith("cfg4_decode"):

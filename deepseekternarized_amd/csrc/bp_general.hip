@@ -129,6 +129,77 @@ __global__ __launch_bounds__(256) void k_pack(uint8_t* __restrict__ packed, cons
   }
 }
 
+
+// ---- pack / unpack with the trit side in 16-byte pieces (K a multiple of 16, 16-byte aligned trits): a workgroup takes
+// SEG_BYTES packed bytes of one row, a thread four of them (16 or 20 trits); the trits cross LDS so that global memory
+// sees them as consecutive 16-byte pieces whatever the 5-trit bytes' stride is. Same values as k_pack / k_unpack.
+constexpr int SEG_BYTES = 1024;
+template <int FMT>
+__global__ __launch_bounds__(256) void k_unpack_seg(int8_t* __restrict__ trits, const uint8_t* __restrict__ packed, int64_t K, int64_t Kp) {
+  constexpr int PER = FMT == BP_TQ2 ? 4 : 5;
+  __shared__ __attribute__((aligned(16))) unsigned seg[256 * PER];
+  const int64_t n = blockIdx.y, b0 = (int64_t)blockIdx.x * SEG_BYTES;
+  const uint8_t* prow = packed + n * Kp + b0;
+  const int64_t left = Kp - b0;  // packed bytes of the row from b0 on
+  unsigned char tb[4 * PER];
+#pragma unroll
+  for (int j = 0; j < 4; ++j) {
+    const int b = 4 * (int)threadIdx.x + j;
+    const unsigned v = b < left ? prow[b] : 0u;
+#pragma unroll
+    for (int d = 0; d < PER; ++d) tb[PER * j + d] = (unsigned char)(FMT == BP_TQ2 ? (int)((v >> (2 * d)) & 3u) - 1 : tq1_trit(v, d));
+  }
+#pragma unroll
+  for (int i = 0; i < PER; ++i)
+    seg[PER * threadIdx.x + i] = (unsigned)tb[4 * i] | ((unsigned)tb[4 * i + 1] << 8) | ((unsigned)tb[4 * i + 2] << 16) | ((unsigned)tb[4 * i + 3] << 24);
+  __syncthreads();
+  const int64_t k0 = b0 * PER;
+  const int64_t count = K - k0 < (int64_t)SEG_BYTES * PER ? K - k0 : (int64_t)SEG_BYTES * PER;  // (a multiple of 16)
+  uint4* dst = (uint4*)(trits + n * K + k0);
+  for (int pc = threadIdx.x; pc < count / 16; pc += 256) dst[pc] = ((const uint4*)seg)[pc];
+}
+
+template <int FMT>
+__global__ __launch_bounds__(256) void k_pack_seg(uint8_t* __restrict__ packed, const int8_t* __restrict__ trits, int64_t K, int64_t Kp) {
+  constexpr int PER = FMT == BP_TQ2 ? 4 : 5;
+  __shared__ __attribute__((aligned(16))) unsigned seg[256 * PER];
+  const int64_t n = blockIdx.y, b0 = (int64_t)blockIdx.x * SEG_BYTES;
+  const int64_t k0 = b0 * PER;
+  const int64_t count = K - k0 < (int64_t)SEG_BYTES * PER ? K - k0 : (int64_t)SEG_BYTES * PER;
+  const uint4* src = (const uint4*)(trits + n * K + k0);
+  for (int pc = threadIdx.x; pc < SEG_BYTES * PER / 16; pc += 256)  // (past the row: trit 0, the pad digit 1)
+    ((uint4*)seg)[pc] = pc < count / 16 ? src[pc] : make_uint4(0u, 0u, 0u, 0u);
+  __syncthreads();
+  unsigned char tb[4 * PER];
+#pragma unroll
+  for (int i = 0; i < PER; ++i) {
+    const unsigned w = seg[PER * threadIdx.x + i];
+    tb[4 * i] = (unsigned char)w; tb[4 * i + 1] = (unsigned char)(w >> 8); tb[4 * i + 2] = (unsigned char)(w >> 16); tb[4 * i + 3] = (unsigned char)(w >> 24);
+  }
+  unsigned out = 0;
+#pragma unroll
+  for (int j = 0; j < 4; ++j) {
+    unsigned v = 0, mul = 1;
+#pragma unroll
+    for (int d = 0; d < PER; ++d) {
+      const unsigned u = (unsigned)(((int)(signed char)tb[PER * j + d] + 1) & 0xff);
+      if (FMT == BP_TQ2) v |= u << (2 * d);
+      else { v += u * mul; mul *= 3u; }
+    }
+    out |= (v & 0xffu) << (8 * j);
+  }
+  const int64_t left = Kp - b0;
+  const int b = 4 * (int)threadIdx.x;
+  uint8_t* prow = packed + n * Kp + b0;
+  if ((((uintptr_t)prow) & 3) == 0 && b + 3 < left) {
+    *(unsigned*)(prow + b) = out;
+  } else {
+#pragma unroll
+    for (int j = 0; j < 4; ++j)
+      if (b + j < left) prow[b + j] = (uint8_t)(out >> (8 * j));
+  }
+}
+
 __global__ __launch_bounds__(256) void k_expand(float* __restrict__ out, const void* __restrict__ in, int dtype, int64_t n) {
   for (int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; i < n; i += (int64_t)gridDim.x * blockDim.x)
     out[i] = load_scale(in, dtype, i);
@@ -286,6 +357,89 @@ __global__ __launch_bounds__(256) void k_absmean_pack(uint8_t* __restrict__ pack
   }
 }
 
+
+// The same with the row staged in LDS as float32 (rows of whole 16-byte pieces at 16-byte aligned addresses that fit: the
+// launcher's choice): the row is read once, in consecutive 16-byte pieces, where the kernel above reads it twice with
+// a stride of one group between neighbouring threads in its first pass. Group g's values sit at g (group + 1) + i, so
+// the threads that add up neighbouring groups - each in ascending k, the order of the kernel above: the same scales
+// bit for bit - read different banks. LDS: K + G floats of the row, then the G rounded scales.
+template <int WDT>
+__global__ __launch_bounds__(256) void k_absmean_pack_lds(uint8_t* __restrict__ packed, void* __restrict__ scale, int8_t* __restrict__ trits,
+                                                          const void* __restrict__ w, int scale_dtype, int64_t K, int64_t Kp,
+                                                          int64_t G, int64_t group, int fmt) {
+  extern __shared__ __attribute__((aligned(16))) float row[];
+  constexpr int EPP = WDT == BP_F32 ? 4 : 8;  // elements per 16-byte piece
+  float* srow = row + K + G;
+  const int64_t n = blockIdx.x;
+  const uint4* src = (const uint4*)((const char*)w + n * K * (WDT == BP_F32 ? 4 : 2));
+  const int grp = (int)group, kk = (int)K;
+  for (int pc = threadIdx.x; pc < kk / EPP; pc += 256) {
+    const uint4 v = src[pc];
+    float f[EPP];
+    if (WDT == BP_F32) {
+      f[0] = __uint_as_float(v.x); f[1] = __uint_as_float(v.y); f[2] = __uint_as_float(v.z); f[3] = __uint_as_float(v.w);
+    } else {
+      const unsigned q[4] = {v.x, v.y, v.z, v.w};
+#pragma unroll
+      for (int j = 0; j < 4; ++j) {
+        f[2 * j % EPP] = WDT == BP_F16 ? f16_bits_to_f32((uint16_t)q[j]) : bf16_bits_to_f32((uint16_t)q[j]);
+        f[(2 * j + 1) % EPP] = WDT == BP_F16 ? f16_bits_to_f32((uint16_t)(q[j] >> 16)) : bf16_bits_to_f32((uint16_t)(q[j] >> 16));
+      }
+    }
+    const int k0 = EPP * pc;
+    int g = k0 / grp, r = k0 - g * grp;
+#pragma unroll
+    for (int j = 0; j < EPP; ++j) {
+      row[k0 + j + g] = f[j];
+      if (++r == grp) { r = 0; ++g; }
+    }
+  }
+  __syncthreads();
+  for (int g = threadIdx.x; g < (int)G; g += 256) {
+    const int k0 = g * grp, cnt = k0 + grp < kk ? grp : kk - k0;
+    const float* p = row + k0 + g;
+    float sum = 0.f;
+    for (int i = 0; i < cnt; ++i) sum += fabsf(p[i]);
+    const float mean = sum / (float)cnt;
+    float rounded;
+    if (scale_dtype == BP_F16) {
+      const _Float16 h = (_Float16)mean;
+      ((_Float16*)scale)[n * G + g] = h;
+      rounded = (float)h;
+    } else {
+      const uint16_t b = f32_to_bf16_bits(mean);
+      ((uint16_t*)scale)[n * G + g] = b;
+      rounded = bf16_bits_to_f32(b);
+    }
+    srow[g] = rounded;
+  }
+  __syncthreads();
+  const int per = fmt == BP_TQ2 ? 4 : 5;
+  for (int c = threadIdx.x; c < (int)Kp; c += 256) {
+    unsigned byte = 0, mul = 1;
+    const int kb = c * per;
+    int g = kb / grp, r = kb - g * grp;
+    for (int i = 0; i < per; ++i) {
+      const int k = kb + i;
+      int t = 0;
+      if (k < kk) {
+        const float s = srow[g];
+        if (s > 0.f) {
+          float q = rintf(row[k + g] / fmaxf(s, 1e-30f));
+          q = q < -1.f ? -1.f : q > 1.f ? 1.f : q;
+          t = (int)q;  // (a NaN weight compares false twice and converts to 0)
+        }
+        if (trits) trits[n * K + k] = (int8_t)t;
+        if (++r == grp) { r = 0; ++g; }
+      }
+      const unsigned u = (unsigned)(t + 1);
+      if (fmt == BP_TQ2) byte |= u << (2 * i);
+      else { byte += u * mul; mul *= 3; }
+    }
+    packed[n * Kp + c] = (uint8_t)byte;
+  }
+}
+
 }  // namespace
 
 int launch_general(const GemmArgs& a, hipStream_t s) {
@@ -320,6 +474,12 @@ extern "C" int bp_unpack_trits(int8_t* trits, const uint8_t* packed, int64_t N, 
   if (int rc = fmt_dims(fmt, N, K, &Kp)) return rc;
   if (N == 0) return BP_OK;
   if (!trits || !packed) return fail(BP_ERR_ARG, "null pointer");
+  if (K % 16 == 0 && ((uintptr_t)trits & 15) == 0 && N <= 65535) {
+    const dim3 grid((unsigned)((Kp + SEG_BYTES - 1) / SEG_BYTES), (unsigned)N);
+    if (fmt == BP_TQ2) hipLaunchKernelGGL(k_unpack_seg<BP_TQ2>, grid, dim3(256), 0, (hipStream_t)stream, trits, packed, K, Kp);
+    else hipLaunchKernelGGL(k_unpack_seg<BP_TQ1>, grid, dim3(256), 0, (hipStream_t)stream, trits, packed, K, Kp);
+    return check_launch("unpack");
+  }
   hipLaunchKernelGGL(k_unpack, dim3(grid_for(N * Kp)), dim3(256), 0, (hipStream_t)stream, trits, packed, N, K, Kp, fmt);
   return check_launch("unpack");
 }
@@ -329,6 +489,12 @@ extern "C" int bp_pack_trits(uint8_t* packed, const int8_t* trits, int64_t N, in
   if (int rc = fmt_dims(fmt, N, K, &Kp)) return rc;
   if (N == 0) return BP_OK;
   if (!trits || !packed) return fail(BP_ERR_ARG, "null pointer");
+  if (K % 16 == 0 && ((uintptr_t)trits & 15) == 0 && N <= 65535) {
+    const dim3 grid((unsigned)((Kp + SEG_BYTES - 1) / SEG_BYTES), (unsigned)N);
+    if (fmt == BP_TQ2) hipLaunchKernelGGL(k_pack_seg<BP_TQ2>, grid, dim3(256), 0, (hipStream_t)stream, packed, trits, K, Kp);
+    else hipLaunchKernelGGL(k_pack_seg<BP_TQ1>, grid, dim3(256), 0, (hipStream_t)stream, packed, trits, K, Kp);
+    return check_launch("pack");
+  }
   hipLaunchKernelGGL(k_pack, dim3(grid_for(N * Kp)), dim3(256), 0, (hipStream_t)stream, packed, trits, N, K, Kp, fmt);
   return check_launch("pack");
 }
@@ -372,6 +538,23 @@ extern "C" int bp_absmean_pack(uint8_t* packed, void* scale, int scale_dtype, in
   if (N > 0x7fffffff) return fail(BP_ERR_ARG, "too many rows");
   if (N == 0) return BP_OK;
   if (!packed || !scale || !w) return fail(BP_ERR_ARG, "null pointer");
+  // rows of whole 16-byte pieces that fit LDS beside their scales: the kernel that reads its row once
+  const int64_t epp = w_dtype == BP_F32 ? 4 : 8;
+  const size_t lds = (size_t)(K + 2 * G) * 4;
+  if (K % epp == 0 && ((uintptr_t)w & 15) == 0 && lds <= 128 * 1024 && K < ((int64_t)1 << 24)) {
+    const dim3 grid((unsigned)N);
+    const hipStream_t st = (hipStream_t)stream;
+#define BP_ABSMEAN(DT)                                                                                                          \
+  {                                                                                                                             \
+    if (const int rc = raise_lds_limit<k_absmean_pack_lds<DT>>(128 * 1024)) return rc;                                          \
+    hipLaunchKernelGGL(k_absmean_pack_lds<DT>, grid, dim3(256), lds, st, packed, scale, trits, w, scale_dtype, K, Kp, G, group, fmt); \
+    return check_launch("absmean_pack");                                                                                       \
+  }
+    if (w_dtype == BP_F32) BP_ABSMEAN(BP_F32)
+    if (w_dtype == BP_F16) BP_ABSMEAN(BP_F16)
+    BP_ABSMEAN(BP_BF16)
+#undef BP_ABSMEAN
+  }
   hipLaunchKernelGGL(k_absmean_pack, dim3((unsigned)N), dim3(256), 0, (hipStream_t)stream, packed, scale, trits, w, w_dtype, scale_dtype, K, Kp,
                      G, group, fmt);
   return check_launch("absmean_pack");

@@ -18,7 +18,7 @@
 namespace bp {
 namespace {
 
-constexpr int HUFF_THREADS = 256;
+constexpr int HUFF_THREADS = 64;  // a wave per workgroup: the blocks are few (4096 symbols each) and spread over as many CUs as they can
 
 template <bool RAW>
 __global__ __launch_bounds__(HUFF_THREADS) void k_huff_decode(uint8_t* __restrict__ out, const uint8_t* __restrict__ stream, int64_t stream_bytes,
@@ -39,20 +39,38 @@ __global__ __launch_bounds__(HUFF_THREADS) void k_huff_decode(uint8_t* __restric
   // bits [pos, pos + have) of the stream sit at the top of `buf`
   uint64_t buf = 0;
   int have = 0;
-  int64_t next_byte = pos >> 3;  // the byte the next refill starts at
-  auto refill = [&]() {  // 32 more bits; past the stream's last byte they are zeros (never decoded: a code must start 4 bytes before the end)
-    if (have > 32 || next_byte >= stream_bytes) return;
-    uint32_t w = 0;
-    if (next_byte + 4 <= stream_bytes) {
-      uint32_t le;
-      __builtin_memcpy(&le, stream + next_byte, 4);
-      w = __builtin_bswap32(le);
+  // The lane's part of the stream travels in 16-byte pieces, requested one piece (four refills, some 30 symbols) before
+  // its first word is wanted: with a few thousand blocks per tensor there are few waves per CU, and a load that a wave
+  // waits for is a microsecond in which it decodes nothing. Past the stream's last byte a piece holds zeros (never
+  // decoded: a code must start 4 bytes before the end).
+  auto load_piece = [&](int64_t byte) -> uint4 {
+    uint4 v = make_uint4(0u, 0u, 0u, 0u);
+    if (byte + 16 <= stream_bytes) {
+      __builtin_memcpy(&v, stream + byte, 16);
     } else {
-      for (int64_t q = next_byte; q < stream_bytes; ++q) w |= (uint32_t)stream[q] << (24 - 8 * (int)(q - next_byte));
+      uint32_t w[4] = {0u, 0u, 0u, 0u};
+      for (int64_t q = byte; q < stream_bytes; ++q) w[(q - byte) >> 2] |= (uint32_t)stream[q] << (8 * (int)((q - byte) & 3));
+      v = make_uint4(w[0], w[1], w[2], w[3]);
     }
+    return v;
+  };
+  int64_t piece_byte = pos >> 3;  // the byte `cur` starts at
+  uint4 cur = load_piece(piece_byte), nxt = load_piece(piece_byte + 16);
+  int words = 4;                  // words of `cur` not yet taken (the next one is cur.x)
+  auto refill = [&]() {  // 32 more bits
+    if (have > 32) return;
+    const uint32_t w = __builtin_bswap32(cur.x);
+    cur.x = cur.y;
+    cur.y = cur.z;
+    cur.z = cur.w;
     buf |= (uint64_t)w << (32 - have);
     have += 32;
-    next_byte += 4;
+    if (--words == 0) {
+      cur = nxt;
+      piece_byte += 16;
+      nxt = load_piece(piece_byte + 16);
+      words = 4;
+    }
   };
   refill();
   {  // drop the bits of the first byte that precede pos
@@ -67,20 +85,38 @@ __global__ __launch_bounds__(HUFF_THREADS) void k_huff_decode(uint8_t* __restric
   while (i < end && !bad) {
     const int chunk = end - i < 16 ? (int)(end - i) : 16;
     uint32_t sy[4] = {0u, 0u, 0u, 0u};
-    for (int j = 0; j < chunk; ++j) {
-      // (the reference: pos >= end bit, or byte > stream_bytes - 4 -> invalid)
-      if (pos >= stop || (pos >> 3) > stream_bytes - 4) { bad = true; break; }
-      if (have < maxlen) { bad = true; break; }  // (cannot happen while the check above holds: 4 bytes from pos >> 3 are in range)
+    // one symbol into byte j of sy (the reference: pos >= end bit, or byte > stream_bytes - 4 -> invalid). After an
+    // invalid code the lane decodes nothing more: it stays inside the table and the stream's pieces whatever it holds.
+    auto symbol = [&](int j) {
+      if (bad) return;
+      if (pos >= stop || (pos >> 3) > stream_bytes - 4) { bad = true; return; }
       const int32_t e = table[(uint32_t)(buf >> (64 - maxlen))];
       const int length = e & 0xff;
-      if (!length || length > stop - pos) { bad = true; break; }
+      if (!length || length > stop - pos) { bad = true; return; }
       sy[j >> 2] |= (uint32_t)((e >> 8) & 0xff) << (8 * (j & 3));
       buf <<= length;
       have -= length;
       pos += length;
       refill();
+    };
+    if (chunk == 16) {  // (unrolled: sy stays in registers)
+#pragma unroll
+      for (int j = 0; j < 16; ++j) symbol(j);
+    } else {
+      uint32_t t4[4] = {0u, 0u, 0u, 0u};
+      for (int j = 0; j < chunk; ++j) {  // the block's last symbols: one at a time into byte 0, moved to its place
+        sy[0] = 0u;
+        symbol(0);
+        const uint32_t v = sy[0] << (8 * (j & 3));
+        t4[0] |= (j >> 2) == 0 ? v : 0u;
+        t4[1] |= (j >> 2) == 1 ? v : 0u;
+        t4[2] |= (j >> 2) == 2 ? v : 0u;
+        t4[3] |= (j >> 2) == 3 ? v : 0u;
+      }
+      sy[0] = t4[0]; sy[1] = t4[1]; sy[2] = t4[2]; sy[3] = t4[3];
     }
     if (bad) break;
+    auto sy_word = [&](int q) { return q == 0 ? sy[0] : q == 1 ? sy[1] : q == 2 ? sy[2] : sy[3]; };  // (no indexed access: sy stays in registers)
     if (RAW) {
       if (vec && chunk == 16) {
         const uint4 r = *(const uint4*)(raw + i);
@@ -96,13 +132,13 @@ __global__ __launch_bounds__(HUFF_THREADS) void k_huff_decode(uint8_t* __restric
       } else {
         for (int j = 0; j < chunk; ++j) {
           out[2 * (i + j)] = raw[i + j];
-          out[2 * (i + j) + 1] = (uint8_t)(sy[j >> 2] >> (8 * (j & 3)));
+          out[2 * (i + j) + 1] = (uint8_t)(sy_word(j >> 2) >> (8 * (j & 3)));
         }
       }
     } else {
       if (vec && chunk == 16) *(uint4*)(out + i) = make_uint4(sy[0], sy[1], sy[2], sy[3]);
       else
-        for (int j = 0; j < chunk; ++j) out[i + j] = (uint8_t)(sy[j >> 2] >> (8 * (j & 3)));
+        for (int j = 0; j < chunk; ++j) out[i + j] = (uint8_t)(sy_word(j >> 2) >> (8 * (j & 3)));
     }
     i += chunk;
   }
