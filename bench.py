@@ -401,7 +401,7 @@ def huff_case(bp, torch, entropy, timed, res, n_sym, repeat, name):
     del parts, sym_d, buf, lut, off_d
 
 
-def run_aux_kernels(bp, torch, a) -> int:
+def aux_kernels(bp, torch, steps, big=True):
     """The kernels either side of the GEMMs - pack / unpack, the scale and activation conversions, the absmean producer,
     GGUF blocks, Mode B's decode, routing - each timed alone on a tensor of config 1's size (16 linears of 2048 x 7168),
     bytes counted as what the operation has to read and write once."""
@@ -424,7 +424,7 @@ def run_aux_kernels(bp, torch, a) -> int:
         torch.cuda.synchronize()
         if check is not None:
             assert check(out), name
-        reps = max(5, min(a.steps, 30))
+        reps = max(5, min(steps, 30))
         ev = [(torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)) for _ in range(reps)]
         for e0, e1 in ev:
             e0.record()
@@ -458,7 +458,7 @@ def run_aux_kernels(bp, torch, a) -> int:
               check=lambda o: torch.equal(o.packed, term.packed) and torch.equal(o.scale, sc256))
         del term, blocks
     # Mode B decode, one-byte format: 64 Mi symbols (16,384 blocks: one lane each, one wave per CU) and 1 Gi symbols
-    for n_sym, rep_, name in ((64 << 20, 1, "huff_decode_u8_64Mi"), (1 << 30, 16, "huff_decode_u8_1Gi")):
+    for n_sym, rep_, name in ((64 << 20, 1, "huff_decode_u8_64Mi"), (1 << 30, 16, "huff_decode_u8_1Gi"))[: 2 if big else 1]:
         huff_case(bp, torch, entropy, timed, res, n_sym, rep_, name)
     # routing: config 3's 12,288 ids over 384 experts, and a million ids
     for n_ids, E in ((12288, 384), (1 << 20, 384)):
@@ -467,6 +467,11 @@ def run_aux_kernels(bp, torch, a) -> int:
     xs = torch.randn(2048, 4096, device="cuda", generator=g).to(torch.bfloat16)
     order, _ = bp.sort_by_expert(torch.randint(0, 384, (12288,), device="cuda", generator=g), 384)
     timed("gather_rows_12288x4096_bf16", lambda: gather_rows(xs, order, 6), 2 * 12288 * 4096 * 2)
+    return res, (N, K)
+
+
+def run_aux_kernels(bp, torch, a) -> int:
+    res, (N, K) = aux_kernels(bp, torch, a.steps)
     worst = min(res, key=lambda k: res[k]["frac_of_hbm_peak"] if res[k]["bytes"] > (64 << 20) else 9.0)
     return emit({
         "metric": "ternary GEMV HBM GB/s (% peak); grouped-expert GEMM TFLOP/s (% MFMA peak)",
@@ -672,6 +677,10 @@ def main() -> int:
                                   "ms_per_layer": round(dt3 * 1e3, 3), "TFLOPs_per_term_count": round(fl3 / dt3 / 1e12, 1),
                                   "frac_of_bf16_mfma_peak": round(fl3 / dt3 / 1e12 / MFMA_BF16_PEAK_TFLOPS, 4)}
         del moe3, x3, lg3
+        torch.cuda.empty_cache()
+        # the producer, format and routing kernels either side of the GEMMs, each alone (us, bytes read + written once per second)
+        aux, _ = aux_kernels(bp, torch, 10, big=False)
+        also["aux_kernels"] = {k: {"us": v["us"], "GBps": v["GBps"]} for k, v in aux.items()}
         torch.cuda.empty_cache()
         # end-to-end timing loop of the reference's `boilerplate bench` on a random-init OLMoE-shaped Mode D decoder
         from deepseekternarized_amd.decoder_harness import DecoderConfig, TernaryDecoder, bench_decoder
