@@ -117,7 +117,9 @@ int bp_set_kernel_policy(int policy);
  * Safe against launches on other threads: they read either the old or the new set, whole. */
 void bp_reload_tuning(void);
 
-/* Name of the kernel the last bp_ternary_grouped_gemm on this thread launched ("" if none). */
+/* Name of the kernel the last bp_ternary_grouped_gemm on this thread launched ("" if none). After bp_moe_layer_*: the
+ * down projection's kernel, with "+glu", "+gather", "+y16" appended where the gate | up launch applied SwiGLU itself, read
+ * its rows through the sort order, and the down launch wrote bf16 rows (diagnostics; the tests read it). */
 const char* bp_last_kernel(void);
 
 /* Packed rows -> int8 trits [N, K]; bit-identical to unpack_tq1/unpack_tq2
