@@ -51,6 +51,21 @@ def test_pack_unpack_bit_exact(bp, fmt, K):
 
 
 @pytest.mark.parametrize("fmt", ["tq2", "tq1"])
+@pytest.mark.parametrize("K", [16, 5120, 5136, 7168, 20496])
+def test_pack_unpack_in_16_byte_pieces_bit_exact(bp, fmt, K):
+    """K a multiple of 16: the kernels that move the trit side in 16-byte pieces through LDS, a workgroup per 1024 packed
+    bytes of a row - one segment, a segment that ends inside a TQ1 byte's five trits, several segments per row."""
+    rng = np.random.default_rng(K)
+    t = rng.integers(-1, 2, (37, K)).astype(np.int8)
+    p = bp.pack(dev(t), fmt)
+    assert np.array_equal(p.cpu().numpy(), orc.pack(t, fmt))
+    assert np.array_equal(bp.unpack(p, fmt, K).cpu().numpy(), t)
+    # every byte value on the unpack side (TQ2 code 3 -> +2, TQ1 bytes >= 243 -> 0), rows of other lengths around it
+    raw = rng.integers(0, 256, (5, bp.packed_cols(fmt, K))).astype(np.uint8)
+    assert np.array_equal(bp.unpack(dev(raw), fmt, K).cpu().numpy(), orc.unpack(raw, fmt, K))
+
+
+@pytest.mark.parametrize("fmt", ["tq2", "tq1"])
 def test_unpack_every_byte_value_bit_exact(bp, fmt):
     """All 256 byte values, incl. TQ2 code 3 (-> +2) and TQ1 bytes >= 243 (-> 0)."""
     per = 4 if fmt == "tq2" else 5
@@ -488,6 +503,28 @@ def test_absmean_and_packed_term_bit_exact(bp, wdtype, sdtype, K, group):
     assert np.array_equal(term.trits.cpu().numpy(), want_trits)
     for fmt in ("tq1", "tq2"):
         pt = bp.packed_term(wt, group, fmt, sdtype)
+        assert np.array_equal(pt.packed.cpu().numpy(), orc.pack(want_trits, fmt))
+        assert torch.equal(pt.scale, term.scale)
+
+
+@pytest.mark.parametrize("wdtype", [torch.float32, torch.bfloat16, torch.float16])
+@pytest.mark.parametrize("K,group", [(7168, 128), (7168, 256), (2048, 96), (1000, 100), (256, 1000), (4096, 4096)])
+def test_absmean_with_the_row_staged_in_lds_bit_exact(bp, wdtype, K, group):
+    """Rows of whole 16-byte pieces: the producer reads its row once into LDS. Groups that end inside a 16-byte piece, a
+    last group shorter than the others, one group longer than the row: scales, trits and packed bytes bit-identical to
+    the oracle (group sums in ascending k)."""
+    rng = np.random.default_rng(K + group)
+    w = rng.standard_normal((21, K)).astype(np.float32) * np.exp(rng.uniform(-3, 3, (21, 1))).astype(np.float32)
+    w[3] = 0.0
+    w[4, K // 3:] = 0.0
+    wt = dev(w).to(wdtype)
+    w_seen = wt.float().cpu().numpy()
+    want_trits, want_scale = orc.absmean_ternary(w_seen, group, "f16")
+    term = bp.absmean_ternary(wt, group, torch.float16)
+    assert np.array_equal(term.scale.float().cpu().numpy(), want_scale)
+    assert np.array_equal(term.trits.cpu().numpy(), want_trits)
+    for fmt in ("tq1", "tq2"):
+        pt = bp.packed_term(wt, group, fmt, torch.float16)
         assert np.array_equal(pt.packed.cpu().numpy(), orc.pack(want_trits, fmt))
         assert torch.equal(pt.scale, term.scale)
 
