@@ -138,7 +138,7 @@ template <int FMT>
 __global__ __launch_bounds__(256) void k_unpack_seg(int8_t* __restrict__ trits, const uint8_t* __restrict__ packed, int64_t K, int64_t Kp) {
   constexpr int PER = FMT == BP_TQ2 ? 4 : 5;
   __shared__ __attribute__((aligned(16))) unsigned seg[256 * PER];
-  const int64_t n = blockIdx.y, b0 = (int64_t)blockIdx.x * SEG_BYTES;
+  const int64_t n = blockIdx.x, b0 = (int64_t)blockIdx.y * SEG_BYTES;
   const uint8_t* prow = packed + n * Kp + b0;
   const int64_t left = Kp - b0;  // packed bytes of the row from b0 on
   unsigned char tb[4 * PER];
@@ -163,7 +163,7 @@ template <int FMT>
 __global__ __launch_bounds__(256) void k_pack_seg(uint8_t* __restrict__ packed, const int8_t* __restrict__ trits, int64_t K, int64_t Kp) {
   constexpr int PER = FMT == BP_TQ2 ? 4 : 5;
   __shared__ __attribute__((aligned(16))) unsigned seg[256 * PER];
-  const int64_t n = blockIdx.y, b0 = (int64_t)blockIdx.x * SEG_BYTES;
+  const int64_t n = blockIdx.x, b0 = (int64_t)blockIdx.y * SEG_BYTES;
   const int64_t k0 = b0 * PER;
   const int64_t count = K - k0 < (int64_t)SEG_BYTES * PER ? K - k0 : (int64_t)SEG_BYTES * PER;
   const uint4* src = (const uint4*)(trits + n * K + k0);
@@ -474,8 +474,8 @@ extern "C" int bp_unpack_trits(int8_t* trits, const uint8_t* packed, int64_t N, 
   if (int rc = fmt_dims(fmt, N, K, &Kp)) return rc;
   if (N == 0) return BP_OK;
   if (!trits || !packed) return fail(BP_ERR_ARG, "null pointer");
-  if (K % 16 == 0 && ((uintptr_t)trits & 15) == 0 && N <= 65535) {
-    const dim3 grid((unsigned)((Kp + SEG_BYTES - 1) / SEG_BYTES), (unsigned)N);
+  if (K % 16 == 0 && ((uintptr_t)trits & 15) == 0 && N <= 0x7fffffff && (Kp + SEG_BYTES - 1) / SEG_BYTES <= 65535) {
+    const dim3 grid((unsigned)N, (unsigned)((Kp + SEG_BYTES - 1) / SEG_BYTES));
     if (fmt == BP_TQ2) hipLaunchKernelGGL(k_unpack_seg<BP_TQ2>, grid, dim3(256), 0, (hipStream_t)stream, trits, packed, K, Kp);
     else hipLaunchKernelGGL(k_unpack_seg<BP_TQ1>, grid, dim3(256), 0, (hipStream_t)stream, trits, packed, K, Kp);
     return check_launch("unpack");
@@ -489,8 +489,8 @@ extern "C" int bp_pack_trits(uint8_t* packed, const int8_t* trits, int64_t N, in
   if (int rc = fmt_dims(fmt, N, K, &Kp)) return rc;
   if (N == 0) return BP_OK;
   if (!trits || !packed) return fail(BP_ERR_ARG, "null pointer");
-  if (K % 16 == 0 && ((uintptr_t)trits & 15) == 0 && N <= 65535) {
-    const dim3 grid((unsigned)((Kp + SEG_BYTES - 1) / SEG_BYTES), (unsigned)N);
+  if (K % 16 == 0 && ((uintptr_t)trits & 15) == 0 && N <= 0x7fffffff && (Kp + SEG_BYTES - 1) / SEG_BYTES <= 65535) {
+    const dim3 grid((unsigned)N, (unsigned)((Kp + SEG_BYTES - 1) / SEG_BYTES));
     if (fmt == BP_TQ2) hipLaunchKernelGGL(k_pack_seg<BP_TQ2>, grid, dim3(256), 0, (hipStream_t)stream, packed, trits, K, Kp);
     else hipLaunchKernelGGL(k_pack_seg<BP_TQ1>, grid, dim3(256), 0, (hipStream_t)stream, packed, trits, K, Kp);
     return check_launch("pack");

@@ -60,6 +60,11 @@ def test_pack_unpack_in_16_byte_pieces_bit_exact(bp, fmt, K):
     p = bp.pack(dev(t), fmt)
     assert np.array_equal(p.cpu().numpy(), orc.pack(t, fmt))
     assert np.array_equal(bp.unpack(p, fmt, K).cpu().numpy(), t)
+    if K == 16:  # more rows than one grid dimension's second extent holds
+        tall = rng.integers(-1, 2, (70001, K)).astype(np.int8)
+        pt = bp.pack(dev(tall), fmt)
+        assert np.array_equal(pt.cpu().numpy(), orc.pack(tall, fmt))
+        assert np.array_equal(bp.unpack(pt, fmt, K).cpu().numpy(), tall)
     # every byte value on the unpack side (TQ2 code 3 -> +2, TQ1 bytes >= 243 -> 0), rows of other lengths around it
     raw = rng.integers(0, 256, (5, bp.packed_cols(fmt, K))).astype(np.uint8)
     assert np.array_equal(bp.unpack(dev(raw), fmt, K).cpu().numpy(), orc.unpack(raw, fmt, K))
