@@ -253,6 +253,29 @@ def test_swiglu_in_the_gate_up_epilogue_equals_the_separate_launch(tune, fmt, te
     assert torch.isfinite(fused.float()).all() and torch.equal(fused, apart)
 
 
+@pytest.mark.parametrize("fmt", ["tq1", "tq2"])
+def test_swiglu_epilogue_with_a_partly_filled_row_block(tune, fmt):
+    """An intermediate size that is not a multiple of the 256 rows a row block takes of either half (1152 = 4.5 blocks): the
+    last block's waves without rows store nothing, and the down projection (K = 1152 is outside the tile kernels) runs
+    on another kernel from the same bf16 h. Bit-identical to the separate SwiGLU launch."""
+    from deepseekternarized_amd import ext
+
+    H, I, E, k, T = 1024, 1152, 8, 2, 150
+    moe, _ = _layer(fmt, "bf16", H, I, E, k, terms=1, seed=77)
+    g = torch.Generator(device="cuda").manual_seed(78)
+    x = torch.randn(T, H, device="cuda", generator=g).to(torch.bfloat16)
+    logits = torch.randn(T, E, device="cuda", generator=g)
+    if fmt == "tq2":
+        tune("BP_TUNE_TQ2G", "fp4")
+    fused = moe(x, logits).clone()
+    assert "+glu" in ext().last_kernel(), ext().last_kernel()
+    tune("BP_TUNE_GLU", "n")
+    apart = moe(x, logits).clone()
+    assert "+glu" not in ext().last_kernel(), ext().last_kernel()
+    assert torch.isfinite(fused.float()).all() and torch.equal(fused, apart)
+    assert _rel(fused, moe.composed(x, logits)) <= 2e-3
+
+
 def test_v4_stages_bit_exact():
     """bp_swiglu_v4 and bp_moe_combine_v4 alone, against their definitions evaluated with torch on the device
     (float32 throughout; expf may differ from torch's by an ulp, which the bf16 rounding rarely sees)."""
