@@ -470,8 +470,43 @@ def aux_kernels(bp, torch, steps, big=True):
     return res, (N, K)
 
 
+def aux_cpu_baseline(K, rows=512):
+    """The NumPy restatements of the same operations on `rows` rows of the same width, one host thread: bytes read +
+    written once per second, for the figure beside the device's."""
+    import numpy as np
+
+    sys.path.insert(0, str(ROOT / "tests"))
+    from _util import orc
+
+    rng = np.random.default_rng(0)
+    trits = rng.integers(-1, 2, (rows, K)).astype(np.int8)
+    w = (rng.standard_normal((rows, K)) * 0.02).astype(np.float32)
+    out = {}
+
+    def timed(name, f, nbytes):
+        f()
+        reps, t0 = 0, time.perf_counter()
+        while time.perf_counter() - t0 < 1.0:
+            f()
+            reps += 1
+        dt = (time.perf_counter() - t0) / reps
+        out[name] = {"GBps": round(nbytes / dt / 1e9, 3), "ms": round(dt * 1e3, 2)}
+
+    for fmt in ("tq1", "tq2"):
+        kp = orc.packed_cols(fmt, K)
+        pk = orc.pack(trits, fmt)
+        timed(f"pack_{fmt}", lambda: orc.pack(trits, fmt), rows * (K + kp))
+        timed(f"unpack_{fmt}", lambda: orc.unpack(pk, fmt, K), rows * (K + kp))
+    timed("absmean_ternary_f32", lambda: orc.absmean_ternary(w, 128, "f16"), rows * (4 * K + K + 2 * K // 128))
+    x = orc.bf16_round(rng.standard_normal((rows, K)).astype(np.float32))
+    timed("quant_act_int8", lambda: orc.quant_act_int8(x), rows * (3 * K + 4))
+    return {"value": out["pack_tq1"]["GBps"], "unit": "GB/s", "cores": 1, "kind": "port",
+            "sample": f"NumPy restatements on {rows} x {K}, about a second each, one host thread", "each": out}
+
+
 def run_aux_kernels(bp, torch, a) -> int:
     res, (N, K) = aux_kernels(bp, torch, a.steps)
+    cpu = None if a.no_cpu else aux_cpu_baseline(K)
     worst = min(res, key=lambda k: res[k]["frac_of_hbm_peak"] if res[k]["bytes"] > (64 << 20) else 9.0)
     return emit({
         "metric": "ternary GEMV HBM GB/s (% peak); grouped-expert GEMM TFLOP/s (% MFMA peak)",
@@ -482,7 +517,7 @@ def run_aux_kernels(bp, torch, a) -> int:
                    "bytes_counted": "inputs read once + outputs written once; median of the timed calls by HIP events, Python wrapper and output allocation included"},
         "roofline": {"bound": "hbm", "achieved": res[worst]["GBps"], "peak": HBM_PEAK_GBPS, "unit": "GB/s", "frac": res[worst]["frac_of_hbm_peak"],
                      "traffic": None, "kernel": worst},
-        "cpu_baseline": None, "also": res})
+        "cpu_baseline": cpu, "also": res})
 
 
 def emit(line) -> int:
