@@ -141,13 +141,29 @@ __global__ __launch_bounds__(256) void k_unpack_seg(int8_t* __restrict__ trits, 
   const int64_t n = blockIdx.x, b0 = (int64_t)blockIdx.y * SEG_BYTES;
   const uint8_t* prow = packed + n * Kp + b0;
   const int64_t left = Kp - b0;  // packed bytes of the row from b0 on
+  // TQ1: a byte's five trits from a table in LDS (entry v: trits 0..3 in one dword, trit 4 in the next), made by the
+  // workgroup's 256 threads - five divisions per byte otherwise
+  __shared__ unsigned digits[FMT == BP_TQ1 ? 512 : 1];
+  if (FMT == BP_TQ1) {
+    const unsigned v = threadIdx.x;
+    digits[2 * v] = (unsigned)(tq1_trit(v, 0) & 0xff) | ((unsigned)(tq1_trit(v, 1) & 0xff) << 8) | ((unsigned)(tq1_trit(v, 2) & 0xff) << 16) |
+                    ((unsigned)(tq1_trit(v, 3) & 0xff) << 24);
+    digits[2 * v + 1] = (unsigned)(tq1_trit(v, 4) & 0xff);
+    __syncthreads();
+  }
   unsigned char tb[4 * PER];
 #pragma unroll
   for (int j = 0; j < 4; ++j) {
     const int b = 4 * (int)threadIdx.x + j;
     const unsigned v = b < left ? prow[b] : 0u;
+    if (FMT == BP_TQ1) {
+      const unsigned lo = digits[2 * v], hi = digits[2 * v + 1];
+      tb[PER * j] = (unsigned char)lo; tb[PER * j + 1] = (unsigned char)(lo >> 8); tb[PER * j + 2] = (unsigned char)(lo >> 16);
+      tb[PER * j + 3] = (unsigned char)(lo >> 24); tb[PER * j + PER - 1] = (unsigned char)hi;
+    } else {
 #pragma unroll
-    for (int d = 0; d < PER; ++d) tb[PER * j + d] = (unsigned char)(FMT == BP_TQ2 ? (int)((v >> (2 * d)) & 3u) - 1 : tq1_trit(v, d));
+      for (int d = 0; d < PER; ++d) tb[PER * j + d] = (unsigned char)((int)((v >> (2 * d)) & 3u) - 1);
+    }
   }
 #pragma unroll
   for (int i = 0; i < PER; ++i)
@@ -399,7 +415,15 @@ __global__ __launch_bounds__(256) void k_absmean_pack_lds(uint8_t* __restrict__ 
     const int k0 = g * grp, cnt = k0 + grp < kk ? grp : kk - k0;
     const float* p = row + k0 + g;
     float sum = 0.f;
-    for (int i = 0; i < cnt; ++i) sum += fabsf(p[i]);
+    int i = 0;
+    for (; i + 16 <= cnt; i += 16) {  // (sixteen reads on their way, then added in ascending k)
+      float v[16];
+#pragma unroll
+      for (int j = 0; j < 16; ++j) v[j] = p[i + j];
+#pragma unroll
+      for (int j = 0; j < 16; ++j) sum += fabsf(v[j]);
+    }
+    for (; i < cnt; ++i) sum += fabsf(p[i]);
     const float mean = sum / (float)cnt;
     float rounded;
     if (scale_dtype == BP_F16) {
@@ -423,12 +447,13 @@ __global__ __launch_bounds__(256) void k_absmean_pack_lds(uint8_t* __restrict__ 
       const int k = kb + i;
       int t = 0;
       if (k < kk) {
-        const float s = srow[g];
-        if (s > 0.f) {
-          float q = rintf(row[k + g] / fmaxf(s, 1e-30f));
-          q = q < -1.f ? -1.f : q > 1.f ? 1.f : q;
-          t = (int)q;  // (a NaN weight compares false twice and converts to 0)
-        }
+        // clamp(rint(w / max(s, 1e-30)), -1, 1) without the division: the rounded quotient exceeds 1/2 (and rounds to
+        // +-1 or beyond) exactly when |w| / se > 1/2 + 2^-25, i.e. |w| - se / 2 > se 2^-25; the difference is exact
+        // wherever the comparison is close (|w| within a factor of two of se / 2), the product always (se >= 1e-30).
+        // A quotient of exactly 1/2 rounds to even, 0. NaN weights compare false: 0, as the conversion of a NaN gives.
+        const float s = srow[g], w = row[k + g];
+        const float se = fmaxf(s, 1e-30f);
+        if (s > 0.f && fabsf(w) - 0.5f * se > se * 0x1p-25f) t = w < 0.f ? -1 : 1;
         if (trits) trits[n * K + k] = (int8_t)t;
         if (++r == grp) { r = 0; ++g; }
       }

@@ -534,6 +534,35 @@ def test_absmean_with_the_row_staged_in_lds_bit_exact(bp, wdtype, K, group):
         assert torch.equal(pt.scale, term.scale)
 
 
+@pytest.mark.parametrize("sdtype", [torch.float16, torch.bfloat16])
+def test_absmean_weights_at_the_rounding_boundary(bp, sdtype):
+    """Weights within a few units in the last place of half their group's scale, where rint(w / s) changes between 0 and
+    +-1 (a quotient of exactly 1/2 rounds to even, 0): the producer decides without dividing, the oracle divides. Groups
+    of 128 whose mean is a power of two (so that the stored scale is the mean exactly), at magnitudes from 2^-20 to 2^10,
+    and a group of NaN / infinite weights."""
+    rng = np.random.default_rng(99)
+    N, K, group = 64, 1024, 128
+    w = np.zeros((N, K), np.float32)
+    for n in range(N):
+        for g in range(K // group):
+            s = np.float32(2.0) ** int(rng.integers(-20, 11))
+            half = np.float32(0.5) * s
+            near = (np.full(64, half, np.float32).view(np.int32) + rng.integers(-3, 4, 64).astype(np.int32)).view(np.float32)
+            near *= rng.choice(np.array([-1, 1], np.float32), 64)
+            # the other 64 weights make the group's mean |w| exactly s: each pair (near, 2 s - |near|) sums to 2 s
+            rest = (2 * s - np.abs(near)).astype(np.float32) * rng.choice(np.array([-1, 1], np.float32), 64)
+            w[n, g * group:(g + 1) * group] = rng.permutation(np.concatenate([near, rest]))
+    w[3, :group] = np.nan
+    w[4, 5] = np.inf
+    w[5, :group] = 0.0
+    wt = dev(w)
+    want_trits, want_scale = orc.absmean_ternary(w, group, "f16" if sdtype == torch.float16 else "bf16")
+    term = bp.absmean_ternary(wt, group, sdtype)
+    assert np.array_equal(term.scale.float().cpu().numpy(), want_scale, equal_nan=True)
+    assert np.array_equal(term.trits.cpu().numpy(), want_trits)
+    assert (np.abs(want_trits[8:]) == 0).mean() > 0.1 and (np.abs(want_trits[8:]) == 1).mean() > 0.5  # (both sides of the boundary occur)
+
+
 def test_packed_term_feeds_the_linear_like_the_training_graph(bp):
     """reference tests/test_qat.py:52-59 (BitLinear training graph == packed engine), K=131, group 64: the packed term
     made on the device, run through TernaryLinear, equals the dequantized product."""
