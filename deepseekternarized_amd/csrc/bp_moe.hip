@@ -290,8 +290,7 @@ static int moe_layer(bool v4, void* out, int out_dtype, float limit, const void*
   const bool prezeroed = aligned16 && !tiles;  // the zero-fill rides along with the gather (the GEMMs over the tile list write instead of accumulate)
   // The gate | up projection as the grouped GEMM over converted activations with SwiGLU in its epilogue (bf16 h written,
   // no float32 gate | up rows), where that kernel takes the call: over the tile list, bf16 activations. Its conversion
-  // pass then also does the row gather (rows read through `order`), unless the preparation kernel of small batches has
-  // done it anyway.
+  // pass then also does the row gather (rows read through `order`): no routed copy of the activations is written.
   GemmArgs fused;
   memset(&fused, 0, sizeof(fused));
   bool fuse = false;
@@ -306,17 +305,18 @@ static int moe_layer(bool v4, void* out, int out_dtype, float limit, const void*
     a.overwrite = 1; a.max_rows = TILE_ROWS;
     a.glu_h = (uint16_t*)p.h; a.glu_v4 = v4 ? 1 : 0; a.glu_limit = limit;
     a.glu_weights = v4 ? (const float*)weights : nullptr; a.glu_order = p.order; a.glu_pairs = n;
-    if (!small && aligned16 && tuning().glu != 'g') {  // (development: BP_TUNE_GLU=g keeps the gather a launch of its own)
+    if (aligned16 && tuning().glu != 'g') {  // (development: BP_TUNE_GLU=g keeps the gather a launch of its own)
       a.x = x; a.x_index = p.order; a.x_div = k; a.x_rows = T;
     }
     fuse = gemm_tiles_supported(a) && gemm_tq2f_applies(a) == BP_OK;
   }
   if (small) {
     const int64_t z0 = prezeroed ? (int64_t)(4 * (size_t)n * 2 * I / 16) : 0, z1 = prezeroed ? (int64_t)(4 * (size_t)n * H / 16) : 0;
-    int64_t g = (z0 + z1 + (int64_t)n * (H / 8) + ROUTE_SMALL_THREADS - 1) / ROUTE_SMALL_THREADS;
+    const int64_t row16 = fuse && fused.x_index ? 0 : H / 8;  // (no rows to copy where the gate | up launch reads them through `order`)
+    int64_t g = (z0 + z1 + (int64_t)n * row16 + ROUTE_SMALL_THREADS - 1) / ROUTE_SMALL_THREADS;
     g = g < 1 ? 1 : (g > 256 ? 256 : g);
     hipLaunchKernelGGL(k_route_small, dim3((unsigned)g), dim3(ROUTE_SMALL_THREADS), 0, s, p.order, p.offsets, p.inv, experts, (int)n, E, bad,
-                       (u32x4*)p.xg, (const u32x4*)x, (int)k, T, H / 8, (u32x4*)p.gu, z0, (u32x4*)p.y, z1, tiles ? p.tiles : nullptr, p.tile_count,
+                       (u32x4*)p.xg, (const u32x4*)x, (int)k, T, row16, (u32x4*)p.gu, z0, (u32x4*)p.y, z1, tiles ? p.tiles : nullptr, p.tile_count,
                        p.tile_cap);
     if ((rc = check_launch("route_small")) != BP_OK) return rc;
   } else {

@@ -419,6 +419,6 @@ def test_small_batch_preparation_kernel_writes_the_tile_list(T, E, k):
     if E == 4:
         logits[:, 1] += 6.0  # expert 1 is in every token's top-2: more than one tile
     got = moe(x, logits)
-    assert ext().last_kernel() == "gemm_tq1f_bf16+glu+y16", ext().last_kernel()
+    assert ext().last_kernel() == "gemm_tq1f_bf16+glu+gather+y16", ext().last_kernel()
     want = moe.composed(x, logits)
     assert torch.isfinite(got.float()).all() and torch.equal(got, want)
