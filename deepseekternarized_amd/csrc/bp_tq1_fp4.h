@@ -42,8 +42,13 @@ __device__ __forceinline__ u32x2 f4_load8(__amdgpu_buffer_rsrc_t r, unsigned lan
   return __builtin_bit_cast(u32x2, __builtin_amdgcn_raw_buffer_load_b64(r, (int)lane_off, (int)wave_off, 0));
 }
 
-// first packed byte (of the chunk's 128) of the byte pair behind half `hf` of A lane quarter `kbA` in instruction j
+// first packed byte (of the chunk's 128) of the byte pair behind half `hf` of A lane quarter `kbA` in instruction j.
+// MAP 0: B lane (n, kb) brings dword j % 4 of the 16-byte quarter kb of the 64-byte window j / 4 (the bytes as a lane
+// loaded them). MAP 1: it brings dword kb of the chunk's 16-byte piece j, so an instruction covers 80 consecutive
+// digits - at most two scale groups (the streaming kernel with four token rows per expert).
+template <int MAP = 0>
 __device__ __forceinline__ int f4_pair_byte(int j, int kbA, int hf) {
+  if (MAP == 1) return 16 * j + 4 * (2 * hf + (kbA >> 1)) + 2 * (kbA & 1);
   return 64 * (j >> 2) + 16 * (2 * hf + (kbA >> 1)) + 4 * (j & 3) + 2 * (kbA & 1);
 }
 
@@ -77,7 +82,7 @@ __device__ __forceinline__ void f4_build_table() {
 // behind the table (from LDS byte AT) by the workgroup's first `builders` waves (the caller synchronises afterwards).
 struct F4Nothing { __device__ __forceinline__ void operator()() const {} };
 // `meanwhile` runs after the wave's first activations are requested and before they are used.
-template <int NTOK, int WAVES, int AT = F4_LUT_BYTES, typename Meanwhile = F4Nothing>
+template <int NTOK, int WAVES, int AT = F4_LUT_BYTES, int MAP = 0, typename Meanwhile = F4Nothing>
 __device__ __forceinline__ void f4_build_tiles(const GemmArgs& a, int64_t tok, int ntok, int nchunks, int cb, int wave, int lane, int builders = WAVES, Meanwhile meanwhile = Meanwhile()) {
   constexpr int PC = f4_pieces(NTOK);
   constexpr int F4_HI_OFF = F4Tile<PC>::HI_OFF, F4_ZERO_OFF = F4Tile<PC>::ZERO_OFF, F4_PRE_OFF = F4Tile<PC>::PRE_OFF;
@@ -91,7 +96,7 @@ __device__ __forceinline__ void f4_build_tiles(const GemmArgs& a, int64_t tok, i
   // maximum over the float bits -> the groups' prescales 2^sh (sh brings the group's largest magnitude into [128, 256))
   // and their inverses -> 3 pieces x (first-group block, second-group block).
   const int blk = lane;
-  const int tt0 = 5 * f4_pair_byte(blk >> 3, (blk >> 1) & 3, blk & 1), glo = tt0 >> 7, ghi = (tt0 + 9) >> 7;
+  const int tt0 = 5 * f4_pair_byte<MAP>(blk >> 3, (blk >> 1) & 3, blk & 1), glo = tt0 >> 7, ghi = (tt0 + 9) >> 7;
   // (a wave with several items requests the next item's activations before it works on the current one's)
   // The lane's 10 activations come as one 20-byte piece (16-bit) or as the three dwords around their 10 bytes (int8)
   // through a buffer over the whole tensor: what lies past it reads as zero, what lies past the row is masked below.
@@ -232,6 +237,30 @@ __device__ __forceinline__ void f4_block_offsets(int r16, int kb, unsigned (&aof
       unsigned o = F4_ZERO_OFF / 16;
       if (am_used && g == glo) o = PC * blk + am_p;
       else if (am_used && g == ghi) o = F4_HI_OFF / 16 + PC * (ghi - 1) + am_p;
+      both |= o << (8 * hf);
+    }
+    if (j & 1) aoff[j >> 1] |= both << 16;
+    else aoff[j >> 1] = both;
+  }
+}
+
+// Four token rows per expert over byte map 1: row 8 s + 2 t + p = piece p of token t (which selects the token's tile, not
+// the block) in group slot s, and slot s of an instruction holds the group of its 80 digits whose number has parity s.
+// An accumulator tile may collect instructions as long as neither slot changes its group: instructions 0-2 (groups 0 | 1),
+// 3 (2 | 1), 4-5 (2 | 3), 6-7 (4 | 3).
+__device__ __forceinline__ void f4_block_offsets4(int r16, int kb, unsigned (&aoff)[4]) {
+  constexpr int PC = 2, F4_HI_OFF = F4Tile<PC>::HI_OFF, F4_ZERO_OFF = F4Tile<PC>::ZERO_OFF;
+  const int am_s = r16 >> 3, am_p = r16 & 1;
+#pragma unroll
+  for (int j = 0; j < 8; ++j) {
+    unsigned both = 0;
+#pragma unroll
+    for (int hf = 0; hf < 2; ++hf) {
+      const int blk = j * 8 + kb * 2 + hf;
+      const int tt0 = 5 * f4_pair_byte<1>(j, kb, hf), glo = tt0 >> 7, ghi = (tt0 + 9) >> 7;
+      unsigned o = F4_ZERO_OFF / 16;
+      if ((glo & 1) == am_s) o = PC * blk + am_p;
+      else if (ghi != glo) o = F4_HI_OFF / 16 + PC * (ghi - 1) + am_p;
       both |= o << (8 * hf);
     }
     if (j & 1) aoff[j >> 1] |= both << 16;

@@ -49,7 +49,12 @@ constexpr int64_t cw_buffer_bytes(int64_t Kp, int64_t G, int64_t scale_bytes) { 
 // and a multiplier's registers hold the pair's chunk (the same 8 x 8 registers).
 template <int SDT, int LPW, int TPB, int NTOK = 1>
 __global__ __launch_bounds__(CW_WAVES * 64) void k_tq1_gemv_cw(GemmArgs a, int nchunks, int groups, int tiles_per_wg, int first_row) {
-  static_assert(NTOK == 1 || NTOK == 2, "one token row per expert, or a pair");
+  static_assert(NTOK == 1 || NTOK == 2 || NTOK == 4, "one token row per expert, a pair, or four");
+  // NTOK = 4: the multipliers read their rows' bytes piece by piece (byte map 1 of bp_tq1_fp4.h), so that a matrix
+  // instruction covers 80 consecutive digits = at most two scale groups and the 16 rows of operand A are 2 group slots x
+  // 4 tokens x 2 pieces; four accumulator tiles per chunk. The four tokens' tiles (108 KiB at K = 7168) are built from
+  // LDS address 0, where the table goes once the multipliers have their operand in registers.
+  constexpr bool M4 = NTOK == 4;
   constexpr int WAVES = CW_WAVES, THREADS = WAVES * 64, NB = 2 * TPB, PC = f4_pieces(NTOK), SB = SDT == BP_F32 ? 4 : 2;
   constexpr int F4_INV_OFF = F4Tile<PC>::INV_OFF, F4_CHUNK_BYTES = F4Tile<PC>::CHUNK_BYTES, AT = CW_LUT_BYTES;
   const int wave = __builtin_amdgcn_readfirstlane((int)(threadIdx.x >> 6)), lane = threadIdx.x & 63;
@@ -88,7 +93,8 @@ __global__ __launch_bounds__(CW_WAVES * 64) void k_tq1_gemv_cw(GemmArgs a, int n
   // operand A tiles, which are built in the buffers' place): read from memory now, parked in LDS before the first
   // barrier, added to there tile by tile, and written back once after the last term - no access to the outputs in the loop.
   const int stream_bytes = groups * NB * (buf_bytes + nchunks * 64 * NTOK), build_bytes = nchunks * NTOK * F4_CHUNK_BYTES;
-  const unsigned stage = (unsigned)(AT + (stream_bytes > build_bytes ? stream_bytes : build_bytes));
+  const unsigned stage = M4 ? (unsigned)(AT + stream_bytes > build_bytes ? AT + stream_bytes : build_bytes)
+                            : (unsigned)(AT + (stream_bytes > build_bytes ? stream_bytes : build_bytes));
   const int n_stage = (int)(tile_end - tile0) * 16 * NTOK;  // (at most CW_STAGE_PER_THREAD x the workgroup's threads: the launcher's bound)
   auto out_index = [&](int o) -> int64_t { return (tok + ((o >> 4) % NTOK)) * a.N + (tile0 + (o >> 4) / NTOK) * 16 + (o & 15); };
   float was[CW_STAGE_PER_THREAD];
@@ -167,10 +173,11 @@ __global__ __launch_bounds__(CW_WAVES * 64) void k_tq1_gemv_cw(GemmArgs a, int n
     setup_term(0);
     request(0, IC<0>{});
     request(1, IC<1>{});
-    build_table();
-  } else {  // (chunk by chunk, by the multipliers; their part of the table while the activations are on their way)
+    if constexpr (!M4) build_table();
+  } else if constexpr (!M4) {  // (chunk by chunk, by the multipliers; their part of the table while the activations are on their way)
     f4_build_tiles<NTOK, WAVES, AT>(a, tok, ntok, nchunks, 0, wave, lane, active, build_table);
   }
+  if constexpr (M4) f4_build_tiles<NTOK, WAVES, 0, 1>(a, tok, ntok, nchunks, 0, wave, lane, WAVES);  // (all waves, where the table will be)
 
 #pragma unroll
   for (int u = 0; u < CW_STAGE_PER_THREAD; ++u) {
@@ -185,12 +192,14 @@ __global__ __launch_bounds__(CW_WAVES * 64) void k_tq1_gemv_cw(GemmArgs a, int n
     // window and of the second (kb and 3, 4, 2, 2 for kb = 0..3; the lanes kb = 3 hold unused rows: their sums are 0)
     i32x8 A[8];
     float inv_a[NTOK], inv_b[NTOK];
-    const int g_w0 = NTOK == 1 ? kb : kb < 3 ? kb : 2, g_w1 = NTOK == 1 ? 4 : kb == 0 ? 3 : kb == 1 ? 4 : 2;
+    float inv_c[2] = {0.f, 0.f};  // (M4: the lane's third group)
+    const int g_w0 = M4 ? kb >> 1 : NTOK == 1 ? kb : kb < 3 ? kb : 2, g_w1 = M4 ? 2 + (kb >> 1) : NTOK == 1 ? 4 : kb == 0 ? 3 : kb == 1 ? 4 : 2;
     {
       unsigned aoff[4];
-      f4_block_offsets<PC>(r16, kb, aoff);
-      const unsigned cbase = (unsigned)(AT + c * NTOK * F4_CHUNK_BYTES);
-      const unsigned mine = cbase + (NTOK == 2 ? (unsigned)(((r16 >> 1) & 1) * F4_CHUNK_BYTES) : 0u);
+      if constexpr (M4) f4_block_offsets4(r16, kb, aoff);
+      else f4_block_offsets<PC>(r16, kb, aoff);
+      const unsigned cbase = (unsigned)((M4 ? 0 : AT) + c * NTOK * F4_CHUNK_BYTES);
+      const unsigned mine = cbase + (M4 ? (unsigned)(((r16 >> 1) & 3) * F4_CHUNK_BYTES) : NTOK == 2 ? (unsigned)(((r16 >> 1) & 1) * F4_CHUNK_BYTES) : 0u);
 #pragma unroll
       for (int j = 0; j < 8; ++j) {
         const u32x4 lo = *(const lds_u32x4*)((((aoff[j >> 1] >> (16 * (j & 1))) & 0xffu) << 4) + mine);
@@ -198,10 +207,21 @@ __global__ __launch_bounds__(CW_WAVES * 64) void k_tq1_gemv_cw(GemmArgs a, int n
         A[j] = i32x8{(int)lo.x, (int)lo.y, (int)lo.z, (int)lo.w, (int)hi.x, (int)hi.y, (int)hi.z, (int)hi.w};
       }
       const float f4th = kb == 3 ? 0.f : kb == 2 ? 1.f / 256.f : 1.f;
+      if constexpr (M4) {  // the lane's two tokens 2 (kb % 2) + t; slot 0 lanes: groups 0, 2, 4, slot 1 lanes: 1, 3
 #pragma unroll
-      for (int tt = 0; tt < NTOK; ++tt) {
-        inv_a[tt] = __uint_as_float(*(const lds_u32*)(cbase + tt * F4_CHUNK_BYTES + F4_INV_OFF + 4 * g_w0));
-        inv_b[tt] = __uint_as_float(*(const lds_u32*)(cbase + tt * F4_CHUNK_BYTES + F4_INV_OFF + 4 * g_w1)) * (NTOK == 1 ? f4th : 1.f);
+        for (int t2 = 0; t2 < 2; ++t2) {
+          const unsigned tile = cbase + (unsigned)((2 * (kb & 1) + t2) * F4_CHUNK_BYTES + F4_INV_OFF);
+          inv_a[t2] = __uint_as_float(*(const lds_u32*)(tile + 4 * g_w0));
+          inv_b[t2] = __uint_as_float(*(const lds_u32*)(tile + 4 * g_w1));
+          inv_c[t2] = (kb >> 1) ? 0.f : __uint_as_float(*(const lds_u32*)(tile + 4 * 4));
+          inv_a[t2 + 2] = inv_b[t2 + 2] = 0.f;
+        }
+      } else {
+#pragma unroll
+        for (int tt = 0; tt < NTOK; ++tt) {
+          inv_a[tt] = __uint_as_float(*(const lds_u32*)(cbase + tt * F4_CHUNK_BYTES + F4_INV_OFF + 4 * g_w0));
+          inv_b[tt] = __uint_as_float(*(const lds_u32*)(cbase + tt * F4_CHUNK_BYTES + F4_INV_OFF + 4 * g_w1)) * (NTOK == 1 ? f4th : 1.f);
+        }
       }
     }
     const unsigned lane4 = (unsigned)lane << 2;
@@ -212,7 +232,14 @@ __global__ __launch_bounds__(CW_WAVES * 64) void k_tq1_gemv_cw(GemmArgs a, int n
     const int64_t ga = (5 * (int64_t)c + g_w0) >> gs, gb = (5 * (int64_t)c + g_w1) >> gs;
     const unsigned rd_sa = (unsigned)(16 * pitch + r16 * (int)(a.G * SB) + SB * (int)(ga < g_last ? ga : g_last));
     const unsigned rd_sb = (unsigned)(16 * pitch + r16 * (int)(a.G * SB) + SB * (int)(gb < g_last ? gb : g_last));
+    const int64_t gc = (5 * (int64_t)c + 4) >> gs;
+    const unsigned rd_sc = (unsigned)(16 * pitch + r16 * (int)(a.G * SB) + SB * (int)(gc < g_last ? gc : g_last));  // (M4)
+    const unsigned rd_w4 = (unsigned)(r16 * pitch + 128 * c + 4 * kb);                                             // (M4: dword kb of piece j at + 16 j)
     __syncthreads();  // (every multiplier has its operand A: the tile buffers may overwrite the tiles)
+    if constexpr (M4) {
+      build_table();
+      __syncthreads();
+    }
 
     for (int term = 0; term < a.n_terms; ++term) {
       const unsigned mis = (unsigned)((uintptr_t)(a.packed[term] + e * a.N * a.Kp) & 3);
@@ -270,11 +297,64 @@ __global__ __launch_bounds__(CW_WAVES * 64) void k_tq1_gemv_cw(GemmArgs a, int n
           if (kb == 0) *(lds_u32*)(red + (unsigned)((((t % NB) * nchunks + c) * NTOK + tt) * 64 + 4 * r16)) = __float_as_uint(v);
         }
       };
+      // Four token rows: instruction j multiplies piece j of the chunk (the lane's dword kb of it and the dword behind it,
+      // for the realignment); accumulator tiles 0 .. 3 take instructions 0-2, 3, 4-5, 6-7. A lane of the result holds
+      // slot kb / 2 of tokens 2 (kb % 2) and 2 (kb % 2) + 1: the sums of the slot's groups under their scales and the
+      // tokens' inverse prescales, and the other slot's lane (kb ^ 2) has the rest of the row's sum.
+      auto multiply4 = [&](int t) {
+        const unsigned rb = gbase + (unsigned)((t % NB) * buf_bytes);
+        const unsigned ra = SB == 4 ? *(const lds_u32*)(rb + rd_sa) : (unsigned)*(const lds_u16*)(rb + rd_sa);
+        const unsigned rbits = SB == 4 ? *(const lds_u32*)(rb + rd_sb) : (unsigned)*(const lds_u16*)(rb + rd_sb);
+        const unsigned rcb = SB == 4 ? *(const lds_u32*)(rb + rd_sc) : (unsigned)*(const lds_u16*)(rb + rd_sc);
+        constexpr int BD = 2;
+        u32x4 Bq[BD + 1];
+        auto lookup = [&](auto j_c) {
+          constexpr int j = decltype(j_c)::value;
+          const unsigned cur = *(const lds_u32*)(rb + rd_w4 + 16 * j), nxt = *(const lds_u32*)(rb + rd_w4 + 16 * j + 4);
+          const unsigned d = __builtin_amdgcn_alignbyte(nxt, cur, dlt);
+#pragma unroll
+          for (int w = 0; w < 4; ++w) Bq[j % (BD + 1)][w] = *(const lds_u32*)__builtin_amdgcn_perm(d, lane4, 0x0c0c0400u + ((unsigned)w << 8));
+        };
+        f32x4 C[4];
+#pragma unroll
+        for (int q = 0; q < 4; ++q) C[q] = f32x4{0.f, 0.f, 0.f, 0.f};
+        lookup(IC<0>{});
+        lookup(IC<1>{});
+        auto stage4 = [&](auto j_c) {
+          constexpr int j = decltype(j_c)::value, ci = j < 3 ? 0 : j == 3 ? 1 : j < 6 ? 2 : 3;
+          __builtin_amdgcn_sched_barrier(0);
+          if (j + BD < 8) lookup(IC<(j + BD < 8 ? j + BD : 0)>{});
+          __builtin_amdgcn_sched_barrier(0);
+          const u32x4 bq = Bq[j % (BD + 1)];
+          const i32x8 B8 = {(int)bq.x, (int)bq.y, (int)bq.z, (int)bq.w, 0, 0, 0, 0};
+          C[ci] = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(A[j], B8, C[ci], 0 /* A: E4M3 */, 4 /* B: E2M1 */, 0, 0, 0, 0);
+        };
+        stage4(IC<0>{}); stage4(IC<1>{}); stage4(IC<2>{}); stage4(IC<3>{}); stage4(IC<4>{}); stage4(IC<5>{}); stage4(IC<6>{}); stage4(IC<7>{});
+        __builtin_amdgcn_sched_barrier(0);
+        auto widen = [&](unsigned r) { return SDT == BP_F32 ? __uint_as_float(r) : SDT == BP_F16 ? f16_bits_to_f32((uint16_t)r) : __uint_as_float(r << 16); };
+        const float sa = widen(ra), sb = widen(rbits), sc = widen(rcb);
+        const bool odd = (kb >> 1) != 0;  // the lane's slot
+#pragma unroll
+        for (int t2 = 0; t2 < 2; ++t2) {
+          const float p0 = C[0][2 * t2] + C[0][2 * t2 + 1], p1 = C[1][2 * t2] + C[1][2 * t2 + 1];
+          const float p2 = C[2][2 * t2] + C[2][2 * t2 + 1], p3 = C[3][2 * t2] + C[3][2 * t2 + 1];
+          // slot 0: group 0 <- tile 0, group 2 <- tiles 1, 2, group 4 <- tile 3; slot 1: group 1 <- tiles 0, 1, group 3 <- tiles 2, 3
+          const float qa = odd ? p0 + p1 : p0, qb = odd ? p2 + p3 : p1 + p2;
+          float v = sa * inv_a[t2] * qa + sb * inv_b[t2] * qb + sc * inv_c[t2] * p3;
+          const auto h32 = __builtin_amdgcn_permlane32_swap(__float_as_uint(v), __float_as_uint(v), false, false);
+          v = __uint_as_float(h32[0]) + __uint_as_float(h32[1]);
+          const int tt = 2 * (kb & 1) + t2;
+          if (kb < 2) *(lds_u32*)(red + (unsigned)((((t % NB) * nchunks + c) * NTOK + tt) * 64 + 4 * r16)) = __float_as_uint(v);
+        }
+      };
       if (term > 0) __syncthreads();  // (the previous term's last tiles have been added)
       for (int i = 0; i < n_int; ++i) {
         __syncthreads();  // (the tiles TPB i .. TPB i + TPB - 1 are in their buffers)
 #pragma unroll
-        for (int u = 0; u < TPB; ++u) multiply(TPB * i + u);
+        for (int u = 0; u < TPB; ++u) {
+          if constexpr (M4) multiply4(TPB * i + u);
+          else multiply(TPB * i + u);
+        }
       }
       __syncthreads();
     }
@@ -283,6 +363,10 @@ __global__ __launch_bounds__(CW_WAVES * 64) void k_tq1_gemv_cw(GemmArgs a, int n
 
   // ---- loaders (and waves without a role, which only keep the barriers' count)
   __syncthreads();  // (the multipliers have their operand A)
+  if constexpr (M4) {
+    build_table();
+    __syncthreads();
+  }
   for (int term = 0; term < a.n_terms; ++term) {
     if (term > 0) setup_term(term);
     // The sums of the tile of iteration t, by the group's first loader: lane (row n, quarter q) adds chunks q, q + 4, ...
@@ -384,6 +468,7 @@ int launch_cw(const GemmArgs& a, hipStream_t s, int64_t nchunks, int cus, int fi
   auto lds_of = [&](int g, int tpb) {
     const int64_t stream = (int64_t)g * 2 * tpb * (buf + nchunks * 64 * NTOK), build = nchunks * NTOK * f4_chunk_bytes(NTOK);
     const int64_t mine = (per + g - 1) / g * g;  // tiles per workgroup with g groups
+    if (NTOK == 4) return (CW_LUT_BYTES + stream > build ? CW_LUT_BYTES + stream : build) + mine * 64 * NTOK;  // (the tiles are built from LDS address 0)
     return (int64_t)CW_LUT_BYTES + (stream > build ? stream : build) + mine * 64 * NTOK;
   };
   auto fits = [&](int g, int tpb) {
@@ -403,12 +488,13 @@ int launch_cw(const GemmArgs& a, hipStream_t s, int64_t nchunks, int cus, int fi
   if (force != 'c' && (groups * nchunks < 10 || per / groups < 48)) return BP_ERR_UNSUPPORTED;
   const dim3 grid((unsigned)((tiles + per - 1) / per), (unsigned)a.E, 1u);
   const size_t lds = (size_t)lds_of(groups, tpb);
-  note_kernel(NTOK == 1 ? "fp4_tq1_t1_cw" : "fp4_tq1_m2_cw");
+  const char* const kname = NTOK == 1 ? "fp4_tq1_t1_cw" : NTOK == 2 ? "fp4_tq1_m2_cw" : "fp4_tq1_m4_cw";
+  note_kernel(kname);
 #define BP_CW_LAUNCH(L, P)                                                                                                                  \
   {                                                                                                                                         \
     if (const int rc = raise_lds_limit<k_tq1_gemv_cw<SDT, L, P, NTOK>>(F4_LDS_MAX)) return rc;                                              \
     hipLaunchKernelGGL((k_tq1_gemv_cw<SDT, L, P, NTOK>), grid, dim3(CW_WAVES * 64), lds, s, a, (int)nchunks, groups, (int)per, first_row); \
-    return check_launch(NTOK == 1 ? "fp4_tq1_t1_cw" : "fp4_tq1_m2_cw");                                                                     \
+    return check_launch(kname);                                                                                                           \
   }
 #define BP_CW_LPW(L)        \
   if (lpw == L) {           \
@@ -424,6 +510,11 @@ int launch_cw(const GemmArgs& a, hipStream_t s, int64_t nchunks, int cus, int fi
 }  // namespace
 
 int launch_tq1_gemv_cw(const GemmArgs& a, hipStream_t s, int ntok, int64_t nchunks, int cus, int first_row) {
+  if (ntok == 4) {  // (2-byte scales)
+    if (a.scale_dtype == BP_F16) return launch_cw<BP_F16, 4>(a, s, nchunks, cus, first_row);
+    if (a.scale_dtype == BP_BF16) return launch_cw<BP_BF16, 4>(a, s, nchunks, cus, first_row);
+    return BP_ERR_UNSUPPORTED;
+  }
   if (ntok != 1 && ntok != 2) return BP_ERR_UNSUPPORTED;
   if (a.scale_dtype == BP_F16) return ntok == 1 ? launch_cw<BP_F16, 1>(a, s, nchunks, cus, first_row) : launch_cw<BP_F16, 2>(a, s, nchunks, cus, first_row);
   if (a.scale_dtype == BP_BF16) return ntok == 1 ? launch_cw<BP_BF16, 1>(a, s, nchunks, cus, first_row) : launch_cw<BP_BF16, 2>(a, s, nchunks, cus, first_row);

@@ -553,6 +553,12 @@ int launch_f4(const GemmArgs& a, hipStream_t s, int first_row = 0) {
       if (rc != BP_ERR_UNSUPPORTED) return rc;
     }
   }
+  if constexpr (NTOK == 4) {  // (four rows per expert in a large call: the same, a matrix instruction per 16-byte piece)
+    if (tuning().tq1 != 'r') {
+      const int rc = launch_tq1_gemv_cw(a, s, 4, nchunks, cus, first_row);
+      if (rc != BP_ERR_UNSUPPORTED) return rc;
+    }
+  }
   if (NTOK > 1) {
     const bool wide = lds > (size_t)F4_LDS_MAX / 2 || ((a.N + 255) / 256) * experts >= 4 * (int64_t)cus;
     const char* name8 = NTOK == 2 ? "fp4_tq1_m2_w8" : NTOK == 4 ? "fp4_tq1_m4_w8" : NTOK == 6 ? "fp4_tq1_m6_w8" : "fp4_tq1_m8_w8";

@@ -202,6 +202,21 @@ def test_tq1_gemv_chunk_per_wave_token_pairs(bp, tune, K, counts, act):
     _check(got, want)
 
 
+@pytest.mark.parametrize("K,counts,act", [(1024, [4, 0, 3], "bf16"), (7168, [4, 3, 1], "int8"), (2304, [3, 4], "bf16"), (4352, [4, 4], "int8"),
+                                          (7168, [4, 4, 4], "bf16")])
+def test_tq1_gemv_chunk_per_wave_four_rows(bp, tune, K, counts, act):
+    """The same kernel with up to four token rows per expert: a matrix instruction per 16-byte piece of a row (80
+    consecutive digits, at most two scale groups), operand rows = 2 group slots x 4 tokens x 2 pieces, four accumulator
+    tiles per chunk; experts with four, three, one and no rows; two stacked terms; N not a multiple of a workgroup's tiles."""
+    tune("BP_TUNE_TQ1", "chunk")
+    got, want, kern = _run(bp, "tq1", len(counts), 2048 + 48, K, counts, act, terms=2, seed=K + 4)
+    assert kern == "fp4_tq1_m4_cw", kern
+    _check(got, want)
+    got, want, kern = _run(bp, "tq1", len(counts), 272, K, counts, act, seed=K + 5, scale_dtype=np.float16, group=256 if K % 512 == 0 and K >= 2048 else 128)
+    assert kern == "fp4_tq1_m4_cw", kern
+    _check(got, want)
+
+
 def test_tq1_gemv_chunk_per_wave_pair_after_launches_of_eight(bp, tune):
     """Up to 10 rows per expert where most experts have few: a launch of 8 rows, then the rows 8 and 9 as a pair."""
     tune("BP_TUNE_TQ1", "chunk")
