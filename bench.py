@@ -85,6 +85,9 @@ WORKLOADS = {
     "cfg1b_tq1_gemv": ("tq1", 7168, 2048, 1, "bf16", 1, 128),
     "cfg1a_tq1_m2": ("tq1", 2048, 7168, 2, "bf16", 1, 128),
     "cfg1a_tq1_m4": ("tq1", 2048, 7168, 4, "bf16", 1, 128),
+    "cfg1a_tq1_m3": ("tq1", 2048, 7168, 3, "bf16", 1, 128),
+    "cfg1a_tq1_m6": ("tq1", 2048, 7168, 6, "bf16", 1, 128),
+    "cfg1a_tq1_m8": ("tq1", 2048, 7168, 8, "bf16", 1, 128),
     "cfg1a_tq1_m16": ("tq1", 2048, 7168, 16, "bf16", 1, 128),
     "cfg1a_tq1_m32": ("tq1", 2048, 7168, 32, "bf16", 1, 128),
     "cfg1b_tq1_m16": ("tq1", 7168, 2048, 16, "bf16", 1, 128),

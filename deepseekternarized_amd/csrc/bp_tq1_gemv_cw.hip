@@ -22,7 +22,7 @@ namespace {
 //    token's operand A in registers (8 instructions x 8 registers) and multiplies chunk c of every tile: no operand A
 //    reads in the loop. A group is nchunks multipliers and its loaders; groups walk over their own tiles (tile index =
 //    group mod groups);
-//  * a multiplier's 16 partial sums of a tile (one per row) go to LDS, and the group's first loader adds the chunks' sums
+//  * a multiplier's 16 partial sums of a tile (one per row) go to LDS, and the group's loaders (token t by loader t mod their number) add the chunks' sums
 //    in a fixed order and adds the result to the row's entry of the workgroup's outputs, which wait in LDS too: read
 //    from memory when the workgroup starts, written back once after the last term.
 // A barrier hands over TPB tiles: two where four tile buffers fit beside the table (the loaders' waits for memory and
@@ -369,14 +369,16 @@ __global__ __launch_bounds__(CW_WAVES * 64) void k_tq1_gemv_cw(GemmArgs a, int n
   }
   for (int term = 0; term < a.n_terms; ++term) {
     if (term > 0) setup_term(term);
-    // The sums of the tile of iteration t, by the group's first loader: lane (row n, quarter q) adds chunks q, q + 4, ...
-    // in that order, the row's four lanes are added in a fixed order too, and the row's entry of the output stage takes
-    // one addition (this wave is the only one that touches its group's entries between the first barrier and the end).
+    // The sums of the tile of iteration t, token tt by the group's loader tt % lpg: lane (row n, quarter q) adds chunks q,
+    // q + 4, ... in that order, the row's four lanes are added in a fixed order too, and the row's entry of the output
+    // stage takes one addition (this wave is the only one that touches its tokens' entries of its group between the
+    // first barrier and the end).
     auto reduce = [&](int t, auto) {
-      if (!loader || lidx != 0) return;  // (uniform)
+      if (!loader) return;  // (uniform)
       const int64_t tile = tile_of(t);
 #pragma unroll
       for (int tt = 0; tt < NTOK; ++tt) {
+        if (tt % lpg != lidx) continue;  // (uniform)
         float v = 0.f;
 #pragma unroll
         for (int q = 0; q < CW_WAVES / 4; ++q) {
@@ -427,14 +429,14 @@ __global__ __launch_bounds__(CW_WAVES * 64) void k_tq1_gemv_cw(GemmArgs a, int n
     if (TPB == 2 || (n_int & 1) == 0) reduce(TPB * n_int - 1, IC<1>{});
     else reduce(n_int - 1, IC<0>{});
   }
-  // ---- the group's first loader writes its tiles' outputs back: the entries it has added to itself (no barrier), four
+  // ---- the group's loaders write their tokens' outputs back: the entries a wave has added to itself (no barrier), four
   // tiles per wave store
-  if (loader && lidx == 0) {
+  if (loader) {
     for (int t = kb; t < n_iter; t += 4) {
       const int64_t tile = tile_of(t);
 #pragma unroll
       for (int tt = 0; tt < NTOK; ++tt) {
-        if (tile < tile_end && tt < ntok)
+        if (tt % lpg == lidx && tile < tile_end && tt < ntok)
           a.out[(tok + tt) * a.N + tile * 16 + r16] = __uint_as_float(*(const lds_u32*)(stage + (unsigned)((((int)(tile - tile0) * NTOK + tt) * 16 + r16) * 4)));
       }
     }
