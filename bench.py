@@ -92,6 +92,9 @@ WORKLOADS = {
     "cfg1a_tq1_m32": ("tq1", 2048, 7168, 32, "bf16", 1, 128),
     "cfg1b_tq1_m16": ("tq1", 7168, 2048, 16, "bf16", 1, 128),
     "cfg1b_tq1_m32": ("tq1", 7168, 2048, 32, "bf16", 1, 128),
+    "cfg1a_tq2_m2": ("tq2", 2048, 7168, 2, "bf16", 1, 128),
+    "cfg1a_tq2_m4": ("tq2", 2048, 7168, 4, "bf16", 1, 128),
+    "cfg1a_tq2_m8": ("tq2", 2048, 7168, 8, "bf16", 1, 128),
     "cfg1a_tq2_m16": ("tq2", 2048, 7168, 16, "bf16", 1, 128),
     "cfg1a_tq2_gemv": ("tq2", 2048, 7168, 1, "bf16", 1, 128),
     "cfg0_tq2_gemv": ("tq2", 2048, 4096, 1, "bf16", 1, 192),
