@@ -92,15 +92,23 @@ __device__ __forceinline__ void kv_widen_run(const GemmArgs& a, const KvRun& r, 
   }
 }
 
-template <int SDT>
+// NTOK = 2: a pair of token rows per expert (bf16 / int8 activations: two fp8 pieces suffice, as in the small-batch TQ1
+// kernels - exact down to 2^-9 of a group's largest magnitude, at most 2^-17 of it dropped below). Row 4 g + 2 t + p of
+// operand A is piece p of token t in group g: the same 4 x 8 registers per wave, one accumulator tile per row tile, and
+// a lane of the result holds both tokens' pieces of group kb.
+template <int SDT, int NTOK = 1>
 __global__ __launch_bounds__(1024) void k_tq2_gemv_ks(GemmArgs a, int nw, int tiles_per_wg) {
+  static_assert(NTOK == 1 || NTOK == 2, "one token row per expert, or a pair");
   constexpr int SB = SDT == BP_F32 ? 4 : 2, NSL = SB / 2;  // bytes per scale; a wave's 16-byte loads of a round's scales
   const int wave = __builtin_amdgcn_readfirstlane((int)(threadIdx.x >> 6)), lane = threadIdx.x & 63;
   const int n = lane & 15, kb = lane >> 4;
   const int64_t e = blockIdx.y;
   const int64_t tok = clamp_i64(a.offsets[e], 0, a.T), o1 = clamp_i64(a.offsets[e + 1], 0, a.T);
   if (tok >= o1) return;  // (uniform: an expert without a token row)
-  const float xsc = a.x_dtype == BP_I8 ? a.x_scale[tok] : 1.f;
+  const int ntok = o1 - tok < NTOK ? (int)(o1 - tok) : NTOK;
+  float xsc[NTOK];
+#pragma unroll
+  for (int tt = 0; tt < NTOK; ++tt) xsc[tt] = a.x_dtype == BP_I8 && tt < ntok ? a.x_scale[tok + tt] : 1.f;
   const int gs = a.group == 256 ? 1 : 0;
   const int64_t tiles = a.N / 16;
   const int64_t tile0 = (int64_t)blockIdx.x * tiles_per_wg;
@@ -109,7 +117,7 @@ __global__ __launch_bounds__(1024) void k_tq2_gemv_ks(GemmArgs a, int nw, int ti
 
   // ---- LDS: two slots of a round's scales, then two of a round's partial sums [tile][wave][row]
   const unsigned row_sb = (unsigned)(a.G * SB), tile_sb = 16 * row_sb, slot_bytes = KV_R * tile_sb;
-  const unsigned RED = 2 * slot_bytes;  // [tile of the workgroup][wave][row]
+  const unsigned RED = 2 * slot_bytes;  // [tile of the workgroup][wave][token][row]
   const int64_t g128 = 2 * KV_S * (int64_t)wave + kb;  // the lane's group of 128 as a column of the result
   const bool g_real = 128 * g128 < a.K;
   const unsigned rd_s = (unsigned)n * row_sb + (unsigned)SB * (unsigned)(g_real ? g128 >> gs : 0);
@@ -118,20 +126,25 @@ __global__ __launch_bounds__(1024) void k_tq2_gemv_ks(GemmArgs a, int nw, int ti
 
   // The lane as a row of operand A: piece p of the wave's group gl (p = 3: unused); its 2 x 16 activations are requested
   // first, the first tiles next, and operand A is built while those are on their way.
-  const int gl = n >> 2, p = n & 3;
+  const int gl = n >> 2, p = NTOK == 2 ? n & 1 : n & 3, trow = NTOK == 2 ? (n >> 1) & 1 : 0;  // (a pair: the lane's token)
   const int64_t kbase = 256 * KV_S * (int64_t)wave + 128 * gl + 64 * (kb >> 1) + 16 * (kb & 1);
-  const KvRun x_lo = kv_load_run(a, tok, kbase), x_hi = kv_load_run(a, tok, kbase + 32);
+  // (an expert with one row of the pair: the absent token's rows of operand A hold zeros, its sums are not stored)
+  const int64_t kx = trow < ntok ? kbase : a.K;
+  const KvRun x_lo = kv_load_run(a, tok + trow, kx), x_hi = kv_load_run(a, tok + trow, kx + 32);
   // Thread o of the workgroup owns output o of the workgroup's rows (up to KV_OPT of them: o + a multiple of the
   // workgroup's threads): what the call adds to is read now and written back once, after the last term.
-  const int n_out = (int)(tile_end - tile0) * 16;
+  // (a pair: output o = ((tile * 2 + token) * 16 + row)
+  const int n_out = (int)(tile_end - tile0) * 16 * NTOK;
+  auto out_at = [&](int o) -> int64_t { return (tok + ((o >> 4) % NTOK)) * a.N + tile0 * 16 + ((o >> 4) / NTOK) * 16 + (o & 15); };
+  auto out_live = [&](int o) { return o < n_out && ((o >> 4) % NTOK) < ntok; };
   float total[KV_OPT];
 #pragma unroll
   for (int u = 0; u < KV_OPT; ++u) {
     const int o = (int)threadIdx.x + u * nw * 64;
-    total[u] = o < n_out ? a.out[tok * a.N + tile0 * 16 + o] : 0.f;
+    total[u] = out_live(o) ? a.out[out_at(o)] : 0.f;
   }
   i32x8 A[2 * KV_S];
-  float cinit[3], inv2;
+  float cinit[4], inv2[NTOK];
 
   // (the expert's rows and scales of a term as buffers of their own: what lies past them reads as zeros)
   __amdgpu_buffer_rsrc_t wrs = make_rsrc(a.packed[0] + e * a.N * a.Kp, a.N * a.Kp);
@@ -158,7 +171,7 @@ __global__ __launch_bounds__(1024) void k_tq2_gemv_ks(GemmArgs a, int nw, int ti
     constexpr int i = decltype(i_c)::value, slot = i % KV_D;
     const unsigned sat = (unsigned)(r & 1) * slot_bytes + (unsigned)i * tile_sb + rd_s;
     const unsigned raw = SB == 4 ? *(const lds_u32*)sat : (unsigned)*(const lds_u16*)sat;
-    f32x4 C = {cinit[0], cinit[1], cinit[2], 0.f};
+    f32x4 C = {cinit[0], cinit[1], cinit[2], NTOK == 2 ? cinit[3] : 0.f};
 #pragma unroll
     for (int s = 0; s < KV_S; ++s) {
       const u32x4 W = ring[slot][s];
@@ -171,9 +184,12 @@ __global__ __launch_bounds__(1024) void k_tq2_gemv_ks(GemmArgs a, int nw, int ti
     }
     request(KV_R * r + i + KV_D, IC<slot>{});
     const float sc = SDT == BP_F32 ? __uint_as_float(raw) : SDT == BP_F16 ? f16_bits_to_f32((uint16_t)raw) : __uint_as_float(raw << 16);
-    float v = g_real ? sc * inv2 * (C[0] + C[1] + C[2] * (1.f / 256.f)) : 0.f;
-    v = kv_quad_sum(v);
-    if (kb == 0) *(lds_u32*)(RED + (unsigned)(((KV_R * r + i) * nw + wave) * 64 + 4 * n)) = __float_as_uint(v);
+#pragma unroll
+    for (int tt = 0; tt < NTOK; ++tt) {
+      float v = !g_real ? 0.f : NTOK == 2 ? sc * inv2[tt] * (C[2 * tt] + C[2 * tt + 1]) : sc * inv2[0] * (C[0] + C[1] + C[2] * (1.f / 256.f));
+      v = kv_quad_sum(v);
+      if (kb == 0) *(lds_u32*)(RED + (unsigned)((((KV_R * r + i) * nw + wave) * NTOK + tt) * 64 + 4 * n)) = __float_as_uint(v);
+    }
   };
 
   auto first_requests = [&] {  // a term's first loads: the scales of round 0, the ring's tiles
@@ -244,8 +260,9 @@ __global__ __launch_bounds__(1024) void k_tq2_gemv_ks(GemmArgs a, int nw, int ti
     hs += __shfl_xor(hs, 16, 64);
     hs += __shfl_xor(hs, 32, 64);
 #pragma unroll
-    for (int i = 0; i < 3; ++i) cinit[i] = -0.5f * __shfl(hs, 4 * kb + i, 64);  // (the lane as a column of the result: group kb)
-    inv2 = __shfl(inv, 4 * kb, 64);
+    for (int i = 0; i < 4; ++i) cinit[i] = -0.5f * __shfl(hs, 4 * kb + i, 64);  // (the lane as a column of the result: group kb; one token: row 3 is unused, its sum 0)
+#pragma unroll
+    for (int tt = 0; tt < NTOK; ++tt) inv2[tt] = __shfl(inv, 4 * kb + 2 * tt, 64);
 #pragma unroll
     for (int j = 0; j < 2 * KV_S; ++j) {
 #pragma unroll
@@ -274,16 +291,17 @@ __global__ __launch_bounds__(1024) void k_tq2_gemv_ks(GemmArgs a, int nw, int ti
     for (int u = 0; u < KV_OPT; ++u) {
       const int o = (int)threadIdx.x + u * nw * 64;
       if (o < n_out) {
+        const int tl = (o >> 4) / NTOK, tt = (o >> 4) % NTOK;
         float v = 0.f;
-        for (int c = 0; c < nw; ++c) v += __uint_as_float(*(const lds_u32*)(RED + (unsigned)((((o >> 4) * nw + c) * 16 + (o & 15)) * 4)));
-        total[u] += a.x_dtype == BP_I8 ? v * xsc : v;
+        for (int c = 0; c < nw; ++c) v += __uint_as_float(*(const lds_u32*)(RED + (unsigned)((((tl * nw + c) * NTOK + tt) * 16 + (o & 15)) * 4)));
+        total[u] += a.x_dtype == BP_I8 ? v * (NTOK == 2 && tt ? xsc[NTOK - 1] : xsc[0]) : v;
       }
     }
   }
 #pragma unroll
   for (int u = 0; u < KV_OPT; ++u) {
     const int o = (int)threadIdx.x + u * nw * 64;
-    if (o < n_out) a.out[tok * a.N + tile0 * 16 + o] = total[u];
+    if (out_live(o)) a.out[out_at(o)] = total[u];
   }
 }
 
@@ -301,13 +319,17 @@ int kv_cus() {  // compute units of the current device (256 if the query fails)
   return known[dev];
 }
 
-template <int SDT>
-int launch_kv(const GemmArgs& a, hipStream_t s, int nw, int64_t per, const dim3& grid, size_t lds) {
-  const char* name = a.x_dtype == BP_I8 ? "fp4_tq2_i8_t1_ks" : "fp4_tq2_t1_ks";
+template <int SDT, int NTOK>
+int launch_kv_n(const GemmArgs& a, hipStream_t s, int nw, int64_t per, const dim3& grid, size_t lds) {
+  const char* name = NTOK == 2 ? (a.x_dtype == BP_I8 ? "fp4_tq2_i8_m2_ks" : "fp4_tq2_m2_ks") : a.x_dtype == BP_I8 ? "fp4_tq2_i8_t1_ks" : "fp4_tq2_t1_ks";
   note_kernel(name);
-  if (const int rc = raise_lds_limit<k_tq2_gemv_ks<SDT>>(160 * 1024)) return rc;
-  hipLaunchKernelGGL((k_tq2_gemv_ks<SDT>), grid, dim3((unsigned)nw * 64), lds, s, a, nw, (int)per);
+  if (const int rc = raise_lds_limit<k_tq2_gemv_ks<SDT, NTOK>>(160 * 1024)) return rc;
+  hipLaunchKernelGGL((k_tq2_gemv_ks<SDT, NTOK>), grid, dim3((unsigned)nw * 64), lds, s, a, nw, (int)per);
   return check_launch(name);
+}
+template <int SDT>
+int launch_kv(const GemmArgs& a, hipStream_t s, int nw, int64_t per, const dim3& grid, size_t lds, int ntok) {
+  return ntok == 2 ? launch_kv_n<SDT, 2>(a, s, nw, per, grid, lds) : launch_kv_n<SDT, 1>(a, s, nw, per, grid, lds);
 }
 
 }  // namespace
@@ -316,7 +338,8 @@ int launch_kv(const GemmArgs& a, hipStream_t s, int nw, int64_t per, const dim3&
 int launch_tq2_gemv_fp4(const GemmArgs& a, hipStream_t s) {
   const char force = tuning().tq2v;
   if (force == 'n') return BP_ERR_UNSUPPORTED;
-  if (a.fmt != BP_TQ2 || a.max_rows != 1 || a.tiles) return BP_ERR_UNSUPPORTED;
+  if (a.fmt != BP_TQ2 || a.max_rows < 1 || a.max_rows > 2 || a.tiles) return BP_ERR_UNSUPPORTED;
+  const int ntok = (int)a.max_rows;
   if (a.x_dtype != BP_BF16 && a.x_dtype != BP_I8) return BP_ERR_UNSUPPORTED;
   if (a.scale_dtype != BP_F16 && a.scale_dtype != BP_BF16 && a.scale_dtype != BP_F32) return BP_ERR_UNSUPPORTED;
   const int64_t sb = a.scale_dtype == BP_F32 ? 4 : 2;
@@ -347,15 +370,16 @@ int launch_tq2_gemv_fp4(const GemmArgs& a, hipStream_t s) {
   if (force != 'k' && (a.K < 2048 || experts * tiles < (a.x_dtype == BP_I8 ? 16 : 2) * (int64_t)cus)) return BP_ERR_UNSUPPORTED;
   // (a thread owns up to KV_OPT outputs; the partial sums of a workgroup's tiles stay in LDS until the term's end)
   const int64_t lds_cap = 160 * 1024 / per_cu;
-  int64_t per_max = 16 * nw < (lds_cap - slots) / (nw * 64) ? 16 * nw : (lds_cap - slots) / (nw * 64);
+  // (a thread owns up to KV_OPT outputs; a pair has two per row)
+  int64_t per_max = 16 * nw / ntok < (lds_cap - slots) / (nw * 64 * ntok) ? 16 * nw / ntok : (lds_cap - slots) / (nw * 64 * ntok);
   per_max = per_max / KV_R * KV_R;
   if (per_max < 2 * KV_R) return BP_ERR_UNSUPPORTED;
   if (per > per_max) per = per_max;
-  const size_t lds = (size_t)(slots + per * nw * 64);
+  const size_t lds = (size_t)(slots + per * nw * 64 * ntok);
   const dim3 grid((unsigned)((tiles + per - 1) / per), (unsigned)a.E, 1u);
   if (a.E > 65535) return BP_ERR_UNSUPPORTED;
-  if (a.scale_dtype == BP_F32) return launch_kv<BP_F32>(a, s, (int)nw, per, grid, lds);
-  return a.scale_dtype == BP_F16 ? launch_kv<BP_F16>(a, s, (int)nw, per, grid, lds) : launch_kv<BP_BF16>(a, s, (int)nw, per, grid, lds);
+  if (a.scale_dtype == BP_F32) return launch_kv<BP_F32>(a, s, (int)nw, per, grid, lds, ntok);
+  return a.scale_dtype == BP_F16 ? launch_kv<BP_F16>(a, s, (int)nw, per, grid, lds, ntok) : launch_kv<BP_BF16>(a, s, (int)nw, per, grid, lds, ntok);
 }
 
 }  // namespace bp

@@ -556,7 +556,8 @@ def test_absmean_weights_at_the_rounding_boundary(bp, sdtype):
     w[4, 5] = np.inf
     w[5, :group] = 0.0
     wt = dev(w)
-    want_trits, want_scale = orc.absmean_ternary(w, group, "f16" if sdtype == torch.float16 else "bf16")
+    with np.errstate(invalid="ignore"):  # (the NaN and infinite weights of rows 3 and 4)
+        want_trits, want_scale = orc.absmean_ternary(w, group, "f16" if sdtype == torch.float16 else "bf16")
     term = bp.absmean_ternary(wt, group, sdtype)
     assert np.array_equal(term.scale.float().cpu().numpy(), want_scale, equal_nan=True)
     assert np.array_equal(term.trits.cpu().numpy(), want_trits)

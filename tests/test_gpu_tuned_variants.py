@@ -523,8 +523,32 @@ def test_tq2_k_split_gemv_is_the_default_for_large_single_token_calls(bp):
         assert kern == ("fp4_tq2_i8_t1_ks" if act == "int8" else "fp4_tq2_t1_ks"), kern
         _check(got, want)
     got, want, kern = _run(bp, "tq2", 64, 1024, 2048, [1] * 63 + [2], "bf16", seed=6, max_rows=2)
+    assert kern == "fp4_tq2_m2_ks", kern  # (a bound of two rows: the pair variant)
+    _check(got, want)
+    got, want, kern = _run(bp, "tq2", 64, 1024, 2048, [1] * 63 + [3], "bf16", seed=7, max_rows=3)
     assert kern.startswith("mfma_tq2"), kern
     _check(got, want)
+
+
+@pytest.mark.parametrize("act", ["bf16", "int8"])
+@pytest.mark.parametrize("E,N,K,group,terms,sdt,counts", [
+    (3, 272, 2048, 128, 1, np.float16, [2, 0, 1]),
+    (2, 144, 1280, 128, 2, "bf16", [2, 2]),
+    (3, 1040, 4096, 256, 2, np.float16, [1, 2, 2]),
+    (2, 2064, 7168, 128, 1, np.float16, [2, 1]),
+    (3, 528, 7168, 128, 2, "f32", [2, 2, 0]),
+])
+def test_tq2_token_pair_gemv_with_k_split_over_the_waves(bp, tune, act, E, N, K, group, terms, sdt, counts):
+    """A pair of token rows per expert on the same kernel (two fp8 pieces per activation, rows 4 g + 2 t + p of operand A):
+    experts with two rows, one row and none; stacked terms; scale types and group sizes."""
+    if act == "int8" and sdt == "f32":
+        pytest.skip("int8 activations with float32 scales stay on the other kernel")
+    tune("BP_TUNE_TQ2V", "k")
+    got, want, kern = _run(bp, "tq2", E, N, K, counts, act, terms=terms, seed=K + N + 1, scale_dtype=sdt, group=group, max_rows=2)
+    assert kern == ("fp4_tq2_i8_m2_ks" if act == "int8" else "fp4_tq2_m2_ks"), kern
+    _check(got, want)
+    if act == "int8":
+        assert rel_l2(got, want) <= 1e-6, rel_l2(got, want)
 
 
 def test_tq2_k_split_gemv_adds_to_the_output_and_keeps_other_rows(bp, tune):
