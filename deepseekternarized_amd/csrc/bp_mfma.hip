@@ -53,7 +53,7 @@ int launch_mfma(const GemmArgs& a, hipStream_t s) {
   if (tuning().r == 1 || tuning().r == 2) R = tuning().r;
   if (tuning().waves == 8 || tuning().waves == 16) waves = tuning().waves;
   if (a.fmt == BP_TQ1) return launch_mfma_tq1(a, s, waves);
-  if (a.max_rows <= 2) {  // decode GEMV of a large call (one token row per expert, or a pair): K split over the waves, weights as fp4
+  if (a.max_rows <= 4) {  // decode GEMV of a large call (up to four token rows per expert): K split over the waves, weights as fp4
     const int rc = launch_tq2_gemv_fp4(a, s);
     if (rc != BP_ERR_UNSUPPORTED) return rc;
   }

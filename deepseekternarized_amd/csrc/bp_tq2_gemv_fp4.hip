@@ -98,7 +98,11 @@ __device__ __forceinline__ void kv_widen_run(const GemmArgs& a, const KvRun& r, 
 // a lane of the result holds both tokens' pieces of group kb.
 template <int SDT, int NTOK = 1>
 __global__ __launch_bounds__(1024) void k_tq2_gemv_ks(GemmArgs a, int nw, int tiles_per_wg) {
-  static_assert(NTOK == 1 || NTOK == 2, "one token row per expert, or a pair");
+  static_assert(NTOK == 1 || NTOK == 2 || NTOK == 4, "one token row per expert, a pair, or four");
+  // NTOK = 4: the matrix instructions of a step (two of a tile's four) meet only that step's two groups, so with an
+  // accumulator tile per step the 16 rows are 2 groups x 4 tokens x 2 pieces: row 8 q + 2 t + p is piece p of token t in
+  // the step's group q, and a lane builds its row for both steps (groups q and 2 + q of the wave's four).
+  constexpr bool M4 = NTOK == 4;
   constexpr int SB = SDT == BP_F32 ? 4 : 2, NSL = SB / 2;  // bytes per scale; a wave's 16-byte loads of a round's scales
   const int wave = __builtin_amdgcn_readfirstlane((int)(threadIdx.x >> 6)), lane = threadIdx.x & 63;
   const int n = lane & 15, kb = lane >> 4;
@@ -118,19 +122,23 @@ __global__ __launch_bounds__(1024) void k_tq2_gemv_ks(GemmArgs a, int nw, int ti
   // ---- LDS: two slots of a round's scales, then two of a round's partial sums [tile][wave][row]
   const unsigned row_sb = (unsigned)(a.G * SB), tile_sb = 16 * row_sb, slot_bytes = KV_R * tile_sb;
   const unsigned RED = 2 * slot_bytes;  // [tile of the workgroup][wave][token][row]
-  const int64_t g128 = 2 * KV_S * (int64_t)wave + kb;  // the lane's group of 128 as a column of the result
-  const bool g_real = 128 * g128 < a.K;
+  // the lane's group of 128 as a column of the result (four tokens: group kb / 2 of the first step, and 2 + kb / 2 of the second)
+  const int64_t g128 = 2 * KV_S * (int64_t)wave + (M4 ? kb >> 1 : kb), g128b = g128 + 2;
+  const bool g_real = 128 * g128 < a.K, g_realb = M4 && 128 * g128b < a.K;
   const unsigned rd_s = (unsigned)n * row_sb + (unsigned)SB * (unsigned)(g_real ? g128 >> gs : 0);
+  const unsigned rd_sb = (unsigned)n * row_sb + (unsigned)SB * (unsigned)(g_realb ? g128b >> gs : 0);
   const unsigned w_lane = (unsigned)n * (unsigned)a.Kp + 16u * (unsigned)kb + 64u * KV_S * (unsigned)wave;
   const unsigned s_off = 16u * (unsigned)(64 * wave + lane), s_step = 1024u * (unsigned)nw;  // (load j of a wave: + j s_step)
 
   // The lane as a row of operand A: piece p of the wave's group gl (p = 3: unused); its 2 x 16 activations are requested
   // first, the first tiles next, and operand A is built while those are on their way.
-  const int gl = n >> 2, p = NTOK == 2 ? n & 1 : n & 3, trow = NTOK == 2 ? (n >> 1) & 1 : 0;  // (a pair: the lane's token)
+  // (several tokens: the lane's token; four: gl is the lane's group of the first step, gl + 2 that of the second)
+  const int gl = M4 ? n >> 3 : n >> 2, p = NTOK >= 2 ? n & 1 : n & 3, trow = M4 ? (n >> 1) & 3 : NTOK == 2 ? (n >> 1) & 1 : 0;
   const int64_t kbase = 256 * KV_S * (int64_t)wave + 128 * gl + 64 * (kb >> 1) + 16 * (kb & 1);
-  // (an expert with one row of the pair: the absent token's rows of operand A hold zeros, its sums are not stored)
-  const int64_t kx = trow < ntok ? kbase : a.K;
+  // (an expert with fewer rows: the absent tokens' rows of operand A hold zeros, their sums are not stored)
+  const int64_t kx = trow < ntok ? kbase : a.K, kxb = M4 && trow < ntok ? kbase + 256 : a.K;
   const KvRun x_lo = kv_load_run(a, tok + trow, kx), x_hi = kv_load_run(a, tok + trow, kx + 32);
+  const KvRun xb_lo = kv_load_run(a, tok + trow, kxb), xb_hi = kv_load_run(a, tok + trow, kxb + 32);  // (four tokens: the second step's group)
   // Thread o of the workgroup owns output o of the workgroup's rows (up to KV_OPT of them: o + a multiple of the
   // workgroup's threads): what the call adds to is read now and written back once, after the last term.
   // (a pair: output o = ((tile * 2 + token) * 16 + row)
@@ -144,7 +152,7 @@ __global__ __launch_bounds__(1024) void k_tq2_gemv_ks(GemmArgs a, int nw, int ti
     total[u] = out_live(o) ? a.out[out_at(o)] : 0.f;
   }
   i32x8 A[2 * KV_S];
-  float cinit[4], inv2[NTOK];
+  float cinit[4], inv2[NTOK], cinitb[4], inv2b[2];  // (b: four tokens, the second step; inv2 / inv2b then hold the lane's two tokens)
 
   // (the expert's rows and scales of a term as buffers of their own: what lies past them reads as zeros)
   __amdgpu_buffer_rsrc_t wrs = make_rsrc(a.packed[0] + e * a.N * a.Kp, a.N * a.Kp);
@@ -171,7 +179,10 @@ __global__ __launch_bounds__(1024) void k_tq2_gemv_ks(GemmArgs a, int nw, int ti
     constexpr int i = decltype(i_c)::value, slot = i % KV_D;
     const unsigned sat = (unsigned)(r & 1) * slot_bytes + (unsigned)i * tile_sb + rd_s;
     const unsigned raw = SB == 4 ? *(const lds_u32*)sat : (unsigned)*(const lds_u16*)sat;
-    f32x4 C = {cinit[0], cinit[1], cinit[2], NTOK == 2 ? cinit[3] : 0.f};
+    const unsigned satb = (unsigned)(r & 1) * slot_bytes + (unsigned)i * tile_sb + rd_sb;
+    const unsigned rawb = !M4 ? 0u : SB == 4 ? *(const lds_u32*)satb : (unsigned)*(const lds_u16*)satb;
+    f32x4 C = {cinit[0], cinit[1], cinit[2], NTOK >= 2 ? cinit[3] : 0.f};
+    f32x4 Cb = {cinitb[0], cinitb[1], cinitb[2], cinitb[3]};  // (four tokens: the second step's accumulator tile)
 #pragma unroll
     for (int s = 0; s < KV_S; ++s) {
       const u32x4 W = ring[slot][s];
@@ -179,16 +190,30 @@ __global__ __launch_bounds__(1024) void k_tq2_gemv_ks(GemmArgs a, int nw, int ti
       for (int h = 0; h < 2; ++h) {
         const unsigned d0 = W[2 * h], d1 = W[2 * h + 1];
         const i32x8 B8 = {(int)(d0 & 0x33333333u), (int)((d0 >> 2) & 0x33333333u), (int)(d1 & 0x33333333u), (int)((d1 >> 2) & 0x33333333u), 0, 0, 0, 0};
-        C = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(A[2 * s + h], B8, C, 0 /* A: E4M3 */, 4 /* B: E2M1 */, 0, 0, 0, 0);
+        if (M4 && s == 1) Cb = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(A[2 * s + h], B8, Cb, 0, 4, 0, 0, 0, 0);
+        else C = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(A[2 * s + h], B8, C, 0 /* A: E4M3 */, 4 /* B: E2M1 */, 0, 0, 0, 0);
       }
     }
     request(KV_R * r + i + KV_D, IC<slot>{});
-    const float sc = SDT == BP_F32 ? __uint_as_float(raw) : SDT == BP_F16 ? f16_bits_to_f32((uint16_t)raw) : __uint_as_float(raw << 16);
+    auto widen = [&](unsigned q) { return SDT == BP_F32 ? __uint_as_float(q) : SDT == BP_F16 ? f16_bits_to_f32((uint16_t)q) : __uint_as_float(q << 16); };
+    const float sc = widen(raw);
+    if constexpr (M4) {  // the lane: group kb / 2 of either step, tokens 2 (kb % 2) and 2 (kb % 2) + 1; the other group's lane is kb ^ 2
+      const float scb = widen(rawb);
 #pragma unroll
-    for (int tt = 0; tt < NTOK; ++tt) {
-      float v = !g_real ? 0.f : NTOK == 2 ? sc * inv2[tt] * (C[2 * tt] + C[2 * tt + 1]) : sc * inv2[0] * (C[0] + C[1] + C[2] * (1.f / 256.f));
-      v = kv_quad_sum(v);
-      if (kb == 0) *(lds_u32*)(RED + (unsigned)((((KV_R * r + i) * nw + wave) * NTOK + tt) * 64 + 4 * n)) = __float_as_uint(v);
+      for (int t2 = 0; t2 < 2; ++t2) {
+        float v = (g_real ? sc * inv2[t2] * (C[2 * t2] + C[2 * t2 + 1]) : 0.f) + (g_realb ? scb * inv2b[t2] * (Cb[2 * t2] + Cb[2 * t2 + 1]) : 0.f);
+        const auto h32 = __builtin_amdgcn_permlane32_swap(__float_as_uint(v), __float_as_uint(v), false, false);
+        v = __uint_as_float(h32[0]) + __uint_as_float(h32[1]);
+        const int tt = 2 * (kb & 1) + t2;
+        if (kb < 2) *(lds_u32*)(RED + (unsigned)((((KV_R * r + i) * nw + wave) * NTOK + tt) * 64 + 4 * n)) = __float_as_uint(v);
+      }
+    } else {
+#pragma unroll
+      for (int tt = 0; tt < NTOK; ++tt) {
+        float v = !g_real ? 0.f : NTOK == 2 ? sc * inv2[tt] * (C[2 * tt] + C[2 * tt + 1]) : sc * inv2[0] * (C[0] + C[1] + C[2] * (1.f / 256.f));
+        v = kv_quad_sum(v);
+        if (kb == 0) *(lds_u32*)(RED + (unsigned)((((KV_R * r + i) * nw + wave) * NTOK + tt) * 64 + 4 * n)) = __float_as_uint(v);
+      }
     }
   };
 
@@ -203,70 +228,100 @@ __global__ __launch_bounds__(1024) void k_tq2_gemv_ks(GemmArgs a, int nw, int ti
 
   // ---- the wave's part of operand A, the starting values of an accumulator tile and the lane's inverse prescale
   {
-    float y[2][16];
-    kv_widen_run(a, x_lo, y[0]);
-    kv_widen_run(a, x_hi, y[1]);
-    unsigned m = 0;
+    // the lane's row for the wave's group gidx: its 2 x 16 activations as pieces (word), the sum of the lane's piece over
+    // the row's four lanes (hs) and the group's doubled inverse prescale (inv)
+    auto build = [&](const KvRun& lo, const KvRun& hi, int gidx, unsigned (&word)[2][4], float& hs, float& inv) {
+      float y[2][16];
+      kv_widen_run(a, lo, y[0]);
+      kv_widen_run(a, hi, y[1]);
+      unsigned m = 0;
 #pragma unroll
-    for (int t = 0; t < 32; ++t) {
-      const unsigned v = __float_as_uint(y[t >> 4][t & 15]) & 0x7fffffffu;
-      m = m > v ? m : v;
-    }
-    {  // the group's largest magnitude: the four lanes of a row hold its 128 activations
-      unsigned o = (unsigned)__shfl_xor((int)m, 16, 64);
-      m = m > o ? m : o;
-      o = (unsigned)__shfl_xor((int)m, 32, 64);
-      m = m > o ? m : o;
-    }
-    const bool real = 256 * KV_S * (int64_t)wave + 128 * gl < a.K;
-    int sh = 0;
-    bool finite = true;
-    if (a.x_dtype != BP_I8) {  // (int8 values fit as they are: prescale 1)
-      const int ex = (int)(m >> 23);
-      finite = ex != 255;  // a NaN or an infinity among the group's activations
-      sh = 134 - ex;
-      sh = sh > 120 ? 120 : sh < -120 ? -120 : sh;
-    }
-    const float pre = __uint_as_float((unsigned)(sh + 127) << 23);
-    // twice the inverse prescale (the weights are multiplied as c / 2); NaN for a group with a non-finite activation,
-    // so the token's outputs are NaN rather than finite and wrong
-    const float inv = !real ? 0.f : finite ? __uint_as_float((unsigned)(128 - sh) << 23) : __uint_as_float(0x7fc00000u);
-    unsigned word[2][4];
-    float hs = 0.f;  // the sum of the lane's piece over its activations
-#pragma unroll
-    for (int h = 0; h < 2; ++h) {
-#pragma unroll
-      for (int vv = 0; vv < 4; ++vv) {
-        float r[4];
-#pragma unroll
-        for (int b = 0; b < 4; ++b) r[b] = y[h][8 * (vv & 1) + 2 * b + (vv >> 1)] * pre;
-        unsigned mine = 0;
-#pragma unroll
-        for (int pp = 0; pp < 3; ++pp) {
-          const float f = pp == 2 ? 256.f : 1.f;
-          int w = __builtin_amdgcn_cvt_pk_fp8_f32(r[0] * f, r[1] * f, 0, false);
-          w = __builtin_amdgcn_cvt_pk_fp8_f32(r[2] * f, r[3] * f, w, true);
-          const float f0 = __builtin_amdgcn_cvt_f32_fp8(w, 0), f1 = __builtin_amdgcn_cvt_f32_fp8(w, 1);
-          const float f2 = __builtin_amdgcn_cvt_f32_fp8(w, 2), f3 = __builtin_amdgcn_cvt_f32_fp8(w, 3);
-          if (pp == p) {
-            mine = (unsigned)w;
-            hs += (f0 + f1) + (f2 + f3);
-          }
-          if (pp < 2) { r[0] -= f0; r[1] -= f1; r[2] -= f2; r[3] -= f3; }
-        }
-        word[h][vv] = mine;
+      for (int t = 0; t < 32; ++t) {
+        const unsigned v = __float_as_uint(y[t >> 4][t & 15]) & 0x7fffffffu;
+        m = m > v ? m : v;
       }
-    }
-    hs += __shfl_xor(hs, 16, 64);
-    hs += __shfl_xor(hs, 32, 64);
+      {  // the group's largest magnitude: the four lanes of a row hold its 128 activations
+        unsigned o = (unsigned)__shfl_xor((int)m, 16, 64);
+        m = m > o ? m : o;
+        o = (unsigned)__shfl_xor((int)m, 32, 64);
+        m = m > o ? m : o;
+      }
+      const bool real = 256 * KV_S * (int64_t)wave + 128 * gidx < a.K;
+      int sh = 0;
+      bool finite = true;
+      if (a.x_dtype != BP_I8) {  // (int8 values fit as they are: prescale 1)
+        const int ex = (int)(m >> 23);
+        finite = ex != 255;  // a NaN or an infinity among the group's activations
+        sh = 134 - ex;
+        sh = sh > 120 ? 120 : sh < -120 ? -120 : sh;
+      }
+      const float pre = __uint_as_float((unsigned)(sh + 127) << 23);
+      // twice the inverse prescale (the weights are multiplied as c / 2); NaN for a group with a non-finite activation,
+      // so the token's outputs are NaN rather than finite and wrong
+      inv = !real ? 0.f : finite ? __uint_as_float((unsigned)(128 - sh) << 23) : __uint_as_float(0x7fc00000u);
+      hs = 0.f;
 #pragma unroll
-    for (int i = 0; i < 4; ++i) cinit[i] = -0.5f * __shfl(hs, 4 * kb + i, 64);  // (the lane as a column of the result: group kb; one token: row 3 is unused, its sum 0)
+      for (int h = 0; h < 2; ++h) {
 #pragma unroll
-    for (int tt = 0; tt < NTOK; ++tt) inv2[tt] = __shfl(inv, 4 * kb + 2 * tt, 64);
+        for (int vv = 0; vv < 4; ++vv) {
+          float r[4];
 #pragma unroll
-    for (int j = 0; j < 2 * KV_S; ++j) {
+          for (int b = 0; b < 4; ++b) r[b] = y[h][8 * (vv & 1) + 2 * b + (vv >> 1)] * pre;
+          unsigned mine = 0;
 #pragma unroll
-      for (int v = 0; v < 8; ++v) A[j][v] = (j >> 1) == (gl >> 1) && (v >> 2) == (gl & 1) && p < 3 ? (int)word[j & 1][v & 3] : 0;
+          for (int pp = 0; pp < 3; ++pp) {
+            const float f = pp == 2 ? 256.f : 1.f;
+            int w = __builtin_amdgcn_cvt_pk_fp8_f32(r[0] * f, r[1] * f, 0, false);
+            w = __builtin_amdgcn_cvt_pk_fp8_f32(r[2] * f, r[3] * f, w, true);
+            const float f0 = __builtin_amdgcn_cvt_f32_fp8(w, 0), f1 = __builtin_amdgcn_cvt_f32_fp8(w, 1);
+            const float f2 = __builtin_amdgcn_cvt_f32_fp8(w, 2), f3 = __builtin_amdgcn_cvt_f32_fp8(w, 3);
+            if (pp == p) {
+              mine = (unsigned)w;
+              hs += (f0 + f1) + (f2 + f3);
+            }
+            if (pp < 2) { r[0] -= f0; r[1] -= f1; r[2] -= f2; r[3] -= f3; }
+          }
+          word[h][vv] = mine;
+        }
+      }
+      hs += __shfl_xor(hs, 16, 64);
+      hs += __shfl_xor(hs, 32, 64);
+    };
+    unsigned word[2][4];
+    float hs, inv;
+    build(x_lo, x_hi, gl, word, hs, inv);
+    // (the lane as a column of the result: rows 4 kb + i; one token: row 3 is unused, its sum 0)
+#pragma unroll
+    for (int i = 0; i < 4; ++i) cinit[i] = -0.5f * __shfl(hs, 4 * kb + i, 64);
+    if constexpr (M4) {
+      unsigned wordb[2][4];
+      float hsb, invb;
+      build(xb_lo, xb_hi, gl + 2, wordb, hsb, invb);
+#pragma unroll
+      for (int i = 0; i < 4; ++i) cinitb[i] = -0.5f * __shfl(hsb, 4 * kb + i, 64);
+#pragma unroll
+      for (int t2 = 0; t2 < 2; ++t2) {
+        inv2[t2] = __shfl(inv, 4 * kb + 2 * t2, 64);
+        inv2b[t2] = __shfl(invb, 4 * kb + 2 * t2, 64);
+      }
+      inv2[2] = inv2[3] = 0.f;
+      // instruction 2 s + h: the step's two groups sit in register halves 0 and 1; the lane's row belongs to half gl
+#pragma unroll
+      for (int jj = 0; jj < 2 * KV_S; ++jj) {
+#pragma unroll
+        for (int v = 0; v < 8; ++v) A[jj][v] = (v >> 2) == gl ? (int)((jj >> 1) ? wordb[jj & 1][v & 3] : word[jj & 1][v & 3]) : 0;
+      }
+    } else {
+#pragma unroll
+      for (int i = 0; i < 4; ++i) cinitb[i] = 0.f;
+      inv2b[0] = inv2b[1] = 0.f;
+#pragma unroll
+      for (int tt = 0; tt < NTOK; ++tt) inv2[tt] = __shfl(inv, 4 * kb + 2 * tt, 64);
+#pragma unroll
+      for (int jj = 0; jj < 2 * KV_S; ++jj) {
+#pragma unroll
+        for (int v = 0; v < 8; ++v) A[jj][v] = (jj >> 1) == (gl >> 1) && (v >> 2) == (gl & 1) && p < 3 ? (int)word[jj & 1][v & 3] : 0;
+      }
     }
   }
 
@@ -294,7 +349,10 @@ __global__ __launch_bounds__(1024) void k_tq2_gemv_ks(GemmArgs a, int nw, int ti
         const int tl = (o >> 4) / NTOK, tt = (o >> 4) % NTOK;
         float v = 0.f;
         for (int c = 0; c < nw; ++c) v += __uint_as_float(*(const lds_u32*)(RED + (unsigned)((((tl * nw + c) * NTOK + tt) * 16 + (o & 15)) * 4)));
-        total[u] += a.x_dtype == BP_I8 ? v * (NTOK == 2 && tt ? xsc[NTOK - 1] : xsc[0]) : v;
+        float xs = xsc[0];  // (the token's activation scale, without indexing the array by a variable)
+#pragma unroll
+        for (int q = 1; q < NTOK; ++q) xs = tt == q ? xsc[q] : xs;
+        total[u] += a.x_dtype == BP_I8 ? v * xs : v;
       }
     }
   }
@@ -321,7 +379,8 @@ int kv_cus() {  // compute units of the current device (256 if the query fails)
 
 template <int SDT, int NTOK>
 int launch_kv_n(const GemmArgs& a, hipStream_t s, int nw, int64_t per, const dim3& grid, size_t lds) {
-  const char* name = NTOK == 2 ? (a.x_dtype == BP_I8 ? "fp4_tq2_i8_m2_ks" : "fp4_tq2_m2_ks") : a.x_dtype == BP_I8 ? "fp4_tq2_i8_t1_ks" : "fp4_tq2_t1_ks";
+  const char* name = NTOK == 4 ? (a.x_dtype == BP_I8 ? "fp4_tq2_i8_m4_ks" : "fp4_tq2_m4_ks") : NTOK == 2 ? (a.x_dtype == BP_I8 ? "fp4_tq2_i8_m2_ks" : "fp4_tq2_m2_ks")
+                                : a.x_dtype == BP_I8 ? "fp4_tq2_i8_t1_ks" : "fp4_tq2_t1_ks";
   note_kernel(name);
   if (const int rc = raise_lds_limit<k_tq2_gemv_ks<SDT, NTOK>>(160 * 1024)) return rc;
   hipLaunchKernelGGL((k_tq2_gemv_ks<SDT, NTOK>), grid, dim3((unsigned)nw * 64), lds, s, a, nw, (int)per);
@@ -329,6 +388,7 @@ int launch_kv_n(const GemmArgs& a, hipStream_t s, int nw, int64_t per, const dim
 }
 template <int SDT>
 int launch_kv(const GemmArgs& a, hipStream_t s, int nw, int64_t per, const dim3& grid, size_t lds, int ntok) {
+  if (ntok == 4) return launch_kv_n<SDT, 4>(a, s, nw, per, grid, lds);
   return ntok == 2 ? launch_kv_n<SDT, 2>(a, s, nw, per, grid, lds) : launch_kv_n<SDT, 1>(a, s, nw, per, grid, lds);
 }
 
@@ -338,8 +398,8 @@ int launch_kv(const GemmArgs& a, hipStream_t s, int nw, int64_t per, const dim3&
 int launch_tq2_gemv_fp4(const GemmArgs& a, hipStream_t s) {
   const char force = tuning().tq2v;
   if (force == 'n') return BP_ERR_UNSUPPORTED;
-  if (a.fmt != BP_TQ2 || a.max_rows < 1 || a.max_rows > 2 || a.tiles) return BP_ERR_UNSUPPORTED;
-  const int ntok = (int)a.max_rows;
+  if (a.fmt != BP_TQ2 || a.max_rows < 1 || a.max_rows > 4 || a.tiles) return BP_ERR_UNSUPPORTED;
+  const int ntok = a.max_rows == 3 ? 4 : (int)a.max_rows;  // (three rows: the variant for four)
   if (a.x_dtype != BP_BF16 && a.x_dtype != BP_I8) return BP_ERR_UNSUPPORTED;
   if (a.scale_dtype != BP_F16 && a.scale_dtype != BP_BF16 && a.scale_dtype != BP_F32) return BP_ERR_UNSUPPORTED;
   const int64_t sb = a.scale_dtype == BP_F32 ? 4 : 2;

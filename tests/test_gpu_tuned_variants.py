@@ -526,6 +526,9 @@ def test_tq2_k_split_gemv_is_the_default_for_large_single_token_calls(bp):
     assert kern == "fp4_tq2_m2_ks", kern  # (a bound of two rows: the pair variant)
     _check(got, want)
     got, want, kern = _run(bp, "tq2", 64, 1024, 2048, [1] * 63 + [3], "bf16", seed=7, max_rows=3)
+    assert kern == "fp4_tq2_m4_ks", kern  # (three or four rows: the variant for four)
+    _check(got, want)
+    got, want, kern = _run(bp, "tq2", 64, 1024, 2048, [1] * 63 + [5], "bf16", seed=8, max_rows=5)
     assert kern.startswith("mfma_tq2"), kern
     _check(got, want)
 
@@ -546,6 +549,28 @@ def test_tq2_token_pair_gemv_with_k_split_over_the_waves(bp, tune, act, E, N, K,
     tune("BP_TUNE_TQ2V", "k")
     got, want, kern = _run(bp, "tq2", E, N, K, counts, act, terms=terms, seed=K + N + 1, scale_dtype=sdt, group=group, max_rows=2)
     assert kern == ("fp4_tq2_i8_m2_ks" if act == "int8" else "fp4_tq2_m2_ks"), kern
+    _check(got, want)
+    if act == "int8":
+        assert rel_l2(got, want) <= 1e-6, rel_l2(got, want)
+
+
+@pytest.mark.parametrize("act", ["bf16", "int8"])
+@pytest.mark.parametrize("E,N,K,group,terms,sdt,counts", [
+    (3, 272, 2048, 128, 1, np.float16, [4, 0, 3]),
+    (2, 144, 2304, 128, 2, "bf16", [4, 1]),
+    (3, 1040, 4096, 256, 2, np.float16, [2, 4, 3]),
+    (2, 2064, 7168, 128, 1, np.float16, [4, 4]),
+    (3, 528, 7168, 128, 2, "f32", [3, 4, 0]),
+])
+def test_tq2_four_token_gemv_with_k_split_over_the_waves(bp, tune, act, E, N, K, group, terms, sdt, counts):
+    """Up to four token rows per expert on the same kernel: an accumulator tile per 64-byte step, rows 8 q + 2 t + p of
+    operand A (the step's group q, token t, piece p); experts with four, three, two, one and no rows; stacked terms; an odd
+    number of steps (the last wave's second step lies past the row)."""
+    if act == "int8" and sdt == "f32":
+        pytest.skip("int8 activations with float32 scales stay on the other kernel")
+    tune("BP_TUNE_TQ2V", "k")
+    got, want, kern = _run(bp, "tq2", E, N, K, counts, act, terms=terms, seed=K + N + 2, scale_dtype=sdt, group=group, max_rows=max(counts))
+    assert kern == ("fp4_tq2_i8_m4_ks" if act == "int8" else "fp4_tq2_m4_ks"), kern
     _check(got, want)
     if act == "int8":
         assert rel_l2(got, want) <= 1e-6, rel_l2(got, want)
