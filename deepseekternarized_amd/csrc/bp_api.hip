@@ -8,6 +8,7 @@
 #include <cstring>
 
 #include "bp_common.h"
+#include "bp_mfma.h"
 
 namespace bp {
 namespace {
@@ -173,7 +174,7 @@ static size_t staged_workspace_bytes(int64_t T, int64_t N, int64_t K, int64_t E,
   if (tuning().tq2g == 'b') return 0;
   // (the launcher's own thresholds, so that a call it would turn down does not make its caller allocate)
   if (fmt == BP_TQ2 && tuning().tq2g != 'f' && (N < 1024 || (T + 31) / 32 * ((N + 511) / 512) < 768)) return 0;  // at least two blocks of 512 output rows, three rounds of one workgroup per CU
-  if (fmt == BP_TQ1 && max_rows <= 8 && tuning().tq2g != 'f') return 0;  // (the small-batch kernels take these)
+  if (fmt == BP_TQ1 && max_rows <= 8 && tuning().tq2g != 'f' && !tq1_rows_on_tiles(max_rows, E, T, N)) return 0;  // (the small-batch kernels take these)
   if (max_rows <= 0 || (max_rows + 31) / 32 * 32 * E > 4 * T + 32 * E) return 0;  // a loose bound on the rows per expert: mostly token tiles that do not exist
   return gemm_tq2f_workspace_bytes(T, K, E);
 }

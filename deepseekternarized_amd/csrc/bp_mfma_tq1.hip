@@ -403,6 +403,10 @@ int launch_mfma_tq1(const GemmArgs& a, hipStream_t s, int waves) {
     return launch_tq1_v<8, 1>(a, s, "mfma_tq1_bf16_t1_w8", "mfma_tq1_bf16_t1_w8_gs");
   }
   if (a.max_rows <= 64) {  // small decode batches: the fp8 x fp4 kernel with one operand tile per token
+    if (a.stage && tuning().tq1 == 0 && tuning().tq2g != 'b' && tq1_rows_on_tiles(a.max_rows, a.E, a.T, a.N)) {  // (dense batches of 7 - 8 rows with a workspace)
+      const int rc = launch_gemm_tq2f(a, s);
+      if (rc != BP_ERR_UNSUPPORTED) return rc;
+    }
     if (tuning().tq1 != 'm' && tuning().tq1 != 'l') {  // (development: "mfma" / "lut" keep the kernels below)
       const int rc = launch_tq1_gemv_fp4(a, s);
       if (rc != BP_ERR_UNSUPPORTED) return rc;

@@ -28,6 +28,7 @@ _BACKENDS = ("auto", "cuda", "hip", "torch", "cpp")
 
 
 _WORKSPACE_CAP = 8 << 30  # bytes of workspace the mirrored grouped call allocates at most
+_DECODE_ROWS = 6  # bf16 / int8 calls of up to this many rows per expert run on the decode kernels: no workspace query
 
 
 class _HipTernary:
@@ -95,7 +96,7 @@ class _HipTernary:
             # fp16 activations run on the bf16 kernels as a pair. The size query answers 0 where the launch would not use
             # one (small calls, a loose max_rows); decode-sized bf16 / int8 calls never do and skip the query.
             need = 0
-            if max_rows > 8 or xdt in (_lib.BP_F16, _lib.BP_F32):
+            if max_rows > _DECODE_ROWS or xdt in (_lib.BP_F16, _lib.BP_F32):
                 need = self.lib.bp_grouped_gemm_workspace_bytes(xdt, T, N, int(K), E, int(fmt), int(max_rows))
                 if need > _WORKSPACE_CAP:  # (about 2.1 bytes per activation: a call this large keeps its memory and runs the kernels without one)
                     need = 0

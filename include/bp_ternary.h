@@ -83,7 +83,7 @@ int bp_ternary_grouped_gemm(float* out, const void* x, int x_dtype, const float*
 /* bp_ternary_grouped_gemm with a workspace of the caller's (the library allocates no device memory). It has no
  * counterpart in the reference. With a workspace of at least bp_grouped_gemm_workspace_bytes(...) bytes (256-byte
  * aligned device memory; contents undefined before and after the call) the grouped GEMM kernels for bf16 activations
- * (TQ2: more than 16 rows per expert; TQ1: more than 8) convert the activations to matrix-instruction operands once, in
+ * (TQ2: more than 16 rows per expert; TQ1: more than 8, and dense batches of 7 or 8) convert the activations to matrix-instruction operands once, in
  * a pass of their own, instead of once per block of output rows; results agree with bp_ternary_grouped_gemm's to
  * float32 rounding of the sums. workspace = NULL, or a size of 0 from bp_grouped_gemm_workspace_bytes (no such kernel
  * for these arguments; a launch too small for it to pay - TQ2: fewer than 1024 output rows, or fewer than 768 blocks

@@ -433,6 +433,32 @@ def test_tq1_fp4_few_large_experts(bp, K, counts, last, act):
     _check(got, want)
 
 
+def test_tq1_dense_batches_of_seven_or_eight_rows_run_on_the_tile_kernel_with_a_workspace(bp):
+    """Seven or eight rows per expert, four or more on average, and at least 512 blocks of 512 output rows: the mirrored
+    call brings a workspace and the call runs on the tile kernel over converted activations (one decode of the weights
+    instead of two launches of the four-row kernel); six rows, few experts or int8 activations stay on the decode kernels."""
+    from deepseekternarized_amd.kernels import _lib
+    E, N, K = 128, 2048, 1024
+    counts = [8] * (E - 3) + [7, 0, 5]
+    T = sum(counts)
+    lib = bp.ext().lib
+    assert lib.bp_grouped_gemm_workspace_bytes(_lib.BP_BF16, T, N, K, E, 1, 8) > 0
+    assert lib.bp_grouped_gemm_workspace_bytes(_lib.BP_BF16, T, N, K, E, 1, 7) > 0
+    assert lib.bp_grouped_gemm_workspace_bytes(_lib.BP_BF16, T, N, K, E, 1, 6) == 0
+    assert lib.bp_grouped_gemm_workspace_bytes(_lib.BP_BF16, 16 * 8, N, K, 16, 1, 8) == 0   # 64 blocks
+    assert lib.bp_grouped_gemm_workspace_bytes(_lib.BP_BF16, 3 * E, N, K, E, 1, 8) == 0     # three rows per expert on average
+    assert lib.bp_grouped_gemm_workspace_bytes(_lib.BP_I8, T, N, K, E, 1, 8) == 0
+    got, want, kern = _run(bp, "tq1", E, N, K, counts, "bf16", seed=77)
+    assert kern == "gemm_tq1f_bf16", kern
+    _check(got, want)
+    got, want, kern = _run(bp, "tq1", E, N, K, counts, "int8", seed=78)
+    assert kern.startswith("fp4_tq1_m"), kern
+    _check(got, want)
+    got, want, kern = _run(bp, "tq1", 16, N, K, [8] * 16, "bf16", seed=79)
+    assert kern.startswith("fp4_tq1_m"), kern
+    _check(got, want)
+
+
 def test_tq1_fp4_upper_bound_max_rows(bp):
     """max_rows as an upper bound (64 for a decode step of 64 tokens) with offsets on the device: 8 launches of 8 rows,
     most of them without any row to take."""
