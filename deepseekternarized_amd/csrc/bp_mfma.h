@@ -43,7 +43,7 @@ int launch_tq1_gemv(const GemmArgs& a, hipStream_t s, int waves);
 // batches: up to 8 token rows per expert, or up to 64 in launches of 8 when the experts average at most 4 rows;
 // BP_ERR_UNSUPPORTED without a message when the call is outside its preconditions
 int launch_tq1_gemv_fp4(const GemmArgs& a, hipStream_t s);
-// bp_tq2_gemv_fp4.hip: TQ2, one token row per expert, on the fp8 x fp4 matrix instruction with K split over the waves;
+// bp_tq2_gemv_fp4.hip: TQ2, one to four token rows per expert, on the fp8 x fp4 matrix instruction with K split over the waves;
 // BP_ERR_UNSUPPORTED without a message when the call is outside its preconditions
 int launch_tq2_gemv_fp4(const GemmArgs& a, hipStream_t s);
 
