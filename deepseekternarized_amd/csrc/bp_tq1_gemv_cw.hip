@@ -466,7 +466,7 @@ int launch_cw(const GemmArgs& a, hipStream_t s, int64_t nchunks, int cus, int fi
   auto loaders_of = [&](int g) { return (CW_WAVES - g * nchunks) / g; };
   // (a workgroup keeps its outputs in LDS: at most CW_STAGE_PER_THREAD per thread, 64 bytes per tile and token)
   const int64_t per_cap = CW_STAGE_PER_THREAD * CW_WAVES * 64 / (16 * NTOK);
-  if (per > per_cap) per = per_cap;
+  for (int64_t k = 2; per > per_cap; ++k) per = (tiles + k * wpe - 1) / (k * wpe);  // (twice, three times ... as many workgroups per expert: whole rounds of one workgroup per CU)
   auto lds_of = [&](int g, int tpb) {
     const int64_t stream = (int64_t)g * 2 * tpb * (buf + nchunks * 64 * NTOK), build = nchunks * NTOK * f4_chunk_bytes(NTOK);
     const int64_t mine = (per + g - 1) / g * g;  // tiles per workgroup with g groups

@@ -434,7 +434,9 @@ int launch_tq2_gemv_fp4(const GemmArgs& a, hipStream_t s) {
   int64_t per_max = 16 * nw / ntok < (lds_cap - slots) / (nw * 64 * ntok) ? 16 * nw / ntok : (lds_cap - slots) / (nw * 64 * ntok);
   per_max = per_max / KV_R * KV_R;
   if (per_max < 2 * KV_R) return BP_ERR_UNSUPPORTED;
-  if (per > per_max) per = per_max;
+  // (ranges too long for a workgroup's LDS: twice, three times ... as many workgroups per expert, so that the launch
+  // stays whole rounds of the resident workgroups - 96 tiles per expert at four rows as 4 x 24, not 3 x 32)
+  for (int64_t k = 2; per > per_max; ++k) per = ((tiles + k * wpe - 1) / (k * wpe) + KV_R - 1) / KV_R * KV_R;
   const size_t lds = (size_t)(slots + per * nw * 64 * ntok);
   const dim3 grid((unsigned)((tiles + per - 1) / per), (unsigned)a.E, 1u);
   if (a.E > 65535) return BP_ERR_UNSUPPORTED;

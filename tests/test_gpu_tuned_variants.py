@@ -602,6 +602,33 @@ def test_tq2_four_token_gemv_with_k_split_over_the_waves(bp, tune, act, E, N, K,
         assert rel_l2(got, want) <= 1e-6, rel_l2(got, want)
 
 
+@pytest.mark.parametrize("fmt,N,rows,switch,off,want", [("tq2", 1536, 4, "BP_TUNE_TQ2V", "n", "fp4_tq2_m4_ks"), ("tq1", 3072, 4, "BP_TUNE_TQ1", "rows", "fp4_tq1_m4_cw")])
+def test_decode_gemv_ranges_capped_by_lds_cover_every_row(bp, tune, fmt, N, rows, switch, off, want):
+    """128 experts x 96 (192) row tiles at four token rows: a workgroup's LDS holds the sums of 32 (64) tiles, so an
+    expert's tiles go to 4 workgroups of 24 (48) rather than 3 of 32 (64) - whole rounds of the resident workgroups. The
+    launch is too large for the CPU kernel in a test's time: checked against the library's other kernel for these calls
+    (each of them is checked against the CPU kernel at smaller sizes), on weights drawn on the device."""
+    E, K = 128, 7168
+    g = torch.Generator(device="cuda").manual_seed(N)
+    packed = torch.empty(E, N, bp.packed_cols(fmt, K), dtype=torch.uint8, device="cuda")
+    for e in range(E):
+        packed[e] = bp.pack(torch.randint(-1, 2, (N, K), device="cuda", generator=g).to(torch.int8), fmt)
+    scale = (0.02 * torch.randn(E, N, K // GROUP, device="cuda", generator=g).abs()).half()
+    x = torch.randn(E * rows, K, device="cuda", generator=g).to(torch.bfloat16)
+    offsets = [rows * e for e in range(E + 1)]
+    got = bp.grouped_ternary_gemm(x, None, offsets, packed, scale, K, GROUP, fmt)
+    assert bp.ext().last_kernel() == want, bp.ext().last_kernel()
+    tune(switch, off)
+    ref = bp.grouped_ternary_gemm(x, None, offsets, packed, scale, K, GROUP, fmt)
+    assert bp.ext().last_kernel() != want
+    got, ref = got.double(), ref.double()
+    assert torch.isfinite(got).all()
+    per_expert = ((got - ref).reshape(E, -1).norm(dim=1) / ref.reshape(E, -1).norm(dim=1)).max().item()
+    assert per_expert <= REL_L2, per_expert
+    per_tile = ((got - ref).reshape(E * rows, N // 16, 16).norm(dim=2) / ref.reshape(E * rows, N // 16, 16).norm(dim=2)).max().item()
+    assert per_tile <= 10 * REL_L2, per_tile  # (no row tile left out or added twice)
+
+
 def test_tq2_k_split_gemv_adds_to_the_output_and_keeps_other_rows(bp, tune):
     """The C-ABI call accumulates (include/bp_ternary.h): the kernel reads what it adds to when a workgroup starts and
     writes once at its end; rows of experts without a token and rows past N / 16 tiles of a workgroup stay as they were."""
@@ -708,6 +735,21 @@ def test_tq2_mfma_variants(bp, act, K, counts):
     got, want, kern = _run(bp, "tq2", 3, 2048 + 16 if K <= 2048 else 64, K, counts, act, terms=2 if K == 4096 else 1, seed=K + len(act))
     assert kern.startswith("gemm_tq2" if max(counts) > 16 else "mfma_tq2"), kern
     _check(got, want)
+
+
+@pytest.mark.parametrize("rows", [3, 5, 7, 11])
+def test_tq2_token_tiles_of_large_calls_stage_every_row(bp, tune, rows):
+    """Large calls run the 16-wave variant of the token-tile kernel, whose activation tile holds 1.5 sixteen-element
+    units per thread with 16-bit activations: with 3 - 7 or 9 - 11 rows per expert the tile is longer than one unit per
+    thread, and every row of it has to be staged (the last rows once were not)."""
+    tune("BP_TUNE_TQ2V", "n")  # (three rows: keep the K-split GEMV out of the way)
+    E, N, K = 8, 4096, 4096
+    got, want, kern = _run(bp, "tq2", E, N, K, [rows] * E, "bf16", seed=rows)
+    assert kern == "mfma_tq2_bf16_r1_m1_w16", kern
+    _check(got, want)
+    for e in range(E):  # (the last row of each expert by itself: a tile's last rows are the ones that were left out)
+        r = (e + 1) * rows - 1
+        assert rel_l2(got[r], want[r]) <= REL_L2, (e, rel_l2(got[r], want[r]))
 
 
 def test_tq2_bf16_scales_and_f32_scales(bp):
