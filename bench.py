@@ -99,6 +99,8 @@ WORKLOADS = {
     "cfg1a_tq2_gemv": ("tq2", 2048, 7168, 1, "bf16", 1, 128),
     "cfg0_tq2_gemv": ("tq2", 2048, 4096, 1, "bf16", 1, 192),
     "cfg1a_tq2_i8_gemv": ("tq2", 2048, 7168, 1, "int8", 1, 128),
+    "cfg1a_tq1_gemv_L256": ("tq1", 2048, 7168, 1, "bf16", 1, 256),  # twice the linears per launch: the launch's fixed part against twice the bytes
+    "cfg1a_tq2_gemv_L256": ("tq2", 2048, 7168, 1, "bf16", 1, 256),
     "cfg1a_tq1_one_linear": ("tq1", 2048, 7168, 1, "bf16", 1, 1),  # what one TernaryLinear call issues (latency-bound: 3 MB)
 }
 
