@@ -23,6 +23,7 @@ __global__ __launch_bounds__(WAVES * 64, 4) void k_mfma_tq2(GemmArgs a, int KC, 
   constexpr int KM = ACT == BP_BF16 ? 8 : 16;  // k per lane per MFMA
   constexpr int NJ = 32 / KM;                  // MFMAs per group
   constexpr int XU = (XKB * 1024 / (16 * XB) + THREADS - 1) / THREADS;  // 16-element units of the activation tile per thread (rounded up: 16 waves and 16-bit activations hold 1.5 each)
+  static_assert(XU * THREADS * 16 * XB >= XKB * 1024, "every unit of the activation tile has a thread that stages it");
 
   // the wave index through readfirstlane: everything derived from it stays in scalar registers
   const int wave = __builtin_amdgcn_readfirstlane((int)(threadIdx.x >> 6)), lane = threadIdx.x & 63;
